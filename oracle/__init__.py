@@ -1,0 +1,352 @@
+"""numpy front-end of the CPU oracle (liboracle.so) and of the compiled
+reference (_ref/libref.so, when it has been built).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by the smoke check and by the
+CPU-baseline leg of the benchmark.  The shipped library never imports it.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "liboracle.so")
+_REF = os.path.join(_HERE, "_ref", "libref.so")
+
+# wire ids (include/quant/types.h:22-66 of the reference) + appended literal formats
+FMT = {
+    "Q_4": 3, "Q_8": 5, "Q_32": 9,
+    "Q_G_2": 38, "Q_G_3": 39, "Q_G_4": 40, "Q_G_8": 42,
+    "Q_3_5": 75, "Q_4_5": 76, "Q_8_5": 78, "Q_G_3_5": 84, "Q_G_4_5": 85, "Q_G_8_5": 87,
+    "B32S4": 105, "B32S8": 106, "SB256A3": 107, "SB256A2": 108,
+}
+# formats that exist in the reference (the compiled reference can run them)
+REF_FORMATS = [k for k, v in FMT.items() if v < 105]
+
+_u8p = C.POINTER(C.c_uint8)
+_f32p = C.POINTER(C.c_float)
+
+
+def build(force: bool = False) -> None:
+    """Compile liboracle.so (and _ref/libref.so where the reference tree exists)."""
+    if force or not os.path.exists(_LIB):
+        subprocess.check_call(["make", "-s", "-C", _HERE, "all"])
+
+
+def _load(path):
+    return C.CDLL(path) if os.path.exists(path) else None
+
+
+build()
+lib = _load(_LIB)
+ref = _load(_REF)
+
+
+def have_ref() -> bool:
+    return ref is not None
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _ptr(a, t):
+    return a.ctypes.data_as(t)
+
+
+lib.orc_f32_to_f16.restype = C.c_uint16
+lib.orc_f32_to_f16.argtypes = [C.c_float]
+lib.orc_f16_to_f32.restype = C.c_float
+lib.orc_f16_to_f32.argtypes = [C.c_uint16]
+lib.orc_block_bytes.restype = C.c_long
+lib.orc_block_bytes.argtypes = [C.c_uint8, C.c_int]
+lib.orc_encode_block.restype = C.c_long
+lib.orc_encode_block.argtypes = [C.c_uint8, _f32p, C.c_int, _u8p, C.c_size_t]
+lib.orc_decode_block.restype = C.c_int
+lib.orc_decode_block.argtypes = [C.c_uint8, _u8p, C.c_size_t, C.c_int, _f32p]
+lib.orc_encode_tensor.restype = C.c_long
+lib.orc_encode_tensor.argtypes = [C.c_uint8, _f32p, C.c_int64, _u8p, C.c_size_t, C.c_int]
+lib.orc_decode_tensor.restype = C.c_int
+lib.orc_decode_tensor.argtypes = [C.c_uint8, _u8p, C.c_size_t, C.c_int64, _f32p, C.c_int]
+lib.orc_matmul.restype = C.c_int
+lib.orc_matmul.argtypes = [C.c_uint8, _u8p, C.c_int64, C.c_int64, _f32p, C.c_int, _f32p, C.c_int]
+lib.orc_matmul_f64.restype = C.c_int
+lib.orc_matmul_f64.argtypes = [C.c_uint8, _u8p, C.c_int64, C.c_int64, _f32p, C.c_int,
+                               C.POINTER(C.c_double), C.c_int]
+lib.orc_rng_normal.argtypes = [C.c_uint64, C.c_int64, C.c_float, _f32p]
+lib.orc_rng_uniform.argtypes = [C.c_uint64, C.c_int64, _f32p]
+lib.orc_rng_u64.argtypes = [C.c_uint64, C.c_int64, C.POINTER(C.c_uint64)]
+lib.orc_rng_laplace.argtypes = [C.c_uint64, C.c_int64, C.c_float, _f32p]
+lib.orc_softmax_topk.argtypes = [_f32p, C.c_int64, C.c_int64, C.c_int64, _f32p,
+                                 C.POINTER(C.c_int64), _f32p]
+lib.orc_silu_mul.argtypes = [_f32p, _f32p, C.c_int64, _f32p]
+lib.orc_moe_ffn.restype = C.c_int
+lib.orc_moe_ffn.argtypes = [C.c_uint8, C.POINTER(_u8p), C.POINTER(_u8p), C.POINTER(_u8p), C.c_int,
+                            C.c_int64, C.c_int64, C.POINTER(C.c_int64), _f32p, C.c_int64, C.c_int64,
+                            _f32p, _f32p, C.c_int, C.c_int]
+lib.orc_quant4_gemm.argtypes = [_u8p, C.POINTER(C.c_uint16), _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+lib.orc_quant8_gemm.argtypes = [_u8p, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+lib.orc_comp8_table.argtypes = [_f32p]
+
+THREADS = min(16, os.cpu_count() or 1)
+
+
+def fmt_id(fmt) -> int:
+    return FMT[fmt] if isinstance(fmt, str) else int(fmt)
+
+
+def f32_to_f16(v: float) -> int:
+    return int(lib.orc_f32_to_f16(float(v)))
+
+
+def f16_to_f32(h: int) -> float:
+    return float(lib.orc_f16_to_f32(int(h)))
+
+
+def comp8_table() -> np.ndarray:
+    out = np.empty(256, np.float32)
+    lib.orc_comp8_table(_ptr(out, _f32p))
+    return out
+
+
+def block_bytes(fmt, n: int = 256) -> int:
+    return int(lib.orc_block_bytes(fmt_id(fmt), n))
+
+
+def encode_block(fmt, w) -> np.ndarray:
+    w = _f32(w)
+    need = block_bytes(fmt, w.size)
+    if need < 0:
+        raise ValueError(f"format {fmt} cannot encode a block of {w.size}")
+    out = np.zeros(need, np.uint8)
+    r = lib.orc_encode_block(fmt_id(fmt), _ptr(w, _f32p), w.size, _ptr(out, _u8p), need)
+    if r != need:
+        raise RuntimeError("oracle encode failed")
+    return out
+
+
+def decode_block(fmt, payload, n: int = 256) -> np.ndarray:
+    payload = np.ascontiguousarray(payload, np.uint8)
+    out = np.empty(n, np.float32)
+    if lib.orc_decode_block(fmt_id(fmt), _ptr(payload, _u8p), payload.size, n, _ptr(out, _f32p)) != 0:
+        raise RuntimeError("oracle decode failed")
+    return out
+
+
+def encode_tensor(fmt, w, threads: int = THREADS) -> np.ndarray:
+    w = _f32(w).reshape(-1)
+    nb = (w.size + 255) // 256
+    tail = w.size - (nb - 1) * 256
+    cap = (nb - 1) * max(block_bytes(fmt, 256), 0) + block_bytes(fmt, tail)
+    out = np.zeros(cap, np.uint8)
+    r = lib.orc_encode_tensor(fmt_id(fmt), _ptr(w, _f32p), w.size, _ptr(out, _u8p), cap, threads)
+    if r != cap:
+        raise RuntimeError("oracle encode_tensor failed")
+    return out
+
+
+def decode_tensor(fmt, payload, total: int, threads: int = THREADS) -> np.ndarray:
+    payload = np.ascontiguousarray(payload, np.uint8)
+    out = np.empty(total, np.float32)
+    if lib.orc_decode_tensor(fmt_id(fmt), _ptr(payload, _u8p), payload.size, total, _ptr(out, _f32p), threads):
+        raise RuntimeError("oracle decode_tensor failed")
+    return out
+
+
+def matmul(fmt, packed, N: int, K: int, X, threads: int = THREADS) -> np.ndarray:
+    """Y[B][N] = X[B][K] . W^T in the reference engine's accumulation order (fp32)."""
+    packed = np.ascontiguousarray(packed, np.uint8)
+    X = _f32(X).reshape(-1, K)
+    Y = np.empty((X.shape[0], N), np.float32)
+    if lib.orc_matmul(fmt_id(fmt), _ptr(packed, _u8p), N, K, _ptr(X, _f32p), X.shape[0], _ptr(Y, _f32p), threads):
+        raise RuntimeError("oracle matmul failed")
+    return Y
+
+
+def matmul_f64(fmt, packed, N: int, K: int, X, threads: int = THREADS) -> np.ndarray:
+    packed = np.ascontiguousarray(packed, np.uint8)
+    X = _f32(X).reshape(-1, K)
+    Y = np.empty((X.shape[0], N), np.float64)
+    if lib.orc_matmul_f64(fmt_id(fmt), _ptr(packed, _u8p), N, K, _ptr(X, _f32p), X.shape[0],
+                          Y.ctypes.data_as(C.POINTER(C.c_double)), threads):
+        raise RuntimeError("oracle matmul_f64 failed")
+    return Y
+
+
+def rng_normal(seed: int, n: int, scale: float = 1.0) -> np.ndarray:
+    out = np.empty(n, np.float32)
+    lib.orc_rng_normal(seed, n, scale, _ptr(out, _f32p))
+    return out
+
+
+def rng_uniform(seed: int, n: int) -> np.ndarray:
+    out = np.empty(n, np.float32)
+    lib.orc_rng_uniform(seed, n, _ptr(out, _f32p))
+    return out
+
+
+def rng_u64(seed: int, n: int) -> np.ndarray:
+    out = np.empty(n, np.uint64)
+    lib.orc_rng_u64(seed, n, out.ctypes.data_as(C.POINTER(C.c_uint64)))
+    return out
+
+
+def rng_laplace(seed: int, n: int, b: float) -> np.ndarray:
+    out = np.empty(n, np.float32)
+    lib.orc_rng_laplace(seed, n, b, _ptr(out, _f32p))
+    return out
+
+
+def bf16_round(a) -> np.ndarray:
+    """fp32 -> nearest-even bf16 -> fp32 (the reference has no bf16 type; this is
+    how 'bf16 activations' enter its fp32 matmul)."""
+    a = _f32(a)
+    u = a.view(np.uint32).astype(np.uint64)
+    finite = (u & 0x7F800000) != 0x7F800000
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000).astype(np.uint32)
+    return np.where(finite, r, a.view(np.uint32)).astype(np.uint32).view(np.float32).reshape(a.shape)
+
+
+def softmax_topk(logits, k: int):
+    logits = _f32(logits)
+    T, E = logits.shape
+    k = max(1, min(k, E))
+    probs = np.empty((T, E), np.float32)
+    idx = np.empty((T, k), np.int64)
+    w = np.empty((T, k), np.float32)
+    lib.orc_softmax_topk(_ptr(logits, _f32p), T, E, k, _ptr(probs, _f32p),
+                         idx.ctypes.data_as(C.POINTER(C.c_int64)), _ptr(w, _f32p))
+    return probs, idx, w
+
+
+def silu_mul(g, u) -> np.ndarray:
+    g, u = _f32(g), _f32(u)
+    out = np.empty_like(g)
+    lib.orc_silu_mul(_ptr(g, _f32p), _ptr(u, _f32p), g.size, _ptr(out, _f32p))
+    return out
+
+
+def moe_ffn(fmt, gate, up, down, D: int, F: int, topk_idx, topk_w, x, mid_bf16: bool = False,
+            threads: int = THREADS) -> np.ndarray:
+    E = len(gate)
+    keep = [np.ascontiguousarray(a, np.uint8) for a in list(gate) + list(up) + list(down)]
+    arr = lambda xs: (_u8p * E)(*[_ptr(a, _u8p) for a in xs])
+    topk_idx = np.ascontiguousarray(topk_idx, np.int64)
+    topk_w = _f32(topk_w)
+    x = _f32(x)
+    T, Kk = topk_idx.shape
+    out = np.empty((T, D), np.float32)
+    r = lib.orc_moe_ffn(fmt_id(fmt), arr(keep[:E]), arr(keep[E:2 * E]), arr(keep[2 * E:]), E, D, F,
+                        topk_idx.ctypes.data_as(C.POINTER(C.c_int64)), _ptr(topk_w, _f32p), T, Kk,
+                        _ptr(x, _f32p), _ptr(out, _f32p), int(mid_bf16), threads)
+    if r:
+        raise RuntimeError("oracle moe_ffn failed")
+    return out
+
+
+def quant4_gemm(w, cb16, act, M: int, N: int, K: int) -> np.ndarray:
+    w = np.ascontiguousarray(w, np.uint8)
+    cb16 = np.ascontiguousarray(cb16, np.uint16)
+    act = _f32(act)
+    out = np.empty((M, N), np.float32)
+    lib.orc_quant4_gemm(_ptr(w, _u8p), cb16.ctypes.data_as(C.POINTER(C.c_uint16)), _ptr(act, _f32p),
+                        _ptr(out, _f32p), M, N, K)
+    return out
+
+
+def quant8_gemm(idx, cb256, act, M: int, N: int, K: int) -> np.ndarray:
+    idx = np.ascontiguousarray(idx, np.uint8)
+    cb256, act = _f32(cb256), _f32(act)
+    out = np.empty((M, N), np.float32)
+    lib.orc_quant8_gemm(_ptr(idx, _u8p), _ptr(cb256, _f32p), _ptr(act, _f32p), _ptr(out, _f32p), M, N, K)
+    return out
+
+
+# ------------------------------------------------------------ compiled reference
+if ref is not None:
+    ref.ref_quantize_block.restype = C.c_long
+    ref.ref_quantize_block.argtypes = [C.c_uint8, _f32p, C.c_int, _u8p, C.c_size_t]
+    ref.ref_dequantize_block.argtypes = [C.c_uint8, _u8p, C.c_size_t, C.c_uint32, _f32p]
+    ref.ref_block_claimed_bytes.restype = C.c_size_t
+    ref.ref_block_claimed_bytes.argtypes = [C.c_uint8, C.c_uint32]
+    ref.ref_format_bpw.restype = C.c_float
+    ref.ref_format_bpw.argtypes = [C.c_uint8]
+    ref.ref_format_name.restype = C.c_char_p
+    ref.ref_format_name.argtypes = [C.c_uint8]
+    ref.ref_registry_quantize.restype = C.c_long
+    ref.ref_registry_quantize.argtypes = [C.c_char_p, _f32p, C.c_int64, _u8p, C.c_size_t,
+                                          C.POINTER(C.c_uint32), C.c_int64]
+    ref.ref_registry_roundtrip.restype = C.c_int
+    ref.ref_registry_roundtrip.argtypes = [C.c_char_p, _f32p, C.c_int64, _f32p]
+    ref.ref_parse_format_id.restype = C.c_int
+    ref.ref_parse_format_id.argtypes = [C.c_char_p]
+    ref.ref_rng_normal.argtypes = [C.c_uint64, C.c_int64, C.c_float, _f32p]
+    ref.ref_rng_uniform.argtypes = [C.c_uint64, C.c_int64, _f32p]
+    ref.ref_rng_u64.argtypes = [C.c_uint64, C.c_int64, C.POINTER(C.c_uint64)]
+    ref.ref_quant4_gemm.argtypes = [_u8p, C.POINTER(C.c_uint16), _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+    ref.ref_quant8_gemm.argtypes = [_u8p, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+    ref.ref_scalar_gemm_bt.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+    ref.ref_gemv_quant4_tiled.argtypes = [_u8p, C.POINTER(C.c_uint16), C.c_float, _f32p, _f32p, C.c_int, C.c_int]
+    ref.ref_gemv_quant8_tiled.argtypes = [_u8p, _f32p, C.c_float, _f32p, _f32p, C.c_int, C.c_int]
+    ref.ref_detect_cpu_isa.restype = C.c_int
+
+
+def ref_encode_block(fmt, w) -> np.ndarray:
+    w = _f32(w)
+    out = np.zeros(w.size * 4 + 64, np.uint8)
+    r = ref.ref_quantize_block(fmt_id(fmt), _ptr(w, _f32p), w.size, _ptr(out, _u8p), out.size)
+    if r < 0:
+        raise RuntimeError(f"reference quantize failed ({r})")
+    return out[:r].copy()
+
+
+def ref_decode_block(fmt, payload, n: int = 256) -> np.ndarray:
+    payload = np.ascontiguousarray(payload, np.uint8)
+    out = np.empty(n, np.float32)
+    ref.ref_dequantize_block(fmt_id(fmt), _ptr(payload, _u8p), payload.size, n, _ptr(out, _f32p))
+    return out
+
+
+def ref_rng_normal(seed: int, n: int, scale: float = 1.0) -> np.ndarray:
+    out = np.empty(n, np.float32)
+    ref.ref_rng_normal(seed, n, scale, _ptr(out, _f32p))
+    return out
+
+
+def ref_rng_uniform(seed: int, n: int) -> np.ndarray:
+    out = np.empty(n, np.float32)
+    ref.ref_rng_uniform(seed, n, _ptr(out, _f32p))
+    return out
+
+
+def ref_registry_quantize(name: str, data):
+    data = _f32(data).reshape(-1)
+    nb = (data.size + 255) // 256
+    out = np.zeros(data.size * 4 + 64 * nb, np.uint8)
+    per = np.zeros(nb, np.uint32)
+    r = ref.ref_registry_quantize(name.encode(), _ptr(data, _f32p), data.size, _ptr(out, _u8p), out.size,
+                                  per.ctypes.data_as(C.POINTER(C.c_uint32)), nb)
+    if r < 0:
+        raise RuntimeError(f"reference registry quantize failed ({r})")
+    return out[:r].copy(), per
+
+
+def ref_quant4_gemm(w, cb16, act, M, N, K) -> np.ndarray:
+    w = np.ascontiguousarray(w, np.uint8)
+    cb16 = np.ascontiguousarray(cb16, np.uint16)
+    act = _f32(act)
+    out = np.empty((M, N), np.float32)
+    ref.ref_quant4_gemm(_ptr(w, _u8p), cb16.ctypes.data_as(C.POINTER(C.c_uint16)), _ptr(act, _f32p),
+                        _ptr(out, _f32p), M, N, K)
+    return out
+
+
+def ref_quant8_gemm(idx, cb256, act, M, N, K) -> np.ndarray:
+    idx = np.ascontiguousarray(idx, np.uint8)
+    cb256, act = _f32(cb256), _f32(act)
+    out = np.empty((M, N), np.float32)
+    ref.ref_quant8_gemm(_ptr(idx, _u8p), _ptr(cb256, _f32p), _ptr(act, _f32p), _ptr(out, _f32p), M, N, K)
+    return out
