@@ -1,0 +1,123 @@
+/*
+ * tfq.h - C ABI of the MI355X (gfx950) backend for the block-quantized weight
+ * matmul: block codec, dequant-fused GEMV / GEMM, MoE expert FFN.
+ *
+ * Every entry point takes plain pointers and sizes.  Unless a name ends in
+ * _host, data pointers are DEVICE pointers and the call is asynchronous on the
+ * given stream (a hipStream_t passed as void*, NULL = the default stream).
+ * Functions return TFQ_OK (0) or a TFQ_ERR_* code; tfq_last_error() returns a
+ * thread-local message for the last failure on the calling thread.  No entry
+ * point falls back to a CPU implementation: without a usable gfx950 device
+ * every compute call fails with TFQ_ERR_DEVICE (the reference's GPU back-ends
+ * behave the same way, "REAL-ONLY": src/backend/backend.cpp:1959-1993).
+ *
+ * Each declaration cites the reference interface it stands behind
+ * (paths relative to the reference tree).
+ */
+#ifndef TFQ_H
+#define TFQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    TFQ_OK = 0,
+    TFQ_ERR_ARG = 1,     /* null pointer, non-positive size, bad dtype          */
+    TFQ_ERR_FORMAT = 2,  /* wire id not handled by this backend                 */
+    TFQ_ERR_SHAPE = 3,   /* K not a multiple of 256, payload size mismatch, ... */
+    TFQ_ERR_DEVICE = 4,  /* no gfx950 device, HIP error                         */
+    TFQ_ERR_NOMEM = 5
+};
+
+/* activation / output element types */
+enum { TFQ_F32 = 0, TFQ_BF16 = 1 };
+
+/* Wire ids.  0..104 are the reference's Format enum (include/quant/types.h:22-66)
+ * and keep their values because they are stored on disk; the four literal
+ * formats are appended after FORMAT_COUNT (105). */
+enum {
+    TFQ_Q_4 = 3, TFQ_Q_8 = 5, TFQ_Q_32 = 9,
+    TFQ_Q_G_2 = 38, TFQ_Q_G_3 = 39, TFQ_Q_G_4 = 40, TFQ_Q_G_8 = 42,
+    TFQ_Q_3_5 = 75, TFQ_Q_4_5 = 76, TFQ_Q_8_5 = 78,
+    TFQ_Q_G_3_5 = 84, TFQ_Q_G_4_5 = 85, TFQ_Q_G_8_5 = 87,
+    TFQ_B32S4 = 105,   /* 32-group symmetric 4-bit, binary16 scale = absmax/7   */
+    TFQ_B32S8 = 106,   /* 32-group symmetric 8-bit, binary16 scale = absmax/127 */
+    TFQ_SB256A3 = 107, /* 256-superblock, 16x16 sub-blocks, 6-bit scale + min, 3-bit codes */
+    TFQ_SB256A2 = 108  /* same with 2-bit codes                                  */
+};
+
+typedef struct tfq_weight tfq_weight_t; /* device-resident packed matrix, opaque */
+typedef void* tfq_stream_t;             /* hipStream_t                           */
+
+/* ---- library / errors ---------------------------------------------------
+ * Error convention follows the reference C API: status + thread-local message
+ * (quant_last_error, src/server/production_core.cpp:29-100). */
+int tfq_init(int device);
+const char* tfq_last_error(void);
+const char* tfq_version(void);
+
+/* ---- format registry ------------------------------------------------------
+ * format_name / format_bpw: include/quant/types.h:168-230.
+ * tfq_format_id: FormatRegistry::parse_format_name + regformat_to_format
+ * (src/codec/format_registry.cpp:462-483, include/quant/format_registry.h:245-280);
+ * accepts "Q_G_4", "QG4", "qg4", "Q4.5"-style spellings; -1 if unknown.
+ * tfq_block_bytes: payload bytes of one block of n weights, the size
+ * quantize_block_all produces (include/quant/block_codec.h:62-70). */
+int tfq_format_id(const char* name);
+const char* tfq_format_name(uint8_t fmt);
+float tfq_format_bpw(uint8_t fmt);
+int tfq_format_supported(uint8_t fmt);
+int tfq_block_bytes(uint8_t fmt, uint32_t n, size_t* out);
+
+/* ---- block codec ------------------------------------------------------------
+ * quantize_block_all / dequantize_block_all (include/quant/block_codec.h:69-77),
+ * applied to a tensor cut into 256-weight blocks the way
+ * FormatRegistry::quantize / dequantize do (src/codec/format_registry.cpp:168-207,
+ * 241-290): payloads are concatenated in block order.  n must be a multiple of
+ * 256.  dst/src and w/out are device pointers. */
+int tfq_encode_blocks(uint8_t fmt, const float* w, int64_t n, uint8_t* dst, size_t cap,
+                      tfq_stream_t stream);
+int tfq_decode_blocks(uint8_t fmt, const uint8_t* src, size_t bytes, int64_t n, float* out,
+                      tfq_stream_t stream);
+/* Same with host pointers (copies in, runs the kernel, copies out, synchronises);
+ * per_block_bytes (may be NULL) receives each block's payload size like
+ * QuantResult::block_idx_bytes (include/quant/format_registry.h:112-125). */
+int tfq_encode_blocks_host(uint8_t fmt, const float* w, int64_t n, uint8_t* dst, size_t cap,
+                           uint32_t* per_block_bytes);
+int tfq_decode_blocks_host(uint8_t fmt, const uint8_t* src, size_t bytes, int64_t n, float* out);
+
+/* ---- packed weight matrices ---------------------------------------------------
+ * W is N rows of K/256 consecutive wire blocks, the layout Qwen35Engine::gemm
+ * walks (src/adapters/tools/qwen35_engine.cpp:58,82-86).  upload copies a host
+ * payload to the device; wrap borrows a device payload (the caller keeps it
+ * alive).  Both return NULL on failure. */
+tfq_weight_t* tfq_weight_upload(uint8_t fmt, int64_t N, int64_t K, const uint8_t* packed_host,
+                                size_t bytes);
+tfq_weight_t* tfq_weight_wrap(uint8_t fmt, int64_t N, int64_t K, const uint8_t* packed_dev,
+                              size_t bytes);
+void tfq_weight_free(tfq_weight_t* w);
+int tfq_weight_info(const tfq_weight_t* w, uint8_t* fmt, int64_t* N, int64_t* K, size_t* bytes);
+/* decoded fp32 matrix [N][K] (device) */
+int tfq_weight_decode(const tfq_weight_t* w, float* out, tfq_stream_t stream);
+
+/* ---- dequant-fused matmul -------------------------------------------------------
+ * y[b][n] = sum_k x[b][k] * W[n][k], fp32 accumulation.
+ * Replaces Qwen35Engine::gemm (src/adapters/tools/qwen35_engine.cpp:54-101):
+ * tfq_gemv is the decode path (B rows, 1 <= B <= 16), tfq_gemm the prefill
+ * path (any M).  x is [B][K], y is [B][N], row-major, dtypes TFQ_F32 / TFQ_BF16. */
+int tfq_gemv(const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, int y_dtype,
+             tfq_stream_t stream);
+int tfq_gemm(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
+             tfq_stream_t stream);
+/* host-pointer form of tfq_gemv/tfq_gemm with fp32 x and y: the exact call
+ * shape of Qwen35Engine::gemm(t, X, Y, B). */
+int tfq_matmul_host(const tfq_weight_t* w, const float* X, float* Y, int B);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TFQ_H */

@@ -1,0 +1,109 @@
+"""Writes the golden fixtures from the COMPILED REFERENCE (oracle/_ref/libref.so,
+built from the reference's own sources by oracle/Makefile).  Run it where the
+reference tree exists; the fixtures it writes are what travels.
+
+    python tests/golden/make_golden.py
+
+codec.npz
+    w            [4 distributions x 8 blocks x 256] fp32 inputs (seeded with the
+                 reference generator: N(0,0.02) seed 42, N(0,1) seed 43,
+                 Laplace(0,0.015) seed 44, heavy-tail mix seed 46)
+    <fmt>_payload  uint8 payload of every block, reference quantize_block_all
+    <fmt>_decoded  fp32 output of reference dequantize_block_all on that payload
+    comp8_levels  the 256-entry companded grid (decoded from a Q_G_8 payload
+                 with codes 0..255 and scale 1.0)
+    f16_all_decoded  binary32 bit patterns the reference decodes all 65,536
+                 binary16 patterns to (each pattern placed as a Q_G_8 group scale
+                 over code 255, whose level is exactly 1.0)
+rng.npz
+    u64_42, uniform_42, normal_42_002, normal_43: first 4096 draws of RNG(seed)
+matmul.npz
+    for Q_G_4 and Q_G_8: y = x.W^T with W 48x512 from the fixture generator,
+    computed by the reference scalar_gemm_bt on the reference-decoded matrix
+"""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+import oracle as O  # noqa: E402
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+FORMATS = ["Q_4", "Q_8", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_8", "Q_32"]
+
+
+def inputs():
+    nb = 8
+    a = O.ref_rng_normal(42, nb * 256, 0.02)
+    b = O.ref_rng_normal(43, nb * 256, 1.0)
+    u = O.ref_rng_uniform(44, nb * 256) - np.float32(0.5)
+    c = (-np.float32(0.015) * np.sign(u) * np.log(np.float32(1) - np.float32(2) * np.abs(u))).astype(np.float32)
+    d = O.ref_rng_normal(46, nb * 256, 0.02)
+    d[::37] *= np.float32(25.0)
+    d[256:512] = 0.0              # an all-zero block
+    d[512:768] = np.float32(0.5)  # a constant block
+    d[768:800] = 0.0              # one zero group inside a live block
+    return np.stack([a, b, c, d]).reshape(4, nb, 256)
+
+
+def main():
+    assert O.have_ref(), "build oracle/_ref first (make -C oracle)"
+    w = inputs()
+    out = {"w": w}
+    for fmt in FORMATS:
+        pays, decs = [], []
+        for blk in w.reshape(-1, 256):
+            p = O.ref_encode_block(fmt, blk)
+            pays.append(p)
+            decs.append(O.ref_decode_block(fmt, p))
+        out[f"{fmt}_payload"] = np.stack(pays)
+        out[f"{fmt}_decoded"] = np.stack(decs)
+    p = np.zeros(272, np.uint8)
+    p[:256] = np.arange(256)
+    p[257:272:2] = 0x3C
+    out["comp8_levels"] = O.ref_decode_block("Q_G_8", p)
+    # binary16 -> binary32 seen through the codec: every 16-bit pattern as a
+    # Q_G_8 group scale over code 255 (level exactly 1.0).
+    dec = np.empty(65536, np.float32)
+    for h0 in range(0, 65536, 8):
+        q = np.zeros(272, np.uint8)
+        q[:256] = 255
+        for g in range(8):
+            q[256 + 2 * g] = (h0 + g) & 0xFF
+            q[256 + 2 * g + 1] = (h0 + g) >> 8
+        dec[h0:h0 + 8] = O.ref_decode_block("Q_G_8", q)[::32]
+    out["f16_all_decoded"] = dec.view(np.uint32)
+    np.savez_compressed(os.path.join(HERE, "codec.npz"), **out)
+
+    rng = {
+        "u64_42": np.empty(4096, np.uint64),
+        "uniform_42": O.ref_rng_uniform(42, 4096),
+        "normal_42_002": O.ref_rng_normal(42, 4096, 0.02),
+        "normal_43": O.ref_rng_normal(43, 4096, 1.0),
+    }
+    import ctypes as C
+    O.ref.ref_rng_u64(42, 4096, rng["u64_42"].ctypes.data_as(C.POINTER(C.c_uint64)))
+    np.savez_compressed(os.path.join(HERE, "rng.npz"), **rng)
+
+    N, K, B = 48, 512, 3
+    W = O.ref_rng_normal(47, N * K, 0.02)
+    X = O.ref_rng_normal(48, B * K, 1.0)
+    mm = {"W": W, "X": X}
+    for fmt in ("Q_G_4", "Q_G_8", "Q_4"):
+        pays = np.concatenate([O.ref_encode_block(fmt, W[i:i + 256]) for i in range(0, N * K, 256)])
+        dec = np.concatenate([O.ref_decode_block(fmt, pays[i:i + len(pays) // (N * K // 256)])
+                              for i in range(0, len(pays), len(pays) // (N * K // 256))])
+        Y = np.empty((B, N), np.float32)
+        _f = C.POINTER(C.c_float)
+        O.ref.ref_scalar_gemm_bt(X.ctypes.data_as(_f), dec.ctypes.data_as(_f), Y.ctypes.data_as(_f), B, N, K)
+        mm[f"{fmt}_payload"] = pays
+        mm[f"{fmt}_y"] = Y
+    np.savez_compressed(os.path.join(HERE, "matmul.npz"), **mm)
+    for f in ("codec.npz", "rng.npz", "matmul.npz"):
+        print(f, os.path.getsize(os.path.join(HERE, f)))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,99 @@
+"""Device codec through the C ABI against the oracle: decoded weights and
+device-encoded codes must be bit-exact."""
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+G = os.path.join(os.path.dirname(__file__), "golden")
+DECODE_FORMATS = ["Q_4", "Q_8", "Q_32", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_8", "Q_4_5", "Q_G_8_5",
+                  "B32S4", "B32S8", "SB256A3", "SB256A2"]
+
+
+def _inputs(O, nblk):
+    rng = np.random.default_rng(31)
+    w = np.concatenate([O.rng_normal(42, nblk * 256, 0.02), O.rng_laplace(44, nblk * 256, 0.015),
+                        rng.standard_normal(nblk * 256).astype(np.float32)])
+    w[256:512] = 0.0
+    w[512:544] = 0.0
+    w[1024:1280] = 0.75
+    return w
+
+
+@pytest.mark.parametrize("fmt", DECODE_FORMATS)
+def test_decode_bit_exact(O, tfq, gpu, fmt):
+    import torch
+    print(f"decode {fmt}", flush=True)
+    w = _inputs(O, 64)
+    pay = O.encode_tensor(fmt, w)
+    want = O.decode_tensor(fmt, pay, w.size)
+    got = tfq.decode(fmt, torch.from_numpy(pay).to(gpu), w.size).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("fmt", ["Q_4", "Q_8", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_8"])
+def test_decode_golden_payloads(tfq, gpu, fmt):
+    import torch
+    c = np.load(os.path.join(G, "codec.npz"))
+    pay, want = c[f"{fmt}_payload"], c[f"{fmt}_decoded"]
+    got = tfq.decode(fmt, torch.from_numpy(pay.reshape(-1)).to(gpu), want.size).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.reshape(-1).view(np.uint32))
+
+
+@pytest.mark.parametrize("fmt", ["Q_4", "Q_8", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_8", "SB256A3", "SB256A2"])
+def test_decode_arbitrary_payload_bits(O, tfq, gpu, fmt):
+    # every payload bit pattern is legal input: random bytes, finite scales
+    import torch
+    rng = np.random.default_rng(17)
+    nb = O.block_bytes(fmt)
+    pay = rng.integers(0, 256, (256, nb), dtype=np.uint8)
+    if fmt in ("Q_G_8",):
+        pay[:, -16:] &= 0x7B
+    elif fmt in ("Q_4", "Q_8"):
+        pay[:, :2] &= 0x7B
+    else:
+        pay[:, -4:] &= 0x7B
+    want = O.decode_tensor(fmt, pay.reshape(-1), 256 * 256)
+    got = tfq.decode(fmt, torch.from_numpy(pay.reshape(-1)).to(gpu), 256 * 256).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_half_subnormal_scales_decode_exactly(O, tfq, gpu):
+    import torch
+    pay = np.zeros((128, 272), np.uint8)
+    pay[:, :256] = 255
+    hs = np.concatenate([np.arange(0, 512), np.arange(0x8000, 0x8000 + 512)]).astype(np.uint16)
+    pay[:, 256:] = hs.reshape(128, 8).view(np.uint8).reshape(128, 16)
+    want = O.decode_tensor("Q_G_8", pay.reshape(-1), 128 * 256)
+    got = tfq.decode("Q_G_8", torch.from_numpy(pay.reshape(-1)).to(gpu), 128 * 256).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("fmt", ["B32S4", "B32S8", "Q_32"])
+def test_device_encoder_codes_bit_exact(O, tfq, gpu, fmt):
+    import torch
+    w = _inputs(O, 64)
+    w[2048:2080] = 1e-9          # scale underflows binary16
+    w[4096] = 3.0e5              # scale overflows binary16 -> inf -> codes 0
+    want = O.encode_tensor(fmt, w)
+    got = tfq.encode(fmt, torch.from_numpy(w).to(gpu)).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
+def test_host_pointer_codec_entry_points(O, tfq, gpu):
+    import ctypes as C
+    w = O.rng_normal(42, 256 * 8, 0.02)
+    L = tfq.lib()
+    dst = np.zeros(8 * 144, np.uint8)
+    per = np.zeros(8, np.uint32)
+    rc = L.tfq_encode_blocks_host(105, w.ctypes.data, w.size, dst.ctypes.data, dst.size, per.ctypes.data)
+    assert rc == 0 and np.all(per == 144)
+    assert np.array_equal(dst, O.encode_tensor("B32S4", w))
+    pay = O.encode_tensor("Q_G_4", w)
+    out = np.zeros(w.size, np.float32)
+    assert L.tfq_decode_blocks_host(40, pay.ctypes.data, pay.size, w.size, out.ctypes.data) == 0
+    assert np.array_equal(out.view(np.uint32), O.decode_tensor("Q_G_4", pay, w.size).view(np.uint32))
+    # an encoder this build does not have must say so, not encode on the CPU
+    assert L.tfq_encode_blocks_host(5, w.ctypes.data, w.size, dst.ctypes.data, dst.size, None) in (2, 3)

@@ -1,0 +1,185 @@
+"""ctypes binding of libtfq.so, the gfx950 backend for the block-quantized
+weight matmul.  PyTorch is used only to own device memory and streams; every
+computation is a hand-written HIP kernel reached through the C ABI declared in
+include/tfq.h.  There is no fallback: importing works without a GPU (so the
+symbol table can be inspected), but every compute call raises TfqError when
+the library or the device is missing.
+
+The directory name contains a hyphen, so import it with
+``importlib.import_module("transformers-fusion_amd")``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtfq.so")
+
+F32, BF16 = 0, 1
+
+FMT = {
+    "Q_4": 3, "Q_8": 5, "Q_32": 9,
+    "Q_G_2": 38, "Q_G_3": 39, "Q_G_4": 40, "Q_G_8": 42,
+    "Q_3_5": 75, "Q_4_5": 76, "Q_8_5": 78, "Q_G_3_5": 84, "Q_G_4_5": 85, "Q_G_8_5": 87,
+    "B32S4": 105, "B32S8": 106, "SB256A3": 107, "SB256A2": 108,
+}
+
+
+class TfqError(RuntimeError):
+    pass
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise TfqError(f"{LIB_PATH} is missing: run __graft_entry__.build() (hipcc) first")
+    lib = C.CDLL(LIB_PATH)
+    vp, u8, i32, i64, sz = C.c_void_p, C.c_uint8, C.c_int, C.c_int64, C.c_size_t
+    sig = {
+        "tfq_init": (i32, [i32]),
+        "tfq_last_error": (C.c_char_p, []),
+        "tfq_version": (C.c_char_p, []),
+        "tfq_format_id": (i32, [C.c_char_p]),
+        "tfq_format_name": (C.c_char_p, [u8]),
+        "tfq_format_bpw": (C.c_float, [u8]),
+        "tfq_format_supported": (i32, [u8]),
+        "tfq_block_bytes": (i32, [u8, C.c_uint32, C.POINTER(sz)]),
+        "tfq_encode_blocks": (i32, [u8, vp, i64, vp, sz, vp]),
+        "tfq_decode_blocks": (i32, [u8, vp, sz, i64, vp, vp]),
+        "tfq_encode_blocks_host": (i32, [u8, vp, i64, vp, sz, vp]),
+        "tfq_decode_blocks_host": (i32, [u8, vp, sz, i64, vp]),
+        "tfq_weight_upload": (vp, [u8, i64, i64, vp, sz]),
+        "tfq_weight_wrap": (vp, [u8, i64, i64, vp, sz]),
+        "tfq_weight_free": (None, [vp]),
+        "tfq_weight_info": (i32, [vp, C.POINTER(u8), C.POINTER(i64), C.POINTER(i64), C.POINTER(sz)]),
+        "tfq_weight_decode": (i32, [vp, vp, vp]),
+        "tfq_gemv": (i32, [vp, vp, i32, i32, vp, i32, vp]),
+        "tfq_gemm": (i32, [vp, vp, i32, i32, vp, i32, vp]),
+        "tfq_matmul_host": (i32, [vp, vp, vp, i32]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        _lib = _load()
+    return _lib
+
+
+def _check(rc: int):
+    if rc != 0:
+        raise TfqError(f"tfq error {rc}: {lib().tfq_last_error().decode()}")
+
+
+def fmt_id(fmt) -> int:
+    return FMT[fmt] if isinstance(fmt, str) else int(fmt)
+
+
+def block_bytes(fmt, n: int = 256) -> int:
+    out = C.c_size_t(0)
+    _check(lib().tfq_block_bytes(fmt_id(fmt), n, C.byref(out)))
+    return out.value
+
+
+def _stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dtype_code(t):
+    import torch
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.bfloat16:
+        return BF16
+    raise TfqError(f"unsupported dtype {t.dtype}")
+
+
+def init(device: int = 0):
+    _check(lib().tfq_init(device))
+
+
+def encode(fmt, w):
+    """fp32 device tensor (numel multiple of 256) -> uint8 device tensor of payloads."""
+    import torch
+    w = w.contiguous()
+    assert w.is_cuda and w.dtype == torch.float32
+    n = w.numel()
+    out = torch.empty((n // 256) * block_bytes(fmt), dtype=torch.uint8, device=w.device)
+    _check(lib().tfq_encode_blocks(fmt_id(fmt), w.data_ptr(), n, out.data_ptr(), out.numel(), _stream()))
+    return out
+
+
+def decode(fmt, payload, n: int):
+    import torch
+    assert payload.is_cuda and payload.dtype == torch.uint8
+    out = torch.empty(n, dtype=torch.float32, device=payload.device)
+    _check(lib().tfq_decode_blocks(fmt_id(fmt), payload.data_ptr(), payload.numel(), n, out.data_ptr(), _stream()))
+    return out
+
+
+class Weight:
+    """Device-resident packed matrix W[N][K] (N rows of K/256 wire blocks)."""
+
+    def __init__(self, fmt, N: int, K: int, packed):
+        import numpy as np
+        import torch
+        self.fmt, self.N, self.K = fmt_id(fmt), int(N), int(K)
+        self._keep = None
+        if isinstance(packed, torch.Tensor) and packed.is_cuda:
+            self._keep = packed  # borrowed device payload
+            h = lib().tfq_weight_wrap(self.fmt, N, K, packed.data_ptr(), packed.numel())
+        else:
+            arr = np.ascontiguousarray(packed.cpu().numpy() if isinstance(packed, torch.Tensor) else packed,
+                                       dtype=np.uint8)
+            h = lib().tfq_weight_upload(self.fmt, N, K, arr.ctypes.data, arr.size)
+        if not h:
+            raise TfqError(lib().tfq_last_error().decode())
+        self.handle = C.c_void_p(h)
+
+    def close(self):
+        if getattr(self, "handle", None):
+            lib().tfq_weight_free(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def decode(self):
+        import torch
+        out = torch.empty((self.N, self.K), dtype=torch.float32, device="cuda")
+        _check(lib().tfq_weight_decode(self.handle, out.data_ptr(), _stream()))
+        return out
+
+    def _mm(self, fn, x, out_dtype):
+        import torch
+        x = x.contiguous()
+        assert x.is_cuda and x.shape[-1] == self.K
+        B = x.numel() // self.K
+        y = torch.empty((B, self.N), dtype=out_dtype or torch.float32, device=x.device)
+        _check(fn(self.handle, x.data_ptr(), _dtype_code(x), B, y.data_ptr(), _dtype_code(y), _stream()))
+        return y
+
+    def gemv(self, x, out_dtype=None, out=None):
+        """y[B][N] = x[B][K] . W^T for 1 <= B <= 16 (decode)."""
+        if out is not None:
+            B = x.numel() // self.K
+            _check(lib().tfq_gemv(self.handle, x.data_ptr(), _dtype_code(x), B, out.data_ptr(),
+                                  _dtype_code(out), _stream()))
+            return out
+        return self._mm(lib().tfq_gemv, x, out_dtype)
+
+    def gemm(self, x, out_dtype=None):
+        """y[M][N] = x[M][K] . W^T for any M (prefill)."""
+        return self._mm(lib().tfq_gemm, x, out_dtype)

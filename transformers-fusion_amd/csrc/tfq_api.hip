@@ -1,0 +1,285 @@
+// C ABI of the backend (include/tfq.h): argument checking, the error channel,
+// the format registry mirror, handle management and host-pointer wrappers.
+// All compute goes to the launchers in tfq_codec.hip / tfq_gemv.hip /
+// tfq_gemm.hip; there is no CPU implementation behind any entry point.
+
+#include "tfq_internal.hpp"
+
+#include <cctype>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <vector>
+
+namespace tfq {
+
+namespace {
+thread_local std::string g_last_error;
+std::mutex g_init_mutex;
+bool g_device_ok[64] = {};
+}  // namespace
+
+int fail(int code, const std::string& msg) {
+    g_last_error = msg;
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    if (e == hipSuccess) return TFQ_OK;
+    return fail(TFQ_ERR_DEVICE, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+// The kernels are built for gfx950 only; any other device (or none) is an
+// error, never a reason to compute elsewhere.
+int ensure_device() {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(TFQ_ERR_DEVICE, std::string("no HIP device: ") + hipGetErrorString(e));
+    if (dev < 0 || dev >= 64) return fail(TFQ_ERR_DEVICE, "device ordinal out of range");
+    if (g_device_ok[dev]) return TFQ_OK;
+    std::lock_guard<std::mutex> lock(g_init_mutex);
+    if (g_device_ok[dev]) return TFQ_OK;
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDeviceProperties");
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(TFQ_ERR_DEVICE, std::string("device is ") + prop.gcnArchName + ", this library holds gfx950 code only");
+    g_device_ok[dev] = true;
+    return TFQ_OK;
+}
+
+namespace {
+
+struct NameRow {
+    const char* name;
+    int id;
+};
+// Canonical names (format_name, include/quant/types.h:168-196) of the ids this
+// backend handles, plus the appended literal formats.
+const NameRow kNames[] = {
+    {"Q_4", TFQ_Q_4}, {"Q_8", TFQ_Q_8}, {"Q_32", TFQ_Q_32},
+    {"Q_G_2", TFQ_Q_G_2}, {"Q_G_3", TFQ_Q_G_3}, {"Q_G_4", TFQ_Q_G_4}, {"Q_G_8", TFQ_Q_G_8},
+    {"Q_3_5", TFQ_Q_3_5}, {"Q_4_5", TFQ_Q_4_5}, {"Q_8_5", TFQ_Q_8_5},
+    {"Q_G_3_5", TFQ_Q_G_3_5}, {"Q_G_4_5", TFQ_Q_G_4_5}, {"Q_G_8_5", TFQ_Q_G_8_5},
+    {"B32S4", TFQ_B32S4}, {"B32S8", TFQ_B32S8}, {"SB256A3", TFQ_SB256A3}, {"SB256A2", TFQ_SB256A2},
+};
+
+std::string normalise(const char* s) {
+    std::string o;
+    for (; *s; ++s) {
+        if (*s == '_' || *s == '.') continue;
+        o.push_back((char)std::toupper((unsigned char)*s));
+    }
+    return o;
+}
+
+}  // namespace
+}  // namespace tfq
+
+using namespace tfq;
+
+extern "C" {
+
+const char* tfq_version(void) { return "tfq 0.1 (gfx950)"; }
+
+const char* tfq_last_error(void) { return g_last_error.c_str(); }
+
+int tfq_init(int device) {
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) return hip_fail(e, "hipSetDevice");
+    return ensure_device();
+}
+
+// The registry's name parser drops '_' and '.' and upper-cases before
+// comparing, so "Q_G_4", "QG4", "qg4" and "Q.G.4" all name one format.  A
+// registry name maps to the base wire id of its family ("Q4.5" is Q_G_4's
+// registry twin Q_4_5 only by layout; the registry itself resolves dotted
+// half-bpw spellings to the grouped single of that name).
+int tfq_format_id(const char* name) {
+    if (!name) return -1;
+    const std::string want = normalise(name);
+    for (const auto& r : kNames)
+        if (normalise(r.name) == want) return r.id;
+    return -1;
+}
+
+const char* tfq_format_name(uint8_t fmt) {
+    for (const auto& r : kNames)
+        if (r.id == fmt) return r.name;
+    return "unknown";
+}
+
+float tfq_format_bpw(uint8_t fmt) { return spec_of(fmt).bpw; }
+
+int tfq_format_supported(uint8_t fmt) { return spec_of(fmt).codec != Codec::None; }
+
+int tfq_block_bytes(uint8_t fmt, uint32_t n, size_t* out) {
+    if (!out) return fail(TFQ_ERR_ARG, "tfq_block_bytes: null out");
+    const Spec sp = spec_of(fmt);
+    if (sp.codec == Codec::None) return fail(TFQ_ERR_FORMAT, "tfq_block_bytes: wire id " + std::to_string(fmt) + " is not handled");
+    if (n != 256) return fail(TFQ_ERR_SHAPE, "tfq_block_bytes: only full 256-weight blocks are handled");
+    *out = (size_t)sp.block_bytes;
+    return TFQ_OK;
+}
+
+static int check_blocks(const char* who, uint8_t fmt, int64_t n, size_t* need) {
+    const Spec sp = spec_of(fmt);
+    if (sp.codec == Codec::None) return fail(TFQ_ERR_FORMAT, std::string(who) + ": wire id " + std::to_string(fmt) + " is not handled");
+    if (n <= 0 || n % 256) return fail(TFQ_ERR_SHAPE, std::string(who) + ": n must be a positive multiple of 256");
+    *need = (size_t)(n / 256) * (size_t)sp.block_bytes;
+    return TFQ_OK;
+}
+
+int tfq_encode_blocks(uint8_t fmt, const float* w, int64_t n, uint8_t* dst, size_t cap, tfq_stream_t stream) {
+    size_t need = 0;
+    if (!w || !dst) return fail(TFQ_ERR_ARG, "tfq_encode_blocks: null pointer");
+    if (int r = check_blocks("tfq_encode_blocks", fmt, n, &need)) return r;
+    if (cap < need) return fail(TFQ_ERR_SHAPE, "tfq_encode_blocks: destination too small");
+    if (int r = ensure_device()) return r;
+    return launch_encode(fmt, w, n / 256, dst, (hipStream_t)stream);
+}
+
+int tfq_decode_blocks(uint8_t fmt, const uint8_t* src, size_t bytes, int64_t n, float* out, tfq_stream_t stream) {
+    size_t need = 0;
+    if (!src || !out) return fail(TFQ_ERR_ARG, "tfq_decode_blocks: null pointer");
+    if (int r = check_blocks("tfq_decode_blocks", fmt, n, &need)) return r;
+    if (bytes < need) return fail(TFQ_ERR_SHAPE, "tfq_decode_blocks: payload shorter than n/256 blocks");
+    if (int r = ensure_device()) return r;
+    return launch_decode(fmt, src, n / 256, out, (hipStream_t)stream);
+}
+
+int tfq_encode_blocks_host(uint8_t fmt, const float* w, int64_t n, uint8_t* dst, size_t cap, uint32_t* per_block_bytes) {
+    size_t need = 0;
+    if (!w || !dst) return fail(TFQ_ERR_ARG, "tfq_encode_blocks_host: null pointer");
+    if (int r = check_blocks("tfq_encode_blocks_host", fmt, n, &need)) return r;
+    if (cap < need) return fail(TFQ_ERR_SHAPE, "tfq_encode_blocks_host: destination too small");
+    if (int r = ensure_device()) return r;
+    float* dw = nullptr;
+    uint8_t* dd = nullptr;
+    TFQ_HIP(hipMalloc(&dw, (size_t)n * 4));
+    hipError_t e = hipMalloc(&dd, need);
+    if (e != hipSuccess) { (void)hipFree(dw); return hip_fail(e, "hipMalloc"); }
+    int rc = hip_fail(hipMemcpy(dw, w, (size_t)n * 4, hipMemcpyHostToDevice), "hipMemcpy H2D");
+    if (!rc) rc = launch_encode(fmt, dw, n / 256, dd, nullptr);
+    if (!rc) rc = hip_fail(hipMemcpy(dst, dd, need, hipMemcpyDeviceToHost), "hipMemcpy D2H");
+    (void)hipFree(dw);
+    (void)hipFree(dd);
+    if (!rc && per_block_bytes)
+        for (int64_t b = 0; b < n / 256; ++b) per_block_bytes[b] = (uint32_t)spec_of(fmt).block_bytes;
+    return rc;
+}
+
+int tfq_decode_blocks_host(uint8_t fmt, const uint8_t* src, size_t bytes, int64_t n, float* out) {
+    size_t need = 0;
+    if (!src || !out) return fail(TFQ_ERR_ARG, "tfq_decode_blocks_host: null pointer");
+    if (int r = check_blocks("tfq_decode_blocks_host", fmt, n, &need)) return r;
+    if (bytes < need) return fail(TFQ_ERR_SHAPE, "tfq_decode_blocks_host: payload shorter than n/256 blocks");
+    if (int r = ensure_device()) return r;
+    uint8_t* ds = nullptr;
+    float* dout = nullptr;
+    TFQ_HIP(hipMalloc(&ds, need));
+    hipError_t e = hipMalloc(&dout, (size_t)n * 4);
+    if (e != hipSuccess) { (void)hipFree(ds); return hip_fail(e, "hipMalloc"); }
+    int rc = hip_fail(hipMemcpy(ds, src, need, hipMemcpyHostToDevice), "hipMemcpy H2D");
+    if (!rc) rc = launch_decode(fmt, ds, n / 256, dout, nullptr);
+    if (!rc) rc = hip_fail(hipMemcpy(out, dout, (size_t)n * 4, hipMemcpyDeviceToHost), "hipMemcpy D2H");
+    (void)hipFree(ds);
+    (void)hipFree(dout);
+    return rc;
+}
+
+static tfq_weight_t* make_weight(const char* who, uint8_t fmt, int64_t N, int64_t K, const uint8_t* packed,
+                                 size_t bytes, bool copy) {
+    const Spec sp = spec_of(fmt);
+    if (sp.codec == Codec::None) { fail(TFQ_ERR_FORMAT, std::string(who) + ": wire id " + std::to_string(fmt) + " is not handled"); return nullptr; }
+    if (!packed || N <= 0 || K <= 0) { fail(TFQ_ERR_ARG, std::string(who) + ": null payload or non-positive shape"); return nullptr; }
+    if (K % 256) { fail(TFQ_ERR_SHAPE, std::string(who) + ": K must be a multiple of 256"); return nullptr; }
+    const size_t need = (size_t)N * (size_t)(K / 256) * (size_t)sp.block_bytes;
+    if (bytes != need) { fail(TFQ_ERR_SHAPE, std::string(who) + ": payload is " + std::to_string(bytes) + " bytes, shape needs " + std::to_string(need)); return nullptr; }
+    if (ensure_device()) return nullptr;
+    tfq_weight_t* w = new (std::nothrow) tfq_weight_t{fmt, N, K, bytes, nullptr, copy};
+    if (!w) { fail(TFQ_ERR_NOMEM, std::string(who) + ": out of host memory"); return nullptr; }
+    if (copy) {
+        hipError_t e = hipMalloc(&w->dev, bytes);
+        if (e == hipSuccess) e = hipMemcpy(w->dev, packed, bytes, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            hip_fail(e, who);
+            if (w->dev) (void)hipFree(w->dev);
+            delete w;
+            return nullptr;
+        }
+    } else {
+        if ((uintptr_t)packed % 16) { fail(TFQ_ERR_ARG, std::string(who) + ": device payload must be 16-byte aligned"); delete w; return nullptr; }
+        w->dev = const_cast<uint8_t*>(packed);
+    }
+    return w;
+}
+
+tfq_weight_t* tfq_weight_upload(uint8_t fmt, int64_t N, int64_t K, const uint8_t* packed_host, size_t bytes) {
+    return make_weight("tfq_weight_upload", fmt, N, K, packed_host, bytes, true);
+}
+
+tfq_weight_t* tfq_weight_wrap(uint8_t fmt, int64_t N, int64_t K, const uint8_t* packed_dev, size_t bytes) {
+    return make_weight("tfq_weight_wrap", fmt, N, K, packed_dev, bytes, false);
+}
+
+void tfq_weight_free(tfq_weight_t* w) {
+    if (!w) return;
+    if (w->owns && w->dev) (void)hipFree(w->dev);
+    delete w;
+}
+
+int tfq_weight_info(const tfq_weight_t* w, uint8_t* fmt, int64_t* N, int64_t* K, size_t* bytes) {
+    if (!w) return fail(TFQ_ERR_ARG, "tfq_weight_info: null handle");
+    if (fmt) *fmt = w->fmt;
+    if (N) *N = w->N;
+    if (K) *K = w->K;
+    if (bytes) *bytes = w->bytes;
+    return TFQ_OK;
+}
+
+int tfq_weight_decode(const tfq_weight_t* w, float* out, tfq_stream_t stream) {
+    if (!w || !out) return fail(TFQ_ERR_ARG, "tfq_weight_decode: null pointer");
+    if (int r = ensure_device()) return r;
+    return launch_decode(w->fmt, w->dev, w->N * (w->K / 256), out, (hipStream_t)stream);
+}
+
+static int check_matmul(const char* who, const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, int y_dtype) {
+    if (!w || !x || !y) return fail(TFQ_ERR_ARG, std::string(who) + ": null pointer");
+    if (B <= 0) return fail(TFQ_ERR_ARG, std::string(who) + ": batch must be positive");
+    if ((x_dtype != TFQ_F32 && x_dtype != TFQ_BF16) || (y_dtype != TFQ_F32 && y_dtype != TFQ_BF16))
+        return fail(TFQ_ERR_ARG, std::string(who) + ": dtype must be TFQ_F32 or TFQ_BF16");
+    if ((uintptr_t)x % 16 || (uintptr_t)y % 4) return fail(TFQ_ERR_ARG, std::string(who) + ": x must be 16-byte aligned, y 4-byte aligned");
+    return ensure_device();
+}
+
+int tfq_gemv(const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, int y_dtype, tfq_stream_t stream) {
+    if (int r = check_matmul("tfq_gemv", w, x, x_dtype, B, y, y_dtype)) return r;
+    if (B > 16) return fail(TFQ_ERR_SHAPE, "tfq_gemv: batch above 16, use tfq_gemm");
+    return launch_gemv(w, x, x_dtype, B, y, y_dtype, (hipStream_t)stream);
+}
+
+int tfq_gemm(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, int y_dtype, tfq_stream_t stream) {
+    if (int r = check_matmul("tfq_gemm", w, x, x_dtype, M, y, y_dtype)) return r;
+    return launch_gemm(w, x, x_dtype, M, y, y_dtype, (hipStream_t)stream);
+}
+
+int tfq_matmul_host(const tfq_weight_t* w, const float* X, float* Y, int B) {
+    if (!w || !X || !Y) return fail(TFQ_ERR_ARG, "tfq_matmul_host: null pointer");
+    if (B <= 0) return fail(TFQ_ERR_ARG, "tfq_matmul_host: batch must be positive");
+    if (int r = ensure_device()) return r;
+    float *dx = nullptr, *dy = nullptr;
+    const size_t xb = (size_t)B * (size_t)w->K * 4, yb = (size_t)B * (size_t)w->N * 4;
+    TFQ_HIP(hipMalloc(&dx, xb));
+    hipError_t e = hipMalloc(&dy, yb);
+    if (e != hipSuccess) { (void)hipFree(dx); return hip_fail(e, "hipMalloc"); }
+    int rc = hip_fail(hipMemcpy(dx, X, xb, hipMemcpyHostToDevice), "hipMemcpy H2D");
+    if (!rc) rc = B <= 16 ? launch_gemv(w, dx, TFQ_F32, B, dy, TFQ_F32, nullptr)
+                          : launch_gemm(w, dx, TFQ_F32, B, dy, TFQ_F32, nullptr);
+    if (!rc) rc = hip_fail(hipMemcpy(Y, dy, yb, hipMemcpyDeviceToHost), "hipMemcpy D2H");
+    (void)hipFree(dx);
+    (void)hipFree(dy);
+    return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,159 @@
+// Shared declarations of the gfx950 backend: format table, error channel,
+// device helpers.  Internal to the library; the public surface is include/tfq.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <string>
+
+#include "../../include/tfq.h"
+
+namespace tfq {
+
+// ------------------------------------------------------------------ formats
+enum class Codec : int { None = 0, Raw32, Lattice, Affine, Grp8, Sym32 };
+
+// Layout parameters of one wire format.  The affine family is the reference's
+// parametric codec quant_affine(bits, w, n, gsz, scb, mb, claimed)
+// (src/codec/block_codec.cpp:1406-1521); Q_G_4, Q_G_3, Q_G_2 and the two
+// superblock formats differ only in these numbers.
+struct Spec {
+    Codec codec;
+    int bits;     // code width
+    int gsz;      // weights per group
+    int scb, mb;  // scale / min code widths (affine)
+    float bpw;    // wire bits per weight of a full 256-block
+    int block_bytes;  // payload bytes of a full 256-block
+};
+
+__host__ __device__ constexpr Spec spec_of(int fmt) {
+    switch (fmt) {
+        case TFQ_Q_32: return {Codec::Raw32, 32, 0, 0, 0, 32.0f, 1024};
+        case TFQ_Q_4: return {Codec::Lattice, 4, 0, 0, 0, 4.0f, 128};
+        case TFQ_Q_8: return {Codec::Lattice, 8, 0, 0, 0, 8.0f, 256};
+        case TFQ_Q_G_4: case TFQ_Q_4_5: case TFQ_Q_G_4_5: return {Codec::Affine, 4, 32, 6, 6, 4.5f, 144};
+        case TFQ_Q_G_3: case TFQ_Q_3_5: case TFQ_Q_G_3_5: return {Codec::Affine, 3, 32, 6, 6, 3.5f, 112};
+        case TFQ_Q_G_2: return {Codec::Affine, 2, 16, 4, 4, 2.625f, 84};
+        case TFQ_Q_G_8: case TFQ_Q_8_5: case TFQ_Q_G_8_5: return {Codec::Grp8, 8, 32, 0, 0, 8.5f, 272};
+        case TFQ_SB256A3: return {Codec::Affine, 3, 16, 6, 6, 3.875f, 124};
+        case TFQ_SB256A2: return {Codec::Affine, 2, 16, 6, 6, 2.875f, 92};
+        case TFQ_B32S4: return {Codec::Sym32, 4, 32, 0, 0, 4.5f, 144};
+        case TFQ_B32S8: return {Codec::Sym32, 8, 32, 0, 0, 8.5f, 272};
+        default: return {Codec::None, 0, 0, 0, 0, 0.0f, 0};
+    }
+}
+
+// Canonical id of a family of wire ids that share one payload layout
+// (Q_4_5 and Q_G_4_5 are byte-identical to Q_G_4, and so on).
+__host__ __device__ constexpr int canonical(int fmt) {
+    switch (fmt) {
+        case TFQ_Q_4_5: case TFQ_Q_G_4_5: return TFQ_Q_G_4;
+        case TFQ_Q_3_5: case TFQ_Q_G_3_5: return TFQ_Q_G_3;
+        case TFQ_Q_8_5: case TFQ_Q_G_8_5: return TFQ_Q_G_8;
+        default: return fmt;
+    }
+}
+
+// --------------------------------------------------------------- error channel
+int fail(int code, const std::string& msg);  // records msg for tfq_last_error, returns code
+int hip_fail(hipError_t e, const char* what);
+#define TFQ_HIP(call)                                         \
+    do {                                                      \
+        hipError_t e_ = (call);                               \
+        if (e_ != hipSuccess) return ::tfq::hip_fail(e_, #call); \
+    } while (0)
+
+int ensure_device();  // TFQ_OK once a gfx950 device is current and tables are loaded
+
+// -------------------------------------------------------------------- handle
+}  // namespace tfq
+
+struct tfq_weight {
+    uint8_t fmt;
+    int64_t N, K;
+    size_t bytes;
+    uint8_t* dev;
+    bool owns;
+};
+
+namespace tfq {
+
+// ------------------------------------------------------------- kernel launchers
+int launch_decode(int fmt, const uint8_t* src, int64_t nblocks, float* out, hipStream_t s);
+int launch_encode(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStream_t s);
+int launch_gemv(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype,
+                hipStream_t s);
+int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
+                hipStream_t s);
+
+// ---------------------------------------------------------------- device helpers
+// binary16 -> binary32 by integer arithmetic: exact for every input including
+// subnormals, independent of the device's denormal mode
+// (f16_to_f32, src/codec/block_codec.cpp:76-99).
+__device__ __forceinline__ float half_bits_to_float(uint32_t h) {
+    const uint32_t sign = (h & 0x8000u) << 16;
+    const uint32_t ex = (h >> 10) & 0x1Fu;
+    const uint32_t man = h & 0x3FFu;
+    uint32_t u;
+    if (ex == 0) {
+        if (man == 0) {
+            u = sign;
+        } else {
+            const int lz = __clz(man) - 21;  // shifts needed to bring bit 10 up
+            const uint32_t m = (man << lz) & 0x3FFu;
+            u = sign | ((uint32_t)(113 - lz) << 23) | (m << 13);
+        }
+    } else if (ex == 31) {
+        u = sign | 0x7F800000u | (man << 13);
+    } else {
+        u = sign | ((ex + 112u) << 23) | (man << 13);
+    }
+    return __uint_as_float(u);
+}
+
+// binary16 -> binary32 with the hardware conversion (v_cvt_f32_f16); used by the
+// matmul kernels, where a flushed subnormal scale would be far below tolerance.
+__device__ __forceinline__ float half_fast(uint32_t h) {
+    return (float)__builtin_bit_cast(_Float16, (unsigned short)h);
+}
+
+// binary32 -> binary16, round to nearest even, with the reference's two quirks:
+// NaN becomes infinity and magnitudes below 2^-24 flush to signed zero
+// (f32_to_f16, src/codec/block_codec.cpp:41-74).
+__device__ __forceinline__ uint32_t float_to_half_bits(float v) {
+    const uint32_t u = __float_as_uint(v);
+    const uint32_t sign = (u >> 16) & 0x8000u;
+    const int e = (int)((u >> 23) & 0xFFu) - 127;
+    const uint32_t man = u & 0x7FFFFFu;
+    if (e > 15) return sign | 0x7C00u;
+    if (e >= -14) {
+        uint32_t h = ((uint32_t)(e + 15) << 10) | (man >> 13);
+        const uint32_t rem = man & 0x1FFFu;
+        if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) ++h;
+        return sign | h;
+    }
+    if (e < -24) return sign;
+    const uint32_t full = man | 0x800000u;
+    const int shift = -e - 1;
+    uint32_t m = full >> shift;
+    const uint32_t rem = full & ((1u << shift) - 1u);
+    const uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (m & 1u))) ++m;
+    return sign | m;
+}
+
+// `count` (<= 25) bits starting at bit `pos` of an LSB-first stream of `size`
+// bytes; bits past the end read as zero (FastBitReader::get,
+// src/codec/block_codec.cpp:147-172).
+__device__ __forceinline__ uint32_t stream_bits(const uint8_t* p, uint32_t size, uint32_t pos, int count) {
+    const uint32_t byte = pos >> 3;
+    uint32_t w = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (byte + i < size) w |= (uint32_t)p[byte + i] << (8 * i);
+    return (w >> (pos & 7)) & ((1u << count) - 1u);
+}
+
+}  // namespace tfq
