@@ -92,9 +92,10 @@ int tfq_decode_blocks_host(uint8_t fmt, const uint8_t* src, size_t bytes, int64_
 
 /* ---- packed weight matrices ---------------------------------------------------
  * W is N rows of K/256 consecutive wire blocks, the layout Qwen35Engine::gemm
- * walks (src/adapters/tools/qwen35_engine.cpp:58,82-86).  upload copies a host
- * payload to the device; wrap borrows a device payload (the caller keeps it
- * alive).  Both return NULL on failure. */
+ * walks (src/adapters/tools/qwen35_engine.cpp:58,82-86).  upload takes a host
+ * payload, wrap a payload that is already in device memory (16-byte aligned).
+ * Both copy it into the handle's own device layout and synchronise, so the
+ * caller may release its buffer when the call returns.  NULL on failure. */
 tfq_weight_t* tfq_weight_upload(uint8_t fmt, int64_t N, int64_t K, const uint8_t* packed_host,
                                 size_t bytes);
 tfq_weight_t* tfq_weight_wrap(uint8_t fmt, int64_t N, int64_t K, const uint8_t* packed_dev,
@@ -113,6 +114,12 @@ int tfq_gemv(const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, 
              tfq_stream_t stream);
 int tfq_gemm(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
              tfq_stream_t stream);
+/* Up to four matrices that share K, format and the activation rows in ONE launch:
+ * ys[i][b][n] = sum_k x[b][k] * ws[i][n][k].  This is the q/k/v step and the
+ * gate/up step of the reference engine, which issue one gemm per matrix on the
+ * same input (src/adapters/tools/qwen35_engine.cpp:662-672 for gate/up). */
+int tfq_gemv_multi(const tfq_weight_t* const* ws, int count, const void* x, int x_dtype, int B,
+                   void* const* ys, int y_dtype, tfq_stream_t stream);
 /* host-pointer form of tfq_gemv/tfq_gemm with fp32 x and y: the exact call
  * shape of Qwen35Engine::gemm(t, X, Y, B). */
 int tfq_matmul_host(const tfq_weight_t* w, const float* X, float* Y, int B);

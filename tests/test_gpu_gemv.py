@@ -114,3 +114,25 @@ def test_gemv_rejects_bad_arguments(O, tfq, gpu):
     with pytest.raises(tfq.TfqError):
         W.gemv(x)
     W.close()
+
+
+@pytest.mark.parametrize("fmt", GEMV_FORMATS)
+@pytest.mark.parametrize("B", [1, 4])
+def test_gemv_multi_matches_single_launches(O, tfq, gpu, fmt, B):
+    """q/k/v style: three matrices of different heights on one input, one launch."""
+    import torch
+    K = 2048
+    shapes = [72, 24, 33]
+    x = torch.from_numpy(O.bf16_round(O.rng_normal(5, B * K, 1.0).reshape(B, K))).to(gpu).bfloat16()
+    Ws, singles = [], []
+    for i, N in enumerate(shapes):
+        pay = O.encode_tensor(fmt, O.rng_normal(60 + i, N * K, 0.02))
+        W = tfq.Weight(fmt, N, K, pay)
+        Ws.append(W)
+        singles.append(W.gemv(x))
+    outs = [torch.zeros(B, N, device=gpu) for N in shapes]
+    tfq.gemv_multi(Ws, x, outs)
+    for got, want in zip(outs, singles):
+        assert torch.equal(got, want)
+    for W in Ws:
+        W.close()

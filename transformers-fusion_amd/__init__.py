@@ -55,6 +55,7 @@ def _load():
         "tfq_weight_decode": (i32, [vp, vp, vp]),
         "tfq_gemv": (i32, [vp, vp, i32, i32, vp, i32, vp]),
         "tfq_gemm": (i32, [vp, vp, i32, i32, vp, i32, vp]),
+        "tfq_gemv_multi": (i32, [vp, i32, vp, i32, i32, vp, i32, vp]),
         "tfq_matmul_host": (i32, [vp, vp, vp, i32]),
     }
     for name, (res, args) in sig.items():
@@ -133,9 +134,8 @@ class Weight:
         import numpy as np
         import torch
         self.fmt, self.N, self.K = fmt_id(fmt), int(N), int(K)
-        self._keep = None
         if isinstance(packed, torch.Tensor) and packed.is_cuda:
-            self._keep = packed  # borrowed device payload
+            # device payload: copied into the handle's own layout, the caller may drop its tensor
             h = lib().tfq_weight_wrap(self.fmt, N, K, packed.data_ptr(), packed.numel())
         else:
             arr = np.ascontiguousarray(packed.cpu().numpy() if isinstance(packed, torch.Tensor) else packed,
@@ -183,3 +183,13 @@ class Weight:
     def gemm(self, x, out_dtype=None):
         """y[M][N] = x[M][K] . W^T for any M (prefill)."""
         return self._mm(lib().tfq_gemm, x, out_dtype)
+
+
+def gemv_multi(weights, x, outs):
+    """One launch for up to four matrices that share K, format and x (q/k/v, gate/up)."""
+    n = len(weights)
+    hs = (C.c_void_p * n)(*[w.handle for w in weights])
+    ys = (C.c_void_p * n)(*[o.data_ptr() for o in outs])
+    B = x.numel() // weights[0].K
+    _check(lib().tfq_gemv_multi(hs, n, x.data_ptr(), _dtype_code(x), B, ys, _dtype_code(outs[0]), _stream()))
+    return outs

@@ -22,7 +22,7 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
-]
+] + os.environ.get("TFQ_EXTRA_HIPCC_FLAGS", "").split()
 
 
 def hipcc() -> str:

@@ -188,29 +188,48 @@ int tfq_decode_blocks_host(uint8_t fmt, const uint8_t* src, size_t bytes, int64_
     return rc;
 }
 
+// The 4-bit matmul formats are kept in the Tiled16 layout; everything else stays in wire order.
+static bool wants_tiled16(uint8_t fmt) {
+    const int c = canonical(fmt);
+    return c == TFQ_Q_G_4 || c == TFQ_B32S4;
+}
+
 static tfq_weight_t* make_weight(const char* who, uint8_t fmt, int64_t N, int64_t K, const uint8_t* packed,
-                                 size_t bytes, bool copy) {
+                                 size_t bytes, bool from_host) {
     const Spec sp = spec_of(fmt);
     if (sp.codec == Codec::None) { fail(TFQ_ERR_FORMAT, std::string(who) + ": wire id " + std::to_string(fmt) + " is not handled"); return nullptr; }
     if (!packed || N <= 0 || K <= 0) { fail(TFQ_ERR_ARG, std::string(who) + ": null payload or non-positive shape"); return nullptr; }
     if (K % 256) { fail(TFQ_ERR_SHAPE, std::string(who) + ": K must be a multiple of 256"); return nullptr; }
     const size_t need = (size_t)N * (size_t)(K / 256) * (size_t)sp.block_bytes;
     if (bytes != need) { fail(TFQ_ERR_SHAPE, std::string(who) + ": payload is " + std::to_string(bytes) + " bytes, shape needs " + std::to_string(need)); return nullptr; }
+    if (!from_host && (uintptr_t)packed % 16) { fail(TFQ_ERR_ARG, std::string(who) + ": device payload must be 16-byte aligned"); return nullptr; }
     if (ensure_device()) return nullptr;
-    tfq_weight_t* w = new (std::nothrow) tfq_weight_t{fmt, N, K, bytes, nullptr, copy};
+    const bool tiled = wants_tiled16(fmt);
+    tfq_weight_t* w = new (std::nothrow) tfq_weight_t{fmt, N, K, bytes, nullptr, 0, tiled ? TFQ_LAYOUT_TILED16 : TFQ_LAYOUT_WIRE, true};
     if (!w) { fail(TFQ_ERR_NOMEM, std::string(who) + ": out of host memory"); return nullptr; }
-    if (copy) {
-        hipError_t e = hipMalloc(&w->dev, bytes);
-        if (e == hipSuccess) e = hipMemcpy(w->dev, packed, bytes, hipMemcpyHostToDevice);
-        if (e != hipSuccess) {
-            hip_fail(e, who);
-            if (w->dev) (void)hipFree(w->dev);
-            delete w;
-            return nullptr;
+    w->dev_bytes = tiled ? (size_t)((N + 15) / 16) * (size_t)(K / 256) * 2304 : bytes;
+    uint8_t* staged = nullptr;  // wire payload on the device, when it has to be permuted
+    hipError_t e = hipMalloc(&w->dev, w->dev_bytes);
+    if (e == hipSuccess && from_host) {
+        if (tiled) {
+            e = hipMalloc(&staged, bytes);
+            if (e == hipSuccess) e = hipMemcpy(staged, packed, bytes, hipMemcpyHostToDevice);
+        } else {
+            e = hipMemcpy(w->dev, packed, bytes, hipMemcpyHostToDevice);
         }
-    } else {
-        if ((uintptr_t)packed % 16) { fail(TFQ_ERR_ARG, std::string(who) + ": device payload must be 16-byte aligned"); delete w; return nullptr; }
-        w->dev = const_cast<uint8_t*>(packed);
+    }
+    int rc = hip_fail(e, who);
+    if (!rc) {
+        const uint8_t* wire = from_host ? staged : packed;
+        if (tiled) rc = launch_tile16(wire, w->dev, N, K, nullptr);
+        else if (!from_host) rc = hip_fail(hipMemcpy(w->dev, packed, bytes, hipMemcpyDeviceToDevice), who);
+        if (!rc) rc = hip_fail(hipDeviceSynchronize(), who);
+    }
+    if (staged) (void)hipFree(staged);
+    if (rc) {
+        if (w->dev) (void)hipFree(w->dev);
+        delete w;
+        return nullptr;
     }
     return w;
 }
@@ -241,7 +260,15 @@ int tfq_weight_info(const tfq_weight_t* w, uint8_t* fmt, int64_t* N, int64_t* K,
 int tfq_weight_decode(const tfq_weight_t* w, float* out, tfq_stream_t stream) {
     if (!w || !out) return fail(TFQ_ERR_ARG, "tfq_weight_decode: null pointer");
     if (int r = ensure_device()) return r;
-    return launch_decode(w->fmt, w->dev, w->N * (w->K / 256), out, (hipStream_t)stream);
+    if (w->layout == TFQ_LAYOUT_WIRE) return launch_decode(w->fmt, w->dev, w->N * (w->K / 256), out, (hipStream_t)stream);
+    // Tiled16: restore wire order in a temporary buffer, then decode it.
+    uint8_t* wire = nullptr;
+    TFQ_HIP(hipMalloc(&wire, w->bytes));
+    int rc = launch_untile16(w->dev, wire, w->N, w->K, (hipStream_t)stream);
+    if (!rc) rc = launch_decode(w->fmt, wire, w->N * (w->K / 256), out, (hipStream_t)stream);
+    if (!rc) rc = hip_fail(hipStreamSynchronize((hipStream_t)stream), "tfq_weight_decode");
+    (void)hipFree(wire);
+    return rc;
 }
 
 static int check_matmul(const char* who, const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, int y_dtype) {
@@ -257,6 +284,15 @@ int tfq_gemv(const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, 
     if (int r = check_matmul("tfq_gemv", w, x, x_dtype, B, y, y_dtype)) return r;
     if (B > 16) return fail(TFQ_ERR_SHAPE, "tfq_gemv: batch above 16, use tfq_gemm");
     return launch_gemv(w, x, x_dtype, B, y, y_dtype, (hipStream_t)stream);
+}
+
+int tfq_gemv_multi(const tfq_weight_t* const* ws, int count, const void* x, int x_dtype, int B, void* const* ys,
+                   int y_dtype, tfq_stream_t stream) {
+    if (!ws || !ys || count < 1 || count > 4) return fail(TFQ_ERR_ARG, "tfq_gemv_multi: 1 to 4 matrices per launch");
+    for (int i = 0; i < count; ++i)
+        if (int r = check_matmul("tfq_gemv_multi", ws[i], x, x_dtype, B, ys[i], y_dtype)) return r;
+    if (B > 16) return fail(TFQ_ERR_SHAPE, "tfq_gemv_multi: batch above 16");
+    return launch_gemv_multi(ws, count, x, x_dtype, B, ys, y_dtype, (hipStream_t)stream);
 }
 
 int tfq_gemm(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, int y_dtype, tfq_stream_t stream) {

@@ -137,6 +137,32 @@ __global__ __launch_bounds__(256) void encode_raw32_kernel(const float* __restri
     reinterpret_cast<float*>(dst)[e] = w[e];
 }
 
+// Wire <-> Tiled16 permutation of 144-byte blocks, one lane per 16-byte piece.
+// piece p of a unit: p < 64 code slot of k-step 0, p < 128 of k-step 1, else header of row p - 128.
+template <bool TO_TILED>
+__global__ __launch_bounds__(256) void tile16_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                     int64_t N, int nblocks, int64_t npieces) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= npieces) return;
+    const int64_t unit = i / 144;
+    const int p = (int)(i - unit * 144);
+    const int64_t tile = unit / nblocks;
+    const int blk = (int)(unit - tile * nblocks);
+    int n, off16;  // row inside the tile, 16-byte piece inside the wire block
+    if (p < 128) {
+        const int l = p & 63;
+        n = l & 15;
+        off16 = (l >> 4) + 4 * (p >> 6);
+    } else {
+        n = p - 128;
+        off16 = 8;
+    }
+    const int64_t row = tile * 16 + n;
+    const int64_t wire = (row * nblocks + blk) * 9 + off16;
+    if (TO_TILED) dst[i] = row < N ? src[wire] : uint4{0, 0, 0, 0};
+    else if (row < N) dst[wire] = src[i];
+}
+
 template <int FMT>
 int run_decode(const uint8_t* src, int64_t nblocks, float* out, hipStream_t s) {
     hipLaunchKernelGGL(decode_kernel<FMT>, dim3((unsigned)nblocks), dim3(256), 0, s, src, out);
@@ -162,6 +188,29 @@ int launch_decode(int fmt, const uint8_t* src, int64_t nblocks, float* out, hipS
         case TFQ_B32S8: return run_decode<TFQ_B32S8>(src, nblocks, out, s);
         default: return fail(TFQ_ERR_FORMAT, "decode: wire id " + std::to_string(fmt) + " is not handled");
     }
+}
+
+static int run_tile16(bool to_tiled, const uint8_t* src, uint8_t* dst, int64_t N, int64_t K, hipStream_t s) {
+    const int nblocks = (int)(K / 256);
+    const int64_t tiles = (N + 15) / 16;
+    const int64_t npieces = tiles * nblocks * 144;
+    const int64_t grid = (npieces + 255) / 256;
+    if (grid > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "matrix too large for one layout pass");
+    if (to_tiled)
+        hipLaunchKernelGGL(tile16_kernel<true>, dim3((unsigned)grid), dim3(256), 0, s, reinterpret_cast<const uint4*>(src),
+                           reinterpret_cast<uint4*>(dst), N, nblocks, npieces);
+    else
+        hipLaunchKernelGGL(tile16_kernel<false>, dim3((unsigned)grid), dim3(256), 0, s, reinterpret_cast<const uint4*>(src),
+                           reinterpret_cast<uint4*>(dst), N, nblocks, npieces);
+    return hip_fail(hipGetLastError(), "layout launch");
+}
+
+int launch_tile16(const uint8_t* wire, uint8_t* tiled, int64_t N, int64_t K, hipStream_t s) {
+    return run_tile16(true, wire, tiled, N, K, s);
+}
+
+int launch_untile16(const uint8_t* tiled, uint8_t* wire, int64_t N, int64_t K, hipStream_t s) {
+    return run_tile16(false, tiled, wire, N, K, s);
 }
 
 int launch_encode(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStream_t s) {

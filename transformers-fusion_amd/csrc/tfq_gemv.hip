@@ -2,33 +2,53 @@
 //   y[b][n] = sum_k x[b][k] * W[n][k],  W packed in 4-bit block formats.
 // Replaces Qwen35Engine::gemm at B <= 16 (src/adapters/tools/qwen35_engine.cpp:54-101).
 //
-// Data layout.  W is used in its wire layout, untouched: a row is K/256
-// consecutive 144-byte blocks, [128 B of nibbles, element 2j low / 2j+1 high]
-// followed by a 16-byte header.  Block size and both parts are multiples of
-// 16 B, so a lane fetches one 32-weight group (16 B of nibbles) and its block's
-// header with two 128-bit loads; a wavefront covers 8 consecutive blocks
-// (1152 contiguous bytes) per step and every fetched cache line is used once.
+// Data layout.  W is held in the Tiled16 layout (tfq_internal.hpp): rows in tiles
+// of 16, and for every tile and 256-wide block column one 2304-byte unit
+//   [ 64 x 16 B codes of k-step 0 ][ 64 x 16 B codes of k-step 1 ][ 16 x 16 B headers ].
+// It is the wire payload permuted at upload (same bytes), arranged so that a
+// wavefront reads a unit as one contiguous run with 128-bit loads: lane l takes
+// code slots l of both k-steps and the header of row l % 16.
 //
-// Arithmetic.  The activation rows are staged once per workgroup in LDS as
-// bf16, permuted so that one 128-bit LDS read returns the four bf16 pairs
-// (x0,x4) (x1,x5) (x2,x6) (x3,x7) that match the nibble pairs obtained from a
-// code dword by (q >> 4t) & 0x000F000F.  OR-ing 0x4300 into each half turns a
-// nibble n into the bf16 value 128+n without a conversion, and v_dot2_f32_bf16
-// accumulates pairs of products in fp32.  Per group
-//   sum_k w_k x_k = a * (D - 128 X) + c * X,   D = sum (128+n_k) x_k,  X = sum x_k
-// with (a, c) = (d*sc/15, -dm*mc) for the affine formats and (d, -8 d) for the
-// symmetric one, so the per-group scale and offset cost two FMAs per lane.
-// fp32 activations are split into a bf16 high and low part (two LDS rows whose
-// results are added), which keeps 16 significant bits of x.
-// Lanes are reduced with wavefront shuffles at the end of each weight row.
+// Arithmetic.  The multiply-accumulate runs on the matrix cores
+// (v_mfma_f32_16x16x32_bf16) with the WEIGHTS as the B operand (16 weight rows
+// = 16 columns) and the ACTIVATIONS as the A operand.  A lane (n, c) of a
+// wavefront (n = lane % 16, c = lane / 16) holds the 16 bytes of group c of
+// row n for the current 128-wide k-step: 4 dwords of 8 nibbles.  OR-ing 0x4300
+// into a masked nibble pair turns nibbles into the bf16 values 128+n without a
+// conversion, so one dword becomes the lane's 8-element B fragment in 7 VALU
+// operations.  The A operand is block diagonal: row 4s+c (s = activation row,
+// c = group) holds x only in k-slot c, so the 32-deep MFMA does not mix the four
+// groups and D[4s+c][n] is the dot product of activation row s with ONE group of
+// weight row n.  Four chained MFMAs (one per dword) finish the 32 weights of a
+// group.  The accumulator starts at -128 X (X = the group's activation sum; -136 X
+// for the symmetric format, whose codes carry an offset of 8), so it ends as the
+// dot product D with the integer codes, and the per-group scale and offset are
+// applied in fp32: a * D + c * X with (a, c) = (d*sc/15, -dm*mc) for the affine
+// formats and (d, 0) for the symmetric one.  Up to four activation rows ride in one
+// pass for free; fp32 activations are split into a bf16 high and low part
+// (two rows whose results are added), which keeps 16 significant bits of x.
+//
+// Work split.  A workgroup of NW <= 16 wavefronts owns T consecutive tiles and
+// wavefront w takes the block columns w, w+NW, ... of every tile.  Each
+// wavefront stages only the activations of ITS block columns, in a private LDS
+// region (bf16 in the nibble-pair order (x0,x4)(x1,x5)(x2,x6)(x3,x7), with the
+// group sums X beside them), so no wavefront waits for another before it starts.
+// It holds the A fragments of the current block column in registers while it
+// walks the tiles, keeps four unit fetches in flight, and adds its partial sums
+// into a private LDS cell per (tile, lane); after the only barrier the NW
+// partials of each output are added in a fixed order (deterministic results).
 
 #include "tfq_internal.hpp"
+
+#include <cstdlib>
 
 namespace tfq {
 
 namespace {
 
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a),
@@ -50,218 +70,388 @@ __device__ __forceinline__ uint4 pair_permute(uint4 v) {
     return p;
 }
 
-// LDS slot (in uint4 units) of the 8 activations starting at k = 8*i: chunks of
-// 2048 weights; inside a chunk lane l owns weights 32l..32l+31 and its four
-// 8-weight quads are stored 64 slots apart, so that the 64 lanes of a wavefront
-// read 64 consecutive slots (no bank conflicts).
-__device__ __forceinline__ int x_slot(int i) {
-    const int c = i >> 8, r = i & 255;
-    return (c << 8) + ((r & 3) << 6) + (r >> 2);
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false);
+    return v + __int_as_float(moved);
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
-    return v;
-}
+// Up to four matrices that share K and the activation rows are served by one
+// launch (q/k/v, or gate/up): their tiles are concatenated into one tile space.
+struct GemvArgs {
+    const uint8_t* W[4];  // Tiled16 buffers
+    void* y[4];
+    int tile_end[4];  // cumulative tile counts, INT_MAX in unused entries
+    int nrows[4];
+    int ntiles;
+    int nmat;
+    int K;
+    int y_bf16;
+    int x_f32;
+    int nslot;         // bf16 activation rows held in LDS: B, or 2B for fp32 input (<= 4)
+    int tiles_per_wg;  // T
+    int cols_base, cols_rem;  // block columns per wavefront: cols_base + (wave < cols_rem)
+};
 
-// Per-group coefficients (a, c) from a block header, for the lane's group g.
+// Matrix lookup without indexed kernel-argument reads (an indexed read is a
+// dependent scalar load from the argument segment, about a microsecond each):
+// everything is fetched once, unconditionally, and selected with compares.
+// Unused tile_end entries hold INT_MAX.
+struct MatrixTable {
+    const uint8_t* W0; const uint8_t* W1; const uint8_t* W2; const uint8_t* W3;
+    int e0, e1, e2;
+    __device__ __forceinline__ explicit MatrixTable(const GemvArgs& a)
+        : W0(a.W[0]), W1(a.W[1]), W2(a.W[2]), W3(a.W[3]), e0(a.tile_end[0]), e1(a.tile_end[1]), e2(a.tile_end[2]) {}
+    __device__ __forceinline__ int index(int tile) const { return (tile >= e0) + (tile >= e1) + (tile >= e2); }
+    __device__ __forceinline__ int first_tile(int m) const { return m == 0 ? 0 : m == 1 ? e0 : m == 2 ? e1 : e2; }
+    __device__ __forceinline__ const uint8_t* base(int m) const { return m == 0 ? W0 : m == 1 ? W1 : m == 2 ? W2 : W3; }
+};
+
+// Bias that the MFMA accumulator starts from, so that it ends as the dot
+// product with the true code values: the bf16 fragments hold 128+n, and the
+// symmetric format's codes are offset by 8.
 template <int FMT>
-__device__ __forceinline__ void group_coeffs(const uint8_t* blk, int g, float& a, float& c) {
+__device__ __forceinline__ f32x4_t accumulator_bias(float4 X) {
+    constexpr float k = FMT == TFQ_B32S4 ? -136.0f : -128.0f;
+    return f32x4_t{k * X.x, k * X.y, k * X.z, k * X.w};
+}
+
+// sum over the four groups r of one k-step: D[r] is the group's dot product with
+// the integer codes (bias already removed), X[r] the group's activation sum
+template <int FMT>
+__device__ __forceinline__ float apply_groups(uint4 h, int khalf, f32x4_t D, float4 X) {
+    float res = 0.0f;
     if constexpr (FMT == TFQ_Q_G_4) {
         // header: 8 x 6-bit sc | 8 x 6-bit (mc+32) | binary16 d | binary16 dm
-        const uint4 h = *reinterpret_cast<const uint4*>(blk + 128);
+        const float xv[4] = {X.x, X.y, X.z, X.w};
         const uint64_t scs = (uint64_t)h.x | ((uint64_t)(h.y & 0xFFFFu) << 32);
         const uint64_t mcs = (uint64_t)(h.y >> 16) | ((uint64_t)h.z << 16);
-        const float sc = (float)(uint32_t)((scs >> (6 * g)) & 63u);
-        const float mc = (float)((int)((mcs >> (6 * g)) & 63u) - 32);
-        const float d = half_fast(h.w & 0xFFFFu);
+        const uint32_t sc24 = (uint32_t)(scs >> (24 * khalf));
+        const uint32_t mc24 = (uint32_t)(mcs >> (24 * khalf));
+        const float d15 = half_fast(h.w & 0xFFFFu) * (1.0f / 15.0f);
         const float dm = half_fast(h.w >> 16);
-        a = d * sc * (1.0f / 15.0f);
-        c = -(dm * mc);
-    } else {  // TFQ_B32S4: header = 8 binary16 scales
-        const unsigned short hs = *reinterpret_cast<const unsigned short*>(blk + 128 + 2 * g);
-        const float d = half_fast(hs);
-        a = d;
-        c = -8.0f * d;
-    }
-}
-
-template <int FMT, int B, bool XF32, bool YBF16>
-__global__ __launch_bounds__(256) void gemv4_kernel(const uint8_t* __restrict__ W,
-                                                    const void* __restrict__ xin,
-                                                    void* __restrict__ yout, int N, int K) {
-    constexpr int ROWS = XF32 ? 2 * B : B;  // LDS activation rows
-    constexpr int R = 2;                    // weight rows in flight per wavefront
-    extern __shared__ uint4 xs[];
-    const int nchunks = (K + 2047) >> 11;
-    const int row_slots = nchunks << 8;
-    const int k8 = K >> 3;
-
-    // ---- stage activations
-    for (int i = threadIdx.x; i < k8; i += 256) {
-        const int slot = x_slot(i);
 #pragma unroll
-        for (int b = 0; b < B; ++b) {
-            if constexpr (XF32) {
-                const float4* xf = reinterpret_cast<const float4*>(xin) + ((size_t)b * K >> 2) + 2 * i;
-                const float4 lo4 = xf[0], hi4 = xf[1];
-                const float f[8] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
-                uint32_t hb[8], lb[8];
+        for (int r = 0; r < 4; ++r) {
+            const float a = d15 * (float)((sc24 >> (6 * r)) & 63u);
+            const float off = dm * (float)(32 - (int)((mc24 >> (6 * r)) & 63u));  // -dm * mc
+            res = __builtin_fmaf(a, D[r], res);
+            res = __builtin_fmaf(off, xv[r], res);
+        }
+    } else {
+        // header: eight binary16 scales, four per k-step
+        const uint32_t hw[2] = {khalf ? h.z : h.x, khalf ? h.w : h.y};
 #pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    hb[t] = bf16_rne(f[t]);
-                    lb[t] = bf16_rne(f[t] - __uint_as_float(hb[t] << 16));
-                }
-                uint4 vh, vl;
-                vh.x = hb[0] | (hb[1] << 16); vh.y = hb[2] | (hb[3] << 16);
-                vh.z = hb[4] | (hb[5] << 16); vh.w = hb[6] | (hb[7] << 16);
-                vl.x = lb[0] | (lb[1] << 16); vl.y = lb[2] | (lb[3] << 16);
-                vl.z = lb[4] | (lb[5] << 16); vl.w = lb[6] | (lb[7] << 16);
-                xs[(2 * b) * row_slots + slot] = pair_permute(vh);
-                xs[(2 * b + 1) * row_slots + slot] = pair_permute(vl);
-            } else {
-                const uint4 v = reinterpret_cast<const uint4*>(xin)[((size_t)b * K >> 3) + i];
-                xs[b * row_slots + slot] = pair_permute(v);
-            }
+        for (int r = 0; r < 4; ++r) {
+            const float d = half_fast((hw[r >> 1] >> (16 * (r & 1))) & 0xFFFFu);
+            res = __builtin_fmaf(d, D[r], res);
         }
     }
-    __syncthreads();
+    return res;
+}
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int g = lane & 7;
-    const int ngroups = K >> 5;
-    const size_t row_bytes = (size_t)(K >> 8) * 144;
-    const uint32_t M = 0x000F000Fu, C = 0x43004300u, ONES = 0x3F803F80u;
+#ifdef TFQ_TRACE
+__device__ unsigned long long g_trace[1024 * 16 * 8];
+#define TRACE(slot) do { if (lane == 0) g_trace[(blockIdx.x * 16 + wave) * 8 + (slot)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define TRACE(slot) do {} while (0)
+#endif
 
-    for (int row0 = (blockIdx.x * 4 + wave) * R; row0 < N; row0 += gridDim.x * 4 * R) {
-        float acc[R][ROWS];
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int t = 0; t < ROWS; ++t) acc[r][t] = 0.0f;
+template <int FMT>
+__global__ __launch_bounds__(1024) void gemv4_kernel(GemvArgs args, const void* __restrict__ xin) {
+    constexpr int WD = 4;  // unit fetches in flight per wavefront
+    extern __shared__ uint4 smem[];
+    // every kernel argument is read here, in one batch of scalar loads
+    const MatrixTable mt(args);
+    const int K = args.K, nslot = args.nslot, T = args.tiles_per_wg, ntiles = args.ntiles;
+    const int cols_base = args.cols_base, cols_rem = args.cols_rem;
+    const bool x_f32 = args.x_f32 != 0, y_bf16 = args.y_bf16 != 0;
+    const int nr0 = args.nrows[0], nr1 = args.nrows[1], nr2 = args.nrows[2], nr3 = args.nrows[3];
+    void* const y0 = args.y[0]; void* const y1 = args.y[1]; void* const y2 = args.y[2]; void* const y3 = args.y[3];
+    asm volatile("" ::"s"(K), "s"(nslot), "s"(T), "s"(ntiles), "s"(cols_base), "s"(cols_rem), "s"(nr0), "s"(nr1),
+                 "s"(nr2), "s"(nr3), "s"(y0), "s"(y1), "s"(y2), "s"(y3), "s"(xin), "s"(mt.W0), "s"(mt.W1), "s"(mt.W2),
+                 "s"(mt.W3), "s"(mt.e0), "s"(mt.e1), "s"(mt.e2));
 
-        for (int ch = 0; ch < nchunks; ++ch) {
-            const int gi = (ch << 6) + lane;
-            if (gi >= ngroups) continue;
-            const size_t off = (size_t)(gi >> 3) * 144;
-            uint4 q[R];
-            float a[R], c[R];
+    const int nblocks = K >> 8;
+    const int NW = blockDim.x >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, q = lane >> 4;
+    const int tile0 = blockIdx.x * T;
+    const int tiles_here = min(T, ntiles - tile0);
+    const int ncols = cols_base + (wave < cols_rem ? 1 : 0);  // block columns wave, wave + NW, ...
+    const int ncols_max = cols_base + (cols_rem ? 1 : 0);
+    const int nitems = ncols * tiles_here;  // block-column major, tiles inside
+    TRACE(0);
+
+    // LDS: per wavefront and block column, A entries [nslot][2 k-steps][4 groups][4] (uint4) and
+    // group sums [4 slots][2][4] (float); then one zero A entry set, then the partial sums [T][NW][64].
+    const int a_per_col = nslot * 32;                   // uint4 entries
+    const int col_stride = a_per_col + 8;               // + 32 floats of group sums
+    uint4* my = smem + (size_t)wave * ncols_max * col_stride;
+    uint4* zero4 = smem + (size_t)NW * ncols_max * col_stride;
+    float* part = reinterpret_cast<float*>(zero4 + 4);
+
+    // ---- this wavefront's activation slices first (tiny, and needed before any arithmetic)
+    // lane l < 32 of a pass owns the 8-element quad l of one (column, slot); a pass covers two slots
+    const int quad = lane & 31, sl_in_pass = lane >> 5;
+    auto x_load = [&](int ci, int s, uint4& lo, uint4& hi) {
+        const size_t k0 = (size_t)(wave + NW * ci) * 256 + (size_t)quad * 8;
+        if (x_f32) {
+            const uint4* xf = reinterpret_cast<const uint4*>(xin) + (((size_t)(s >> 1) * K + k0) >> 2);
+            lo = xf[0];
+            hi = xf[1];
+        } else {
+            lo = reinterpret_cast<const uint4*>(xin)[((size_t)s * K + k0) >> 3];
+        }
+    };
+    uint4 xlo = {0, 0, 0, 0}, xhi = {0, 0, 0, 0};
+    if (ncols > 0 && sl_in_pass < nslot) x_load(0, sl_in_pass, xlo, xhi);
+    TRACE(1);
+
+    // ---- stage this wavefront's activations: bf16 in nibble-pair order, group sums beside them
+    const uint32_t ONES = 0x3F803F80u;
+    if (tid < 4) zero4[tid] = uint4{0, 0, 0, 0};
+    for (int t = 0; t < tiles_here; ++t) part[(t * NW + wave) * 64 + lane] = 0.0f;  // this wavefront's own cells
+    for (int ci = 0; ci < ncols; ++ci) {
+        uint4* col = my + (size_t)ci * col_stride;
+        float* colX = reinterpret_cast<float*>(col + a_per_col);
+        for (int s0 = 0; s0 < 4; s0 += 2) {
+            const int s = s0 + sl_in_pass;
+            float sum = 0.0f;
+            if (s < nslot) {
+                if (ci != 0 || s0 != 0) x_load(ci, s, xlo, xhi);
+                uint4 v = xlo;
+                if (x_f32) {
+                    const float f[8] = {__uint_as_float(xlo.x), __uint_as_float(xlo.y), __uint_as_float(xlo.z),
+                                        __uint_as_float(xlo.w), __uint_as_float(xhi.x), __uint_as_float(xhi.y),
+                                        __uint_as_float(xhi.z), __uint_as_float(xhi.w)};
+                    uint32_t e[8];
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int row = min(row0 + r, N - 1);
-                const uint8_t* blk = W + (size_t)row * row_bytes + off;
-                q[r] = *reinterpret_cast<const uint4*>(blk + 16 * g);
-                group_coeffs<FMT>(blk, g, a[r], c[r]);
-                c[r] = __builtin_fmaf(-128.0f, a[r], c[r]);
-            }
-#pragma unroll
-            for (int t = 0; t < ROWS; ++t) {
-                uint4 xq[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) xq[j] = xs[t * row_slots + (ch << 8) + (j << 6) + lane];
-                float X = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    X = dot2(ONES, xq[j].x, X); X = dot2(ONES, xq[j].y, X);
-                    X = dot2(ONES, xq[j].z, X); X = dot2(ONES, xq[j].w, X);
+                    for (int t = 0; t < 8; ++t) {
+                        const uint32_t hb = bf16_rne(f[t]);
+                        e[t] = (s & 1) ? bf16_rne(f[t] - __uint_as_float(hb << 16)) : hb;
+                    }
+                    v.x = e[0] | (e[1] << 16); v.y = e[2] | (e[3] << 16);
+                    v.z = e[4] | (e[5] << 16); v.w = e[6] | (e[7] << 16);
                 }
+                const uint4 p = pair_permute(v);
+                col[s * 32 + quad] = p;  // quad = (k-step, group, dword) in that order
+                sum = dot2(ONES, p.x, 0.0f);
+                sum = dot2(ONES, p.y, sum);
+                sum = dot2(ONES, p.z, sum);
+                sum = dot2(ONES, p.w, sum);
+            }
+            sum = dpp_add<0xB1>(sum);  // the four dwords of a group sit in adjacent lanes
+            sum = dpp_add<0x4E>(sum);
+            if ((quad & 3) == 0) colX[s * 8 + (quad >> 2)] = sum;  // zero for unused slots
+        }
+    }
+    // ---- unit fetch cursor.  The weight stream starts only now: a vector load that hits
+    // in L2 still returns behind every older miss of the compute unit, so activations
+    // requested after the flood would arrive microseconds late
+    int f_ci = 0, f_t = 0;
+    auto fetch = [&](uint4& c0, uint4& c1, uint4& hd) {
+        const int tile = tile0 + f_t;
+        const int m = mt.index(tile);
+        const int ltile = tile - mt.first_tile(m);
+        const uint8_t* u = mt.base(m) + ((size_t)ltile * nblocks + (size_t)(wave + NW * f_ci)) * 2304;
+        c0 = *reinterpret_cast<const uint4*>(u + 16 * lane);
+        c1 = *reinterpret_cast<const uint4*>(u + 1024 + 16 * lane);
+        hd = *reinterpret_cast<const uint4*>(u + 2048 + 16 * n);
+        if (++f_t == tiles_here) { f_t = 0; ++f_ci; }
+    };
+    uint4 c0[WD], c1[WD], hd[WD];
 #pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    const uint32_t qq[4] = {q[r].x, q[r].y, q[r].z, q[r].w};
-                    float D = 0.0f;
+    for (int u = 0; u < WD; ++u)
+        if (u < nitems) fetch(c0[u], c1[u], hd[u]);
+
+    TRACE(2);
+    TRACE(3);
+
+    // ---- per-lane operand addressing
+    // A operand: lane (i = n, kc = q) is non-zero only on the diagonal c == kc of activation row s
+    const int s_a = n >> 2, c_a = n & 3;
+    const bool a_live = (c_a == q) && (s_a < nslot);
+
+    const uint32_t M = 0x000F000Fu;
+    uint32_t C = 0x43004300u;
+    asm volatile("" : "+v"(C));  // keep the bias in a VGPR so (v & M) | C is one v_and_or_b32
+    uint4 av[2][4];
+    float4 xv[2];
+    f32x4_t bias[2];
+    int c_ci = 0, c_t = 0;
+    for (int it0 = 0; it0 < nitems; it0 += WD) {
+#pragma unroll
+        for (int u = 0; u < WD; ++u) {
+            if (it0 + u < nitems) {
+                if (c_t == 0) {  // new block column: its two k-steps' A fragments and group sums
+                    const uint4* col = my + (size_t)c_ci * col_stride;
+                    const float* colX = reinterpret_cast<const float*>(col + a_per_col);
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const uint4* src = a_live ? col + s_a * 32 + h * 16 + q * 4 : zero4;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) av[h][j] = src[j];
+                        xv[h] = *reinterpret_cast<const float4*>(colX + q * 8 + h * 4);
+                        bias[h] = accumulator_bias<FMT>(xv[h]);
+                    }
+                }
+                float res = 0.0f;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const uint4 cw = h ? c1[u] : c0[u];
+                    const uint32_t qq[4] = {cw.x, cw.y, cw.z, cw.w};
+                    f32x4_t Dv = bias[h];
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const uint32_t v = qq[j];
-                        D = dot2((v & M) | C, xq[j].x, D);
-                        D = dot2(((v >> 4) & M) | C, xq[j].y, D);
-                        D = dot2(((v >> 8) & M) | C, xq[j].z, D);
-                        D = dot2(((v >> 12) & M) | C, xq[j].w, D);
+                        const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
+                        Dv = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[h][j]),
+                                                                     __builtin_bit_cast(bf16x8_t, wv), Dv, 0, 0, 0);
                     }
-                    acc[r][t] = __builtin_fmaf(a[r], D, acc[r][t]);
-                    acc[r][t] = __builtin_fmaf(c[r], X, acc[r][t]);
+                    res += apply_groups<FMT>(hd[u], h, Dv, xv[h]);
                 }
-            }
-        }
-
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int row = row0 + r;
-#pragma unroll
-            for (int b = 0; b < B; ++b) {
-                float v;
-                if constexpr (XF32) v = wave_sum(acc[r][2 * b] + acc[r][2 * b + 1]);
-                else v = wave_sum(acc[r][b]);
-                if (lane == 0 && row < N) {
-                    if constexpr (YBF16) reinterpret_cast<unsigned short*>(yout)[(size_t)b * N + row] = (unsigned short)bf16_rne(v);
-                    else reinterpret_cast<float*>(yout)[(size_t)b * N + row] = v;
-                }
+                float* cell = part + (c_t * NW + wave) * 64 + lane;
+                *cell += res;
+                if (it0 + u == 0) TRACE(4);
+                if (++c_t == tiles_here) { c_t = 0; ++c_ci; }
+                if (it0 + u + WD < nitems) fetch(c0[u], c1[u], hd[u]);
             }
         }
     }
-}
+    TRACE(5);
+    __syncthreads();
+    TRACE(6);
 
-template <int FMT, int B, bool XF32, bool YBF16>
-int run_gemv4(const tfq_weight* w, const void* x, void* y, hipStream_t s) {
-    const int N = (int)w->N, K = (int)w->K;
-    constexpr int ROWS = XF32 ? 2 * B : B;
-    const int nchunks = (K + 2047) >> 11;
-    const size_t lds = (size_t)ROWS * nchunks * 256 * 16;
-    if (lds > 160 * 1024) return fail(TFQ_ERR_SHAPE, "gemv: activation rows do not fit LDS");
-    auto kern = gemv4_kernel<FMT, B, XF32, YBF16>;
-    if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
+    // ---- add the wavefronts' partials and store: 16 lanes per output, lane w reads wavefront w's
+    // cell(s), then a fixed-order DPP tree inside the 16-lane row
+    const int rows_per_out = x_f32 ? 2 : 1;  // fp32 input: high and low part live in adjacent activation rows
+    const int nb = nslot / rows_per_out;
+    const int nout = tiles_here * nb * 16;
+    for (int o = tid >> 4; o < ((nout + 63) & ~63); o += blockDim.x >> 4) {
+        const int w = tid & 15;
+        const int t = o / (nb * 16), rem = o - t * (nb * 16);
+        const int b = rem >> 4, nn = rem & 15;
+        float v = 0.0f;
+        if (o < nout && w < NW)
+            for (int h = 0; h < rows_per_out; ++h) v += part[(t * NW + w) * 64 + (b * rows_per_out + h) * 16 + nn];
+        v = dpp_add<0xB1>(v);
+        v = dpp_add<0x4E>(v);
+        v = dpp_add<0x141>(v);  // row_half_mirror
+        v = dpp_add<0x140>(v);  // row_mirror
+        if (o < nout && w == 0) {
+            const int tile = tile0 + t;
+            const int m = mt.index(tile);
+            const int row = (tile - mt.first_tile(m)) * 16 + nn;
+            const int nr = m == 0 ? nr0 : m == 1 ? nr1 : m == 2 ? nr2 : nr3;
+            void* yp = m == 0 ? y0 : m == 1 ? y1 : m == 2 ? y2 : y3;
+            if (row < nr) {
+                const size_t off = (size_t)b * (size_t)nr + (size_t)row;
+                if (y_bf16) reinterpret_cast<unsigned short*>(yp)[off] = (unsigned short)bf16_rne(v);
+                else reinterpret_cast<float*>(yp)[off] = v;
+            }
+        }
     }
-    const int tiles = (N + 7) / 8;
-    const int grid = tiles < 2048 ? tiles : 2048;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, s, w->dev, x, y, N, K);
-    return hip_fail(hipGetLastError(), "gemv launch");
-}
-
-template <int FMT, int B>
-int pick_io(const tfq_weight* w, const void* x, int xd, void* y, int yd, hipStream_t s) {
-    if (xd == TFQ_F32) return yd == TFQ_BF16 ? run_gemv4<FMT, B, true, true>(w, x, y, s)
-                                             : run_gemv4<FMT, B, true, false>(w, x, y, s);
-    return yd == TFQ_BF16 ? run_gemv4<FMT, B, false, true>(w, x, y, s)
-                          : run_gemv4<FMT, B, false, false>(w, x, y, s);
+    TRACE(7);
 }
 
 template <int FMT>
-int gemv4_batched(const tfq_weight* w, const void* x, int xd, int B, void* y, int yd, hipStream_t s) {
-    // Activation rows are processed in slices of at most 4 (2 for fp32 input at
-    // large K) so that a slice fits LDS.
-    const size_t xe = xd == TFQ_F32 ? 4 : 2, ye = yd == TFQ_F32 ? 4 : 2;
-    const int nchunks = (int)((w->K + 2047) >> 11);
-    int step = 4;
-    while (step > 1 && (size_t)step * (xd == TFQ_F32 ? 2 : 1) * nchunks * 4096 > 128 * 1024) step >>= 1;
-    for (int b0 = 0; b0 < B;) {
-        int nb = B - b0 < step ? B - b0 : step;
-        if (nb == 3) nb = 2;
-        const void* xb = (const uint8_t*)x + (size_t)b0 * w->K * xe;
-        void* yb = (uint8_t*)y + (size_t)b0 * w->N * ye;
-        int rc;
-        switch (nb) {
-            case 1: rc = pick_io<FMT, 1>(w, xb, xd, yb, yd, s); break;
-            case 2: rc = pick_io<FMT, 2>(w, xb, xd, yb, yd, s); break;
-            default: rc = pick_io<FMT, 4>(w, xb, xd, yb, yd, s); break;
+int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
+    const int ntiles = a.ntiles;
+    const int nblocks = a.K >> 8;
+    static const int num_cu = [] { const char* e = getenv("TFQ_GEMV_WGS"); return e ? atoi(e) : 256; }();
+    // wavefronts per workgroup: the count in 8..16 that splits the block columns most evenly
+    int NW = nblocks < 16 ? nblocks : 16;
+    if (nblocks > 16) {
+        int best_waste = 1 << 30;
+        for (int w = 16; w >= 8; --w) {
+            const int waste = (nblocks + w - 1) / w * w - nblocks;
+            if (waste < best_waste) { best_waste = waste; NW = w; }
         }
-        if (rc) return rc;
-        b0 += nb;
+    }
+    a.cols_base = nblocks / NW;
+    a.cols_rem = nblocks % NW;
+    const int ncols_max = a.cols_base + (a.cols_rem ? 1 : 0);
+    const size_t x_bytes = ((size_t)NW * ncols_max * (a.nslot * 32 + 8) + 4) * 16;
+    int T = (ntiles + num_cu - 1) / num_cu;
+    while (T > 1 && x_bytes + (size_t)T * NW * 256 > 160 * 1024) --T;
+    const size_t lds = x_bytes + (size_t)T * NW * 256;
+    if (lds > 160 * 1024) return fail(TFQ_ERR_SHAPE, "gemv: K too large for the LDS activation stage");
+    a.tiles_per_wg = T;
+    auto kern = gemv4_kernel<FMT>;
+    // Raise the dynamic-LDS limit once per kernel (not per launch: the call is
+    // not allowed while a stream is being captured into a graph).
+    static bool lds_limit_raised = false;
+    if (!lds_limit_raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
+        lds_limit_raised = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((ntiles + T - 1) / T), dim3(64 * NW), lds, s, a, x);
+    return hip_fail(hipGetLastError(), "gemv launch");
+}
+
+template <int FMT>
+int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t s) {
+    // One launch carries four bf16 activation rows (two fp32 rows).
+    const size_t xe = xd == TFQ_F32 ? 4 : 2, ye = yd == TFQ_F32 ? 4 : 2;
+    const int step = xd == TFQ_F32 ? 2 : 4;
+    a.y_bf16 = yd == TFQ_BF16;
+    a.x_f32 = xd == TFQ_F32;
+    for (int b0 = 0; b0 < B; b0 += step) {
+        const int nb = B - b0 < step ? B - b0 : step;
+        GemvArgs ab = a;
+        ab.nslot = a.x_f32 ? 2 * nb : nb;
+        for (int m = 0; m < a.nmat; ++m) ab.y[m] = (uint8_t*)a.y[m] + (size_t)b0 * (size_t)a.nrows[m] * ye;
+        const void* xb = (const uint8_t*)x + (size_t)b0 * a.K * xe;
+        if (int rc = run_gemv4<FMT>(ab, xb, s)) return rc;
     }
     return TFQ_OK;
 }
 
 }  // namespace
 
-int launch_gemv(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype, hipStream_t s) {
-    switch (canonical(w->fmt)) {
-        case TFQ_Q_G_4: return gemv4_batched<TFQ_Q_G_4>(w, x, x_dtype, B, y, y_dtype, s);
-        case TFQ_B32S4: return gemv4_batched<TFQ_B32S4>(w, x, x_dtype, B, y, y_dtype, s);
-        default:
-            return fail(TFQ_ERR_FORMAT, std::string("gemv: no kernel for format ") + tfq_format_name(w->fmt));
+int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
+                      void* const* ys, int y_dtype, hipStream_t s) {
+    GemvArgs a{};
+    int64_t tiles = 0;
+    for (int m = 0; m < nmat; ++m) {
+        if (canonical(ws[m]->fmt) != canonical(ws[0]->fmt) || ws[m]->K != ws[0]->K)
+            return fail(TFQ_ERR_SHAPE, "gemv: matrices of one launch must share format and K");
+        if (ws[m]->layout != TFQ_LAYOUT_TILED16)
+            return fail(TFQ_ERR_FORMAT, std::string("gemv: no kernel for format ") + tfq_format_name(ws[m]->fmt));
+        tiles += (ws[m]->N + 15) / 16;
+        if (tiles > 0x7FFFFFF || ws[m]->N > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "gemv: too many rows");
+        a.W[m] = ws[m]->dev;
+        a.y[m] = ys[m];
+        a.tile_end[m] = (int)tiles;
+        a.nrows[m] = (int)ws[m]->N;
     }
+    for (int m = nmat; m < 4; ++m) {
+        a.W[m] = a.W[0];
+        a.y[m] = a.y[0];
+        a.tile_end[m] = 0x7FFFFFFF;
+    }
+    a.ntiles = (int)tiles;
+    a.nmat = nmat;
+    a.K = (int)ws[0]->K;
+    switch (canonical(ws[0]->fmt)) {
+        case TFQ_Q_G_4: return gemv4_batched<TFQ_Q_G_4>(a, x, x_dtype, B, y_dtype, s);
+        case TFQ_B32S4: return gemv4_batched<TFQ_B32S4>(a, x, x_dtype, B, y_dtype, s);
+        default:
+            return fail(TFQ_ERR_FORMAT, std::string("gemv: no kernel for format ") + tfq_format_name(ws[0]->fmt));
+    }
+}
+
+#ifdef TFQ_TRACE
+extern "C" int tfq_debug_trace(unsigned long long* out) {
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_trace), sizeof(g_trace));
+}
+#endif
+
+int launch_gemv(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype, hipStream_t s) {
+    return launch_gemv_multi(&w, 1, x, x_dtype, B, &y, y_dtype, s);
 }
 
 int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype, hipStream_t s) {

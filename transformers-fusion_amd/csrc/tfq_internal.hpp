@@ -70,11 +70,26 @@ int ensure_device();  // TFQ_OK once a gfx950 device is current and tables are l
 // -------------------------------------------------------------------- handle
 }  // namespace tfq
 
+// Device layouts of a packed matrix.
+//   Wire:    the payload as the codec writes it, N rows of K/256 consecutive blocks.
+//   Tiled16: for the 4-bit matmul formats (144-byte blocks).  Rows are grouped in
+//            tiles of 16 (the last tile is zero padded); the 16 blocks that a tile
+//            holds at one block column form a 2304-byte unit
+//              [ 64 x 16 B codes of k-step 0 ][ 64 x 16 B codes of k-step 1 ][ 16 x 16 B headers ]
+//            where code slot l = n + 16 q holds group q (k-step 0) or q + 4
+//            (k-step 1) of row n, and header slot n is row n's 16-byte block
+//            header.  Units are ordered tile-major.  Same bytes as the wire
+//            layout (apart from the padding rows), permuted so that one
+//            wavefront reads one unit as a contiguous run.
+enum : int { TFQ_LAYOUT_WIRE = 0, TFQ_LAYOUT_TILED16 = 1 };
+
 struct tfq_weight {
     uint8_t fmt;
     int64_t N, K;
-    size_t bytes;
-    uint8_t* dev;
+    size_t bytes;      // wire payload bytes
+    uint8_t* dev;      // device buffer in `layout`
+    size_t dev_bytes;
+    int layout;
     bool owns;
 };
 
@@ -82,9 +97,13 @@ namespace tfq {
 
 // ------------------------------------------------------------- kernel launchers
 int launch_decode(int fmt, const uint8_t* src, int64_t nblocks, float* out, hipStream_t s);
+int launch_tile16(const uint8_t* wire, uint8_t* tiled, int64_t N, int64_t K, hipStream_t s);
+int launch_untile16(const uint8_t* tiled, uint8_t* wire, int64_t N, int64_t K, hipStream_t s);
 int launch_encode(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStream_t s);
 int launch_gemv(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype,
                 hipStream_t s);
+int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
+                      void* const* ys, int y_dtype, hipStream_t s);
 int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
                 hipStream_t s);
 
