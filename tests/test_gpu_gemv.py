@@ -8,6 +8,7 @@ pytestmark = pytest.mark.gpu
 
 TOL_F32, TOL_BF16 = 1e-3, 1e-2
 GEMV_FORMATS = ["Q_G_4", "B32S4"]
+OTHER_FORMATS = ["Q_G_8", "B32S8", "Q_G_3", "Q_G_2", "SB256A3", "SB256A2", "Q_4", "Q_8", "Q_32", "Q_4_5", "Q_G_8_5"]
 
 
 def rel_err(y, ref):
@@ -136,3 +137,43 @@ def test_gemv_multi_matches_single_launches(O, tfq, gpu, fmt, B):
         assert torch.equal(got, want)
     for W in Ws:
         W.close()
+
+
+@pytest.mark.parametrize("fmt", OTHER_FORMATS)
+@pytest.mark.parametrize("N,K,B,xdt", [(48, 512, 1, "bf16"), (33, 1024, 3, "bf16"), (20, 2304, 8, "f32"), (16, 4096, 16, "bf16")])
+def test_gemv_other_formats(O, tfq, gpu, fmt, N, K, B, xdt):
+    """8-bit, 3-bit, 2-bit, plain lattice and raw blocks: every registered format the
+    codec handles also runs through the matmul entry point."""
+    import torch
+    print(f"gemv {fmt} N={N} K={K} B={B} {xdt}", flush=True)
+    dist = O.rng_laplace(44, N * K, 0.015) if fmt.startswith("SB256") or fmt in ("Q_G_3", "Q_G_2") else O.rng_normal(42, N * K, 0.02)
+    x = O.rng_normal(43, B * K, 1.0).reshape(B, K)
+    pay = O.encode_tensor(fmt, dist)
+    W = tfq.Weight(fmt, N, K, pay)
+    if xdt == "bf16":
+        x = O.bf16_round(x)
+        y = W.gemv(torch.from_numpy(x).to(gpu).bfloat16()).cpu().numpy()
+        tol = TOL_BF16
+    else:
+        y = W.gemv(torch.from_numpy(x).to(gpu)).cpu().numpy()
+        tol = TOL_F32
+    ref = O.matmul(fmt, pay, N, K, x)
+    assert rel_err(y, ref) <= min(tol, 1e-4)   # exact decode, fp32 products: only summation order differs
+    assert np.array_equal(W.decode().cpu().numpy().reshape(-1).view(np.uint32),
+                          O.decode_tensor(fmt, pay, N * K).view(np.uint32))
+    W.close()
+
+
+@pytest.mark.parametrize("fmt,bits", [("SB256A3", 3), ("SB256A2", 2), ("Q_G_3", 3), ("Q_G_2", 2)])
+def test_config4_lowbit_superblock_shapes(O, tfq, gpu, fmt, bits):
+    """Laplace(0, 0.015) weights, 14336-wide rows (a slice of the 14336x4096 matrix), batch 1 and 8."""
+    import torch
+    N, K = 256, 4096
+    w = O.rng_laplace(44, N * K, 0.015)
+    pay = O.encode_tensor(fmt, w)
+    W = tfq.Weight(fmt, N, K, pay)
+    for B in (1, 8):
+        x = O.bf16_round(O.rng_normal(43, B * K, 1.0).reshape(B, K))
+        y = W.gemv(torch.from_numpy(x).to(gpu).bfloat16()).cpu().numpy()
+        assert rel_err(y, O.matmul(fmt, pay, N, K, x)) <= 1e-4
+    W.close()

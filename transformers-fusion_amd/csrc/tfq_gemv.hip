@@ -414,6 +414,11 @@ int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t 
 
 int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
                       void* const* ys, int y_dtype, hipStream_t s) {
+    if (ws[0]->layout == TFQ_LAYOUT_WIRE) {  // formats without a tiled kernel: one launch per matrix
+        for (int m = 0; m < nmat; ++m)
+            if (int rc = launch_gemv_generic(ws[m], x, x_dtype, B, ys[m], y_dtype, s)) return rc;
+        return TFQ_OK;
+    }
     GemvArgs a{};
     int64_t tiles = 0;
     for (int m = 0; m < nmat; ++m) {

@@ -1,0 +1,130 @@
+// Dequant-fused GEMV for the formats that have no specialised kernel yet
+// (8-bit, 3-bit, 2-bit, plain lattice and raw fp32 blocks), on the wire layout:
+//   y[b][n] = sum_k x[b][k] * W[n][k]
+// Replaces Qwen35Engine::gemm (src/adapters/tools/qwen35_engine.cpp:54-101) for
+// those formats.  One wavefront owns a weight row; lane l decodes weights
+// 4l..4l+3 of every 256-weight block with the codec's own per-weight decode
+// (tfq_decode.hpp, the exact reference arithmetic) and multiplies them into up
+// to four activation rows in fp32.  The 64 lane sums are reduced with DPP adds.
+// Decoding costs a few tens of VALU operations per weight here; this kernel is
+// about coverage and exactness, the 4-bit formats have the fast path.
+
+#include "tfq_decode.hpp"
+
+namespace tfq {
+
+namespace {
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, false);
+    return v + __int_as_float(moved);
+}
+// total ends up in lane 63
+__device__ __forceinline__ float wave_sum_lane63(float v) {
+    v = dpp_add<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x141, 0xF>(v);  // row_half_mirror
+    v = dpp_add<0x140, 0xF>(v);  // row_mirror
+    v = dpp_add<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
+    v = dpp_add<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+__device__ __forceinline__ uint32_t bf16_rne(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+
+template <int FMT, int BT, bool XF32>
+__global__ __launch_bounds__(256) void gemv_generic_kernel(const uint8_t* __restrict__ W,
+                                                           const void* __restrict__ xin,
+                                                           void* __restrict__ yout, int N, int K, int y_bf16) {
+    constexpr int BB = spec_of(FMT).block_bytes;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nblk = K >> 8;
+    for (int row = blockIdx.x * 4 + wave; row < N; row += gridDim.x * 4) {
+        float acc[BT];
+#pragma unroll
+        for (int b = 0; b < BT; ++b) acc[b] = 0.0f;
+        const uint8_t* prow = W + (size_t)row * (size_t)nblk * BB;
+        for (int blk = 0; blk < nblk; ++blk) {
+            const uint8_t* p = prow + (size_t)blk * BB;
+            float w[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) w[t] = decode_weight<FMT>(p, 4 * lane + t);
+            const size_t k0 = (size_t)blk * 256 + 4 * lane;
+#pragma unroll
+            for (int b = 0; b < BT; ++b) {
+                float xv[4];
+                if constexpr (XF32) {
+                    const float4 v = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(xin) + (size_t)b * K + k0);
+                    xv[0] = v.x; xv[1] = v.y; xv[2] = v.z; xv[3] = v.w;
+                } else {
+                    const uint2 v = *reinterpret_cast<const uint2*>(reinterpret_cast<const unsigned short*>(xin) + (size_t)b * K + k0);
+                    xv[0] = __uint_as_float(v.x << 16); xv[1] = __uint_as_float(v.x & 0xFFFF0000u);
+                    xv[2] = __uint_as_float(v.y << 16); xv[3] = __uint_as_float(v.y & 0xFFFF0000u);
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[b] = __builtin_fmaf(w[t], xv[t], acc[b]);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            const float v = wave_sum_lane63(acc[b]);
+            if (lane == 63) {
+                if (y_bf16) reinterpret_cast<unsigned short*>(yout)[(size_t)b * N + row] = (unsigned short)bf16_rne(v);
+                else reinterpret_cast<float*>(yout)[(size_t)b * N + row] = v;
+            }
+        }
+    }
+}
+
+template <int FMT, int BT>
+int run(const tfq_weight* w, const void* x, int xd, void* y, int yd, hipStream_t s) {
+    const int N = (int)w->N, K = (int)w->K;
+    const int grid = (N + 3) / 4 < 4096 ? (N + 3) / 4 : 4096;
+    if (xd == TFQ_F32)
+        hipLaunchKernelGGL((gemv_generic_kernel<FMT, BT, true>), dim3(grid), dim3(256), 0, s, w->dev, x, y, N, K, yd == TFQ_BF16);
+    else
+        hipLaunchKernelGGL((gemv_generic_kernel<FMT, BT, false>), dim3(grid), dim3(256), 0, s, w->dev, x, y, N, K, yd == TFQ_BF16);
+    return hip_fail(hipGetLastError(), "gemv launch");
+}
+
+template <int FMT>
+int batched(const tfq_weight* w, const void* x, int xd, int B, void* y, int yd, hipStream_t s) {
+    const size_t xe = xd == TFQ_F32 ? 4 : 2, ye = yd == TFQ_F32 ? 4 : 2;
+    for (int b0 = 0; b0 < B;) {
+        const int left = B - b0;
+        const int nb = left >= 4 ? 4 : left >= 2 ? 2 : 1;
+        const void* xb = (const uint8_t*)x + (size_t)b0 * w->K * xe;
+        void* yb = (uint8_t*)y + (size_t)b0 * w->N * ye;
+        const int rc = nb == 4 ? run<FMT, 4>(w, xb, xd, yb, yd, s) : nb == 2 ? run<FMT, 2>(w, xb, xd, yb, yd, s)
+                                                                            : run<FMT, 1>(w, xb, xd, yb, yd, s);
+        if (rc) return rc;
+        b0 += nb;
+    }
+    return TFQ_OK;
+}
+
+}  // namespace
+
+int launch_gemv_generic(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype, hipStream_t s) {
+    if (w->layout != TFQ_LAYOUT_WIRE) return fail(TFQ_ERR_FORMAT, "gemv: generic kernel expects the wire layout");
+    if (w->N > 0x7FFFFFFF || w->K > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "gemv: shape too large");
+    switch (canonical(w->fmt)) {
+        case TFQ_Q_32: return batched<TFQ_Q_32>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_4: return batched<TFQ_Q_4>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_8: return batched<TFQ_Q_8>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_G_2: return batched<TFQ_Q_G_2>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_G_3: return batched<TFQ_Q_G_3>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_G_8: return batched<TFQ_Q_G_8>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_SB256A3: return batched<TFQ_SB256A3>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_SB256A2: return batched<TFQ_SB256A2>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_B32S8: return batched<TFQ_B32S8>(w, x, x_dtype, B, y, y_dtype, s);
+        default:
+            return fail(TFQ_ERR_FORMAT, std::string("gemv: no kernel for format ") + tfq_format_name(w->fmt));
+    }
+}
+
+}  // namespace tfq

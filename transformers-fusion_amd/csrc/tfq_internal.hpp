@@ -104,6 +104,8 @@ int launch_gemv(const tfq_weight* w, const void* x, int x_dtype, int B, void* y,
                 hipStream_t s);
 int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
                       void* const* ys, int y_dtype, hipStream_t s);
+int launch_gemv_generic(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype,
+                        hipStream_t s);
 int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
                 hipStream_t s);
 
