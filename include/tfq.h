@@ -124,6 +124,30 @@ int tfq_gemv_multi(const tfq_weight_t* const* ws, int count, const void* x, int 
  * shape of Qwen35Engine::gemm(t, X, Y, B). */
 int tfq_matmul_host(const tfq_weight_t* w, const float* X, float* Y, int B);
 
+/* ---- MoE expert path ------------------------------------------------------------
+ * tfq_moe_route: router softmax + top-k on the device, softmax_with_topk
+ * (src/model/moe_core.cpp:98-149): probs [T][E], idx [T][k] (descending
+ * probability, lowest expert id first on ties), weights = the selected
+ * probabilities, not renormalised.  All pointers are device pointers.
+ *
+ * tfq_moe_ffn: the inference branch of moe_dispatch_batched
+ * (src/model/moe_core.cpp:289-343) with ExpertFFN::forward (:78-92) over
+ * block-quantized experts: gate/up are E matrices F x D, down E matrices D x F;
+ * out[t] = sum over the experts e of token t, ascending e, of
+ * w(t,e) * down_e( silu(gate_e x_t) * (up_e x_t) ).  topk_idx [T][k] and topk_w
+ * [T][k] are HOST arrays like the reference's (int64 expert ids; ids outside
+ * 0..E-1 and weights <= 0 are skipped); x [T][D] and y [T][D] are device
+ * pointers.  mid_dtype is the type the SwiGLU product is rounded to before the
+ * down projection (TFQ_F32 or TFQ_BF16).  workspace is device memory of at
+ * least tfq_moe_workspace_bytes(T, k, D, F) bytes, 256-byte aligned. */
+int tfq_moe_route(const float* logits, int T, int E, int k, float* probs, int32_t* idx, float* weights,
+                  tfq_stream_t stream);
+size_t tfq_moe_workspace_bytes(int T, int k, int64_t D, int64_t F);
+int tfq_moe_ffn(const tfq_weight_t* const* gate, const tfq_weight_t* const* up,
+                const tfq_weight_t* const* down, int E, const int64_t* topk_idx, const float* topk_w,
+                int T, int k, const void* x, int x_dtype, void* y, int y_dtype, int mid_dtype,
+                void* workspace, size_t workspace_bytes, tfq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

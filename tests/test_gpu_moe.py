@@ -1,0 +1,132 @@
+"""MoE expert path through the C ABI against the oracle (reference dispatch order)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_err(y, ref):
+    return float(np.abs(y.astype(np.float64) - ref).max() / np.abs(ref).max())
+
+
+def test_route_matches_reference_softmax_topk(O, tfq, gpu):
+    import torch
+    T, E, K = 16, 8, 2
+    logits = O.rng_normal(45, T * E, 1.0).reshape(T, E)
+    probs, idx, w = O.softmax_topk(logits, K)
+    p_d, i_d, w_d = tfq.moe_route(torch.from_numpy(logits).to(gpu), K)
+    assert np.array_equal(i_d.cpu().numpy().astype(np.int64), idx)
+    assert np.abs(p_d.cpu().numpy() - probs).max() <= 2e-7
+    assert np.abs(w_d.cpu().numpy() - w).max() <= 2e-7
+    # closed form: rows sum to one, weights are the k largest probabilities, not renormalised
+    pn = p_d.cpu().numpy()
+    assert np.abs(pn.sum(axis=1) - 1).max() < 1e-6
+    assert np.allclose(np.sort(pn, axis=1)[:, ::-1][:, :K], w_d.cpu().numpy(), atol=0, rtol=0)
+    # k is clamped into 1..E like the reference does
+    assert tfq.moe_route(torch.from_numpy(logits).to(gpu), 99)[1].shape == (T, E)
+
+
+def _experts(O, tfq, fmt, E, D, F, seed):
+    gate, up, down, hg, hu, hd = [], [], [], [], [], []
+    for e in range(E):
+        for lst, hst, n, k, off in ((gate, hg, F, D, 0), (up, hu, F, D, 1), (down, hd, D, F, 2)):
+            pay = O.encode_tensor(fmt, O.rng_normal(seed + 10 * e + off, n * k, 0.02))
+            hst.append(pay)
+            lst.append(tfq.Weight(fmt, n, k, pay))
+    return gate, up, down, hg, hu, hd
+
+
+@pytest.mark.parametrize("fmt", ["Q_G_4", "B32S4"])
+@pytest.mark.parametrize("xdt,mid_bf16,tol", [("bf16", True, 1e-2), ("f32", False, 1e-3)])
+def test_moe_ffn_small(O, tfq, gpu, fmt, xdt, mid_bf16, tol):
+    """8 experts, top-2, 16 tokens: the Mixtral-style configuration at reduced width."""
+    import torch
+    E, Ktop, T, D, F = 8, 2, 16, 512, 1024
+    gate, up, down, hg, hu, hd = _experts(O, tfq, fmt, E, D, F, 300)
+    logits = O.rng_normal(45, T * E, 1.0).reshape(T, E)
+    _, idx, w = O.softmax_topk(logits, Ktop)
+    x = O.rng_normal(43, T * D, 1.0).reshape(T, D)
+    if xdt == "bf16":
+        x = O.bf16_round(x)
+        xt = torch.from_numpy(x).to(gpu).bfloat16()
+    else:
+        xt = torch.from_numpy(x).to(gpu)
+    ref = O.moe_ffn(fmt, hg, hu, hd, D, F, idx, w, x, mid_bf16=mid_bf16)
+    y = tfq.moe_ffn(gate, up, down, idx, w, xt, mid_dtype=torch.bfloat16 if mid_bf16 else torch.float32).cpu().numpy()
+    assert rel_err(y, ref) <= tol
+    # invariants: every (token, slot) pair is dispatched once; weights in (0, 1]
+    assert sum((idx == e).sum() for e in range(E)) == T * Ktop and np.all((w > 0) & (w <= 1))
+    # an expert nobody routes to, a dropped (non-positive) weight and an out-of-range id are skipped
+    idx2, w2 = idx.copy(), w.copy()
+    idx2[idx2 == 3] = 5
+    w2[0, 0] = 0.0
+    idx2[1, 1] = 99
+    for t in range(T):  # keep the two slots of a token distinct
+        if idx2[t, 0] == idx2[t, 1]:
+            idx2[t, 1] = (idx2[t, 0] + 1) % E if (idx2[t, 0] + 1) % E != 3 else (idx2[t, 0] + 2) % E
+    ref2 = O.moe_ffn(fmt, hg, hu, hd, D, F, idx2, w2, x, mid_bf16=mid_bf16)
+    y2 = tfq.moe_ffn(gate, up, down, idx2, w2, xt, mid_dtype=torch.bfloat16 if mid_bf16 else torch.float32).cpu().numpy()
+    assert rel_err(y2, ref2) <= tol
+    yb = tfq.moe_ffn(gate, up, down, idx, w, xt, out_dtype=torch.bfloat16,
+                     mid_dtype=torch.bfloat16 if mid_bf16 else torch.float32).float().cpu().numpy()
+    assert rel_err(yb, ref) <= 1e-2
+    for wl in gate + up + down:
+        wl.close()
+
+
+def test_moe_single_token_equals_plain_mlp(O, tfq, gpu):
+    """One token, one expert, weight 1: the MoE path reduces to the SwiGLU MLP step."""
+    import torch
+    fmt, D, F = "B32S4", 512, 768
+    gate, up, down, hg, hu, hd = _experts(O, tfq, fmt, 1, D, F, 500)
+    x = O.bf16_round(O.rng_normal(7, D, 1.0).reshape(1, D))
+    xt = torch.from_numpy(x).to(gpu).bfloat16()
+    y = tfq.moe_ffn(gate, up, down, np.zeros((1, 1), np.int64), np.ones((1, 1), np.float32), xt,
+                    mid_dtype=torch.float32).cpu().numpy()
+    g = O.matmul(fmt, hg[0], F, D, x)
+    u = O.matmul(fmt, hu[0], F, D, x)
+    want = O.matmul(fmt, hd[0], D, F, O.silu_mul(g, u))
+    assert rel_err(y, want) <= 1e-3
+    for wl in gate + up + down:
+        wl.close()
+
+
+def test_config5_mixtral_layer_full_size(tfq, gpu):
+    """8 experts, top-2, 16 tokens, gate/up 14336x4096 and down 4096x14336, B32S4 weights from
+    N(0, 0.02), bf16 activations: checked against a dense torch evaluation of the same decoded
+    weights (the oracle takes minutes at this size), plus conservation under weight scaling."""
+    import torch
+    E, Ktop, T, D, F = 8, 2, 16, 4096, 14336
+    g = torch.Generator(device="cuda").manual_seed(5)
+    gate, up, down = [], [], []
+    for e in range(E):
+        for lst, n, k in ((gate, F, D), (up, F, D), (down, D, F)):
+            w = torch.randn(n * k, device=gpu, generator=g) * 0.02
+            lst.append(tfq.Weight("B32S4", n, k, tfq.encode("B32S4", w)))
+            del w
+    logits = torch.randn(T, E, device=gpu, generator=g)
+    _, idx, wts = tfq.moe_route(logits, Ktop)
+    idx_h, w_h = idx.cpu().numpy().astype(np.int64), wts.cpu().numpy()
+    x = torch.randn(T, D, device=gpu, generator=g).bfloat16()
+    y = tfq.moe_ffn(gate, up, down, idx_h, w_h, x, mid_dtype=torch.bfloat16)
+    want = torch.zeros(T, D, device=gpu, dtype=torch.float64)
+    xf = x.double()
+    for e in range(E):
+        toks = [t for t in range(T) if e in idx_h[t]]
+        if not toks:
+            continue
+        Wg, Wu, Wd = gate[e].decode().double(), up[e].decode().double(), down[e].decode().double()
+        xe = xf[toks]
+        gg, uu = (xe @ Wg.T).float(), (xe @ Wu.T).float()
+        h = (gg / (1 + torch.exp(-gg)) * uu).bfloat16().double()
+        o = h @ Wd.T
+        for i, t in enumerate(toks):
+            want[t] += float(w_h[t][list(idx_h[t]).index(e)]) * o[i]
+        del Wg, Wu, Wd
+    err = float((y.double() - want).abs().max() / want.abs().max())
+    assert err <= 1e-2, err
+    # linear in the routing weights: doubling them doubles the output exactly (power of two)
+    y2 = tfq.moe_ffn(gate, up, down, idx_h, 2 * w_h, x, mid_dtype=torch.bfloat16)
+    assert torch.equal(y2, 2 * y)
+    for wl in gate + up + down:
+        wl.close()

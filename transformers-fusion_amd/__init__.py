@@ -57,6 +57,9 @@ def _load():
         "tfq_gemm": (i32, [vp, vp, i32, i32, vp, i32, vp]),
         "tfq_gemv_multi": (i32, [vp, i32, vp, i32, i32, vp, i32, vp]),
         "tfq_matmul_host": (i32, [vp, vp, vp, i32]),
+        "tfq_moe_route": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
+        "tfq_moe_workspace_bytes": (sz, [i32, i32, i64, i64]),
+        "tfq_moe_ffn": (i32, [vp, vp, vp, i32, vp, vp, i32, i32, vp, i32, vp, i32, i32, vp, sz, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -193,3 +196,37 @@ def gemv_multi(weights, x, outs):
     B = x.numel() // weights[0].K
     _check(lib().tfq_gemv_multi(hs, n, x.data_ptr(), _dtype_code(x), B, ys, _dtype_code(outs[0]), _stream()))
     return outs
+
+
+def moe_route(logits, k: int):
+    """Device softmax + top-k: returns (probs [T][E], idx [T][k] int32, weights [T][k])."""
+    import torch
+    logits = logits.contiguous().float()
+    T, E = logits.shape
+    k = max(1, min(k, E))
+    probs = torch.empty_like(logits)
+    idx = torch.empty((T, k), dtype=torch.int32, device=logits.device)
+    w = torch.empty((T, k), dtype=torch.float32, device=logits.device)
+    _check(lib().tfq_moe_route(logits.data_ptr(), T, E, k, probs.data_ptr(), idx.data_ptr(), w.data_ptr(), _stream()))
+    return probs, idx, w
+
+
+def moe_ffn(gate, up, down, topk_idx, topk_w, x, out_dtype=None, mid_dtype=None):
+    """MoE expert FFN.  gate/up/down: lists of Weight; topk_idx/topk_w: host arrays [T][k]; x: device [T][D]."""
+    import numpy as np
+    import torch
+    E = len(gate)
+    idx = np.ascontiguousarray(topk_idx, np.int64)
+    wts = np.ascontiguousarray(topk_w, np.float32)
+    T, k = idx.shape
+    D, F = gate[0].K, gate[0].N
+    x = x.contiguous()
+    y = torch.empty((T, D), dtype=out_dtype or torch.float32, device=x.device)
+    mid = BF16 if (mid_dtype or x.dtype) == torch.bfloat16 else F32
+    nbytes = lib().tfq_moe_workspace_bytes(T, k, D, F)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    arr = lambda ws_: (C.c_void_p * E)(*[w.handle for w in ws_])
+    _check(lib().tfq_moe_ffn(arr(gate), arr(up), arr(down), E, idx.ctypes.data, wts.ctypes.data, T, k,
+                             x.data_ptr(), _dtype_code(x), y.data_ptr(), _dtype_code(y), mid,
+                             ws.data_ptr(), nbytes, _stream()))
+    return y

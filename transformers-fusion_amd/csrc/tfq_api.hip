@@ -300,6 +300,37 @@ int tfq_gemm(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, 
     return launch_gemm(w, x, x_dtype, M, y, y_dtype, (hipStream_t)stream);
 }
 
+int tfq_moe_route(const float* logits, int T, int E, int k, float* probs, int32_t* idx, float* weights, tfq_stream_t stream) {
+    if (!logits || !probs || !idx || !weights) return fail(TFQ_ERR_ARG, "tfq_moe_route: null pointer");
+    if (T <= 0 || E <= 0) return fail(TFQ_ERR_ARG, "tfq_moe_route: T and E must be positive");
+    if (k < 1) k = 1;  // the reference clamps k into 1..E
+    if (k > E) k = E;
+    if (int r = ensure_device()) return r;
+    return launch_moe_route(logits, T, E, k, probs, idx, weights, (hipStream_t)stream);
+}
+
+size_t tfq_moe_workspace_bytes(int T, int k, int64_t D, int64_t F) {
+    if (T <= 0 || k <= 0 || D <= 0 || F <= 0) return 0;
+    return moe_workspace_bytes(T, k, D, F);
+}
+
+int tfq_moe_ffn(const tfq_weight_t* const* gate, const tfq_weight_t* const* up, const tfq_weight_t* const* down, int E,
+                const int64_t* topk_idx, const float* topk_w, int T, int k, const void* x, int x_dtype, void* y,
+                int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes, tfq_stream_t stream) {
+    if (!gate || !up || !down || !topk_idx || !topk_w || !x || !y || !workspace)
+        return fail(TFQ_ERR_ARG, "tfq_moe_ffn: null pointer");
+    if (E <= 0 || T <= 0 || k <= 0) return fail(TFQ_ERR_ARG, "tfq_moe_ffn: E, T and k must be positive");
+    if ((x_dtype != TFQ_F32 && x_dtype != TFQ_BF16) || (y_dtype != TFQ_F32 && y_dtype != TFQ_BF16) ||
+        (mid_dtype != TFQ_F32 && mid_dtype != TFQ_BF16))
+        return fail(TFQ_ERR_ARG, "tfq_moe_ffn: dtype must be TFQ_F32 or TFQ_BF16");
+    for (int e = 0; e < E; ++e)
+        if (!gate[e] || !up[e] || !down[e]) return fail(TFQ_ERR_ARG, "tfq_moe_ffn: null expert handle");
+    if ((uintptr_t)x % 16 || (uintptr_t)workspace % 256) return fail(TFQ_ERR_ARG, "tfq_moe_ffn: x must be 16-byte, workspace 256-byte aligned");
+    if (int r = ensure_device()) return r;
+    return launch_moe_ffn(gate, up, down, E, topk_idx, topk_w, T, k, x, x_dtype, y, y_dtype, mid_dtype, workspace,
+                          workspace_bytes, (hipStream_t)stream);
+}
+
 int tfq_matmul_host(const tfq_weight_t* w, const float* X, float* Y, int B) {
     if (!w || !X || !Y) return fail(TFQ_ERR_ARG, "tfq_matmul_host: null pointer");
     if (B <= 0) return fail(TFQ_ERR_ARG, "tfq_matmul_host: batch must be positive");

@@ -106,6 +106,11 @@ int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int 
                       void* const* ys, int y_dtype, hipStream_t s);
 int launch_gemv_generic(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype,
                         hipStream_t s);
+size_t moe_workspace_bytes(int T, int Ktop, int64_t D, int64_t F);
+int launch_moe_route(const float* logits, int T, int E, int k, float* probs, int* idx, float* wts, hipStream_t s);
+int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E,
+                   const int64_t* topk_idx, const float* topk_w, int T, int Ktop, const void* x, int x_dtype,
+                   void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes, hipStream_t s);
 int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
                 hipStream_t s);
 
