@@ -459,17 +459,4 @@ int launch_gemv(const tfq_weight* w, const void* x, int x_dtype, int B, void* y,
     return launch_gemv_multi(&w, 1, x, x_dtype, B, &y, y_dtype, s);
 }
 
-int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype, hipStream_t s) {
-    // Until the MFMA prefill kernel exists, a tall activation matrix is cut into
-    // 16-row slices for the GEMV kernel.
-    const size_t xe = x_dtype == TFQ_F32 ? 4 : 2, ye = y_dtype == TFQ_F32 ? 4 : 2;
-    for (int m0 = 0; m0 < M; m0 += 16) {
-        const int mb = M - m0 < 16 ? M - m0 : 16;
-        const int rc = launch_gemv(w, (const uint8_t*)x + (size_t)m0 * w->K * xe, x_dtype, mb,
-                                   (uint8_t*)y + (size_t)m0 * w->N * ye, y_dtype, s);
-        if (rc) return rc;
-    }
-    return TFQ_OK;
-}
-
 }  // namespace tfq
