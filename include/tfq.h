@@ -148,6 +148,40 @@ int tfq_moe_ffn(const tfq_weight_t* const* gate, const tfq_weight_t* const* up,
                 int T, int k, const void* x, int x_dtype, void* y, int y_dtype, int mid_dtype,
                 void* workspace, size_t workspace_bytes, tfq_stream_t stream);
 
+/* ---- codebook-lookup operators ----------------------------------------------------
+ * Weights are BITS-wide indices into one small table of centroids.  packed / idx,
+ * act / X and out / Y are device pointers; the codebook is a HOST pointer (it is
+ * passed to the kernel by value).
+ *
+ * tfq_lut4_gemm: kernel::quant4_gemm (include/quant/kernel.h:30-34,
+ *   src/kernel/kernel_quant4.cpp:18-47): out[m*N+n] = sum_k f16(cb[nib(m*N+n, k)]) * act[n*K+k],
+ *   where the packed row of the pair (m,n) starts at byte ((m*N+n)*K)/2 and nibble k
+ *   is the low half of byte k/2 for even k.  codebook = 16 binary16 values.
+ * tfq_lut8_gemm: kernel::quant8_gemm (include/quant/kernel.h:24-28,
+ *   src/kernel/kernel_quant8.cpp:14-32): out[m*N+n] = sum_k cb[idx[n*K+k]] * act[m*K+k].
+ *   codebook = 256 floats.
+ * tfq_lut_gemv_batch: prod::gemv_quant_batch / gemv_quant4_batch / gemv_quant8_batch and,
+ *   with N = 1, the _tiled forms (include/quant/kernel_production.h:25-51; semantics =
+ *   the scalar loops src/kernel/kernel_production.cpp:68-117): Y[n*M+m] = scale *
+ *   sum_k cb[idx(m,k)] * X[n*K+k]; rows of ceil(K*bits/8) bytes.  bits = 2 (codes
+ *   0,1,2,3 = -1,0,+1,+1; codebook ignored), 4 (16 binary16) or 8 (256 floats). */
+int tfq_lut4_gemm(const uint8_t* packed, const uint16_t* codebook, const float* act, float* out, int M,
+                  int N, int K, tfq_stream_t stream);
+int tfq_lut8_gemm(const uint8_t* idx, const float* codebook, const float* act, float* out, int M, int N,
+                  int K, tfq_stream_t stream);
+int tfq_lut_gemv_batch(int bits, const uint8_t* packed, const void* codebook, float scale, const float* X,
+                       float* Y, int M, int N, int K, tfq_stream_t stream);
+
+/* ---- device memory for hosts without a HIP toolchain ---------------------------------
+ * The reference's operators take host pointers (include/quant/kernel.h:24-54); a
+ * caller compiled without HIP moves its buffers with these.  tfq_malloc returns
+ * NULL on failure (see tfq_last_error).  Copies are synchronous. */
+void* tfq_malloc(size_t bytes);
+void tfq_free(void* dev);
+int tfq_copy_to_device(void* dev, const void* host, size_t bytes);
+int tfq_copy_to_host(void* host, const void* dev, size_t bytes);
+int tfq_stream_sync(tfq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

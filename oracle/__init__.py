@@ -89,6 +89,7 @@ lib.orc_moe_ffn.argtypes = [C.c_uint8, C.POINTER(_u8p), C.POINTER(_u8p), C.POINT
                             _f32p, _f32p, C.c_int, C.c_int]
 lib.orc_quant4_gemm.argtypes = [_u8p, C.POINTER(C.c_uint16), _f32p, _f32p, C.c_int, C.c_int, C.c_int]
 lib.orc_quant8_gemm.argtypes = [_u8p, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+lib.orc_lut_gemv_batch.argtypes = [C.c_int, _u8p, C.c_void_p, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
 lib.orc_comp8_table.argtypes = [_f32p]
 
 THREADS = min(16, os.cpu_count() or 1)
@@ -262,6 +263,20 @@ def quant8_gemm(idx, cb256, act, M: int, N: int, K: int) -> np.ndarray:
     cb256, act = _f32(cb256), _f32(act)
     out = np.empty((M, N), np.float32)
     lib.orc_quant8_gemm(_ptr(idx, _u8p), _ptr(cb256, _f32p), _ptr(act, _f32p), _ptr(out, _f32p), M, N, K)
+    return out
+
+
+def lut_gemv_batch(bits: int, packed, cb, scale: float, X, M: int, N: int, K: int) -> np.ndarray:
+    """Y[N][M] of the production batch GEMV (scalar semantics); cb: 16 uint16 (bits 4), 256 float (bits 8), None (bits 2)."""
+    packed = np.ascontiguousarray(packed, np.uint8)
+    X = _f32(X)
+    out = np.empty((N, M), np.float32)
+    if bits == 4:
+        cb = np.ascontiguousarray(cb, np.uint16)
+    elif bits == 8:
+        cb = _f32(cb)
+    cbp = C.c_void_p(cb.ctypes.data) if bits != 2 else C.c_void_p(0)
+    lib.orc_lut_gemv_batch(bits, _ptr(packed, _u8p), cbp, C.c_float(scale), _ptr(X, _f32p), _ptr(out, _f32p), M, N, K)
     return out
 
 

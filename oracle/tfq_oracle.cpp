@@ -1028,4 +1028,33 @@ void orc_quant8_gemm(const uint8_t* idx, const float* cb256, const float* act, f
         }
 }
 
+// Batch GEMV of the production kernels, scalar semantics
+// (gemv_quant_tiled_scalar / gemv_quant4_tiled_scalar / gemv_quant8_tiled_scalar and
+// the _batch loops, src/kernel/kernel_production.cpp:68-117, 334-353):
+// Y[n*M+m] = scale * sum_k value(m,k) * X[n*K+k], rows of ceil(K*bits/8) bytes.
+// bits = 2: codes 0,1,2,3 = -1,0,+1,+1 (decode_quant :55-58); bits = 4: 16 binary16
+// centroids, low nibble first; bits = 8: 256 float centroids.
+void orc_lut_gemv_batch(int bits, const uint8_t* packed, const void* cb, float scale, const float* X, float* Y,
+                        int M, int N, int K) {
+    float tab[256] = {};
+    if (bits == 2) {
+        tab[0] = -1.0f; tab[1] = 0.0f; tab[2] = 1.0f; tab[3] = 1.0f;
+    } else if (bits == 4) {
+        for (int i = 0; i < 16; ++i) tab[i] = half_to_float(static_cast<const uint16_t*>(cb)[i]);
+    } else {
+        for (int i = 0; i < 256; ++i) tab[i] = static_cast<const float*>(cb)[i];
+    }
+    const size_t row_bytes = ((size_t)K * (size_t)bits + 7) / 8;
+    const int per = 8 / bits;
+    const unsigned mask = (1u << bits) - 1u;
+    for (int n = 0; n < N; ++n)
+        for (int m = 0; m < M; ++m) {
+            const uint8_t* row = packed + (size_t)m * row_bytes;
+            const float* x = X + (size_t)n * (size_t)K;
+            float s = 0.0f;
+            for (int k = 0; k < K; ++k) s += tab[(row[k / per] >> ((k % per) * bits)) & mask] * x[k];
+            Y[(size_t)n * (size_t)M + (size_t)m] = s * scale;
+        }
+}
+
 }  // extern "C"

@@ -1,0 +1,49 @@
+"""The C++ shim library must export the reference's own (mangled) names, so that it links in
+place of the reference's translation units.  The expected names are what g++ emits for the
+declarations in include/quant/block_codec.h:69-83, include/quant/kernel.h:24-34 and
+include/quant/kernel_production.h:25-51; where the compiled reference is built they are also
+looked up in it."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SHIMS = os.path.join(ROOT, "transformers-fusion_amd", "libtfq_shims.so")
+REF = os.path.join(ROOT, "oracle", "_ref", "libref.so")
+
+EXPECTED = [
+    "_ZN5quant16block_actual_bpwEjmm",
+    "_ZN5quant18quantize_block_allENS_6FormatEPKfiRSt6vectorIhSaIhEES6_",
+    "_ZN5quant19block_claimed_bytesENS_6FormatEj",
+    "_ZN5quant20dequantize_block_allENS_6FormatEPKhmS2_mjPf",
+    "_ZN5quant6kernel11quant4_gemmEPKhPKtPKfPfiii",
+    "_ZN5quant6kernel11quant8_gemmEPKhPKfS4_Pfiii",
+    "_ZN5quant8adapters4prod16gemv_quant_batchEPKhfPKfPfiii",
+    "_ZN5quant8adapters4prod16gemv_quant_tiledEPKhfPKfPfiii",
+    "_ZN5quant8adapters4prod17gemv_quant4_batchEPKhPKtfPKfPfiii",
+    "_ZN5quant8adapters4prod17gemv_quant4_tiledEPKhPKtfPKfPfiii",
+    "_ZN5quant8adapters4prod17gemv_quant8_batchEPKhPKffS5_Pfiii",
+    "_ZN5quant8adapters4prod17gemv_quant8_tiledEPKhPKffS5_Pfiii",
+]
+
+
+def defined(path):
+    out = subprocess.check_output(["nm", "-D", "--defined-only", path], text=True)
+    return {line.split()[-1] for line in out.splitlines() if line.strip()}
+
+
+def test_shims_export_the_reference_names():
+    if not os.path.exists(SHIMS):
+        pytest.skip("libtfq_shims.so not built")
+    have = defined(SHIMS)
+    missing = [s for s in EXPECTED if s not in have]
+    assert not missing, missing
+
+
+def test_the_compiled_reference_defines_the_same_names():
+    if not os.path.exists(REF):
+        pytest.skip("compiled reference not built on this machine")
+    have = defined(REF)
+    missing = [s for s in EXPECTED if s not in have]
+    assert not missing, missing

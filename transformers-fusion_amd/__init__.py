@@ -60,6 +60,14 @@ def _load():
         "tfq_moe_route": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "tfq_moe_workspace_bytes": (sz, [i32, i32, i64, i64]),
         "tfq_moe_ffn": (i32, [vp, vp, vp, i32, vp, vp, i32, i32, vp, i32, vp, i32, i32, vp, sz, vp]),
+        "tfq_lut4_gemm": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
+        "tfq_lut8_gemm": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
+        "tfq_lut_gemv_batch": (i32, [i32, vp, vp, C.c_float, vp, vp, i32, i32, i32, vp]),
+        "tfq_malloc": (vp, [sz]),
+        "tfq_free": (None, [vp]),
+        "tfq_copy_to_device": (i32, [vp, vp, sz]),
+        "tfq_copy_to_host": (i32, [vp, vp, sz]),
+        "tfq_stream_sync": (i32, [vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -230,3 +238,39 @@ def moe_ffn(gate, up, down, topk_idx, topk_w, x, out_dtype=None, mid_dtype=None)
                              x.data_ptr(), _dtype_code(x), y.data_ptr(), _dtype_code(y), mid,
                              ws.data_ptr(), nbytes, _stream()))
     return y
+
+
+def lut4_gemm(packed, codebook16, act, M: int, N: int, K: int):
+    """kernel::quant4_gemm on the device: packed (uint8) and act (fp32 [N][K]) are device tensors, codebook16 a host uint16[16]."""
+    import numpy as np
+    import torch
+    cb = np.ascontiguousarray(codebook16, np.uint16)
+    out = torch.empty((M, N), dtype=torch.float32, device=act.device)
+    _check(lib().tfq_lut4_gemm(packed.data_ptr(), cb.ctypes.data, act.data_ptr(), out.data_ptr(), M, N, K, _stream()))
+    return out
+
+
+def lut8_gemm(idx, codebook256, act, M: int, N: int, K: int):
+    """kernel::quant8_gemm on the device: idx uint8 [N][K], act fp32 [M][K] device tensors, codebook256 a host float[256]."""
+    import numpy as np
+    import torch
+    cb = np.ascontiguousarray(codebook256, np.float32)
+    out = torch.empty((M, N), dtype=torch.float32, device=act.device)
+    _check(lib().tfq_lut8_gemm(idx.data_ptr(), cb.ctypes.data, act.data_ptr(), out.data_ptr(), M, N, K, _stream()))
+    return out
+
+
+def lut_gemv_batch(bits: int, packed, codebook, scale: float, X, M: int, N: int, K: int):
+    """prod::gemv_quant{,4,8}_batch on the device: Y[N][M] = scale * W . X^T."""
+    import numpy as np
+    import torch
+    cbp = None
+    if bits == 4:
+        cb = np.ascontiguousarray(codebook, np.uint16)
+        cbp = cb.ctypes.data
+    elif bits == 8:
+        cb = np.ascontiguousarray(codebook, np.float32)
+        cbp = cb.ctypes.data
+    out = torch.empty((N, M), dtype=torch.float32, device=X.device)
+    _check(lib().tfq_lut_gemv_batch(bits, packed.data_ptr(), cbp, scale, X.data_ptr(), out.data_ptr(), M, N, K, _stream()))
+    return out

@@ -13,7 +13,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtfq.so")
 
-SOURCES = ["tfq_api.hip", "tfq_codec.hip", "tfq_gemv.hip", "tfq_gemv_generic.hip", "tfq_moe.hip", "tfq_gemm.hip"]
+SOURCES = ["tfq_api.hip", "tfq_codec.hip", "tfq_gemv.hip", "tfq_gemv_generic.hip", "tfq_moe.hip", "tfq_gemm.hip",
+           "tfq_lut.hip"]
 
 # -ffp-contract=off: the decode arithmetic is ordered to match the reference
 #   bit for bit, fusion happens only where the source says fmaf.
@@ -58,5 +59,19 @@ def build_library(verbose: bool = False) -> str:
     return LIB
 
 
+SHIMS = os.path.join(HERE, "libtfq_shims.so")
+
+
+def build_shims(verbose: bool = False) -> str:
+    """Host C++ (g++, no HIP): the reference-named C++ entry points over the C ABI."""
+    cmd = ["g++", "-std=c++20", "-O2", "-fPIC", "-Wall", "-shared", os.path.join(CSRC, "tfq_shims.cpp"),
+           "-o", SHIMS, "-L" + HERE, "-ltfq", "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return SHIMS
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_shims(verbose=True))

@@ -349,4 +349,57 @@ int tfq_matmul_host(const tfq_weight_t* w, const float* X, float* Y, int B) {
     return rc;
 }
 
+static int check_lut(const char* who, const void* w, const void* x, const void* y, int M, int N, int K) {
+    if (!w || !x || !y) return fail(TFQ_ERR_ARG, std::string(who) + ": null pointer");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(TFQ_ERR_ARG, std::string(who) + ": M, N and K must be positive");
+    return ensure_device();
+}
+
+int tfq_lut4_gemm(const uint8_t* packed, const uint16_t* codebook, const float* act, float* out, int M, int N, int K,
+                  tfq_stream_t stream) {
+    if (!codebook) return fail(TFQ_ERR_ARG, "tfq_lut4_gemm: null codebook");
+    if (int r = check_lut("tfq_lut4_gemm", packed, act, out, M, N, K)) return r;
+    return launch_lut4_gemm(packed, codebook, act, out, M, N, K, (hipStream_t)stream);
+}
+
+int tfq_lut8_gemm(const uint8_t* idx, const float* codebook, const float* act, float* out, int M, int N, int K,
+                  tfq_stream_t stream) {
+    if (!codebook) return fail(TFQ_ERR_ARG, "tfq_lut8_gemm: null codebook");
+    if (int r = check_lut("tfq_lut8_gemm", idx, act, out, M, N, K)) return r;
+    return launch_lut8_gemm(idx, codebook, act, out, M, N, K, (hipStream_t)stream);
+}
+
+int tfq_lut_gemv_batch(int bits, const uint8_t* packed, const void* codebook, float scale, const float* X, float* Y,
+                       int M, int N, int K, tfq_stream_t stream) {
+    if (bits != 2 && bits != 4 && bits != 8) return fail(TFQ_ERR_ARG, "tfq_lut_gemv_batch: bits must be 2, 4 or 8");
+    if (bits != 2 && !codebook) return fail(TFQ_ERR_ARG, "tfq_lut_gemv_batch: null codebook");
+    if (int r = check_lut("tfq_lut_gemv_batch", packed, X, Y, M, N, K)) return r;
+    return launch_lut_gemv_batch(bits, packed, codebook, scale, X, Y, M, N, K, (hipStream_t)stream);
+}
+
+void* tfq_malloc(size_t bytes) {
+    if (ensure_device()) return nullptr;
+    void* p = nullptr;
+    if (hip_fail(hipMalloc(&p, bytes ? bytes : 1), "tfq_malloc")) return nullptr;
+    return p;
+}
+
+void tfq_free(void* dev) {
+    if (dev) (void)hipFree(dev);
+}
+
+int tfq_copy_to_device(void* dev, const void* host, size_t bytes) {
+    if (!bytes) return TFQ_OK;
+    if (!dev || !host) return fail(TFQ_ERR_ARG, "tfq_copy_to_device: null pointer");
+    return hip_fail(hipMemcpy(dev, host, bytes, hipMemcpyHostToDevice), "tfq_copy_to_device");
+}
+
+int tfq_copy_to_host(void* host, const void* dev, size_t bytes) {
+    if (!bytes) return TFQ_OK;
+    if (!dev || !host) return fail(TFQ_ERR_ARG, "tfq_copy_to_host: null pointer");
+    return hip_fail(hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost), "tfq_copy_to_host");
+}
+
+int tfq_stream_sync(tfq_stream_t stream) { return hip_fail(hipStreamSynchronize((hipStream_t)stream), "tfq_stream_sync"); }
+
 }  // extern "C"

@@ -113,6 +113,12 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
                    void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes, hipStream_t s);
 int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
                 hipStream_t s);
+int launch_lut4_gemm(const uint8_t* packed, const uint16_t* cb16, const float* act, float* out, int M, int N, int K,
+                     hipStream_t s);
+int launch_lut8_gemm(const uint8_t* idx, const float* cb, const float* act, float* out, int M, int N, int K,
+                     hipStream_t s);
+int launch_lut_gemv_batch(int bits, const uint8_t* packed, const void* cb, float scale, const float* X, float* Y,
+                          int M, int Nb, int K, hipStream_t s);
 
 // ---------------------------------------------------------------- device helpers
 // binary16 -> binary32 by integer arithmetic: exact for every input including

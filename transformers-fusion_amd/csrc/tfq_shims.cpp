@@ -1,0 +1,204 @@
+// Definitions of the reference-named entry points declared in include/tfq_shims.hpp.
+// Host C++ only (built with g++, linked against libtfq.so): each function moves the
+// caller's host buffers to the device through the C ABI, runs the HIP path and
+// moves the result back.  There is no CPU computation in this file.
+
+#include "../../include/tfq_shims.hpp"
+
+#include <cmath>
+#include <cstring>
+
+namespace {
+
+// Device buffers of one call; released on scope exit.
+struct DeviceBuffers {
+    std::vector<void*> ptrs;
+    ~DeviceBuffers() {
+        for (void* p : ptrs) tfq_free(p);
+    }
+    void* alloc(size_t bytes) {
+        void* p = tfq_malloc(bytes);
+        if (p) ptrs.push_back(p);
+        return p;
+    }
+    void* upload(const void* host, size_t bytes) {
+        void* p = alloc(bytes);
+        if (p && tfq_copy_to_device(p, host, bytes) != TFQ_OK) return nullptr;
+        return p;
+    }
+};
+
+void lut_batch(int bits, const uint8_t* packed, const void* codebook, float scale, const float* X, float* Y, int M,
+               int N, int K) {
+    if (!packed || !X || !Y || M <= 0 || N <= 0 || K <= 0) return;
+    DeviceBuffers d;
+    const size_t row_bytes = ((size_t)K * (size_t)bits + 7) / 8;
+    const uint8_t* dw = static_cast<const uint8_t*>(d.upload(packed, (size_t)M * row_bytes));
+    const float* dx = static_cast<const float*>(d.upload(X, (size_t)N * (size_t)K * 4));
+    float* dy = static_cast<float*>(d.alloc((size_t)N * (size_t)M * 4));
+    if (!dw || !dx || !dy) return;
+    if (tfq_lut_gemv_batch(bits, dw, codebook, scale, dx, dy, M, N, K, nullptr) != TFQ_OK) return;
+    tfq_copy_to_host(Y, dy, (size_t)N * (size_t)M * 4);
+}
+
+}  // namespace
+
+namespace quant {
+
+bool quantize_block_all(Format fmt, const float* w, int n, std::vector<uint8_t>& indices,
+                        std::vector<uint8_t>& codebook) {
+    indices.clear();
+    codebook.clear();
+    size_t bytes = 0;
+    if (!w || n <= 0 || tfq_block_bytes((uint8_t)fmt, (uint32_t)n, &bytes) != TFQ_OK) return false;
+    indices.resize(bytes);
+    if (tfq_encode_blocks_host((uint8_t)fmt, w, n, indices.data(), bytes, nullptr) != TFQ_OK) {
+        indices.clear();
+        return false;
+    }
+    return true;
+}
+
+// Pre-zeroes `out`, treats bytes past the payload as zero and leaves zeros for an
+// unhandled format, as the reference does (src/codec/block_codec.cpp:2869-2890).
+void dequantize_block_all(Format fmt, const uint8_t* indices, size_t idx_bytes, const uint8_t* /*codebook*/,
+                          size_t /*cb_bytes*/, uint32_t nw, float* out) {
+    if (!out || nw == 0) return;
+    std::memset(out, 0, (size_t)nw * sizeof(float));
+    size_t bytes = 0;
+    if (tfq_block_bytes((uint8_t)fmt, nw, &bytes) != TFQ_OK) return;
+    std::vector<uint8_t> padded(bytes, 0);
+    if (indices) std::memcpy(padded.data(), indices, idx_bytes < bytes ? idx_bytes : bytes);
+    std::vector<float> tmp(nw);
+    if (tfq_decode_blocks_host((uint8_t)fmt, padded.data(), bytes, nw, tmp.data()) == TFQ_OK)
+        std::memcpy(out, tmp.data(), (size_t)nw * sizeof(float));
+}
+
+float block_actual_bpw(uint32_t nw, size_t idx_bytes, size_t cb_bytes) {
+    if (nw == 0) return 0.0f;
+    return (float)((double)(idx_bytes + cb_bytes) * 8.0 / (double)nw);
+}
+
+size_t block_claimed_bytes(Format fmt, uint32_t n) {
+    return (size_t)std::ceil(tfq_format_bpw((uint8_t)fmt) * (float)n / 8.0f);
+}
+
+namespace kernel {
+
+void quant8_gemm(const uint8_t* indices, const float* codebook, const float* activations, float* output, int M,
+                 int N, int K) {
+    if (!indices || !codebook || !activations || !output || M <= 0 || N <= 0 || K <= 0) return;
+    DeviceBuffers d;
+    const uint8_t* dw = static_cast<const uint8_t*>(d.upload(indices, (size_t)N * (size_t)K));
+    const float* dx = static_cast<const float*>(d.upload(activations, (size_t)M * (size_t)K * 4));
+    float* dy = static_cast<float*>(d.alloc((size_t)M * (size_t)N * 4));
+    if (!dw || !dx || !dy) return;
+    if (tfq_lut8_gemm(dw, codebook, dx, dy, M, N, K, nullptr) != TFQ_OK) return;
+    tfq_copy_to_host(output, dy, (size_t)M * (size_t)N * 4);
+}
+
+void quant4_gemm(const uint8_t* packed_indices, const uint16_t* codebook, const float* activations, float* output,
+                 int M, int N, int K) {
+    if (!packed_indices || !codebook || !activations || !output || M <= 0 || N <= 0 || K <= 0) return;
+    DeviceBuffers d;
+    const size_t wbytes = ((size_t)M * (size_t)N * (size_t)K + 1) / 2;  // one packed row per (m, n) pair
+    const uint8_t* dw = static_cast<const uint8_t*>(d.upload(packed_indices, wbytes));
+    const float* dx = static_cast<const float*>(d.upload(activations, (size_t)N * (size_t)K * 4));
+    float* dy = static_cast<float*>(d.alloc((size_t)M * (size_t)N * 4));
+    if (!dw || !dx || !dy) return;
+    if (tfq_lut4_gemm(dw, codebook, dx, dy, M, N, K, nullptr) != TFQ_OK) return;
+    tfq_copy_to_host(output, dy, (size_t)M * (size_t)N * 4);
+}
+
+}  // namespace kernel
+
+namespace adapters {
+namespace prod {
+
+void gemv_quant_tiled(const uint8_t* w, float scale, const float* x, float* y, int M, int K, int) {
+    lut_batch(2, w, nullptr, scale, x, y, M, 1, K);
+}
+void gemv_quant4_tiled(const uint8_t* w, const uint16_t* cb, float scale, const float* x, float* y, int M, int K, int) {
+    if (cb) lut_batch(4, w, cb, scale, x, y, M, 1, K);
+}
+void gemv_quant8_tiled(const uint8_t* w, const float* cb, float scale, const float* x, float* y, int M, int K, int) {
+    if (cb) lut_batch(8, w, cb, scale, x, y, M, 1, K);
+}
+void gemv_quant_batch(const uint8_t* w, float scale, const float* X, float* Y, int M, int N, int K) {
+    lut_batch(2, w, nullptr, scale, X, Y, M, N, K);
+}
+void gemv_quant4_batch(const uint8_t* w, const uint16_t* cb, float scale, const float* X, float* Y, int M, int N,
+                       int K) {
+    if (cb) lut_batch(4, w, cb, scale, X, Y, M, N, K);
+}
+void gemv_quant8_batch(const uint8_t* w, const float* cb, float scale, const float* X, float* Y, int M, int N, int K) {
+    if (cb) lut_batch(8, w, cb, scale, X, Y, M, N, K);
+}
+
+}  // namespace prod
+}  // namespace adapters
+
+}  // namespace quant
+
+namespace tfq {
+
+BlockRowMatmul::BlockRowMatmul(uint8_t wire_format, int64_t rows, int64_t cols, const uint8_t* payload, size_t bytes)
+    : rows_(rows), cols_(cols) {
+    handle_ = tfq_weight_upload(wire_format, rows, cols, payload, bytes);
+}
+
+BlockRowMatmul::~BlockRowMatmul() { tfq_weight_free(handle_); }
+
+void BlockRowMatmul::gemm(const float* X, float* Y, int B) const {
+    if (!handle_ || !X || !Y || B <= 0 || B > MAX_BATCH) return;
+    tfq_matmul_host(handle_, X, Y, B);
+}
+
+void BlockRowMatmul::mlp_step(const BlockRowMatmul& gate, const BlockRowMatmul& up, const BlockRowMatmul& down,
+                              const float* x, float* out) {
+    if (!gate.ok() || !up.ok() || !down.ok() || !x || !out) return;
+    if (gate.rows() != up.rows() || gate.cols() != up.cols() || down.cols() != gate.rows()) return;
+    // One expert, one token, weight 1: the MoE entry point is exactly this chain on the device.
+    const tfq_weight_t* g = gate.handle();
+    const tfq_weight_t* u = up.handle();
+    const tfq_weight_t* dn = down.handle();
+    const int64_t idx = 0;
+    const float wt = 1.0f;
+    const int64_t D = gate.cols(), F = gate.rows();
+    if (down.rows() != D) return;
+    DeviceBuffers d;
+    const size_t wsb = tfq_moe_workspace_bytes(1, 1, D, F);
+    void* ws = d.alloc(wsb);
+    const float* dx = static_cast<const float*>(d.upload(x, (size_t)D * 4));
+    float* dy = static_cast<float*>(d.alloc((size_t)D * 4));
+    if (!ws || !dx || !dy) return;
+    if (tfq_moe_ffn(&g, &u, &dn, 1, &idx, &wt, 1, 1, dx, TFQ_F32, dy, TFQ_F32, TFQ_F32, ws, wsb, nullptr) != TFQ_OK) return;
+    if (tfq_stream_sync(nullptr) != TFQ_OK) return;
+    tfq_copy_to_host(out, dy, (size_t)D * 4);
+}
+
+TensorPayload TensorCodec::quantize(uint8_t wire_format, const float* data, int64_t n) {
+    TensorPayload p;
+    p.num_elements = n;
+    size_t per = 0;
+    if (!data || n <= 0 || n % 256 || tfq_block_bytes(wire_format, 256, &per) != TFQ_OK) return p;
+    const size_t blocks = (size_t)(n / 256);
+    p.indices.resize(blocks * per);
+    p.block_idx_bytes.resize(blocks);
+    if (tfq_encode_blocks_host(wire_format, data, n, p.indices.data(), p.indices.size(), p.block_idx_bytes.data()) != TFQ_OK) {
+        p.indices.clear();
+        p.block_idx_bytes.clear();
+        return p;
+    }
+    p.success = true;
+    return p;
+}
+
+void TensorCodec::dequantize(uint8_t wire_format, const TensorPayload& p, float* output, int64_t n) {
+    if (!output || n <= 0) return;
+    std::memset(output, 0, (size_t)n * sizeof(float));
+    if (!p.success || n % 256 || n > p.num_elements) return;
+    tfq_decode_blocks_host(wire_format, p.indices.data(), p.indices.size(), n, output);
+}
+
+}  // namespace tfq
