@@ -177,3 +177,30 @@ def test_config4_lowbit_superblock_shapes(O, tfq, gpu, fmt, bits):
         y = W.gemv(torch.from_numpy(x).to(gpu).bfloat16()).cpu().numpy()
         assert rel_err(y, O.matmul(fmt, pay, N, K, x)) <= 1e-4
     W.close()
+
+
+@pytest.mark.parametrize("fmt", GEMV_FORMATS)
+@pytest.mark.parametrize("N,K,B", [(16 * 256 * 2, 256, 1), (16 * 256 * 7, 256, 3), (16 * 256 * 5 + 40, 512, 4),
+                                   (16 * 300, 4096, 2), (48, 14336, 4), (16 * 256 * 3, 1024, 16)])
+def test_gemv_many_tiles_per_workgroup(O, tfq, gpu, fmt, N, K, B):
+    """More than 256 row tiles (a workgroup then walks several tiles, in groups of fetches with a
+    partial last group) and K = 14336 (four block columns per wavefront): checked against a dense
+    torch product of the device-decoded matrix, which the codec tests hold bit-exact."""
+    import torch
+    print(f"gemv tiles {fmt} N={N} K={K} B={B}", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(N + K + B)
+    if fmt == "B32S4":
+        w = torch.randn(N * K, device=gpu, generator=g) * 0.02
+        pay = tfq.encode(fmt, w)
+    else:  # random valid payloads: any code bytes, small finite binary16 d and dm
+        bb = tfq.block_bytes(fmt)
+        pay = torch.randint(0, 256, (N * K // 256, bb), device=gpu, dtype=torch.uint8, generator=g)
+        pay[:, -4:] = torch.tensor([0x00, 0x20, 0x00, 0x20], dtype=torch.uint8, device=gpu)
+        pay = pay.reshape(-1)
+    W = tfq.Weight(fmt, N, K, pay)
+    x = torch.randn(B, K, device=gpu, generator=g).bfloat16()
+    y = W.gemv(x)
+    want = x.double() @ W.decode().double().T
+    err = float((y.double() - want).abs().max() / want.abs().max())
+    assert err <= 1e-4, err
+    W.close()

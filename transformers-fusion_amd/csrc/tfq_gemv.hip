@@ -49,6 +49,7 @@ namespace {
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
 
 __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a),
@@ -93,6 +94,23 @@ struct GemvArgs {
     int cols_base, cols_rem;  // block columns per wavefront: cols_base + (wave < cols_rem)
 };
 
+// What the kernel receives: the same, flattened.  No arrays on purpose: a chain of selects over
+// array elements is folded by the optimizer into an indexed read of the argument block, which
+// costs a dependent memory access (or a private-memory copy of the block) per lookup.
+struct GemvKernArgs {
+    const uint8_t *W0, *W1, *W2, *W3;
+    void *y0, *y1, *y2, *y3;
+    int e0, e1, e2;
+    int nr0, nr1, nr2, nr3;
+    int ntiles, K, y_bf16, nslot, tiles_per_wg, cols_base, cols_rem;
+    explicit GemvKernArgs(const GemvArgs& a)
+        : W0(a.W[0]), W1(a.W[1]), W2(a.W[2]), W3(a.W[3]), y0(a.y[0]), y1(a.y[1]), y2(a.y[2]), y3(a.y[3]),
+          e0(a.tile_end[0]), e1(a.tile_end[1]), e2(a.tile_end[2]),
+          nr0(a.nrows[0]), nr1(a.nrows[1]), nr2(a.nrows[2]), nr3(a.nrows[3]),
+          ntiles(a.ntiles), K(a.K), y_bf16(a.y_bf16), nslot(a.nslot), tiles_per_wg(a.tiles_per_wg),
+          cols_base(a.cols_base), cols_rem(a.cols_rem) {}
+};
+
 // Matrix lookup without indexed kernel-argument reads (an indexed read is a
 // dependent scalar load from the argument segment, about a microsecond each):
 // everything is fetched once, unconditionally, and selected with compares.
@@ -100,8 +118,8 @@ struct GemvArgs {
 struct MatrixTable {
     const uint8_t* W0; const uint8_t* W1; const uint8_t* W2; const uint8_t* W3;
     int e0, e1, e2;
-    __device__ __forceinline__ explicit MatrixTable(const GemvArgs& a)
-        : W0(a.W[0]), W1(a.W[1]), W2(a.W[2]), W3(a.W[3]), e0(a.tile_end[0]), e1(a.tile_end[1]), e2(a.tile_end[2]) {}
+    __device__ __forceinline__ explicit MatrixTable(const GemvKernArgs& a)
+        : W0(a.W0), W1(a.W1), W2(a.W2), W3(a.W3), e0(a.e0), e1(a.e1), e2(a.e2) {}
     __device__ __forceinline__ int index(int tile) const { return (tile >= e0) + (tile >= e1) + (tile >= e2); }
     __device__ __forceinline__ int first_tile(int m) const { return m == 0 ? 0 : m == 1 ? e0 : m == 2 ? e1 : e2; }
     __device__ __forceinline__ const uint8_t* base(int m) const { return m == 0 ? W0 : m == 1 ? W1 : m == 2 ? W2 : W3; }
@@ -138,13 +156,14 @@ __device__ __forceinline__ float apply_groups(uint4 h, int khalf, f32x4_t D, flo
             res = __builtin_fmaf(off, xv[r], res);
         }
     } else {
-        // header: eight binary16 scales, four per k-step
-        const uint32_t hw[2] = {khalf ? h.z : h.x, khalf ? h.w : h.y};
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const float d = half_fast((hw[r >> 1] >> (16 * (r & 1))) & 0xFFFFu);
-            res = __builtin_fmaf(d, D[r], res);
-        }
+        // header: eight binary16 scales, four per k-step; the conversion rides in the multiply-add
+        // (v_fma_mix_f32 reads either half of a dword as binary16)
+        const f16x2_t s01 = __builtin_bit_cast(f16x2_t, khalf ? h.z : h.x);
+        const f16x2_t s23 = __builtin_bit_cast(f16x2_t, khalf ? h.w : h.y);
+        res = __builtin_fmaf((float)s01.x, D[0], res);
+        res = __builtin_fmaf((float)s01.y, D[1], res);
+        res = __builtin_fmaf((float)s23.x, D[2], res);
+        res = __builtin_fmaf((float)s23.y, D[3], res);
     }
     return res;
 }
@@ -156,17 +175,18 @@ __device__ unsigned long long g_trace[1024 * 16 * 8];
 #define TRACE(slot) do {} while (0)
 #endif
 
-template <int FMT>
-__global__ __launch_bounds__(1024) void gemv4_kernel(GemvArgs args, const void* __restrict__ xin) {
-    constexpr int WD = 4;  // unit fetches in flight per wavefront
+// WD = unit fetches in flight per wavefront; the first WD are requested unconditionally, so the host
+// chooses WD <= the number of units of a full wavefront (a short one re-reads a unit it never uses).
+template <int FMT, bool XF32, int WD>
+__global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin) {
     extern __shared__ uint4 smem[];
     // every kernel argument is read here, in one batch of scalar loads
     const MatrixTable mt(args);
     const int K = args.K, nslot = args.nslot, T = args.tiles_per_wg, ntiles = args.ntiles;
     const int cols_base = args.cols_base, cols_rem = args.cols_rem;
-    const bool x_f32 = args.x_f32 != 0, y_bf16 = args.y_bf16 != 0;
-    const int nr0 = args.nrows[0], nr1 = args.nrows[1], nr2 = args.nrows[2], nr3 = args.nrows[3];
-    void* const y0 = args.y[0]; void* const y1 = args.y[1]; void* const y2 = args.y[2]; void* const y3 = args.y[3];
+    const bool y_bf16 = args.y_bf16 != 0;
+    const int nr0 = args.nr0, nr1 = args.nr1, nr2 = args.nr2, nr3 = args.nr3;
+    void* const y0 = args.y0; void* const y1 = args.y1; void* const y2 = args.y2; void* const y3 = args.y3;
     asm volatile("" ::"s"(K), "s"(nslot), "s"(T), "s"(ntiles), "s"(cols_base), "s"(cols_rem), "s"(nr0), "s"(nr1),
                  "s"(nr2), "s"(nr3), "s"(y0), "s"(y1), "s"(y2), "s"(y3), "s"(xin), "s"(mt.W0), "s"(mt.W1), "s"(mt.W2),
                  "s"(mt.W3), "s"(mt.e0), "s"(mt.e1), "s"(mt.e2));
@@ -184,19 +204,28 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvArgs args, const void* 
     TRACE(0);
 
     // LDS: per wavefront and block column, A entries [nslot][2 k-steps][4 groups][4] (uint4) and
-    // group sums [4 slots][2][4] (float); then one zero A entry set, then the partial sums [T][NW][64].
+    // group sums [4 slots][2][4] (float); then one zero A entry set per wavefront, then the partial sums [T][NW][64].
     const int a_per_col = nslot * 32;                   // uint4 entries
     const int col_stride = a_per_col + 8;               // + 32 floats of group sums
     uint4* my = smem + (size_t)wave * ncols_max * col_stride;
-    uint4* zero4 = smem + (size_t)NW * ncols_max * col_stride;
-    float* part = reinterpret_cast<float*>(zero4 + 4);
+    uint4* zero4 = smem + (size_t)NW * ncols_max * col_stride + 4 * wave;  // this wavefront's own zero A entries
+    float* part = reinterpret_cast<float*>(smem + (size_t)NW * ncols_max * col_stride + 4 * NW);
 
-    // ---- this wavefront's activation slices first (tiny, and needed before any arithmetic)
-    // lane l < 32 of a pass owns the 8-element quad l of one (column, slot); a pass covers two slots
+    // ---- this wavefront's activation slices are requested first (tiny, and needed before any
+    // arithmetic), the first unit fetches right behind them, and the activations are staged while
+    // the weights are in flight.
+    // A pass covers two activation slots of one block column: lane l < 32 owns the 8-element quad l
+    // of slot s0, lane l + 32 the same quad of slot s0 + 1.
+    constexpr int XP = 4;  // passes whose loads are issued before the weight stream
     const int quad = lane & 31, sl_in_pass = lane >> 5;
-    auto x_load = [&](int ci, int s, uint4& lo, uint4& hi) {
+    const int npc = (nslot + 1) >> 1;  // passes per block column
+    const int npass = ncols * npc;
+    auto x_load = [&](int pass, uint4& lo, uint4& hi) __attribute__((always_inline)) {
+        const int ci = npc == 1 ? pass : pass >> 1;
+        const int s = (npc == 1 ? 0 : (pass & 1) * 2) + sl_in_pass;
+        if (s >= nslot) return;
         const size_t k0 = (size_t)(wave + NW * ci) * 256 + (size_t)quad * 8;
-        if (x_f32) {
+        if constexpr (XF32) {
             const uint4* xf = reinterpret_cast<const uint4*>(xin) + (((size_t)(s >> 1) * K + k0) >> 2);
             lo = xf[0];
             hi = xf[1];
@@ -204,66 +233,80 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvArgs args, const void* 
             lo = reinterpret_cast<const uint4*>(xin)[((size_t)s * K + k0) >> 3];
         }
     };
-    uint4 xlo = {0, 0, 0, 0}, xhi = {0, 0, 0, 0};
-    if (ncols > 0 && sl_in_pass < nslot) x_load(0, sl_in_pass, xlo, xhi);
+    uint4 pxlo[XP], pxhi[XP];
+#pragma unroll
+    for (int p = 0; p < XP; ++p) {
+        pxlo[p] = uint4{0, 0, 0, 0};
+        pxhi[p] = uint4{0, 0, 0, 0};
+        if (p < npass) x_load(p, pxlo[p], pxhi[p]);
+    }
     TRACE(1);
 
-    // ---- stage this wavefront's activations: bf16 in nibble-pair order, group sums beside them
-    const uint32_t ONES = 0x3F803F80u;
-    if (tid < 4) zero4[tid] = uint4{0, 0, 0, 0};
-    for (int t = 0; t < tiles_here; ++t) part[(t * NW + wave) * 64 + lane] = 0.0f;  // this wavefront's own cells
-    for (int ci = 0; ci < ncols; ++ci) {
-        uint4* col = my + (size_t)ci * col_stride;
-        float* colX = reinterpret_cast<float*>(col + a_per_col);
-        for (int s0 = 0; s0 < 4; s0 += 2) {
-            const int s = s0 + sl_in_pass;
-            float sum = 0.0f;
-            if (s < nslot) {
-                if (ci != 0 || s0 != 0) x_load(ci, s, xlo, xhi);
-                uint4 v = xlo;
-                if (x_f32) {
-                    const float f[8] = {__uint_as_float(xlo.x), __uint_as_float(xlo.y), __uint_as_float(xlo.z),
-                                        __uint_as_float(xlo.w), __uint_as_float(xhi.x), __uint_as_float(xhi.y),
-                                        __uint_as_float(xhi.z), __uint_as_float(xhi.w)};
-                    uint32_t e[8];
-#pragma unroll
-                    for (int t = 0; t < 8; ++t) {
-                        const uint32_t hb = bf16_rne(f[t]);
-                        e[t] = (s & 1) ? bf16_rne(f[t] - __uint_as_float(hb << 16)) : hb;
-                    }
-                    v.x = e[0] | (e[1] << 16); v.y = e[2] | (e[3] << 16);
-                    v.z = e[4] | (e[5] << 16); v.w = e[6] | (e[7] << 16);
-                }
-                const uint4 p = pair_permute(v);
-                col[s * 32 + quad] = p;  // quad = (k-step, group, dword) in that order
-                sum = dot2(ONES, p.x, 0.0f);
-                sum = dot2(ONES, p.y, sum);
-                sum = dot2(ONES, p.z, sum);
-                sum = dot2(ONES, p.w, sum);
-            }
-            sum = dpp_add<0xB1>(sum);  // the four dwords of a group sit in adjacent lanes
-            sum = dpp_add<0x4E>(sum);
-            if ((quad & 3) == 0) colX[s * 8 + (quad >> 2)] = sum;  // zero for unused slots
-        }
-    }
-    // ---- unit fetch cursor.  The weight stream starts only now: a vector load that hits
-    // in L2 still returns behind every older miss of the compute unit, so activations
-    // requested after the flood would arrive microseconds late
+    // ---- unit fetch cursor
     int f_ci = 0, f_t = 0;
-    auto fetch = [&](uint4& c0, uint4& c1, uint4& hd) {
+    auto fetch = [&](uint4& c0, uint4& c1, uint4& hd) __attribute__((always_inline)) {
         const int tile = tile0 + f_t;
         const int m = mt.index(tile);
         const int ltile = tile - mt.first_tile(m);
-        const uint8_t* u = mt.base(m) + ((size_t)ltile * nblocks + (size_t)(wave + NW * f_ci)) * 2304;
+        const int ci = min(f_ci, ncols - 1);  // past the end: a unit of this wavefront again, never used
+        const uint8_t* u = mt.base(m) + ((size_t)ltile * nblocks + (size_t)(wave + NW * ci)) * 2304;
         c0 = *reinterpret_cast<const uint4*>(u + 16 * lane);
         c1 = *reinterpret_cast<const uint4*>(u + 1024 + 16 * lane);
         hd = *reinterpret_cast<const uint4*>(u + 2048 + 16 * n);
         if (++f_t == tiles_here) { f_t = 0; ++f_ci; }
     };
+    // Every fetch is unconditional: the number of loads younger than any operand is then a
+    // compile-time constant, so staging waits for the activations alone and a unit is consumed as
+    // soon as IT has arrived (behind a conditional fetch the compiler waits for everything in flight).
     uint4 c0[WD], c1[WD], hd[WD];
 #pragma unroll
-    for (int u = 0; u < WD; ++u)
-        if (u < nitems) fetch(c0[u], c1[u], hd[u]);
+    for (int u = 0; u < WD; ++u) fetch(c0[u], c1[u], hd[u]);
+
+    // ---- stage this wavefront's activations: bf16 in nibble-pair order, group sums beside them
+    const uint32_t ONES = 0x3F803F80u;
+    if (lane < 4) zero4[lane] = uint4{0, 0, 0, 0};
+    for (int t = 0; t < tiles_here; ++t) part[(t * NW + wave) * 64 + lane] = 0.0f;  // this wavefront's own cells
+    auto stage = [&](int pass, uint4 xlo, uint4 xhi) __attribute__((always_inline)) {
+        const int ci = npc == 1 ? pass : pass >> 1;
+        const int s = (npc == 1 ? 0 : (pass & 1) * 2) + sl_in_pass;
+        uint4* col = my + (size_t)ci * col_stride;
+        float* colX = reinterpret_cast<float*>(col + a_per_col);
+        float sum = 0.0f;
+        if (s < nslot) {
+            uint4 v = xlo;
+            if constexpr (XF32) {
+                const float f[8] = {__uint_as_float(xlo.x), __uint_as_float(xlo.y), __uint_as_float(xlo.z),
+                                    __uint_as_float(xlo.w), __uint_as_float(xhi.x), __uint_as_float(xhi.y),
+                                    __uint_as_float(xhi.z), __uint_as_float(xhi.w)};
+                uint32_t e[8];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const uint32_t hb = bf16_rne(f[t]);
+                    e[t] = (s & 1) ? bf16_rne(f[t] - __uint_as_float(hb << 16)) : hb;
+                }
+                v.x = e[0] | (e[1] << 16); v.y = e[2] | (e[3] << 16);
+                v.z = e[4] | (e[5] << 16); v.w = e[6] | (e[7] << 16);
+            }
+            const uint4 p = pair_permute(v);
+            col[s * 32 + quad] = p;  // quad = (k-step, group, dword) in that order
+            sum = dot2(ONES, p.x, 0.0f);
+            sum = dot2(ONES, p.y, sum);
+            sum = dot2(ONES, p.z, sum);
+            sum = dot2(ONES, p.w, sum);
+        }
+        sum = dpp_add<0xB1>(sum);  // the four dwords of a group sit in adjacent lanes
+        sum = dpp_add<0x4E>(sum);
+        if ((quad & 3) == 0) colX[s * 8 + (quad >> 2)] = sum;  // zero for an unused slot of the pass
+        if (npc == 1 && (quad & 3) == 0) colX[(s + 2) * 8 + (quad >> 2)] = 0.0f;  // slots 2, 3 are never staged
+    };
+#pragma unroll
+    for (int p = 0; p < XP; ++p)
+        if (p < npass) stage(p, pxlo[p], pxhi[p]);
+    for (int p = XP; p < npass; ++p) {
+        uint4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+        x_load(p, lo, hi);
+        stage(p, lo, hi);
+    }
 
     TRACE(2);
     TRACE(3);
@@ -278,78 +321,81 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvArgs args, const void* 
     asm volatile("" : "+v"(C));  // keep the bias in a VGPR so (v & M) | C is one v_and_or_b32
     uint4 av[2][4];
     float4 xv[2];
-    f32x4_t bias[2];
     int c_ci = 0, c_t = 0;
-    for (int it0 = 0; it0 < nitems; it0 += WD) {
+    auto consume = [&](int u) __attribute__((always_inline)) {
+        if (c_t == 0) {  // new block column: its two k-steps' A fragments and group sums
+            const uint4* col = my + (size_t)c_ci * col_stride;
+            const float* colX = reinterpret_cast<const float*>(col + a_per_col);
 #pragma unroll
-        for (int u = 0; u < WD; ++u) {
-            if (it0 + u < nitems) {
-                if (c_t == 0) {  // new block column: its two k-steps' A fragments and group sums
-                    const uint4* col = my + (size_t)c_ci * col_stride;
-                    const float* colX = reinterpret_cast<const float*>(col + a_per_col);
+            for (int h = 0; h < 2; ++h) {
+                const uint4* src = a_live ? col + s_a * 32 + h * 16 + q * 4 : zero4;
 #pragma unroll
-                    for (int h = 0; h < 2; ++h) {
-                        const uint4* src = a_live ? col + s_a * 32 + h * 16 + q * 4 : zero4;
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) av[h][j] = src[j];
-                        xv[h] = *reinterpret_cast<const float4*>(colX + q * 8 + h * 4);
-                        bias[h] = accumulator_bias<FMT>(xv[h]);
-                    }
-                }
-                float res = 0.0f;
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const uint4 cw = h ? c1[u] : c0[u];
-                    const uint32_t qq[4] = {cw.x, cw.y, cw.z, cw.w};
-                    f32x4_t Dv = bias[h];
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const uint32_t v = qq[j];
-                        const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
-                        Dv = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[h][j]),
-                                                                     __builtin_bit_cast(bf16x8_t, wv), Dv, 0, 0, 0);
-                    }
-                    res += apply_groups<FMT>(hd[u], h, Dv, xv[h]);
-                }
-                float* cell = part + (c_t * NW + wave) * 64 + lane;
-                *cell += res;
-                if (it0 + u == 0) TRACE(4);
-                if (++c_t == tiles_here) { c_t = 0; ++c_ci; }
-                if (it0 + u + WD < nitems) fetch(c0[u], c1[u], hd[u]);
+                for (int j = 0; j < 4; ++j) av[h][j] = src[j];
+                xv[h] = *reinterpret_cast<const float4*>(colX + q * 8 + h * 4);
             }
         }
+        float res = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint4 cw = h ? c1[u] : c0[u];
+            const uint32_t qq[4] = {cw.x, cw.y, cw.z, cw.w};
+            f32x4_t Dv = accumulator_bias<FMT>(xv[h]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t v = qq[j];
+                const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
+                Dv = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[h][j]),
+                                                             __builtin_bit_cast(bf16x8_t, wv), Dv, 0, 0, 0);
+            }
+            res += apply_groups<FMT>(hd[u], h, Dv, xv[h]);
+        }
+        float* cell = part + (c_t * NW + wave) * 64 + lane;
+        *cell += res;
+        if (++c_t == tiles_here) { c_t = 0; ++c_ci; }
+    };
+    // Units are taken in groups of WD; only the last group can be partial.
+    const int groups = (nitems + WD - 1) / WD;
+    for (int g = 1; g < groups; ++g) {
+#pragma unroll
+        for (int u = 0; u < WD; ++u) {
+            consume(u);
+            fetch(c0[u], c1[u], hd[u]);
+        }
     }
+    TRACE(4);
+    const int last0 = (groups - 1) * WD;
+#pragma unroll
+    for (int u = 0; u < WD; ++u)
+        if (last0 + u < nitems) consume(u);
+    // ---- add the wavefronts' partials and store.  One lane per output (tile t, activation row b,
+    // weight row nn), b padded to a power of two so the split is shifts only; the lane adds the NW
+    // partials in wavefront order (deterministic).  Only as many wavefronts as there are outputs / 64
+    // run this: instructions issued by all sixteen wavefronts would cost four times as long per SIMD.
+    constexpr int rows_per_out = XF32 ? 2 : 1;  // fp32 input: high and low part live in adjacent activation rows
+    const int nb = nslot / rows_per_out;
+    const int bshift = nb > 2 ? 2 : nb - 1;  // log2 of nb rounded up to a power of two
+    const int nout = tiles_here << (4 + bshift);
     TRACE(5);
     __syncthreads();
     TRACE(6);
-
-    // ---- add the wavefronts' partials and store: 16 lanes per output, lane w reads wavefront w's
-    // cell(s), then a fixed-order DPP tree inside the 16-lane row
-    const int rows_per_out = x_f32 ? 2 : 1;  // fp32 input: high and low part live in adjacent activation rows
-    const int nb = nslot / rows_per_out;
-    const int nout = tiles_here * nb * 16;
-    for (int o = tid >> 4; o < ((nout + 63) & ~63); o += blockDim.x >> 4) {
-        const int w = tid & 15;
-        const int t = o / (nb * 16), rem = o - t * (nb * 16);
-        const int b = rem >> 4, nn = rem & 15;
+    for (int o = tid; o < nout; o += blockDim.x) {
+        const int t = o >> (4 + bshift), b = (o >> 4) & ((1 << bshift) - 1), nn = o & 15;
+        if (b >= nb) continue;
+        const float* cell = part + t * NW * 64 + b * rows_per_out * 16 + nn;
         float v = 0.0f;
-        if (o < nout && w < NW)
-            for (int h = 0; h < rows_per_out; ++h) v += part[(t * NW + w) * 64 + (b * rows_per_out + h) * 16 + nn];
-        v = dpp_add<0xB1>(v);
-        v = dpp_add<0x4E>(v);
-        v = dpp_add<0x141>(v);  // row_half_mirror
-        v = dpp_add<0x140>(v);  // row_mirror
-        if (o < nout && w == 0) {
-            const int tile = tile0 + t;
-            const int m = mt.index(tile);
-            const int row = (tile - mt.first_tile(m)) * 16 + nn;
-            const int nr = m == 0 ? nr0 : m == 1 ? nr1 : m == 2 ? nr2 : nr3;
-            void* yp = m == 0 ? y0 : m == 1 ? y1 : m == 2 ? y2 : y3;
-            if (row < nr) {
-                const size_t off = (size_t)b * (size_t)nr + (size_t)row;
-                if (y_bf16) reinterpret_cast<unsigned short*>(yp)[off] = (unsigned short)bf16_rne(v);
-                else reinterpret_cast<float*>(yp)[off] = v;
-            }
+        for (int w = 0; w < NW; ++w) {
+#pragma unroll
+            for (int h = 0; h < rows_per_out; ++h) v += cell[w * 64 + h * 16];
+        }
+        const int tile = tile0 + t;
+        const int m = mt.index(tile);
+        const int row = (tile - mt.first_tile(m)) * 16 + nn;
+        const int nr = m == 0 ? nr0 : m == 1 ? nr1 : m == 2 ? nr2 : nr3;
+        void* yp = m == 0 ? y0 : m == 1 ? y1 : m == 2 ? y2 : y3;
+        if (row < nr) {
+            const size_t off = (size_t)b * (size_t)nr + (size_t)row;
+            if (y_bf16) reinterpret_cast<unsigned short*>(yp)[off] = (unsigned short)bf16_rne(v);
+            else reinterpret_cast<float*>(yp)[off] = v;
         }
     }
     TRACE(7);
@@ -372,23 +418,30 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     a.cols_base = nblocks / NW;
     a.cols_rem = nblocks % NW;
     const int ncols_max = a.cols_base + (a.cols_rem ? 1 : 0);
-    const size_t x_bytes = ((size_t)NW * ncols_max * (a.nslot * 32 + 8) + 4) * 16;
+    const size_t x_bytes = ((size_t)NW * ncols_max * (a.nslot * 32 + 8) + 4 * NW) * 16;
     int T = (ntiles + num_cu - 1) / num_cu;
     while (T > 1 && x_bytes + (size_t)T * NW * 256 > 160 * 1024) --T;
     const size_t lds = x_bytes + (size_t)T * NW * 256;
     if (lds > 160 * 1024) return fail(TFQ_ERR_SHAPE, "gemv: K too large for the LDS activation stage");
     a.tiles_per_wg = T;
-    auto kern = gemv4_kernel<FMT>;
+    const int full_items = a.cols_base * T;  // units of a wavefront with the fewest block columns in a full workgroup
+    const int wd = full_items >= 4 ? 4 : full_items >= 2 ? 2 : 1;
+    using Kernel = void (*)(GemvKernArgs, const void*);
+    static const Kernel kernels[2][3] = {
+        {gemv4_kernel<FMT, false, 1>, gemv4_kernel<FMT, false, 2>, gemv4_kernel<FMT, false, 4>},
+        {gemv4_kernel<FMT, true, 1>, gemv4_kernel<FMT, true, 2>, gemv4_kernel<FMT, true, 4>}};
+    const int xi = a.x_f32 ? 1 : 0, wi = wd == 4 ? 2 : wd == 2 ? 1 : 0;
+    const Kernel kern = kernels[xi][wi];
     // Raise the dynamic-LDS limit once per kernel (not per launch: the call is
     // not allowed while a stream is being captured into a graph).
-    static bool lds_limit_raised = false;
-    if (!lds_limit_raised) {
+    static bool lds_limit_raised[2][3] = {};
+    if (!lds_limit_raised[xi][wi]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
-        lds_limit_raised = true;
+        lds_limit_raised[xi][wi] = true;
     }
-    hipLaunchKernelGGL(kern, dim3((ntiles + T - 1) / T), dim3(64 * NW), lds, s, a, x);
+    hipLaunchKernelGGL(kern, dim3((ntiles + T - 1) / T), dim3(64 * NW), lds, s, GemvKernArgs(a), x);
     return hip_fail(hipGetLastError(), "gemv launch");
 }
 
