@@ -40,7 +40,6 @@
 
 #include "tfq_internal.hpp"
 
-#include <cstdlib>
 
 namespace tfq {
 
@@ -78,13 +77,13 @@ __device__ __forceinline__ float dpp_add(float v) {
 }
 
 // Up to four matrices that share K and the activation rows are served by one
-// launch (q/k/v, or gate/up): their tiles are concatenated into one tile space.
+// launch (q/k/v, or gate/up).  Every workgroup works inside ONE matrix: the grid is
+// the concatenation of the matrices' workgroup ranges.
 struct GemvArgs {
     const uint8_t* W[4];  // Tiled16 buffers
     void* y[4];
-    int tile_end[4];  // cumulative tile counts, INT_MAX in unused entries
     int nrows[4];
-    int ntiles;
+    int ntiles;  // all matrices together
     int nmat;
     int K;
     int y_bf16;
@@ -94,35 +93,16 @@ struct GemvArgs {
     int cols_base, cols_rem;  // block columns per wavefront: cols_base + (wave < cols_rem)
 };
 
-// What the kernel receives: the same, flattened.  No arrays on purpose: a chain of selects over
-// array elements is folded by the optimizer into an indexed read of the argument block, which
-// costs a dependent memory access (or a private-memory copy of the block) per lookup.
+// What the kernel receives, flattened.  No arrays on purpose: a chain of selects over array
+// elements is folded by the optimizer into an indexed read of the argument block, which costs a
+// dependent memory access (or a private-memory copy of the block) per lookup.  g0..g2 are the
+// cumulative workgroup counts of matrices 0..2 (INT_MAX when unused).
 struct GemvKernArgs {
     const uint8_t *W0, *W1, *W2, *W3;
     void *y0, *y1, *y2, *y3;
-    int e0, e1, e2;
+    int g0, g1, g2;
     int nr0, nr1, nr2, nr3;
-    int ntiles, K, y_bf16, nslot, tiles_per_wg, cols_base, cols_rem;
-    explicit GemvKernArgs(const GemvArgs& a)
-        : W0(a.W[0]), W1(a.W[1]), W2(a.W[2]), W3(a.W[3]), y0(a.y[0]), y1(a.y[1]), y2(a.y[2]), y3(a.y[3]),
-          e0(a.tile_end[0]), e1(a.tile_end[1]), e2(a.tile_end[2]),
-          nr0(a.nrows[0]), nr1(a.nrows[1]), nr2(a.nrows[2]), nr3(a.nrows[3]),
-          ntiles(a.ntiles), K(a.K), y_bf16(a.y_bf16), nslot(a.nslot), tiles_per_wg(a.tiles_per_wg),
-          cols_base(a.cols_base), cols_rem(a.cols_rem) {}
-};
-
-// Matrix lookup without indexed kernel-argument reads (an indexed read is a
-// dependent scalar load from the argument segment, about a microsecond each):
-// everything is fetched once, unconditionally, and selected with compares.
-// Unused tile_end entries hold INT_MAX.
-struct MatrixTable {
-    const uint8_t* W0; const uint8_t* W1; const uint8_t* W2; const uint8_t* W3;
-    int e0, e1, e2;
-    __device__ __forceinline__ explicit MatrixTable(const GemvKernArgs& a)
-        : W0(a.W0), W1(a.W1), W2(a.W2), W3(a.W3), e0(a.e0), e1(a.e1), e2(a.e2) {}
-    __device__ __forceinline__ int index(int tile) const { return (tile >= e0) + (tile >= e1) + (tile >= e2); }
-    __device__ __forceinline__ int first_tile(int m) const { return m == 0 ? 0 : m == 1 ? e0 : m == 2 ? e1 : e2; }
-    __device__ __forceinline__ const uint8_t* base(int m) const { return m == 0 ? W0 : m == 1 ? W1 : m == 2 ? W2 : W3; }
+    int K, y_bf16, nslot, tiles_per_wg, cols_base, cols_rem;
 };
 
 // Bias that the MFMA accumulator starts from, so that it ends as the dot
@@ -180,24 +160,25 @@ __device__ unsigned long long g_trace[1024 * 16 * 8];
 template <int FMT, bool XF32, int WD>
 __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin) {
     extern __shared__ uint4 smem[];
-    // every kernel argument is read here, in one batch of scalar loads
-    const MatrixTable mt(args);
-    const int K = args.K, nslot = args.nslot, T = args.tiles_per_wg, ntiles = args.ntiles;
+    const int K = args.K, nslot = args.nslot, T = args.tiles_per_wg;
     const int cols_base = args.cols_base, cols_rem = args.cols_rem;
     const bool y_bf16 = args.y_bf16 != 0;
-    const int nr0 = args.nr0, nr1 = args.nr1, nr2 = args.nr2, nr3 = args.nr3;
-    void* const y0 = args.y0; void* const y1 = args.y1; void* const y2 = args.y2; void* const y3 = args.y3;
-    asm volatile("" ::"s"(K), "s"(nslot), "s"(T), "s"(ntiles), "s"(cols_base), "s"(cols_rem), "s"(nr0), "s"(nr1),
-                 "s"(nr2), "s"(nr3), "s"(y0), "s"(y1), "s"(y2), "s"(y3), "s"(xin), "s"(mt.W0), "s"(mt.W1), "s"(mt.W2),
-                 "s"(mt.W3), "s"(mt.e0), "s"(mt.e1), "s"(mt.e2));
+
+    // ---- this workgroup's matrix, selected once with compares
+    const int bid = blockIdx.x;
+    const int m = (bid >= args.g0) + (bid >= args.g1) + (bid >= args.g2);
+    const int wg_first = m == 0 ? 0 : m == 1 ? args.g0 : m == 2 ? args.g1 : args.g2;
+    const uint8_t* Wm = m == 0 ? args.W0 : m == 1 ? args.W1 : m == 2 ? args.W2 : args.W3;
+    void* const ym = m == 0 ? args.y0 : m == 1 ? args.y1 : m == 2 ? args.y2 : args.y3;
+    const int nrm = m == 0 ? args.nr0 : m == 1 ? args.nr1 : m == 2 ? args.nr2 : args.nr3;
 
     const int nblocks = K >> 8;
     const int NW = blockDim.x >> 6;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, q = lane >> 4;
-    const int tile0 = blockIdx.x * T;
-    const int tiles_here = min(T, ntiles - tile0);
+    const int tile0 = (bid - wg_first) * T;              // inside the matrix
+    const int tiles_here = min(T, ((nrm + 15) >> 4) - tile0);
     const int ncols = cols_base + (wave < cols_rem ? 1 : 0);  // block columns wave, wave + NW, ...
     const int ncols_max = cols_base + (cols_rem ? 1 : 0);
     const int nitems = ncols * tiles_here;  // block-column major, tiles inside
@@ -215,23 +196,25 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     // arithmetic), the first unit fetches right behind them, and the activations are staged while
     // the weights are in flight.
     // A pass covers two activation slots of one block column: lane l < 32 owns the 8-element quad l
-    // of slot s0, lane l + 32 the same quad of slot s0 + 1.
+    // of slot s0, lane l + 32 the same quad of slot s0 + 1 (clamped to the last slot: the load is
+    // unconditional and staging drops what it does not need).
     constexpr int XP = 4;  // passes whose loads are issued before the weight stream
     const int quad = lane & 31, sl_in_pass = lane >> 5;
     const int npc = (nslot + 1) >> 1;  // passes per block column
     const int npass = ncols * npc;
+    constexpr int XE = XF32 ? 4 : 2;   // bytes per activation element
+    const uint8_t* xbytes = static_cast<const uint8_t*>(xin);
+    // per-lane byte offset inside a pass, and the per-pass scalar offset
     auto x_load = [&](int pass, uint4& lo, uint4& hi) __attribute__((always_inline)) {
         const int ci = npc == 1 ? pass : pass >> 1;
-        const int s = (npc == 1 ? 0 : (pass & 1) * 2) + sl_in_pass;
-        if (s >= nslot) return;
-        const size_t k0 = (size_t)(wave + NW * ci) * 256 + (size_t)quad * 8;
-        if constexpr (XF32) {
-            const uint4* xf = reinterpret_cast<const uint4*>(xin) + (((size_t)(s >> 1) * K + k0) >> 2);
-            lo = xf[0];
-            hi = xf[1];
-        } else {
-            lo = reinterpret_cast<const uint4*>(xin)[((size_t)s * K + k0) >> 3];
-        }
+        const int s0 = npc == 1 ? 0 : (pass & 1) * 2;
+        const int s = min(s0 + sl_in_pass, nslot - 1);
+        const int row = XF32 ? s >> 1 : s;
+        const uint32_t lane_off = ((uint32_t)row * (uint32_t)K + (uint32_t)quad * 8u) * XE;
+        const uint8_t* base = xbytes + (size_t)(wave + NW * ci) * (256 * XE);
+        const uint4* src = reinterpret_cast<const uint4*>(base + lane_off);
+        lo = src[0];
+        if constexpr (XF32) hi = src[1];
     };
     uint4 pxlo[XP], pxhi[XP];
 #pragma unroll
@@ -242,22 +225,28 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     }
     TRACE(1);
 
-    // ---- unit fetch cursor
+    // ---- unit fetch cursor: a pointer that walks the tiles of a block column, then moves to the
+    // wavefront's next column.  Past the end it keeps walking the last column again (valid units
+    // of this wavefront, cache hits, never used): every fetch is unconditional, so the number of
+    // loads younger than any operand is a compile-time constant, staging waits for the
+    // activations alone and a unit is consumed as soon as IT has arrived (behind a conditional
+    // fetch the compiler waits for everything in flight).
+    const size_t tile_stride = (size_t)nblocks * 2304;
+    const uint8_t* col_ptr = Wm + ((size_t)tile0 * nblocks + (size_t)wave) * 2304;
+    const uint8_t* f_ptr = col_ptr;
     int f_ci = 0, f_t = 0;
+    const uint32_t off_c = 16u * lane, off_h = 2048u + 16u * n;
     auto fetch = [&](uint4& c0, uint4& c1, uint4& hd) __attribute__((always_inline)) {
-        const int tile = tile0 + f_t;
-        const int m = mt.index(tile);
-        const int ltile = tile - mt.first_tile(m);
-        const int ci = min(f_ci, ncols - 1);  // past the end: a unit of this wavefront again, never used
-        const uint8_t* u = mt.base(m) + ((size_t)ltile * nblocks + (size_t)(wave + NW * ci)) * 2304;
-        c0 = *reinterpret_cast<const uint4*>(u + 16 * lane);
-        c1 = *reinterpret_cast<const uint4*>(u + 1024 + 16 * lane);
-        hd = *reinterpret_cast<const uint4*>(u + 2048 + 16 * n);
-        if (++f_t == tiles_here) { f_t = 0; ++f_ci; }
+        c0 = *reinterpret_cast<const uint4*>(f_ptr + off_c);
+        c1 = *reinterpret_cast<const uint4*>(f_ptr + off_c + 1024);
+        hd = *reinterpret_cast<const uint4*>(f_ptr + off_h);
+        f_ptr += tile_stride;
+        if (++f_t == tiles_here) {
+            f_t = 0;
+            if (++f_ci < ncols) col_ptr += (size_t)NW * 2304;
+            f_ptr = col_ptr;
+        }
     };
-    // Every fetch is unconditional: the number of loads younger than any operand is then a
-    // compile-time constant, so staging waits for the activations alone and a unit is consumed as
-    // soon as IT has arrived (behind a conditional fetch the compiler waits for everything in flight).
     uint4 c0[WD], c1[WD], hd[WD];
 #pragma unroll
     for (int u = 0; u < WD; ++u) fetch(c0[u], c1[u], hd[u]);
@@ -265,7 +254,6 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     // ---- stage this wavefront's activations: bf16 in nibble-pair order, group sums beside them
     const uint32_t ONES = 0x3F803F80u;
     if (lane < 4) zero4[lane] = uint4{0, 0, 0, 0};
-    for (int t = 0; t < tiles_here; ++t) part[(t * NW + wave) * 64 + lane] = 0.0f;  // this wavefront's own cells
     auto stage = [&](int pass, uint4 xlo, uint4 xhi) __attribute__((always_inline)) {
         const int ci = npc == 1 ? pass : pass >> 1;
         const int s = (npc == 1 ? 0 : (pass & 1) * 2) + sl_in_pass;
@@ -307,7 +295,6 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
         x_load(p, lo, hi);
         stage(p, lo, hi);
     }
-
     TRACE(2);
     TRACE(3);
 
@@ -321,7 +308,9 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     asm volatile("" : "+v"(C));  // keep the bias in a VGPR so (v & M) | C is one v_and_or_b32
     uint4 av[2][4];
     float4 xv[2];
+    f32x4_t bias[2];
     int c_ci = 0, c_t = 0;
+    float* cell = part + wave * 64 + lane;  // this wavefront's cell of tile c_t
     auto consume = [&](int u) __attribute__((always_inline)) {
         if (c_t == 0) {  // new block column: its two k-steps' A fragments and group sums
             const uint4* col = my + (size_t)c_ci * col_stride;
@@ -332,6 +321,7 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
 #pragma unroll
                 for (int j = 0; j < 4; ++j) av[h][j] = src[j];
                 xv[h] = *reinterpret_cast<const float4*>(colX + q * 8 + h * 4);
+                bias[h] = accumulator_bias<FMT>(xv[h]);
             }
         }
         float res = 0.0f;
@@ -339,7 +329,7 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
         for (int h = 0; h < 2; ++h) {
             const uint4 cw = h ? c1[u] : c0[u];
             const uint32_t qq[4] = {cw.x, cw.y, cw.z, cw.w};
-            f32x4_t Dv = accumulator_bias<FMT>(xv[h]);
+            f32x4_t Dv = bias[h];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t v = qq[j];
@@ -349,9 +339,11 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
             }
             res += apply_groups<FMT>(hd[u], h, Dv, xv[h]);
         }
-        float* cell = part + (c_t * NW + wave) * 64 + lane;
-        *cell += res;
-        if (++c_t == tiles_here) { c_t = 0; ++c_ci; }
+        // the first block column writes the cell, later ones add to it (no zero fill, no read)
+        if (c_ci == 0) *cell = res;
+        else *cell += res;
+        cell += NW * 64;
+        if (++c_t == tiles_here) { c_t = 0; ++c_ci; cell = part + wave * 64 + lane; }
     };
     // Units are taken in groups of WD; only the last group can be partial.
     const int groups = (nitems + WD - 1) / WD;
@@ -367,6 +359,7 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
 #pragma unroll
     for (int u = 0; u < WD; ++u)
         if (last0 + u < nitems) consume(u);
+
     // ---- add the wavefronts' partials and store.  One lane per output (tile t, activation row b,
     // weight row nn), b padded to a power of two so the split is shifts only; the lane adds the NW
     // partials in wavefront order (deterministic).  Only as many wavefronts as there are outputs / 64
@@ -380,32 +373,25 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     TRACE(6);
     for (int o = tid; o < nout; o += blockDim.x) {
         const int t = o >> (4 + bshift), b = (o >> 4) & ((1 << bshift) - 1), nn = o & 15;
-        if (b >= nb) continue;
-        const float* cell = part + t * NW * 64 + b * rows_per_out * 16 + nn;
+        const int row = (tile0 + t) * 16 + nn;
+        if (b >= nb || row >= nrm) continue;
+        const float* src = part + t * NW * 64 + b * rows_per_out * 16 + nn;
         float v = 0.0f;
         for (int w = 0; w < NW; ++w) {
 #pragma unroll
-            for (int h = 0; h < rows_per_out; ++h) v += cell[w * 64 + h * 16];
+            for (int h = 0; h < rows_per_out; ++h) v += src[w * 64 + h * 16];
         }
-        const int tile = tile0 + t;
-        const int m = mt.index(tile);
-        const int row = (tile - mt.first_tile(m)) * 16 + nn;
-        const int nr = m == 0 ? nr0 : m == 1 ? nr1 : m == 2 ? nr2 : nr3;
-        void* yp = m == 0 ? y0 : m == 1 ? y1 : m == 2 ? y2 : y3;
-        if (row < nr) {
-            const size_t off = (size_t)b * (size_t)nr + (size_t)row;
-            if (y_bf16) reinterpret_cast<unsigned short*>(yp)[off] = (unsigned short)bf16_rne(v);
-            else reinterpret_cast<float*>(yp)[off] = v;
-        }
+        const size_t off = (size_t)b * (size_t)nrm + (size_t)row;
+        if (y_bf16) reinterpret_cast<unsigned short*>(ym)[off] = (unsigned short)bf16_rne(v);
+        else reinterpret_cast<float*>(ym)[off] = v;
     }
     TRACE(7);
 }
 
 template <int FMT>
 int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
-    const int ntiles = a.ntiles;
     const int nblocks = a.K >> 8;
-    static const int num_cu = [] { const char* e = getenv("TFQ_GEMV_WGS"); return e ? atoi(e) : 256; }();
+    constexpr int num_cu = 256;  // compute units of an MI355X
     // wavefronts per workgroup: the count in 8..16 that splits the block columns most evenly
     int NW = nblocks < 16 ? nblocks : 16;
     if (nblocks > 16) {
@@ -419,11 +405,31 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     a.cols_rem = nblocks % NW;
     const int ncols_max = a.cols_base + (a.cols_rem ? 1 : 0);
     const size_t x_bytes = ((size_t)NW * ncols_max * (a.nslot * 32 + 8) + 4 * NW) * 16;
-    int T = (ntiles + num_cu - 1) / num_cu;
+    if (x_bytes + (size_t)NW * 256 > 160 * 1024) return fail(TFQ_ERR_SHAPE, "gemv: K too large for the LDS activation stage");
+    // tiles per workgroup: one round of workgroups over the compute units where LDS allows it;
+    // every workgroup stays inside one matrix
+    auto grid_for = [&](int T) {
+        int g = 0;
+        for (int m = 0; m < a.nmat; ++m) g += ((a.nrows[m] + 15) / 16 + T - 1) / T;
+        return g;
+    };
+    int T = (a.ntiles + num_cu - 1) / num_cu;
+    while (grid_for(T) > num_cu && x_bytes + (size_t)(T + 1) * NW * 256 <= 160 * 1024) ++T;
     while (T > 1 && x_bytes + (size_t)T * NW * 256 > 160 * 1024) --T;
     const size_t lds = x_bytes + (size_t)T * NW * 256;
-    if (lds > 160 * 1024) return fail(TFQ_ERR_SHAPE, "gemv: K too large for the LDS activation stage");
     a.tiles_per_wg = T;
+    GemvKernArgs k{};
+    k.W0 = a.W[0]; k.W1 = a.W[1]; k.W2 = a.W[2]; k.W3 = a.W[3];
+    k.y0 = a.y[0]; k.y1 = a.y[1]; k.y2 = a.y[2]; k.y3 = a.y[3];
+    k.nr0 = a.nrows[0]; k.nr1 = a.nrows[1]; k.nr2 = a.nrows[2]; k.nr3 = a.nrows[3];
+    int ends[3], g = 0;
+    for (int m = 0; m < 3; ++m) {
+        if (m < a.nmat) g += ((a.nrows[m] + 15) / 16 + T - 1) / T;
+        ends[m] = m < a.nmat ? g : 0x7FFFFFFF;
+    }
+    k.g0 = ends[0]; k.g1 = ends[1]; k.g2 = ends[2];
+    k.K = a.K; k.y_bf16 = a.y_bf16; k.nslot = a.nslot; k.tiles_per_wg = T;
+    k.cols_base = a.cols_base; k.cols_rem = a.cols_rem;
     const int full_items = a.cols_base * T;  // units of a wavefront with the fewest block columns in a full workgroup
     const int wd = full_items >= 4 ? 4 : full_items >= 2 ? 2 : 1;
     using Kernel = void (*)(GemvKernArgs, const void*);
@@ -441,7 +447,7 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
         lds_limit_raised[xi][wi] = true;
     }
-    hipLaunchKernelGGL(kern, dim3((ntiles + T - 1) / T), dim3(64 * NW), lds, s, GemvKernArgs(a), x);
+    hipLaunchKernelGGL(kern, dim3(grid_for(T)), dim3(64 * NW), lds, s, k, x);
     return hip_fail(hipGetLastError(), "gemv launch");
 }
 
@@ -483,13 +489,11 @@ int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int 
         if (tiles > 0x7FFFFFF || ws[m]->N > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "gemv: too many rows");
         a.W[m] = ws[m]->dev;
         a.y[m] = ys[m];
-        a.tile_end[m] = (int)tiles;
         a.nrows[m] = (int)ws[m]->N;
     }
     for (int m = nmat; m < 4; ++m) {
         a.W[m] = a.W[0];
         a.y[m] = a.y[0];
-        a.tile_end[m] = 0x7FFFFFFF;
     }
     a.ntiles = (int)tiles;
     a.nmat = nmat;
