@@ -5,21 +5,20 @@
 //
 // A workgroup of 8 wavefronts owns a 256 x 128 output tile and walks K in steps
 // of 32 (one scale group per weight row).  Per step it
-//   * copies the 256 x 32 activation tile to LDS (bf16, each run of 8 stored in
-//     the nibble-pair order (x0,x4)(x1,x5)(x2,x6)(x3,x7)),
+//   * copies the 256 x 32 activation tile to LDS (bf16),
 //   * decodes the 128 x 32 weight tile: one lane takes one code dword (8 weights),
-//     turns the nibbles into bf16 128+n by OR-ing 0x4300 into masked nibble
-//     pairs, applies the group's scale and offset in fp32
-//         w = a * (128+n) + (c - 128 a),   (a, c) = (d, -8d) or (d*sc/15, -dm*mc)
-//     rounds to bf16 (v_cvt_pk_bf16_f32) and stores the 8 weights to LDS in the
-//     same order,
+//     converts the nibbles with v_cvt_f32_ubyte, applies the group's scale and
+//     offset in fp32
+//         w = a * n + c,   (a, c) = (d, -8d) or (d*sc/15, -dm*mc)
+//     packs to bf16 (v_cvt_pk_bf16_f32) and stores the 8 weights to LDS,
 //   * runs 16 v_mfma_f32_16x16x32_bf16 per wavefront (a 64 x 64 sub-tile).
-// The next step's global loads are issued before the current step's MFMAs, so
-// HBM / L2 latency overlaps with arithmetic.  Weights are read from the
+// Global loads run three steps ahead of their use in a ring of four register
+// sets (a step's loads have two full steps to arrive before they are written
+// to LDS), so HBM / L2 latency overlaps with arithmetic.  Weights are read from the
 // Tiled16 layout, where the 16 rows of a tile hold a group as 256 contiguous bytes.
-// Workgroups are numbered so that the 8 row-tiles of one 128-column strip run on
-// the same XCD back to back: the strip's packed weights are fetched from HBM
-// once and then served from that XCD's L2.
+// Workgroups are numbered so that the ones running together on an XCD share a
+// token tile: the activations, the larger operand by bytes, are then served from
+// that XCD's L2 and only the packed weights stream from HBM.
 
 #include "tfq_internal.hpp"
 
@@ -29,6 +28,9 @@ namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
 
 constexpr int BM = 256, BN = 128, BK = 32, THREADS = 512;
 
@@ -37,20 +39,31 @@ __device__ __forceinline__ uint32_t bf16_rne(float f) {
     return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
 }
 
-__device__ __forceinline__ uint4 pair_permute(uint4 v) {
-    uint4 p;
-    p.x = (v.x & 0xFFFFu) | (v.z << 16);
-    p.y = (v.x >> 16) | (v.z & 0xFFFF0000u);
-    p.z = (v.y & 0xFFFFu) | (v.w << 16);
-    p.w = (v.y >> 16) | (v.w & 0xFFFF0000u);
-    return p;
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
 }
 
-// two bf16 (128+n) in one dword -> two scaled weights, rounded to bf16
-__device__ __forceinline__ uint32_t scale_pair(uint32_t pair, float a, float c) {
-    const float lo = __builtin_fmaf(a, __uint_as_float(pair << 16), c);
-    const float hi = __builtin_fmaf(a, __uint_as_float(pair & 0xFFFF0000u), c);
-    return bf16_rne(lo) | (bf16_rne(hi) << 16);
+// byte B of a dword as float (v_cvt_f32_ubyteB); written as an instruction because the optimizer
+// otherwise rebuilds every nibble with a bit-field extract of its own, two operations per weight
+template <int B>
+__device__ __forceinline__ float ubyte_to_float(uint32_t v) {
+    float f;
+    if constexpr (B == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(v));
+    else if constexpr (B == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(v));
+    else if constexpr (B == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(v));
+    else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(v));
+    return f;
+}
+
+// one code dword (nibble t = weight t) -> eight bf16 weights in k order: 3 + 8 + 8 + 4 operations
+__device__ __forceinline__ uint4 decode8(uint32_t v, float a, float c) {
+    const uint32_t ev = v & 0x0F0F0F0Fu, od = (v >> 4) & 0x0F0F0F0Fu;  // nibbles 0,2,4,6 / 1,3,5,7 as bytes
+    uint4 o;
+    o.x = pack_bf16(__builtin_fmaf(a, ubyte_to_float<0>(ev), c), __builtin_fmaf(a, ubyte_to_float<0>(od), c));
+    o.y = pack_bf16(__builtin_fmaf(a, ubyte_to_float<1>(ev), c), __builtin_fmaf(a, ubyte_to_float<1>(od), c));
+    o.z = pack_bf16(__builtin_fmaf(a, ubyte_to_float<2>(ev), c), __builtin_fmaf(a, ubyte_to_float<2>(od), c));
+    o.w = pack_bf16(__builtin_fmaf(a, ubyte_to_float<3>(ev), c), __builtin_fmaf(a, ubyte_to_float<3>(od), c));
+    return o;
 }
 
 struct GemmArgs {
@@ -62,7 +75,7 @@ struct GemmArgs {
     int tiles_m, tiles_n;
 };
 
-// (a, c) of group g (0..7) of a block from its 16-byte header
+// (a, c) of group g (0..7) of a block from its 16-byte header: weight = a * code + c
 template <int FMT>
 __device__ __forceinline__ void group_coeffs(uint4 h, int g, float& a, float& c) {
     if constexpr (FMT == TFQ_Q_G_4) {
@@ -71,11 +84,11 @@ __device__ __forceinline__ void group_coeffs(uint4 h, int g, float& a, float& c)
         const float sc = (float)(uint32_t)((scs >> (6 * g)) & 63u);
         const float mc = (float)((int)((mcs >> (6 * g)) & 63u) - 32);
         a = half_fast(h.w & 0xFFFFu) * sc * (1.0f / 15.0f);
-        c = __builtin_fmaf(-128.0f, a, -(half_fast(h.w >> 16) * mc));
+        c = -(half_fast(h.w >> 16) * mc);
     } else {
         const uint32_t hw[4] = {h.x, h.y, h.z, h.w};
         a = half_fast((hw[g >> 1] >> (16 * (g & 1))) & 0xFFFFu);
-        c = -136.0f * a;
+        c = -8.0f * a;
     }
 }
 
@@ -85,51 +98,58 @@ __global__ __launch_bounds__(THREADS) void gemm4_kernel(GemmArgs args) {
     __shared__ uint4 wsm[2][BN * 4];
     const int M = args.M, N = args.N, K = args.K;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    // workgroup -> (column strip, row tile): strips are dealt to XCDs, row tiles of a strip run consecutively
+    // workgroup -> (token tile, weight strip).  Workgroups are dealt to the 8 XCDs round robin, and the
+    // activation tile is the big operand of a step (16 KB against 2.3 KB of packed weights), so each
+    // XCD is given a contiguous run of the token-tile-major work list: the workgroups that run
+    // together on an XCD walk the same 256 token rows and share them through that XCD's L2, while
+    // the packed weight strips stream from HBM.
     const int wg = blockIdx.x;
     const int xcd = wg & 7, slot = wg >> 3;
-    const int strips_per_xcd = (args.tiles_n + 7) >> 3;
-    const int strip = xcd * strips_per_xcd + slot / args.tiles_m;
-    const int tm = slot % args.tiles_m;
-    if (strip >= args.tiles_n) return;
+    const int items = args.tiles_m * args.tiles_n;
+    const int per_xcd = (items + 7) >> 3;
+    const int item = xcd * per_xcd + slot;
+    if (item >= items) return;
+    const int tm = item / args.tiles_n, strip = item - tm * args.tiles_n;
     const int m0 = tm * BM, n0 = strip * BN;
     const int nblocks = K >> 8;
     const int ntiles16 = (N + 15) >> 4;
 
     // ---- global -> register stage of one k-step
     // activations: thread handles (row, 16-byte segment) pairs idx = tid and tid + 512
-    const int xr0 = tid >> 2, xseg = tid & 3;
+    // LDS tiles are stored as [row / 8][16-byte segment][row % 8]: the 8 lanes that an LDS access
+    // serves together (consecutive rows, same segment) then touch 128 consecutive bytes, all banks
+    // once; with plain [row][segment] rows 64 bytes apart they would share banks four ways.
+    // Threads are matched to (row, segment) so that their writes follow the same rule.
+    auto lds_index = [](int row, int seg) { return ((row >> 3) << 5) + (seg << 3) + (row & 7); };
+    const int xr0 = (tid & 7) + ((tid >> 5) << 3), xseg = (tid >> 3) & 3;
     const unsigned short* xp0 = args.X + (size_t)min(m0 + xr0, M - 1) * K + xseg * 8;
     const unsigned short* xp1 = args.X + (size_t)min(m0 + xr0 + 128, M - 1) * K + xseg * 8;
     // weights: thread handles code dword j of row wr of the strip
-    const int wr = tid >> 2, wj = tid & 3;
+    const int wr = xr0, wj = xseg;
     const int wtile = min((n0 + wr) >> 4, ntiles16 - 1), wn = (n0 + wr) & 15;
     const uint8_t* wbase = args.W + (size_t)wtile * nblocks * 2304;
 
-    uint4 gx0, gx1, hdr = {0, 0, 0, 0};
-    uint32_t gw;
-    auto load_step = [&](int ks) {  // ks = K offset / 32
-        gx0 = *reinterpret_cast<const uint4*>(xp0 + (size_t)ks * BK);
-        gx1 = *reinterpret_cast<const uint4*>(xp1 + (size_t)ks * BK);
+    // ring of four register sets: set r holds the loads of a step with ks % 4 == r
+    uint4 rx0[4], rx1[4];
+    uint32_t rw[4];
+    uint4 hdr = {0, 0, 0, 0}, hnext = {0, 0, 0, 0};
+    const int nsteps = K / BK;
+    auto load_step = [&](int ks_, uint4& x0, uint4& x1, uint32_t& w) __attribute__((always_inline)) {  // ks = K offset / 32
+        const int ks = min(ks_, nsteps - 1);  // past the end: the last step again, no branch
+        x0 = *reinterpret_cast<const uint4*>(xp0 + (size_t)ks * BK);
+        x1 = *reinterpret_cast<const uint4*>(xp1 + (size_t)ks * BK);
         const int blk = ks >> 3, g = ks & 7;
         const uint8_t* unit = wbase + (size_t)blk * 2304;
-        gw = *reinterpret_cast<const uint32_t*>(unit + (g >> 2) * 1024 + (wn + 16 * (g & 3)) * 16 + 4 * wj);
-        if (g == 0) hdr = *reinterpret_cast<const uint4*>(unit + 2048 + 16 * wn);
+        w = *reinterpret_cast<const uint32_t*>(unit + (g >> 2) * 1024 + (wn + 16 * (g & 3)) * 16 + 4 * wj);
+        if (g == 0) hnext = *reinterpret_cast<const uint4*>(unit + 2048 + 16 * wn);
     };
-    const uint32_t MK = 0x000F000Fu;
-    uint32_t C = 0x43004300u;
-    asm volatile("" : "+v"(C));
-    auto store_step = [&](int buf, int ks) {
-        xs[buf][xr0 * 4 + xseg] = pair_permute(gx0);
-        xs[buf][(xr0 + 128) * 4 + xseg] = pair_permute(gx1);
+    auto store_step = [&](int buf, int ks, uint4 x0, uint4 x1, uint32_t w) __attribute__((always_inline)) {
+        xs[buf][lds_index(xr0, xseg)] = x0;
+        xs[buf][lds_index(xr0 + 128, xseg)] = x1;
+        if ((ks & 7) == 0) hdr = hnext;
         float a, c;
         group_coeffs<FMT>(hdr, ks & 7, a, c);
-        uint4 o;
-        o.x = scale_pair((gw & MK) | C, a, c);
-        o.y = scale_pair(((gw >> 4) & MK) | C, a, c);
-        o.z = scale_pair(((gw >> 8) & MK) | C, a, c);
-        o.w = scale_pair(((gw >> 12) & MK) | C, a, c);
-        wsm[buf][wr * 4 + wj] = o;
+        wsm[buf][lds_index(wr, wj)] = decode8(w, a, c);
     };
 
     // wavefront sub-tile: 4 (M) x 2 (N) wavefronts, each 64 x 64 = 4 x 4 MFMA tiles
@@ -141,26 +161,30 @@ __global__ __launch_bounds__(THREADS) void gemm4_kernel(GemmArgs args) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    const int nsteps = K / BK;
-    load_step(0);
-    store_step(0, 0);
+    load_step(0, rx0[0], rx1[0], rw[0]);
+    load_step(1, rx0[1], rx1[1], rw[1]);
+    load_step(2, rx0[2], rx1[2], rw[2]);
+    store_step(0, 0, rx0[0], rx1[0], rw[0]);
     __syncthreads();
-    for (int ks = 0; ks < nsteps; ++ks) {
-        const int buf = ks & 1;
-        if (ks + 1 < nsteps) load_step(ks + 1);
-        uint4 af[4], bfr[4];
+    for (int ks0 = 0; ks0 < nsteps; ks0 += 4) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) af[i] = xs[buf][(wm * 64 + i * 16 + fr) * 4 + fk];
+        for (int u = 0; u < 4; ++u) {
+            const int ks = ks0 + u, buf = u & 1;
+            load_step(ks + 3, rx0[(u + 3) & 3], rx1[(u + 3) & 3], rw[(u + 3) & 3]);
+            uint4 af[4], bfr[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) bfr[j] = wsm[buf][(wn_ * 64 + j * 16 + fr) * 4 + fk];
+            for (int i = 0; i < 4; ++i) af[i] = xs[buf][lds_index(wm * 64 + i * 16 + fr, fk)];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+            for (int j = 0; j < 4; ++j) bfr[j] = wsm[buf][lds_index(wn_ * 64 + j * 16 + fr, fk)];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[i]),
-                                                                    __builtin_bit_cast(bf16x8_t, bfr[j]), acc[i][j], 0, 0, 0);
-        if (ks + 1 < nsteps) store_step(buf ^ 1, ks + 1);
-        __syncthreads();
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[i]),
+                                                                        __builtin_bit_cast(bf16x8_t, bfr[j]), acc[i][j], 0, 0, 0);
+            store_step(buf ^ 1, ks + 1, rx0[(u + 1) & 3], rx1[(u + 1) & 3], rw[(u + 1) & 3]);  // past the end: written, never read
+            __syncthreads();
+        }
     }
 
     // ---- store: lane holds column fr, rows 4 fk + r of each 16 x 16 tile
@@ -193,8 +217,7 @@ int run(const tfq_weight* w, const void* x, int M, void* y, int yd, hipStream_t 
     a.y_bf16 = yd == TFQ_BF16;
     a.tiles_m = (M + BM - 1) / BM;
     a.tiles_n = (a.N + BN - 1) / BN;
-    const int strips_per_xcd = (a.tiles_n + 7) / 8;
-    const int grid = 8 * strips_per_xcd * a.tiles_m;
+    const int grid = 8 * ((a.tiles_m * a.tiles_n + 7) / 8);
     hipLaunchKernelGGL(gemm4_kernel<FMT>, dim3(grid), dim3(THREADS), 0, s, a);
     return hip_fail(hipGetLastError(), "gemm launch");
 }
