@@ -3,15 +3,16 @@
 // Replaces Qwen35Engine::gemm on the prefill path, which the reference runs in
 // chunks of 512 rows (src/adapters/tools/qwen35_engine.cpp:54-101, :681-686).
 //
-// A workgroup of 8 wavefronts owns a 256 x 128 output tile and walks K in steps
+// A workgroup of 8 wavefronts owns a 256 x 256 output tile and walks K in steps
 // of 32 (one scale group per weight row).  Per step it
 //   * copies the 256 x 32 activation tile to LDS (bf16),
-//   * decodes the 128 x 32 weight tile: one lane takes one code dword (8 weights),
+//   * decodes the 256 x 32 weight tile: one lane takes two code dwords (8 weights each),
 //     converts the nibbles with v_cvt_f32_ubyte, applies the group's scale and
 //     offset in fp32
 //         w = a * n + c,   (a, c) = (d, -8d) or (d*sc/15, -dm*mc)
 //     packs to bf16 (v_cvt_pk_bf16_f32) and stores the 8 weights to LDS,
-//   * runs 16 v_mfma_f32_16x16x32_bf16 per wavefront (a 64 x 64 sub-tile).
+//   * runs 32 v_mfma_f32_16x16x32_bf16 per wavefront (a 128 x 64 sub-tile: LDS reads per MFMA
+//     are what bounds this kernel, and they shrink with the sub-tile's size).
 // Global loads run three steps ahead of their use in a ring of four register
 // sets (a step's loads have two full steps to arrive before they are written
 // to LDS), so HBM / L2 latency overlaps with arithmetic.  Weights are read from the
@@ -32,7 +33,7 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
 
-constexpr int BM = 256, BN = 128, BK = 32, THREADS = 512;
+constexpr int BM = 256, BK = 32, THREADS = 512;  // the weight-strip width BN (256 or 128) is a template parameter
 
 __device__ __forceinline__ uint32_t bf16_rne(float f) {
     const uint32_t u = __float_as_uint(f);
@@ -92,10 +93,14 @@ __device__ __forceinline__ void group_coeffs(uint4 h, int g, float& a, float& c)
     }
 }
 
-template <int FMT>
+template <int FMT, int BN>
 __global__ __launch_bounds__(THREADS) void gemm4_kernel(GemmArgs args) {
-    __shared__ uint4 xs[2][BM * 4];  // [buf][row][4 x 16 B]
-    __shared__ uint4 wsm[2][BN * 4];
+    constexpr int WROWS = BN / 128;      // weight rows decoded per thread and step
+    constexpr int MI = BN == 256 ? 8 : 4;  // 16-row token fragments per wavefront: sub-tile 128 x 64 or 64 x 64
+    // activations: four buffers of a 256 x 32 bf16 step (copied three steps ahead); weights: two buffers
+    extern __shared__ uint4 smem[];
+    uint4* const xs = smem;                 // [4][BM * 4]
+    uint4* const wsm = smem + 4 * BM * 4;   // [2][BN * 4]
     const int M = args.M, N = args.N, K = args.K;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // workgroup -> (token tile, weight strip).  Workgroups are dealt to the 8 XCDs round robin, and the
@@ -124,78 +129,108 @@ __global__ __launch_bounds__(THREADS) void gemm4_kernel(GemmArgs args) {
     const int xr0 = (tid & 7) + ((tid >> 5) << 3), xseg = (tid >> 3) & 3;
     const unsigned short* xp0 = args.X + (size_t)min(m0 + xr0, M - 1) * K + xseg * 8;
     const unsigned short* xp1 = args.X + (size_t)min(m0 + xr0 + 128, M - 1) * K + xseg * 8;
-    // weights: thread handles code dword j of row wr of the strip
+    // weights: thread handles code dword j of rows wr and wr + 128 of the strip (same row inside their 16-row tiles)
     const int wr = xr0, wj = xseg;
-    const int wtile = min((n0 + wr) >> 4, ntiles16 - 1), wn = (n0 + wr) & 15;
-    const uint8_t* wbase = args.W + (size_t)wtile * nblocks * 2304;
+    const int wn = (n0 + wr) & 15;
+    const uint8_t* wbase0 = args.W + (size_t)min((n0 + wr) >> 4, ntiles16 - 1) * nblocks * 2304;
+    const uint8_t* wbase1 = args.W + (size_t)min((n0 + wr + (WROWS - 1) * 128) >> 4, ntiles16 - 1) * nblocks * 2304;
 
     // ring of four register sets: set r holds the loads of a step with ks % 4 == r
-    uint4 rx0[4], rx1[4];
-    uint32_t rw[4];
-    uint4 hdr = {0, 0, 0, 0}, hnext = {0, 0, 0, 0};
+    uint32_t rw0[4], rw1[4];
+    uint4 hdr0 = {0, 0, 0, 0}, hdr1 = {0, 0, 0, 0}, hnext0 = {0, 0, 0, 0}, hnext1 = {0, 0, 0, 0};
     const int nsteps = K / BK;
-    auto load_step = [&](int ks_, uint4& x0, uint4& x1, uint32_t& w) __attribute__((always_inline)) {  // ks = K offset / 32
+    // The activation copies go global -> LDS without passing registers (global_load_lds); they are
+    // written as instructions so that the compiler does not count them: it would make every LDS
+    // read wait for copies that are in flight on purpose.  They are waited for by hand (below).
+    const uint32_t lds_x = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)xs;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    auto copy_x = [&](int ks_) __attribute__((always_inline)) {
         const int ks = min(ks_, nsteps - 1);  // past the end: the last step again, no branch
-        x0 = *reinterpret_cast<const uint4*>(xp0 + (size_t)ks * BK);
-        x1 = *reinterpret_cast<const uint4*>(xp1 + (size_t)ks * BK);
-        const int blk = ks >> 3, g = ks & 7;
-        const uint8_t* unit = wbase + (size_t)blk * 2304;
-        w = *reinterpret_cast<const uint32_t*>(unit + (g >> 2) * 1024 + (wn + 16 * (g & 3)) * 16 + 4 * wj);
-        if (g == 0) hnext = *reinterpret_cast<const uint4*>(unit + 2048 + 16 * wn);
+        const uint32_t dst = lds_x + (uint32_t)(((ks_ & 3) * BM * 4 + 64 * wave_u) * 16);
+        const unsigned short* s0 = xp0 + (size_t)ks * BK;
+        const unsigned short* s1 = xp1 + (size_t)ks * BK;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(s0) : "memory");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst + 512 * 16), "v"(s1) : "memory");
     };
-    auto store_step = [&](int buf, int ks, uint4 x0, uint4 x1, uint32_t w) __attribute__((always_inline)) {
-        xs[buf][lds_index(xr0, xseg)] = x0;
-        xs[buf][lds_index(xr0 + 128, xseg)] = x1;
-        if ((ks & 7) == 0) hdr = hnext;
+    // g = ks % 8 is passed separately: a compile-time constant where the loop is unrolled over a block
+    auto load_step = [&](int ks_, int g, uint32_t& w0, uint32_t& w1) __attribute__((always_inline)) {  // ks = K offset / 32
+        const int ks = min(ks_, nsteps - 8 + g);  // past the end: the last block again, no branch
+        const int blk = ks >> 3;
+        const size_t off = (size_t)blk * 2304;
+        const int coff = (g >> 2) * 1024 + (wn + 16 * (g & 3)) * 16 + 4 * wj;
+        w0 = *reinterpret_cast<const uint32_t*>(wbase0 + off + coff);
+        if constexpr (WROWS == 2) w1 = *reinterpret_cast<const uint32_t*>(wbase1 + off + coff);
+        if (g == 0) {
+            hnext0 = *reinterpret_cast<const uint4*>(wbase0 + off + 2048 + 16 * wn);
+            if constexpr (WROWS == 2) hnext1 = *reinterpret_cast<const uint4*>(wbase1 + off + 2048 + 16 * wn);
+        }
+    };
+    auto store_step = [&](int buf, int g, uint32_t w0, uint32_t w1) __attribute__((always_inline)) {
+        if (g == 0) { hdr0 = hnext0; hdr1 = hnext1; }
         float a, c;
-        group_coeffs<FMT>(hdr, ks & 7, a, c);
-        wsm[buf][lds_index(wr, wj)] = decode8(w, a, c);
+        group_coeffs<FMT>(hdr0, g, a, c);
+        wsm[buf * BN * 4 + lds_index(wr, wj)] = decode8(w0, a, c);
+        if constexpr (WROWS == 2) {
+            group_coeffs<FMT>(hdr1, g, a, c);
+            wsm[buf * BN * 4 + lds_index(wr + 128, wj)] = decode8(w1, a, c);
+        }
     };
 
-    // wavefront sub-tile: 4 (M) x 2 (N) wavefronts, each 64 x 64 = 4 x 4 MFMA tiles
-    const int wm = wave >> 1, wn_ = wave & 1;
+    // wavefront sub-tile: 2 (M) x 4 (N) wavefronts of 128 x 64, or 4 x 2 wavefronts of 64 x 64
+    const int wm = BN == 256 ? wave >> 2 : wave >> 1, wn_ = BN == 256 ? wave & 3 : wave & 1;
     const int fr = lane & 15, fk = lane >> 4;
-    f32x4_t acc[4][4];
+    f32x4_t acc[MI][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    load_step(0, rx0[0], rx1[0], rw[0]);
-    load_step(1, rx0[1], rx1[1], rw[1]);
-    load_step(2, rx0[2], rx1[2], rw[2]);
-    store_step(0, 0, rx0[0], rx1[0], rw[0]);
+    copy_x(0); load_step(0, 0, rw0[0], rw1[0]);
+    copy_x(1); load_step(1, 1, rw0[1], rw1[1]);
+    copy_x(2); load_step(2, 2, rw0[2], rw1[2]);
+    store_step(0, 0, rw0[0], rw1[0]);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    for (int ks0 = 0; ks0 < nsteps; ks0 += 4) {
+    // The affine format's header fields are cheapest to extract at a static group index, so its loop
+    // is unrolled over a whole 256-wide block; the symmetric one keeps the shorter body.
+    constexpr int UNR = FMT == TFQ_Q_G_4 ? 8 : 4;
+    for (int ks0 = 0; ks0 < nsteps; ks0 += UNR) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < UNR; ++u) {
             const int ks = ks0 + u, buf = u & 1;
-            load_step(ks + 3, rx0[(u + 3) & 3], rx1[(u + 3) & 3], rw[(u + 3) & 3]);
-            uint4 af[4], bfr[4];
+            const int gbase = UNR == 8 ? 0 : (ks0 & 4);
+            // buffer (ks + 3) % 4 was read during step ks - 1, which every wavefront has left
+            copy_x(ks + 3);
+            load_step(ks + 3, (gbase + u + 3) & 7, rw0[(u + 3) & 3], rw1[(u + 3) & 3]);
+            uint4 af[MI], bfr[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) af[i] = xs[buf][lds_index(wm * 64 + i * 16 + fr, fk)];
+            for (int j = 0; j < 4; ++j) bfr[j] = wsm[buf * BN * 4 + lds_index(wn_ * 64 + j * 16 + fr, fk)];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) bfr[j] = wsm[buf][lds_index(wn_ * 64 + j * 16 + fr, fk)];
+            for (int i = 0; i < MI; ++i) af[i] = xs[(u & 3) * BM * 4 + lds_index(wm * (MI * 16) + i * 16 + fr, fk)];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < MI; ++i)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[i]),
                                                                         __builtin_bit_cast(bf16x8_t, bfr[j]), acc[i][j], 0, 0, 0);
-            store_step(buf ^ 1, ks + 1, rx0[(u + 1) & 3], rx1[(u + 1) & 3], rw[(u + 1) & 3]);  // past the end: written, never read
+            store_step(buf ^ 1, (gbase + u + 1) & 7, rw0[(u + 1) & 3], rw1[(u + 1) & 3]);  // past the end: written, never read
+            // step ks + 1's activation copies were issued two steps ago; behind them at least the
+            // 2 + 4 + 4 = 10 loads of this and the previous step have been issued, 8 is a safe bound
+            asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
             __syncthreads();
         }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may land in LDS after the workgroup is gone
 
     // ---- store: lane holds column fr, rows 4 fk + r of each 16 x 16 tile
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int col = n0 + wn_ * 64 + j * 16 + fr;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int row = m0 + wm * 64 + i * 16 + 4 * fk + r;
+                const int row = m0 + wm * (MI * 16) + i * 16 + 4 * fk + r;
                 if (row < M && col < N) {
                     const size_t o = (size_t)row * N + col;
                     if (args.y_bf16) reinterpret_cast<unsigned short*>(args.Y)[o] = (unsigned short)bf16_rne(acc[i][j][r]);
@@ -203,6 +238,22 @@ __global__ __launch_bounds__(THREADS) void gemm4_kernel(GemmArgs args) {
                 }
             }
         }
+}
+
+template <int FMT, int BN>
+int run_tiles(GemmArgs a, hipStream_t s) {
+    a.tiles_n = (a.N + BN - 1) / BN;
+    const int grid = 8 * ((a.tiles_m * a.tiles_n + 7) / 8);
+    constexpr size_t lds = (size_t)(4 * BM * 4 + 2 * BN * 4) * 16;  // 96 KB or 80 KB
+    static bool lds_limit_raised = false;  // once: not allowed while a stream is being captured
+    if (!lds_limit_raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm4_kernel<FMT, BN>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
+        lds_limit_raised = true;
+    }
+    hipLaunchKernelGGL((gemm4_kernel<FMT, BN>), dim3(grid), dim3(THREADS), lds, s, a);
+    return hip_fail(hipGetLastError(), "gemm launch");
 }
 
 template <int FMT>
@@ -216,10 +267,10 @@ int run(const tfq_weight* w, const void* x, int M, void* y, int yd, hipStream_t 
     a.K = (int)w->K;
     a.y_bf16 = yd == TFQ_BF16;
     a.tiles_m = (M + BM - 1) / BM;
-    a.tiles_n = (a.N + BN - 1) / BN;
-    const int grid = 8 * ((a.tiles_m * a.tiles_n + 7) / 8);
-    hipLaunchKernelGGL(gemm4_kernel<FMT>, dim3(grid), dim3(THREADS), 0, s, a);
-    return hip_fail(hipGetLastError(), "gemm launch");
+    // 256-wide weight strips read LDS less per MFMA; they are used when they still give every
+    // compute unit a workgroup, otherwise the 128-wide ones double the number of workgroups
+    const int wide = a.tiles_m * ((a.N + 255) / 256);
+    return wide >= 256 ? run_tiles<FMT, 256>(a, s) : run_tiles<FMT, 128>(a, s);
 }
 
 }  // namespace
