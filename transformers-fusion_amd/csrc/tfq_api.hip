@@ -188,11 +188,8 @@ int tfq_decode_blocks_host(uint8_t fmt, const uint8_t* src, size_t bytes, int64_
     return rc;
 }
 
-// The 4-bit matmul formats are kept in the Tiled16 layout; everything else stays in wire order.
-static bool wants_tiled16(uint8_t fmt) {
-    const int c = canonical(fmt);
-    return c == TFQ_Q_G_4 || c == TFQ_B32S4;
-}
+// The formats with a matrix-core matmul kernel are kept in the Tiled16 layout; everything else stays in wire order.
+static bool wants_tiled16(uint8_t fmt) { return tiled_header_bytes(fmt) != 0; }
 
 static tfq_weight_t* make_weight(const char* who, uint8_t fmt, int64_t N, int64_t K, const uint8_t* packed,
                                  size_t bytes, bool from_host) {
@@ -207,7 +204,7 @@ static tfq_weight_t* make_weight(const char* who, uint8_t fmt, int64_t N, int64_
     const bool tiled = wants_tiled16(fmt);
     tfq_weight_t* w = new (std::nothrow) tfq_weight_t{fmt, N, K, bytes, nullptr, 0, tiled ? TFQ_LAYOUT_TILED16 : TFQ_LAYOUT_WIRE, true};
     if (!w) { fail(TFQ_ERR_NOMEM, std::string(who) + ": out of host memory"); return nullptr; }
-    w->dev_bytes = tiled ? (size_t)((N + 15) / 16) * (size_t)(K / 256) * 2304 : bytes;
+    w->dev_bytes = tiled ? (size_t)((N + 15) / 16) * (size_t)(K / 256) * (size_t)tiled_unit_bytes(fmt) : bytes;
     uint8_t* staged = nullptr;  // wire payload on the device, when it has to be permuted
     hipError_t e = hipMalloc(&w->dev, w->dev_bytes);
     if (e == hipSuccess && from_host) {
@@ -221,7 +218,7 @@ static tfq_weight_t* make_weight(const char* who, uint8_t fmt, int64_t N, int64_
     int rc = hip_fail(e, who);
     if (!rc) {
         const uint8_t* wire = from_host ? staged : packed;
-        if (tiled) rc = launch_tile16(wire, w->dev, N, K, nullptr);
+        if (tiled) rc = launch_tile16(fmt, wire, w->dev, N, K, nullptr);
         else if (!from_host) rc = hip_fail(hipMemcpy(w->dev, packed, bytes, hipMemcpyDeviceToDevice), who);
         if (!rc) rc = hip_fail(hipDeviceSynchronize(), who);
     }
@@ -261,14 +258,7 @@ int tfq_weight_decode(const tfq_weight_t* w, float* out, tfq_stream_t stream) {
     if (!w || !out) return fail(TFQ_ERR_ARG, "tfq_weight_decode: null pointer");
     if (int r = ensure_device()) return r;
     if (w->layout == TFQ_LAYOUT_WIRE) return launch_decode(w->fmt, w->dev, w->N * (w->K / 256), out, (hipStream_t)stream);
-    // Tiled16: restore wire order in a temporary buffer, then decode it.
-    uint8_t* wire = nullptr;
-    TFQ_HIP(hipMalloc(&wire, w->bytes));
-    int rc = launch_untile16(w->dev, wire, w->N, w->K, (hipStream_t)stream);
-    if (!rc) rc = launch_decode(w->fmt, wire, w->N * (w->K / 256), out, (hipStream_t)stream);
-    if (!rc) rc = hip_fail(hipStreamSynchronize((hipStream_t)stream), "tfq_weight_decode");
-    (void)hipFree(wire);
-    return rc;
+    return launch_decode_tiled(w->fmt, w->dev, w->N, w->K, out, (hipStream_t)stream);
 }
 
 static int check_matmul(const char* who, const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, int y_dtype) {

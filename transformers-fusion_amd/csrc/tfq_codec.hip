@@ -1,6 +1,6 @@
 // Block codec on the device: bit-exact decode of every supported wire format
-// (per-weight arithmetic in tfq_decode.hpp), the closed-form encoders, and the
-// wire <-> Tiled16 layout permutation.  Decode and encode use one workgroup of
+// (per-weight arithmetic in tfq_decode.hpp), the closed-form encoders, the wire ->
+// Tiled16 layout conversion and the decode from that layout.  Decode and encode use one workgroup of
 // 256 lanes per 256-weight block, one lane per weight; the payload of a block is
 // at most 1 KB, so these kernels are bound by the fp32 side (4 B per weight).
 
@@ -63,30 +63,84 @@ __global__ __launch_bounds__(256) void encode_raw32_kernel(const float* __restri
     reinterpret_cast<float*>(dst)[e] = w[e];
 }
 
-// Wire <-> Tiled16 permutation of 144-byte blocks, one lane per 16-byte piece.
-// piece p of a unit: p < 64 code slot of k-step 0, p < 128 of k-step 1, else header of row p - 128.
-template <bool TO_TILED>
-__global__ __launch_bounds__(256) void tile16_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+// Wire -> Tiled16: one lane per 16-byte piece of the tiled buffer.  Piece p of a unit: p < 64 code
+// slot of k-step 0, p < 128 of k-step 1, else a 16-byte part of a row header.  Codes narrower
+// than 4 bits are widened to nibbles.
+template <int FMT>
+__global__ __launch_bounds__(256) void tile16_kernel(const uint8_t* __restrict__ wire, uint4* __restrict__ tiled,
                                                      int64_t N, int nblocks, int64_t npieces) {
+    constexpr Spec sp = spec_of(FMT);
+    constexpr int HB = tiled_header_bytes(FMT), HP = HB / 16, PIECES = 128 + 16 * HP;
+    constexpr uint32_t BB = sp.block_bytes, code_bytes = 256u * sp.bits / 8;
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= npieces) return;
-    const int64_t unit = i / 144;
-    const int p = (int)(i - unit * 144);
+    const int64_t unit = i / PIECES;
+    const int p = (int)(i - unit * PIECES);
     const int64_t tile = unit / nblocks;
     const int blk = (int)(unit - tile * nblocks);
-    int n, off16;  // row inside the tile, 16-byte piece inside the wire block
+    uint32_t o[4] = {0, 0, 0, 0};
     if (p < 128) {
-        const int l = p & 63;
-        n = l & 15;
-        off16 = (l >> 4) + 4 * (p >> 6);
+        const int l = p & 63, n = l & 15, g32 = (l >> 4) + 4 * (p >> 6);
+        const int64_t row = tile * 16 + n;
+        if (row < N) {
+            const uint8_t* src = wire + (row * nblocks + blk) * (int64_t)BB;
+#pragma unroll
+            for (int j = 0; j < 32; ++j) {
+                const uint32_t code = stream_bits(src, code_bytes, (uint32_t)(32 * g32 + j) * sp.bits, sp.bits);
+                o[j >> 3] |= code << (4 * (j & 7));
+            }
+        }
     } else {
-        n = p - 128;
-        off16 = 8;
+        const int n = (p - 128) / HP, part = (p - 128) % HP;
+        const int64_t row = tile * 16 + n;
+        if (row < N) {
+            const uint8_t* src = wire + (row * nblocks + blk) * (int64_t)BB;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const uint32_t off = code_bytes + 16 * part + j;
+                if (off < BB) o[j >> 2] |= (uint32_t)src[off] << (8 * (j & 3));
+            }
+        }
     }
-    const int64_t row = tile * 16 + n;
-    const int64_t wire = (row * nblocks + blk) * 9 + off16;
-    if (TO_TILED) dst[i] = row < N ? src[wire] : uint4{0, 0, 0, 0};
-    else if (row < N) dst[wire] = src[i];
+    tiled[i] = uint4{o[0], o[1], o[2], o[3]};
+}
+
+// Decode straight from the Tiled16 layout: one workgroup per (row, block), one lane per weight,
+// the arithmetic of decode_weight on the same header bytes.
+template <int FMT>
+__global__ __launch_bounds__(256) void decode_tiled_kernel(const uint8_t* __restrict__ tiled, float* __restrict__ out,
+                                                           int nblocks) {
+    constexpr Spec sp = spec_of(FMT);
+    constexpr int HB = tiled_header_bytes(FMT), UB = tiled_unit_bytes(FMT);
+    const int64_t rb = blockIdx.x;  // row * nblocks + blk
+    const int64_t row = rb / nblocks;
+    const int blk = (int)(rb - row * nblocks);
+    const uint32_t i = threadIdx.x;
+    const uint8_t* unit = tiled + ((row >> 4) * nblocks + blk) * (int64_t)UB;
+    const int n = (int)(row & 15);
+    const uint32_t g32 = i >> 5, j = i & 31;
+    const uint8_t* codes = unit + (g32 >> 2) * 1024 + (n + 16 * (g32 & 3)) * 16;
+    const uint32_t idx = (codes[j >> 1] >> ((j & 1u) * 4)) & 15u;
+    const uint8_t* h = unit + 2048 + n * HB;
+    float v;
+    if constexpr (sp.codec == Codec::Sym32) {
+        const float d = half_bits_to_float((uint32_t)h[2 * g32] | ((uint32_t)h[2 * g32 + 1] << 8));
+        v = (float)((int)idx - 8) * d;
+    } else {
+        constexpr uint32_t ng = 256 / sp.gsz;
+        constexpr uint32_t sc_bits = ((ng * sp.scb + 7) / 8) * 8;
+        constexpr uint32_t mn_bits = ((ng * sp.mb + 7) / 8) * 8;
+        constexpr int bias = (1 << sp.mb) / 2;
+        const uint32_t g = i / sp.gsz;
+        const float sc = (float)stream_bits(h, HB, g * sp.scb, sp.scb);
+        const float mc = (float)stream_bits(h, HB, sc_bits + g * sp.mb, sp.mb) - (float)bias;
+        const float d = half_bits_to_float(stream_bits(h, HB, sc_bits + mn_bits, 16));
+        const float dm = half_bits_to_float(stream_bits(h, HB, sc_bits + mn_bits + 16, 16));
+        const float es = d * sc;
+        const float neg = -(dm * mc);
+        v = __builtin_fmaf(es, unit_level(sp.bits, idx), neg);
+    }
+    out[rb * 256 + i] = v;
 }
 
 template <int FMT>
@@ -116,27 +170,49 @@ int launch_decode(int fmt, const uint8_t* src, int64_t nblocks, float* out, hipS
     }
 }
 
-static int run_tile16(bool to_tiled, const uint8_t* src, uint8_t* dst, int64_t N, int64_t K, hipStream_t s) {
+template <int FMT>
+static int run_tile16(const uint8_t* wire, uint8_t* tiled, int64_t N, int64_t K, hipStream_t s) {
     const int nblocks = (int)(K / 256);
     const int64_t tiles = (N + 15) / 16;
-    const int64_t npieces = tiles * nblocks * 144;
+    const int64_t npieces = tiles * nblocks * (tiled_unit_bytes(FMT) / 16);
     const int64_t grid = (npieces + 255) / 256;
     if (grid > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "matrix too large for one layout pass");
-    if (to_tiled)
-        hipLaunchKernelGGL(tile16_kernel<true>, dim3((unsigned)grid), dim3(256), 0, s, reinterpret_cast<const uint4*>(src),
-                           reinterpret_cast<uint4*>(dst), N, nblocks, npieces);
-    else
-        hipLaunchKernelGGL(tile16_kernel<false>, dim3((unsigned)grid), dim3(256), 0, s, reinterpret_cast<const uint4*>(src),
-                           reinterpret_cast<uint4*>(dst), N, nblocks, npieces);
+    hipLaunchKernelGGL(tile16_kernel<FMT>, dim3((unsigned)grid), dim3(256), 0, s, wire, reinterpret_cast<uint4*>(tiled), N,
+                       nblocks, npieces);
     return hip_fail(hipGetLastError(), "layout launch");
 }
 
-int launch_tile16(const uint8_t* wire, uint8_t* tiled, int64_t N, int64_t K, hipStream_t s) {
-    return run_tile16(true, wire, tiled, N, K, s);
+int launch_tile16(int fmt, const uint8_t* wire, uint8_t* tiled, int64_t N, int64_t K, hipStream_t s) {
+    switch (canonical(fmt)) {
+        case TFQ_Q_G_4: return run_tile16<TFQ_Q_G_4>(wire, tiled, N, K, s);
+        case TFQ_B32S4: return run_tile16<TFQ_B32S4>(wire, tiled, N, K, s);
+        case TFQ_Q_G_3: return run_tile16<TFQ_Q_G_3>(wire, tiled, N, K, s);
+        case TFQ_Q_G_2: return run_tile16<TFQ_Q_G_2>(wire, tiled, N, K, s);
+        case TFQ_SB256A3: return run_tile16<TFQ_SB256A3>(wire, tiled, N, K, s);
+        case TFQ_SB256A2: return run_tile16<TFQ_SB256A2>(wire, tiled, N, K, s);
+        default: return fail(TFQ_ERR_FORMAT, "layout: wire id " + std::to_string(fmt) + " has no tiled layout");
+    }
 }
 
-int launch_untile16(const uint8_t* tiled, uint8_t* wire, int64_t N, int64_t K, hipStream_t s) {
-    return run_tile16(false, tiled, wire, N, K, s);
+template <int FMT>
+static int run_decode_tiled(const uint8_t* tiled, int64_t N, int64_t K, float* out, hipStream_t s) {
+    const int nblocks = (int)(K / 256);
+    const int64_t grid = N * nblocks;
+    if (grid > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "decode: more than 2^31-1 blocks in one call");
+    hipLaunchKernelGGL(decode_tiled_kernel<FMT>, dim3((unsigned)grid), dim3(256), 0, s, tiled, out, nblocks);
+    return hip_fail(hipGetLastError(), "decode launch");
+}
+
+int launch_decode_tiled(int fmt, const uint8_t* tiled, int64_t N, int64_t K, float* out, hipStream_t s) {
+    switch (canonical(fmt)) {
+        case TFQ_Q_G_4: return run_decode_tiled<TFQ_Q_G_4>(tiled, N, K, out, s);
+        case TFQ_B32S4: return run_decode_tiled<TFQ_B32S4>(tiled, N, K, out, s);
+        case TFQ_Q_G_3: return run_decode_tiled<TFQ_Q_G_3>(tiled, N, K, out, s);
+        case TFQ_Q_G_2: return run_decode_tiled<TFQ_Q_G_2>(tiled, N, K, out, s);
+        case TFQ_SB256A3: return run_decode_tiled<TFQ_SB256A3>(tiled, N, K, out, s);
+        case TFQ_SB256A2: return run_decode_tiled<TFQ_SB256A2>(tiled, N, K, out, s);
+        default: return fail(TFQ_ERR_FORMAT, "decode: wire id " + std::to_string(fmt) + " has no tiled layout");
+    }
 }
 
 int launch_encode(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStream_t s) {

@@ -276,7 +276,7 @@ int run(const tfq_weight* w, const void* x, int M, void* y, int yd, hipStream_t 
 }  // namespace
 
 int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype, hipStream_t s) {
-    const bool mfma_path = w->layout == TFQ_LAYOUT_TILED16 && x_dtype == TFQ_BF16 && M > 16;
+    const bool mfma_path = w->layout == TFQ_LAYOUT_TILED16 && tiled_unit_bytes(w->fmt) == 2304 && x_dtype == TFQ_BF16 && M > 16;
     if (mfma_path) {
         if (w->N > 0x7FFFFFF0 || w->K > 0x7FFFFFF0) return fail(TFQ_ERR_SHAPE, "gemm: shape too large");
         switch (canonical(w->fmt)) {

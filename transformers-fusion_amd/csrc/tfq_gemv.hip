@@ -105,45 +105,72 @@ struct GemvKernArgs {
     int K, y_bf16, nslot, tiles_per_wg, cols_base, cols_rem;
 };
 
-// Bias that the MFMA accumulator starts from, so that it ends as the dot
-// product with the true code values: the bf16 fragments hold 128+n, and the
-// symmetric format's codes are offset by 8.
+// Per-format constants of the kernel.
+//   HB   header bytes per row and block in the Tiled16 layout (16 or 32)
+//   GS   weights per scale group (32 or 16)
+//   OFFS what the bf16 operand (128 + code) overshoots the true code value by: the MFMA
+//        accumulator starts at -OFFS * X so that it ends as the dot product with the codes
 template <int FMT>
-__device__ __forceinline__ f32x4_t accumulator_bias(float4 X) {
-    constexpr float k = FMT == TFQ_B32S4 ? -136.0f : -128.0f;
-    return f32x4_t{k * X.x, k * X.y, k * X.z, k * X.w};
+struct Fmt {
+    static constexpr int HB = tiled_header_bytes(FMT);
+    static constexpr int HV = HB / 16;  // uint4 registers per header
+    static constexpr int GS = spec_of(FMT).gsz == 16 ? 16 : 32;
+    static constexpr int NG = 256 / GS;  // groups per block: 8 or 16
+    static constexpr float OFFS = FMT == TFQ_B32S4 ? 136.0f : 128.0f;
+};
+
+// `count` bits at bit `pos` (both compile-time after unrolling) of the little-endian bit string w[0], w[1], ...
+__device__ __forceinline__ uint32_t field(const uint32_t* w, int pos, int count) {
+    const int i = pos >> 5, sh = pos & 31;
+    uint32_t v = w[i] >> sh;
+    if (sh + count > 32) v |= w[i + 1] << (32 - sh);
+    return count >= 32 ? v : v & ((1u << count) - 1u);
 }
 
-// sum over the four groups r of one k-step: D[r] is the group's dot product with
-// the integer codes (bias already removed), X[r] the group's activation sum
+// Contribution of k-step `khalf` of one unit to the lane's output: the sum over the k-step's
+// groups of a * D + c * X, where D is the group's dot product with the integer codes, X the
+// group's activation sum and (a, c) the group's scale and offset:
+//   affine formats     a = d * sc / top,  c = -dm * mc      (top = 15, 7 or 3)
+//   symmetric format   a = d,             c = 0             (the code offset 8 is part of OFFS)
+// With 32-weight groups DA[r] is the dot product of group r (DB is unused); with 16-weight
+// groups DA[r] / DB[r] are the two halves of 32-slot r, i.e. groups 2r and 2r + 1, and X
+// holds the eight activation sums in group order.
 template <int FMT>
-__device__ __forceinline__ float apply_groups(uint4 h, int khalf, f32x4_t D, float4 X) {
+__device__ __forceinline__ float apply_groups(const uint4* hv, int khalf, f32x4_t DA, f32x4_t DB, const float* X) {
+    constexpr Spec sp = spec_of(FMT);
     float res = 0.0f;
-    if constexpr (FMT == TFQ_Q_G_4) {
-        // header: 8 x 6-bit sc | 8 x 6-bit (mc+32) | binary16 d | binary16 dm
-        const float xv[4] = {X.x, X.y, X.z, X.w};
-        const uint64_t scs = (uint64_t)h.x | ((uint64_t)(h.y & 0xFFFFu) << 32);
-        const uint64_t mcs = (uint64_t)(h.y >> 16) | ((uint64_t)h.z << 16);
-        const uint32_t sc24 = (uint32_t)(scs >> (24 * khalf));
-        const uint32_t mc24 = (uint32_t)(mcs >> (24 * khalf));
-        const float d15 = half_fast(h.w & 0xFFFFu) * (1.0f / 15.0f);
-        const float dm = half_fast(h.w >> 16);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const float a = d15 * (float)((sc24 >> (6 * r)) & 63u);
-            const float off = dm * (float)(32 - (int)((mc24 >> (6 * r)) & 63u));  // -dm * mc
-            res = __builtin_fmaf(a, D[r], res);
-            res = __builtin_fmaf(off, xv[r], res);
-        }
-    } else {
+    if constexpr (FMT == TFQ_B32S4) {
         // header: eight binary16 scales, four per k-step; the conversion rides in the multiply-add
         // (v_fma_mix_f32 reads either half of a dword as binary16)
-        const f16x2_t s01 = __builtin_bit_cast(f16x2_t, khalf ? h.z : h.x);
-        const f16x2_t s23 = __builtin_bit_cast(f16x2_t, khalf ? h.w : h.y);
-        res = __builtin_fmaf((float)s01.x, D[0], res);
-        res = __builtin_fmaf((float)s01.y, D[1], res);
-        res = __builtin_fmaf((float)s23.x, D[2], res);
-        res = __builtin_fmaf((float)s23.y, D[3], res);
+        const f16x2_t s01 = __builtin_bit_cast(f16x2_t, khalf ? hv[0].z : hv[0].x);
+        const f16x2_t s23 = __builtin_bit_cast(f16x2_t, khalf ? hv[0].w : hv[0].y);
+        res = __builtin_fmaf((float)s01.x, DA[0], res);
+        res = __builtin_fmaf((float)s01.y, DA[1], res);
+        res = __builtin_fmaf((float)s23.x, DA[2], res);
+        res = __builtin_fmaf((float)s23.y, DA[3], res);
+    } else {
+        // header: NG scale codes of scb bits | NG offset codes of mb bits (biased) | binary16 d | binary16 dm
+        constexpr int NG = Fmt<FMT>::NG, PER = NG / 2;  // groups per k-step
+        constexpr int sc_bits = ((NG * sp.scb + 7) / 8) * 8, mn_bits = ((NG * sp.mb + 7) / 8) * 8;
+        constexpr int mbias = (1 << sp.mb) / 2;
+        constexpr float inv_top = sp.bits == 4 ? 1.0f / 15.0f : sp.bits == 3 ? 1.0f / 7.0f : 1.0f / 3.0f;
+        uint32_t w[8];
+#pragma unroll
+        for (int i = 0; i < Fmt<FMT>::HV; ++i) {
+            w[4 * i] = hv[i].x; w[4 * i + 1] = hv[i].y; w[4 * i + 2] = hv[i].z; w[4 * i + 3] = hv[i].w;
+        }
+        const uint32_t dd = field(w, sc_bits + mn_bits, 32);
+        const float dtop = half_fast(dd & 0xFFFFu) * inv_top;
+        const float dm = half_fast(dd >> 16);
+#pragma unroll
+        for (int t = 0; t < PER; ++t) {
+            const int g = khalf * PER + t;
+            const float a = dtop * (float)field(w, g * sp.scb, sp.scb);
+            const float off = dm * (float)(mbias - (int)field(w, sc_bits + g * sp.mb, sp.mb));  // -dm * mc
+            const float D = Fmt<FMT>::GS == 32 ? DA[t] : (t & 1) ? DB[t >> 1] : DA[t >> 1];
+            res = __builtin_fmaf(a, D, res);
+            res = __builtin_fmaf(off, X[t], res);
+        }
     }
     return res;
 }
@@ -160,6 +187,9 @@ __device__ unsigned long long g_trace[1024 * 16 * 8];
 template <int FMT, bool XF32, int WD>
 __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin) {
     extern __shared__ uint4 smem[];
+    using F = Fmt<FMT>;
+    constexpr int UB = 2048 + 16 * F::HB;  // bytes of a unit
+    constexpr int NG = F::NG, PER = NG / 2;  // scale groups per block / per k-step
     const int K = args.K, nslot = args.nslot, T = args.tiles_per_wg;
     const int cols_base = args.cols_base, cols_rem = args.cols_rem;
     const bool y_bf16 = args.y_bf16 != 0;
@@ -184,10 +214,10 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     const int nitems = ncols * tiles_here;  // block-column major, tiles inside
     TRACE(0);
 
-    // LDS: per wavefront and block column, A entries [nslot][2 k-steps][4 groups][4] (uint4) and
-    // group sums [4 slots][2][4] (float); then one zero A entry set per wavefront, then the partial sums [T][NW][64].
+    // LDS: per wavefront and block column, A entries [nslot][2 k-steps][4 slots of 32][4] (uint4) and
+    // group sums [4 slots][NG] (float); then one zero A entry set per wavefront, then the partial sums [T][NW][64].
     const int a_per_col = nslot * 32;                   // uint4 entries
-    const int col_stride = a_per_col + 8;               // + 32 floats of group sums
+    const int col_stride = a_per_col + NG;              // + 4 NG floats of group sums
     uint4* my = smem + (size_t)wave * ncols_max * col_stride;
     uint4* zero4 = smem + (size_t)NW * ncols_max * col_stride + 4 * wave;  // this wavefront's own zero A entries
     float* part = reinterpret_cast<float*>(smem + (size_t)NW * ncols_max * col_stride + 4 * NW);
@@ -231,23 +261,24 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     // loads younger than any operand is a compile-time constant, staging waits for the
     // activations alone and a unit is consumed as soon as IT has arrived (behind a conditional
     // fetch the compiler waits for everything in flight).
-    const size_t tile_stride = (size_t)nblocks * 2304;
-    const uint8_t* col_ptr = Wm + ((size_t)tile0 * nblocks + (size_t)wave) * 2304;
+    const size_t tile_stride = (size_t)nblocks * UB;
+    const uint8_t* col_ptr = Wm + ((size_t)tile0 * nblocks + (size_t)wave) * UB;
     const uint8_t* f_ptr = col_ptr;
     int f_ci = 0, f_t = 0;
-    const uint32_t off_c = 16u * lane, off_h = 2048u + 16u * n;
-    auto fetch = [&](uint4& c0, uint4& c1, uint4& hd) __attribute__((always_inline)) {
+    const uint32_t off_c = 16u * lane, off_h = 2048u + (uint32_t)F::HB * n;
+    auto fetch = [&](uint4& c0, uint4& c1, uint4 (&hd)[F::HV]) __attribute__((always_inline)) {
         c0 = *reinterpret_cast<const uint4*>(f_ptr + off_c);
         c1 = *reinterpret_cast<const uint4*>(f_ptr + off_c + 1024);
-        hd = *reinterpret_cast<const uint4*>(f_ptr + off_h);
+#pragma unroll
+        for (int i = 0; i < F::HV; ++i) hd[i] = *reinterpret_cast<const uint4*>(f_ptr + off_h + 16 * i);
         f_ptr += tile_stride;
         if (++f_t == tiles_here) {
             f_t = 0;
-            if (++f_ci < ncols) col_ptr += (size_t)NW * 2304;
+            if (++f_ci < ncols) col_ptr += (size_t)NW * UB;
             f_ptr = col_ptr;
         }
     };
-    uint4 c0[WD], c1[WD], hd[WD];
+    uint4 c0[WD], c1[WD], hd[WD][F::HV];
 #pragma unroll
     for (int u = 0; u < WD; ++u) fetch(c0[u], c1[u], hd[u]);
 
@@ -282,10 +313,14 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
             sum = dot2(ONES, p.z, sum);
             sum = dot2(ONES, p.w, sum);
         }
-        sum = dpp_add<0xB1>(sum);  // the four dwords of a group sit in adjacent lanes
-        sum = dpp_add<0x4E>(sum);
-        if ((quad & 3) == 0) colX[s * 8 + (quad >> 2)] = sum;  // zero for an unused slot of the pass
-        if (npc == 1 && (quad & 3) == 0) colX[(s + 2) * 8 + (quad >> 2)] = 0.0f;  // slots 2, 3 are never staged
+        // a lane holds 8 elements; the lanes of a 16- or 32-weight group are adjacent
+        sum = dpp_add<0xB1>(sum);
+        if constexpr (F::GS == 32) sum = dpp_add<0x4E>(sum);
+        constexpr int LPG = F::GS / 8;  // lanes per group
+        if ((quad & (LPG - 1)) == 0) {
+            colX[s * NG + quad / LPG] = sum;  // zero for an unused slot of the pass
+            if (npc == 1) colX[(s + 2) * NG + quad / LPG] = 0.0f;  // slots 2, 3 are never staged
+        }
     };
 #pragma unroll
     for (int p = 0; p < XP; ++p)
@@ -307,8 +342,7 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     uint32_t C = 0x43004300u;
     asm volatile("" : "+v"(C));  // keep the bias in a VGPR so (v & M) | C is one v_and_or_b32
     uint4 av[2][4];
-    float4 xv[2];
-    f32x4_t bias[2];
+    float xv[2][PER];
     int c_ci = 0, c_t = 0;
     float* cell = part + wave * 64 + lane;  // this wavefront's cell of tile c_t
     auto consume = [&](int u) __attribute__((always_inline)) {
@@ -320,8 +354,11 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
                 const uint4* src = a_live ? col + s_a * 32 + h * 16 + q * 4 : zero4;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) av[h][j] = src[j];
-                xv[h] = *reinterpret_cast<const float4*>(colX + q * 8 + h * 4);
-                bias[h] = accumulator_bias<FMT>(xv[h]);
+#pragma unroll
+                for (int t = 0; t < PER; t += 4) {
+                    const float4 f = *reinterpret_cast<const float4*>(colX + q * NG + h * PER + t);
+                    xv[h][t] = f.x; xv[h][t + 1] = f.y; xv[h][t + 2] = f.z; xv[h][t + 3] = f.w;
+                }
             }
         }
         float res = 0.0f;
@@ -329,15 +366,27 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
         for (int h = 0; h < 2; ++h) {
             const uint4 cw = h ? c1[u] : c0[u];
             const uint32_t qq[4] = {cw.x, cw.y, cw.z, cw.w};
-            f32x4_t Dv = bias[h];
+            // accumulators start at -OFFS * X; with 16-weight groups dwords 0, 1 and 2, 3 of a
+            // 32-slot belong to different groups and get an accumulator each
+            f32x4_t DA, DB = {0.0f, 0.0f, 0.0f, 0.0f};
+            if constexpr (F::GS == 32) {
+                DA = f32x4_t{-F::OFFS * xv[h][0], -F::OFFS * xv[h][1], -F::OFFS * xv[h][2], -F::OFFS * xv[h][3]};
+            } else {
+                DA = f32x4_t{-F::OFFS * xv[h][0], -F::OFFS * xv[h][2], -F::OFFS * xv[h][4], -F::OFFS * xv[h][6]};
+                DB = f32x4_t{-F::OFFS * xv[h][1], -F::OFFS * xv[h][3], -F::OFFS * xv[h][5], -F::OFFS * xv[h][7]};
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t v = qq[j];
                 const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
-                Dv = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[h][j]),
-                                                             __builtin_bit_cast(bf16x8_t, wv), Dv, 0, 0, 0);
+                if (F::GS == 32 || j < 2)
+                    DA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[h][j]),
+                                                                 __builtin_bit_cast(bf16x8_t, wv), DA, 0, 0, 0);
+                else
+                    DB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[h][j]),
+                                                                 __builtin_bit_cast(bf16x8_t, wv), DB, 0, 0, 0);
             }
-            res += apply_groups<FMT>(hd[u], h, Dv, xv[h]);
+            res += apply_groups<FMT>(hd[u], h, DA, DB, xv[h]);
         }
         // the first block column writes the cell, later ones add to it (no zero fill, no read)
         if (c_ci == 0) *cell = res;
@@ -404,7 +453,7 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     a.cols_base = nblocks / NW;
     a.cols_rem = nblocks % NW;
     const int ncols_max = a.cols_base + (a.cols_rem ? 1 : 0);
-    const size_t x_bytes = ((size_t)NW * ncols_max * (a.nslot * 32 + 8) + 4 * NW) * 16;
+    const size_t x_bytes = ((size_t)NW * ncols_max * (a.nslot * 32 + Fmt<FMT>::NG) + 4 * NW) * 16;
     if (x_bytes + (size_t)NW * 256 > 160 * 1024) return fail(TFQ_ERR_SHAPE, "gemv: K too large for the LDS activation stage");
     // tiles per workgroup: one round of workgroups over the compute units where LDS allows it;
     // every workgroup stays inside one matrix
@@ -431,11 +480,13 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     k.K = a.K; k.y_bf16 = a.y_bf16; k.nslot = a.nslot; k.tiles_per_wg = T;
     k.cols_base = a.cols_base; k.cols_rem = a.cols_rem;
     const int full_items = a.cols_base * T;  // units of a wavefront with the fewest block columns in a full workgroup
-    const int wd = full_items >= 4 ? 4 : full_items >= 2 ? 2 : 1;
+    // formats with a 32-byte header hold two more registers per unit in flight: at most two units
+    const int wd = full_items >= 4 && Fmt<FMT>::HV == 1 ? 4 : full_items >= 2 ? 2 : 1;
     using Kernel = void (*)(GemvKernArgs, const void*);
+    constexpr int WDMAX = Fmt<FMT>::HV == 1 ? 4 : 2;
     static const Kernel kernels[2][3] = {
-        {gemv4_kernel<FMT, false, 1>, gemv4_kernel<FMT, false, 2>, gemv4_kernel<FMT, false, 4>},
-        {gemv4_kernel<FMT, true, 1>, gemv4_kernel<FMT, true, 2>, gemv4_kernel<FMT, true, 4>}};
+        {gemv4_kernel<FMT, false, 1>, gemv4_kernel<FMT, false, 2>, gemv4_kernel<FMT, false, WDMAX>},
+        {gemv4_kernel<FMT, true, 1>, gemv4_kernel<FMT, true, 2>, gemv4_kernel<FMT, true, WDMAX>}};
     const int xi = a.x_f32 ? 1 : 0, wi = wd == 4 ? 2 : wd == 2 ? 1 : 0;
     const Kernel kern = kernels[xi][wi];
     // Raise the dynamic-LDS limit once per kernel (not per launch: the call is
@@ -501,6 +552,10 @@ int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int 
     switch (canonical(ws[0]->fmt)) {
         case TFQ_Q_G_4: return gemv4_batched<TFQ_Q_G_4>(a, x, x_dtype, B, y_dtype, s);
         case TFQ_B32S4: return gemv4_batched<TFQ_B32S4>(a, x, x_dtype, B, y_dtype, s);
+        case TFQ_Q_G_3: return gemv4_batched<TFQ_Q_G_3>(a, x, x_dtype, B, y_dtype, s);
+        case TFQ_Q_G_2: return gemv4_batched<TFQ_Q_G_2>(a, x, x_dtype, B, y_dtype, s);
+        case TFQ_SB256A3: return gemv4_batched<TFQ_SB256A3>(a, x, x_dtype, B, y_dtype, s);
+        case TFQ_SB256A2: return gemv4_batched<TFQ_SB256A2>(a, x, x_dtype, B, y_dtype, s);
         default:
             return fail(TFQ_ERR_FORMAT, std::string("gemv: no kernel for format ") + tfq_format_name(ws[0]->fmt));
     }

@@ -72,16 +72,33 @@ int ensure_device();  // TFQ_OK once a gfx950 device is current and tables are l
 
 // Device layouts of a packed matrix.
 //   Wire:    the payload as the codec writes it, N rows of K/256 consecutive blocks.
-//   Tiled16: for the 4-bit matmul formats (144-byte blocks).  Rows are grouped in
-//            tiles of 16 (the last tile is zero padded); the 16 blocks that a tile
-//            holds at one block column form a 2304-byte unit
-//              [ 64 x 16 B codes of k-step 0 ][ 64 x 16 B codes of k-step 1 ][ 16 x 16 B headers ]
-//            where code slot l = n + 16 q holds group q (k-step 0) or q + 4
-//            (k-step 1) of row n, and header slot n is row n's 16-byte block
-//            header.  Units are ordered tile-major.  Same bytes as the wire
-//            layout (apart from the padding rows), permuted so that one
-//            wavefront reads one unit as a contiguous run.
+//   Tiled16: for the formats with 2- to 4-bit codes and per-group scales.  Rows are
+//            grouped in tiles of 16 (the last tile is zero padded); the 16 blocks
+//            that a tile holds at one block column form a unit of 2048 + 16 HB bytes
+//              [ 64 x 16 B codes of k-step 0 ][ 64 x 16 B codes of k-step 1 ][ 16 x HB B headers ]
+//            where code slot l = n + 16 q holds the 32 codes k = 32 (q + 4 kstep) .. + 31
+//            of row n as nibbles (code 2j in the low half of byte j), and header
+//            slot n holds row n's block header, the wire bytes behind the codes,
+//            zero padded to HB = 16 or 32 bytes.  2- and 3-bit codes are widened to
+//            nibbles here (the matmul kernel turns a nibble into a bf16 operand with
+//            one operation; the wire bit streams straddle every register boundary).
+//            Units are ordered tile-major, so one wavefront reads one unit as a
+//            contiguous run.  For the 4-bit formats this is a permutation of the
+//            wire bytes.
 enum : int { TFQ_LAYOUT_WIRE = 0, TFQ_LAYOUT_TILED16 = 1 };
+
+namespace tfq {
+// header bytes per row and block in the Tiled16 layout; 0 = the format stays in wire order
+__host__ __device__ constexpr int tiled_header_bytes(int fmt) {
+    switch (fmt) {
+        case TFQ_Q_G_4: case TFQ_Q_4_5: case TFQ_Q_G_4_5: case TFQ_B32S4:
+        case TFQ_Q_G_3: case TFQ_Q_3_5: case TFQ_Q_G_3_5: return 16;
+        case TFQ_Q_G_2: case TFQ_SB256A3: case TFQ_SB256A2: return 32;
+        default: return 0;
+    }
+}
+__host__ __device__ constexpr int tiled_unit_bytes(int fmt) { return 2048 + 16 * tiled_header_bytes(fmt); }
+}  // namespace tfq
 
 struct tfq_weight {
     uint8_t fmt;
@@ -97,8 +114,8 @@ namespace tfq {
 
 // ------------------------------------------------------------- kernel launchers
 int launch_decode(int fmt, const uint8_t* src, int64_t nblocks, float* out, hipStream_t s);
-int launch_tile16(const uint8_t* wire, uint8_t* tiled, int64_t N, int64_t K, hipStream_t s);
-int launch_untile16(const uint8_t* tiled, uint8_t* wire, int64_t N, int64_t K, hipStream_t s);
+int launch_tile16(int fmt, const uint8_t* wire, uint8_t* tiled, int64_t N, int64_t K, hipStream_t s);
+int launch_decode_tiled(int fmt, const uint8_t* tiled, int64_t N, int64_t K, float* out, hipStream_t s);
 int launch_encode(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStream_t s);
 int launch_gemv(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype,
                 hipStream_t s);
