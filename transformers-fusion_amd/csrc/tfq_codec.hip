@@ -70,7 +70,8 @@ template <int FMT>
 __global__ __launch_bounds__(256) void tile16_kernel(const uint8_t* __restrict__ wire, uint4* __restrict__ tiled,
                                                      int64_t N, int nblocks, int64_t npieces) {
     constexpr Spec sp = spec_of(FMT);
-    constexpr int HB = tiled_header_bytes(FMT), HP = HB / 16, PIECES = 128 + 16 * HP;
+    constexpr int HB = tiled_header_bytes(FMT), HP = HB / 16, NP = tiled_planes(FMT);
+    constexpr int CP = 128 * NP, PIECES = CP + 16 * HP;  // code pieces, all pieces of a unit
     constexpr uint32_t BB = sp.block_bytes, code_bytes = 256u * sp.bits / 8;
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= npieces) return;
@@ -79,19 +80,25 @@ __global__ __launch_bounds__(256) void tile16_kernel(const uint8_t* __restrict__
     const int64_t tile = unit / nblocks;
     const int blk = (int)(unit - tile * nblocks);
     uint32_t o[4] = {0, 0, 0, 0};
-    if (p < 128) {
-        const int l = p & 63, n = l & 15, g32 = (l >> 4) + 4 * (p >> 6);
+    if (p < CP) {
+        const int plane = p >> 7, l = p & 63, n = l & 15, g32 = (l >> 4) + 4 * ((p >> 6) & 1);
         const int64_t row = tile * 16 + n;
         if (row < N) {
             const uint8_t* src = wire + (row * nblocks + blk) * (int64_t)BB;
 #pragma unroll
             for (int j = 0; j < 32; ++j) {
-                const uint32_t code = stream_bits(src, code_bytes, (uint32_t)(32 * g32 + j) * sp.bits, sp.bits);
+                uint32_t code;
+                if constexpr (NP == 2) {  // int8 code + 128, split into nibbles
+                    const uint32_t u = (uint32_t)src[32 * g32 + j] ^ 0x80u;
+                    code = plane ? u >> 4 : u & 15u;
+                } else {
+                    code = stream_bits(src, code_bytes, (uint32_t)(32 * g32 + j) * sp.bits, sp.bits);
+                }
                 o[j >> 3] |= code << (4 * (j & 7));
             }
         }
     } else {
-        const int n = (p - 128) / HP, part = (p - 128) % HP;
+        const int n = (p - CP) / HP, part = (p - CP) % HP;
         const int64_t row = tile * 16 + n;
         if (row < N) {
             const uint8_t* src = wire + (row * nblocks + blk) * (int64_t)BB;
@@ -121,11 +128,13 @@ __global__ __launch_bounds__(256) void decode_tiled_kernel(const uint8_t* __rest
     const uint32_t g32 = i >> 5, j = i & 31;
     const uint8_t* codes = unit + (g32 >> 2) * 1024 + (n + 16 * (g32 & 3)) * 16;
     const uint32_t idx = (codes[j >> 1] >> ((j & 1u) * 4)) & 15u;
-    const uint8_t* h = unit + 2048 + n * HB;
+    const uint8_t* h = unit + 2048 * tiled_planes(FMT) + n * HB;
     float v;
     if constexpr (sp.codec == Codec::Sym32) {
         const float d = half_bits_to_float((uint32_t)h[2 * g32] | ((uint32_t)h[2 * g32 + 1] << 8));
-        v = (float)((int)idx - 8) * d;
+        int q = (int)idx - 8;
+        if constexpr (tiled_planes(FMT) == 2) q = (int)(idx | (((codes[2048 + (j >> 1)] >> ((j & 1u) * 4)) & 15u) << 4)) - 128;
+        v = (float)q * d;
     } else {
         constexpr uint32_t ng = 256 / sp.gsz;
         constexpr uint32_t sc_bits = ((ng * sp.scb + 7) / 8) * 8;
@@ -186,6 +195,7 @@ int launch_tile16(int fmt, const uint8_t* wire, uint8_t* tiled, int64_t N, int64
     switch (canonical(fmt)) {
         case TFQ_Q_G_4: return run_tile16<TFQ_Q_G_4>(wire, tiled, N, K, s);
         case TFQ_B32S4: return run_tile16<TFQ_B32S4>(wire, tiled, N, K, s);
+        case TFQ_B32S8: return run_tile16<TFQ_B32S8>(wire, tiled, N, K, s);
         case TFQ_Q_G_3: return run_tile16<TFQ_Q_G_3>(wire, tiled, N, K, s);
         case TFQ_Q_G_2: return run_tile16<TFQ_Q_G_2>(wire, tiled, N, K, s);
         case TFQ_SB256A3: return run_tile16<TFQ_SB256A3>(wire, tiled, N, K, s);
@@ -207,6 +217,7 @@ int launch_decode_tiled(int fmt, const uint8_t* tiled, int64_t N, int64_t K, flo
     switch (canonical(fmt)) {
         case TFQ_Q_G_4: return run_decode_tiled<TFQ_Q_G_4>(tiled, N, K, out, s);
         case TFQ_B32S4: return run_decode_tiled<TFQ_B32S4>(tiled, N, K, out, s);
+        case TFQ_B32S8: return run_decode_tiled<TFQ_B32S8>(tiled, N, K, out, s);
         case TFQ_Q_G_3: return run_decode_tiled<TFQ_Q_G_3>(tiled, N, K, out, s);
         case TFQ_Q_G_2: return run_decode_tiled<TFQ_Q_G_2>(tiled, N, K, out, s);
         case TFQ_SB256A3: return run_decode_tiled<TFQ_SB256A3>(tiled, N, K, out, s);

@@ -108,15 +108,18 @@ struct GemvKernArgs {
 // Per-format constants of the kernel.
 //   HB   header bytes per row and block in the Tiled16 layout (16 or 32)
 //   GS   weights per scale group (32 or 16)
-//   OFFS what the bf16 operand (128 + code) overshoots the true code value by: the MFMA
-//        accumulator starts at -OFFS * X so that it ends as the dot product with the codes
+//   OFFS what the bf16 operands (128 + nibble) overshoot the true code value by in total: the
+//        MFMA accumulator starts at -OFFS * X so that it ends as the dot product with the codes
 template <int FMT>
 struct Fmt {
     static constexpr int HB = tiled_header_bytes(FMT);
     static constexpr int HV = HB / 16;  // uint4 registers per header
     static constexpr int GS = spec_of(FMT).gsz == 16 ? 16 : 32;
     static constexpr int NG = 256 / GS;  // groups per block: 8 or 16
-    static constexpr float OFFS = FMT == TFQ_B32S4 ? 136.0f : 128.0f;
+    static constexpr int NP = tiled_planes(FMT);  // nibble planes of the codes (2: low and high nibble of code + 128)
+    // 4-bit symmetric: 128 + 8; 8-bit symmetric: code = 16 hi + lo - 128 with both nibbles carrying
+    // +128, so 16 * 128 + 128 + 128; affine: 128
+    static constexpr float OFFS = FMT == TFQ_B32S4 ? 136.0f : FMT == TFQ_B32S8 ? 2304.0f : 128.0f;
 };
 
 // `count` bits at bit `pos` (both compile-time after unrolling) of the little-endian bit string w[0], w[1], ...
@@ -132,18 +135,22 @@ __device__ __forceinline__ uint32_t field(const uint32_t* w, int pos, int count)
 // group's activation sum and (a, c) the group's scale and offset:
 //   affine formats     a = d * sc / top,  c = -dm * mc      (top = 15, 7 or 3)
 //   symmetric format   a = d,             c = 0             (the code offset 8 is part of OFFS)
-// With 32-weight groups DA[r] is the dot product of group r (DB is unused); with 16-weight
-// groups DA[r] / DB[r] are the two halves of 32-slot r, i.e. groups 2r and 2r + 1, and X
-// holds the eight activation sums in group order.
+// With 32-weight groups DA[r] is the dot product of group r; with 16-weight groups DA[r] / DB[r]
+// are the two halves of 32-slot r, i.e. groups 2r and 2r + 1, and X holds the eight activation
+// sums in group order.  For the 8-bit format DA / DB are the low / high nibble planes.
 template <int FMT>
 __device__ __forceinline__ float apply_groups(const uint4* hv, int khalf, f32x4_t DA, f32x4_t DB, const float* X) {
     constexpr Spec sp = spec_of(FMT);
     float res = 0.0f;
-    if constexpr (FMT == TFQ_B32S4) {
+    if constexpr (FMT == TFQ_B32S4 || FMT == TFQ_B32S8) {
         // header: eight binary16 scales, four per k-step; the conversion rides in the multiply-add
         // (v_fma_mix_f32 reads either half of a dword as binary16)
         const f16x2_t s01 = __builtin_bit_cast(f16x2_t, khalf ? hv[0].z : hv[0].x);
         const f16x2_t s23 = __builtin_bit_cast(f16x2_t, khalf ? hv[0].w : hv[0].y);
+        if constexpr (FMT == TFQ_B32S8) {  // DB holds the high-nibble plane's dot products
+#pragma unroll
+            for (int r = 0; r < 4; ++r) DA[r] = __builtin_fmaf(16.0f, DB[r], DA[r]);
+        }
         res = __builtin_fmaf((float)s01.x, DA[0], res);
         res = __builtin_fmaf((float)s01.y, DA[1], res);
         res = __builtin_fmaf((float)s23.x, DA[2], res);
@@ -188,7 +195,8 @@ template <int FMT, bool XF32, int WD>
 __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
-    constexpr int UB = 2048 + 16 * F::HB;  // bytes of a unit
+    constexpr int UB = tiled_unit_bytes(FMT);  // bytes of a unit
+    constexpr int NC = 2 * F::NP;              // 1 KB code pieces of a unit: [plane][k-step]
     constexpr int NG = F::NG, PER = NG / 2;  // scale groups per block / per k-step
     const int K = args.K, nslot = args.nslot, T = args.tiles_per_wg;
     const int cols_base = args.cols_base, cols_rem = args.cols_rem;
@@ -265,10 +273,10 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     const uint8_t* col_ptr = Wm + ((size_t)tile0 * nblocks + (size_t)wave) * UB;
     const uint8_t* f_ptr = col_ptr;
     int f_ci = 0, f_t = 0;
-    const uint32_t off_c = 16u * lane, off_h = 2048u + (uint32_t)F::HB * n;
-    auto fetch = [&](uint4& c0, uint4& c1, uint4 (&hd)[F::HV]) __attribute__((always_inline)) {
-        c0 = *reinterpret_cast<const uint4*>(f_ptr + off_c);
-        c1 = *reinterpret_cast<const uint4*>(f_ptr + off_c + 1024);
+    const uint32_t off_c = 16u * lane, off_h = 1024u * NC + (uint32_t)F::HB * n;
+    auto fetch = [&](uint4 (&cc)[NC], uint4 (&hd)[F::HV]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NC; ++i) cc[i] = *reinterpret_cast<const uint4*>(f_ptr + off_c + 1024 * i);
 #pragma unroll
         for (int i = 0; i < F::HV; ++i) hd[i] = *reinterpret_cast<const uint4*>(f_ptr + off_h + 16 * i);
         f_ptr += tile_stride;
@@ -278,9 +286,9 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
             f_ptr = col_ptr;
         }
     };
-    uint4 c0[WD], c1[WD], hd[WD][F::HV];
+    uint4 cc[WD][NC], hd[WD][F::HV];
 #pragma unroll
-    for (int u = 0; u < WD; ++u) fetch(c0[u], c1[u], hd[u]);
+    for (int u = 0; u < WD; ++u) fetch(cc[u], hd[u]);
 
     // ---- stage this wavefront's activations: bf16 in nibble-pair order, group sums beside them
     const uint32_t ONES = 0x3F803F80u;
@@ -364,7 +372,7 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
         float res = 0.0f;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const uint4 cw = h ? c1[u] : c0[u];
+            const uint4 cw = cc[u][h];
             const uint32_t qq[4] = {cw.x, cw.y, cw.z, cw.w};
             // accumulators start at -OFFS * X; with 16-weight groups dwords 0, 1 and 2, 3 of a
             // 32-slot belong to different groups and get an accumulator each
@@ -386,6 +394,17 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
                     DB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[h][j]),
                                                                  __builtin_bit_cast(bf16x8_t, wv), DB, 0, 0, 0);
             }
+            if constexpr (F::NP == 2) {  // second nibble plane, same activation fragments
+                const uint4 ch = cc[u][2 + h];
+                const uint32_t qh[4] = {ch.x, ch.y, ch.z, ch.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t v = qh[j];
+                    const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
+                    DB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[h][j]),
+                                                                 __builtin_bit_cast(bf16x8_t, wv), DB, 0, 0, 0);
+                }
+            }
             res += apply_groups<FMT>(hd[u], h, DA, DB, xv[h]);
         }
         // the first block column writes the cell, later ones add to it (no zero fill, no read)
@@ -400,7 +419,7 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
 #pragma unroll
         for (int u = 0; u < WD; ++u) {
             consume(u);
-            fetch(c0[u], c1[u], hd[u]);
+            fetch(cc[u], hd[u]);
         }
     }
     TRACE(4);
@@ -481,9 +500,9 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     k.cols_base = a.cols_base; k.cols_rem = a.cols_rem;
     const int full_items = a.cols_base * T;  // units of a wavefront with the fewest block columns in a full workgroup
     // formats with a 32-byte header hold two more registers per unit in flight: at most two units
-    const int wd = full_items >= 4 && Fmt<FMT>::HV == 1 ? 4 : full_items >= 2 ? 2 : 1;
+    constexpr int WDMAX = Fmt<FMT>::HV == 1 && Fmt<FMT>::NP == 1 ? 4 : 2;
+    const int wd = full_items >= 4 && WDMAX == 4 ? 4 : full_items >= 2 ? 2 : 1;
     using Kernel = void (*)(GemvKernArgs, const void*);
-    constexpr int WDMAX = Fmt<FMT>::HV == 1 ? 4 : 2;
     static const Kernel kernels[2][3] = {
         {gemv4_kernel<FMT, false, 1>, gemv4_kernel<FMT, false, 2>, gemv4_kernel<FMT, false, WDMAX>},
         {gemv4_kernel<FMT, true, 1>, gemv4_kernel<FMT, true, 2>, gemv4_kernel<FMT, true, WDMAX>}};
@@ -552,6 +571,7 @@ int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int 
     switch (canonical(ws[0]->fmt)) {
         case TFQ_Q_G_4: return gemv4_batched<TFQ_Q_G_4>(a, x, x_dtype, B, y_dtype, s);
         case TFQ_B32S4: return gemv4_batched<TFQ_B32S4>(a, x, x_dtype, B, y_dtype, s);
+        case TFQ_B32S8: return gemv4_batched<TFQ_B32S8>(a, x, x_dtype, B, y_dtype, s);
         case TFQ_Q_G_3: return gemv4_batched<TFQ_Q_G_3>(a, x, x_dtype, B, y_dtype, s);
         case TFQ_Q_G_2: return gemv4_batched<TFQ_Q_G_2>(a, x, x_dtype, B, y_dtype, s);
         case TFQ_SB256A3: return gemv4_batched<TFQ_SB256A3>(a, x, x_dtype, B, y_dtype, s);

@@ -75,7 +75,7 @@ int ensure_device();  // TFQ_OK once a gfx950 device is current and tables are l
 //   Tiled16: for the formats with 2- to 4-bit codes and per-group scales.  Rows are
 //            grouped in tiles of 16 (the last tile is zero padded); the 16 blocks
 //            that a tile holds at one block column form a unit of 2048 + 16 HB bytes
-//              [ 64 x 16 B codes of k-step 0 ][ 64 x 16 B codes of k-step 1 ][ 16 x HB B headers ]
+//              [ 64 x 16 B codes of k-step 0 ][ 64 x 16 B codes of k-step 1 ] (x nibble planes) [ 16 x HB B headers ]
 //            where code slot l = n + 16 q holds the 32 codes k = 32 (q + 4 kstep) .. + 31
 //            of row n as nibbles (code 2j in the low half of byte j), and header
 //            slot n holds row n's block header, the wire bytes behind the codes,
@@ -91,13 +91,16 @@ namespace tfq {
 // header bytes per row and block in the Tiled16 layout; 0 = the format stays in wire order
 __host__ __device__ constexpr int tiled_header_bytes(int fmt) {
     switch (fmt) {
-        case TFQ_Q_G_4: case TFQ_Q_4_5: case TFQ_Q_G_4_5: case TFQ_B32S4:
+        case TFQ_Q_G_4: case TFQ_Q_4_5: case TFQ_Q_G_4_5: case TFQ_B32S4: case TFQ_B32S8:
         case TFQ_Q_G_3: case TFQ_Q_3_5: case TFQ_Q_G_3_5: return 16;
         case TFQ_Q_G_2: case TFQ_SB256A3: case TFQ_SB256A2: return 32;
         default: return 0;
     }
 }
-__host__ __device__ constexpr int tiled_unit_bytes(int fmt) { return 2048 + 16 * tiled_header_bytes(fmt); }
+// nibble planes of the code area: the 8-bit symmetric format is stored as two, the low and the
+// high nibble of (code + 128), each laid out like a 4-bit format's codes
+__host__ __device__ constexpr int tiled_planes(int fmt) { return fmt == TFQ_B32S8 ? 2 : 1; }
+__host__ __device__ constexpr int tiled_unit_bytes(int fmt) { return 2048 * tiled_planes(fmt) + 16 * tiled_header_bytes(fmt); }
 }  // namespace tfq
 
 struct tfq_weight {
