@@ -25,7 +25,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes moved per algorithmic byte for the GEMV launches of this workload, from
 # rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy kernel (summary under profiles/)
-HBM_TRAFFIC_RATIO = 1.009
+HBM_TRAFFIC_RATIO = 1.0075
 # (name, N, K, input) per decoder layer
 PROJ = [("q", 4096, 4096, "x"), ("k", 1024, 4096, "x"), ("v", 1024, 4096, "x"), ("o", 4096, 4096, "a"),
         ("gate", 14336, 4096, "x"), ("up", 14336, 4096, "x"), ("down", 4096, 14336, "h")]
@@ -45,6 +45,7 @@ def main():
     ap.add_argument("--fmt", default="B32S4")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM figure")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one elementwise kernel that reads and writes 1 GiB (counter calibration)")
     args = ap.parse_args()
@@ -150,9 +151,38 @@ def main():
                      "alg_bytes_per_launch": int(bytes_per_step / launches_per_step)},
     }
 
+    if not args.no_prefill:
+        res["prefill"] = prefill_gemm(tfq, torch, layers[0], gen)
     if not args.no_cpu:
         res["cpu_baseline"] = cpu_baseline(host_layer0, fmt, B, acts, bpw)
     print(json.dumps(res), flush=True)
+
+
+MFMA_PEAK_TFLOPS = 2500.0
+
+
+def prefill_gemm(tfq, torch, layer, gen, M=2048, reps=10):
+    """The prefill GEMM on the same weights: M = 2048 bf16 tokens through gate (14336x4096) and down
+    (4096x14336), bf16 output, fp32 accumulation on the matrix cores.  A side figure, not `value`."""
+    out = {"tokens": M, "peak_tflops": MFMA_PEAK_TFLOPS, "bound": "mfma"}
+    for name in ("gate", "down"):
+        W = layer[name]
+        x = torch.randn(M, W.K, device="cuda", generator=gen).bfloat16()
+        for _ in range(3):
+            y = W.gemm(x, out_dtype=torch.bfloat16)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            y = W.gemm(x, out_dtype=torch.bfloat16)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        tf = 2.0 * M * W.N * W.K / (ms * 1e-3) / 1e12
+        out[name] = {"shape": "%dx%d" % (W.N, W.K), "us": round(ms * 1e3, 1), "tflops": round(tf, 1),
+                     "frac": round(tf / MFMA_PEAK_TFLOPS, 4)}
+        del x, y
+    return out
 
 
 def cpu_baseline(layer, fmt, B, acts, bpw, budget_s=12.0):

@@ -264,28 +264,31 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     TRACE(1);
 
     // ---- unit fetch cursor: a pointer that walks the tiles of a block column, then moves to the
-    // wavefront's next column.  Past the end it keeps walking the last column again (valid units
-    // of this wavefront, cache hits, never used): every fetch is unconditional, so the number of
-    // loads younger than any operand is a compile-time constant, staging waits for the
+    // wavefront's next column.  Past the end it stays on the last unit (requested a moment ago, so
+    // the repeat is served by the caches and never used): every fetch is unconditional, so the
+    // number of loads younger than any operand is a compile-time constant, staging waits for the
     // activations alone and a unit is consumed as soon as IT has arrived (behind a conditional
     // fetch the compiler waits for everything in flight).
     const size_t tile_stride = (size_t)nblocks * UB;
     const uint8_t* col_ptr = Wm + ((size_t)tile0 * nblocks + (size_t)wave) * UB;
     const uint8_t* f_ptr = col_ptr;
-    int f_ci = 0, f_t = 0;
+    int f_t = 0, f_left = nitems;
     const uint32_t off_c = 16u * lane, off_h = 1024u * NC + (uint32_t)F::HB * n;
     auto fetch = [&](uint4 (&cc)[NC], uint4 (&hd)[F::HV]) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < NC; ++i) cc[i] = *reinterpret_cast<const uint4*>(f_ptr + off_c + 1024 * i);
 #pragma unroll
         for (int i = 0; i < F::HV; ++i) hd[i] = *reinterpret_cast<const uint4*>(f_ptr + off_h + 16 * i);
-        f_ptr += tile_stride;
-        if (++f_t == tiles_here) {
-            f_t = 0;
-            if (++f_ci < ncols) col_ptr += (size_t)NW * UB;
-            f_ptr = col_ptr;
+        if (--f_left > 0) {
+            f_ptr += tile_stride;
+            if (++f_t == tiles_here) {
+                f_t = 0;
+                col_ptr += (size_t)NW * UB;
+                f_ptr = col_ptr;
+            }
         }
     };
+    // WD fetches in flight
     uint4 cc[WD][NC], hd[WD][F::HV];
 #pragma unroll
     for (int u = 0; u < WD; ++u) fetch(cc[u], hd[u]);
