@@ -191,8 +191,10 @@ __device__ unsigned long long g_trace[1024 * 16 * 8];
 
 // WD = unit fetches in flight per wavefront; the first WD are requested unconditionally, so the host
 // chooses WD <= the number of units of a full wavefront (a short one re-reads a unit it never uses).
-template <int FMT, bool XF32, int WD>
-__global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin) {
+// SETS = sets of four activation slots that ride in one pass (1, 2 or 4: up to 16 bf16 rows).  More
+// than one set keeps that many A fragments in registers, which fits at 8 wavefronts per workgroup.
+template <int FMT, bool XF32, int WD, int SETS = 1>
+__global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
     constexpr int UB = tiled_unit_bytes(FMT);  // bytes of a unit
@@ -223,9 +225,10 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     TRACE(0);
 
     // LDS: per wavefront and block column, A entries [nslot][2 k-steps][4 slots of 32][4] (uint4) and
-    // group sums [4 slots][NG] (float); then one zero A entry set per wavefront, then the partial sums [T][NW][64].
+    // group sums [4 SETS slots][NG] (float); then one zero A entry set per wavefront, then the partial
+    // sums [T][NW][SETS][64].
     const int a_per_col = nslot * 32;                   // uint4 entries
-    const int col_stride = a_per_col + NG;              // + 4 NG floats of group sums
+    const int col_stride = a_per_col + SETS * NG;       // + 4 SETS NG floats of group sums
     uint4* my = smem + (size_t)wave * ncols_max * col_stride;
     uint4* zero4 = smem + (size_t)NW * ncols_max * col_stride + 4 * wave;  // this wavefront's own zero A entries
     float* part = reinterpret_cast<float*>(smem + (size_t)NW * ncols_max * col_stride + 4 * NW);
@@ -238,14 +241,16 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     // unconditional and staging drops what it does not need).
     constexpr int XP = 4;  // passes whose loads are issued before the weight stream
     const int quad = lane & 31, sl_in_pass = lane >> 5;
-    const int npc = (nslot + 1) >> 1;  // passes per block column
+    // passes per block column: a power of two, so that a pass index splits with shifts
+    const int npc = SETS == 1 ? (nslot + 1) >> 1 : 2 * SETS;
+    const int npc_shift = SETS == 1 ? npc - 1 : SETS == 2 ? 2 : 3;
     const int npass = ncols * npc;
     constexpr int XE = XF32 ? 4 : 2;   // bytes per activation element
     const uint8_t* xbytes = static_cast<const uint8_t*>(xin);
     // per-lane byte offset inside a pass, and the per-pass scalar offset
     auto x_load = [&](int pass, uint4& lo, uint4& hi) __attribute__((always_inline)) {
-        const int ci = npc == 1 ? pass : pass >> 1;
-        const int s0 = npc == 1 ? 0 : (pass & 1) * 2;
+        const int ci = pass >> npc_shift;
+        const int s0 = (pass & (npc - 1)) * 2;
         const int s = min(s0 + sl_in_pass, nslot - 1);
         const int row = XF32 ? s >> 1 : s;
         const uint32_t lane_off = ((uint32_t)row * (uint32_t)K + (uint32_t)quad * 8u) * XE;
@@ -297,8 +302,8 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     const uint32_t ONES = 0x3F803F80u;
     if (lane < 4) zero4[lane] = uint4{0, 0, 0, 0};
     auto stage = [&](int pass, uint4 xlo, uint4 xhi) __attribute__((always_inline)) {
-        const int ci = npc == 1 ? pass : pass >> 1;
-        const int s = (npc == 1 ? 0 : (pass & 1) * 2) + sl_in_pass;
+        const int ci = pass >> npc_shift;
+        const int s = (pass & (npc - 1)) * 2 + sl_in_pass;
         uint4* col = my + (size_t)ci * col_stride;
         float* colX = reinterpret_cast<float*>(col + a_per_col);
         float sum = 0.0f;
@@ -347,74 +352,84 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     // ---- per-lane operand addressing
     // A operand: lane (i = n, kc = q) is non-zero only on the diagonal c == kc of activation row s
     const int s_a = n >> 2, c_a = n & 3;
-    const bool a_live = (c_a == q) && (s_a < nslot);
 
     const uint32_t M = 0x000F000Fu;
     uint32_t C = 0x43004300u;
     asm volatile("" : "+v"(C));  // keep the bias in a VGPR so (v & M) | C is one v_and_or_b32
-    uint4 av[2][4];
-    float xv[2][PER];
+    uint4 av[SETS][2][4];
+    float xv[SETS][2][PER];
     int c_ci = 0, c_t = 0;
-    float* cell = part + wave * 64 + lane;  // this wavefront's cell of tile c_t
+    float* cell = part + wave * SETS * 64 + lane;  // this wavefront's cells of tile c_t, one per slot set
     auto consume = [&](int u) __attribute__((always_inline)) {
         if (c_t == 0) {  // new block column: its two k-steps' A fragments and group sums
             const uint4* col = my + (size_t)c_ci * col_stride;
             const float* colX = reinterpret_cast<const float*>(col + a_per_col);
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const uint4* src = a_live ? col + s_a * 32 + h * 16 + q * 4 : zero4;
+            for (int st = 0; st < SETS; ++st) {
+                const bool live = (c_a == q) && (4 * st + s_a < nslot);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) av[h][j] = src[j];
+                for (int h = 0; h < 2; ++h) {
+                    const uint4* src = live ? col + (4 * st + s_a) * 32 + h * 16 + q * 4 : zero4;
 #pragma unroll
-                for (int t = 0; t < PER; t += 4) {
-                    const float4 f = *reinterpret_cast<const float4*>(colX + q * NG + h * PER + t);
-                    xv[h][t] = f.x; xv[h][t + 1] = f.y; xv[h][t + 2] = f.z; xv[h][t + 3] = f.w;
+                    for (int j = 0; j < 4; ++j) av[st][h][j] = src[j];
+#pragma unroll
+                    for (int t = 0; t < PER; t += 4) {
+                        const float4 f = *reinterpret_cast<const float4*>(colX + (4 * st + q) * NG + h * PER + t);
+                        xv[st][h][t] = f.x; xv[st][h][t + 1] = f.y; xv[st][h][t + 2] = f.z; xv[st][h][t + 3] = f.w;
+                    }
                 }
             }
         }
-        float res = 0.0f;
+        float res[SETS];
+#pragma unroll
+        for (int st = 0; st < SETS; ++st) res[st] = 0.0f;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const uint4 cw = cc[u][h];
-            const uint32_t qq[4] = {cw.x, cw.y, cw.z, cw.w};
             // accumulators start at -OFFS * X; with 16-weight groups dwords 0, 1 and 2, 3 of a
             // 32-slot belong to different groups and get an accumulator each
-            f32x4_t DA, DB = {0.0f, 0.0f, 0.0f, 0.0f};
-            if constexpr (F::GS == 32) {
-                DA = f32x4_t{-F::OFFS * xv[h][0], -F::OFFS * xv[h][1], -F::OFFS * xv[h][2], -F::OFFS * xv[h][3]};
-            } else {
-                DA = f32x4_t{-F::OFFS * xv[h][0], -F::OFFS * xv[h][2], -F::OFFS * xv[h][4], -F::OFFS * xv[h][6]};
-                DB = f32x4_t{-F::OFFS * xv[h][1], -F::OFFS * xv[h][3], -F::OFFS * xv[h][5], -F::OFFS * xv[h][7]};
-            }
+            f32x4_t DA[SETS], DB[SETS];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t v = qq[j];
-                const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
-                if (F::GS == 32 || j < 2)
-                    DA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[h][j]),
-                                                                 __builtin_bit_cast(bf16x8_t, wv), DA, 0, 0, 0);
-                else
-                    DB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[h][j]),
-                                                                 __builtin_bit_cast(bf16x8_t, wv), DB, 0, 0, 0);
-            }
-            if constexpr (F::NP == 2) {  // second nibble plane, same activation fragments
-                const uint4 ch = cc[u][2 + h];
-                const uint32_t qh[4] = {ch.x, ch.y, ch.z, ch.w};
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint32_t v = qh[j];
-                    const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
-                    DB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[h][j]),
-                                                                 __builtin_bit_cast(bf16x8_t, wv), DB, 0, 0, 0);
+            for (int st = 0; st < SETS; ++st) {
+                const float* X = xv[st][h];
+                DB[st] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                if constexpr (F::GS == 32) {
+                    DA[st] = f32x4_t{-F::OFFS * X[0], -F::OFFS * X[1], -F::OFFS * X[2], -F::OFFS * X[3]};
+                } else {
+                    DA[st] = f32x4_t{-F::OFFS * X[0], -F::OFFS * X[2], -F::OFFS * X[4], -F::OFFS * X[6]};
+                    DB[st] = f32x4_t{-F::OFFS * X[1], -F::OFFS * X[3], -F::OFFS * X[5], -F::OFFS * X[7]};
                 }
             }
-            res += apply_groups<FMT>(hd[u], h, DA, DB, xv[h]);
+#pragma unroll
+            for (int pl = 0; pl < F::NP; ++pl) {  // nibble planes: the second one accumulates into DB
+                const uint4 cw = cc[u][2 * pl + h];
+                const uint32_t qq[4] = {cw.x, cw.y, cw.z, cw.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t v = qq[j];
+                    const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
+                    const bool second = pl == 1 || (F::GS == 16 && j >= 2);
+#pragma unroll
+                    for (int st = 0; st < SETS; ++st) {
+                        if (!second)
+                            DA[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[st][h][j]),
+                                                                             __builtin_bit_cast(bf16x8_t, wv), DA[st], 0, 0, 0);
+                        else
+                            DB[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[st][h][j]),
+                                                                             __builtin_bit_cast(bf16x8_t, wv), DB[st], 0, 0, 0);
+                    }
+                }
+            }
+#pragma unroll
+            for (int st = 0; st < SETS; ++st) res[st] += apply_groups<FMT>(hd[u], h, DA[st], DB[st], xv[st][h]);
         }
-        // the first block column writes the cell, later ones add to it (no zero fill, no read)
-        if (c_ci == 0) *cell = res;
-        else *cell += res;
-        cell += NW * 64;
-        if (++c_t == tiles_here) { c_t = 0; ++c_ci; cell = part + wave * 64 + lane; }
+        // the first block column writes the cells, later ones add to them (no zero fill, no read)
+#pragma unroll
+        for (int st = 0; st < SETS; ++st) {
+            if (c_ci == 0) cell[st * 64] = res[st];
+            else cell[st * 64] += res[st];
+        }
+        cell += NW * SETS * 64;
+        if (++c_t == tiles_here) { c_t = 0; ++c_ci; cell = part + wave * SETS * 64 + lane; }
     };
     // Units are taken in groups of WD; only the last group can be partial.
     const int groups = (nitems + WD - 1) / WD;
@@ -437,7 +452,7 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     // run this: instructions issued by all sixteen wavefronts would cost four times as long per SIMD.
     constexpr int rows_per_out = XF32 ? 2 : 1;  // fp32 input: high and low part live in adjacent activation rows
     const int nb = nslot / rows_per_out;
-    const int bshift = nb > 2 ? 2 : nb - 1;  // log2 of nb rounded up to a power of two
+    const int bshift = nb > 8 ? 4 : nb > 4 ? 3 : nb > 2 ? 2 : nb - 1;  // log2 of nb rounded up to a power of two
     const int nout = tiles_here << (4 + bshift);
     TRACE(5);
     __syncthreads();
@@ -446,11 +461,12 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
         const int t = o >> (4 + bshift), b = (o >> 4) & ((1 << bshift) - 1), nn = o & 15;
         const int row = (tile0 + t) * 16 + nn;
         if (b >= nb || row >= nrm) continue;
-        const float* src = part + t * NW * 64 + b * rows_per_out * 16 + nn;
+        const int s0 = b * rows_per_out;  // first activation slot of the output row
+        const float* src = part + (t * NW * SETS + (s0 >> 2)) * 64 + (s0 & 3) * 16 + nn;
         float v = 0.0f;
         for (int w = 0; w < NW; ++w) {
 #pragma unroll
-            for (int h = 0; h < rows_per_out; ++h) v += src[w * 64 + h * 16];
+            for (int h = 0; h < rows_per_out; ++h) v += src[w * SETS * 64 + h * 16];
         }
         const size_t off = (size_t)b * (size_t)nrm + (size_t)row;
         if (y_bf16) reinterpret_cast<unsigned short*>(ym)[off] = (unsigned short)bf16_rne(v);
@@ -459,24 +475,36 @@ __global__ __launch_bounds__(1024) void gemv4_kernel(GemvKernArgs args, const vo
     TRACE(7);
 }
 
+// Formats whose kernel is also built with several slot sets per pass (up to 16 bf16 rows).
 template <int FMT>
-int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
-    const int nblocks = a.K >> 8;
+constexpr bool kWide = FMT == TFQ_B32S4 || FMT == TFQ_B32S8 || FMT == TFQ_Q_G_4;
+
+struct GemvPlan {
+    int NW, T, sets;
+    size_t lds;
+};
+
+// Workgroup shape for `nslot` activation slots; lds == 0 if they do not fit in LDS.
+template <int FMT>
+GemvPlan plan_gemv4(const GemvArgs& a, int nslot) {
     constexpr int num_cu = 256;  // compute units of an MI355X
-    // wavefronts per workgroup: the count in 8..16 that splits the block columns most evenly
-    int NW = nblocks < 16 ? nblocks : 16;
-    if (nblocks > 16) {
+    const int nblocks = a.K >> 8;
+    GemvPlan p{};
+    p.sets = nslot <= 4 ? 1 : nslot <= 8 ? 2 : 4;
+    // wavefronts per workgroup: the count in max/2..max that splits the block columns most evenly;
+    // several slot sets need the registers of two wavefronts, so at most 8 then
+    const int max_nw = p.sets == 1 ? 16 : 8;
+    p.NW = nblocks < max_nw ? nblocks : max_nw;
+    if (nblocks > max_nw) {
         int best_waste = 1 << 30;
-        for (int w = 16; w >= 8; --w) {
+        for (int w = max_nw; w >= max_nw / 2; --w) {
             const int waste = (nblocks + w - 1) / w * w - nblocks;
-            if (waste < best_waste) { best_waste = waste; NW = w; }
+            if (waste < best_waste) { best_waste = waste; p.NW = w; }
         }
     }
-    a.cols_base = nblocks / NW;
-    a.cols_rem = nblocks % NW;
-    const int ncols_max = a.cols_base + (a.cols_rem ? 1 : 0);
-    const size_t x_bytes = ((size_t)NW * ncols_max * (a.nslot * 32 + Fmt<FMT>::NG) + 4 * NW) * 16;
-    if (x_bytes + (size_t)NW * 256 > 160 * 1024) return fail(TFQ_ERR_SHAPE, "gemv: K too large for the LDS activation stage");
+    const int ncols_max = (nblocks + p.NW - 1) / p.NW;
+    const size_t x_bytes = ((size_t)p.NW * ncols_max * (nslot * 32 + p.sets * Fmt<FMT>::NG) + 4 * p.NW) * 16;
+    const size_t per_tile = (size_t)p.NW * p.sets * 256;
     // tiles per workgroup: one round of workgroups over the compute units where LDS allows it;
     // every workgroup stays inside one matrix
     auto grid_for = [&](int T) {
@@ -485,9 +513,22 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
         return g;
     };
     int T = (a.ntiles + num_cu - 1) / num_cu;
-    while (grid_for(T) > num_cu && x_bytes + (size_t)(T + 1) * NW * 256 <= 160 * 1024) ++T;
-    while (T > 1 && x_bytes + (size_t)T * NW * 256 > 160 * 1024) --T;
-    const size_t lds = x_bytes + (size_t)T * NW * 256;
+    while (grid_for(T) > num_cu && x_bytes + (size_t)(T + 1) * per_tile <= 160 * 1024) ++T;
+    while (T > 1 && x_bytes + (size_t)T * per_tile > 160 * 1024) --T;
+    p.T = T;
+    p.lds = x_bytes + (size_t)T * per_tile;
+    if (p.lds > 160 * 1024) p.lds = 0;
+    return p;
+}
+
+template <int FMT>
+int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
+    const int nblocks = a.K >> 8;
+    const GemvPlan p = plan_gemv4<FMT>(a, a.nslot);
+    if (p.lds == 0) return fail(TFQ_ERR_SHAPE, "gemv: K too large for the LDS activation stage");
+    const int NW = p.NW, T = p.T;
+    a.cols_base = nblocks / NW;
+    a.cols_rem = nblocks % NW;
     a.tiles_per_wg = T;
     GemvKernArgs k{};
     k.W0 = a.W[0]; k.W1 = a.W[1]; k.W2 = a.W[2]; k.W3 = a.W[3];
@@ -499,10 +540,12 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
         ends[m] = m < a.nmat ? g : 0x7FFFFFFF;
     }
     k.g0 = ends[0]; k.g1 = ends[1]; k.g2 = ends[2];
+    int grid = g;
+    if (a.nmat == 4) grid += ((a.nrows[3] + 15) / 16 + T - 1) / T;
     k.K = a.K; k.y_bf16 = a.y_bf16; k.nslot = a.nslot; k.tiles_per_wg = T;
     k.cols_base = a.cols_base; k.cols_rem = a.cols_rem;
     const int full_items = a.cols_base * T;  // units of a wavefront with the fewest block columns in a full workgroup
-    // formats with a 32-byte header hold two more registers per unit in flight: at most two units
+    // formats with a 32-byte header or two nibble planes hold more registers per unit in flight: at most two units
     constexpr int WDMAX = Fmt<FMT>::HV == 1 && Fmt<FMT>::NP == 1 ? 4 : 2;
     const int wd = full_items >= 4 && WDMAX == 4 ? 4 : full_items >= 2 ? 2 : 1;
     using Kernel = void (*)(GemvKernArgs, const void*);
@@ -510,27 +553,41 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
         {gemv4_kernel<FMT, false, 1>, gemv4_kernel<FMT, false, 2>, gemv4_kernel<FMT, false, WDMAX>},
         {gemv4_kernel<FMT, true, 1>, gemv4_kernel<FMT, true, 2>, gemv4_kernel<FMT, true, WDMAX>}};
     const int xi = a.x_f32 ? 1 : 0, wi = wd == 4 ? 2 : wd == 2 ? 1 : 0;
-    const Kernel kern = kernels[xi][wi];
+    Kernel kern = kernels[xi][wi];
+    int slot = xi * 3 + wi;  // which kernel's LDS limit is being raised
+    if constexpr (kWide<FMT>) {
+        if (p.sets > 1) {
+            kern = p.sets == 2 ? gemv4_kernel<FMT, false, 2, 2> : gemv4_kernel<FMT, false, 1, 4>;
+            slot = p.sets == 2 ? 6 : 7;
+        }
+    }
     // Raise the dynamic-LDS limit once per kernel (not per launch: the call is
     // not allowed while a stream is being captured into a graph).
-    static bool lds_limit_raised[2][3] = {};
-    if (!lds_limit_raised[xi][wi]) {
+    static bool lds_limit_raised[8] = {};
+    if (!lds_limit_raised[slot]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
-        lds_limit_raised[xi][wi] = true;
+        lds_limit_raised[slot] = true;
     }
-    hipLaunchKernelGGL(kern, dim3(grid_for(T)), dim3(64 * NW), lds, s, k, x);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), p.lds, s, k, x);
     return hip_fail(hipGetLastError(), "gemv launch");
 }
 
 template <int FMT>
 int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t s) {
-    // One launch carries four bf16 activation rows (two fp32 rows).
+    // One launch carries four bf16 activation rows (two fp32 rows); for the formats built with
+    // several slot sets, up to sixteen bf16 rows when their staged activations fit in LDS.
     const size_t xe = xd == TFQ_F32 ? 4 : 2, ye = yd == TFQ_F32 ? 4 : 2;
-    const int step = xd == TFQ_F32 ? 2 : 4;
     a.y_bf16 = yd == TFQ_BF16;
     a.x_f32 = xd == TFQ_F32;
+    int step = a.x_f32 ? 2 : 4;
+    if constexpr (kWide<FMT>) {
+        if (!a.x_f32 && B > 4) {
+            for (int rows = 16; rows > 4; rows >>= 1)
+                if (plan_gemv4<FMT>(a, rows).lds != 0) { step = rows; break; }
+        }
+    }
     for (int b0 = 0; b0 < B; b0 += step) {
         const int nb = B - b0 < step ? B - b0 : step;
         GemvArgs ab = a;
