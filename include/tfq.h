@@ -172,6 +172,19 @@ int tfq_lut8_gemm(const uint8_t* idx, const float* codebook, const float* act, f
 int tfq_lut_gemv_batch(int bits, const uint8_t* packed, const void* codebook, float scale, const float* X,
                        float* Y, int M, int N, int K, tfq_stream_t stream);
 
+/* tfq_lutn_gemm: kernel::q3_gemm / q6_gemm / q12_gemm / q24_gemm (include/quant/kernel.h:36-54;
+ *   src/kernel/kernel_q3.cpp:27-72, kernel_q6.cpp:28-68, kernel_q12.cpp:30-71, kernel_q24.cpp:47-68):
+ *   out[m*N+n] = sum_k value(m*N+n, k) * act[n*K+k]; the packed row of the pair (m,n) has
+ *   ceil(K*bits/8) bytes, an LSB-first stream of bits-wide indices.  bits = 3 (codebook: 8 floats),
+ *   6 (64 floats), 12 (4096 binary16) or 24 (no codebook: a weight is the top 24 bits of a
+ *   binary32, big-endian).  Synchronises the stream (the table is staged in device memory).
+ * tfq_fp24_encode / tfq_fp24_decode: kernel::q24_encode / q24_decode (kernel_q24.cpp:28-45, 152-193),
+ *   truncation to the top 24 bits.  Device pointers. */
+int tfq_lutn_gemm(int bits, const uint8_t* packed, const void* codebook, const float* act, float* out, int M,
+                  int N, int K, tfq_stream_t stream);
+int tfq_fp24_encode(const float* w, uint8_t* packed, int64_t count, tfq_stream_t stream);
+int tfq_fp24_decode(const uint8_t* packed, float* w, int64_t count, tfq_stream_t stream);
+
 /* ---- device memory for hosts without a HIP toolchain ---------------------------------
  * The reference's operators take host pointers (include/quant/kernel.h:24-54); a
  * caller compiled without HIP moves its buffers with these.  tfq_malloc returns

@@ -8,6 +8,8 @@
 //   quant::quantize_block_all / dequantize_block_all / block_claimed_bytes /
 //   block_actual_bpw                 include/quant/block_codec.h:69-83   (src/codec/block_codec.cpp)
 //   quant::kernel::quant4_gemm / quant8_gemm   include/quant/kernel.h:24-34   (src/kernel/kernel_quant{4,8}.cpp)
+//   quant::kernel::q3_gemm / q6_gemm / q12_gemm / q24_gemm / q24_encode / q24_decode
+//                                    include/quant/kernel.h:36-54   (src/kernel/kernel_q{3,6,12,24}.cpp)
 //   quant::adapters::prod::gemv_quant*_tiled / _batch
 //                                    include/quant/kernel_production.h:25-51 (src/kernel/kernel_production.cpp)
 //   tfq::BlockRowMatmul              the call shape of Qwen35Engine::gemm,
@@ -49,6 +51,15 @@ void quant8_gemm(const uint8_t* indices, const float* codebook, const float* act
                  int N, int K);
 void quant4_gemm(const uint8_t* packed_indices, const uint16_t* codebook, const float* activations, float* output,
                  int M, int N, int K);
+void q3_gemm(const uint8_t* packed_indices, const float* codebook, const float* activations, float* output, int M, int N,
+             int K);
+void q6_gemm(const uint8_t* packed_indices, const float* codebook, const float* activations, float* output, int M, int N,
+             int K);
+void q12_gemm(const uint8_t* packed_indices, const uint16_t* codebook_fp16, const float* activations, float* output,
+              int M, int N, int K);
+void q24_gemm(const uint8_t* packed_weights, const float* activations, float* output, int M, int N, int K);
+void q24_encode(const float* weights, uint8_t* packed, int count);
+void q24_decode(const uint8_t* packed, float* weights, int count);
 }  // namespace kernel
 
 namespace adapters {

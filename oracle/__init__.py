@@ -90,6 +90,9 @@ lib.orc_moe_ffn.argtypes = [C.c_uint8, C.POINTER(_u8p), C.POINTER(_u8p), C.POINT
 lib.orc_quant4_gemm.argtypes = [_u8p, C.POINTER(C.c_uint16), _f32p, _f32p, C.c_int, C.c_int, C.c_int]
 lib.orc_quant8_gemm.argtypes = [_u8p, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
 lib.orc_lut_gemv_batch.argtypes = [C.c_int, _u8p, C.c_void_p, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+lib.orc_lutn_gemm.argtypes = [C.c_int, _u8p, C.c_void_p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+lib.orc_fp24_encode.argtypes = [_f32p, _u8p, C.c_int64]
+lib.orc_fp24_decode.argtypes = [_u8p, _f32p, C.c_int64]
 lib.orc_comp8_table.argtypes = [_f32p]
 
 THREADS = min(16, os.cpu_count() or 1)
@@ -280,6 +283,38 @@ def lut_gemv_batch(bits: int, packed, cb, scale: float, X, M: int, N: int, K: in
     return out
 
 
+def _lutn_codebook(bits, cb):
+    if bits == 24:
+        return None, C.c_void_p(0)
+    cb = np.ascontiguousarray(cb, np.uint16 if bits == 12 else np.float32)
+    assert cb.size == 1 << bits
+    return cb, C.c_void_p(cb.ctypes.data)
+
+
+def lutn_gemm(bits: int, packed, cb, act, M: int, N: int, K: int) -> np.ndarray:
+    """q3_gemm / q6_gemm / q12_gemm / q24_gemm (scalar semantics): packed row per (m, n), activation row n."""
+    packed = np.ascontiguousarray(packed, np.uint8)
+    act = _f32(act)
+    keep, cbp = _lutn_codebook(bits, cb)
+    out = np.empty((M, N), np.float32)
+    lib.orc_lutn_gemm(bits, _ptr(packed, _u8p), cbp, _ptr(act, _f32p), _ptr(out, _f32p), M, N, K)
+    return out
+
+
+def fp24_encode(w) -> np.ndarray:
+    w = _f32(w).reshape(-1)
+    out = np.empty(3 * w.size, np.uint8)
+    lib.orc_fp24_encode(_ptr(w, _f32p), _ptr(out, _u8p), w.size)
+    return out
+
+
+def fp24_decode(packed) -> np.ndarray:
+    packed = np.ascontiguousarray(packed, np.uint8)
+    out = np.empty(packed.size // 3, np.float32)
+    lib.orc_fp24_decode(_ptr(packed, _u8p), _ptr(out, _f32p), out.size)
+    return out
+
+
 # ------------------------------------------------------------ compiled reference
 if ref is not None:
     ref.ref_quantize_block.restype = C.c_long
@@ -365,3 +400,24 @@ def ref_quant8_gemm(idx, cb256, act, M, N, K) -> np.ndarray:
     out = np.empty((M, N), np.float32)
     ref.ref_quant8_gemm(_ptr(idx, _u8p), _ptr(cb256, _f32p), _ptr(act, _f32p), _ptr(out, _f32p), M, N, K)
     return out
+
+
+def ref_lutn_gemm(bits: int, packed, cb, act, M, N, K) -> np.ndarray:
+    packed = np.ascontiguousarray(packed, np.uint8)
+    act = _f32(act)
+    keep, cbp = _lutn_codebook(bits, cb)
+    out = np.empty((M, N), np.float32)
+    ref.ref_lutn_gemm.argtypes = [C.c_int, _u8p, C.c_void_p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+    ref.ref_lutn_gemm(bits, _ptr(packed, _u8p), cbp, _ptr(act, _f32p), _ptr(out, _f32p), M, N, K)
+    return out
+
+
+def ref_fp24_round_trip(w):
+    w = _f32(w).reshape(-1)
+    packed = np.empty(3 * w.size, np.uint8)
+    back = np.empty(w.size, np.float32)
+    ref.ref_fp24_encode.argtypes = [_f32p, _u8p, C.c_int]
+    ref.ref_fp24_decode.argtypes = [_u8p, _f32p, C.c_int]
+    ref.ref_fp24_encode(_ptr(w, _f32p), _ptr(packed, _u8p), w.size)
+    ref.ref_fp24_decode(_ptr(packed, _u8p), _ptr(back, _f32p), w.size)
+    return packed, back

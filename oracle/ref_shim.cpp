@@ -109,4 +109,12 @@ void ref_gemv_quant8_batch(const uint8_t* w, const float* cb, float scale, const
 }
 int ref_detect_cpu_isa() { return quant::adapters::prod::detect_cpu_isa(); }
 
+void ref_lutn_gemm(int bits, const uint8_t* w, const void* cb, const float* act, float* out, int M, int N, int K) {
+    if (bits == 3) quant::kernel::q3_gemm(w, static_cast<const float*>(cb), act, out, M, N, K);
+    else if (bits == 6) quant::kernel::q6_gemm(w, static_cast<const float*>(cb), act, out, M, N, K);
+    else if (bits == 12) quant::kernel::q12_gemm(w, static_cast<const uint16_t*>(cb), act, out, M, N, K);
+    else quant::kernel::q24_gemm(w, act, out, M, N, K);
+}
+void ref_fp24_encode(const float* w, uint8_t* packed, int count) { quant::kernel::q24_encode(w, packed, count); }
+void ref_fp24_decode(const uint8_t* packed, float* w, int count) { quant::kernel::q24_decode(packed, w, count); }
 }  // extern "C"

@@ -1057,4 +1057,61 @@ void orc_lut_gemv_batch(int bits, const uint8_t* packed, const void* cb, float s
         }
 }
 
+// Packed-row lookup GEMMs with 3-, 6- and 12-bit indices and the 24-bit float rows
+// (q3_gemm_scalar src/kernel/kernel_q3.cpp:27-72, q6_gemm_scalar kernel_q6.cpp:28-68,
+// q12_gemm_scalar kernel_q12.cpp:30-71, q24_gemm_scalar kernel_q24.cpp:47-68):
+// out[m*N+n] = sum_k value(m*N+n, k) * act[n*K+k]; the packed row of the pair (m,n) has
+// ceil(K*bits/8) bytes (3K for 24 bits), indices form an LSB-first bit stream (the reference
+// unpacks 24-bit little-endian groups, which is the same thing), a 24-bit weight is the top
+// three bytes of a binary32, most significant byte first.
+void orc_lutn_gemm(int bits, const uint8_t* packed, const void* cb, const float* act, float* out, int M, int N, int K) {
+    std::vector<float> tab;
+    if (bits == 12) {
+        tab.resize(4096);
+        for (int i = 0; i < 4096; ++i) tab[i] = half_to_float(static_cast<const uint16_t*>(cb)[i]);
+    } else if (bits != 24) {
+        tab.assign(static_cast<const float*>(cb), static_cast<const float*>(cb) + ((size_t)1 << bits));
+    }
+    const size_t row_bytes = ((size_t)K * (size_t)bits + 7) / 8;
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) {
+            const uint8_t* row = packed + ((size_t)m * (size_t)N + (size_t)n) * row_bytes;
+            const float* a = act + (size_t)n * (size_t)K;
+            float s = 0.0f;
+            for (int k = 0; k < K; ++k) {
+                float w;
+                if (bits == 24) {
+                    const uint32_t u = ((uint32_t)row[3 * k] << 24) | ((uint32_t)row[3 * k + 1] << 16) | ((uint32_t)row[3 * k + 2] << 8);
+                    std::memcpy(&w, &u, 4);
+                } else {
+                    const size_t pos = (size_t)k * (size_t)bits;
+                    uint32_t v = 0;
+                    for (size_t b = 0; b < 3; ++b)
+                        if ((pos >> 3) + b < row_bytes) v |= (uint32_t)row[(pos >> 3) + b] << (8 * b);
+                    w = tab[(v >> (pos & 7)) & ((1u << bits) - 1u)];
+                }
+                s += w * a[k];
+            }
+            out[(size_t)m * (size_t)N + (size_t)n] = s;
+        }
+}
+
+// float_to_fp24 / fp24_to_float (src/kernel/kernel_q24.cpp:28-45): truncation, no rounding
+void orc_fp24_encode(const float* w, uint8_t* packed, int64_t count) {
+    for (int64_t i = 0; i < count; ++i) {
+        uint32_t u;
+        std::memcpy(&u, &w[i], 4);
+        packed[3 * i] = (uint8_t)(u >> 24);
+        packed[3 * i + 1] = (uint8_t)(u >> 16);
+        packed[3 * i + 2] = (uint8_t)(u >> 8);
+    }
+}
+
+void orc_fp24_decode(const uint8_t* packed, float* w, int64_t count) {
+    for (int64_t i = 0; i < count; ++i) {
+        const uint32_t u = ((uint32_t)packed[3 * i] << 24) | ((uint32_t)packed[3 * i + 1] << 16) | ((uint32_t)packed[3 * i + 2] << 8);
+        std::memcpy(&w[i], &u, 4);
+    }
+}
+
 }  // extern "C"

@@ -29,6 +29,14 @@ void drv_quant4_gemm(const uint8_t* w, const uint16_t* cb, const float* act, flo
 void drv_quant8_gemm(const uint8_t* w, const float* cb, const float* act, float* out, int M, int N, int K) {
     quant::kernel::quant8_gemm(w, cb, act, out, M, N, K);
 }
+void drv_lutn_gemm(int bits, const uint8_t* w, const void* cb, const float* act, float* out, int M, int N, int K) {
+    if (bits == 3) quant::kernel::q3_gemm(w, static_cast<const float*>(cb), act, out, M, N, K);
+    if (bits == 6) quant::kernel::q6_gemm(w, static_cast<const float*>(cb), act, out, M, N, K);
+    if (bits == 12) quant::kernel::q12_gemm(w, static_cast<const uint16_t*>(cb), act, out, M, N, K);
+    if (bits == 24) quant::kernel::q24_gemm(w, act, out, M, N, K);
+}
+void drv_q24_encode(const float* w, uint8_t* packed, int count) { quant::kernel::q24_encode(w, packed, count); }
+void drv_q24_decode(const uint8_t* packed, float* w, int count) { quant::kernel::q24_decode(packed, w, count); }
 void drv_gemv_quant_tiled(const uint8_t* w, float s, const float* x, float* y, int M, int K) {
     quant::adapters::prod::gemv_quant_tiled(w, s, x, y, M, K);
 }

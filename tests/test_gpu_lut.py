@@ -57,6 +57,37 @@ def test_lut_gemv_batch(O, tfq, gpu, bits, M, N, K):
     assert rel_err(y.cpu().numpy(), ref) <= TOL
 
 
+@pytest.mark.parametrize("bits", [3, 6, 12, 24])
+@pytest.mark.parametrize("M,N,K", [(1, 1, 8), (3, 4, 64), (3, 4, 37), (2, 16, 4096), (5, 3, 1000), (64, 8, 512)])
+def test_lutn_gemm(O, tfq, gpu, bits, M, N, K):
+    """kernel::q3_gemm / q6_gemm / q12_gemm / q24_gemm (include/quant/kernel.h:36-54)."""
+    import torch
+    print(f"lutn_gemm bits={bits} M={M} N={N} K={K}", flush=True)
+    rs = np.random.RandomState(bits * 100 + K)
+    row_bytes = (K * bits + 7) // 8
+    act = rs.randn(N, K).astype(np.float32)
+    if bits == 24:
+        packed, cb = O.fp24_encode(rs.randn(M * N * K).astype(np.float32)), None
+    else:
+        packed = rs.randint(0, 256, M * N * row_bytes).astype(np.uint8)
+        cb = half_bits(rs.randn(4096)) if bits == 12 else rs.randn(1 << bits).astype(np.float32)
+    ref = O.lutn_gemm(bits, packed, cb, act, M, N, K)
+    y = tfq.lutn_gemm(bits, torch.from_numpy(packed).to(gpu), cb, torch.from_numpy(act).to(gpu), M, N, K)
+    assert rel_err(y.cpu().numpy(), ref) <= TOL
+
+
+@pytest.mark.parametrize("count", [1, 255, 4096, 1000003])
+def test_fp24_encode_decode_bit_exact(O, tfq, gpu, count):
+    import torch
+    print(f"fp24 count={count}", flush=True)
+    rs = np.random.RandomState(count % 1000)
+    w = (rs.randn(count) * 10.0 ** rs.randint(-10, 10, count)).astype(np.float32)
+    packed = tfq.fp24_encode(torch.from_numpy(w).to(gpu))
+    assert np.array_equal(packed.cpu().numpy(), O.fp24_encode(w))
+    back = tfq.fp24_decode(packed).cpu().numpy()
+    assert np.array_equal(back.view(np.uint32), O.fp24_decode(O.fp24_encode(w)).view(np.uint32))
+
+
 def test_lut_rejects_bad_arguments(tfq, gpu):
     import torch
     x = torch.zeros(64, device=gpu)
@@ -65,6 +96,8 @@ def test_lut_rejects_bad_arguments(tfq, gpu):
         tfq.lut_gemv_batch(3, w, np.zeros(16, np.uint16), 1.0, x, 1, 1, 64)
     with pytest.raises(tfq.TfqError):
         tfq.lut4_gemm(w, np.zeros(16, np.uint16), x, 0, 1, 64)
+    with pytest.raises(tfq.TfqError):
+        tfq.lutn_gemm(5, w, np.zeros(32, np.float32), x, 1, 1, 64)
 
 
 def test_device_memory_helpers_round_trip(tfq, gpu):

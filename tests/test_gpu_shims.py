@@ -39,6 +39,9 @@ def drv(gpu):
     d.drv_claimed_bytes.argtypes = [C.c_uint8, C.c_uint32]
     d.drv_quant4_gemm.argtypes = [u8p, C.POINTER(C.c_uint16), f32p, f32p, C.c_int, C.c_int, C.c_int]
     d.drv_quant8_gemm.argtypes = [u8p, f32p, f32p, f32p, C.c_int, C.c_int, C.c_int]
+    d.drv_lutn_gemm.argtypes = [C.c_int, u8p, C.c_void_p, f32p, f32p, C.c_int, C.c_int, C.c_int]
+    d.drv_q24_encode.argtypes = [f32p, u8p, C.c_int]
+    d.drv_q24_decode.argtypes = [u8p, f32p, C.c_int]
     d.drv_gemv_quant_tiled.argtypes = [u8p, C.c_float, f32p, f32p, C.c_int, C.c_int]
     d.drv_gemv_quant4_tiled.argtypes = [u8p, C.POINTER(C.c_uint16), C.c_float, f32p, f32p, C.c_int, C.c_int]
     d.drv_gemv_quant8_tiled.argtypes = [u8p, f32p, C.c_float, f32p, f32p, C.c_int, C.c_int]
@@ -110,6 +113,31 @@ def test_lookup_gemms(O, drv):
     act8 = rs.randn(M, K).astype(np.float32)
     drv.drv_quant8_gemm(p8(idx), pf(cb), pf(act8), pf(out), M, N, K)
     assert rel_err(out, O.quant8_gemm(idx, cb, act8, M, N, K)) <= TOL
+
+
+def test_wide_lookup_gemms_and_fp24(O, drv):
+    """q3_gemm / q6_gemm / q12_gemm / q24_gemm / q24_encode / q24_decode (include/quant/kernel.h:36-54)."""
+    rs = np.random.RandomState(8)
+    M, N, K = 3, 5, 200
+    act = rs.randn(N, K).astype(np.float32)
+    w = rs.randn(M * N * K).astype(np.float32)
+    packed24 = np.zeros(3 * w.size, np.uint8)
+    drv.drv_q24_encode(pf(w), p8(packed24), w.size)
+    assert np.array_equal(packed24, O.fp24_encode(w))
+    back = np.zeros_like(w)
+    drv.drv_q24_decode(p8(packed24), pf(back), w.size)
+    assert np.array_equal(back.view(np.uint32), O.fp24_decode(packed24).view(np.uint32))
+    for bits in (3, 6, 12, 24):
+        print(f"shim lutn bits={bits}", flush=True)
+        if bits == 24:
+            packed, cb, cbp = packed24, None, None
+        else:
+            packed = rs.randint(0, 256, M * N * ((K * bits + 7) // 8)).astype(np.uint8)
+            cb = rs.randn(4096).astype(np.float16).view(np.uint16) if bits == 12 else rs.randn(1 << bits).astype(np.float32)
+            cbp = cb.ctypes.data
+        out = np.zeros((M, N), np.float32)
+        drv.drv_lutn_gemm(bits, p8(packed), cbp, pf(act), pf(out), M, N, K)
+        assert rel_err(out, O.lutn_gemm(bits, packed, cb, act, M, N, K)) <= TOL
 
 
 def test_production_gemvs(O, drv):

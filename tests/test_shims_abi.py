@@ -19,6 +19,12 @@ EXPECTED = [
     "_ZN5quant20dequantize_block_allENS_6FormatEPKhmS2_mjPf",
     "_ZN5quant6kernel11quant4_gemmEPKhPKtPKfPfiii",
     "_ZN5quant6kernel11quant8_gemmEPKhPKfS4_Pfiii",
+    "_ZN5quant6kernel7q3_gemmEPKhPKfS4_Pfiii",
+    "_ZN5quant6kernel7q6_gemmEPKhPKfS4_Pfiii",
+    "_ZN5quant6kernel8q12_gemmEPKhPKtPKfPfiii",
+    "_ZN5quant6kernel8q24_gemmEPKhPKfPfiii",
+    "_ZN5quant6kernel10q24_encodeEPKfPhi",
+    "_ZN5quant6kernel10q24_decodeEPKhPfi",
     "_ZN5quant8adapters4prod16gemv_quant_batchEPKhfPKfPfiii",
     "_ZN5quant8adapters4prod16gemv_quant_tiledEPKhfPKfPfiii",
     "_ZN5quant8adapters4prod17gemv_quant4_batchEPKhPKtfPKfPfiii",

@@ -63,6 +63,9 @@ def _load():
         "tfq_lut4_gemm": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
         "tfq_lut8_gemm": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
         "tfq_lut_gemv_batch": (i32, [i32, vp, vp, C.c_float, vp, vp, i32, i32, i32, vp]),
+        "tfq_lutn_gemm": (i32, [i32, vp, vp, vp, vp, i32, i32, i32, vp]),
+        "tfq_fp24_encode": (i32, [vp, vp, i64, vp]),
+        "tfq_fp24_decode": (i32, [vp, vp, i64, vp]),
         "tfq_malloc": (vp, [sz]),
         "tfq_free": (None, [vp]),
         "tfq_copy_to_device": (i32, [vp, vp, sz]),
@@ -273,4 +276,33 @@ def lut_gemv_batch(bits: int, packed, codebook, scale: float, X, M: int, N: int,
         cbp = cb.ctypes.data
     out = torch.empty((N, M), dtype=torch.float32, device=X.device)
     _check(lib().tfq_lut_gemv_batch(bits, packed.data_ptr(), cbp, scale, X.data_ptr(), out.data_ptr(), M, N, K, _stream()))
+    return out
+
+
+def lutn_gemm(bits: int, packed, codebook, act, M: int, N: int, K: int):
+    """kernel::q3_gemm / q6_gemm / q12_gemm / q24_gemm on the device (bits = 3, 6, 12, 24): packed uint8 and
+    act fp32 [N][K] are device tensors, codebook a host array (float32, or uint16 binary16 bits for 12; None for 24)."""
+    import numpy as np
+    import torch
+    cbp = None
+    if bits != 24:
+        cb = np.ascontiguousarray(codebook, np.uint16 if bits == 12 else np.float32)
+        cbp = cb.ctypes.data
+    out = torch.empty((M, N), dtype=torch.float32, device=act.device)
+    _check(lib().tfq_lutn_gemm(bits, packed.data_ptr(), cbp, act.data_ptr(), out.data_ptr(), M, N, K, _stream()))
+    return out
+
+
+def fp24_encode(w):
+    import torch
+    w = w.contiguous().float()
+    out = torch.empty(3 * w.numel(), dtype=torch.uint8, device=w.device)
+    _check(lib().tfq_fp24_encode(w.data_ptr(), out.data_ptr(), w.numel(), _stream()))
+    return out
+
+
+def fp24_decode(packed):
+    import torch
+    out = torch.empty(packed.numel() // 3, dtype=torch.float32, device=packed.device)
+    _check(lib().tfq_fp24_decode(packed.data_ptr(), out.data_ptr(), out.numel(), _stream()))
     return out

@@ -359,6 +359,26 @@ int tfq_lut8_gemm(const uint8_t* idx, const float* codebook, const float* act, f
     return launch_lut8_gemm(idx, codebook, act, out, M, N, K, (hipStream_t)stream);
 }
 
+int tfq_lutn_gemm(int bits, const uint8_t* packed, const void* codebook, const float* act, float* out, int M, int N,
+                  int K, tfq_stream_t stream) {
+    if (bits != 3 && bits != 6 && bits != 12 && bits != 24) return fail(TFQ_ERR_ARG, "tfq_lutn_gemm: bits must be 3, 6, 12 or 24");
+    if (bits != 24 && !codebook) return fail(TFQ_ERR_ARG, "tfq_lutn_gemm: null codebook");
+    if (int r = check_lut("tfq_lutn_gemm", packed, act, out, M, N, K)) return r;
+    return launch_lutn_gemm(bits, packed, codebook, act, out, M, N, K, (hipStream_t)stream);
+}
+
+int tfq_fp24_encode(const float* w, uint8_t* packed, int64_t count, tfq_stream_t stream) {
+    if (count < 0 || (count > 0 && (!w || !packed))) return fail(TFQ_ERR_ARG, "tfq_fp24_encode: bad arguments");
+    if (int r = ensure_device()) return r;
+    return launch_fp24_convert(true, w, packed, count, (hipStream_t)stream);
+}
+
+int tfq_fp24_decode(const uint8_t* packed, float* w, int64_t count, tfq_stream_t stream) {
+    if (count < 0 || (count > 0 && (!w || !packed))) return fail(TFQ_ERR_ARG, "tfq_fp24_decode: bad arguments");
+    if (int r = ensure_device()) return r;
+    return launch_fp24_convert(false, packed, w, count, (hipStream_t)stream);
+}
+
 int tfq_lut_gemv_batch(int bits, const uint8_t* packed, const void* codebook, float scale, const float* X, float* Y,
                        int M, int N, int K, tfq_stream_t stream) {
     if (bits != 2 && bits != 4 && bits != 8) return fail(TFQ_ERR_ARG, "tfq_lut_gemv_batch: bits must be 2, 4 or 8");

@@ -137,6 +137,9 @@ int launch_lut4_gemm(const uint8_t* packed, const uint16_t* cb16, const float* a
                      hipStream_t s);
 int launch_lut8_gemm(const uint8_t* idx, const float* cb, const float* act, float* out, int M, int N, int K,
                      hipStream_t s);
+int launch_lutn_gemm(int bits, const uint8_t* packed, const void* codebook, const float* act, float* out, int M, int N,
+                     int K, hipStream_t s);
+int launch_fp24_convert(bool encode, const void* src, void* dst, int64_t count, hipStream_t s);
 int launch_lut_gemv_batch(int bits, const uint8_t* packed, const void* cb, float scale, const float* X, float* Y,
                           int M, int Nb, int K, hipStream_t s);
 

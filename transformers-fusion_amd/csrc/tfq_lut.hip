@@ -23,6 +23,8 @@
 
 #include "tfq_internal.hpp"
 
+#include <vector>
+
 namespace tfq {
 
 namespace {
@@ -117,6 +119,76 @@ __global__ __launch_bounds__(kWaves * 64) void lut_rows_kernel(LutArgs a, Table<
     }
 }
 
+// Packed-row lookup operators whose index width does not divide a register: 3, 6 and 12 bits
+// (kernel::q3_gemm, q6_gemm, q12_gemm: src/kernel/kernel_q3.cpp:27-72, kernel_q6.cpp:28-68,
+// kernel_q12.cpp:30-71), and the 24-bit float rows of kernel::q24_gemm (kernel_q24.cpp:28-68).
+// All share quant4_gemm's convention: out[m*N+n] uses packed row (m*N+n), of ceil(K*BITS/8)
+// bytes, against activation row n; indices are an LSB-first bit stream.  One wavefront per
+// packed row; a lane takes 8 consecutive weights, which are exactly BITS bytes.
+// BITS == 24: no table, a weight is the top 24 bits of a binary32, stored big-endian.
+template <int BITS>
+__global__ __launch_bounds__(kWaves * 64) void lutn_rows_kernel(const uint8_t* __restrict__ W, const float* __restrict__ tab_g,
+                                                               const float* __restrict__ X, float* __restrict__ Y,
+                                                               int64_t R, int N, int K) {
+    extern __shared__ float tab[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if constexpr (BITS != 24) {
+        for (int i = threadIdx.x; i < (1 << BITS); i += kWaves * 64) tab[i] = tab_g[i];
+        __syncthreads();
+    }
+    const int64_t r = (int64_t)blockIdx.x * kWaves + wave;
+    if (r >= R) return;
+    const int64_t row_bytes = ((int64_t)K * BITS + 7) / 8;
+    const uint8_t* row = W + r * row_bytes;
+    const float* x = X + (r % N) * (int64_t)K;
+    float acc = 0.0f;
+    for (int k0 = lane * 8; k0 < K; k0 += 64 * 8) {
+        const uint8_t* p = row + (int64_t)k0 * BITS / 8;  // 8 weights start on a byte boundary
+        const int cnt = K - k0 < 8 ? K - k0 : 8;
+        const int64_t avail = row_bytes - (int64_t)k0 * BITS / 8;
+        uint32_t w[BITS / 4 + 1] = {};
+#pragma unroll
+        for (int b = 0; b < BITS; ++b)
+            if (b < avail) w[b >> 2] |= (uint32_t)p[b] << (8 * (b & 3));
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (j >= cnt) break;
+            float v;
+            if constexpr (BITS == 24) {
+                const uint32_t b0 = (w[(3 * j) >> 2] >> (8 * ((3 * j) & 3))) & 0xFFu;
+                const uint32_t b1 = (w[(3 * j + 1) >> 2] >> (8 * ((3 * j + 1) & 3))) & 0xFFu;
+                const uint32_t b2 = (w[(3 * j + 2) >> 2] >> (8 * ((3 * j + 2) & 3))) & 0xFFu;
+                v = __uint_as_float((b0 << 24) | (b1 << 16) | (b2 << 8));
+            } else {
+                const int pos = j * BITS, i = pos >> 5, sh = pos & 31;
+                uint32_t idx = w[i] >> sh;
+                if (sh + BITS > 32) idx |= w[i + 1] << (32 - sh);
+                v = tab[idx & ((1u << BITS) - 1u)];
+            }
+            acc = fmaf(v, x[k0 + j], acc);
+        }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 64);
+    if (lane == 0) Y[r] = acc;
+}
+
+// q24_encode / q24_decode (src/kernel/kernel_q24.cpp:28-45, 152-193): top 24 bits of the binary32, big-endian
+__global__ void fp24_encode_kernel(const float* __restrict__ w, uint8_t* __restrict__ packed, int64_t count) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    const uint32_t u = __float_as_uint(w[i]);
+    packed[3 * i] = (uint8_t)(u >> 24);
+    packed[3 * i + 1] = (uint8_t)(u >> 16);
+    packed[3 * i + 2] = (uint8_t)(u >> 8);
+}
+
+__global__ void fp24_decode_kernel(const uint8_t* __restrict__ packed, float* __restrict__ w, int64_t count) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    w[i] = __uint_as_float(((uint32_t)packed[3 * i] << 24) | ((uint32_t)packed[3 * i + 1] << 16) | ((uint32_t)packed[3 * i + 2] << 8));
+}
+
 template <int BITS, int BT>
 void launch_bt(const LutArgs& a, const Table<(1 << BITS)>& cb, bool vec, hipStream_t s) {
     const dim3 grid((unsigned)((a.R + kWaves - 1) / kWaves)), block(kWaves * 64);
@@ -160,6 +232,45 @@ float half_to_float_host(uint16_t h) {
 }
 
 }  // namespace
+
+// codebook: 8 or 64 floats (3, 6 bits), 4096 binary16 (12 bits), none (24 bits); device scratch for the table
+int launch_lutn_gemm(int bits, const uint8_t* packed, const void* codebook, const float* act, float* out, int M, int N,
+                     int K, hipStream_t s) {
+    const int64_t R = (int64_t)M * N;
+    if ((R + kWaves - 1) / kWaves > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "lookup matmul: too many packed rows for one launch");
+    const dim3 grid((unsigned)((R + kWaves - 1) / kWaves)), block(kWaves * 64);
+    if (bits == 24) {
+        hipLaunchKernelGGL(lutn_rows_kernel<24>, grid, block, 0, s, packed, (const float*)nullptr, act, out, R, N, K);
+        return hip_fail(hipGetLastError(), "lookup matmul launch");
+    }
+    const int entries = 1 << bits;
+    std::vector<float> host(entries);
+    for (int i = 0; i < entries; ++i)
+        host[i] = bits == 12 ? half_to_float_host(static_cast<const uint16_t*>(codebook)[i]) : static_cast<const float*>(codebook)[i];
+    float* tab = nullptr;
+    TFQ_HIP(hipMalloc(&tab, entries * sizeof(float)));
+    int rc = hip_fail(hipMemcpyAsync(tab, host.data(), entries * sizeof(float), hipMemcpyHostToDevice, s), "table upload");
+    if (!rc) rc = hip_fail(hipStreamSynchronize(s), "table upload");  // `host` goes out of scope below
+    if (!rc) {
+        const size_t lds = entries * sizeof(float);
+        if (bits == 3) hipLaunchKernelGGL(lutn_rows_kernel<3>, grid, block, lds, s, packed, tab, act, out, R, N, K);
+        else if (bits == 6) hipLaunchKernelGGL(lutn_rows_kernel<6>, grid, block, lds, s, packed, tab, act, out, R, N, K);
+        else hipLaunchKernelGGL(lutn_rows_kernel<12>, grid, block, lds, s, packed, tab, act, out, R, N, K);
+        rc = hip_fail(hipGetLastError(), "lookup matmul launch");
+        if (!rc) rc = hip_fail(hipStreamSynchronize(s), "lookup matmul");  // the table is freed below
+    }
+    (void)hipFree(tab);
+    return rc;
+}
+
+int launch_fp24_convert(bool encode, const void* src, void* dst, int64_t count, hipStream_t s) {
+    if (count <= 0) return TFQ_OK;
+    const int64_t grid = (count + 255) / 256;
+    if (grid > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "fp24: too many elements for one launch");
+    if (encode) hipLaunchKernelGGL(fp24_encode_kernel, dim3((unsigned)grid), dim3(256), 0, s, (const float*)src, (uint8_t*)dst, count);
+    else hipLaunchKernelGGL(fp24_decode_kernel, dim3((unsigned)grid), dim3(256), 0, s, (const uint8_t*)src, (float*)dst, count);
+    return hip_fail(hipGetLastError(), "fp24 launch");
+}
 
 int launch_lut4_gemm(const uint8_t* packed, const uint16_t* cb16, const float* act, float* out, int M, int N, int K,
                      hipStream_t s) {

@@ -110,6 +110,42 @@ void quant4_gemm(const uint8_t* packed_indices, const uint16_t* codebook, const 
     tfq_copy_to_host(output, dy, (size_t)M * (size_t)N * 4);
 }
 
+static void lutn(int bits, const uint8_t* packed, const void* codebook, const float* activations, float* output, int M,
+                 int N, int K) {
+    if (!packed || !activations || !output || M <= 0 || N <= 0 || K <= 0 || (bits != 24 && !codebook)) return;
+    DeviceBuffers d;
+    const size_t row_bytes = ((size_t)K * (size_t)bits + 7) / 8;
+    const uint8_t* dw = static_cast<const uint8_t*>(d.upload(packed, (size_t)M * (size_t)N * row_bytes));
+    const float* dx = static_cast<const float*>(d.upload(activations, (size_t)N * (size_t)K * 4));
+    float* dy = static_cast<float*>(d.alloc((size_t)M * (size_t)N * 4));
+    if (!dw || !dx || !dy) return;
+    if (tfq_lutn_gemm(bits, dw, codebook, dx, dy, M, N, K, nullptr) != TFQ_OK) return;
+    tfq_copy_to_host(output, dy, (size_t)M * (size_t)N * 4);
+}
+
+void q3_gemm(const uint8_t* p, const float* cb, const float* a, float* o, int M, int N, int K) { lutn(3, p, cb, a, o, M, N, K); }
+void q6_gemm(const uint8_t* p, const float* cb, const float* a, float* o, int M, int N, int K) { lutn(6, p, cb, a, o, M, N, K); }
+void q12_gemm(const uint8_t* p, const uint16_t* cb, const float* a, float* o, int M, int N, int K) { lutn(12, p, cb, a, o, M, N, K); }
+void q24_gemm(const uint8_t* p, const float* a, float* o, int M, int N, int K) { lutn(24, p, nullptr, a, o, M, N, K); }
+
+void q24_encode(const float* weights, uint8_t* packed, int count) {
+    if (!weights || !packed || count <= 0) return;
+    DeviceBuffers d;
+    const float* dw = static_cast<const float*>(d.upload(weights, (size_t)count * 4));
+    uint8_t* dp = static_cast<uint8_t*>(d.alloc((size_t)count * 3));
+    if (!dw || !dp || tfq_fp24_encode(dw, dp, count, nullptr) != TFQ_OK) return;
+    tfq_copy_to_host(packed, dp, (size_t)count * 3);
+}
+
+void q24_decode(const uint8_t* packed, float* weights, int count) {
+    if (!weights || !packed || count <= 0) return;
+    DeviceBuffers d;
+    const uint8_t* dp = static_cast<const uint8_t*>(d.upload(packed, (size_t)count * 3));
+    float* dw = static_cast<float*>(d.alloc((size_t)count * 4));
+    if (!dw || !dp || tfq_fp24_decode(dp, dw, count, nullptr) != TFQ_OK) return;
+    tfq_copy_to_host(weights, dw, (size_t)count * 4);
+}
+
 }  // namespace kernel
 
 namespace adapters {
