@@ -40,10 +40,14 @@ enum { TFQ_F32 = 0, TFQ_BF16 = 1 };
  * and keep their values because they are stored on disk; the four literal
  * formats are appended after FORMAT_COUNT (105). */
 enum {
-    TFQ_Q_4 = 3, TFQ_Q_8 = 5, TFQ_Q_32 = 9,
-    TFQ_Q_G_2 = 38, TFQ_Q_G_3 = 39, TFQ_Q_G_4 = 40, TFQ_Q_G_8 = 42,
-    TFQ_Q_3_5 = 75, TFQ_Q_4_5 = 76, TFQ_Q_8_5 = 78,
-    TFQ_Q_G_3_5 = 84, TFQ_Q_G_4_5 = 85, TFQ_Q_G_8_5 = 87,
+    TFQ_Q_2 = 1, TFQ_Q_4 = 3, TFQ_Q_8 = 5, TFQ_Q_32 = 9,
+    TFQ_Q_G_2 = 38, TFQ_Q_G_3 = 39, TFQ_Q_G_4 = 40, TFQ_Q_G_6 = 41, TFQ_Q_G_8 = 42,
+    TFQ_Q_G_2_K_L = 49, TFQ_Q_G_2_K_M = 50, TFQ_Q_G_2_K_H = 51,
+    TFQ_Q_G_3_K_L = 52, TFQ_Q_G_3_K_M = 53, TFQ_Q_G_3_K_H = 54,
+    TFQ_Q_G_4_K_L = 55, TFQ_Q_G_4_K_M = 56, TFQ_Q_G_4_K_H = 57,
+    TFQ_Q_G_6_K_L = 58, TFQ_Q_G_6_K_M = 59, TFQ_Q_G_6_K_H = 60,
+    TFQ_Q_2_5 = 74, TFQ_Q_3_5 = 75, TFQ_Q_4_5 = 76, TFQ_Q_6_5 = 77, TFQ_Q_8_5 = 78,
+    TFQ_Q_G_2_5 = 83, TFQ_Q_G_3_5 = 84, TFQ_Q_G_4_5 = 85, TFQ_Q_G_6_5 = 86, TFQ_Q_G_8_5 = 87,
     TFQ_B32S4 = 105,   /* 32-group symmetric 4-bit, binary16 scale = absmax/7   */
     TFQ_B32S8 = 106,   /* 32-group symmetric 8-bit, binary16 scale = absmax/127 */
     TFQ_SB256A3 = 107, /* 256-superblock, 16x16 sub-blocks, 6-bit scale + min, 3-bit codes */
@@ -77,8 +81,10 @@ int tfq_block_bytes(uint8_t fmt, uint32_t n, size_t* out);
  * quantize_block_all / dequantize_block_all (include/quant/block_codec.h:69-77),
  * applied to a tensor cut into 256-weight blocks the way
  * FormatRegistry::quantize / dequantize do (src/codec/format_registry.cpp:168-207,
- * 241-290): payloads are concatenated in block order.  n must be a multiple of
- * 256.  dst/src and w/out are device pointers. */
+ * 241-290): payloads are concatenated in block order.  Encoding needs n to be a
+ * multiple of 256; decoding also takes a short last block of n % 256 weights in
+ * the layout the reference's codec chooses for that size (tfq_block_bytes gives
+ * its byte count).  dst/src and w/out are device pointers. */
 int tfq_encode_blocks(uint8_t fmt, const float* w, int64_t n, uint8_t* dst, size_t cap,
                       tfq_stream_t stream);
 int tfq_decode_blocks(uint8_t fmt, const uint8_t* src, size_t bytes, int64_t n, float* out,

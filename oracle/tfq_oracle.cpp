@@ -55,14 +55,16 @@ namespace {
 // Wire ids 0..104 are the reference's (include/quant/types.h:22-66).  The four
 // literal formats are appended after FORMAT_COUNT.
 enum : uint8_t {
-    F_Q_4 = 3, F_Q_8 = 5, F_Q_32 = 9,
-    F_Q_G_2 = 38, F_Q_G_3 = 39, F_Q_G_4 = 40, F_Q_G_8 = 42,
-    F_Q_3_5 = 75, F_Q_4_5 = 76, F_Q_8_5 = 78,
-    F_Q_G_3_5 = 84, F_Q_G_4_5 = 85, F_Q_G_8_5 = 87,
+    F_Q_2 = 1, F_Q_4 = 3, F_Q_8 = 5, F_Q_32 = 9,
+    F_Q_G_2 = 38, F_Q_G_3 = 39, F_Q_G_4 = 40, F_Q_G_6 = 41, F_Q_G_8 = 42,
+    F_Q_G_2_K_L = 49, F_Q_G_2_K_H = 51, F_Q_G_3_K_L = 52, F_Q_G_3_K_H = 54, F_Q_G_4_K_L = 55, F_Q_G_4_K_H = 57,
+    F_Q_G_6_K_L = 58, F_Q_G_6_K_M = 59, F_Q_G_6_K_H = 60,
+    F_Q_2_5 = 74, F_Q_3_5 = 75, F_Q_4_5 = 76, F_Q_6_5 = 77, F_Q_8_5 = 78,
+    F_Q_G_2_5 = 83, F_Q_G_3_5 = 84, F_Q_G_4_5 = 85, F_Q_G_6_5 = 86, F_Q_G_8_5 = 87,
     F_B32S4 = 105, F_B32S8 = 106, F_SB256A3 = 107, F_SB256A2 = 108,
 };
 
-enum class Codec { Raw32, Lattice, Affine, Grp8, Sym32 };
+enum class Codec { Raw32, Lattice, Affine, Grp8, Sym32, Q6K };
 
 struct Spec {
     Codec codec;
@@ -70,11 +72,13 @@ struct Spec {
     int gsz;        // group size (Affine, Sym32)
     int scb, mb;    // scale / min code widths (Affine)
     float claimed;  // claimed bits per weight
+    int tier = 0;   // encoder search tier of the _K_L/_K_M/_K_H ids (0, 1, 2); the wire layout is the base id's
 };
 
 bool spec_for(uint8_t fmt, Spec* s) {
     switch (fmt) {
         case F_Q_32:  *s = {Codec::Raw32, 32, 0, 0, 0, 32.0f}; return true;
+        case F_Q_2:   *s = {Codec::Lattice, 2, 0, 0, 0, 2.0f}; return true;
         case F_Q_4:   *s = {Codec::Lattice, 4, 0, 0, 0, 4.0f}; return true;
         case F_Q_8:   *s = {Codec::Lattice, 8, 0, 0, 0, 8.0f}; return true;
         case F_Q_G_4: case F_Q_4_5: case F_Q_G_4_5:
@@ -84,6 +88,17 @@ bool spec_for(uint8_t fmt, Spec* s) {
         case F_Q_G_2: *s = {Codec::Affine, 2, 16, 4, 4, 2.625f}; return true;
         case F_Q_G_8: case F_Q_8_5: case F_Q_G_8_5:
             *s = {Codec::Grp8, 8, 32, 0, 0, 8.5f}; return true;
+        // Claims below the affine header's size: every block takes the grouped-lattice
+        // fallback layout (src/codec/block_codec.cpp:1408-1411, :1622-1625), so the three
+        // tiers of one width are byte-identical (:2676-2730).
+        case F_Q_2_5: case F_Q_G_2_5: *s = {Codec::Affine, 2, 16, 4, 4, 2.5f}; return true;
+        case F_Q_6_5: case F_Q_G_6_5: *s = {Codec::Affine, 6, 32, 8, 8, 6.5f}; return true;
+        case F_Q_G_2_K_L: case F_Q_G_2_K_L + 1: case F_Q_G_2_K_H: *s = {Codec::Affine, 2, 16, 4, 4, 2.4375f}; return true;
+        case F_Q_G_3_K_L: case F_Q_G_3_K_L + 1: case F_Q_G_3_K_H: *s = {Codec::Affine, 3, 32, 6, 6, 3.4375f}; return true;
+        case F_Q_G_4_K_L: case F_Q_G_4_K_L + 1: case F_Q_G_4_K_H: *s = {Codec::Affine, 4, 32, 6, 6, 4.4375f}; return true;
+        case F_Q_G_6: case F_Q_G_6_K_L: *s = {Codec::Q6K, 6, 16, 8, 0, 6.5625f, 0}; return true;
+        case F_Q_G_6_K_M: *s = {Codec::Q6K, 6, 16, 8, 0, 6.5625f, 1}; return true;
+        case F_Q_G_6_K_H: *s = {Codec::Q6K, 6, 16, 8, 0, 6.5625f, 2}; return true;
         case F_SB256A3: *s = {Codec::Affine, 3, 16, 6, 6, 3.875f}; return true;
         case F_SB256A2: *s = {Codec::Affine, 2, 16, 6, 6, 2.875f}; return true;
         case F_B32S4: *s = {Codec::Sym32, 4, 32, 0, 0, 4.5f}; return true;
@@ -411,6 +426,337 @@ void grp8_decode(const uint8_t* bytes, size_t size, int n, float* out) {
     }
 }
 
+// ----------------------------------------- grouped lattice fallback ("grp16")
+// quant_grp16 / dequant_grp16 (src/codec/block_codec.cpp:739-945): groups of 8
+// weights, a 3-bit scale code per group and one binary16 d, on the plain
+// lattice grid (grid_value).  It is what the affine family degrades to when
+// its header does not fit ceil(claimed * n / 8): tails, and every block of the
+// ids whose claim is below the affine size.  Layout by n and budget:
+//   n < 8, or no room for d:        raw levels, implied d = 1
+//   no room for the group scales:   levels, d in the last two bytes
+//   otherwise:                      levels, n/8 3-bit scales, d, one bit stream
+constexpr int kGrp16 = 8;
+
+float grp16_top(int bits) { return bits == 2 ? 1.5104f : bits == 4 ? 2.7178f : 8.0f; }
+
+// :750-786: 4 x (assign, least-squares refit), +-15 % polish in 5 % steps by plain MSE, closing refit
+void grp16_fit_scale(int bits, const float* w, int cnt, float* s_out) {
+    float maxa = 0.0f;
+    for (int i = 0; i < cnt; ++i) maxa = std::max(maxa, std::fabs(w[i]));
+    float s = (maxa > 1e-30f) ? maxa / grp16_top(bits) : 0.0f;
+    if (!(std::fabs(s) > 1e-30f)) { *s_out = 0.0f; return; }
+    uint32_t idx[256];
+    auto refit = [&]() {
+        double num = 0.0, den = 0.0;
+        for (int i = 0; i < cnt; ++i) {
+            const float l = grid_value(bits, idx[i]);
+            num += (double)w[i] * (double)l;
+            den += (double)l * (double)l;
+        }
+        if (den > 1e-20) s = (float)(num / den);
+    };
+    for (int iter = 0; iter < 4; ++iter) {
+        for (int i = 0; i < cnt; ++i) idx[i] = grid_nearest(w[i] / s, bits);
+        refit();
+    }
+    float best_s = s;
+    double best = 1e300;
+    for (int k = -3; k <= 3; ++k) {
+        if (k == 0) continue;
+        const float cs = s * (1.0f + 0.05f * (float)k);
+        double e = 0.0;
+        for (int i = 0; i < cnt; ++i) {
+            const float l = grid_value(bits, grid_nearest(w[i] / cs, bits));
+            const float diff = cs * l - w[i];
+            e += (double)diff * diff;
+        }
+        if (e < best) { best = e; best_s = cs; }
+    }
+    s = best_s;
+    for (int i = 0; i < cnt; ++i) idx[i] = grid_nearest(w[i] / s, bits);
+    refit();
+    *s_out = s;
+}
+
+struct Grp16Sizes {
+    size_t levels, sc, total;
+    int ng;
+    bool scales, d;
+};
+
+Grp16Sizes grp16_sizes(int bits, int n, float claimed) {
+    Grp16Sizes z{};
+    z.levels = ((size_t)n * (size_t)bits + 7) / 8;
+    z.ng = (n >= kGrp16) ? n / kGrp16 : 0;
+    z.sc = (size_t)((z.ng * 3 + 7) / 8);
+    const size_t budget = (size_t)std::ceil(claimed * (double)n / 8.0);
+    z.scales = (n == 256) || (n >= kGrp16 && z.levels + z.sc + 2 <= budget);
+    z.d = (n >= 8) && (z.levels + 2 <= budget);
+    z.total = z.levels + (z.scales ? z.sc : 0) + ((z.scales || z.d) ? 2 : 0);
+    return z;
+}
+
+bool grp16_encode(int bits, const float* w, int n, float claimed, uint8_t* out, size_t nbytes) {
+    const Grp16Sizes z = grp16_sizes(bits, n, claimed);
+    if (nbytes != z.total) return false;
+    std::memset(out, 0, nbytes);
+    const float eps = 1e-15f;
+    BitSink bs(out, nbytes);
+    if (n < 8 || (!z.scales && !z.d)) {
+        for (int i = 0; i < n; ++i) bs.put(grid_nearest(w[i], bits), bits);
+        return !bs.overflow;
+    }
+    if (!z.scales) {
+        float d = 1.0f;
+        grp16_fit_scale(bits, w, n, &d);
+        if (!(std::fabs(d) > eps)) d = 0.0f;
+        for (int i = 0; i < n; ++i) bs.put((d == 0.0f) ? 0u : grid_nearest(w[i] / d, bits), bits);
+        const uint16_t dh = half_from_float(d);
+        out[z.levels] = (uint8_t)(dh & 0xFF);
+        out[z.levels + 1] = (uint8_t)(dh >> 8);
+        return !bs.overflow;
+    }
+    const int ng = z.ng;
+    std::vector<float> s((size_t)ng, 0.0f);
+    std::vector<int> sc((size_t)ng, 0);
+    float max_abs = 0.0f;
+    for (int g = 0; g < ng; ++g) {
+        grp16_fit_scale(bits, w + g * kGrp16, kGrp16, &s[(size_t)g]);
+        max_abs = std::max(max_abs, std::fabs(s[(size_t)g]));
+    }
+    float d = 1.0f;
+    auto snap = [&]() {
+        for (int g = 0; g < ng; ++g)
+            sc[(size_t)g] = (s[(size_t)g] == 0.0f) ? 0 : std::max(0, std::min(7, (int)std::lround(s[(size_t)g] / d)));
+    };
+    if (max_abs <= eps) {
+        d = 0.0f;
+    } else {
+        d = half_to_float(half_from_float(max_abs / 7.0f));
+        snap();
+        for (int iter = 0; iter < 5; ++iter) {
+            for (int g = 0; g < ng; ++g) {
+                const int st = g * kGrp16;
+                const float eff = d * (float)sc[(size_t)g];
+                if (eff == 0.0f) continue;
+                double num = 0.0, den = 0.0;
+                for (int i = 0; i < kGrp16; ++i) {
+                    const float l = grid_value(bits, grid_nearest(w[st + i] / eff, bits));
+                    num += (double)w[st + i] * (double)l;
+                    den += (double)l * (double)l;
+                }
+                s[(size_t)g] = (den > 1e-20) ? (float)(num / den) : 0.0f;
+            }
+            snap();
+            double num = 0.0, den = 0.0;
+            for (int g = 0; g < ng; ++g) {
+                num += (double)s[(size_t)g] * (double)sc[(size_t)g];
+                den += (double)sc[(size_t)g] * (double)sc[(size_t)g];
+            }
+            d = (den > 1e-20) ? (float)(num / den) : 0.0f;
+            d = half_to_float(half_from_float(d));
+            if (std::fabs(d) <= eps) d = 0.0f;
+        }
+    }
+    for (int i = 0; i < n; ++i) {
+        const float eff = d * (float)sc[(size_t)std::min(i / kGrp16, ng - 1)];
+        bs.put((eff == 0.0f) ? 0u : grid_nearest(w[i] / eff, bits), bits);
+    }
+    for (int g = 0; g < ng; ++g) bs.put((uint32_t)sc[(size_t)g], 3);
+    bs.put(half_from_float(d), 16);
+    return !bs.overflow;
+}
+
+void grp16_decode(int bits, const uint8_t* bytes, size_t size, int n, float* out) {
+    const size_t levels = ((size_t)n * (size_t)bits + 7) / 8;
+    const int ng = (n >= kGrp16) ? n / kGrp16 : 0;
+    const size_t scb = (size_t)((ng * 3 + 7) / 8);
+    float d = 1.0f;
+    std::vector<float> sc((size_t)std::max(ng, 1), 1.0f);
+    if (n >= kGrp16 && size >= levels + scb + 2) {
+        BitSource hdr(bytes, size);
+        for (int i = 0; i < n; ++i) hdr.take(bits);
+        for (int g = 0; g < ng; ++g) sc[(size_t)g] = (float)hdr.take(3);
+        d = half_to_float((uint16_t)hdr.take(16));
+    } else if (n >= 8 && size >= levels + 2) {
+        d = half_to_float((uint16_t)((uint16_t)bytes[size - 2] | ((uint16_t)bytes[size - 1] << 8)));
+    }
+    BitSource br(bytes, size);
+    const int last = std::max(ng - 1, 0);
+    for (int i = 0; i < n; ++i) {
+        const uint32_t idx = br.take(bits);
+        out[i] = grid_value(bits, idx) * d * sc[(size_t)std::min(i / kGrp16, last)];
+    }
+}
+
+// ------------------------------------------------------------ Q_G_6 codec
+// quant_6k / dequant_6k (src/codec/block_codec.cpp:1046-1303): 6-bit levels
+// stored +32, one int8 scale per 16 weights, one binary16 d; a full block is
+// 192 + 16 + 2 = 210 bytes.  value = (d * sc[g]) * (level - 32).
+int q6k_round(float v) {  // :1059-1063, round to nearest even through the 1.5 * 2^23 bias
+    const float biased = v + 12582912.f;
+    int i;
+    std::memcpy(&i, &biased, sizeof(int));
+    return (i & 0x007fffff) - 0x00400000;
+}
+
+int q6k_level(float ratio) {
+    ratio = std::max(-4000.0f, std::min(4000.0f, ratio));
+    return std::max(-32, std::min(31, q6k_round(ratio)));
+}
+
+struct Q6kSizes {
+    size_t levels, total;
+    int sc_count;
+    bool scales, d;
+};
+
+Q6kSizes q6k_sizes(int n) {
+    Q6kSizes z{};
+    z.d = n >= 8;
+    z.sc_count = (n >= 32) ? n / 16 : 0;
+    z.levels = ((size_t)n * 6 + 7) / 8;
+    const size_t budget = (size_t)std::ceil(6.5625 * (double)n / 8.0);
+    z.scales = (n == 256) || (n >= 32 && z.levels + (size_t)z.sc_count + 2 <= budget);
+    z.total = z.levels + (z.scales ? (size_t)z.sc_count : 0) + (z.d ? 2 : 0);
+    return z;
+}
+
+bool q6k_encode(const float* w, int n, uint8_t* out, size_t nbytes, int passes = 2, int giters = 4, int polish = 3,
+                int joint = 3) {
+    const Q6kSizes z = q6k_sizes(n);
+    if (nbytes != z.total) return false;
+    std::memset(out, 0, nbytes);
+    const float eps = 1e-15f;
+    BitSink bs(out, nbytes);
+    if (n < 8) {
+        for (int i = 0; i < n; ++i) bs.put((uint32_t)(q6k_level(w[i]) + 32), 6);
+        return !bs.overflow;
+    }
+    if (!z.scales) {  // one weighted least-squares d for the whole block (:1095-1125)
+        float av = 0.0f;
+        for (int i = 0; i < n; ++i) av += std::fabs(w[i]);
+        av /= (float)n;
+        float maxa = 0.0f;
+        for (int i = 0; i < n; ++i) maxa = std::max(maxa, std::fabs(w[i]));
+        float d = maxa / 32.0f;
+        for (int pass = 0; pass < passes; ++pass) {
+            double num = 0.0, den = 0.0;
+            for (int i = 0; i < n; ++i) {
+                const int l = q6k_level(w[i] / d);
+                const double wgt = (double)(av + std::fabs(w[i]));
+                num += wgt * (double)w[i] * (double)l;
+                den += wgt * (double)l * (double)l;
+            }
+            if (den > 1e-20) d = (float)(num / den);
+        }
+        if (!(std::fabs(d) > eps)) d = 0.0f;
+        for (int i = 0; i < n; ++i) bs.put((uint32_t)(((d == 0.0f) ? 0 : q6k_level(w[i] / d)) + 32), 6);
+        const uint16_t dh = half_from_float(d);
+        out[z.levels] = (uint8_t)(dh & 0xFF);
+        out[z.levels + 1] = (uint8_t)(dh >> 8);
+        return !bs.overflow;
+    }
+    const int ng = z.sc_count;
+    std::vector<float> s((size_t)ng, 0.0f);
+    std::vector<int> sc8((size_t)ng, 0);
+    float max_abs = 0.0f;
+    auto refit16 = [&](const float* x, float scale, float* s_out) {
+        double num = 0.0, den = 0.0;
+        for (int i = 0; i < 16; ++i) {
+            const int l = q6k_level(x[i] / scale);
+            num += (double)x[i] * (double)l;
+            den += (double)l * (double)l;
+        }
+        if (den > 1e-20) *s_out = (float)(num / den);
+    };
+    for (int g = 0; g < ng; ++g) {
+        const float* x = w + g * 16;
+        float maxa = 0.0f;
+        for (int i = 0; i < 16; ++i) maxa = std::max(maxa, std::fabs(x[i]));
+        float sg = (maxa > eps) ? maxa / 32.0f : 0.0f;
+        if (std::fabs(sg) <= eps) { s[(size_t)g] = 0.0f; continue; }
+        for (int iter = 0; iter < giters; ++iter) refit16(x, sg, &sg);
+        float best_s = sg;
+        double best = 1e300;
+        for (int k = -polish; k <= polish; ++k) {
+            if (k == 0) continue;
+            const float cs = sg * (1.0f + 0.05f * (float)k);
+            double e = 0.0;
+            for (int i = 0; i < 16; ++i) {
+                const float diff = cs * (float)q6k_level(x[i] / cs) - x[i];
+                e += (double)diff * diff;
+            }
+            if (e < best) { best = e; best_s = cs; }
+        }
+        sg = best_s;
+        refit16(x, sg, &sg);
+        s[(size_t)g] = sg;
+        max_abs = std::max(max_abs, std::fabs(sg));
+    }
+    float d = 1.0f;
+    if (max_abs <= eps) {
+        d = 0.0f;
+    } else {
+        const float iscale = -128.0f / max_abs;
+        d = 1.0f / iscale;
+        for (int g = 0; g < ng; ++g) sc8[(size_t)g] = std::max(-127, std::min(127, q6k_round(iscale * s[(size_t)g])));
+        for (int iter = 0; iter < joint; ++iter) {
+            for (int g = 0; g < ng; ++g) {
+                const float eff = d * (float)sc8[(size_t)g];
+                if (eff == 0.0f) continue;
+                float fitted = 0.0f;  // stays 0 when the refit has no support
+                refit16(w + g * 16, eff, &fitted);
+                s[(size_t)g] = fitted;
+            }
+            for (int g = 0; g < ng; ++g)
+                sc8[(size_t)g] = (d == 0.0f) ? 0 : std::max(-127, std::min(127, q6k_round(s[(size_t)g] / d)));
+            double num = 0.0, den = 0.0;
+            for (int g = 0; g < ng; ++g) {
+                num += (double)s[(size_t)g] * (double)sc8[(size_t)g];
+                den += (double)sc8[(size_t)g] * (double)sc8[(size_t)g];
+            }
+            d = (den > 1e-20) ? (float)(num / den) : 0.0f;
+            if (std::fabs(d) <= eps) d = 0.0f;
+        }
+    }
+    for (int i = 0; i < n; ++i) {
+        const float eff = d * (float)sc8[(size_t)std::min(i / 16, ng - 1)];
+        bs.put((uint32_t)(((eff == 0.0f) ? 0 : q6k_level(w[i] / eff)) + 32), 6);
+    }
+    size_t off = z.levels;
+    for (int g = 0; g < ng; ++g) out[off++] = (uint8_t)(int8_t)sc8[(size_t)g];
+    const uint16_t dh = half_from_float(d);
+    out[off] = (uint8_t)(dh & 0xFF);
+    out[off + 1] = (uint8_t)(dh >> 8);
+    return !bs.overflow;
+}
+
+void q6k_decode(const uint8_t* bytes, size_t size, int n, float* out) {
+    const int sc_count = (n >= 32) ? n / 16 : 0;
+    const size_t levels = ((size_t)n * 6 + 7) / 8;
+    const int groups = (n + 15) / 16;
+    float d = 1.0f;
+    std::vector<float> sc((size_t)groups, 1.0f);
+    if (n >= 8 && size >= levels + 2) {
+        d = half_to_float((uint16_t)((uint16_t)bytes[size - 2] | ((uint16_t)bytes[size - 1] << 8)));
+        const int stored = (size >= levels + 2 + (size_t)sc_count) ? sc_count : 0;
+        for (int g = 0; g < stored; ++g) sc[(size_t)g] = (float)(int8_t)bytes[size - 2 - (size_t)stored + (size_t)g];
+        if (stored > 0)
+            for (int g = stored; g < groups; ++g) sc[(size_t)g] = sc[(size_t)stored - 1];
+    }
+    BitSource br(bytes, size);
+    for (int i = 0; i < n; ++i) {
+        const float e = d * sc[(size_t)(i / 16)];
+        const float v = e * (float)((int)(br.take(6) & 63u) - 32);
+        // The reference's vector path (:1278-1295, full groups of 16 under AVX2) computes
+        // e * level + 0, which turns a negative zero into +0; its scalar path for a
+        // partial last group keeps the sign.
+        const bool full_group = (i / 16) * 16 + 16 <= n;
+        out[i] = (full_group && v == 0.0f) ? 0.0f : v;
+    }
+}
+
 // ------------------------------------------------------ affine grouped codec
 // w ~= d*sc[g]*lv - dm*mc[g], lv on a uniform [0,1] grid, sc unsigned, mc
 // signed (stored with a bias).  Layout: levels, scale codes, min codes, d, dm.
@@ -503,7 +849,8 @@ void affine_fit_group(int bits, const float* w, int cnt, float* s_out, float* m_
 
 bool affine_encode(const Spec& sp, const float* w, int n, uint8_t* out, size_t nbytes) {
     const AffineSizes z = affine_sizes(sp, n);
-    if (!z.ok || nbytes != z.total) return false;
+    if (!z.ok) return grp16_encode(sp.bits, w, n, sp.claimed, out, nbytes);
+    if (nbytes != z.total) return false;
     std::memset(out, 0, nbytes);
     const int bits = sp.bits, gsz = sp.gsz, ng = z.ng;
     const float eps = 1e-15f;
@@ -599,7 +946,7 @@ bool affine_encode(const Spec& sp, const float* w, int n, uint8_t* out, size_t n
 
 bool affine_decode(const Spec& sp, const uint8_t* bytes, size_t size, int n, float* out) {
     const AffineSizes z = affine_sizes(sp, n);
-    if (!z.ok) return false;
+    if (!z.ok) { grp16_decode(sp.bits, bytes, size, n, out); return true; }
     const int ng = z.ng, gsz = sp.gsz;
     const int bias = ((1 << sp.mb)) / 2;
     BitSource br(bytes, size);
@@ -672,14 +1019,51 @@ bool sym32_decode(int bits, const uint8_t* bytes, size_t size, int n, float* out
 }
 
 // ------------------------------------------------------------------ dispatch
+// A Q_G_8 block whose size is not a multiple of 32 is written by the affine codec
+// with 8-bit levels (src/codec/block_codec.cpp:2501-2510, :2957-2962).
+const Spec kGrp8Tail = {Codec::Affine, 8, 32, 6, 6, 8.5f};
+
+long affine_bytes(const Spec& sp, int n) {
+    const AffineSizes z = affine_sizes(sp, n);
+    return z.ok ? (long)z.total : (long)grp16_sizes(sp.bits, n, sp.claimed).total;
+}
+
+double mean_sq_err(const float* a, const float* b, int n) {
+    double e = 0.0;
+    for (int i = 0; i < n; ++i) { const double d = (double)a[i] - b[i]; e += d * d; }
+    return n > 0 ? e / (double)n : 0.0;
+}
+
+// Q_G_6_K_M / _K_H: the base encoding, then one or two longer searches, keeping a
+// candidate only when its decoded error is strictly smaller (:2733-2755).
+bool q6k_encode_tier(int tier, const float* w, int n, uint8_t* out, size_t nbytes) {
+    if (!q6k_encode(w, n, out, nbytes)) return false;
+    if (tier <= 0) return true;
+    std::vector<float> dec((size_t)n);
+    std::vector<uint8_t> cand(nbytes);
+    q6k_decode(out, nbytes, n, dec.data());
+    double best = mean_sq_err(w, dec.data(), n);
+    const int kp[2][4] = {{5, 8, 5, 6}, {10, 14, 8, 10}};
+    for (int c = 0; c < (tier >= 2 ? 2 : 1); ++c) {
+        if (!q6k_encode(w, n, cand.data(), nbytes, kp[c][0], kp[c][1], kp[c][2], kp[c][3])) return false;
+        q6k_decode(cand.data(), nbytes, n, dec.data());
+        const double e = mean_sq_err(w, dec.data(), n);
+        if (e < best) { best = e; std::memcpy(out, cand.data(), nbytes); }
+    }
+    return true;
+}
+
 long block_bytes(uint8_t fmt, int n) {
     Spec sp;
     if (n <= 0 || !spec_for(fmt, &sp)) return -1;
     switch (sp.codec) {
         case Codec::Raw32: return (long)n * 4;
         case Codec::Lattice: return (long)lattice_bytes(sp.bits, n);
-        case Codec::Grp8: return grp8_fits(n) ? (long)n + (long)(n / 32) * 2 : -1;
-        case Codec::Affine: { const AffineSizes z = affine_sizes(sp, n); return z.ok ? (long)z.total : -1; }
+        case Codec::Grp8:
+            if (grp8_fits(n)) return (long)n + (long)(n / 32) * 2;
+            return affine_bytes(kGrp8Tail, n);
+        case Codec::Affine: return affine_bytes(sp, n);
+        case Codec::Q6K: return (long)q6k_sizes(n).total;
         case Codec::Sym32: return (n >= 32 && n % 32 == 0) ? (long)sym32_bytes(sp.bits, n) : -1;
     }
     return -1;
@@ -694,8 +1078,12 @@ long encode_block(uint8_t fmt, const float* w, int n, uint8_t* out, size_t cap) 
     switch (sp.codec) {
         case Codec::Raw32: std::memcpy(out, w, (size_t)n * 4); break;
         case Codec::Lattice: ok = lattice_encode(sp.bits, w, n, out, (size_t)need); break;
-        case Codec::Grp8: grp8_encode(w, n, out); break;
+        case Codec::Grp8:
+            if (grp8_fits(n)) grp8_encode(w, n, out);
+            else ok = affine_encode(kGrp8Tail, w, n, out, (size_t)need);
+            break;
         case Codec::Affine: ok = affine_encode(sp, w, n, out, (size_t)need); break;
+        case Codec::Q6K: ok = q6k_encode_tier(sp.tier, w, n, out, (size_t)need); break;
         case Codec::Sym32: ok = sym32_encode(sp.bits, w, n, out); break;
     }
     return ok ? need : -1;
@@ -710,7 +1098,11 @@ int decode_block(uint8_t fmt, const uint8_t* bytes, size_t size, int n, float* o
     switch (sp.codec) {
         case Codec::Raw32: if (size >= (size_t)n * 4) std::memcpy(out, bytes, (size_t)n * 4); return 0;
         case Codec::Lattice: lattice_decode(sp.bits, bytes, size, n, out); return 0;
-        case Codec::Grp8: if (!grp8_fits(n)) return -1; grp8_decode(bytes, size, n, out); return 0;
+        case Codec::Grp8:
+            if (!grp8_fits(n)) return affine_decode(kGrp8Tail, bytes, size, n, out) ? 0 : -1;
+            grp8_decode(bytes, size, n, out);
+            return 0;
+        case Codec::Q6K: q6k_decode(bytes, size, n, out); return 0;
         case Codec::Affine: return affine_decode(sp, bytes, size, n, out) ? 0 : -1;
         case Codec::Sym32: return sym32_decode(sp.bits, bytes, size, n, out) ? 0 : -1;
     }

@@ -17,6 +17,12 @@ codec.npz
                  over code 255, whose level is exactly 1.0)
 rng.npz
     u64_42, uniform_42, normal_42_002, normal_43: first 4096 draws of RNG(seed)
+tails.npz
+    blocks of n <= 256 weights (the first n of two of the inputs above) through the
+    reference codec, one row of `index` = (wire id, n, input, payload offset, payload
+    bytes, decoded offset) into the flat `payloads` / `decoded` arrays: the short-block
+    layouts (raw levels, one scale, grouped-lattice fallback), Q_2, Q_G_6 and the ids
+    whose claim is below the affine header's size
 matmul.npz
     for Q_G_4 and Q_G_8: y = x.W^T with W 48x512 from the fixture generator,
     computed by the reference scalar_gemm_bt on the reference-decoded matrix
@@ -48,9 +54,32 @@ def inputs():
     return np.stack([a, b, c, d]).reshape(4, nb, 256)
 
 
+TAIL_FORMATS = ["Q_2", "Q_4", "Q_8", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_6", "Q_G_8", "Q_G_2_K_H", "Q_G_3_K_L",
+                "Q_G_4_K_M", "Q_G_6_K_M", "Q_G_6_K_H", "Q_2_5", "Q_6_5"]
+TAIL_SIZES = [1, 7, 8, 15, 16, 31, 32, 33, 100, 160, 250, 255, 256]
+
+
+def tails(w):
+    src = [w[0].reshape(-1), w[2].reshape(-1) + np.float32(0.01)]
+    index, pays, decs, poff, doff = [], [], [], 0, 0
+    for fmt in TAIL_FORMATS:
+        for n in TAIL_SIZES:
+            for which, x in enumerate(src):
+                p = O.ref_encode_block(fmt, x[300:300 + n])
+                index.append((O.FMT[fmt], n, which, poff, p.size, doff))
+                pays.append(p)
+                decs.append(O.ref_decode_block(fmt, p, n))
+                poff += p.size
+                doff += n
+    np.savez_compressed(os.path.join(HERE, "tails.npz"), src=np.stack([s[300:556] for s in src]),
+                        index=np.array(index, np.int64), payloads=np.concatenate(pays),
+                        decoded=np.concatenate(decs))
+
+
 def main():
     assert O.have_ref(), "build oracle/_ref first (make -C oracle)"
     w = inputs()
+    tails(w)
     out = {"w": w}
     for fmt in FORMATS:
         pays, decs = [], []
@@ -101,7 +130,7 @@ def main():
         mm[f"{fmt}_payload"] = pays
         mm[f"{fmt}_y"] = Y
     np.savez_compressed(os.path.join(HERE, "matmul.npz"), **mm)
-    for f in ("codec.npz", "rng.npz", "matmul.npz"):
+    for f in ("codec.npz", "rng.npz", "matmul.npz", "tails.npz"):
         print(f, os.path.getsize(os.path.join(HERE, f)))
 
 

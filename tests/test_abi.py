@@ -43,11 +43,13 @@ def test_errors_are_reported_not_swallowed(tfq):
     out = C.c_size_t(0)
     assert L.tfq_block_bytes(0, 256, C.byref(out)) == 2            # TFQ_ERR_FORMAT: Q_1 is not handled
     assert b"not handled" in L.tfq_last_error()
-    assert L.tfq_block_bytes(40, 100, C.byref(out)) == 3           # TFQ_ERR_SHAPE
+    assert L.tfq_block_bytes(40, 100, C.byref(out)) == 0 and out.value == 57   # short block: grouped-lattice fallback
+    assert L.tfq_block_bytes(40, 257, C.byref(out)) == 3           # TFQ_ERR_SHAPE
+    assert L.tfq_block_bytes(105, 100, C.byref(out)) == 3          # literal formats need whole groups of 32
     assert L.tfq_gemv(None, None, 0, 1, None, 0, None) == 1        # TFQ_ERR_ARG
     assert L.tfq_weight_upload(40, 4, 100, None, 0) is None        # null payload
     with pytest.raises(tfq.TfqError):
-        tfq.block_bytes("Q_G_4", 17)
+        tfq.block_bytes("Q_G_4", 300)
 
 
 def test_no_cpu_fallback_without_device(tfq):

@@ -8,7 +8,8 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 G = os.path.join(os.path.dirname(__file__), "golden")
-DECODE_FORMATS = ["Q_4", "Q_8", "Q_32", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_8", "Q_4_5", "Q_G_8_5",
+DECODE_FORMATS = ["Q_2", "Q_4", "Q_8", "Q_32", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_6", "Q_G_8", "Q_4_5", "Q_G_8_5",
+                  "Q_G_2_K_M", "Q_G_3_K_L", "Q_G_4_K_H", "Q_G_6_K_H", "Q_2_5", "Q_G_6_5",
                   "B32S4", "B32S8", "SB256A3", "SB256A2"]
 
 
@@ -42,7 +43,8 @@ def test_decode_golden_payloads(tfq, gpu, fmt):
     assert np.array_equal(got.view(np.uint32), want.reshape(-1).view(np.uint32))
 
 
-@pytest.mark.parametrize("fmt", ["Q_4", "Q_8", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_8", "SB256A3", "SB256A2"])
+@pytest.mark.parametrize("fmt", ["Q_2", "Q_4", "Q_8", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_6", "Q_G_8", "Q_G_2_K_L", "Q_G_3_K_M",
+                                 "Q_G_4_K_L", "Q_6_5", "SB256A3", "SB256A2"])
 def test_decode_arbitrary_payload_bits(O, tfq, gpu, fmt):
     # every payload bit pattern is legal input: random bytes, finite scales
     import torch
@@ -51,13 +53,49 @@ def test_decode_arbitrary_payload_bits(O, tfq, gpu, fmt):
     pay = rng.integers(0, 256, (256, nb), dtype=np.uint8)
     if fmt in ("Q_G_8",):
         pay[:, -16:] &= 0x7B
-    elif fmt in ("Q_4", "Q_8"):
+    elif fmt in ("Q_2", "Q_4", "Q_8"):
         pay[:, :2] &= 0x7B
     else:
         pay[:, -4:] &= 0x7B
     want = O.decode_tensor(fmt, pay.reshape(-1), 256 * 256)
     got = tfq.decode(fmt, torch.from_numpy(pay.reshape(-1)).to(gpu), 256 * 256).cpu().numpy()
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+TAIL_FORMATS = ["Q_2", "Q_4", "Q_8", "Q_32", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_6", "Q_G_8", "Q_G_2_K_H", "Q_G_4_K_M",
+                "Q_G_6_K_L", "Q_6_5", "SB256A3"]
+
+
+@pytest.mark.parametrize("fmt", TAIL_FORMATS)
+def test_decode_with_a_short_last_block(O, tfq, gpu, fmt):
+    """Tensors whose size is not a multiple of 256: the last block uses the layout the codec chooses
+    for its size (no header, one scale, grouped-lattice fallback, ...)."""
+    import torch
+    w = _inputs(O, 2)
+    for n in (1, 5, 8, 15, 16, 17, 31, 32, 33, 64, 100, 160, 200, 224, 250, 255, 256 + 7, 512 + 250):
+        print(f"decode {fmt} n={n}", flush=True)
+        pay = O.encode_tensor(fmt, w[:n])
+        assert tfq.block_bytes(fmt, n % 256 or 256) == O.block_bytes(fmt, n % 256 or 256)
+        want = O.decode_tensor(fmt, pay, n)
+        got = tfq.decode(fmt, torch.from_numpy(pay).to(gpu), n).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), n
+        rnd = np.random.default_rng(n).integers(0, 256, pay.size, dtype=np.uint8)
+        want = O.decode_tensor(fmt, rnd, n)
+        got = tfq.decode(fmt, torch.from_numpy(rnd).to(gpu), n).cpu().numpy()
+        keep = ~(np.isnan(want) & np.isnan(got))
+        assert np.array_equal(got.view(np.uint32)[keep], want.view(np.uint32)[keep]), n
+
+
+def test_decode_short_blocks_golden(tfq, gpu):
+    """The fixture written from the compiled reference (tests/golden/tails.npz)."""
+    import torch
+    t = np.load(os.path.join(G, "tails.npz"))
+    for fmt, n, which, poff, plen, doff in t["index"]:
+        pay = np.ascontiguousarray(t["payloads"][poff:poff + plen])
+        want = t["decoded"][doff:doff + n]
+        assert tfq.block_bytes(int(fmt), int(n)) == plen, (fmt, n)
+        got = tfq.decode(int(fmt), torch.from_numpy(pay).to(gpu), int(n)).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (fmt, n, which)
 
 
 def test_half_subnormal_scales_decode_exactly(O, tfq, gpu):

@@ -19,9 +19,12 @@ LIB_PATH = os.path.join(_HERE, "libtfq.so")
 F32, BF16 = 0, 1
 
 FMT = {
-    "Q_4": 3, "Q_8": 5, "Q_32": 9,
-    "Q_G_2": 38, "Q_G_3": 39, "Q_G_4": 40, "Q_G_8": 42,
-    "Q_3_5": 75, "Q_4_5": 76, "Q_8_5": 78, "Q_G_3_5": 84, "Q_G_4_5": 85, "Q_G_8_5": 87,
+    "Q_2": 1, "Q_4": 3, "Q_8": 5, "Q_32": 9,
+    "Q_G_2": 38, "Q_G_3": 39, "Q_G_4": 40, "Q_G_6": 41, "Q_G_8": 42,
+    "Q_G_2_K_L": 49, "Q_G_2_K_M": 50, "Q_G_2_K_H": 51, "Q_G_3_K_L": 52, "Q_G_3_K_M": 53, "Q_G_3_K_H": 54,
+    "Q_G_4_K_L": 55, "Q_G_4_K_M": 56, "Q_G_4_K_H": 57, "Q_G_6_K_L": 58, "Q_G_6_K_M": 59, "Q_G_6_K_H": 60,
+    "Q_2_5": 74, "Q_3_5": 75, "Q_4_5": 76, "Q_6_5": 77, "Q_8_5": 78,
+    "Q_G_2_5": 83, "Q_G_3_5": 84, "Q_G_4_5": 85, "Q_G_6_5": 86, "Q_G_8_5": 87,
     "B32S4": 105, "B32S8": 106, "SB256A3": 107, "SB256A2": 108,
 }
 

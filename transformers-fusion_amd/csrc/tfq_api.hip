@@ -57,10 +57,15 @@ struct NameRow {
 // Canonical names (format_name, include/quant/types.h:168-196) of the ids this
 // backend handles, plus the appended literal formats.
 const NameRow kNames[] = {
-    {"Q_4", TFQ_Q_4}, {"Q_8", TFQ_Q_8}, {"Q_32", TFQ_Q_32},
-    {"Q_G_2", TFQ_Q_G_2}, {"Q_G_3", TFQ_Q_G_3}, {"Q_G_4", TFQ_Q_G_4}, {"Q_G_8", TFQ_Q_G_8},
-    {"Q_3_5", TFQ_Q_3_5}, {"Q_4_5", TFQ_Q_4_5}, {"Q_8_5", TFQ_Q_8_5},
-    {"Q_G_3_5", TFQ_Q_G_3_5}, {"Q_G_4_5", TFQ_Q_G_4_5}, {"Q_G_8_5", TFQ_Q_G_8_5},
+    {"Q_2", TFQ_Q_2}, {"Q_4", TFQ_Q_4}, {"Q_8", TFQ_Q_8}, {"Q_32", TFQ_Q_32},
+    {"Q_G_2", TFQ_Q_G_2}, {"Q_G_3", TFQ_Q_G_3}, {"Q_G_4", TFQ_Q_G_4}, {"Q_G_6", TFQ_Q_G_6}, {"Q_G_8", TFQ_Q_G_8},
+    {"Q_G_2_K_L", TFQ_Q_G_2_K_L}, {"Q_G_2_K_M", TFQ_Q_G_2_K_M}, {"Q_G_2_K_H", TFQ_Q_G_2_K_H},
+    {"Q_G_3_K_L", TFQ_Q_G_3_K_L}, {"Q_G_3_K_M", TFQ_Q_G_3_K_M}, {"Q_G_3_K_H", TFQ_Q_G_3_K_H},
+    {"Q_G_4_K_L", TFQ_Q_G_4_K_L}, {"Q_G_4_K_M", TFQ_Q_G_4_K_M}, {"Q_G_4_K_H", TFQ_Q_G_4_K_H},
+    {"Q_G_6_K_L", TFQ_Q_G_6_K_L}, {"Q_G_6_K_M", TFQ_Q_G_6_K_M}, {"Q_G_6_K_H", TFQ_Q_G_6_K_H},
+    {"Q_2_5", TFQ_Q_2_5}, {"Q_3_5", TFQ_Q_3_5}, {"Q_4_5", TFQ_Q_4_5}, {"Q_6_5", TFQ_Q_6_5}, {"Q_8_5", TFQ_Q_8_5},
+    {"Q_G_2_5", TFQ_Q_G_2_5}, {"Q_G_3_5", TFQ_Q_G_3_5}, {"Q_G_4_5", TFQ_Q_G_4_5}, {"Q_G_6_5", TFQ_Q_G_6_5},
+    {"Q_G_8_5", TFQ_Q_G_8_5},
     {"B32S4", TFQ_B32S4}, {"B32S8", TFQ_B32S8}, {"SB256A3", TFQ_SB256A3}, {"SB256A2", TFQ_SB256A2},
 };
 
@@ -117,8 +122,26 @@ int tfq_block_bytes(uint8_t fmt, uint32_t n, size_t* out) {
     if (!out) return fail(TFQ_ERR_ARG, "tfq_block_bytes: null out");
     const Spec sp = spec_of(fmt);
     if (sp.codec == Codec::None) return fail(TFQ_ERR_FORMAT, "tfq_block_bytes: wire id " + std::to_string(fmt) + " is not handled");
-    if (n != 256) return fail(TFQ_ERR_SHAPE, "tfq_block_bytes: only full 256-weight blocks are handled");
-    *out = (size_t)sp.block_bytes;
+    BlockLayout L;
+    if (!block_layout(fmt, (int)(n > 256 ? 0 : n), &L))
+        return fail(TFQ_ERR_SHAPE, "tfq_block_bytes: wire id " + std::to_string(fmt) + " cannot hold a block of " + std::to_string(n) + " weights");
+    *out = (size_t)L.bytes;
+    return TFQ_OK;
+}
+
+// Payload bytes of a tensor of n weights cut into 256-blocks, the last one possibly short
+// (FormatRegistry::quantize, src/codec/format_registry.cpp:168-207).
+static int check_tensor(const char* who, uint8_t fmt, int64_t n, size_t* need, BlockLayout* tail) {
+    const Spec sp = spec_of(fmt);
+    if (sp.codec == Codec::None) return fail(TFQ_ERR_FORMAT, std::string(who) + ": wire id " + std::to_string(fmt) + " is not handled");
+    if (n <= 0) return fail(TFQ_ERR_SHAPE, std::string(who) + ": n must be positive");
+    *need = (size_t)(n / 256) * (size_t)sp.block_bytes;
+    tail->n = 0;
+    if (n % 256) {
+        if (!block_layout(fmt, (int)(n % 256), tail))
+            return fail(TFQ_ERR_SHAPE, std::string(who) + ": the format cannot hold a last block of " + std::to_string(n % 256) + " weights");
+        *need += (size_t)tail->bytes;
+    }
     return TFQ_OK;
 }
 
@@ -141,11 +164,14 @@ int tfq_encode_blocks(uint8_t fmt, const float* w, int64_t n, uint8_t* dst, size
 
 int tfq_decode_blocks(uint8_t fmt, const uint8_t* src, size_t bytes, int64_t n, float* out, tfq_stream_t stream) {
     size_t need = 0;
+    BlockLayout tail;
     if (!src || !out) return fail(TFQ_ERR_ARG, "tfq_decode_blocks: null pointer");
-    if (int r = check_blocks("tfq_decode_blocks", fmt, n, &need)) return r;
-    if (bytes < need) return fail(TFQ_ERR_SHAPE, "tfq_decode_blocks: payload shorter than n/256 blocks");
+    if (int r = check_tensor("tfq_decode_blocks", fmt, n, &need, &tail)) return r;
+    if (bytes < need) return fail(TFQ_ERR_SHAPE, "tfq_decode_blocks: payload shorter than the blocks of n weights");
     if (int r = ensure_device()) return r;
-    return launch_decode(fmt, src, n / 256, out, (hipStream_t)stream);
+    if (int r = launch_decode(fmt, src, n / 256, out, (hipStream_t)stream)) return r;
+    if (!tail.n) return TFQ_OK;
+    return launch_decode_short(tail, src + need - (size_t)tail.bytes, out + (n / 256) * 256, (hipStream_t)stream);
 }
 
 int tfq_encode_blocks_host(uint8_t fmt, const float* w, int64_t n, uint8_t* dst, size_t cap, uint32_t* per_block_bytes) {
@@ -171,9 +197,10 @@ int tfq_encode_blocks_host(uint8_t fmt, const float* w, int64_t n, uint8_t* dst,
 
 int tfq_decode_blocks_host(uint8_t fmt, const uint8_t* src, size_t bytes, int64_t n, float* out) {
     size_t need = 0;
+    BlockLayout tail;
     if (!src || !out) return fail(TFQ_ERR_ARG, "tfq_decode_blocks_host: null pointer");
-    if (int r = check_blocks("tfq_decode_blocks_host", fmt, n, &need)) return r;
-    if (bytes < need) return fail(TFQ_ERR_SHAPE, "tfq_decode_blocks_host: payload shorter than n/256 blocks");
+    if (int r = check_tensor("tfq_decode_blocks_host", fmt, n, &need, &tail)) return r;
+    if (bytes < need) return fail(TFQ_ERR_SHAPE, "tfq_decode_blocks_host: payload shorter than the blocks of n weights");
     if (int r = ensure_device()) return r;
     uint8_t* ds = nullptr;
     float* dout = nullptr;
@@ -182,6 +209,7 @@ int tfq_decode_blocks_host(uint8_t fmt, const uint8_t* src, size_t bytes, int64_
     if (e != hipSuccess) { (void)hipFree(ds); return hip_fail(e, "hipMalloc"); }
     int rc = hip_fail(hipMemcpy(ds, src, need, hipMemcpyHostToDevice), "hipMemcpy H2D");
     if (!rc) rc = launch_decode(fmt, ds, n / 256, dout, nullptr);
+    if (!rc && tail.n) rc = launch_decode_short(tail, ds + need - (size_t)tail.bytes, dout + (n / 256) * 256, nullptr);
     if (!rc) rc = hip_fail(hipMemcpy(out, dout, (size_t)n * 4, hipMemcpyDeviceToHost), "hipMemcpy D2H");
     (void)hipFree(ds);
     (void)hipFree(dout);

@@ -6,6 +6,8 @@
 
 #include "tfq_decode.hpp"
 
+#include <cmath>
+
 namespace tfq {
 
 namespace {
@@ -16,6 +18,11 @@ __global__ __launch_bounds__(256) void decode_kernel(const uint8_t* __restrict__
     constexpr Spec sp = spec_of(FMT);
     const int64_t blk = blockIdx.x;
     out[blk * 256 + threadIdx.x] = decode_weight<FMT>(src + blk * (int64_t)sp.block_bytes, threadIdx.x);
+}
+
+__global__ __launch_bounds__(256) void decode_short_kernel(BlockLayout L, const uint8_t* __restrict__ src,
+                                                           float* __restrict__ out) {
+    if ((int)threadIdx.x < L.n) out[threadIdx.x] = decode_weight_short(L, src, threadIdx.x);
 }
 
 // Literal symmetric block-32 formats, closed form per 32 weights:
@@ -160,10 +167,71 @@ int run_decode(const uint8_t* src, int64_t nblocks, float* out, hipStream_t s) {
 
 }  // namespace
 
+// Sizes as the reference's encoders choose them (src/codec/block_codec.cpp): lattice :443-455,
+// affine :1394-1411, grouped-lattice fallback :788-815, Q_G_6 :1070-1082, Q_G_8 :2501-2510.
+static bool affine_or_fallback(int bits, int gsz, int scb, int mb, double claimed, int n, BlockLayout* L) {
+    const int levels = (n * bits + 7) / 8;
+    const int budget = (int)std::ceil(claimed * (double)n / 8.0);
+    const int ng = n >= gsz ? n / gsz : 0;
+    const int total = levels + (ng * scb + 7) / 8 + (ng * mb + 7) / 8 + 4;
+    if (ng > 0 && total <= budget) {
+        *L = {BK_AFFINE, bits, n, total, gsz, ng, scb, mb, 0};
+        return true;
+    }
+    const int ng8 = n >= 8 ? n / 8 : 0;
+    const int sc_bytes = (ng8 * 3 + 7) / 8;
+    const bool scales = n == 256 || (n >= 8 && levels + sc_bytes + 2 <= budget);
+    const bool d_only = n >= 8 && levels + 2 <= budget;
+    *L = {BK_GRP16, bits, n, levels + (scales ? sc_bytes : 0) + ((scales || d_only) ? 2 : 0), 8, ng8, 3, 0,
+          scales ? 2 : d_only ? 1 : 0};
+    return true;
+}
+
+bool block_layout(int fmt, int n, BlockLayout* L) {
+    const Spec sp = spec_of(fmt);
+    if (n <= 0 || n > 256) return false;
+    switch (sp.codec) {
+        case Codec::Raw32: *L = {BK_RAW32, 32, n, n * 4, 0, 0, 0, 0, 0}; return true;
+        case Codec::Lattice:
+            *L = {n < 16 ? BK_LEVELS : BK_LATTICE, sp.bits, n, ((int)std::ceil(sp.bpw * (double)n) + 7) / 8, 0, 0, 0, 0, 0};
+            return true;
+        case Codec::Affine: case Codec::Grp16:
+            return affine_or_fallback(sp.bits, sp.gsz, sp.scb, sp.mb, (double)sp.bpw, n, L);
+        case Codec::Grp8:
+            if (n >= 32 && n % 32 == 0) { *L = {BK_GRP8, 8, n, n + (n / 32) * 2, 32, n / 32, 0, 0, 0}; return true; }
+            return affine_or_fallback(8, 32, 6, 6, 8.5, n, L);
+        case Codec::Q6K: {
+            const int levels = (n * 6 + 7) / 8, sc_count = n >= 32 ? n / 16 : 0;
+            const int budget = (int)std::ceil(6.5625 * (double)n / 8.0);
+            const bool scales = n == 256 || (n >= 32 && levels + sc_count + 2 <= budget);
+            *L = {BK_Q6K, 6, n, levels + (scales ? sc_count : 0) + (n >= 8 ? 2 : 0), 16, sc_count, 8, 0,
+                  (n >= 8 ? 1 : 0) | ((scales ? sc_count : 0) << 8)};
+            return true;
+        }
+        case Codec::Sym32:
+            if (n < 32 || n % 32) return false;
+            *L = {BK_SYM32, sp.bits, n, n * sp.bits / 8 + (n / 32) * 2, 32, n / 32, 0, 0, 0};
+            return true;
+        default: return false;
+    }
+}
+
+int launch_decode_short(const BlockLayout& L, const uint8_t* src, float* out, hipStream_t s) {
+    if (L.n <= 0 || L.n > 256 || L.bytes <= 0) return fail(TFQ_ERR_SHAPE, "decode: bad short-block layout");
+    hipLaunchKernelGGL(decode_short_kernel, dim3(1), dim3(256), 0, s, L, src, out);
+    return hip_fail(hipGetLastError(), "decode launch");
+}
+
 int launch_decode(int fmt, const uint8_t* src, int64_t nblocks, float* out, hipStream_t s) {
     if (nblocks <= 0) return TFQ_OK;
     if (nblocks > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "decode: more than 2^31-1 blocks in one call");
     switch (canonical(fmt)) {
+        case TFQ_Q_2: return run_decode<TFQ_Q_2>(src, nblocks, out, s);
+        case TFQ_Q_G_6: return run_decode<TFQ_Q_G_6>(src, nblocks, out, s);
+        case TFQ_Q_G_2_K_L: return run_decode<TFQ_Q_G_2_K_L>(src, nblocks, out, s);
+        case TFQ_Q_G_3_K_L: return run_decode<TFQ_Q_G_3_K_L>(src, nblocks, out, s);
+        case TFQ_Q_G_4_K_L: return run_decode<TFQ_Q_G_4_K_L>(src, nblocks, out, s);
+        case TFQ_Q_6_5: return run_decode<TFQ_Q_6_5>(src, nblocks, out, s);
         case TFQ_Q_32: return run_decode<TFQ_Q_32>(src, nblocks, out, s);
         case TFQ_Q_4: return run_decode<TFQ_Q_4>(src, nblocks, out, s);
         case TFQ_Q_8: return run_decode<TFQ_Q_8>(src, nblocks, out, s);

@@ -6,6 +6,10 @@
 //   Q_4 / Q_8           dequant_lattice                       :499-529
 //   Q_G_8 family        dequant_grp8_compound                 :390-427
 //   Q_G_4/3/2, SB256A*  dequant_affine                        :1620-1687
+//   Q_G_6 (+ _K_*)      dequant_6k                            :1240-1303
+//   Q_G_{2,3,4}_K_*, Q_2_5, Q_6_5   dequant_grp16             :916-945
+// decode_weight_short() does the same for a block of n <= 256 weights whose layout
+// (BlockLayout) was chosen on the host from (format, n).
 // Arithmetic is ordered exactly as there (fp32 multiply, then one fused
 // multiply-add); the library is compiled with -ffp-contract=off so the
 // compiler adds no fusion of its own.
@@ -22,6 +26,17 @@ __device__ __constant__ static const uint32_t kComp8Bits[256] = {
 __device__ __constant__ static const float kGrid4[16] = {
     -2.7178f, -2.0522f, -1.5995f, -1.2392f, -0.9275f, -0.6508f, -0.3976f, -0.1260f,
     0.1260f,  0.3976f,  0.6508f,  0.9275f,  1.2392f,  1.5995f,  2.0522f,  2.7178f};
+
+__device__ __constant__ static const float kGrid2[4] = {-1.5104f, -0.4528f, 0.4528f, 1.5104f};
+
+// plain lattice grid (level_value, src/codec/block_codec.cpp:182-188): Lloyd-Max tables
+// for 2 and 4 bits, -8 + 16 i / (2^bits - 1) otherwise
+__device__ __forceinline__ float grid_value(int bits, uint32_t idx) {
+    if (bits == 2) return kGrid2[min(idx, 3u)];
+    if (bits == 4) return kGrid4[min(idx, 15u)];
+    const uint32_t top = bits >= 24 ? 16777215u : ((1u << bits) - 1u);
+    return -8.0f + 16.0f * (float)idx / (float)top;
+}
 
 // uniform [0,1] grid of the affine family (level_value_affine,
 // src/codec/block_codec.cpp:1316-1324): (float)idx * (1.0f / top)
@@ -52,7 +67,7 @@ __device__ __forceinline__ float decode_weight(const uint8_t* __restrict__ p, ui
         uint32_t idx = stream_bits(p, BB, pos, sp.bits - (slot ? 1 : 0));
         if (slot) idx <<= 1;
         if constexpr (sp.bits == 8) v = scale * __uint_as_float(kComp8Bits[min(idx, 255u)]);
-        else v = kGrid4[min(idx, 15u)] * scale;
+        else v = grid_value(sp.bits, idx) * scale;
     } else if constexpr (sp.codec == Codec::Grp8) {
         const uint32_t g = i >> 5;
         const uint32_t h = (uint32_t)p[256 + 2 * g] | ((uint32_t)p[256 + 2 * g + 1] << 8);
@@ -72,6 +87,20 @@ __device__ __forceinline__ float decode_weight(const uint8_t* __restrict__ p, ui
         const float es = d * sc;
         const float neg = -(dm * mc);
         v = __builtin_fmaf(es, unit_level(sp.bits, idx), neg);
+    } else if constexpr (sp.codec == Codec::Grp16) {
+        // [256 levels][32 x 3-bit scale][binary16 d], one bit stream (byte aligned at each part here)
+        constexpr uint32_t lev_bits = 256u * sp.bits;
+        const uint32_t idx = stream_bits(p, BB, i * sp.bits, sp.bits);
+        const float sc = (float)stream_bits(p, BB, lev_bits + (i >> 3) * 3u, 3);
+        const float d = half_bits_to_float(stream_bits(p, BB, lev_bits + 96u, 16));
+        v = grid_value(sp.bits, idx) * d * sc;
+    } else if constexpr (sp.codec == Codec::Q6K) {
+        // [192 B levels stored +32][16 int8 scales][binary16 d]
+        const uint32_t code = stream_bits(p, BB, i * 6u, 6);
+        const float sc = (float)(int)(int8_t)p[192 + (i >> 4)];
+        const float d = half_bits_to_float((uint32_t)p[208] | ((uint32_t)p[209] << 8));
+        v = (d * sc) * (float)((int)code - 32);
+        v = v + 0.0f;  // the reference computes e * level + 0 here: never -0
     } else if constexpr (sp.codec == Codec::Sym32) {
         constexpr uint32_t code_bytes = 256u * sp.bits / 8;
         const uint32_t g = i >> 5;
@@ -83,6 +112,81 @@ __device__ __forceinline__ float decode_weight(const uint8_t* __restrict__ p, ui
         v = (float)q * d;
     }
     return v;
+}
+
+// Weight i of a block of L.n <= 256 weights.  Every part of such a block is one
+// LSB-first bit stream without byte alignment between the parts, except where the
+// reference's encoder places a trailer at a byte offset (noted below).
+__device__ __forceinline__ float decode_weight_short(const BlockLayout& L, const uint8_t* __restrict__ p, uint32_t i) {
+    const uint32_t size = (uint32_t)L.bytes, bits = (uint32_t)L.bits, n = (uint32_t)L.n;
+    switch (L.kind) {
+        case BK_RAW32:
+            return __uint_as_float(stream_bits(p, size, i * 32, 16) | (stream_bits(p, size, i * 32 + 16, 16) << 16));
+        case BK_LEVELS:  // fewer than 16 weights: no header, implied scale 1 (:450-455, :508-511)
+            return grid_value(L.bits, stream_bits(p, size, i * bits, L.bits));
+        case BK_LATTICE: {
+            // 16 slots spread by is_slot (:176-180): weight i is one when floor(16 (i + 1) / n) steps
+            const uint32_t before = (i * 16u) / n;
+            const bool slot = ((i + 1u) * 16u) / n != before;
+            const float scale = half_bits_to_float(stream_bits(p, size, 0, 16));
+            uint32_t idx = stream_bits(p, size, 16u + bits * i - before, L.bits - (slot ? 1 : 0));
+            if (slot) idx <<= 1;
+            if (L.bits == 8) return scale * __uint_as_float(kComp8Bits[min(idx, 255u)]);
+            return grid_value(L.bits, idx) * scale;
+        }
+        case BK_AFFINE: {
+            // the decoder reads n levels, then ng scale codes, ng min codes, d, dm; weights past
+            // the last whole group stay zero (:1626-1687)
+            const uint32_t g = i / (uint32_t)L.gsz, ng = (uint32_t)L.ng;
+            if (g >= ng) return 0.0f;
+            const uint32_t base = n * bits;
+            const uint32_t idx = stream_bits(p, size, i * bits, L.bits);
+            const float sc = (float)stream_bits(p, size, base + g * L.scb, L.scb);
+            const float mc = (float)stream_bits(p, size, base + ng * L.scb + g * L.mb, L.mb) - (float)((1 << L.mb) / 2);
+            const uint32_t tail = base + ng * (uint32_t)(L.scb + L.mb);
+            const float d = half_bits_to_float(stream_bits(p, size, tail, 16));
+            const float dm = half_bits_to_float(stream_bits(p, size, tail + 16, 16));
+            const float es = d * sc;
+            const float neg = -(dm * mc);
+            return __builtin_fmaf(es, unit_level(L.bits, idx), neg);
+        }
+        case BK_GRP16: {
+            const uint32_t idx = stream_bits(p, size, i * bits, L.bits);
+            float d = 1.0f, sc = 1.0f;
+            if (L.aux == 2) {
+                const uint32_t ng = n >> 3;
+                sc = (float)stream_bits(p, size, n * bits + min(i >> 3, ng - 1u) * 3u, 3);
+                d = half_bits_to_float(stream_bits(p, size, n * bits + ng * 3u, 16));
+            } else if (L.aux == 1) {
+                d = half_bits_to_float((uint32_t)p[size - 2] | ((uint32_t)p[size - 1] << 8));  // byte aligned trailer
+            }
+            return grid_value(L.bits, idx) * d * sc;
+        }
+        case BK_Q6K: {
+            const uint32_t code = stream_bits(p, size, i * 6u, 6);
+            float d = 1.0f, sc = 1.0f;
+            if (L.aux & 1) {
+                d = half_bits_to_float((uint32_t)p[size - 2] | ((uint32_t)p[size - 1] << 8));
+                const uint32_t stored = (uint32_t)L.aux >> 8;
+                if (stored) sc = (float)(int)(int8_t)p[size - 2 - stored + min(i >> 4, stored - 1u)];
+            }
+            float v = (d * sc) * (float)((int)code - 32);
+            // whole groups of 16 go through the reference's e * level + 0 path (never -0), a
+            // partial last group through a plain multiply (:1278-1301)
+            if ((i | 15u) < n) v = v + 0.0f;
+            return v;
+        }
+        case BK_GRP8: {
+            const uint32_t h = (uint32_t)p[n + 2 * (i >> 5)] | ((uint32_t)p[n + 2 * (i >> 5) + 1] << 8);
+            return half_bits_to_float(h) * __uint_as_float(kComp8Bits[p[i]]);
+        }
+        default: {  // BK_SYM32
+            const uint32_t code_bytes = n * bits / 8;
+            const uint32_t h = (uint32_t)p[code_bytes + 2 * (i >> 5)] | ((uint32_t)p[code_bytes + 2 * (i >> 5) + 1] << 8);
+            const int q = L.bits == 4 ? (int)((p[i >> 1] >> ((i & 1u) * 4)) & 15u) - 8 : (int)(int8_t)p[i];
+            return (float)q * half_bits_to_float(h);
+        }
+    }
 }
 
 }  // namespace tfq

@@ -114,6 +114,12 @@ int launch_gemv_generic(const tfq_weight* w, const void* x, int x_dtype, int B, 
     if (w->N > 0x7FFFFFFF || w->K > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "gemv: shape too large");
     switch (canonical(w->fmt)) {
         case TFQ_Q_32: return batched<TFQ_Q_32>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_2: return batched<TFQ_Q_2>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_G_6: return batched<TFQ_Q_G_6>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_G_2_K_L: return batched<TFQ_Q_G_2_K_L>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_G_3_K_L: return batched<TFQ_Q_G_3_K_L>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_G_4_K_L: return batched<TFQ_Q_G_4_K_L>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_6_5: return batched<TFQ_Q_6_5>(w, x, x_dtype, B, y, y_dtype, s);
         case TFQ_Q_4: return batched<TFQ_Q_4>(w, x, x_dtype, B, y, y_dtype, s);
         case TFQ_Q_8: return batched<TFQ_Q_8>(w, x, x_dtype, B, y, y_dtype, s);
         case TFQ_Q_G_2: return batched<TFQ_Q_G_2>(w, x, x_dtype, B, y, y_dtype, s);

@@ -13,7 +13,7 @@
 namespace tfq {
 
 // ------------------------------------------------------------------ formats
-enum class Codec : int { None = 0, Raw32, Lattice, Affine, Grp8, Sym32 };
+enum class Codec : int { None = 0, Raw32, Lattice, Affine, Grp8, Sym32, Grp16, Q6K };
 
 // Layout parameters of one wire format.  The affine family is the reference's
 // parametric codec quant_affine(bits, w, n, gsz, scb, mb, claimed)
@@ -24,19 +24,34 @@ struct Spec {
     int bits;     // code width
     int gsz;      // weights per group
     int scb, mb;  // scale / min code widths (affine)
-    float bpw;    // wire bits per weight of a full 256-block
+    float bpw;    // claimed bits per weight
     int block_bytes;  // payload bytes of a full 256-block
 };
+
+// Grp16 is the layout the affine family degrades to when its header does not fit the
+// claim (quant_grp16 / dequant_grp16, src/codec/block_codec.cpp:788-945): groups of 8,
+// a 3-bit scale code each, one binary16 d.  The ids that claim 1/16 bit less than the
+// affine layout needs (Q_G_{2,3,4}_K_*, Q_2_5, Q_6_5) use it for every block.
+// Q6K is Q_G_6 (quant_6k / dequant_6k, :1046-1303): 6-bit levels, int8 scale per 16.
 
 __host__ __device__ constexpr Spec spec_of(int fmt) {
     switch (fmt) {
         case TFQ_Q_32: return {Codec::Raw32, 32, 0, 0, 0, 32.0f, 1024};
+        case TFQ_Q_2: return {Codec::Lattice, 2, 0, 0, 0, 2.0f, 64};
         case TFQ_Q_4: return {Codec::Lattice, 4, 0, 0, 0, 4.0f, 128};
         case TFQ_Q_8: return {Codec::Lattice, 8, 0, 0, 0, 8.0f, 256};
         case TFQ_Q_G_4: case TFQ_Q_4_5: case TFQ_Q_G_4_5: return {Codec::Affine, 4, 32, 6, 6, 4.5f, 144};
         case TFQ_Q_G_3: case TFQ_Q_3_5: case TFQ_Q_G_3_5: return {Codec::Affine, 3, 32, 6, 6, 3.5f, 112};
         case TFQ_Q_G_2: return {Codec::Affine, 2, 16, 4, 4, 2.625f, 84};
         case TFQ_Q_G_8: case TFQ_Q_8_5: case TFQ_Q_G_8_5: return {Codec::Grp8, 8, 32, 0, 0, 8.5f, 272};
+        case TFQ_Q_G_6: case TFQ_Q_G_6_K_L: case TFQ_Q_G_6_K_M: case TFQ_Q_G_6_K_H:
+            return {Codec::Q6K, 6, 16, 8, 0, 6.5625f, 210};
+        // scb / mb keep the affine parameters: a short block of these ids may still fit the affine layout
+        case TFQ_Q_G_2_K_L: case TFQ_Q_G_2_K_M: case TFQ_Q_G_2_K_H: return {Codec::Grp16, 2, 16, 4, 4, 2.4375f, 78};
+        case TFQ_Q_2_5: case TFQ_Q_G_2_5: return {Codec::Grp16, 2, 16, 4, 4, 2.5f, 78};
+        case TFQ_Q_G_3_K_L: case TFQ_Q_G_3_K_M: case TFQ_Q_G_3_K_H: return {Codec::Grp16, 3, 32, 6, 6, 3.4375f, 110};
+        case TFQ_Q_G_4_K_L: case TFQ_Q_G_4_K_M: case TFQ_Q_G_4_K_H: return {Codec::Grp16, 4, 32, 6, 6, 4.4375f, 142};
+        case TFQ_Q_6_5: case TFQ_Q_G_6_5: return {Codec::Grp16, 6, 32, 8, 8, 6.5f, 206};
         case TFQ_SB256A3: return {Codec::Affine, 3, 16, 6, 6, 3.875f, 124};
         case TFQ_SB256A2: return {Codec::Affine, 2, 16, 6, 6, 2.875f, 92};
         case TFQ_B32S4: return {Codec::Sym32, 4, 32, 0, 0, 4.5f, 144};
@@ -52,6 +67,11 @@ __host__ __device__ constexpr int canonical(int fmt) {
         case TFQ_Q_4_5: case TFQ_Q_G_4_5: return TFQ_Q_G_4;
         case TFQ_Q_3_5: case TFQ_Q_G_3_5: return TFQ_Q_G_3;
         case TFQ_Q_8_5: case TFQ_Q_G_8_5: return TFQ_Q_G_8;
+        case TFQ_Q_G_6_K_L: case TFQ_Q_G_6_K_M: case TFQ_Q_G_6_K_H: return TFQ_Q_G_6;
+        case TFQ_Q_G_2_K_M: case TFQ_Q_G_2_K_H: case TFQ_Q_2_5: case TFQ_Q_G_2_5: return TFQ_Q_G_2_K_L;
+        case TFQ_Q_G_3_K_M: case TFQ_Q_G_3_K_H: return TFQ_Q_G_3_K_L;
+        case TFQ_Q_G_4_K_M: case TFQ_Q_G_4_K_H: return TFQ_Q_G_4_K_L;
+        case TFQ_Q_G_6_5: return TFQ_Q_6_5;
         default: return fmt;
     }
 }
@@ -115,8 +135,25 @@ struct tfq_weight {
 
 namespace tfq {
 
+// Layout of one block of n <= 256 weights, as the reference's codecs choose it from
+// (format, n): short blocks drop or shrink their headers.  Filled on the host, passed
+// to the short-block decode kernel by value.
+enum : int { BK_RAW32 = 0, BK_LEVELS, BK_LATTICE, BK_AFFINE, BK_GRP16, BK_Q6K, BK_GRP8, BK_SYM32 };
+struct BlockLayout {
+    int kind;
+    int bits;   // code width
+    int n;      // weights in the block
+    int bytes;  // payload bytes
+    int gsz, ng, scb, mb;  // affine: group size, group count, scale / min code widths
+    int aux;    // BK_GRP16: 0 raw levels, 1 one d, 2 group scales + d.  BK_Q6K: bit 0 d present, bits 8.. stored scale count
+};
+// false when the format cannot hold a block of n weights
+bool block_layout(int fmt, int n, BlockLayout* out);
+
 // ------------------------------------------------------------- kernel launchers
 int launch_decode(int fmt, const uint8_t* src, int64_t nblocks, float* out, hipStream_t s);
+// one block of L.n <= 256 weights in the layout L
+int launch_decode_short(const BlockLayout& L, const uint8_t* src, float* out, hipStream_t s);
 int launch_tile16(int fmt, const uint8_t* wire, uint8_t* tiled, int64_t N, int64_t K, hipStream_t s);
 int launch_decode_tiled(int fmt, const uint8_t* tiled, int64_t N, int64_t K, float* out, hipStream_t s);
 int launch_encode(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStream_t s);
