@@ -77,6 +77,43 @@ float tfq_format_bpw(uint8_t fmt);
 int tfq_format_supported(uint8_t fmt);
 int tfq_block_bytes(uint8_t fmt, uint32_t n, size_t* out);
 
+/* ---- .quant container ------------------------------------------------------
+ * QUANTReader (include/quant/quant_format.h:64-149, src/codec/quant_format.cpp:319-640):
+ * header, per-block format table, tensor table, block records
+ * [u32 weights][u32 cb_bytes][codebook][u32 idx_bytes][payload] (write_block, :249-263).
+ * Every file-controlled count and range is checked; a corrupt value gives an error
+ * status, never an access outside the image.  A stored format byte outside the
+ * enum, or 19, reads as Q_32 (read_block, :430-434); ids 105..108 are this library's
+ * appended formats.  open / from_memory return NULL only when the image cannot be
+ * read; an image that fails validation is returned with tfq_container_valid == 0,
+ * like QUANTReader::valid(). */
+typedef struct tfq_container tfq_container_t;
+tfq_container_t* tfq_container_open(const char* path);
+tfq_container_t* tfq_container_from_memory(const void* image, size_t bytes); /* copies the image */
+void tfq_container_close(tfq_container_t* c);
+int tfq_container_valid(const tfq_container_t* c);
+int tfq_container_header(const tfq_container_t* c, uint32_t* version, uint32_t* flags,
+                         const uint8_t** config, size_t* config_size);
+int64_t tfq_container_num_blocks(const tfq_container_t* c);
+int tfq_container_num_tensors(const tfq_container_t* c);
+/* tensor_names (:579-596): copies name `index` (NUL terminated), returns its length or -status */
+int tfq_container_tensor_name(const tfq_container_t* c, int index, char* buf, size_t cap);
+/* tensor_blocks (:463-491) */
+int tfq_container_tensor_blocks(const tfq_container_t* c, const char* name, uint32_t* start, uint32_t* count);
+/* block_sizes / block_ptr / format_entry (:440-461); idx points into the container's image */
+int tfq_container_block(const tfq_container_t* c, uint32_t block_id, uint8_t* format, uint32_t* weights,
+                        uint32_t* cb_bytes, uint32_t* idx_bytes, const uint8_t** idx);
+/* sum of the stored block sizes of a tensor, or -status */
+int64_t tfq_container_tensor_weights(const tfq_container_t* c, const char* name);
+/* read_tensor (:515-577), decoded on the device; out is a device (resp. host) buffer of cap floats */
+int tfq_container_read_tensor(const tfq_container_t* c, const char* name, float* out, int64_t cap,
+                              tfq_stream_t stream);
+int tfq_container_read_tensor_host(const tfq_container_t* c, const char* name, float* out, int64_t cap);
+/* Qwen35Engine::resolve (src/adapters/tools/qwen35_engine.cpp:116-150) + upload: the tensor's
+ * first rows * cols / 256 blocks as a device-resident matrix.  All of them must be full blocks
+ * of one format. */
+tfq_weight_t* tfq_container_weight(const tfq_container_t* c, const char* name, int64_t rows, int64_t cols);
+
 /* ---- block codec ------------------------------------------------------------
  * quantize_block_all / dequantize_block_all (include/quant/block_codec.h:69-77),
  * applied to a tensor cut into 256-weight blocks the way

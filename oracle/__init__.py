@@ -424,3 +424,50 @@ def ref_fp24_round_trip(w):
     ref.ref_fp24_encode(_ptr(w, _f32p), _ptr(packed, _u8p), w.size)
     ref.ref_fp24_decode(_ptr(packed, _u8p), _ptr(back, _f32p), w.size)
     return packed, back
+
+
+def ref_container_write(path: str, tensors, block_fmt, config: bytes = b"", version: int = 1 << 22) -> int:
+    """tensors: list of (name, fp32 array); block_fmt: wire id of every 256-block of the file, in order."""
+    names = (C.c_char_p * len(tensors))(*[n.encode() for n, _ in tensors])
+    data = np.concatenate([_f32(w).reshape(-1) for _, w in tensors])
+    sizes = np.array([np.size(w) for _, w in tensors], np.int64)
+    offsets = np.concatenate([[0], np.cumsum(sizes)[:-1]]).astype(np.int64)
+    fm = np.array([fmt_id(f) for f in block_fmt], np.uint8)
+    assert fm.size == int(((sizes + 255) // 256).sum())
+    i64p = C.POINTER(C.c_int64)
+    ref.ref_container_write.argtypes = [C.c_char_p, C.c_int, C.POINTER(C.c_char_p), _f32p, i64p, i64p, _u8p,
+                                        C.c_char_p, C.c_uint32, C.c_uint32]
+    return ref.ref_container_write(path.encode(), len(tensors), names, _ptr(data, _f32p), offsets.ctypes.data_as(i64p),
+                                   sizes.ctypes.data_as(i64p), _ptr(fm, _u8p), config, len(config), version)
+
+
+def ref_container_info(path: str):
+    out = np.zeros(5, np.int64)
+    ref.ref_container_info.argtypes = [C.c_char_p, C.POINTER(C.c_int64)]
+    ref.ref_container_info(path.encode(), out.ctypes.data_as(C.POINTER(C.c_int64)))
+    return dict(valid=bool(out[0]), blocks=int(out[1]), tensors=int(out[2]), version=int(out[3]), config_size=int(out[4]))
+
+
+def ref_container_tensor_blocks(path: str, name: str):
+    s, k = C.c_uint32(0), C.c_uint32(0)
+    ref.ref_container_tensor_blocks.argtypes = [C.c_char_p, C.c_char_p, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
+    ok = ref.ref_container_tensor_blocks(path.encode(), name.encode(), C.byref(s), C.byref(k))
+    return (s.value, k.value) if ok else None
+
+
+def ref_container_block(path: str, block_id: int):
+    out = np.zeros(5, np.int64)
+    ref.ref_container_block.argtypes = [C.c_char_p, C.c_uint32, C.POINTER(C.c_int64)]
+    if ref.ref_container_block(path.encode(), block_id, out.ctypes.data_as(C.POINTER(C.c_int64))) != 0:
+        return None
+    return dict(format=int(out[0]), weights=int(out[1]), cb_bytes=int(out[2]), idx_bytes=int(out[3]), offset=int(out[4]))
+
+
+def ref_container_read_tensor(path: str, name: str, cap: int = 1 << 22) -> np.ndarray:
+    out = np.empty(cap, np.float32)
+    ref.ref_container_read_tensor.restype = C.c_int64
+    ref.ref_container_read_tensor.argtypes = [C.c_char_p, C.c_char_p, _f32p, C.c_int64]
+    n = ref.ref_container_read_tensor(path.encode(), name.encode(), _ptr(out, _f32p), cap)
+    if n < 0:
+        raise RuntimeError("reference read_tensor: destination too small")
+    return out[:n].copy()

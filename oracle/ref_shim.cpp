@@ -14,11 +14,13 @@
 //       (include/quant/kernel.h:24-60)
 //   quant::adapters::prod::gemv_quant{4,8}_{tiled,batch}
 //       (include/quant/kernel_production.h:25-51)
+//   quant::QUANTWriter / quant::QUANTReader (include/quant/quant_format.h:43-149)
 
 #include "quant/block_codec.h"
 #include "quant/format_registry.h"
 #include "quant/kernel.h"
 #include "quant/kernel_production.h"
+#include "quant/quant_format.h"
 #include "quant/random.h"
 
 #include <cstring>
@@ -117,4 +119,94 @@ void ref_lutn_gemm(int bits, const uint8_t* w, const void* cb, const float* act,
 }
 void ref_fp24_encode(const float* w, uint8_t* packed, int count) { quant::kernel::q24_encode(w, packed, count); }
 void ref_fp24_decode(const uint8_t* packed, float* w, int count) { quant::kernel::q24_decode(packed, w, count); }
+// ---- .quant container: written with QUANTWriter in the reader's order (header,
+// format table, tensor table, block records; tools/convert.cpp:458-540), read
+// back with QUANTReader.
+// tensors: `count` of them, tensor t has sizes[t] weights at data + offsets[t], named
+// names[t], and is cut into 256-blocks; block b of the file is encoded as block_fmt[b].
+int ref_container_write(const char* path, int count, const char* const* names, const float* data,
+                        const int64_t* offsets, const int64_t* sizes, const uint8_t* block_fmt,
+                        const uint8_t* config, uint32_t config_size, uint32_t version) {
+    using namespace quant;
+    std::vector<FormatBlockEntry> ft;
+    std::vector<TensorEntry> te;
+    std::vector<std::string> nm;
+    std::vector<BlockData> blocks;
+    uint32_t bid = 0;
+    for (int t = 0; t < count; ++t) {
+        const int64_t nb = (sizes[t] + 255) / 256;
+        TensorEntry e;
+        e.name_len = (uint16_t)std::strlen(names[t]);
+        e.block_start = bid;
+        e.num_blocks = (uint32_t)nb;
+        te.push_back(e);
+        nm.push_back(names[t]);
+        for (int64_t b = 0; b < nb; ++b, ++bid) {
+            const int64_t st = b * 256, n = std::min<int64_t>(256, sizes[t] - st);
+            BlockData bd;
+            bd.format = (Format)block_fmt[bid];
+            bd.num_weights = (uint32_t)n;
+            if (!quantize_block_all(bd.format, data + offsets[t] + st, (int)n, bd.indices, bd.codebook)) return -1;
+            FormatBlockEntry f;
+            f.block_id = bid;
+            f.format = block_fmt[bid];
+            f.cb_bytes = (uint32_t)bd.codebook.size();
+            ft.push_back(f);
+            blocks.push_back(std::move(bd));
+        }
+    }
+    QUANTWriter w(path);
+    QUANTHeader h;
+    std::memcpy(h.magic, "QUA1", 4);
+    h.version = version;
+    h.flags = 0;
+    h.config_size = config_size;
+    w.write_header(h, config);
+    w.write_format_table(ft);
+    w.write_tensor_table(te, nm);
+    for (const auto& b : blocks) w.write_block(b);
+    w.close();
+    return (int)bid;
+}
+
+// valid, num_blocks, tensors, version, config_size
+int ref_container_info(const char* path, int64_t* out5) {
+    quant::QUANTReader r(path);
+    out5[0] = r.valid() ? 1 : 0;
+    out5[1] = (int64_t)r.num_blocks();
+    out5[2] = (int64_t)r.tensor_names().size();
+    out5[3] = r.valid() ? (int64_t)r.header().version : 0;
+    out5[4] = r.valid() ? (int64_t)r.header().config_size : 0;
+    return 0;
+}
+
+int ref_container_tensor_blocks(const char* path, const char* name, uint32_t* start, uint32_t* count) {
+    quant::QUANTReader r(path);
+    return r.tensor_blocks(name, *start, *count) ? 1 : 0;
+}
+
+// format byte as the readers see it (clamped), nw, cb_bytes, idx_bytes, file offset; -1 when out of range
+int ref_container_block(const char* path, uint32_t block_id, int64_t* out5) {
+    quant::QUANTReader r(path);
+    uint32_t cb = 0, idx = 0;
+    if (!r.block_sizes(block_id, &cb, &idx)) return -1;
+    const quant::BlockData bd = r.read_block(block_id);
+    out5[0] = (int64_t)(uint8_t)bd.format;
+    out5[1] = bd.num_weights;
+    out5[2] = cb;
+    out5[3] = idx;
+    out5[4] = (int64_t)r.block_offset(block_id);
+    return 0;
+}
+
+// decoded weights of a named tensor; returns their count (0 = empty tensor), -1 if cap is too small
+int64_t ref_container_read_tensor(const char* path, const char* name, float* out, int64_t cap) {
+    quant::QUANTReader r(path);
+    quant::Tensor t = r.read_tensor(name);
+    const int64_t n = t.numel();
+    if (n > cap) return -1;
+    if (n > 0) std::memcpy(out, t.data<float>(), (size_t)n * 4);
+    return n;
+}
+
 }  // extern "C"

@@ -23,6 +23,11 @@ tails.npz
     bytes, decoded offset) into the flat `payloads` / `decoded` arrays: the short-block
     layouts (raw levels, one scale, grouped-lattice fallback), Q_2, Q_G_6 and the ids
     whose claim is below the affine header's size
+sample.quant, sample_quant.npz
+    a container written by the reference's QUANTWriter (header with a 5-byte config,
+    format table, tensor table, block records): tensor "blk.0.ffn_gate" 4 x 512 in Q_G_4,
+    "mixed" whose blocks alternate formats, "tail" of 300 weights in Q_G_8 and "raw" of 40
+    weights in Q_32; the npz holds what QUANTReader::read_tensor returns for each name
 matmul.npz
     for Q_G_4 and Q_G_8: y = x.W^T with W 48x512 from the fixture generator,
     computed by the reference scalar_gemm_bt on the reference-decoded matrix
@@ -76,10 +81,22 @@ def tails(w):
                         decoded=np.concatenate(decs))
 
 
+def container(w):
+    flat = w.reshape(-1)
+    tensors = [("blk.0.ffn_gate", flat[:2048]), ("mixed", flat[2048:2048 + 1280]), ("tail", flat[4096:4396]),
+               ("raw", flat[5000:5040])]
+    fmts = ["Q_G_4"] * 8 + ["Q_G_4", "Q_G_8", "Q_4", "Q_G_6", "Q_G_3_K_L"] + ["Q_G_8", "Q_G_8"] + ["Q_32"]
+    path = os.path.join(HERE, "sample.quant")
+    assert O.ref_container_write(path, tensors, fmts, config=b"hello") == len(fmts)
+    np.savez_compressed(os.path.join(HERE, "sample_quant.npz"),
+                        **{name: O.ref_container_read_tensor(path, name) for name, _ in tensors})
+
+
 def main():
     assert O.have_ref(), "build oracle/_ref first (make -C oracle)"
     w = inputs()
     tails(w)
+    container(w)
     out = {"w": w}
     for fmt in FORMATS:
         pays, decs = [], []
@@ -130,7 +147,7 @@ def main():
         mm[f"{fmt}_payload"] = pays
         mm[f"{fmt}_y"] = Y
     np.savez_compressed(os.path.join(HERE, "matmul.npz"), **mm)
-    for f in ("codec.npz", "rng.npz", "matmul.npz", "tails.npz"):
+    for f in ("codec.npz", "rng.npz", "matmul.npz", "tails.npz", "sample.quant", "sample_quant.npz"):
         print(f, os.path.getsize(os.path.join(HERE, f)))
 
 

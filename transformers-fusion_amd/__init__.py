@@ -69,6 +69,21 @@ def _load():
         "tfq_lutn_gemm": (i32, [i32, vp, vp, vp, vp, i32, i32, i32, vp]),
         "tfq_fp24_encode": (i32, [vp, vp, i64, vp]),
         "tfq_fp24_decode": (i32, [vp, vp, i64, vp]),
+        "tfq_container_open": (vp, [C.c_char_p]),
+        "tfq_container_from_memory": (vp, [vp, sz]),
+        "tfq_container_close": (None, [vp]),
+        "tfq_container_valid": (i32, [vp]),
+        "tfq_container_header": (i32, [vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(vp), C.POINTER(sz)]),
+        "tfq_container_num_blocks": (i64, [vp]),
+        "tfq_container_num_tensors": (i32, [vp]),
+        "tfq_container_tensor_name": (i32, [vp, i32, C.c_char_p, sz]),
+        "tfq_container_tensor_blocks": (i32, [vp, C.c_char_p, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
+        "tfq_container_block": (i32, [vp, C.c_uint32, C.POINTER(u8), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32),
+                                      C.POINTER(C.c_uint32), C.POINTER(vp)]),
+        "tfq_container_tensor_weights": (i64, [vp, C.c_char_p]),
+        "tfq_container_read_tensor": (i32, [vp, C.c_char_p, vp, i64, vp]),
+        "tfq_container_read_tensor_host": (i32, [vp, C.c_char_p, vp, i64]),
+        "tfq_container_weight": (vp, [vp, C.c_char_p, i64, i64]),
         "tfq_malloc": (vp, [sz]),
         "tfq_free": (None, [vp]),
         "tfq_copy_to_device": (i32, [vp, vp, sz]),
@@ -147,10 +162,13 @@ def decode(fmt, payload, n: int):
 class Weight:
     """Device-resident packed matrix W[N][K] (N rows of K/256 wire blocks)."""
 
-    def __init__(self, fmt, N: int, K: int, packed):
+    def __init__(self, fmt, N: int, K: int, packed, handle=None):
         import numpy as np
         import torch
         self.fmt, self.N, self.K = fmt_id(fmt), int(N), int(K)
+        if handle is not None:  # adopted from tfq_container_weight
+            self.handle = C.c_void_p(handle)
+            return
         if isinstance(packed, torch.Tensor) and packed.is_cuda:
             # device payload: copied into the handle's own layout, the caller may drop its tensor
             h = lib().tfq_weight_wrap(self.fmt, N, K, packed.data_ptr(), packed.numel())
@@ -200,6 +218,83 @@ class Weight:
     def gemm(self, x, out_dtype=None):
         """y[M][N] = x[M][K] . W^T for any M (prefill)."""
         return self._mm(lib().tfq_gemm, x, out_dtype)
+
+
+class Container:
+    """A .quant file (QUANTReader, include/quant/quant_format.h:64-149): host-side tables, tensors decoded or
+    uploaded on the device."""
+
+    def __init__(self, path=None, image=None):
+        if path is not None:
+            h = lib().tfq_container_open(os.fsencode(path))
+        else:
+            image = bytes(image)
+            h = lib().tfq_container_from_memory(image, len(image))
+        if not h:
+            raise TfqError(lib().tfq_last_error().decode())
+        self.handle = C.c_void_p(h)
+
+    def close(self):
+        if getattr(self, "handle", None):
+            lib().tfq_container_close(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def valid(self) -> bool:
+        return bool(lib().tfq_container_valid(self.handle))
+
+    @property
+    def num_blocks(self) -> int:
+        return int(lib().tfq_container_num_blocks(self.handle))
+
+    def header(self):
+        ver, flags, cfg, n = C.c_uint32(0), C.c_uint32(0), C.c_void_p(0), C.c_size_t(0)
+        _check(lib().tfq_container_header(self.handle, C.byref(ver), C.byref(flags), C.byref(cfg), C.byref(n)))
+        return ver.value, flags.value, (C.string_at(cfg.value, n.value) if n.value else b"")
+
+    def tensor_names(self):
+        buf = C.create_string_buffer(1 << 16)
+        out = []
+        for i in range(lib().tfq_container_num_tensors(self.handle)):
+            n = lib().tfq_container_tensor_name(self.handle, i, buf, len(buf))
+            if n < 0:
+                raise TfqError(lib().tfq_last_error().decode())
+            out.append(buf.raw[:n].decode("utf-8", "replace"))
+        return out
+
+    def tensor_blocks(self, name: str):
+        s, k = C.c_uint32(0), C.c_uint32(0)
+        _check(lib().tfq_container_tensor_blocks(self.handle, name.encode(), C.byref(s), C.byref(k)))
+        return s.value, k.value
+
+    def block(self, block_id: int):
+        """(format as the readers see it, weights, cb_bytes, payload bytes)"""
+        f, nw, cb, ib, p = C.c_uint8(0), C.c_uint32(0), C.c_uint32(0), C.c_uint32(0), C.c_void_p(0)
+        _check(lib().tfq_container_block(self.handle, block_id, C.byref(f), C.byref(nw), C.byref(cb), C.byref(ib), C.byref(p)))
+        return f.value, nw.value, cb.value, C.string_at(p.value, ib.value)
+
+    def read_tensor(self, name: str, device="cuda"):
+        import torch
+        n = lib().tfq_container_tensor_weights(self.handle, name.encode())
+        if n < 0:
+            raise TfqError(lib().tfq_last_error().decode())
+        out = torch.empty(n, dtype=torch.float32, device=device)
+        _check(lib().tfq_container_read_tensor(self.handle, name.encode(), out.data_ptr(), n, _stream()))
+        return out
+
+    def weight(self, name: str, rows: int, cols: int) -> "Weight":
+        h = lib().tfq_container_weight(self.handle, name.encode(), rows, cols)
+        if not h:
+            raise TfqError(lib().tfq_last_error().decode())
+        f, n, k, b = C.c_uint8(0), C.c_int64(0), C.c_int64(0), C.c_size_t(0)
+        lib().tfq_weight_info(h, C.byref(f), C.byref(n), C.byref(k), C.byref(b))
+        return Weight(f.value, n.value, k.value, None, handle=h)
 
 
 def gemv_multi(weights, x, outs):
