@@ -77,6 +77,42 @@ float tfq_format_bpw(uint8_t fmt);
 int tfq_format_supported(uint8_t fmt);
 int tfq_block_bytes(uint8_t fmt, uint32_t n, size_t* out);
 
+/* ---- in-memory codebook engines ---------------------------------------------
+ * engines::Q4Engine / Q8Engine (include/quant/quant_engines.h:33-100;
+ * src/codec/quant_engines_quant4.cpp:102-150, :213-261; quant_engines_quant8.cpp:92-227):
+ * a shared codebook of 16 (bits = 4) or 256 (bits = 8) fp32 centroids, passed as a host
+ * array; everything else is device memory.  Bit-exact with the reference.
+ *   quantize_per_block   one index byte per weight; scales = (center, half_range) per block
+ *                        for bits 4, absmax per block for bits 8
+ *   quantize_tensor      nearest centroid per value; bits 4 packs two codes per byte
+ *   quant_gemm           C[M][N] = A[M][K] . codebook[codes[K][N]]  (codes of bits 4 packed
+ *                        flat, element k*N+n)
+ * These calls return after the stream has finished (the codebook staging buffer is theirs). */
+int tfq_engine_quantize_per_block(int bits, const float* codebook, const float* data, int64_t n, int64_t block_size,
+                                  uint8_t* indices, float* scales, tfq_stream_t stream);
+int tfq_engine_dequantize_per_block(int bits, const float* codebook, const uint8_t* indices, const float* scales,
+                                    int64_t n, int64_t block_size, float* out, tfq_stream_t stream);
+int tfq_engine_quantize_tensor(int bits, const float* codebook, const float* data, int64_t n, uint8_t* out,
+                               tfq_stream_t stream);
+int tfq_engine_dequant_tensor(int bits, const float* codebook, const uint8_t* indices, int64_t n, float* out,
+                              tfq_stream_t stream);
+int tfq_engine_quant_gemm(int bits, const float* codebook, const float* a, const uint8_t* b_idx, int64_t M, int64_t N,
+                          int64_t K, float* c, tfq_stream_t stream);
+/* quant8::Q8Encoder::encode_tensor / Q8Decoder::decode_blocks (engines/quant/codec.cpp:19-78) with
+ * CodebookQ8::train / quantize (src/codec/codebook.cpp:70-185): a 256-entry k-means codebook
+ * per block of block_size <= 256 weights; centroids is [blocks][256] fp32.  Bit-exact. */
+int tfq_q8codec_encode(const float* data, int64_t total, int block_size, float* centroids, uint8_t* indices,
+                       tfq_stream_t stream);
+int tfq_q8codec_decode(const float* centroids, const uint8_t* indices, int64_t total, int block_size, float* out,
+                       tfq_stream_t stream);
+/* quant8::quantize_activations / quantize_tensor (batch = 1) / dequantize
+ * (engines/quant/quantize.cpp:14-101): per row of [batch][per_row], affine uint8
+ * (dst_f32 = 0) or the x * 127/absmax fp32 form (dst_f32 = 1); params (device) receives
+ * (scale, inv_scale, zero_point) per row, dequantize reads one such triple. */
+int tfq_q8_quantize_rows(const float* src, int64_t batch, int64_t per_row, int dst_f32, void* dst, float* params,
+                         tfq_stream_t stream);
+int tfq_q8_dequantize(const void* src, int64_t n, int src_f32, const float* params, float* out, tfq_stream_t stream);
+
 /* ---- .quant container ------------------------------------------------------
  * QUANTReader (include/quant/quant_format.h:64-149, src/codec/quant_format.cpp:319-640):
  * header, per-block format table, tensor table, block records

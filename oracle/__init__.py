@@ -471,3 +471,93 @@ def ref_container_read_tensor(path: str, name: str, cap: int = 1 << 22) -> np.nd
     if n < 0:
         raise RuntimeError("reference read_tensor: destination too small")
     return out[:n].copy()
+
+
+# ---- in-memory codebook engines (Q4Engine / Q8Engine, quant8 codec): oracle and compiled reference share signatures
+def _engine_lib(use_ref):
+    return ref if use_ref else lib
+
+
+def _pfx(use_ref):
+    return "ref_" if use_ref else "orc_"
+
+
+def engine_quantize_per_block(bits, cb, data, block_size, use_ref=False):
+    cb, data = _f32(cb), _f32(data).reshape(-1)
+    nb = (data.size + block_size - 1) // block_size
+    idx = np.zeros(data.size, np.uint8)
+    scales = np.zeros(nb * (2 if bits == 4 else 1), np.float32)
+    fn = getattr(_engine_lib(use_ref), _pfx(use_ref) + "engine_quantize_per_block")
+    fn.argtypes = [C.c_int, _f32p, _f32p, C.c_int64, C.c_int64, _u8p, _f32p]
+    fn(bits, _ptr(cb, _f32p), _ptr(data, _f32p), data.size, block_size, _ptr(idx, _u8p), _ptr(scales, _f32p))
+    return idx, scales
+
+
+def engine_dequantize_per_block(bits, cb, idx, scales, block_size, use_ref=False):
+    cb, scales = _f32(cb), _f32(scales)
+    idx = np.ascontiguousarray(idx, np.uint8)
+    out = np.zeros(idx.size, np.float32)
+    fn = getattr(_engine_lib(use_ref), _pfx(use_ref) + "engine_dequantize_per_block")
+    fn.argtypes = [C.c_int, _f32p, _u8p, _f32p, C.c_int64, C.c_int64, _f32p]
+    fn(bits, _ptr(cb, _f32p), _ptr(idx, _u8p), _ptr(scales, _f32p), idx.size, block_size, _ptr(out, _f32p))
+    return out
+
+
+def engine_quantize_tensor(bits, cb, data, use_ref=False):
+    cb, data = _f32(cb), _f32(data).reshape(-1)
+    out = np.zeros(data.size if bits == 8 else (data.size + 1) // 2, np.uint8)
+    fn = getattr(_engine_lib(use_ref), _pfx(use_ref) + "engine_quantize_tensor")
+    fn.argtypes = [C.c_int, _f32p, _f32p, C.c_int64, _u8p]
+    fn(bits, _ptr(cb, _f32p), _ptr(data, _f32p), data.size, _ptr(out, _u8p))
+    return out
+
+
+def engine_dequant_tensor(bits, cb, idx, n, use_ref=False):
+    cb = _f32(cb)
+    idx = np.ascontiguousarray(idx, np.uint8)
+    out = np.zeros(n, np.float32)
+    fn = getattr(_engine_lib(use_ref), _pfx(use_ref) + "engine_dequant_tensor")
+    fn.argtypes = [C.c_int, _f32p, _u8p, C.c_int64, _f32p]
+    fn(bits, _ptr(cb, _f32p), _ptr(idx, _u8p), n, _ptr(out, _f32p))
+    return out
+
+
+def engine_quant_gemm(bits, cb, a, b_idx, M, N, K, use_ref=False):
+    cb, a = _f32(cb), _f32(a)
+    b_idx = np.ascontiguousarray(b_idx, np.uint8)
+    out = np.zeros((M, N), np.float32)
+    fn = getattr(_engine_lib(use_ref), _pfx(use_ref) + "engine_quant_gemm")
+    fn.argtypes = [C.c_int, _f32p, _f32p, _u8p, C.c_int64, C.c_int64, C.c_int64, _f32p]
+    fn(bits, _ptr(cb, _f32p), _ptr(a, _f32p), _ptr(b_idx, _u8p), M, N, K, _ptr(out, _f32p))
+    return out
+
+
+def q8codec_block(w, use_ref=False):
+    """(centroids[256], indices, decoded) of Q8Encoder::encode / Q8Decoder::decode on one block of <= 256 weights."""
+    w = _f32(w).reshape(-1)
+    cent, idx, dec = np.zeros(256, np.float32), np.zeros(w.size, np.uint8), np.zeros(w.size, np.float32)
+    fn = getattr(_engine_lib(use_ref), _pfx(use_ref) + "q8codec_block")
+    fn.argtypes = [_f32p, C.c_uint32, _f32p, _u8p, _f32p]
+    fn(_ptr(w, _f32p), w.size, _ptr(cent, _f32p), _ptr(idx, _u8p), _ptr(dec, _f32p))
+    return cent, idx, dec
+
+
+def q8_quantize_rows(src, dst_f32=False, use_ref=False):
+    src = _f32(src)
+    batch, per = src.shape
+    dst = np.zeros((batch, per), np.float32 if dst_f32 else np.uint8)
+    params = np.zeros((batch, 3), np.float32)
+    fn = getattr(_engine_lib(use_ref), _pfx(use_ref) + "q8_quantize_rows")
+    fn.argtypes = [_f32p, C.c_int64, C.c_int64, C.c_int, C.c_void_p, _f32p]
+    fn(_ptr(src, _f32p), batch, per, int(dst_f32), dst.ctypes.data, _ptr(params, _f32p))
+    return dst, params
+
+
+def q8_dequantize(src, params3, use_ref=False):
+    src = np.ascontiguousarray(src)
+    params3 = _f32(params3)
+    out = np.zeros(src.size, np.float32)
+    fn = getattr(_engine_lib(use_ref), _pfx(use_ref) + "q8_dequantize")
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_int, _f32p, _f32p]
+    fn(src.ctypes.data, src.size, int(src.dtype == np.float32), _ptr(params3, _f32p), _ptr(out, _f32p))
+    return out

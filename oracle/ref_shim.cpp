@@ -15,16 +15,30 @@
 //   quant::adapters::prod::gemv_quant{4,8}_{tiled,batch}
 //       (include/quant/kernel_production.h:25-51)
 //   quant::QUANTWriter / quant::QUANTReader (include/quant/quant_format.h:43-149)
+//   quant::engines::Q4Engine / Q8Engine (include/quant/quant_engines.h:33-100)
+//   quant::quant8::Q8Encoder / Q8Decoder (engines/quant/codec.h), quantize_tensor /
+//       quantize_activations / dequantize (engines/quant/quantize.h)
 
 #include "quant/block_codec.h"
 #include "quant/format_registry.h"
 #include "quant/kernel.h"
 #include "quant/kernel_production.h"
 #include "quant/quant_format.h"
+#include "quant/quant_engines.h"
+#include "codec.h"
+#include "quantize.h"
 #include "quant/random.h"
 
 #include <cstring>
 #include <vector>
+
+// The engines keep their codebook private; the wrappers below write the caller's
+// centroids through the const accessor.
+template <class E>
+static void set_codebook(E& e, const float* cb, int count) {
+    auto& v = const_cast<std::vector<float>&>(e.codebook());
+    v.assign(cb, cb + count);
+}
 
 extern "C" {
 
@@ -207,6 +221,80 @@ int64_t ref_container_read_tensor(const char* path, const char* name, float* out
     if (n > cap) return -1;
     if (n > 0) std::memcpy(out, t.data<float>(), (size_t)n * 4);
     return n;
+}
+
+// ---- in-memory codebook engines
+
+void ref_engine_quantize_per_block(int bits, const float* cb, const float* data, int64_t n, int64_t bs,
+                                   uint8_t* idx, float* scales) {
+    if (bits == 4) { quant::engines::Q4Engine e; set_codebook(e, cb, 16); e.quantize_per_block(data, n, bs, idx, scales); }
+    else { quant::engines::Q8Engine e; set_codebook(e, cb, 256); e.quantize_per_block(data, n, bs, idx, scales); }
+}
+
+void ref_engine_dequantize_per_block(int bits, const float* cb, const uint8_t* idx, const float* scales, int64_t n,
+                                     int64_t bs, float* out) {
+    if (bits == 4) { quant::engines::Q4Engine e; set_codebook(e, cb, 16); e.dequantize_per_block(idx, scales, n, bs, out); }
+    else { quant::engines::Q8Engine e; set_codebook(e, cb, 256); e.dequantize_per_block(idx, scales, n, bs, out); }
+}
+
+void ref_engine_quantize_tensor(int bits, const float* cb, const float* data, int64_t n, uint8_t* out) {
+    quant::Tensor t;
+    if (bits == 4) { quant::engines::Q4Engine e; set_codebook(e, cb, 16); t = e.quantize_tensor(data, n); }
+    else { quant::engines::Q8Engine e; set_codebook(e, cb, 256); t = e.quantize_tensor(data, n); }
+    std::memcpy(out, t.data<uint8_t>(), (size_t)t.numel());
+}
+
+void ref_engine_dequant_tensor(int bits, const float* cb, const uint8_t* idx, int64_t n, float* out) {
+    quant::Tensor t;
+    if (bits == 4) { quant::engines::Q4Engine e; set_codebook(e, cb, 16); t = e.dequant_tensor(idx, n); }
+    else { quant::engines::Q8Engine e; set_codebook(e, cb, 256); t = e.dequant_tensor(idx, n); }
+    std::memcpy(out, t.data<float>(), (size_t)n * 4);
+}
+
+void ref_engine_quant_gemm(int bits, const float* cb, const float* a, const uint8_t* b_idx, int64_t M, int64_t N,
+                           int64_t K, float* c) {
+    quant::Tensor at(quant::Shape{M, K}, quant::DType::F32);
+    std::memcpy(at.data<float>(), a, (size_t)(M * K) * 4);
+    quant::Tensor ct;
+    if (bits == 4) { quant::engines::Q4Engine e; set_codebook(e, cb, 16); ct = e.quant_gemm(at, b_idx, M, N, K); }
+    else { quant::engines::Q8Engine e; set_codebook(e, cb, 256); ct = e.quant_gemm(at, b_idx, M, N, K); }
+    std::memcpy(c, ct.data<float>(), (size_t)(M * N) * 4);
+}
+
+// Q8Encoder::encode + Q8Decoder::decode of one block of at most 256 weights
+void ref_q8codec_block(const float* w, uint32_t n, float* centroids256, uint8_t* idx, float* decoded) {
+    quant::quant8::Q8Encoder enc;
+    quant::quant8::EncodedBlock b = enc.encode(w, n, 0);
+    std::memcpy(centroids256, b.codebook.centroids, 256 * 4);
+    std::memcpy(idx, b.indices.data(), n);
+    quant::quant8::Q8Decoder dec;
+    quant::Tensor t = dec.decode(b);
+    std::memcpy(decoded, t.data<float>(), (size_t)n * 4);
+}
+
+// quant8::quantize_activations on [batch][per] (batch == 1: quantize_tensor), params = (scale, inv_scale, zero_point) per row
+void ref_q8_quantize_rows(const float* src, int64_t batch, int64_t per, int dst_f32, void* dst, float* params3) {
+    quant::Tensor s(quant::Shape{batch, per}, quant::DType::F32);
+    std::memcpy(s.data<float>(), src, (size_t)(batch * per) * 4);
+    quant::Tensor d(quant::Shape{batch, per}, dst_f32 ? quant::DType::F32 : quant::DType::U8);
+    std::vector<quant::quant8::QuantizeParams> ps = quant::quant8::quantize_activations(s, d);
+    for (int64_t b = 0; b < batch; ++b) {
+        params3[3 * b] = ps[(size_t)b].scale;
+        params3[3 * b + 1] = ps[(size_t)b].inv_scale;
+        params3[3 * b + 2] = ps[(size_t)b].zero_point;
+    }
+    std::memcpy(dst, d.data(), (size_t)(batch * per) * (dst_f32 ? 4 : 1));
+}
+
+void ref_q8_dequantize(const void* src, int64_t n, int src_f32, const float* params3, float* out) {
+    quant::Tensor s(quant::Shape{n}, src_f32 ? quant::DType::F32 : quant::DType::U8);
+    std::memcpy(s.data(), src, (size_t)n * (src_f32 ? 4 : 1));
+    quant::quant8::QuantizeParams p;
+    p.scale = params3[0];
+    p.inv_scale = params3[1];
+    p.zero_point = params3[2];
+    quant::Tensor t = quant::quant8::dequantize(s, p);
+    std::memcpy(out, t.data<float>(), (size_t)n * 4);
 }
 
 }  // extern "C"

@@ -47,6 +47,7 @@
 #include <cstdint>
 #include <cstring>
 #include <thread>
+#include <limits>
 #include <vector>
 
 namespace {
@@ -1504,6 +1505,174 @@ void orc_fp24_decode(const uint8_t* packed, float* w, int64_t count) {
         const uint32_t u = ((uint32_t)packed[3 * i] << 24) | ((uint32_t)packed[3 * i + 1] << 16) | ((uint32_t)packed[3 * i + 2] << 8);
         std::memcpy(&w[i], &u, 4);
     }
+}
+
+// ---- in-memory codebook engines: engines::Q4Engine / Q8Engine
+// (src/codec/quant_engines_quant4.cpp:102-150, :226-261; quant_engines_quant8.cpp:92-227; the
+// AVX2 helpers of quant_engines_core.cpp are compiled out: include/quant/simd_math.h:229-231
+// undefines QUANT_HAS_AVX2 before those files test it, so the scalar loops are what runs).
+// Index of the first centroid at the smallest |v - c|; 0 when no distance is below 1e10.
+static int nearest_abs(const float* cb, int count, float v) {
+    int best = 0;
+    float best_dist = 1e10f;
+    for (int j = 0; j < count; ++j) {
+        const float dist = std::fabs(v - cb[j]);
+        if (dist < best_dist) { best_dist = dist; best = j; }
+    }
+    return best;
+}
+
+// 4-bit: scales = (center, half_range) per block from min/max; 8-bit: scale = absmax.
+// One index byte per weight in both engines.
+void orc_engine_quantize_per_block(int bits, const float* cb, const float* data, int64_t n, int64_t bs,
+                                   uint8_t* idx, float* scales) {
+    const int64_t nb = (n + bs - 1) / bs;
+    for (int64_t b = 0; b < nb; ++b) {
+        const int64_t st = b * bs, en = std::min(st + bs, n);
+        if (bits == 4) {
+            float lo = data[st], hi = data[st];
+            for (int64_t i = st + 1; i < en; ++i) { lo = std::min(lo, data[i]); hi = std::max(hi, data[i]); }
+            float half = (hi - lo) * 0.5f;
+            const float center = (hi + lo) * 0.5f;
+            if (half < 1e-10f) half = 1.0f;
+            scales[2 * b] = center;
+            scales[2 * b + 1] = half;
+            for (int64_t i = st; i < en; ++i) idx[i] = (uint8_t)nearest_abs(cb, 16, (data[i] - center) / half);
+        } else {
+            float amax = 0.0f;
+            for (int64_t i = st; i < en; ++i) amax = std::max(amax, std::fabs(data[i]));
+            if (amax < 1e-10f) amax = 1.0f;
+            scales[b] = amax;
+            for (int64_t i = st; i < en; ++i) idx[i] = (uint8_t)nearest_abs(cb, 256, data[i] / amax);
+        }
+    }
+}
+
+void orc_engine_dequantize_per_block(int bits, const float* cb, const uint8_t* idx, const float* scales, int64_t n,
+                                     int64_t bs, float* out) {
+    for (int64_t i = 0; i < n; ++i) {
+        const int64_t b = i / bs;
+        // codebook * half_range + center is one fused multiply-add in the reference's Release build
+        if (bits == 4) out[i] = std::fma(cb[idx[i]], scales[2 * b + 1], scales[2 * b]);
+        else out[i] = cb[idx[i]] * scales[b];
+    }
+}
+
+void orc_engine_quantize_tensor(int bits, const float* cb, const float* data, int64_t n, uint8_t* out) {
+    if (bits == 8) {
+        for (int64_t i = 0; i < n; ++i) out[i] = (uint8_t)nearest_abs(cb, 256, data[i]);
+        return;
+    }
+    for (int64_t i = 0; i < n; i += 2) {
+        const int lo = nearest_abs(cb, 16, data[i]);
+        const int hi = (i + 1 < n) ? nearest_abs(cb, 16, data[i + 1]) : 0;
+        out[i / 2] = (uint8_t)(lo | (hi << 4));
+    }
+}
+
+void orc_engine_dequant_tensor(int bits, const float* cb, const uint8_t* idx, int64_t n, float* out) {
+    for (int64_t i = 0; i < n; ++i)
+        out[i] = bits == 8 ? cb[idx[i]] : cb[(i % 2 == 0) ? (idx[i / 2] & 0xF) : (idx[i / 2] >> 4)];
+}
+
+// C[m][n] = sum_k a[m][k] * codebook[code(k * N + n)], the code matrix is [K][N]; zero activations are skipped
+void orc_engine_quant_gemm(int bits, const float* cb, const float* a, const uint8_t* b_idx, int64_t M, int64_t N,
+                           int64_t K, float* c) {
+    std::fill(c, c + M * N, 0.0f);
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t k = 0; k < K; ++k) {
+            const float av = a[m * K + k];
+            if (av == 0.0f) continue;
+            for (int64_t nn = 0; nn < N; ++nn) {
+                const int64_t flat = k * N + nn;
+                const float w = bits == 8 ? cb[b_idx[flat]]
+                                          : cb[(flat % 2 == 0) ? (b_idx[flat / 2] & 0xF) : (b_idx[flat / 2] >> 4)];
+                c[m * N + nn] = std::fma(av, w, c[m * N + nn]);
+            }
+        }
+}
+
+// quant8::Q8Encoder::encode + Q8Decoder::decode (engines/quant/codec.cpp:19-50) on one block of
+// n <= 256 weights: CodebookQ8::train (src/codec/codebook.cpp:70-129) seeds centroid c with
+// weight c (the rest with weight 0; the random permutation is only drawn for n > 256, from a
+// process-entropy seed), runs at most 20 Lloyd steps on squared distance with double sums in
+// index order, stops when no centroid moves by more than 1e-7; indices are the first nearest
+// centroid of the trained codebook (:166-180).
+int orc_q8codec_block(const float* w, uint32_t n, float* centroids, uint8_t* idx, float* decoded) {
+    if (n == 0 || n > 256) return -1;
+    for (uint32_t c = 0; c < 256; ++c) centroids[c] = c < n ? w[c] : w[0];
+    auto nearest_sq = [&](float v) {
+        float best = std::numeric_limits<float>::max();
+        int arg = 0;
+        for (int c = 0; c < 256; ++c) {
+            const float d = v - centroids[c];
+            const float dist = d * d;
+            if (dist < best) { best = dist; arg = c; }
+        }
+        return arg;
+    };
+    std::vector<uint8_t> assign(n);
+    for (int iter = 0; iter < 20; ++iter) {
+        for (uint32_t i = 0; i < n; ++i) assign[i] = (uint8_t)nearest_sq(w[i]);
+        double sums[256] = {};
+        int counts[256] = {};
+        for (uint32_t i = 0; i < n; ++i) { sums[assign[i]] += w[i]; counts[assign[i]]++; }
+        bool changed = false;
+        for (int c = 0; c < 256; ++c)
+            if (counts[c] > 0) {
+                const float nv = (float)(sums[c] / (double)counts[c]);
+                if (std::fabs(nv - centroids[c]) > 1e-7f) changed = true;
+                centroids[c] = nv;
+            }
+        if (!changed) break;
+    }
+    for (uint32_t i = 0; i < n; ++i) {
+        idx[i] = (uint8_t)nearest_sq(w[i]);
+        decoded[i] = centroids[idx[i]];
+    }
+    return 0;
+}
+
+// quant8::quantize_tensor per row of [batch][per] (quantize_activations), engines/quant/quantize.cpp:14-83.
+// params3 = (scale, inv_scale, zero_point) per row.
+void orc_q8_quantize_rows(const float* src, int64_t batch, int64_t per, int dst_f32, void* dst, float* params3) {
+    for (int64_t b = 0; b < batch; ++b) {
+        const float* x = src + b * per;
+        float lo = 0.0f, hi = 0.0f;
+        if (per > 0) {
+            lo = hi = x[0];
+            for (int64_t i = 1; i < per; ++i) { lo = std::min(lo, x[i]); hi = std::max(hi, x[i]); }
+        }
+        float range = hi - lo;
+        if (range < 1e-12f) range = 1.0f;
+        float inv_scale = range / 255.0f;
+        float scale = 1.0f / inv_scale;
+        float zp = -lo * scale;
+        if (!dst_f32) {
+            uint8_t* d = static_cast<uint8_t*>(dst) + b * per;
+            for (int64_t i = 0; i < per; ++i) {
+                const float q = std::round(std::fma(x[i], scale, zp));  // one fused operation in the Release build
+                d[i] = (uint8_t)std::min(255.0f, std::max(0.0f, q));
+            }
+        } else {
+            float* d = static_cast<float*>(dst) + b * per;
+            float max_abs = std::max(std::fabs(lo), std::fabs(hi));
+            if (max_abs < 1e-12f) max_abs = 1.0f;
+            scale = 127.0f / max_abs;
+            inv_scale = max_abs / 127.0f;
+            zp = 0.0f;
+            for (int64_t i = 0; i < per; ++i) d[i] = x[i] * scale;
+        }
+        params3[3 * b] = scale;
+        params3[3 * b + 1] = inv_scale;
+        params3[3 * b + 2] = zp;
+    }
+}
+
+void orc_q8_dequantize(const void* src, int64_t n, int src_f32, const float* params3, float* out) {
+    for (int64_t i = 0; i < n; ++i)
+        out[i] = src_f32 ? static_cast<const float*>(src)[i] * params3[1]
+                         : ((float)static_cast<const uint8_t*>(src)[i] - params3[2]) * params3[1];
 }
 
 }  // extern "C"

@@ -69,6 +69,15 @@ def _load():
         "tfq_lutn_gemm": (i32, [i32, vp, vp, vp, vp, i32, i32, i32, vp]),
         "tfq_fp24_encode": (i32, [vp, vp, i64, vp]),
         "tfq_fp24_decode": (i32, [vp, vp, i64, vp]),
+        "tfq_engine_quantize_per_block": (i32, [i32, vp, vp, i64, i64, vp, vp, vp]),
+        "tfq_engine_dequantize_per_block": (i32, [i32, vp, vp, vp, i64, i64, vp, vp]),
+        "tfq_engine_quantize_tensor": (i32, [i32, vp, vp, i64, vp, vp]),
+        "tfq_engine_dequant_tensor": (i32, [i32, vp, vp, i64, vp, vp]),
+        "tfq_engine_quant_gemm": (i32, [i32, vp, vp, vp, i64, i64, i64, vp, vp]),
+        "tfq_q8codec_encode": (i32, [vp, i64, i32, vp, vp, vp]),
+        "tfq_q8codec_decode": (i32, [vp, vp, i64, i32, vp, vp]),
+        "tfq_q8_quantize_rows": (i32, [vp, i64, i64, i32, vp, vp, vp]),
+        "tfq_q8_dequantize": (i32, [vp, i64, i32, vp, vp, vp]),
         "tfq_container_open": (vp, [C.c_char_p]),
         "tfq_container_from_memory": (vp, [vp, sz]),
         "tfq_container_close": (None, [vp]),
@@ -403,4 +412,92 @@ def fp24_decode(packed):
     import torch
     out = torch.empty(packed.numel() // 3, dtype=torch.float32, device=packed.device)
     _check(lib().tfq_fp24_decode(packed.data_ptr(), out.data_ptr(), out.numel(), _stream()))
+    return out
+
+
+class CodebookEngine:
+    """engines::Q4Engine (bits=4) / Q8Engine (bits=8) with the given centroids; tensors live on the device."""
+
+    def __init__(self, bits: int, codebook):
+        import numpy as np
+        self.bits = bits
+        self.cb = np.ascontiguousarray(codebook, np.float32)
+        assert self.cb.size == 1 << bits
+
+    def quantize_per_block(self, data, block_size: int):
+        import torch
+        data = data.contiguous().float()
+        n = data.numel()
+        nb = (n + block_size - 1) // block_size
+        idx = torch.empty(n, dtype=torch.uint8, device=data.device)
+        scales = torch.empty(nb * (2 if self.bits == 4 else 1), dtype=torch.float32, device=data.device)
+        _check(lib().tfq_engine_quantize_per_block(self.bits, self.cb.ctypes.data, data.data_ptr(), n, block_size,
+                                                   idx.data_ptr(), scales.data_ptr(), _stream()))
+        return idx, scales
+
+    def dequantize_per_block(self, idx, scales, block_size: int):
+        import torch
+        out = torch.empty(idx.numel(), dtype=torch.float32, device=idx.device)
+        _check(lib().tfq_engine_dequantize_per_block(self.bits, self.cb.ctypes.data, idx.data_ptr(), scales.data_ptr(),
+                                                     idx.numel(), block_size, out.data_ptr(), _stream()))
+        return out
+
+    def quantize_tensor(self, data):
+        import torch
+        data = data.contiguous().float()
+        n = data.numel()
+        out = torch.empty(n if self.bits == 8 else (n + 1) // 2, dtype=torch.uint8, device=data.device)
+        _check(lib().tfq_engine_quantize_tensor(self.bits, self.cb.ctypes.data, data.data_ptr(), n, out.data_ptr(), _stream()))
+        return out
+
+    def dequant_tensor(self, idx, n: int):
+        import torch
+        out = torch.empty(n, dtype=torch.float32, device=idx.device)
+        _check(lib().tfq_engine_dequant_tensor(self.bits, self.cb.ctypes.data, idx.data_ptr(), n, out.data_ptr(), _stream()))
+        return out
+
+    def quant_gemm(self, a, b_idx, M: int, N: int, K: int):
+        import torch
+        a = a.contiguous().float()
+        out = torch.empty((M, N), dtype=torch.float32, device=a.device)
+        _check(lib().tfq_engine_quant_gemm(self.bits, self.cb.ctypes.data, a.data_ptr(), b_idx.data_ptr(), M, N, K,
+                                           out.data_ptr(), _stream()))
+        return out
+
+
+def q8codec_encode(data, block_size: int = 256):
+    """Q8Encoder::encode_tensor: (centroids [blocks][256], indices)."""
+    import torch
+    data = data.contiguous().float()
+    n = data.numel()
+    nb = (n + block_size - 1) // block_size
+    cent = torch.empty((nb, 256), dtype=torch.float32, device=data.device)
+    idx = torch.empty(n, dtype=torch.uint8, device=data.device)
+    _check(lib().tfq_q8codec_encode(data.data_ptr(), n, block_size, cent.data_ptr(), idx.data_ptr(), _stream()))
+    return cent, idx
+
+
+def q8codec_decode(cent, idx, block_size: int = 256):
+    import torch
+    out = torch.empty(idx.numel(), dtype=torch.float32, device=idx.device)
+    _check(lib().tfq_q8codec_decode(cent.data_ptr(), idx.data_ptr(), idx.numel(), block_size, out.data_ptr(), _stream()))
+    return out
+
+
+def q8_quantize_rows(src, dst_f32: bool = False):
+    """quant8::quantize_activations: (quantized [batch][per], params [batch][3] = scale, inv_scale, zero_point)."""
+    import torch
+    src = src.contiguous().float()
+    batch, per = src.shape
+    dst = torch.empty((batch, per), dtype=torch.float32 if dst_f32 else torch.uint8, device=src.device)
+    params = torch.empty((batch, 3), dtype=torch.float32, device=src.device)
+    _check(lib().tfq_q8_quantize_rows(src.data_ptr(), batch, per, int(dst_f32), dst.data_ptr(), params.data_ptr(), _stream()))
+    return dst, params
+
+
+def q8_dequantize(src, params3):
+    import torch
+    out = torch.empty(src.numel(), dtype=torch.float32, device=src.device)
+    _check(lib().tfq_q8_dequantize(src.data_ptr(), src.numel(), int(src.dtype == torch.float32), params3.data_ptr(),
+                                   out.data_ptr(), _stream()))
     return out
