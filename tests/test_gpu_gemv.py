@@ -159,7 +159,9 @@ def test_gemv_other_formats(O, tfq, gpu, fmt, N, K, B, xdt):
         y = W.gemv(torch.from_numpy(x).to(gpu)).cpu().numpy()
         tol = TOL_F32
     ref = O.matmul(fmt, pay, N, K, x)
-    assert rel_err(y, ref) <= min(tol, 1e-4)   # exact decode, fp32 products: only summation order differs
+    # exact weights and (bf16-split) products: only the summation order differs.  The companded 8-bit grid is
+    # multiplied through a line fitted to its 256 levels (7.5e-5 relative per weight), so those get a wider gate.
+    assert rel_err(y, ref) <= (3e-4 if fmt in ("Q_G_8", "Q_8", "Q_8_5", "Q_G_8_5") else 1e-4)
     assert np.array_equal(W.decode().cpu().numpy().reshape(-1).view(np.uint32),
                           O.decode_tensor(fmt, pay, N * K).view(np.uint32))
     W.close()
@@ -178,6 +180,38 @@ def test_config4_lowbit_superblock_shapes(O, tfq, gpu, fmt, bits):
         y = W.gemv(torch.from_numpy(x).to(gpu).bfloat16()).cpu().numpy()
         assert rel_err(y, O.matmul(fmt, pay, N, K, x)) <= 1e-4
     W.close()
+
+
+@pytest.mark.parametrize("fmt", ["Q_G_8", "Q_8", "B32S8"])
+@pytest.mark.parametrize("N,K", [(256, 4096), (48, 14336), (1040, 1024)])
+def test_config2_eight_bit_formats(O, tfq, gpu, fmt, N, K):
+    """8-bit formats at the projection widths, batch 1, 4, 8, 16 with bf16 activations and batch 1, 3 with
+    fp32 activations.  Q_G_8 / Q_8 multiply through the fitted line of the companded grid: the error
+    against the exact-table oracle stays under a third of the fp32 gate."""
+    import torch
+    w = O.rng_normal(42, N * K, 0.02)
+    pay = O.encode_tensor(fmt, w)
+    W = tfq.Weight(fmt, N, K, pay)
+    assert np.array_equal(W.decode().cpu().numpy().reshape(-1).view(np.uint32), O.decode_tensor(fmt, pay, N * K).view(np.uint32))
+    for B in (1, 4, 8, 16):
+        print(f"gemv 8-bit {fmt} N={N} K={K} B={B} bf16", flush=True)
+        x = O.bf16_round(O.rng_normal(43, B * K, 1.0).reshape(B, K))
+        y = W.gemv(torch.from_numpy(x).to(gpu).bfloat16()).cpu().numpy()
+        assert rel_err(y, O.matmul(fmt, pay, N, K, x)) <= 3e-4
+    for B in (1, 3):
+        print(f"gemv 8-bit {fmt} N={N} K={K} B={B} f32", flush=True)
+        x = O.rng_normal(45, B * K, 1.0).reshape(B, K)
+        y = W.gemv(torch.from_numpy(x).to(gpu)).cpu().numpy()
+        assert rel_err(y, O.matmul(fmt, pay, N, K, x)) <= 3e-4
+    # all-positive activations and weights: nothing cancels, the systematic part of the line fit shows in full
+    wp = np.abs(w)
+    payp = O.encode_tensor(fmt, wp)
+    Wp = tfq.Weight(fmt, N, K, payp)
+    x = np.abs(O.bf16_round(O.rng_normal(43, K, 1.0))).reshape(1, K)
+    y = Wp.gemv(torch.from_numpy(x).to(gpu).bfloat16()).cpu().numpy()
+    assert rel_err(y, O.matmul(fmt, payp, N, K, x)) <= 3e-4
+    W.close()
+    Wp.close()
 
 
 @pytest.mark.parametrize("fmt", GEMV_FORMATS)

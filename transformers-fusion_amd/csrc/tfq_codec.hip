@@ -95,8 +95,18 @@ __global__ __launch_bounds__(256) void tile16_kernel(const uint8_t* __restrict__
 #pragma unroll
             for (int j = 0; j < 32; ++j) {
                 uint32_t code;
-                if constexpr (NP == 2) {  // int8 code + 128, split into nibbles
-                    const uint32_t u = (uint32_t)src[32 * g32 + j] ^ 0x80u;
+                if constexpr (NP == 2) {  // 8-bit code as an unsigned byte, split into nibbles
+                    uint32_t u;
+                    if constexpr (sp.codec == Codec::Sym32) {
+                        u = (uint32_t)src[32 * g32 + j] ^ 0x80u;  // int8 code + 128
+                    } else if constexpr (sp.codec == Codec::Grp8) {
+                        u = src[32 * g32 + j];
+                    } else {  // plain Q_8: every 16th weight is a 7-bit slot that decodes as an even index
+                        const uint32_t e = (uint32_t)(32 * g32 + j);
+                        const bool slot = (e & 15u) == 15u;
+                        u = stream_bits(src, BB, 16u + 8u * e - (e >> 4), slot ? 7 : 8);
+                        if (slot) u <<= 1;
+                    }
                     code = plane ? u >> 4 : u & 15u;
                 } else {
                     code = stream_bits(src, code_bytes, (uint32_t)(32 * g32 + j) * sp.bits, sp.bits);
@@ -109,10 +119,15 @@ __global__ __launch_bounds__(256) void tile16_kernel(const uint8_t* __restrict__
         const int64_t row = tile * 16 + n;
         if (row < N) {
             const uint8_t* src = wire + (row * nblocks + blk) * (int64_t)BB;
+            if constexpr (sp.codec == Codec::Lattice) {  // the block's one binary16 scale, for each of the 8 groups
+                const uint32_t s2 = (uint32_t)src[0] | ((uint32_t)src[1] << 8);
+                o[0] = o[1] = o[2] = o[3] = s2 | (s2 << 16);
+            } else {
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const uint32_t off = code_bytes + 16 * part + j;
-                if (off < BB) o[j >> 2] |= (uint32_t)src[off] << (8 * (j & 3));
+                for (int j = 0; j < 16; ++j) {
+                    const uint32_t off = code_bytes + 16 * part + j;
+                    if (off < BB) o[j >> 2] |= (uint32_t)src[off] << (8 * (j & 3));
+                }
             }
         }
     }
@@ -137,7 +152,11 @@ __global__ __launch_bounds__(256) void decode_tiled_kernel(const uint8_t* __rest
     const uint32_t idx = (codes[j >> 1] >> ((j & 1u) * 4)) & 15u;
     const uint8_t* h = unit + 2048 * tiled_planes(FMT) + n * HB;
     float v;
-    if constexpr (sp.codec == Codec::Sym32) {
+    if constexpr (sp.codec == Codec::Grp8 || sp.codec == Codec::Lattice) {
+        const float d = half_bits_to_float((uint32_t)h[2 * g32] | ((uint32_t)h[2 * g32 + 1] << 8));
+        const uint32_t u = idx | (((codes[2048 + (j >> 1)] >> ((j & 1u) * 4)) & 15u) << 4);
+        v = d * __uint_as_float(kComp8Bits[u]);
+    } else if constexpr (sp.codec == Codec::Sym32) {
         const float d = half_bits_to_float((uint32_t)h[2 * g32] | ((uint32_t)h[2 * g32 + 1] << 8));
         int q = (int)idx - 8;
         if constexpr (tiled_planes(FMT) == 2) q = (int)(idx | (((codes[2048 + (j >> 1)] >> ((j & 1u) * 4)) & 15u) << 4)) - 128;
@@ -264,6 +283,8 @@ int launch_tile16(int fmt, const uint8_t* wire, uint8_t* tiled, int64_t N, int64
         case TFQ_Q_G_4: return run_tile16<TFQ_Q_G_4>(wire, tiled, N, K, s);
         case TFQ_B32S4: return run_tile16<TFQ_B32S4>(wire, tiled, N, K, s);
         case TFQ_B32S8: return run_tile16<TFQ_B32S8>(wire, tiled, N, K, s);
+        case TFQ_Q_G_8: return run_tile16<TFQ_Q_G_8>(wire, tiled, N, K, s);
+        case TFQ_Q_8: return run_tile16<TFQ_Q_8>(wire, tiled, N, K, s);
         case TFQ_Q_G_3: return run_tile16<TFQ_Q_G_3>(wire, tiled, N, K, s);
         case TFQ_Q_G_2: return run_tile16<TFQ_Q_G_2>(wire, tiled, N, K, s);
         case TFQ_SB256A3: return run_tile16<TFQ_SB256A3>(wire, tiled, N, K, s);
@@ -286,6 +307,8 @@ int launch_decode_tiled(int fmt, const uint8_t* tiled, int64_t N, int64_t K, flo
         case TFQ_Q_G_4: return run_decode_tiled<TFQ_Q_G_4>(tiled, N, K, out, s);
         case TFQ_B32S4: return run_decode_tiled<TFQ_B32S4>(tiled, N, K, out, s);
         case TFQ_B32S8: return run_decode_tiled<TFQ_B32S8>(tiled, N, K, out, s);
+        case TFQ_Q_G_8: return run_decode_tiled<TFQ_Q_G_8>(tiled, N, K, out, s);
+        case TFQ_Q_8: return run_decode_tiled<TFQ_Q_8>(tiled, N, K, out, s);
         case TFQ_Q_G_3: return run_decode_tiled<TFQ_Q_G_3>(tiled, N, K, out, s);
         case TFQ_Q_G_2: return run_decode_tiled<TFQ_Q_G_2>(tiled, N, K, out, s);
         case TFQ_SB256A3: return run_decode_tiled<TFQ_SB256A3>(tiled, N, K, out, s);

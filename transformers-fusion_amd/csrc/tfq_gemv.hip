@@ -119,8 +119,18 @@ struct Fmt {
     static constexpr int NP = tiled_planes(FMT);  // nibble planes of the codes (2: low and high nibble of code + 128)
     // 4-bit symmetric: 128 + 8; 8-bit symmetric: code = 16 hi + lo - 128 with both nibbles carrying
     // +128, so 16 * 128 + 128 + 128; affine: 128
-    static constexpr float OFFS = FMT == TFQ_B32S4 ? 136.0f : FMT == TFQ_B32S8 ? 2304.0f : 128.0f;
+    // companded 8-bit (Q_G_8, Q_8): code j = 16 hi + lo stands for the level (j - 127.5) * kComp8Gain, so
+    // 16 * 128 + 128 + 127.5
+    static constexpr bool COMP8 = FMT == TFQ_Q_G_8 || FMT == TFQ_Q_8;
+    static constexpr float OFFS = FMT == TFQ_B32S4 ? 136.0f : FMT == TFQ_B32S8 ? 2304.0f : COMP8 ? 2303.5f : 128.0f;
 };
+
+// The 8-bit companded grid is tanh(0.02 t) / tanh(0.02), t = (j - 127.5) / 127.5
+// (comp8_table, src/codec/block_codec.cpp:224-237).  With so flat a compander the level over t is
+// a + b t^2 with a - 1 = 1.48e-4 and a + b = 1, so one slope c = 1.0000742 reproduces every level
+// to 7.5e-5 relative; the matmul uses that line (codes as integers on the matrix cores, the slope
+// in the scale), which costs under a tenth of the 1e-3 output tolerance.  Decode keeps the table.
+constexpr float kComp8Gain = 1.0000742443371564f / 127.5f;
 
 // `count` bits at bit `pos` (both compile-time after unrolling) of the little-endian bit string w[0], w[1], ...
 __device__ __forceinline__ uint32_t field(const uint32_t* w, int pos, int count) {
@@ -142,12 +152,12 @@ template <int FMT>
 __device__ __forceinline__ float apply_groups(const uint4* hv, int khalf, f32x4_t DA, f32x4_t DB, const float* X) {
     constexpr Spec sp = spec_of(FMT);
     float res = 0.0f;
-    if constexpr (FMT == TFQ_B32S4 || FMT == TFQ_B32S8) {
+    if constexpr (FMT == TFQ_B32S4 || Fmt<FMT>::NP == 2) {
         // header: eight binary16 scales, four per k-step; the conversion rides in the multiply-add
         // (v_fma_mix_f32 reads either half of a dword as binary16)
         const f16x2_t s01 = __builtin_bit_cast(f16x2_t, khalf ? hv[0].z : hv[0].x);
         const f16x2_t s23 = __builtin_bit_cast(f16x2_t, khalf ? hv[0].w : hv[0].y);
-        if constexpr (FMT == TFQ_B32S8) {  // DB holds the high-nibble plane's dot products
+        if constexpr (Fmt<FMT>::NP == 2) {  // DB holds the high-nibble plane's dot products
 #pragma unroll
             for (int r = 0; r < 4; ++r) DA[r] = __builtin_fmaf(16.0f, DB[r], DA[r]);
         }
@@ -155,6 +165,7 @@ __device__ __forceinline__ float apply_groups(const uint4* hv, int khalf, f32x4_
         res = __builtin_fmaf((float)s01.y, DA[1], res);
         res = __builtin_fmaf((float)s23.x, DA[2], res);
         res = __builtin_fmaf((float)s23.y, DA[3], res);
+        if constexpr (Fmt<FMT>::COMP8) res *= kComp8Gain;
     } else {
         // header: NG scale codes of scb bits | NG offset codes of mb bits (biased) | binary16 d | binary16 dm
         constexpr int NG = Fmt<FMT>::NG, PER = NG / 2;  // groups per k-step
@@ -477,7 +488,7 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
 
 // Formats whose kernel is also built with several slot sets per pass (up to 16 bf16 rows).
 template <int FMT>
-constexpr bool kWide = FMT == TFQ_B32S4 || FMT == TFQ_B32S8 || FMT == TFQ_Q_G_4;
+constexpr bool kWide = FMT == TFQ_B32S4 || FMT == TFQ_B32S8 || FMT == TFQ_Q_G_4 || FMT == TFQ_Q_G_8 || FMT == TFQ_Q_8;
 
 struct GemvPlan {
     int NW, T, sets;
@@ -632,6 +643,8 @@ int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int 
         case TFQ_Q_G_4: return gemv4_batched<TFQ_Q_G_4>(a, x, x_dtype, B, y_dtype, s);
         case TFQ_B32S4: return gemv4_batched<TFQ_B32S4>(a, x, x_dtype, B, y_dtype, s);
         case TFQ_B32S8: return gemv4_batched<TFQ_B32S8>(a, x, x_dtype, B, y_dtype, s);
+        case TFQ_Q_G_8: return gemv4_batched<TFQ_Q_G_8>(a, x, x_dtype, B, y_dtype, s);
+        case TFQ_Q_8: return gemv4_batched<TFQ_Q_8>(a, x, x_dtype, B, y_dtype, s);
         case TFQ_Q_G_3: return gemv4_batched<TFQ_Q_G_3>(a, x, x_dtype, B, y_dtype, s);
         case TFQ_Q_G_2: return gemv4_batched<TFQ_Q_G_2>(a, x, x_dtype, B, y_dtype, s);
         case TFQ_SB256A3: return gemv4_batched<TFQ_SB256A3>(a, x, x_dtype, B, y_dtype, s);

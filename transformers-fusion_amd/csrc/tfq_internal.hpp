@@ -112,14 +112,19 @@ namespace tfq {
 __host__ __device__ constexpr int tiled_header_bytes(int fmt) {
     switch (fmt) {
         case TFQ_Q_G_4: case TFQ_Q_4_5: case TFQ_Q_G_4_5: case TFQ_B32S4: case TFQ_B32S8:
-        case TFQ_Q_G_3: case TFQ_Q_3_5: case TFQ_Q_G_3_5: return 16;
+        case TFQ_Q_G_3: case TFQ_Q_3_5: case TFQ_Q_G_3_5:
+        case TFQ_Q_G_8: case TFQ_Q_8_5: case TFQ_Q_G_8_5: case TFQ_Q_8: return 16;
         case TFQ_Q_G_2: case TFQ_SB256A3: case TFQ_SB256A2: return 32;
         default: return 0;
     }
 }
 // nibble planes of the code area: the 8-bit symmetric format is stored as two, the low and the
 // high nibble of (code + 128), each laid out like a 4-bit format's codes
-__host__ __device__ constexpr int tiled_planes(int fmt) { return fmt == TFQ_B32S8 ? 2 : 1; }
+// (the companded 8-bit formats store their code 0..255 the same way; plain Q_8 has its slot codes
+// widened to 8 bits and its one scale repeated for the eight groups)
+__host__ __device__ constexpr int tiled_planes(int fmt) {
+    return fmt == TFQ_B32S8 || fmt == TFQ_Q_G_8 || fmt == TFQ_Q_8_5 || fmt == TFQ_Q_G_8_5 || fmt == TFQ_Q_8 ? 2 : 1;
+}
 __host__ __device__ constexpr int tiled_unit_bytes(int fmt) { return 2048 * tiled_planes(fmt) + 16 * tiled_header_bytes(fmt); }
 }  // namespace tfq
 
