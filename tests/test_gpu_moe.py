@@ -74,6 +74,29 @@ def test_moe_ffn_small(O, tfq, gpu, fmt, xdt, mid_bf16, tol):
         wl.close()
 
 
+@pytest.mark.parametrize("fmt", ["B32S4", "Q_G_8", "Q_G_3"])
+def test_moe_ffn_skewed_routing(O, tfq, gpu, fmt):
+    """One expert takes most tokens (more rows than one pass of the GEMV carries, so its rows are cut into
+    chunks), some experts take none; formats with the grouped launch and one without it."""
+    import torch
+    E, Ktop, T, D, F = 6, 2, 24, 512, 1024
+    gate, up, down, hg, hu, hd = _experts(O, tfq, fmt, E, D, F, 700)
+    logits = O.rng_normal(46, T * E, 1.0).reshape(T, E)
+    logits[:, 2] += 6.0      # every token picks expert 2 first
+    logits[:, 4] -= 20.0     # nobody picks expert 4
+    _, idx, w = O.softmax_topk(logits, Ktop)
+    assert (idx == 2).sum() == T and (idx == 4).sum() == 0
+    x = O.bf16_round(O.rng_normal(43, T * D, 1.0).reshape(T, D))
+    ref = O.moe_ffn(fmt, hg, hu, hd, D, F, idx, w, x, mid_bf16=True)
+    y = tfq.moe_ffn(gate, up, down, idx, w, torch.from_numpy(x).to(gpu).bfloat16(), mid_dtype=torch.bfloat16).cpu().numpy()
+    assert rel_err(y, ref) <= 1e-2
+    ref32 = O.moe_ffn(fmt, hg, hu, hd, D, F, idx, w, x, mid_bf16=False)
+    y32 = tfq.moe_ffn(gate, up, down, idx, w, torch.from_numpy(x).to(gpu), mid_dtype=torch.float32).cpu().numpy()
+    assert rel_err(y32, ref32) <= 1e-3
+    for wl in gate + up + down:
+        wl.close()
+
+
 def test_moe_single_token_equals_plain_mlp(O, tfq, gpu):
     """One token, one expert, weight 1: the MoE path reduces to the SwiGLU MLP step."""
     import torch

@@ -105,6 +105,20 @@ struct GemvKernArgs {
     int K, y_bf16, nslot, tiles_per_wg, cols_base, cols_rem;
 };
 
+// Grouped launch: many independent problems (matrix, activation rows, output) of one format and
+// K in one grid, e.g. all experts of a mixture layer.  The kernel then receives a device table of
+// problems and a map workgroup -> problem instead of the flattened arguments (W0 = table,
+// W1 = map); both reads are uniform per workgroup.
+struct GemvProb {
+    const uint8_t* W;
+    void* y;
+    const void* x;
+    int nrows;
+    int nslot;
+    int wg_first;  // first workgroup of this problem
+    int pad;
+};
+
 // Per-format constants of the kernel.
 //   HB   header bytes per row and block in the Tiled16 layout (16 or 32)
 //   GS   weights per scale group (32 or 16)
@@ -204,24 +218,38 @@ __device__ unsigned long long g_trace[1024 * 16 * 8];
 // chooses WD <= the number of units of a full wavefront (a short one re-reads a unit it never uses).
 // SETS = sets of four activation slots that ride in one pass (1, 2 or 4: up to 16 bf16 rows).  More
 // than one set keeps that many A fragments in registers, which fits at 8 wavefronts per workgroup.
-template <int FMT, bool XF32, int WD, int SETS = 1>
-__global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin) {
+template <int FMT, bool XF32, int WD, int SETS = 1, bool GROUPED = false>
+__global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin_arg) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
     constexpr int UB = tiled_unit_bytes(FMT);  // bytes of a unit
     constexpr int NC = 2 * F::NP;              // 1 KB code pieces of a unit: [plane][k-step]
     constexpr int NG = F::NG, PER = NG / 2;  // scale groups per block / per k-step
-    const int K = args.K, nslot = args.nslot, T = args.tiles_per_wg;
+    const int K = args.K, T = args.tiles_per_wg;
     const int cols_base = args.cols_base, cols_rem = args.cols_rem;
     const bool y_bf16 = args.y_bf16 != 0;
 
-    // ---- this workgroup's matrix, selected once with compares
+    // ---- this workgroup's matrix, selected once with compares (or read from the problem table)
     const int bid = blockIdx.x;
-    const int m = (bid >= args.g0) + (bid >= args.g1) + (bid >= args.g2);
-    const int wg_first = m == 0 ? 0 : m == 1 ? args.g0 : m == 2 ? args.g1 : args.g2;
-    const uint8_t* Wm = m == 0 ? args.W0 : m == 1 ? args.W1 : m == 2 ? args.W2 : args.W3;
-    void* const ym = m == 0 ? args.y0 : m == 1 ? args.y1 : m == 2 ? args.y2 : args.y3;
-    const int nrm = m == 0 ? args.nr0 : m == 1 ? args.nr1 : m == 2 ? args.nr2 : args.nr3;
+    int wg_first, nrm, nslot;
+    const uint8_t* Wm;
+    void* ym;
+    const void* xin;
+    if constexpr (GROUPED) {
+        const GemvProb* table = reinterpret_cast<const GemvProb*>(args.W0);
+        const int* wg_map = reinterpret_cast<const int*>(args.W1);
+        const GemvProb pr = table[wg_map[bid]];
+        wg_first = pr.wg_first; nrm = pr.nrows; nslot = pr.nslot;
+        Wm = pr.W; ym = pr.y; xin = pr.x;
+    } else {
+        const int m = (bid >= args.g0) + (bid >= args.g1) + (bid >= args.g2);
+        wg_first = m == 0 ? 0 : m == 1 ? args.g0 : m == 2 ? args.g1 : args.g2;
+        Wm = m == 0 ? args.W0 : m == 1 ? args.W1 : m == 2 ? args.W2 : args.W3;
+        ym = m == 0 ? args.y0 : m == 1 ? args.y1 : m == 2 ? args.y2 : args.y3;
+        nrm = m == 0 ? args.nr0 : m == 1 ? args.nr1 : m == 2 ? args.nr2 : args.nr3;
+        nslot = args.nslot;
+        xin = xin_arg;
+    }
 
     const int nblocks = K >> 8;
     const int NW = blockDim.x >> 6;
@@ -610,7 +638,106 @@ int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t 
     return TFQ_OK;
 }
 
+// ---- grouped launch
+template <int FMT>
+int plan_grouped(int K, bool x_f32, const int* nrows, const int* nrows_x, int nprob, GemvGroupPlan* gp) {
+    const int nblocks = K >> 8;
+    int max_rows = 1;
+    for (int i = 0; i < nprob; ++i) max_rows = nrows_x[i] > max_rows ? nrows_x[i] : max_rows;
+    const int nslot = x_f32 ? 2 * max_rows : max_rows;
+    if (nslot > 16 || (nslot > 4 && (x_f32 || !kWide<FMT>))) return fail(TFQ_ERR_SHAPE, "gemv group: too many activation rows in one problem");
+    GemvArgs a{};
+    a.K = K;
+    a.nmat = 1;
+    a.nrows[0] = nrows[0];
+    a.ntiles = (nrows[0] + 15) / 16;
+    GemvPlan p = plan_gemv4<FMT>(a, nslot);
+    if (p.lds == 0) return fail(TFQ_ERR_SHAPE, "gemv group: the activation rows of one problem do not fit in LDS");
+    // tiles per workgroup: about 256 KB of packed weights each, within what LDS leaves for the partial sums
+    const size_t per_tile = (size_t)p.NW * p.sets * 256, x_bytes = p.lds - (size_t)p.T * per_tile;
+    int T = (int)((256 * 1024 + (size_t)nblocks * tiled_unit_bytes(FMT) - 1) / ((size_t)nblocks * tiled_unit_bytes(FMT)));
+    while (T > 1 && x_bytes + (size_t)T * per_tile > 160 * 1024) --T;
+    gp->NW = p.NW; gp->T = T; gp->sets = p.sets; gp->lds = x_bytes + (size_t)T * per_tile;
+    gp->x_f32 = x_f32;
+    gp->K = K;
+    int grid = 0;
+    for (int i = 0; i < nprob; ++i) grid += ((nrows[i] + 15) / 16 + T - 1) / T;
+    gp->grid = grid;
+    return TFQ_OK;
+}
+
+template <int FMT>
+int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_bf16, hipStream_t s) {
+    const int nblocks = gp.K >> 8;
+    GemvKernArgs k{};
+    k.W0 = static_cast<const uint8_t*>(d_table);
+    k.W1 = reinterpret_cast<const uint8_t*>(d_map);
+    k.K = gp.K; k.y_bf16 = y_bf16; k.nslot = 0; k.tiles_per_wg = gp.T;
+    k.cols_base = nblocks / gp.NW; k.cols_rem = nblocks % gp.NW;
+    using Kernel = void (*)(GemvKernArgs, const void*);
+    constexpr int WDG = 2;  // two unit fetches in flight: every format's kernel holds that many without spilling
+    Kernel kern = gp.x_f32 ? gemv4_kernel<FMT, true, WDG, 1, true> : gemv4_kernel<FMT, false, WDG, 1, true>;
+    int slot = gp.x_f32 ? 1 : 0;
+    if constexpr (kWide<FMT>) {
+        if (gp.sets == 2) { kern = gemv4_kernel<FMT, false, 2, 2, true>; slot = 2; }
+        if (gp.sets == 4) { kern = gemv4_kernel<FMT, false, 1, 4, true>; slot = 3; }
+    }
+    static bool lds_limit_raised[4] = {};
+    if (!lds_limit_raised[slot]) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
+        lds_limit_raised[slot] = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(gp.grid), dim3(64 * gp.NW), gp.lds, s, k, nullptr);
+    return hip_fail(hipGetLastError(), "gemv group launch");
+}
+
 }  // namespace
+
+bool gemv_grouped_supported(int fmt) {
+    switch (canonical(fmt)) {
+        case TFQ_Q_G_4: case TFQ_B32S4: case TFQ_B32S8: case TFQ_Q_G_8: return true;
+        default: return false;
+    }
+}
+
+int plan_gemv_grouped(int fmt, int K, bool x_f32, const int* nrows, const int* nrows_x, int nprob, GemvGroupPlan* gp) {
+    if (nprob <= 0) return fail(TFQ_ERR_ARG, "gemv group: no problems");
+    switch (canonical(fmt)) {
+        case TFQ_Q_G_4: return plan_grouped<TFQ_Q_G_4>(K, x_f32, nrows, nrows_x, nprob, gp);
+        case TFQ_B32S4: return plan_grouped<TFQ_B32S4>(K, x_f32, nrows, nrows_x, nprob, gp);
+        case TFQ_B32S8: return plan_grouped<TFQ_B32S8>(K, x_f32, nrows, nrows_x, nprob, gp);
+        case TFQ_Q_G_8: return plan_grouped<TFQ_Q_G_8>(K, x_f32, nrows, nrows_x, nprob, gp);
+        default: return fail(TFQ_ERR_FORMAT, "gemv group: no grouped kernel for this format");
+    }
+}
+
+// Fills the host images of the problem table (nprob entries of gemv_group_entry_bytes() each) and of the
+// workgroup map (gp.grid ints).
+void fill_gemv_group(const GemvGroupPlan& gp, const tfq_weight* const* ws, const void* const* xs, void* const* ys,
+                     const int* nrows_x, int nprob, void* table_host, int* map_host) {
+    GemvProb* t = static_cast<GemvProb*>(table_host);
+    int wg = 0;
+    for (int i = 0; i < nprob; ++i) {
+        const int n = ((int)((ws[i]->N + 15) / 16) + gp.T - 1) / gp.T;
+        t[i] = GemvProb{ws[i]->dev, ys[i], xs[i], (int)ws[i]->N, gp.x_f32 ? 2 * nrows_x[i] : nrows_x[i], wg, 0};
+        for (int j = 0; j < n; ++j) map_host[wg + j] = i;
+        wg += n;
+    }
+}
+
+size_t gemv_group_entry_bytes() { return sizeof(GemvProb); }
+
+int launch_gemv_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s) {
+    const int yb = y_dtype == TFQ_BF16;
+    switch (canonical(fmt)) {
+        case TFQ_Q_G_4: return run_grouped<TFQ_Q_G_4>(gp, d_table, d_map, yb, s);
+        case TFQ_B32S4: return run_grouped<TFQ_B32S4>(gp, d_table, d_map, yb, s);
+        case TFQ_B32S8: return run_grouped<TFQ_B32S8>(gp, d_table, d_map, yb, s);
+        case TFQ_Q_G_8: return run_grouped<TFQ_Q_G_8>(gp, d_table, d_map, yb, s);
+        default: return fail(TFQ_ERR_FORMAT, "gemv group: no grouped kernel for this format");
+    }
+}
 
 int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
                       void* const* ys, int y_dtype, hipStream_t s) {

@@ -168,6 +168,20 @@ int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int 
                       void* const* ys, int y_dtype, hipStream_t s);
 int launch_gemv_generic(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype,
                         hipStream_t s);
+// Grouped GEMV: many (matrix, activation rows, output) problems of one format and K in one launch.
+// plan -> fill the host images of the problem table and the workgroup map -> copy both to the
+// device -> launch.  nrows[i] = weight rows of problem i, nrows_x[i] = its activation rows.
+struct GemvGroupPlan {
+    int NW, T, sets, grid, K;
+    bool x_f32;
+    size_t lds;
+};
+bool gemv_grouped_supported(int fmt);
+int plan_gemv_grouped(int fmt, int K, bool x_f32, const int* nrows, const int* nrows_x, int nprob, GemvGroupPlan* gp);
+size_t gemv_group_entry_bytes();
+void fill_gemv_group(const GemvGroupPlan& gp, const tfq_weight* const* ws, const void* const* xs, void* const* ys,
+                     const int* nrows_x, int nprob, void* table_host, int* map_host);
+int launch_gemv_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s);
 size_t moe_workspace_bytes(int T, int Ktop, int64_t D, int64_t F);
 int launch_moe_route(const float* logits, int T, int E, int k, float* probs, int* idx, float* wts, hipStream_t s);
 int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E,

@@ -14,7 +14,10 @@
 // down GEMVs run one after the other on their slices of those buffers, SwiGLU is one
 // launch over all pairs, and one launch combines: the lane that owns out[t][d] adds its
 // token's pairs in ascending expert order, which is the reference's accumulation order
-// (expert-major), without atomics, so results are deterministic.
+// (expert-major), without atomics, so results are deterministic.  For the formats with a
+// grouped GEMV kernel all experts' gate/up products are ONE launch and all down products
+// another (a table of problems, one per expert, matrix and chunk of activation rows), so
+// the weight stream of the whole layer is not interrupted by launch boundaries.
 //
 // Routing (softmax_with_topk, src/model/moe_core.cpp:98-149): max-subtracted
 // softmax in fp32, the k largest probabilities in descending order (lowest
@@ -23,6 +26,7 @@
 
 #include "tfq_internal.hpp"
 
+#include <algorithm>
 #include <vector>
 
 namespace tfq {
@@ -117,7 +121,8 @@ struct Workspace {
     float* u;      // [P][F]
     uint8_t* h;    // [P][F] mid activations
     float* o;      // [P][D]
-    int* lists;    // rows[P] | tok_pairs[P] | tok_first[T + 1] | weights[P] (float bits)
+    int* lists;    // rows[P] | tok_pairs[P] | tok_first[T + 1] | weights[P] (float bits) | grouped-launch tables
+    size_t list_bytes;
     size_t total;
 };
 
@@ -131,7 +136,11 @@ Workspace carve(void* base, int T, int Ktop, int64_t D, int64_t F) {
     ws.u = (float*)take(P * F * 4);
     ws.h = take(P * F * 4);
     ws.o = (float*)take(P * D * 4);
-    ws.lists = (int*)take((3 * P + (size_t)T + 1) * 4);
+    // grouped launches: at most 2P gate/up problems and P down problems, one map entry per workgroup
+    // (at most one per 16-row tile of a problem)
+    ws.list_bytes = (3 * P + (size_t)T + 1) * 4 + 64 + 3 * P * gemv_group_entry_bytes() +
+                    (2 * P * (size_t)((F + 15) / 16) + P * (size_t)((D + 15) / 16)) * 4;
+    ws.lists = (int*)take(ws.list_bytes);
     ws.total = off;
     return ws;
 }
@@ -178,7 +187,68 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
         first[e + 1] = (int)rows.size();
     }
     const int P = (int)rows.size();  // <= T * Ktop; slots naming an expert outside 0..E-1 are dropped
-    std::vector<int> lists((size_t)3 * P + T + 1);
+    const size_t he = mid_dtype == TFQ_BF16 ? 2 : 4;
+
+    // Grouped launches: problems in expert order, an expert's rows cut into chunks of `cap` rows
+    // (what one pass of the kernel carries at this K)
+    const bool grouped = P > 0 && gemv_grouped_supported(gate[0]->fmt) && gemv_grouped_supported(down[0]->fmt) &&
+                         canonical(gate[0]->fmt) == canonical(up[0]->fmt);
+    GemvGroupPlan planA{}, planB{};
+    std::vector<const tfq_weight*> wA, wB;
+    std::vector<const void*> xA, xB;
+    std::vector<void*> yA, yB;
+    std::vector<int> nA, nB, rA, rB;
+    if (grouped) {
+        int max_nt = 1;
+        for (int e = 0; e < E; ++e) max_nt = std::max(max_nt, first[e + 1] - first[e]);
+        auto chunk_cap = [&](int fmt, int K, bool f32, int nrows) {
+            if (f32) return 2;
+            for (int cap = 16; cap > 4; cap >>= 1) {
+                if (cap / 2 >= max_nt) continue;  // a smaller pass already holds every expert's rows
+                GemvGroupPlan probe{};
+                const int one = cap;
+                if (plan_gemv_grouped(fmt, K, false, &nrows, &one, 1, &probe) == TFQ_OK) return cap;
+            }
+            return 4;
+        };
+        const int capA = chunk_cap(gate[0]->fmt, (int)D, x_dtype == TFQ_F32, (int)F);
+        const int capB = chunk_cap(down[0]->fmt, (int)F, mid_dtype == TFQ_F32, (int)D);
+        for (int e = 0; e < E; ++e) {
+            const int p0 = first[e], nt = first[e + 1] - first[e];
+            for (int b0 = 0; b0 < nt; b0 += capA) {
+                const int nb = std::min(capA, nt - b0);
+                for (int m = 0; m < 2; ++m) {
+                    wA.push_back(m ? up[e] : gate[e]);
+                    xA.push_back(ws.xe + (size_t)(p0 + b0) * D * xe_bytes);
+                    yA.push_back((m ? ws.u : ws.g) + (size_t)(p0 + b0) * F);
+                    nA.push_back((int)F);
+                    rA.push_back(nb);
+                }
+            }
+            for (int b0 = 0; b0 < nt; b0 += capB) {
+                const int nb = std::min(capB, nt - b0);
+                wB.push_back(down[e]);
+                xB.push_back(ws.h + (size_t)(p0 + b0) * F * he);
+                yB.push_back(ws.o + (size_t)(p0 + b0) * D);
+                nB.push_back((int)D);
+                rB.push_back(nb);
+            }
+        }
+        if (int rc = plan_gemv_grouped(gate[0]->fmt, (int)D, x_dtype == TFQ_F32, nA.data(), rA.data(), (int)nA.size(), &planA)) return rc;
+        if (int rc = plan_gemv_grouped(down[0]->fmt, (int)F, mid_dtype == TFQ_F32, nB.data(), rB.data(), (int)nB.size(), &planB)) return rc;
+    }
+    const size_t eb = gemv_group_entry_bytes();
+    const size_t base_ints = ((size_t)3 * P + T + 1 + 1) & ~(size_t)1;  // tables start 8-byte aligned
+    const size_t tabA = base_ints * 4, tabB = tabA + wA.size() * eb;
+    const size_t mapA = tabB + wB.size() * eb, mapB = mapA + (size_t)planA.grid * 4;
+    const size_t list_bytes = grouped ? mapB + (size_t)planB.grid * 4 : base_ints * 4;
+    if (list_bytes > ws.list_bytes) return fail(TFQ_ERR_SHAPE, "moe: routing tables exceed the workspace");
+    std::vector<int> lists(list_bytes / 4 + 2);
+    if (grouped) {
+        uint8_t* lb = reinterpret_cast<uint8_t*>(lists.data());
+        fill_gemv_group(planA, wA.data(), xA.data(), yA.data(), rA.data(), (int)wA.size(), lb + tabA, reinterpret_cast<int*>(lb + mapA));
+        fill_gemv_group(planB, wB.data(), xB.data(), yB.data(), rB.data(), (int)wB.size(), lb + tabB, reinterpret_cast<int*>(lb + mapB));
+    }
     int* h_rows = lists.data();
     int* h_pairs = h_rows + P;
     int* h_first = h_pairs + P;
@@ -193,7 +263,7 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
     int* d_first = d_pairs + P;
     float* d_w = reinterpret_cast<float*>(d_first + T + 1);
     // The source is pageable host memory: wait for the copy before the vectors go out of scope.
-    TFQ_HIP(hipMemcpyAsync(ws.lists, lists.data(), lists.size() * 4, hipMemcpyHostToDevice, s));
+    TFQ_HIP(hipMemcpyAsync(ws.lists, lists.data(), list_bytes, hipMemcpyHostToDevice, s));
     TFQ_HIP(hipStreamSynchronize(s));
 
     if (P) {
@@ -202,7 +272,11 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
         hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)((ng + 255) / 256)), dim3(256), 0, s,
                            (const uint4*)x, (uint4*)ws.xe, d_rows, P, row_u4);
     }
-    for (int e = 0; e < E; ++e) {
+    const uint8_t* d_lists = reinterpret_cast<const uint8_t*>(ws.lists);
+    if (grouped) {
+        if (int rc = launch_gemv_grouped(gate[0]->fmt, planA, d_lists + tabA, reinterpret_cast<const int*>(d_lists + mapA), TFQ_F32, s)) return rc;
+    }
+    for (int e = 0; e < E && !grouped; ++e) {
         const int p0 = first[e], nt = first[e + 1] - first[e];
         for (int b0 = 0; b0 < nt; b0 += 16) {  // the GEMV entry takes up to 16 rows
             const int nb = nt - b0 < 16 ? nt - b0 : 16;
@@ -218,8 +292,10 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
         else
             hipLaunchKernelGGL(silu_mul_kernel<false>, dim3((unsigned)((nh + 255) / 256)), dim3(256), 0, s, ws.g, ws.u, (void*)ws.h, nh);
     }
-    const size_t he = mid_dtype == TFQ_BF16 ? 2 : 4;
-    for (int e = 0; e < E; ++e) {
+    if (grouped) {
+        if (int rc = launch_gemv_grouped(down[0]->fmt, planB, d_lists + tabB, reinterpret_cast<const int*>(d_lists + mapB), TFQ_F32, s)) return rc;
+    }
+    for (int e = 0; e < E && !grouped; ++e) {
         const int p0 = first[e], nt = first[e + 1] - first[e];
         for (int b0 = 0; b0 < nt; b0 += 16) {
             const int nb = nt - b0 < 16 ? nt - b0 : 16;
