@@ -20,6 +20,19 @@ __global__ __launch_bounds__(256) void decode_kernel(const uint8_t* __restrict__
     out[blk * 256 + threadIdx.x] = decode_weight<FMT>(src + blk * (int64_t)sp.block_bytes, threadIdx.x);
 }
 
+// Four blocks per workgroup, a wavefront per block, four weights per lane from two aligned dword reads.
+template <int FMT>
+__global__ __launch_bounds__(256) void decode_quad_kernel(const uint8_t* __restrict__ src, float* __restrict__ out,
+                                                          int64_t nblocks) {
+    constexpr Spec sp = spec_of(FMT);
+    const int64_t blk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (blk >= nblocks) return;
+    const uint32_t lane = threadIdx.x & 63;
+    float v[4];
+    decode_quad<FMT>(src + blk * (int64_t)sp.block_bytes, lane, v, src + nblocks * (int64_t)sp.block_bytes);
+    *reinterpret_cast<float4*>(out + blk * 256 + 4 * lane) = float4{v[0], v[1], v[2], v[3]};
+}
+
 __global__ __launch_bounds__(256) void decode_short_kernel(BlockLayout L, const uint8_t* __restrict__ src,
                                                            float* __restrict__ out) {
     if ((int)threadIdx.x < L.n) out[threadIdx.x] = decode_weight_short(L, src, threadIdx.x);
@@ -180,6 +193,14 @@ __global__ __launch_bounds__(256) void decode_tiled_kernel(const uint8_t* __rest
 
 template <int FMT>
 int run_decode(const uint8_t* src, int64_t nblocks, float* out, hipStream_t s) {
+    if constexpr (kHasQuad<FMT>) {
+        // dword reads need a 4-byte aligned payload and a 16-byte aligned destination; anything else
+        // takes the byte-wise kernel
+        if ((reinterpret_cast<uintptr_t>(src) & 3u) == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0) {
+            hipLaunchKernelGGL(decode_quad_kernel<FMT>, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, s, src, out, nblocks);
+            return hip_fail(hipGetLastError(), "decode launch");
+        }
+    }
     hipLaunchKernelGGL(decode_kernel<FMT>, dim3((unsigned)nblocks), dim3(256), 0, s, src, out);
     return hip_fail(hipGetLastError(), "decode launch");
 }

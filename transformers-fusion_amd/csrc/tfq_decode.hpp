@@ -114,6 +114,66 @@ __device__ __forceinline__ float decode_weight(const uint8_t* __restrict__ p, ui
     return v;
 }
 
+// ---- four weights per lane from aligned dword reads
+// Formats that stay in wire order have their codes in one LSB-first stream; the four weights
+// 4 l .. 4 l + 3 of lane l are at most 32 consecutive bits of it.  window32() fetches them with two
+// aligned dword loads instead of one byte load per byte touched; `limit` is the end of the payload
+// buffer (a dword that would straddle it is assembled from what lies inside).  Payload buffers
+// must be 4-byte aligned.
+__device__ __forceinline__ uint32_t safe_dword(const uint8_t* q, const uint8_t* limit) {
+    if (q + 4 <= limit) return *reinterpret_cast<const uint32_t*>(q);
+    return q + 2 <= limit ? (uint32_t)*reinterpret_cast<const uint16_t*>(q) : 0u;
+}
+__device__ __forceinline__ uint32_t window32(const uint8_t* p, uint32_t pos, const uint8_t* limit) {
+    const uint8_t* a = p + (pos >> 3);
+    const uint8_t* a4 = reinterpret_cast<const uint8_t*>(reinterpret_cast<uintptr_t>(a) & ~(uintptr_t)3);
+    const uint32_t sh = (uint32_t)(reinterpret_cast<uintptr_t>(a) & 3u) * 8u + (pos & 7u);
+    const uint64_t v = (uint64_t)safe_dword(a4, limit) | ((uint64_t)safe_dword(a4 + 4, limit) << 32);
+    return (uint32_t)(v >> sh);
+}
+__device__ __forceinline__ uint32_t half_at(const uint8_t* p) { return *reinterpret_cast<const uint16_t*>(p); }
+
+template <int FMT>
+constexpr bool kHasQuad = spec_of(FMT).codec == Codec::Raw32 || spec_of(FMT).codec == Codec::Lattice ||
+                          spec_of(FMT).codec == Codec::Grp16 || spec_of(FMT).codec == Codec::Q6K;
+
+// v[t] = decode_weight<FMT>(p, 4 * lane + t), the same arithmetic on the same operands
+template <int FMT>
+__device__ __forceinline__ void decode_quad(const uint8_t* __restrict__ p, uint32_t lane, float (&v)[4],
+                                            const uint8_t* limit) {
+    constexpr Spec sp = spec_of(FMT);
+    constexpr uint32_t bits = sp.bits;
+    if constexpr (sp.codec == Codec::Raw32) {
+        const uint4 q = *reinterpret_cast<const uint4*>(p + 16 * lane);
+        v[0] = __uint_as_float(q.x); v[1] = __uint_as_float(q.y); v[2] = __uint_as_float(q.z); v[3] = __uint_as_float(q.w);
+    } else if constexpr (sp.codec == Codec::Lattice) {
+        const float scale = half_bits_to_float(half_at(p));
+        const uint32_t i0 = 4 * lane;
+        const uint32_t w = window32(p, 16u + bits * i0 - (i0 >> 4), limit);
+#pragma unroll
+        for (uint32_t t = 0; t < 4; ++t) {
+            const bool slot = t == 3 && (lane & 3u) == 3u;  // weight i is a slot when i % 16 == 15
+            uint32_t idx = (w >> (bits * t)) & ((1u << (bits - (slot ? 1 : 0))) - 1u);
+            if (slot) idx <<= 1;
+            if constexpr (bits == 8) v[t] = scale * __uint_as_float(kComp8Bits[min(idx, 255u)]);
+            else v[t] = grid_value(bits, idx) * scale;
+        }
+    } else if constexpr (sp.codec == Codec::Grp16) {
+        constexpr uint32_t lev_bits = 256u * bits;
+        const uint32_t w = window32(p, 4u * bits * lane, limit);
+        const float sc = (float)(window32(p, lev_bits + (lane >> 1) * 3u, limit) & 7u);
+        const float d = half_bits_to_float(half_at(p + lev_bits / 8 + 12));
+#pragma unroll
+        for (uint32_t t = 0; t < 4; ++t) v[t] = grid_value(bits, (w >> (bits * t)) & ((1u << bits) - 1u)) * d * sc;
+    } else {  // Q6K
+        const uint32_t w = window32(p, 24u * lane, limit);
+        const float sc = (float)(int)(int8_t)p[192 + (lane >> 2)];
+        const float e = half_bits_to_float(half_at(p + 208)) * sc;
+#pragma unroll
+        for (uint32_t t = 0; t < 4; ++t) v[t] = e * (float)((int)((w >> (6u * t)) & 63u) - 32) + 0.0f;
+    }
+}
+
 // Weight i of a block of L.n <= 256 weights.  Every part of such a block is one
 // LSB-first bit stream without byte alignment between the parts, except where the
 // reference's encoder places a trailer at a byte offset (noted below).

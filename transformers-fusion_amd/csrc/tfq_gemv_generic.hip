@@ -1,13 +1,14 @@
-// Dequant-fused GEMV for the formats that have no specialised kernel yet
-// (8-bit, 3-bit, 2-bit, plain lattice and raw fp32 blocks), on the wire layout:
+// Dequant-fused GEMV for the formats that have no matrix-core kernel (plain 2- and 4-bit lattice,
+// Q_G_6, the grouped-lattice fallback ids and raw fp32 blocks), on the wire layout:
 //   y[b][n] = sum_k x[b][k] * W[n][k]
 // Replaces Qwen35Engine::gemm (src/adapters/tools/qwen35_engine.cpp:54-101) for
 // those formats.  One wavefront owns a weight row; lane l decodes weights
-// 4l..4l+3 of every 256-weight block with the codec's own per-weight decode
-// (tfq_decode.hpp, the exact reference arithmetic) and multiplies them into up
-// to four activation rows in fp32.  The 64 lane sums are reduced with DPP adds.
-// Decoding costs a few tens of VALU operations per weight here; this kernel is
-// about coverage and exactness, the 4-bit formats have the fast path.
+// 4l..4l+3 of every 256-weight block with the codec's own arithmetic
+// (decode_quad in tfq_decode.hpp: the lane's codes come in with two aligned dword
+// reads) and multiplies them into up to four activation rows in fp32.  The 64 lane
+// sums are reduced with DPP adds.  The weights are exact here (fp32, no bf16
+// operand), which is what this kernel is for; the formats of the benchmark
+// configurations have the matrix-core path.
 
 #include "tfq_decode.hpp"
 
@@ -43,16 +44,22 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const uint8_t* __rest
     constexpr int BB = spec_of(FMT).block_bytes;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int nblk = K >> 8;
+    const uint8_t* limit = W + (size_t)N * (size_t)nblk * BB;
     for (int row = blockIdx.x * 4 + wave; row < N; row += gridDim.x * 4) {
         float acc[BT];
 #pragma unroll
         for (int b = 0; b < BT; ++b) acc[b] = 0.0f;
         const uint8_t* prow = W + (size_t)row * (size_t)nblk * BB;
+#pragma unroll 4
         for (int blk = 0; blk < nblk; ++blk) {
             const uint8_t* p = prow + (size_t)blk * BB;
             float w[4];
+            if constexpr (kHasQuad<FMT>) {
+                decode_quad<FMT>(p, lane, w, limit);
+            } else {
 #pragma unroll
-            for (int t = 0; t < 4; ++t) w[t] = decode_weight<FMT>(p, 4 * lane + t);
+                for (int t = 0; t < 4; ++t) w[t] = decode_weight<FMT>(p, 4 * lane + t);
+            }
             const size_t k0 = (size_t)blk * 256 + 4 * lane;
 #pragma unroll
             for (int b = 0; b < BT; ++b) {
@@ -121,13 +128,6 @@ int launch_gemv_generic(const tfq_weight* w, const void* x, int x_dtype, int B, 
         case TFQ_Q_G_4_K_L: return batched<TFQ_Q_G_4_K_L>(w, x, x_dtype, B, y, y_dtype, s);
         case TFQ_Q_6_5: return batched<TFQ_Q_6_5>(w, x, x_dtype, B, y, y_dtype, s);
         case TFQ_Q_4: return batched<TFQ_Q_4>(w, x, x_dtype, B, y, y_dtype, s);
-        case TFQ_Q_8: return batched<TFQ_Q_8>(w, x, x_dtype, B, y, y_dtype, s);
-        case TFQ_Q_G_2: return batched<TFQ_Q_G_2>(w, x, x_dtype, B, y, y_dtype, s);
-        case TFQ_Q_G_3: return batched<TFQ_Q_G_3>(w, x, x_dtype, B, y, y_dtype, s);
-        case TFQ_Q_G_8: return batched<TFQ_Q_G_8>(w, x, x_dtype, B, y, y_dtype, s);
-        case TFQ_SB256A3: return batched<TFQ_SB256A3>(w, x, x_dtype, B, y, y_dtype, s);
-        case TFQ_SB256A2: return batched<TFQ_SB256A2>(w, x, x_dtype, B, y, y_dtype, s);
-        case TFQ_B32S8: return batched<TFQ_B32S8>(w, x, x_dtype, B, y, y_dtype, s);
         default:
             return fail(TFQ_ERR_FORMAT, std::string("gemv: no kernel for format ") + tfq_format_name(w->fmt));
     }
