@@ -40,7 +40,13 @@ enum { TFQ_F32 = 0, TFQ_BF16 = 1 };
  * and keep their values because they are stored on disk; the four literal
  * formats are appended after FORMAT_COUNT (105). */
 enum {
-    TFQ_Q_2 = 1, TFQ_Q_4 = 3, TFQ_Q_8 = 5, TFQ_Q_32 = 9,
+    TFQ_Q_1 = 0, TFQ_Q_2 = 1, TFQ_Q_4 = 3, TFQ_Q_8 = 5, TFQ_Q_16 = 7, TFQ_Q_24 = 8, TFQ_Q_32 = 9,
+    TFQ_Q_1_K_L = 10, TFQ_Q_1_K_M = 11, TFQ_Q_1_K_H = 12,
+    TFQ_Q_16_K_L = 31, TFQ_Q_16_K_M = 32, TFQ_Q_16_K_H = 33, TFQ_Q_24_K_L = 34, TFQ_Q_24_K_M = 35, TFQ_Q_24_K_H = 36,
+    TFQ_Q_G_1 = 37, TFQ_Q_G_16 = 44, TFQ_Q_G_24 = 45, TFQ_Q_G_1_K_L = 46, TFQ_Q_G_1_K_M = 47, TFQ_Q_G_1_K_H = 48,
+    TFQ_Q_G_16_K_L = 67, TFQ_Q_G_16_K_M = 68, TFQ_Q_G_16_K_H = 69,
+    TFQ_Q_G_24_K_L = 70, TFQ_Q_G_24_K_M = 71, TFQ_Q_G_24_K_H = 72,
+    TFQ_Q_1_5 = 73, TFQ_Q_16_5 = 80, TFQ_Q_24_5 = 81, TFQ_Q_G_1_5 = 82, TFQ_Q_G_16_5 = 89, TFQ_Q_G_24_5 = 90,
     TFQ_Q_G_2 = 38, TFQ_Q_G_3 = 39, TFQ_Q_G_4 = 40, TFQ_Q_G_6 = 41, TFQ_Q_G_8 = 42,
     TFQ_Q_G_2_K_L = 49, TFQ_Q_G_2_K_M = 50, TFQ_Q_G_2_K_H = 51,
     TFQ_Q_G_3_K_L = 52, TFQ_Q_G_3_K_M = 53, TFQ_Q_G_3_K_H = 54,

@@ -18,7 +18,12 @@ _REF = os.path.join(_HERE, "_ref", "libref.so")
 
 # wire ids (include/quant/types.h:22-66 of the reference) + appended literal formats
 FMT = {
-    "Q_2": 1, "Q_4": 3, "Q_8": 5, "Q_32": 9,
+    "Q_1": 0, "Q_2": 1, "Q_4": 3, "Q_8": 5, "Q_16": 7, "Q_24": 8, "Q_32": 9,
+    "Q_1_K_L": 10, "Q_1_K_M": 11, "Q_1_K_H": 12, "Q_16_K_L": 31, "Q_16_K_M": 32, "Q_16_K_H": 33,
+    "Q_24_K_L": 34, "Q_24_K_M": 35, "Q_24_K_H": 36, "Q_G_1": 37, "Q_G_16": 44, "Q_G_24": 45,
+    "Q_G_1_K_L": 46, "Q_G_1_K_M": 47, "Q_G_1_K_H": 48, "Q_G_16_K_L": 67, "Q_G_16_K_M": 68, "Q_G_16_K_H": 69,
+    "Q_G_24_K_L": 70, "Q_G_24_K_M": 71, "Q_G_24_K_H": 72, "Q_1_5": 73, "Q_16_5": 80, "Q_24_5": 81,
+    "Q_G_1_5": 82, "Q_G_16_5": 89, "Q_G_24_5": 90,
     "Q_G_2": 38, "Q_G_3": 39, "Q_G_4": 40, "Q_G_6": 41, "Q_G_8": 42,
     "Q_G_2_K_L": 49, "Q_G_2_K_M": 50, "Q_G_2_K_H": 51, "Q_G_3_K_L": 52, "Q_G_3_K_M": 53, "Q_G_3_K_H": 54,
     "Q_G_4_K_L": 55, "Q_G_4_K_M": 56, "Q_G_4_K_H": 57, "Q_G_6_K_L": 58, "Q_G_6_K_M": 59, "Q_G_6_K_H": 60,

@@ -56,7 +56,11 @@ namespace {
 // Wire ids 0..104 are the reference's (include/quant/types.h:22-66).  The four
 // literal formats are appended after FORMAT_COUNT.
 enum : uint8_t {
-    F_Q_2 = 1, F_Q_4 = 3, F_Q_8 = 5, F_Q_32 = 9,
+    F_Q_1 = 0, F_Q_2 = 1, F_Q_4 = 3, F_Q_8 = 5, F_Q_16 = 7, F_Q_24 = 8, F_Q_32 = 9,
+    F_Q_1_K_L = 10, F_Q_1_K_M = 11, F_Q_1_K_H = 12, F_Q_16_K_L = 31, F_Q_16_K_H = 33, F_Q_24_K_L = 34, F_Q_24_K_H = 36,
+    F_Q_G_1 = 37, F_Q_G_16 = 44, F_Q_G_24 = 45, F_Q_G_1_K_L = 46, F_Q_G_1_K_M = 47, F_Q_G_1_K_H = 48,
+    F_Q_G_16_K_L = 67, F_Q_G_16_K_H = 69, F_Q_G_24_K_L = 70, F_Q_G_24_K_H = 72,
+    F_Q_1_5 = 73, F_Q_16_5 = 80, F_Q_24_5 = 81, F_Q_G_1_5 = 82, F_Q_G_16_5 = 89, F_Q_G_24_5 = 90,
     F_Q_G_2 = 38, F_Q_G_3 = 39, F_Q_G_4 = 40, F_Q_G_6 = 41, F_Q_G_8 = 42,
     F_Q_G_2_K_L = 49, F_Q_G_2_K_H = 51, F_Q_G_3_K_L = 52, F_Q_G_3_K_H = 54, F_Q_G_4_K_L = 55, F_Q_G_4_K_H = 57,
     F_Q_G_6_K_L = 58, F_Q_G_6_K_M = 59, F_Q_G_6_K_H = 60,
@@ -65,7 +69,7 @@ enum : uint8_t {
     F_B32S4 = 105, F_B32S8 = 106, F_SB256A3 = 107, F_SB256A2 = 108,
 };
 
-enum class Codec { Raw32, Lattice, Affine, Grp8, Sym32, Q6K };
+enum class Codec { Raw32, Lattice, Affine, Grp8, Sym32, Q6K, Q1, Wide };
 
 struct Spec {
     Codec codec;
@@ -79,6 +83,23 @@ struct Spec {
 bool spec_for(uint8_t fmt, Spec* s) {
     switch (fmt) {
         case F_Q_32:  *s = {Codec::Raw32, 32, 0, 0, 0, 32.0f}; return true;
+        // sign formats: tier = effort of the scale search (src/codec/block_codec.cpp:270-299, :2434-2449,
+        // :2523-2549, :2670-2675); Q_1 itself takes the RMS scale, marked by tier -1
+        case F_Q_1:   *s = {Codec::Q1, 1, 0, 0, 0, 1.0f, -1}; return true;
+        case F_Q_G_1: case F_Q_1_K_L: case F_Q_G_1_K_L: *s = {Codec::Q1, 1, 0, 0, 0, 1.0f, 0}; return true;
+        case F_Q_1_K_M: case F_Q_G_1_K_M: *s = {Codec::Q1, 1, 0, 0, 0, 1.0f, 1}; return true;
+        case F_Q_1_K_H: case F_Q_G_1_K_H: *s = {Codec::Q1, 1, 0, 0, 0, 1.0f, 2}; return true;
+        case F_Q_1_5: case F_Q_G_1_5: *s = {Codec::Affine, 1, 32, 6, 6, 1.5f}; return true;
+        // 16- and 24-bit formats (:1690-1873): gsz = 1 marks the ids that append per-32 residual
+        // means when the claim leaves room, claimed = what the payload is padded to
+        case F_Q_16: case F_Q_16_K_L: case F_Q_16_K_L + 1: case F_Q_16_K_H: *s = {Codec::Wide, 16, 0, 0, 0, 16.0f}; return true;
+        case F_Q_16_5: case F_Q_G_16_5: *s = {Codec::Wide, 16, 0, 0, 0, 16.5f}; return true;
+        case F_Q_G_16: *s = {Codec::Wide, 16, 1, 0, 0, 16.5f}; return true;
+        case F_Q_G_16_K_L: case F_Q_G_16_K_L + 1: case F_Q_G_16_K_H: *s = {Codec::Wide, 16, 1, 0, 0, 16.0f}; return true;
+        case F_Q_24: case F_Q_24_K_L: case F_Q_24_K_L + 1: case F_Q_24_K_H: *s = {Codec::Wide, 24, 0, 0, 0, 24.0f}; return true;
+        case F_Q_24_5: case F_Q_G_24_5: *s = {Codec::Wide, 24, 0, 0, 0, 24.5f}; return true;
+        case F_Q_G_24: *s = {Codec::Wide, 24, 1, 0, 0, 24.5f}; return true;
+        case F_Q_G_24_K_L: case F_Q_G_24_K_L + 1: case F_Q_G_24_K_H: *s = {Codec::Wide, 24, 1, 0, 0, 24.0f}; return true;
         case F_Q_2:   *s = {Codec::Lattice, 2, 0, 0, 0, 2.0f}; return true;
         case F_Q_4:   *s = {Codec::Lattice, 4, 0, 0, 0, 4.0f}; return true;
         case F_Q_8:   *s = {Codec::Lattice, 8, 0, 0, 0, 8.0f}; return true;
@@ -424,6 +445,247 @@ void grp8_decode(const uint8_t* bytes, size_t size, int n, float* out) {
         const int g = i >> 5;
         const uint16_t h = (uint16_t)(sc[2 * g] | ((uint16_t)sc[2 * g + 1] << 8));
         out[i] = half_to_float(h) * comp8().lv[bytes[i]];
+    }
+}
+
+// ------------------------------------------------------------ sign formats
+// Q_1 / Q_G_1 (+ _K_*): [binary16 scale][one sign bit per kept weight]; 16 positions carry no bit and
+// decode to zero.  Fewer than 32 weights: sign bits only, +-1.
+// The encoder skips the positions is_slot() names (src/codec/block_codec.cpp:176-180), the decoder
+// the positions ceil((s + 1) n / 16) - 1 (:1560-1564); they agree when 16 divides n.
+size_t q1_bytes(int n) { return (size_t)(n + 7) / 8; }
+
+float q1_fit_scale(const float* w, int n, int effort) {  // :270-299
+    double sum_abs = 0.0;
+    int kept = 0;
+    for (int i = 0; i < n; ++i)
+        if (!slot_at(i, n, 16)) { sum_abs += std::fabs((double)w[i]); ++kept; }
+    if (!kept) return 0.0f;
+    const uint16_t h0 = half_from_float((float)(sum_abs / kept));
+    float best = half_to_float(h0);
+    auto err = [&](float sc) {
+        double e = 0.0;
+        for (int i = 0; i < n; ++i) {
+            if (slot_at(i, n, 16)) continue;
+            const double v = (w[i] >= 0 ? sc : -sc);
+            const double d = (double)w[i] - v;
+            e += d * d;
+        }
+        return e;
+    };
+    double best_e = err(best);
+    const int rad = effort <= 0 ? 4 : (effort == 1 ? 10 : 24);
+    for (int delta = -rad; delta <= rad; ++delta) {
+        if (delta == 0) continue;
+        const int hc = (int)h0 + delta;
+        if (hc < 0 || hc > 0xFFFF) continue;
+        const float cand = half_to_float((uint16_t)hc);
+        const double e = err(cand);
+        if (e < best_e) { best_e = e; best = cand; }
+    }
+    return best;
+}
+
+bool q1_encode(int tier, const float* w, int n, uint8_t* out, size_t nbytes) {
+    if (nbytes != q1_bytes(n)) return false;
+    std::memset(out, 0, nbytes);
+    BitSink bs(out, nbytes);
+    if (n < 32) {
+        for (int i = 0; i < n; ++i) bs.put(w[i] >= 0.0f ? 1u : 0u, 1);
+        return !bs.overflow;
+    }
+    float scale;
+    if (tier < 0) {  // rms_scale, :213-218
+        double sum = 0.0;
+        for (int i = 0; i < n; ++i) sum += (double)w[i] * w[i];
+        scale = (float)std::sqrt(sum / (double)n);
+    } else {
+        scale = q1_fit_scale(w, n, tier);
+    }
+    bs.put(half_from_float(scale), 16);
+    for (int i = 0; i < n; ++i)
+        if (!slot_at(i, n, 16)) bs.put(w[i] >= 0.0f ? 1u : 0u, 1);
+    return !bs.overflow;
+}
+
+void q1_decode(const uint8_t* bytes, size_t size, int n, float* out) {  // :1530-1618
+    if (n < 32) {
+        uint64_t win = 0;
+        std::memcpy(&win, bytes, std::min<size_t>(8, size));
+        for (int i = 0; i < n; ++i) out[i] = ((win >> i) & 1u) ? 1.0f : -1.0f;
+        return;
+    }
+    BitSource br(bytes, size);
+    const float scale = half_to_float((uint16_t)br.take(16));
+    std::vector<char> slot((size_t)n, 0);
+    for (int s = 0; s < 16; ++s) {
+        const int64_t pos = ((int64_t)(s + 1) * (int64_t)n + 15) / 16 - 1;
+        if (pos >= 0 && pos < n) slot[(size_t)pos] = 1;
+    }
+    for (int i = 0; i < n; ++i) {
+        if (slot[(size_t)i]) { out[i] = 0.0f; continue; }
+        out[i] = br.take(1) ? scale : -scale;
+    }
+}
+
+// ------------------------------------------------ 16- and 24-bit formats
+// Q_24: the top three bytes of the binary32, low byte first (:1809-1873).
+// Q_16: per 256 weights [binary32 min][binary32 max], then groups of four weights in 63 bits:
+// three 16-bit and one 15-bit uniform code over [min, max]; a tensor piece that is not a
+// multiple of 256 is stored as raw binary16 instead (:1690-1807).
+// The grouped ids append one binary16 mean of (w - decoded) per 32 weights when the claim has room.
+size_t q16_packed_bytes(int n) {
+    size_t packed = 0;
+    for (int start = 0; start < n; start += 256) {
+        const int end = std::min(start + 256, n);
+        packed += 8 + ((size_t)((end - start + 3) / 4) * 63 + 7) / 8;
+    }
+    return packed;
+}
+
+void q16_encode(const float* w, int n, uint8_t* out) {  // out: 2 n bytes
+    std::memset(out, 0, (size_t)n * 2);
+    if (q16_packed_bytes(n) > (size_t)n * 2) {
+        for (int i = 0; i < n; ++i) {
+            const uint16_t h = half_from_float(w[i]);
+            out[2 * i] = (uint8_t)(h & 0xFF);
+            out[2 * i + 1] = (uint8_t)(h >> 8);
+        }
+        return;
+    }
+    BitSink bs(out, (size_t)n * 2);
+    for (int start = 0; start < n; start += 256) {
+        const int end = std::min(start + 256, n);
+        float vmin = 1e30f, vmax = -1e30f;
+        for (int i = start; i < end; ++i) { vmin = std::min(vmin, w[i]); vmax = std::max(vmax, w[i]); }
+        if (vmin > vmax) { vmin = 0; vmax = 0; }
+        uint32_t imin, imax;
+        std::memcpy(&imin, &vmin, 4);
+        std::memcpy(&imax, &vmax, 4);
+        bs.put(imin, 32);
+        bs.put(imax, 32);
+        const float range = vmax - vmin;
+        const float scale16 = range > 0 ? 65535.0f / range : 0.0f;
+        const float scale15 = range > 0 ? 32767.0f / range : 0.0f;
+        for (int i = start; i < end; i += 4) {
+            uint64_t group = 0;
+            for (int k = 0; k < 4 && i + k < end; ++k) {
+                if (k == 3) {
+                    const int q = std::max(0, std::min(32767, (int)std::lround((w[i + k] - vmin) * scale15)));
+                    group |= (uint64_t)q << 48;
+                } else {
+                    const int q = std::max(0, std::min(65535, (int)std::lround((w[i + k] - vmin) * scale16)));
+                    group |= (uint64_t)q << (16 * k);
+                }
+            }
+            bs.put((uint32_t)(group & 0xFFFFFFFFu), 32);
+            bs.put((uint32_t)(group >> 32), 31);
+        }
+    }
+}
+
+void q16_decode(const uint8_t* bytes, size_t size, int n, float* out) {
+    if (q16_packed_bytes(n) > (size_t)n * 2) {
+        const size_t avail = std::min(size, (size_t)n * 2);
+        for (int i = 0; i < n; ++i) {
+            uint16_t h = 0;
+            if ((size_t)i * 2 + 1 < avail) h = (uint16_t)((uint16_t)bytes[2 * i] | ((uint16_t)bytes[2 * i + 1] << 8));
+            else if ((size_t)i * 2 < avail) h = bytes[2 * i];
+            out[i] = half_to_float(h);
+        }
+        return;
+    }
+    BitSource br(bytes, size);
+    for (int start = 0; start < n; start += 256) {
+        const int end = std::min(start + 256, n);
+        const uint32_t imin = br.take(32), imax = br.take(32);
+        float vmin, vmax;
+        std::memcpy(&vmin, &imin, 4);
+        std::memcpy(&vmax, &imax, 4);
+        const float range = vmax - vmin;
+        const float scale16 = range > 0 ? range / 65535.0f : 0.0f;
+        const float scale15 = range > 0 ? range / 32767.0f : 0.0f;
+        for (int i = start; i < end; i += 4) {
+            const uint64_t group = (uint64_t)br.take(32) | ((uint64_t)br.take(31) << 32);
+            for (int k = 0; k < 4 && i + k < end; ++k) {
+                // one fused multiply-add in the reference's Release build
+                if (k == 3) out[i + k] = std::fma((float)(uint32_t)((group >> 48) & 0x7FFFu), scale15, vmin);
+                else out[i + k] = std::fma((float)(uint32_t)((group >> (16 * k)) & 0xFFFFu), scale16, vmin);
+            }
+        }
+    }
+}
+
+void q24_encode(const float* w, int n, uint8_t* out) {
+    for (int i = 0; i < n; ++i) {
+        uint32_t u;
+        std::memcpy(&u, &w[i], 4);
+        out[3 * i] = (uint8_t)(u >> 8);
+        out[3 * i + 1] = (uint8_t)(u >> 16);
+        out[3 * i + 2] = (uint8_t)(u >> 24);
+    }
+}
+
+void q24_decode(const uint8_t* bytes, size_t size, int n, float* out) {
+    // the reference's vector path stops at the first group of eight that the payload does not
+    // fully hold and its scalar tail at the first missing triple: everything after stays zero
+    for (int i = 0; i < n; ++i) {
+        if ((size_t)i * 3 + 2 >= size) break;
+        const uint32_t u = ((uint32_t)bytes[3 * i] << 8) | ((uint32_t)bytes[3 * i + 1] << 16) | ((uint32_t)bytes[3 * i + 2] << 24);
+        std::memcpy(&out[i], &u, 4);
+    }
+}
+
+struct WideSizes {
+    size_t plain, total;
+    bool residual;
+};
+
+WideSizes wide_sizes(const Spec& sp, int n) {
+    WideSizes z{};
+    z.plain = (size_t)n * (size_t)(sp.bits / 8);
+    const size_t claimed = (size_t)std::ceil((double)sp.claimed * (double)n / 8.0);
+    z.residual = sp.gsz == 1 && claimed > z.plain && n % 32 == 0;
+    z.total = std::max(z.plain, claimed);
+    if (sp.claimed == (float)sp.bits && sp.gsz == 0) z.total = z.plain;
+    return z;
+}
+
+bool wide_encode(const Spec& sp, const float* w, int n, uint8_t* out, size_t nbytes) {
+    const WideSizes z = wide_sizes(sp, n);
+    if (nbytes != z.total) return false;
+    std::memset(out, 0, nbytes);
+    std::vector<float> plain((size_t)n, 0.0f);
+    if (sp.bits == 16) { q16_encode(w, n, out); q16_decode(out, z.plain, n, plain.data()); }
+    else { q24_encode(w, n, out); q24_decode(out, z.plain, n, plain.data()); }
+    if (z.residual) {
+        uint8_t* p = out + z.plain;
+        for (int g = 0; g < n / 32; ++g) {
+            double mean = 0;
+            for (int i = 0; i < 32; ++i) mean += (double)w[g * 32 + i] - plain[(size_t)(g * 32 + i)];
+            mean /= 32.0;
+            const uint16_t h = half_from_float((float)mean);
+            p[0] = (uint8_t)(h & 0xFF);
+            p[1] = (uint8_t)(h >> 8);
+            p += 2;
+        }
+    }
+    return true;
+}
+
+void wide_decode(const Spec& sp, const uint8_t* bytes, size_t size, int n, float* out) {
+    const size_t plain = (size_t)n * (size_t)(sp.bits / 8);
+    const size_t claimed = (size_t)std::ceil((double)sp.claimed * (double)n / 8.0);
+    const bool residual = sp.gsz == 1 && n % 32 == 0 && size >= claimed && claimed > plain;
+    const size_t use = residual ? plain : size;
+    if (sp.bits == 16) q16_decode(bytes, use, n, out);
+    else q24_decode(bytes, use, n, out);
+    if (residual) {
+        const uint8_t* p = bytes + plain;
+        for (int g = 0; g < n / 32; ++g, p += 2) {
+            const float m = half_to_float((uint16_t)((uint16_t)p[0] | ((uint16_t)p[1] << 8)));
+            for (int i = 0; i < 32; ++i) out[g * 32 + i] += m;
+        }
     }
 }
 
@@ -1065,6 +1327,8 @@ long block_bytes(uint8_t fmt, int n) {
             return affine_bytes(kGrp8Tail, n);
         case Codec::Affine: return affine_bytes(sp, n);
         case Codec::Q6K: return (long)q6k_sizes(n).total;
+        case Codec::Q1: return (long)q1_bytes(n);
+        case Codec::Wide: return (long)wide_sizes(sp, n).total;
         case Codec::Sym32: return (n >= 32 && n % 32 == 0) ? (long)sym32_bytes(sp.bits, n) : -1;
     }
     return -1;
@@ -1085,6 +1349,8 @@ long encode_block(uint8_t fmt, const float* w, int n, uint8_t* out, size_t cap) 
             break;
         case Codec::Affine: ok = affine_encode(sp, w, n, out, (size_t)need); break;
         case Codec::Q6K: ok = q6k_encode_tier(sp.tier, w, n, out, (size_t)need); break;
+        case Codec::Q1: ok = q1_encode(sp.tier, w, n, out, (size_t)need); break;
+        case Codec::Wide: ok = wide_encode(sp, w, n, out, (size_t)need); break;
         case Codec::Sym32: ok = sym32_encode(sp.bits, w, n, out); break;
     }
     return ok ? need : -1;
@@ -1104,6 +1370,8 @@ int decode_block(uint8_t fmt, const uint8_t* bytes, size_t size, int n, float* o
             grp8_decode(bytes, size, n, out);
             return 0;
         case Codec::Q6K: q6k_decode(bytes, size, n, out); return 0;
+        case Codec::Q1: q1_decode(bytes, size, n, out); return 0;
+        case Codec::Wide: wide_decode(sp, bytes, size, n, out); return 0;
         case Codec::Affine: return affine_decode(sp, bytes, size, n, out) ? 0 : -1;
         case Codec::Sym32: return sym32_decode(sp.bits, bytes, size, n, out) ? 0 : -1;
     }

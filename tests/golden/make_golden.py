@@ -21,8 +21,9 @@ tails.npz
     blocks of n <= 256 weights (the first n of two of the inputs above) through the
     reference codec, one row of `index` = (wire id, n, input, payload offset, payload
     bytes, decoded offset) into the flat `payloads` / `decoded` arrays: the short-block
-    layouts (raw levels, one scale, grouped-lattice fallback), Q_2, Q_G_6 and the ids
-    whose claim is below the affine header's size
+    layouts (raw levels, one scale, grouped-lattice fallback), Q_2, Q_G_6, the ids
+    whose claim is below the affine header's size, the sign formats and the 16- and
+    24-bit formats
 sample.quant, sample_quant.npz
     a container written by the reference's QUANTWriter (header with a 5-byte config,
     format table, tensor table, block records): tensor "blk.0.ffn_gate" 4 x 512 in Q_G_4,
@@ -60,7 +61,8 @@ def inputs():
 
 
 TAIL_FORMATS = ["Q_2", "Q_4", "Q_8", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_6", "Q_G_8", "Q_G_2_K_H", "Q_G_3_K_L",
-                "Q_G_4_K_M", "Q_G_6_K_M", "Q_G_6_K_H", "Q_2_5", "Q_6_5"]
+                "Q_G_4_K_M", "Q_G_6_K_M", "Q_G_6_K_H", "Q_2_5", "Q_6_5",
+                "Q_1", "Q_G_1_K_H", "Q_1_5", "Q_16", "Q_G_16", "Q_24", "Q_G_24"]
 TAIL_SIZES = [1, 7, 8, 15, 16, 31, 32, 33, 100, 160, 250, 255, 256]
 
 

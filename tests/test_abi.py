@@ -41,7 +41,7 @@ def test_registry_mirror_without_gpu(tfq):
 def test_errors_are_reported_not_swallowed(tfq):
     L = tfq.lib()
     out = C.c_size_t(0)
-    assert L.tfq_block_bytes(0, 256, C.byref(out)) == 2            # TFQ_ERR_FORMAT: Q_1 is not handled
+    assert L.tfq_block_bytes(2, 256, C.byref(out)) == 2            # TFQ_ERR_FORMAT: Q_3 is not handled
     assert b"not handled" in L.tfq_last_error()
     assert L.tfq_block_bytes(40, 100, C.byref(out)) == 0 and out.value == 57   # short block: grouped-lattice fallback
     assert L.tfq_block_bytes(40, 257, C.byref(out)) == 3           # TFQ_ERR_SHAPE

@@ -10,6 +10,8 @@ pytestmark = pytest.mark.gpu
 G = os.path.join(os.path.dirname(__file__), "golden")
 DECODE_FORMATS = ["Q_2", "Q_4", "Q_8", "Q_32", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_6", "Q_G_8", "Q_4_5", "Q_G_8_5",
                   "Q_G_2_K_M", "Q_G_3_K_L", "Q_G_4_K_H", "Q_G_6_K_H", "Q_2_5", "Q_G_6_5",
+                  "Q_1", "Q_G_1", "Q_G_1_K_H", "Q_1_5", "Q_16", "Q_16_5", "Q_G_16", "Q_G_16_K_M", "Q_24", "Q_G_24_5", "Q_G_24",
+                  "Q_G_24_K_L",
                   "B32S4", "B32S8", "SB256A3", "SB256A2"]
 
 
@@ -44,7 +46,8 @@ def test_decode_golden_payloads(tfq, gpu, fmt):
 
 
 @pytest.mark.parametrize("fmt", ["Q_2", "Q_4", "Q_8", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_6", "Q_G_8", "Q_G_2_K_L", "Q_G_3_K_M",
-                                 "Q_G_4_K_L", "Q_6_5", "SB256A3", "SB256A2"])
+                                 "Q_G_4_K_L", "Q_6_5", "SB256A3", "SB256A2", "Q_1", "Q_1_5", "Q_16", "Q_G_16", "Q_24",
+                                 "Q_G_24"])
 def test_decode_arbitrary_payload_bits(O, tfq, gpu, fmt):
     # every payload bit pattern is legal input: random bytes, finite scales
     import torch
@@ -53,7 +56,13 @@ def test_decode_arbitrary_payload_bits(O, tfq, gpu, fmt):
     pay = rng.integers(0, 256, (256, nb), dtype=np.uint8)
     if fmt in ("Q_G_8",):
         pay[:, -16:] &= 0x7B
-    elif fmt in ("Q_2", "Q_4", "Q_8"):
+    elif fmt in ("Q_16", "Q_G_16"):   # binary32 min / max with small exponents, finite residual means
+        pay[:, [3, 7]] &= 0x3F
+        pay[:, -16:] &= 0x7B
+    elif fmt in ("Q_24", "Q_G_24"):   # the top byte of every weight, finite residual means
+        pay[:, 2:768:3] &= 0xBF
+        pay[:, -16:] &= 0x7B
+    elif fmt in ("Q_1", "Q_2", "Q_4", "Q_8"):
         pay[:, :2] &= 0x7B
     else:
         pay[:, -4:] &= 0x7B
@@ -63,7 +72,8 @@ def test_decode_arbitrary_payload_bits(O, tfq, gpu, fmt):
 
 
 TAIL_FORMATS = ["Q_2", "Q_4", "Q_8", "Q_32", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_6", "Q_G_8", "Q_G_2_K_H", "Q_G_4_K_M",
-                "Q_G_6_K_L", "Q_6_5", "SB256A3"]
+                "Q_G_6_K_L", "Q_6_5", "SB256A3", "Q_1", "Q_G_1_K_M", "Q_1_5", "Q_16", "Q_G_16", "Q_16_5", "Q_24", "Q_G_24",
+                "Q_G_24_K_H"]
 
 
 @pytest.mark.parametrize("fmt", TAIL_FORMATS)
@@ -109,7 +119,9 @@ def test_half_subnormal_scales_decode_exactly(O, tfq, gpu):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
-@pytest.mark.parametrize("fmt", ["B32S4", "B32S8", "Q_32"])
+@pytest.mark.parametrize("fmt", ["B32S4", "B32S8", "Q_32", "Q_24", "Q_24_5", "Q_G_24", "Q_G_24_K_M", "Q_16", "Q_G_16_5", "Q_G_16",
+                                 "Q_G_16_K_L", "Q_1", "Q_G_1", "Q_1_K_M", "Q_G_1_K_H",
+                                 "Q_G_4", "Q_4_5", "Q_G_3", "Q_G_2", "SB256A3", "SB256A2", "Q_1_5"])
 def test_device_encoder_codes_bit_exact(O, tfq, gpu, fmt):
     import torch
     w = _inputs(O, 64)
@@ -118,6 +130,21 @@ def test_device_encoder_codes_bit_exact(O, tfq, gpu, fmt):
     want = O.encode_tensor(fmt, w)
     got = tfq.encode(fmt, torch.from_numpy(w).to(gpu)).cpu().numpy()
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("fmt", ["Q_G_4", "Q_G_3", "Q_G_2", "SB256A3", "SB256A2"])
+def test_affine_encoder_many_blocks(O, tfq, gpu, fmt):
+    """The iterative affine encoder (per-group Lloyd fit, joint refinement) on 8192 blocks of four
+    distributions: every payload byte equals the oracle's."""
+    import torch
+    rs = np.random.RandomState(11)
+    n = 2048 * 256
+    w = np.concatenate([(rs.randn(n) * 0.02), rs.randn(n), rs.laplace(0, 0.015, n) + 0.01, np.abs(rs.randn(n)) * 0.3]).astype(np.float32)
+    got = tfq.encode(fmt, torch.from_numpy(w).to(gpu)).cpu().numpy()
+    want = O.encode_tensor(fmt, w)
+    bb = O.block_bytes(fmt)
+    bad = np.nonzero((got.reshape(-1, bb) != want.reshape(-1, bb)).any(1))[0]
+    assert bad.size == 0, f"{bad.size} of {w.size // 256} blocks differ, first {bad[:5]}"
 
 
 def test_host_pointer_codec_entry_points(O, tfq, gpu):

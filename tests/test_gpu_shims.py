@@ -60,7 +60,7 @@ def test_claimed_bytes_are_ceil_of_bpw(O, drv):
         assert drv.drv_claimed_bytes(O.FMT[name], 256) == want
 
 
-@pytest.mark.parametrize("fmt", ["B32S4", "B32S8", "Q_32"])
+@pytest.mark.parametrize("fmt", ["B32S4", "B32S8", "Q_32", "Q_G_4", "Q_G_3", "Q_G_2", "SB256A3", "Q_16", "Q_G_24", "Q_1", "Q_G_1_K_H"])
 def test_quantize_block_all_codes_bit_exact(O, drv, fmt):
     w = O.rng_normal(7, 256, 0.02)
     want = O.encode_block(fmt, w)

@@ -57,7 +57,17 @@ struct NameRow {
 // Canonical names (format_name, include/quant/types.h:168-196) of the ids this
 // backend handles, plus the appended literal formats.
 const NameRow kNames[] = {
-    {"Q_2", TFQ_Q_2}, {"Q_4", TFQ_Q_4}, {"Q_8", TFQ_Q_8}, {"Q_32", TFQ_Q_32},
+    {"Q_1", TFQ_Q_1}, {"Q_2", TFQ_Q_2}, {"Q_4", TFQ_Q_4}, {"Q_8", TFQ_Q_8}, {"Q_16", TFQ_Q_16}, {"Q_24", TFQ_Q_24},
+    {"Q_32", TFQ_Q_32},
+    {"Q_1_K_L", TFQ_Q_1_K_L}, {"Q_1_K_M", TFQ_Q_1_K_M}, {"Q_1_K_H", TFQ_Q_1_K_H},
+    {"Q_16_K_L", TFQ_Q_16_K_L}, {"Q_16_K_M", TFQ_Q_16_K_M}, {"Q_16_K_H", TFQ_Q_16_K_H},
+    {"Q_24_K_L", TFQ_Q_24_K_L}, {"Q_24_K_M", TFQ_Q_24_K_M}, {"Q_24_K_H", TFQ_Q_24_K_H},
+    {"Q_G_1", TFQ_Q_G_1}, {"Q_G_16", TFQ_Q_G_16}, {"Q_G_24", TFQ_Q_G_24},
+    {"Q_G_1_K_L", TFQ_Q_G_1_K_L}, {"Q_G_1_K_M", TFQ_Q_G_1_K_M}, {"Q_G_1_K_H", TFQ_Q_G_1_K_H},
+    {"Q_G_16_K_L", TFQ_Q_G_16_K_L}, {"Q_G_16_K_M", TFQ_Q_G_16_K_M}, {"Q_G_16_K_H", TFQ_Q_G_16_K_H},
+    {"Q_G_24_K_L", TFQ_Q_G_24_K_L}, {"Q_G_24_K_M", TFQ_Q_G_24_K_M}, {"Q_G_24_K_H", TFQ_Q_G_24_K_H},
+    {"Q_1_5", TFQ_Q_1_5}, {"Q_16_5", TFQ_Q_16_5}, {"Q_24_5", TFQ_Q_24_5},
+    {"Q_G_1_5", TFQ_Q_G_1_5}, {"Q_G_16_5", TFQ_Q_G_16_5}, {"Q_G_24_5", TFQ_Q_G_24_5},
     {"Q_G_2", TFQ_Q_G_2}, {"Q_G_3", TFQ_Q_G_3}, {"Q_G_4", TFQ_Q_G_4}, {"Q_G_6", TFQ_Q_G_6}, {"Q_G_8", TFQ_Q_G_8},
     {"Q_G_2_K_L", TFQ_Q_G_2_K_L}, {"Q_G_2_K_M", TFQ_Q_G_2_K_M}, {"Q_G_2_K_H", TFQ_Q_G_2_K_H},
     {"Q_G_3_K_L", TFQ_Q_G_3_K_L}, {"Q_G_3_K_M", TFQ_Q_G_3_K_M}, {"Q_G_3_K_H", TFQ_Q_G_3_K_H},

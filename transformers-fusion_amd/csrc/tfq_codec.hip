@@ -83,6 +83,343 @@ __global__ __launch_bounds__(256) void encode_raw32_kernel(const float* __restri
     reinterpret_cast<float*>(dst)[e] = w[e];
 }
 
+// Closed-form encoders of the 16- and 24-bit formats (quant_q16_enhanced / quant_q24,
+// src/codec/block_codec.cpp:1690-1757, :1809-1820) and of the residual means the grouped ids append
+// (:2450-2493): per 32 weights the binary16 of mean(w - decoded), summed in double in index order.
+// One workgroup per block: lane i owns weight i, then output byte pairs, then (8 lanes) a group.
+template <int FMT>
+__global__ __launch_bounds__(256) void encode_wide_kernel(const float* __restrict__ w, uint8_t* __restrict__ dst) {
+    constexpr Spec sp = spec_of(FMT);
+    constexpr int plain = 256 * sp.bits / 8;
+    __shared__ uint32_t code[256];
+    __shared__ float dec[256];
+    __shared__ float red[8];
+    const int64_t blk = blockIdx.x;
+    const uint32_t i = threadIdx.x;
+    uint8_t* p = dst + blk * (int64_t)sp.block_bytes;
+    const float x = w[blk * 256 + i];
+    if constexpr (sp.bits == 24) {
+        const uint32_t u = __float_as_uint(x);
+        p[3 * i] = (uint8_t)(u >> 8);
+        p[3 * i + 1] = (uint8_t)(u >> 16);
+        p[3 * i + 2] = (uint8_t)(u >> 24);
+        dec[i] = __uint_as_float(u & 0xFFFFFF00u);
+    } else {
+        // min and max are order independent; the encoder starts them at +-1e30
+        float lo = fminf(1e30f, x), hi = fmaxf(-1e30f, x);
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) { lo = fminf(lo, __shfl_xor(lo, m, 64)); hi = fmaxf(hi, __shfl_xor(hi, m, 64)); }
+        if ((i & 63u) == 0) { red[i >> 6] = lo; red[4 + (i >> 6)] = hi; }
+        __syncthreads();
+        lo = fminf(fminf(red[0], red[1]), fminf(red[2], red[3]));
+        hi = fmaxf(fmaxf(red[4], red[5]), fmaxf(red[6], red[7]));
+        if (lo > hi) { lo = 0.0f; hi = 0.0f; }
+        const float range = hi - lo;
+        const bool narrow = (i & 3u) == 3u;
+        const float top = narrow ? 32767.0f : 65535.0f;
+        const float scale = range > 0 ? top / range : 0.0f;
+        long q = lroundf((x - lo) * scale);
+        q = q < 0 ? 0 : q > (long)top ? (long)top : q;
+        code[i] = (uint32_t)q;
+        const float dscale = range > 0 ? range / top : 0.0f;
+        dec[i] = __builtin_fmaf((float)(uint32_t)q, dscale, lo);
+        __syncthreads();
+        // output bytes 2 i and 2 i + 1: bits 16 i .. 16 i + 15 of [min][max][64 groups of 63 bits]
+        uint32_t out16 = 0;
+#pragma unroll
+        for (uint32_t b = 0; b < 16; ++b) {
+            const uint32_t pos = 16 * i + b;
+            uint32_t bit;
+            if (pos < 32) bit = (__float_as_uint(lo) >> pos) & 1u;
+            else if (pos < 64) bit = (__float_as_uint(hi) >> (pos - 32)) & 1u;
+            else {
+                const uint32_t g = (pos - 64) / 63, r = (pos - 64) - 63 * g;
+                const uint32_t k = r < 48 ? r >> 4 : 3;
+                bit = g < 64 ? (code[4 * g + k] >> (r - 16 * k)) & 1u : 0u;
+            }
+            out16 |= bit << b;
+        }
+        p[2 * i] = (uint8_t)(out16 & 0xFF);
+        p[2 * i + 1] = (uint8_t)(out16 >> 8);
+    }
+    if constexpr (sp.block_bytes > plain) {
+        __syncthreads();
+        if (i < 8) {
+            uint32_t h = 0;
+            if constexpr (sp.scb == 1) {
+                double mean = 0.0;
+                for (int j = 0; j < 32; ++j) mean += (double)w[blk * 256 + 32 * i + j] - (double)dec[32 * i + j];
+                mean /= 32.0;
+                h = float_to_half_bits((float)mean);
+            }
+            p[plain + 2 * i] = (uint8_t)(h & 0xFF);  // ids without residuals pad with zeros
+            p[plain + 2 * i + 1] = (uint8_t)(h >> 8);
+        }
+    }
+}
+
+// Sign formats (src/codec/block_codec.cpp:2434-2449, :2523-2549): binary16 scale, then the sign bits of
+// the weights that are not slots.  tier < 0: Q_1, scale = sqrt(mean w^2) (rms_scale, :213-218); otherwise
+// the mean |w| of the kept weights snapped to binary16 and the best of the 2 * radius neighbouring
+// binary16 values by squared error (q1_fit_scale_fp16, :270-299), radius 4, 10 or 24.  Every sum runs
+// in double in index order; lane c evaluates candidate c, lane 0 picks the first strict minimum in the
+// reference's order (centre, then -radius .. +radius).
+__global__ __launch_bounds__(256) void encode_q1_kernel(const float* __restrict__ w, uint8_t* __restrict__ dst, int tier) {
+    __shared__ float x[256];
+    __shared__ double err[64];
+    __shared__ uint32_t scale_bits;
+    const int64_t blk = blockIdx.x;
+    const uint32_t i = threadIdx.x;
+    x[i] = w[blk * 256 + i];
+    __syncthreads();
+    if (tier < 0) {
+        if (i == 0) {
+            double sum = 0.0;
+            for (int j = 0; j < 256; ++j) sum += (double)x[j] * (double)x[j];
+            scale_bits = float_to_half_bits((float)sqrt(sum / 256.0));
+        }
+    } else {
+        const int rad = tier == 0 ? 4 : tier == 1 ? 10 : 24;
+        __shared__ uint32_t h0s;
+        if (i == 0) {
+            double sum_abs = 0.0;
+            for (int j = 0; j < 256; ++j)
+                if ((j & 15) != 15) sum_abs += fabs((double)x[j]);
+            h0s = float_to_half_bits((float)(sum_abs / 240.0));
+        }
+        __syncthreads();
+        const int h0 = (int)h0s;
+        // candidate c: 0 = h0, 1 .. rad = h0 - rad .. h0 - 1, rad + 1 .. 2 rad = h0 + 1 .. h0 + rad
+        if ((int)i <= 2 * rad) {
+            const int delta = i == 0 ? 0 : (int)i <= rad ? (int)i - rad - 1 : (int)i - rad;
+            const int hc = h0 + delta;
+            double e = -1.0;  // out of range: skipped
+            if (hc >= 0 && hc <= 0xFFFF) {
+                const float sc = half_bits_to_float((uint32_t)hc);
+                e = 0.0;
+                for (int j = 0; j < 256; ++j) {
+                    if ((j & 15) == 15) continue;
+                    const double v = x[j] >= 0 ? (double)sc : -(double)sc;
+                    const double d = (double)x[j] - v;
+                    e = __builtin_fma(d, d, e);  // fused in the reference's Release build
+                }
+            }
+            err[i] = e;
+        }
+        __syncthreads();
+        if (i == 0) {
+            int best = h0;
+            double best_e = err[0];
+            for (int c = 1; c <= 2 * rad; ++c) {
+                const int delta = c <= rad ? c - rad - 1 : c - rad;
+                if (err[c] >= 0.0 && err[c] < best_e) { best_e = err[c]; best = h0 + delta; }
+            }
+            scale_bits = (uint32_t)best;  // a binary16 pattern converts back to itself
+        }
+    }
+    __syncthreads();
+    uint8_t* p = dst + blk * 32;
+    if (i < 32) {
+        uint32_t byte = 0;
+#pragma unroll
+        for (uint32_t b = 0; b < 8; ++b) {
+            const uint32_t pos = 8 * i + b;
+            uint32_t bit;
+            if (pos < 16) bit = (scale_bits >> pos) & 1u;
+            else {
+                const uint32_t j = pos - 16;        // kept index -> weight index (15 kept weights per 16)
+                bit = x[j + j / 15] >= 0.0f ? 1u : 0u;
+            }
+            byte |= bit << b;
+        }
+        p[i] = (uint8_t)byte;
+    }
+}
+
+// Affine family encoder: quant_affine with grp16_fit_affine (src/codec/block_codec.cpp:1337-1521) for
+// Q_G_4 / Q_G_3 / Q_G_2, the superblock formats and Q_1_5.  One wavefront per block; lane g owns group g
+// (8 or 16 lanes work): the per-group Lloyd fit (4 x assign + least-squares refit, +-15 % scale polish,
+// closing refit) and the per-group part of the 5 joint refinements run sequentially in that lane, in the
+// reference's order, with double sums; lane 0 does the sums over groups.  Multiply-adds are fused exactly
+// where the reference's Release build (GCC, -ffp-contract=fast) fuses them and nowhere else.  The payload
+// is then assembled a byte per lane from the codes in LDS.
+__device__ __forceinline__ uint32_t unit_nearest_dev(float value, int bits) {
+    const float v = fmaxf(0.0f, fminf(1.0f, value));
+    const float top = bits == 1 ? 1.0f : bits == 4 ? 15.0f : bits == 3 ? 7.0f : bits == 6 ? 63.0f : bits == 8 ? 255.0f : 3.0f;
+    return (uint32_t)lroundf(v * top);
+}
+__device__ __forceinline__ double fms2(double a, double b, double c, double d) {  // a b - c d, first product fused
+    return __builtin_fma(a, b, -(c * d));
+}
+
+template <int FMT>
+__global__ __launch_bounds__(64) void encode_affine_kernel(const float* __restrict__ wg, uint8_t* __restrict__ dst) {
+    constexpr Spec sp = spec_of(FMT);
+    constexpr int bits = sp.bits, gsz = sp.gsz, ng = 256 / gsz;
+    constexpr int scq = (1 << sp.scb) - 1, mq = (1 << sp.mb) - 1, bias = (mq + 1) / 2;
+    constexpr float eps = 1e-15f;
+    __shared__ float w[256];
+    __shared__ float s_[16], m_[16];
+    __shared__ int sc_[16], mc_[16];
+    __shared__ float dd[2];
+    __shared__ uint8_t code[256];
+    const int64_t blk = blockIdx.x;
+    const int t = threadIdx.x;
+    for (int i = t; i < 256; i += 64) w[i] = wg[blk * 256 + i];
+    __syncthreads();
+    const float* x = w + t * gsz;
+
+    // ---- per-group fit
+    if (t < ng) {
+        float maxw = -1e30f, minw = 1e30f;
+        for (int i = 0; i < gsz; ++i) { maxw = fmaxf(maxw, x[i]); minw = fminf(minw, x[i]); }
+        float s = maxw - minw, m = minw;
+        if (!(fabsf(s) > 1e-30f)) { s = 0.0f; m = 0.0f; }
+        else {
+            // assign levels with (am, as), then refit (s, m) by least squares over (level, weight)
+            auto assign_refit = [&](float am, float as) __attribute__((always_inline)) {
+                double sw = 0, sl = 0, sl2 = 0, sx = 0, sxl = 0;
+                for (int i = 0; i < gsz; ++i) {
+                    const double l = (double)unit_level(bits, unit_nearest_dev((x[i] - am) / as, bits));
+                    sw += 1.0; sl += l; sl2 = __builtin_fma(l, l, sl2);
+                    sx += (double)x[i]; sxl = __builtin_fma((double)x[i], l, sxl);
+                }
+                const double D = fms2(sw, sl2, sl, sl);
+                if (D > 1e-20) {
+                    s = (float)(fms2(sw, sxl, sx, sl) / D);
+                    m = (float)(fms2(sl2, sx, sl, sxl) / D);
+                }
+            };
+            for (int iter = 0; iter < 4; ++iter) assign_refit(m, s);
+            float best_s = s;
+            const float best_m = m;
+            double best = 1e300;
+            for (int k = -3; k <= 3; ++k) {
+                if (k == 0) continue;
+                const float cs = s * __builtin_fmaf(0.05f, (float)k, 1.0f);
+                double e = 0.0;
+                for (int i = 0; i < gsz; ++i) {
+                    const float l = unit_level(bits, unit_nearest_dev((x[i] - m) / cs, bits));
+                    const float d = __builtin_fmaf(cs, l, m) - x[i];
+                    e = __builtin_fma((double)d, (double)d, e);
+                }
+                if (e < best) { best = e; best_s = cs; }
+            }
+            s = best_s;
+            assign_refit(best_m, s);
+        }
+        s_[t] = s;
+        m_[t] = m;
+        sc_[t] = 0;
+        mc_[t] = 0;
+    }
+    __syncthreads();
+
+    // ---- global d / dm and the joint refinement
+    if (t == 0) {
+        float max_s = 0.0f, max_m = 0.0f;
+        for (int g = 0; g < ng; ++g) { max_s = fmaxf(max_s, fabsf(s_[g])); max_m = fmaxf(max_m, fabsf(m_[g])); }
+        float d = 1.0f, dm = 1.0f;
+        if (max_s <= eps) d = 0.0f;
+        else {
+            d = half_bits_to_float(float_to_half_bits(max_s / (float)scq));
+            if (max_m > eps) dm = half_bits_to_float(float_to_half_bits(max_m / (float)bias));
+        }
+        dd[0] = d;
+        dd[1] = (max_s <= eps) ? 1.0f : dm;
+        code[0] = (uint8_t)((max_s <= eps ? 1 : 0) | (max_m > eps ? 2 : 0));
+    }
+    __syncthreads();
+    const bool dead = (code[0] & 1) != 0;          // all scales vanish: d = 0, codes 0, dm stays 1
+    const bool have_min = (code[0] & 2) != 0;
+    __syncthreads();
+    auto snap_scale = [&](float s, float d) __attribute__((always_inline)) {
+        return (s == 0.0f) ? 0 : max(0, min(scq, (int)lroundf(s / d)));
+    };
+    auto snap_min = [&](float m, float dm) __attribute__((always_inline)) {
+        return max(-bias, min(mq - bias, (int)lroundf(-m / dm)));
+    };
+    if (!dead) {
+        if (t < ng) {
+            sc_[t] = snap_scale(s_[t], dd[0]);
+            if (have_min) mc_[t] = snap_min(m_[t], dd[1]);
+        }
+        __syncthreads();
+        for (int iter = 0; iter < 5; ++iter) {
+            const float d = dd[0], dm = dd[1];
+            if (t < ng) {
+                const float eff_s = d * (float)sc_[t];
+                const float eff_m = -dm * (float)mc_[t];
+                if (eff_s != 0.0f) {
+                    double sw = 0, sl = 0, sl2 = 0, sx = 0, sxl = 0;
+                    for (int i = 0; i < gsz; ++i) {
+                        const float l = unit_level(bits, unit_nearest_dev((x[i] - eff_m) / eff_s, bits));
+                        sw += 1.0; sl += l; sl2 += l * l;  // the square is a float product here, not fused
+                        sx += (double)x[i]; sxl = __builtin_fma((double)x[i], (double)l, sxl);
+                    }
+                    const double D = fms2(sw, sl2, sl, sl);
+                    if (D > 1e-20) {
+                        s_[t] = (float)(fms2(sw, sxl, sx, sl) / D);
+                        m_[t] = (float)(fms2(sl2, sx, sl, sxl) / D);
+                    }
+                }
+                sc_[t] = snap_scale(s_[t], d);
+            }
+            __syncthreads();
+            if (t == 0) {
+                double num = 0, den = 0;
+                for (int g = 0; g < ng; ++g) {
+                    num = __builtin_fma((double)s_[g], (double)sc_[g], num);
+                    den = __builtin_fma((double)sc_[g], (double)sc_[g], den);
+                }
+                float nd = (den > 1e-20) ? half_bits_to_float(float_to_half_bits((float)(num / den))) : 0.0f;
+                if (fabsf(nd) <= eps) nd = 0.0f;
+                dd[0] = nd;
+            }
+            if (t < ng) mc_[t] = (fabsf(dm) > eps) ? snap_min(m_[t], dm) : 0;
+            __syncthreads();
+            if (t == 0) {
+                double num2 = 0, den2 = 0;
+                for (int g = 0; g < ng; ++g) {
+                    num2 = __builtin_fma(-(double)m_[g], (double)mc_[g], num2);
+                    den2 = __builtin_fma((double)mc_[g], (double)mc_[g], den2);
+                }
+                float ndm = (den2 > 1e-20) ? half_bits_to_float(float_to_half_bits((float)(num2 / den2))) : 0.0f;
+                if (fabsf(ndm) <= eps) ndm = 0.0f;
+                dd[1] = ndm;
+            }
+            __syncthreads();
+        }
+    }
+    // ---- codes
+    const float d = dd[0], dm = dd[1];
+    if (t < ng) {
+        const float eff_s = d * (float)sc_[t];
+        const float eff_m = -dm * (float)mc_[t];
+        for (int i = 0; i < gsz; ++i)
+            code[t * gsz + i] = (eff_s == 0.0f) ? 0 : (uint8_t)unit_nearest_dev((x[i] - eff_m) / eff_s, bits);
+    }
+    __syncthreads();
+    // ---- payload: levels | scale codes | biased min codes | binary16 d | binary16 dm, one LSB-first stream
+    constexpr int lev_bits = 256 * bits, sc_end = lev_bits + ng * sp.scb, mn_end = sc_end + ng * sp.mb;
+    const uint32_t dh = float_to_half_bits(d) | (float_to_half_bits(dm) << 16);
+    uint8_t* p = dst + blk * (int64_t)sp.block_bytes;
+    for (int byte = t; byte < sp.block_bytes; byte += 64) {
+        uint32_t v = 0;
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const int pos = 8 * byte + b;
+            uint32_t bit;
+            if (pos < lev_bits) bit = ((uint32_t)code[pos / bits] >> (pos % bits)) & 1u;
+            else if (pos < sc_end) bit = ((uint32_t)sc_[(pos - lev_bits) / sp.scb] >> ((pos - lev_bits) % sp.scb)) & 1u;
+            else if (pos < mn_end) bit = ((uint32_t)(mc_[(pos - sc_end) / sp.mb] + bias) >> ((pos - sc_end) % sp.mb)) & 1u;
+            else bit = (dh >> (pos - mn_end)) & 1u;
+            v |= bit << b;
+        }
+        p[byte] = (uint8_t)v;
+    }
+}
+
 // Wire -> Tiled16: one lane per 16-byte piece of the tiled buffer.  Piece p of a unit: p < 64 code
 // slot of k-step 0, p < 128 of k-step 1, else a 16-byte part of a row header.  Codes narrower
 // than 4 bits are widened to nibbles.
@@ -248,6 +585,16 @@ bool block_layout(int fmt, int n, BlockLayout* L) {
                   (n >= 8 ? 1 : 0) | ((scales ? sc_count : 0) << 8)};
             return true;
         }
+        case Codec::Q1: *L = {BK_Q1, 1, n, (n + 7) / 8, 0, 0, 0, 0, 0}; return true;
+        case Codec::Q16: case Codec::Q24: {
+            // plain part, padded to the claim; the grouped ids fill the padding with residual means
+            // when the block is a whole number of 32-groups (src/codec/block_codec.cpp:2450-2493, :2836-2847)
+            const int plain = n * sp.bits / 8, claimed = (int)std::ceil((double)sp.bpw * (double)n / 8.0);
+            const bool residual = sp.scb == 1 && claimed > plain && n % 32 == 0;
+            *L = {BK_WIDE, sp.bits, n, claimed > plain ? claimed : plain, 0, 0, 0, 0,
+                  (residual ? 1 : 0) | (sp.bits == 16 && n == 256 ? 2 : 0)};
+            return true;
+        }
         case Codec::Sym32:
             if (n < 32 || n % 32) return false;
             *L = {BK_SYM32, sp.bits, n, n * sp.bits / 8 + (n / 32) * 2, 32, n / 32, 0, 0, 0};
@@ -266,6 +613,14 @@ int launch_decode(int fmt, const uint8_t* src, int64_t nblocks, float* out, hipS
     if (nblocks <= 0) return TFQ_OK;
     if (nblocks > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "decode: more than 2^31-1 blocks in one call");
     switch (canonical(fmt)) {
+        case TFQ_Q_1: return run_decode<TFQ_Q_1>(src, nblocks, out, s);
+        case TFQ_Q_1_5: return run_decode<TFQ_Q_1_5>(src, nblocks, out, s);
+        case TFQ_Q_16: return run_decode<TFQ_Q_16>(src, nblocks, out, s);
+        case TFQ_Q_16_5: return run_decode<TFQ_Q_16_5>(src, nblocks, out, s);
+        case TFQ_Q_G_16: return run_decode<TFQ_Q_G_16>(src, nblocks, out, s);
+        case TFQ_Q_24: return run_decode<TFQ_Q_24>(src, nblocks, out, s);
+        case TFQ_Q_24_5: return run_decode<TFQ_Q_24_5>(src, nblocks, out, s);
+        case TFQ_Q_G_24: return run_decode<TFQ_Q_G_24>(src, nblocks, out, s);
         case TFQ_Q_2: return run_decode<TFQ_Q_2>(src, nblocks, out, s);
         case TFQ_Q_G_6: return run_decode<TFQ_Q_G_6>(src, nblocks, out, s);
         case TFQ_Q_G_2_K_L: return run_decode<TFQ_Q_G_2_K_L>(src, nblocks, out, s);
@@ -346,6 +701,24 @@ int launch_encode(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStr
         case TFQ_Q_32: hipLaunchKernelGGL(encode_raw32_kernel, grid, block, 0, s, w, dst); break;
         case TFQ_B32S4: hipLaunchKernelGGL(encode_sym32_kernel<TFQ_B32S4>, grid, block, 0, s, w, dst); break;
         case TFQ_B32S8: hipLaunchKernelGGL(encode_sym32_kernel<TFQ_B32S8>, grid, block, 0, s, w, dst); break;
+        case TFQ_Q_G_4: hipLaunchKernelGGL(encode_affine_kernel<TFQ_Q_G_4>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_Q_G_3: hipLaunchKernelGGL(encode_affine_kernel<TFQ_Q_G_3>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_Q_G_2: hipLaunchKernelGGL(encode_affine_kernel<TFQ_Q_G_2>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_SB256A3: hipLaunchKernelGGL(encode_affine_kernel<TFQ_SB256A3>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_SB256A2: hipLaunchKernelGGL(encode_affine_kernel<TFQ_SB256A2>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_Q_1_5: hipLaunchKernelGGL(encode_affine_kernel<TFQ_Q_1_5>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_Q_24: hipLaunchKernelGGL(encode_wide_kernel<TFQ_Q_24>, grid, block, 0, s, w, dst); break;
+        case TFQ_Q_24_5: hipLaunchKernelGGL(encode_wide_kernel<TFQ_Q_24_5>, grid, block, 0, s, w, dst); break;
+        case TFQ_Q_G_24: hipLaunchKernelGGL(encode_wide_kernel<TFQ_Q_G_24>, grid, block, 0, s, w, dst); break;
+        case TFQ_Q_16: hipLaunchKernelGGL(encode_wide_kernel<TFQ_Q_16>, grid, block, 0, s, w, dst); break;
+        case TFQ_Q_16_5: hipLaunchKernelGGL(encode_wide_kernel<TFQ_Q_16_5>, grid, block, 0, s, w, dst); break;
+        case TFQ_Q_G_16: hipLaunchKernelGGL(encode_wide_kernel<TFQ_Q_G_16>, grid, block, 0, s, w, dst); break;
+        case TFQ_Q_1: {
+            const int tier = fmt == TFQ_Q_1 ? -1 : (fmt == TFQ_Q_1_K_M || fmt == TFQ_Q_G_1_K_M) ? 1
+                             : (fmt == TFQ_Q_1_K_H || fmt == TFQ_Q_G_1_K_H) ? 2 : 0;
+            hipLaunchKernelGGL(encode_q1_kernel, grid, block, 0, s, w, dst, tier);
+            break;
+        }
         default:
             return fail(TFQ_ERR_FORMAT, "encode: wire id " + std::to_string(fmt) +
                                             " has no device encoder in this build");

@@ -101,6 +101,25 @@ __device__ __forceinline__ float decode_weight(const uint8_t* __restrict__ p, ui
         const float d = half_bits_to_float((uint32_t)p[208] | ((uint32_t)p[209] << 8));
         v = (d * sc) * (float)((int)code - 32);
         v = v + 0.0f;  // the reference computes e * level + 0 here: never -0
+    } else if constexpr (sp.codec == Codec::Q1) {
+        // [binary16 scale][240 sign bits]; weights 15, 31, ... carry no bit and are zero
+        const float scale = half_bits_to_float(stream_bits(p, BB, 0, 16));
+        if ((i & 15u) == 15u) v = 0.0f;
+        else v = stream_bits(p, BB, 16u + i - (i >> 4), 1) ? scale : -scale;
+    } else if constexpr (sp.codec == Codec::Q16) {
+        const float vmin = __uint_as_float(stream_bits(p, BB, 0, 16) | (stream_bits(p, BB, 16, 16) << 16));
+        const float vmax = __uint_as_float(stream_bits(p, BB, 32, 16) | (stream_bits(p, BB, 48, 16) << 16));
+        const float range = vmax - vmin;
+        const bool narrow = (i & 3u) == 3u;  // the fourth code of a group has 15 bits
+        const float scale = range > 0 ? range / (narrow ? 32767.0f : 65535.0f) : 0.0f;
+        const uint32_t qv = stream_bits(p, 8 + 504, 64u + 63u * (i >> 2) + 16u * (i & 3u), narrow ? 15 : 16);
+        v = __builtin_fmaf((float)qv, scale, vmin);  // fused in the reference's Release build
+        if constexpr (sp.scb == 1 && sp.block_bytes > 512)
+            v += half_bits_to_float((uint32_t)p[512 + 2 * (i >> 5)] | ((uint32_t)p[512 + 2 * (i >> 5) + 1] << 8));
+    } else if constexpr (sp.codec == Codec::Q24) {
+        v = __uint_as_float(((uint32_t)p[3 * i] << 8) | ((uint32_t)p[3 * i + 1] << 16) | ((uint32_t)p[3 * i + 2] << 24));
+        if constexpr (sp.scb == 1 && sp.block_bytes > 768)
+            v += half_bits_to_float((uint32_t)p[768 + 2 * (i >> 5)] | ((uint32_t)p[768 + 2 * (i >> 5) + 1] << 8));
     } else if constexpr (sp.codec == Codec::Sym32) {
         constexpr uint32_t code_bytes = 256u * sp.bits / 8;
         const uint32_t g = i >> 5;
@@ -239,6 +258,31 @@ __device__ __forceinline__ float decode_weight_short(const BlockLayout& L, const
         case BK_GRP8: {
             const uint32_t h = (uint32_t)p[n + 2 * (i >> 5)] | ((uint32_t)p[n + 2 * (i >> 5) + 1] << 8);
             return half_bits_to_float(h) * __uint_as_float(kComp8Bits[p[i]]);
+        }
+        case BK_Q1: {
+            if (n < 32) return stream_bits(p, size, i, 1) ? 1.0f : -1.0f;  // sign bits only
+            const uint32_t before = (i * 16u) / n;
+            if (((i + 1u) * 16u) / n != before) return 0.0f;
+            const float scale = half_bits_to_float(stream_bits(p, size, 0, 16));
+            return stream_bits(p, size, 16u + i - before, 1) ? scale : -scale;
+        }
+        case BK_WIDE: {
+            const uint32_t plain = n * (bits / 8);
+            float v;
+            if (bits == 24) {
+                v = __uint_as_float(((uint32_t)p[3 * i] << 8) | ((uint32_t)p[3 * i + 1] << 16) | ((uint32_t)p[3 * i + 2] << 24));
+            } else if (L.aux & 2) {  // 256 weights: min, max, groups of 63 bits
+                const float vmin = __uint_as_float(stream_bits(p, plain, 0, 16) | (stream_bits(p, plain, 16, 16) << 16));
+                const float vmax = __uint_as_float(stream_bits(p, plain, 32, 16) | (stream_bits(p, plain, 48, 16) << 16));
+                const float range = vmax - vmin;
+                const bool narrow = (i & 3u) == 3u;
+                const float scale = range > 0 ? range / (narrow ? 32767.0f : 65535.0f) : 0.0f;
+                v = __builtin_fmaf((float)stream_bits(p, plain, 64u + 63u * (i >> 2) + 16u * (i & 3u), narrow ? 15 : 16), scale, vmin);
+            } else {  // fewer than 256 weights: raw binary16
+                v = half_bits_to_float((uint32_t)p[2 * i] | ((uint32_t)p[2 * i + 1] << 8));
+            }
+            if (L.aux & 1) v += half_bits_to_float((uint32_t)p[plain + 2 * (i >> 5)] | ((uint32_t)p[plain + 2 * (i >> 5) + 1] << 8));
+            return v;
         }
         default: {  // BK_SYM32
             const uint32_t code_bytes = n * bits / 8;

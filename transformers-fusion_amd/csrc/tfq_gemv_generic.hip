@@ -121,6 +121,14 @@ int launch_gemv_generic(const tfq_weight* w, const void* x, int x_dtype, int B, 
     if (w->N > 0x7FFFFFFF || w->K > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "gemv: shape too large");
     switch (canonical(w->fmt)) {
         case TFQ_Q_32: return batched<TFQ_Q_32>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_1: return batched<TFQ_Q_1>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_1_5: return batched<TFQ_Q_1_5>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_16: return batched<TFQ_Q_16>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_16_5: return batched<TFQ_Q_16_5>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_G_16: return batched<TFQ_Q_G_16>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_24: return batched<TFQ_Q_24>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_24_5: return batched<TFQ_Q_24_5>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_G_24: return batched<TFQ_Q_G_24>(w, x, x_dtype, B, y, y_dtype, s);
         case TFQ_Q_2: return batched<TFQ_Q_2>(w, x, x_dtype, B, y, y_dtype, s);
         case TFQ_Q_G_6: return batched<TFQ_Q_G_6>(w, x, x_dtype, B, y, y_dtype, s);
         case TFQ_Q_G_2_K_L: return batched<TFQ_Q_G_2_K_L>(w, x, x_dtype, B, y, y_dtype, s);

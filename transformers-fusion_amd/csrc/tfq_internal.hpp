@@ -13,7 +13,7 @@
 namespace tfq {
 
 // ------------------------------------------------------------------ formats
-enum class Codec : int { None = 0, Raw32, Lattice, Affine, Grp8, Sym32, Grp16, Q6K };
+enum class Codec : int { None = 0, Raw32, Lattice, Affine, Grp8, Sym32, Grp16, Q6K, Q1, Q16, Q24 };
 
 // Layout parameters of one wire format.  The affine family is the reference's
 // parametric codec quant_affine(bits, w, n, gsz, scb, mb, claimed)
@@ -33,10 +33,25 @@ struct Spec {
 // a 3-bit scale code each, one binary16 d.  The ids that claim 1/16 bit less than the
 // affine layout needs (Q_G_{2,3,4}_K_*, Q_2_5, Q_6_5) use it for every block.
 // Q6K is Q_G_6 (quant_6k / dequant_6k, :1046-1303): 6-bit levels, int8 scale per 16.
+// Q1: binary16 scale + one sign bit per weight, every 16th weight decodes to zero (:1526-1618).
+// Q16: binary32 min and max, then per four weights 16 + 16 + 16 + 15 bits of uniform code (:1690-1807).
+// Q24: the top three bytes of the binary32 (:1809-1873).  For Q16 / Q24, scb = 1 marks the ids that
+// append a binary16 residual mean per 32 weights when the claimed size leaves room.
 
 __host__ __device__ constexpr Spec spec_of(int fmt) {
     switch (fmt) {
         case TFQ_Q_32: return {Codec::Raw32, 32, 0, 0, 0, 32.0f, 1024};
+        case TFQ_Q_1: case TFQ_Q_1_K_L: case TFQ_Q_1_K_M: case TFQ_Q_1_K_H:
+        case TFQ_Q_G_1: case TFQ_Q_G_1_K_L: case TFQ_Q_G_1_K_M: case TFQ_Q_G_1_K_H: return {Codec::Q1, 1, 0, 0, 0, 1.0f, 32};
+        case TFQ_Q_1_5: case TFQ_Q_G_1_5: return {Codec::Affine, 1, 32, 6, 6, 1.5f, 48};
+        case TFQ_Q_16: case TFQ_Q_16_K_L: case TFQ_Q_16_K_M: case TFQ_Q_16_K_H: return {Codec::Q16, 16, 0, 0, 0, 16.0f, 512};
+        case TFQ_Q_16_5: case TFQ_Q_G_16_5: return {Codec::Q16, 16, 0, 0, 0, 16.5f, 528};
+        case TFQ_Q_G_16: return {Codec::Q16, 16, 0, 1, 0, 16.5f, 528};
+        case TFQ_Q_G_16_K_L: case TFQ_Q_G_16_K_M: case TFQ_Q_G_16_K_H: return {Codec::Q16, 16, 0, 1, 0, 16.0f, 512};
+        case TFQ_Q_24: case TFQ_Q_24_K_L: case TFQ_Q_24_K_M: case TFQ_Q_24_K_H: return {Codec::Q24, 24, 0, 0, 0, 24.0f, 768};
+        case TFQ_Q_24_5: case TFQ_Q_G_24_5: return {Codec::Q24, 24, 0, 0, 0, 24.5f, 784};
+        case TFQ_Q_G_24: return {Codec::Q24, 24, 0, 1, 0, 24.5f, 784};
+        case TFQ_Q_G_24_K_L: case TFQ_Q_G_24_K_M: case TFQ_Q_G_24_K_H: return {Codec::Q24, 24, 0, 1, 0, 24.0f, 768};
         case TFQ_Q_2: return {Codec::Lattice, 2, 0, 0, 0, 2.0f, 64};
         case TFQ_Q_4: return {Codec::Lattice, 4, 0, 0, 0, 4.0f, 128};
         case TFQ_Q_8: return {Codec::Lattice, 8, 0, 0, 0, 8.0f, 256};
@@ -72,6 +87,15 @@ __host__ __device__ constexpr int canonical(int fmt) {
         case TFQ_Q_G_3_K_M: case TFQ_Q_G_3_K_H: return TFQ_Q_G_3_K_L;
         case TFQ_Q_G_4_K_M: case TFQ_Q_G_4_K_H: return TFQ_Q_G_4_K_L;
         case TFQ_Q_G_6_5: return TFQ_Q_6_5;
+        case TFQ_Q_1_K_L: case TFQ_Q_1_K_M: case TFQ_Q_1_K_H:
+        case TFQ_Q_G_1: case TFQ_Q_G_1_K_L: case TFQ_Q_G_1_K_M: case TFQ_Q_G_1_K_H: return TFQ_Q_1;
+        case TFQ_Q_G_1_5: return TFQ_Q_1_5;
+        case TFQ_Q_16_K_L: case TFQ_Q_16_K_M: case TFQ_Q_16_K_H:
+        case TFQ_Q_G_16_K_L: case TFQ_Q_G_16_K_M: case TFQ_Q_G_16_K_H: return TFQ_Q_16;  // a claim of 16 bits leaves no room for residuals
+        case TFQ_Q_G_16_5: return TFQ_Q_16_5;
+        case TFQ_Q_24_K_L: case TFQ_Q_24_K_M: case TFQ_Q_24_K_H:
+        case TFQ_Q_G_24_K_L: case TFQ_Q_G_24_K_M: case TFQ_Q_G_24_K_H: return TFQ_Q_24;
+        case TFQ_Q_G_24_5: return TFQ_Q_24_5;
         default: return fmt;
     }
 }
@@ -143,14 +167,15 @@ namespace tfq {
 // Layout of one block of n <= 256 weights, as the reference's codecs choose it from
 // (format, n): short blocks drop or shrink their headers.  Filled on the host, passed
 // to the short-block decode kernel by value.
-enum : int { BK_RAW32 = 0, BK_LEVELS, BK_LATTICE, BK_AFFINE, BK_GRP16, BK_Q6K, BK_GRP8, BK_SYM32 };
+enum : int { BK_RAW32 = 0, BK_LEVELS, BK_LATTICE, BK_AFFINE, BK_GRP16, BK_Q6K, BK_GRP8, BK_SYM32, BK_Q1, BK_WIDE };
 struct BlockLayout {
     int kind;
     int bits;   // code width
     int n;      // weights in the block
     int bytes;  // payload bytes
     int gsz, ng, scb, mb;  // affine: group size, group count, scale / min code widths
-    int aux;    // BK_GRP16: 0 raw levels, 1 one d, 2 group scales + d.  BK_Q6K: bit 0 d present, bits 8.. stored scale count
+    int aux;    // BK_GRP16: 0 raw levels, 1 one d, 2 group scales + d.  BK_Q6K: bit 0 d present, bits 8.. stored scale count.
+                // BK_WIDE: bit 0 residual means follow the plain part, bit 1 packed 16-bit layout (else raw binary16 / 24-bit)
 };
 // false when the format cannot hold a block of n weights
 bool block_layout(int fmt, int n, BlockLayout* out);
