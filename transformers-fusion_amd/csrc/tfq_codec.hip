@@ -420,6 +420,525 @@ __global__ __launch_bounds__(64) void encode_affine_kernel(const float* __restri
     }
 }
 
+// Companded 8-bit encoders: Q_G_8 (quant_grp8_compound, src/codec/block_codec.cpp:365-388, a scale per 32
+// weights) and Q_8 (quant_lattice with bits = 8, :458-470, one scale per block, 7-bit slots), both on
+// comp8_fit_scale_fp16 (:306-358): three least-squares seeds, 14 golden-section steps on the true squared
+// error over [0.75 s, 1.25 s], then the +-4 neighbouring binary16 values.  One wavefront per scale group.
+// Every evaluation is split so that the result is the reference's: the lanes do the per-weight part in
+// parallel (nearest level by bisection, residual r = level * s - w as one fused multiply-add in double),
+// lane 0 then adds r * r in index order with the same fused operations the reference's Release build uses.
+// The search state lives in every lane (all decisions come from values lane 0 publishes).
+template <int CNT>
+struct Comp8Team {
+    float* lv;       // 256 levels, LDS
+    double* buf;     // 2 * CNT doubles, LDS
+    double* res;     // 2 doubles, LDS
+    const float* w;  // this group's weights, LDS
+    int lane;
+    static constexpr int PER = CNT / 64 ? CNT / 64 : 1;  // weights per lane
+    __device__ __forceinline__ bool mine(int k, int* i) const { *i = lane * PER + k; return *i < CNT; }
+    __device__ __forceinline__ uint32_t nearest(float v) const {
+        if (v <= lv[0]) return 0;
+        if (v >= lv[255]) return 255;
+        int lo = 0, hi = 255;
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) / 2;
+            if (lv[mid] <= v) lo = mid; else hi = mid;
+        }
+        return (v - lv[lo] <= lv[hi] - v) ? (uint32_t)lo : (uint32_t)hi;
+    }
+    __device__ double sq_err(double s) const {
+        const double inv = 1.0 / s;
+        for (int k = 0; k < PER; ++k) {
+            int i;
+            if (mine(k, &i)) buf[i] = __builtin_fma((double)lv[nearest((float)((double)w[i] * inv))], s, -(double)w[i]);
+        }
+        __syncthreads();
+        if (lane == 0) {
+            double err = 0.0;
+            for (int i = 0; i < CNT; ++i) err = __builtin_fma(buf[i], buf[i], err);
+            res[0] = err;
+        }
+        __syncthreads();
+        const double e = res[0];
+        __syncthreads();
+        return e;
+    }
+    // false when the refit has no support (den <= 1e-20)
+    __device__ bool seed(double s, double* out) const {
+        for (int k = 0; k < PER; ++k) {
+            int i;
+            if (mine(k, &i)) buf[i] = (double)lv[nearest((float)((double)w[i] / s))];
+        }
+        __syncthreads();
+        if (lane == 0) {
+            double num = 0.0, den = 0.0;
+            for (int i = 0; i < CNT; ++i) {
+                num = __builtin_fma((double)w[i], buf[i], num);
+                den = __builtin_fma(buf[i], buf[i], den);
+            }
+            res[0] = num;
+            res[1] = den;
+        }
+        __syncthreads();
+        const double num = res[0], den = res[1];
+        __syncthreads();
+        if (!(den > 1e-20)) return false;
+        *out = num / den;
+        return true;
+    }
+    __device__ float fit(double maxa) const {
+        if (!(maxa > 0.0)) return 0.0f;
+        const double hi = maxa * 1.0000001;
+        double s = maxa;
+        for (int it = 0; it < 3; ++it) {
+            double ls;
+            if (!seed(s, &ls)) break;
+            s = ls < hi ? ls : hi;
+        }
+        double a = s * 0.75, b = s * 1.25;
+        const double phi = 0.6180339887498949;
+        double c = __builtin_fma(-phi, b - a, b), d = __builtin_fma(phi, b - a, a);
+        double fc = sq_err(c), fd = sq_err(d);
+        for (int it = 0; it < 14 && (b - a) > 1e-11 * (a + b); ++it) {
+            if (fc < fd) {
+                b = d; d = c; fd = fc;
+                c = __builtin_fma(-phi, b - a, b); fc = sq_err(c);
+            } else {
+                a = c; c = d; fc = fd;
+                d = __builtin_fma(phi, b - a, a); fd = sq_err(d);
+            }
+        }
+        double raw = 0.5 * (a + b);
+        const double fraw = sq_err(raw);
+        if (fraw > fc && fc <= fd) raw = c;
+        else if (fraw > fd) raw = d;
+        const uint32_t hf = float_to_half_bits((float)raw);
+        float best = half_bits_to_float(hf);
+        double best_e = sq_err((double)best);
+        for (int delta = -4; delta <= 4; ++delta) {
+            if (delta == 0) continue;
+            const int hc = (int)hf + delta;
+            if (hc < 0 || hc > 0xFFFF) continue;
+            const float cand = half_bits_to_float((uint32_t)hc);
+            if (!(cand > 0.0f) || !((double)cand <= hi * 1.02)) continue;
+            const double e = sq_err((double)cand);
+            if (e < best_e) { best_e = e; best = cand; }
+        }
+        return best;
+    }
+};
+
+// FMT = Q_G_8: grid = 8 groups per block, a wavefront each (32 lanes hold a weight).  FMT = Q_8: a wavefront
+// per block, four weights per lane.
+template <int FMT>
+__global__ __launch_bounds__(64) void encode_comp8_kernel(const float* __restrict__ wg, uint8_t* __restrict__ dst) {
+    constexpr bool GROUPED = spec_of(FMT).codec == Codec::Grp8;
+    constexpr int CNT = GROUPED ? 32 : 256;
+    __shared__ float lv[256];
+    __shared__ float w[CNT];
+    __shared__ double buf[CNT];
+    __shared__ double res[2];
+    __shared__ uint8_t code[CNT];
+    const int lane = threadIdx.x;
+    const int64_t unit = blockIdx.x;  // group or block
+    for (int i = lane; i < 256; i += 64) lv[i] = __uint_as_float(kComp8Bits[i]);
+    for (int i = lane; i < CNT; i += 64) w[i] = wg[unit * CNT + i];
+    __syncthreads();
+    float m = 0.0f;
+    for (int i = lane; i < CNT; i += 64) m = fmaxf(m, fabsf(w[i]));
+#pragma unroll
+    for (int sft = 32; sft >= 1; sft >>= 1) m = fmaxf(m, __shfl_xor(m, sft, 64));
+    Comp8Team<CNT> team{lv, buf, res, w, lane};
+    const float s = team.fit((double)m);
+    for (int i = lane; i < CNT; i += 64) code[i] = (uint8_t)((s > 0.0f) ? team.nearest(w[i] / s) : 0u);
+    __syncthreads();
+    const uint32_t h = float_to_half_bits(s);
+    if constexpr (GROUPED) {
+        uint8_t* p = dst + (unit >> 3) * 272;
+        const int g = (int)(unit & 7);
+        if (lane < 32) p[32 * g + lane] = code[lane];
+        if (lane == 0) { p[256 + 2 * g] = (uint8_t)(h & 0xFF); p[257 + 2 * g] = (uint8_t)(h >> 8); }
+    } else {
+        // [binary16 scale][256 codes, every 16th with 7 bits (the even index below it)]: 16 + 16 * 127 bits
+        uint8_t* p = dst + unit * 256;
+        for (int byte = lane; byte < 256; byte += 64) {
+            uint32_t v = 0;
+#pragma unroll
+            for (int b = 0; b < 8; ++b) {
+                const int pos = 8 * byte + b;
+                uint32_t bit;
+                if (pos < 16) bit = (h >> pos) & 1u;
+                else {
+                    const int q = pos - 16, c = q / 127, r = q - 127 * c;
+                    const int k = r / 8 < 15 ? r / 8 : 15, off = r - 8 * k;
+                    const uint32_t idx = code[16 * c + k];
+                    bit = ((k == 15 ? idx >> 1 : idx) >> off) & 1u;
+                }
+                v |= bit << b;
+            }
+            p[byte] = (uint8_t)v;
+        }
+    }
+}
+
+// Plain lattice encoders Q_4 / Q_2 (quant_lattice, src/codec/block_codec.cpp:443-497): s = absmax / top level,
+// two least-squares refits over the nearest levels, binary16; codes are the nearest level of w / s, slots
+// (every 16th weight) keep the even index below.  A wavefront per block; sums in index order on lane 0.
+template <int FMT>
+__global__ __launch_bounds__(64) void encode_lattice_kernel(const float* __restrict__ wg, uint8_t* __restrict__ dst) {
+    constexpr int bits = spec_of(FMT).bits, BB = spec_of(FMT).block_bytes, CHUNK = 16 * bits - 1;
+    __shared__ float w[256];
+    __shared__ float lev[256];
+    __shared__ float sres;
+    __shared__ uint8_t code[256];
+    const int lane = threadIdx.x;
+    const int64_t blk = blockIdx.x;
+    for (int i = lane; i < 256; i += 64) w[i] = wg[blk * 256 + i];
+    __syncthreads();
+    float m = 0.0f;
+    for (int i = lane; i < 256; i += 64) m = fmaxf(m, fabsf(w[i]));
+#pragma unroll
+    for (int sft = 32; sft >= 1; sft >>= 1) m = fmaxf(m, __shfl_xor(m, sft, 64));
+    auto nearest = [&](float v) __attribute__((always_inline)) {
+        uint32_t best = 0;
+        float bd = fabsf(v - grid_value(bits, 0));
+        for (int i = 1; i < (1 << bits); ++i) {
+            const float d = fabsf(v - grid_value(bits, (uint32_t)i));
+            if (d < bd) { bd = d; best = (uint32_t)i; }
+        }
+        return best;
+    };
+    float s = (m > 1e-30f) ? m / (bits == 2 ? 1.5104f : 2.7178f) : 0.0f;
+    if (s > 0.0f) {
+        for (int it = 0; it < 2; ++it) {
+            for (int i = lane; i < 256; i += 64) lev[i] = grid_value(bits, nearest(w[i] / s));
+            __syncthreads();
+            if (lane == 0) {
+                double num = 0.0, den = 0.0;
+                for (int i = 0; i < 256; ++i) {
+                    num = __builtin_fma((double)w[i], (double)lev[i], num);
+                    den = __builtin_fma((double)lev[i], (double)lev[i], den);
+                }
+                sres = (den > 1e-20) ? (float)(num / den) : s;
+            }
+            __syncthreads();
+            s = sres;
+            __syncthreads();
+        }
+    }
+    if (!(s > 0.0f)) s = 0.0f;
+    for (int i = lane; i < 256; i += 64) code[i] = (uint8_t)nearest((s == 0.0f) ? 0.0f : w[i] / s);
+    __syncthreads();
+    const uint32_t h = float_to_half_bits(s);
+    uint8_t* p = dst + blk * BB;
+    for (int byte = lane; byte < BB; byte += 64) {
+        uint32_t v = 0;
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const int pos = 8 * byte + b;
+            uint32_t bit;
+            if (pos < 16) bit = (h >> pos) & 1u;
+            else {
+                const int q = pos - 16, c = q / CHUNK, r = q - CHUNK * c;
+                const int k = r / bits < 15 ? r / bits : 15, off = r - bits * k;
+                const uint32_t idx = code[16 * c + k];
+                bit = ((k == 15 ? idx >> 1 : idx) >> off) & 1u;
+            }
+            v |= bit << b;
+        }
+        p[byte] = (uint8_t)v;
+    }
+}
+
+// Grouped-lattice fallback encoder (quant_grp16 with grp16_fit_scale, src/codec/block_codec.cpp:739-914) for
+// the ids that use that layout for full blocks, and the Q_G_6 encoder (quant_6k, :1070-1238).  Same shape as
+// the affine encoder: a wavefront per block, lane g owns group g (32 groups of 8, or 16 groups of 16), lane 0
+// the sums over groups; fused operations where GCC's Release build fuses.
+template <int FMT>
+__global__ __launch_bounds__(64) void encode_grp16_kernel(const float* __restrict__ wg, uint8_t* __restrict__ dst) {
+    constexpr Spec sp = spec_of(FMT);
+    constexpr int bits = sp.bits, ng = 32;
+    constexpr float eps = 1e-15f;
+    constexpr float top_level = bits == 2 ? 1.5104f : bits == 4 ? 2.7178f : 8.0f;
+    __shared__ float w[256];
+    __shared__ float s_[32];
+    __shared__ int sc_[32];
+    __shared__ float dsh;
+    __shared__ uint8_t code[256];
+    const int64_t blk = blockIdx.x;
+    const int t = threadIdx.x;
+    for (int i = t; i < 256; i += 64) w[i] = wg[blk * 256 + i];
+    __syncthreads();
+    const float* x = w + (t & 31) * 8;
+    auto nearest = [&](float v) __attribute__((always_inline)) -> uint32_t {
+        if constexpr (bits == 2 || bits == 4) {
+            uint32_t best = 0;
+            float bd = fabsf(v - grid_value(bits, 0));
+            for (int i = 1; i < (1 << bits); ++i) {
+                const float d = fabsf(v - grid_value(bits, (uint32_t)i));
+                if (d < bd) { bd = d; best = (uint32_t)i; }
+            }
+            return best;
+        } else {
+            constexpr float top = (float)((1u << bits) - 1u);
+            const float c = fmaxf(-8.0f, fminf(8.0f, v));
+            return (uint32_t)lroundf((c + 8.0f) * top / 16.0f);
+        }
+    };
+    if (t < ng) {
+        float maxa = 0.0f;
+        for (int i = 0; i < 8; ++i) maxa = fmaxf(maxa, fabsf(x[i]));
+        float s = (maxa > 1e-30f) ? maxa / top_level : 0.0f;
+        if (!(fabsf(s) > 1e-30f)) s = 0.0f;
+        else {
+            auto assign_refit = [&](float as) __attribute__((always_inline)) {
+                double num = 0.0, den = 0.0;
+                for (int i = 0; i < 8; ++i) {
+                    const float l = grid_value(bits, nearest(x[i] / as));
+                    num = __builtin_fma((double)x[i], (double)l, num);
+                    den = __builtin_fma((double)l, (double)l, den);
+                }
+                if (den > 1e-20) s = (float)(num / den);
+            };
+            for (int iter = 0; iter < 4; ++iter) assign_refit(s);
+            float best_s = s;
+            double best = 1e300;
+            for (int k = -3; k <= 3; ++k) {
+                if (k == 0) continue;
+                const float cs = s * __builtin_fmaf(0.05f, (float)k, 1.0f);
+                double e = 0.0;
+                for (int i = 0; i < 8; ++i) {
+                    const float l = grid_value(bits, nearest(x[i] / cs));
+                    const float d = __builtin_fmaf(cs, l, -x[i]);
+                    e = __builtin_fma((double)d, (double)d, e);
+                }
+                if (e < best) { best = e; best_s = cs; }
+            }
+            s = best_s;
+            assign_refit(s);
+        }
+        s_[t] = s;
+        sc_[t] = 0;
+    }
+    __syncthreads();
+    if (t == 0) {
+        float max_abs = 0.0f;
+        for (int g = 0; g < ng; ++g) max_abs = fmaxf(max_abs, fabsf(s_[g]));
+        dsh = (max_abs <= eps) ? 0.0f : half_bits_to_float(float_to_half_bits(max_abs / 7.0f));
+    }
+    __syncthreads();
+    // once d has collapsed to zero the reference's (int)lround(s / 0) comes out as 0 after its clamp
+    auto snap = [&](float s, float d) __attribute__((always_inline)) {
+        return (s == 0.0f || d == 0.0f) ? 0 : max(0, min(7, (int)lroundf(s / d)));
+    };
+    if (dsh != 0.0f) {  // an all-zero block keeps d = 0 and every code 0
+        if (t < ng) sc_[t] = snap(s_[t], dsh);
+        __syncthreads();
+        for (int iter = 0; iter < 5; ++iter) {
+            const float d = dsh;
+            if (t < ng) {
+                const float eff = d * (float)sc_[t];
+                if (eff != 0.0f) {
+                    double num = 0.0, den = 0.0;
+                    for (int i = 0; i < 8; ++i) {
+                        const float l = grid_value(bits, nearest(x[i] / eff));
+                        num = __builtin_fma((double)x[i], (double)l, num);
+                        den = __builtin_fma((double)l, (double)l, den);
+                    }
+                    s_[t] = (den > 1e-20) ? (float)(num / den) : 0.0f;
+                }
+                sc_[t] = snap(s_[t], d);
+            }
+            __syncthreads();
+            if (t == 0) {
+                double num = 0.0, den = 0.0;
+                for (int g = 0; g < ng; ++g) {
+                    num = __builtin_fma((double)s_[g], (double)sc_[g], num);
+                    den = __builtin_fma((double)sc_[g], (double)sc_[g], den);
+                }
+                float nd = (den > 1e-20) ? (float)(num / den) : 0.0f;
+                nd = half_bits_to_float(float_to_half_bits(nd));
+                if (fabsf(nd) <= eps) nd = 0.0f;
+                dsh = nd;
+            }
+            __syncthreads();
+        }
+    }
+    const float d = dsh;
+    if (t < ng) {
+        const float eff = d * (float)sc_[t];
+        for (int i = 0; i < 8; ++i) code[t * 8 + i] = (eff == 0.0f) ? 0 : (uint8_t)nearest(x[i] / eff);
+    }
+    __syncthreads();
+    constexpr int lev_bits = 256 * bits, sc_end = lev_bits + 96;
+    const uint32_t dh = float_to_half_bits(d);
+    uint8_t* p = dst + blk * (int64_t)sp.block_bytes;
+    for (int byte = t; byte < sp.block_bytes; byte += 64) {
+        uint32_t v = 0;
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const int pos = 8 * byte + b;
+            uint32_t bit;
+            if (pos < lev_bits) bit = ((uint32_t)code[pos / bits] >> (pos % bits)) & 1u;
+            else if (pos < sc_end) bit = ((uint32_t)sc_[(pos - lev_bits) / 3] >> ((pos - lev_bits) % 3)) & 1u;
+            else bit = (dh >> (pos - sc_end)) & 1u;
+            v |= bit << b;
+        }
+        p[byte] = (uint8_t)v;
+    }
+}
+
+__device__ __forceinline__ int q6k_round_dev(float v) {  // round to nearest even through the 1.5 * 2^23 bias
+    return (int)(__float_as_uint(v + 12582912.f) & 0x007fffffu) - 0x00400000;
+}
+__device__ __forceinline__ int q6k_level_dev(float ratio) {
+    ratio = fmaxf(-4000.0f, fminf(4000.0f, ratio));
+    return max(-32, min(31, q6k_round_dev(ratio)));
+}
+
+// passes / giters / polish / joint: the search effort (2, 4, 3, 3 for Q_G_6 and _K_L)
+__global__ __launch_bounds__(64) void encode_q6k_kernel(const float* __restrict__ wg, uint8_t* __restrict__ dst,
+                                                        int giters, int polish, int joint) {
+    constexpr int ng = 16;
+    constexpr float eps = 1e-15f;
+    __shared__ float w[256];
+    __shared__ float s_[16];
+    __shared__ int sc_[16];
+    __shared__ float dsh;
+    __shared__ uint8_t code[256];
+    const int64_t blk = blockIdx.x;
+    const int t = threadIdx.x;
+    for (int i = t; i < 256; i += 64) w[i] = wg[blk * 256 + i];
+    __syncthreads();
+    const float* x = w + (t & 15) * 16;
+    auto refit16 = [&](float scale, float* out) __attribute__((always_inline)) {
+        double num = 0.0, den = 0.0;
+        for (int i = 0; i < 16; ++i) {
+            const int l = q6k_level_dev(x[i] / scale);
+            num = __builtin_fma((double)x[i], (double)l, num);
+            den = __builtin_fma((double)l, (double)l, den);
+        }
+        if (den > 1e-20) *out = (float)(num / den);
+    };
+    if (t < ng) {
+        float maxa = 0.0f;
+        for (int i = 0; i < 16; ++i) maxa = fmaxf(maxa, fabsf(x[i]));
+        float sg = (maxa > eps) ? maxa / 32.0f : 0.0f;
+        if (fabsf(sg) <= eps) sg = 0.0f;
+        else {
+            for (int iter = 0; iter < giters; ++iter) refit16(sg, &sg);
+            float best_s = sg;
+            double best = 1e300;
+            for (int k = -polish; k <= polish; ++k) {
+                if (k == 0) continue;
+                const float cs = sg * __builtin_fmaf(0.05f, (float)k, 1.0f);
+                double e = 0.0;
+                for (int i = 0; i < 16; ++i) {
+                    const float d = __builtin_fmaf(cs, (float)q6k_level_dev(x[i] / cs), -x[i]);
+                    e = __builtin_fma((double)d, (double)d, e);
+                }
+                if (e < best) { best = e; best_s = cs; }
+            }
+            sg = best_s;
+            refit16(sg, &sg);
+        }
+        s_[t] = sg;
+        sc_[t] = 0;
+    }
+    __syncthreads();
+    float max_abs = 0.0f;
+    for (int g = 0; g < ng; ++g) max_abs = fmaxf(max_abs, fabsf(s_[g]));
+    if (max_abs <= eps) {
+        if (t == 0) dsh = 0.0f;
+        __syncthreads();
+    } else {
+        const float iscale = -128.0f / max_abs;
+        if (t == 0) dsh = 1.0f / iscale;
+        // the product feeds the rounding add directly: one fused operation in the reference's build
+        if (t < ng) sc_[t] = max(-127, min(127, (int)(__float_as_uint(__builtin_fmaf(iscale, s_[t], 12582912.f)) & 0x007fffffu) - 0x00400000));
+        __syncthreads();
+        for (int iter = 0; iter < joint; ++iter) {
+            const float d = dsh;
+            if (t < ng) {
+                const float eff = d * (float)sc_[t];
+                if (eff != 0.0f) {
+                    float fitted = 0.0f;
+                    refit16(eff, &fitted);
+                    s_[t] = fitted;
+                }
+                sc_[t] = (d == 0.0f) ? 0 : max(-127, min(127, q6k_round_dev(s_[t] / d)));
+            }
+            __syncthreads();
+            if (t == 0) {
+                double num = 0.0, den = 0.0;
+                for (int g = 0; g < ng; ++g) {
+                    num = __builtin_fma((double)s_[g], (double)sc_[g], num);
+                    den = __builtin_fma((double)sc_[g], (double)sc_[g], den);
+                }
+                float nd = (den > 1e-20) ? (float)(num / den) : 0.0f;
+                if (fabsf(nd) <= eps) nd = 0.0f;
+                dsh = nd;
+            }
+            __syncthreads();
+        }
+    }
+    const float d = dsh;
+    if (t < ng) {
+        const float eff = d * (float)sc_[t];
+        for (int i = 0; i < 16; ++i) code[t * 16 + i] = (uint8_t)(((eff == 0.0f) ? 0 : q6k_level_dev(x[i] / eff)) + 32);
+    }
+    __syncthreads();
+    const uint32_t dh = float_to_half_bits(d);
+    uint8_t* p = dst + blk * 210;
+    for (int byte = t; byte < 210; byte += 64) {
+        uint32_t v = 0;
+        if (byte < 192) {
+#pragma unroll
+            for (int b = 0; b < 8; ++b) {
+                const int pos = 8 * byte + b;
+                v |= (((uint32_t)code[pos / 6] >> (pos % 6)) & 1u) << b;
+            }
+        } else if (byte < 208) {
+            v = (uint32_t)(uint8_t)(int8_t)sc_[byte - 192];
+        } else {
+            v = (dh >> (8 * (byte - 208))) & 0xFFu;
+        }
+        p[byte] = (uint8_t)v;
+    }
+}
+
+// Q_G_6_K_M / _K_H (src/codec/block_codec.cpp:2733-2755): a candidate payload replaces the current one when
+// its decoded mean squared error (double, index order, fused like the reference's k_mse) is strictly smaller.
+// One wavefront per block: lanes decode both payloads, lane 0 compares, all lanes copy.
+__global__ __launch_bounds__(64) void keep_better_q6k_kernel(const float* __restrict__ wg, uint8_t* __restrict__ cur,
+                                                             const uint8_t* __restrict__ cand) {
+    __shared__ float dc[256], dn[256];
+    __shared__ int take;
+    const int64_t blk = blockIdx.x;
+    const int t = threadIdx.x;
+    uint8_t* pc = cur + blk * 210;
+    const uint8_t* pn = cand + blk * 210;
+    for (int i = t; i < 256; i += 64) {
+        dc[i] = decode_weight<TFQ_Q_G_6>(pc, i);
+        dn[i] = decode_weight<TFQ_Q_G_6>(pn, i);
+    }
+    __syncthreads();
+    if (t == 0) {
+        double ec = 0.0, en = 0.0;
+        for (int i = 0; i < 256; ++i) {
+            const double w = (double)wg[blk * 256 + i];
+            const double a = w - (double)dc[i], b = w - (double)dn[i];
+            ec = __builtin_fma(a, a, ec);
+            en = __builtin_fma(b, b, en);
+        }
+        take = (en / 256.0) < (ec / 256.0);
+    }
+    __syncthreads();
+    if (take)
+        for (int i = t; i < 210; i += 64) pc[i] = pn[i];
+}
+
 // Wire -> Tiled16: one lane per 16-byte piece of the tiled buffer.  Piece p of a unit: p < 64 code
 // slot of k-step 0, p < 128 of k-step 1, else a 16-byte part of a row header.  Codes narrower
 // than 4 bits are widened to nibbles.
@@ -707,6 +1226,35 @@ int launch_encode(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStr
         case TFQ_SB256A3: hipLaunchKernelGGL(encode_affine_kernel<TFQ_SB256A3>, grid, dim3(64), 0, s, w, dst); break;
         case TFQ_SB256A2: hipLaunchKernelGGL(encode_affine_kernel<TFQ_SB256A2>, grid, dim3(64), 0, s, w, dst); break;
         case TFQ_Q_1_5: hipLaunchKernelGGL(encode_affine_kernel<TFQ_Q_1_5>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_Q_G_8:
+            if (nblocks * 8 > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "encode: too many groups in one call");
+            hipLaunchKernelGGL(encode_comp8_kernel<TFQ_Q_G_8>, dim3((unsigned)(nblocks * 8)), dim3(64), 0, s, w, dst);
+            break;
+        case TFQ_Q_8: hipLaunchKernelGGL(encode_comp8_kernel<TFQ_Q_8>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_Q_4: hipLaunchKernelGGL(encode_lattice_kernel<TFQ_Q_4>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_Q_2: hipLaunchKernelGGL(encode_lattice_kernel<TFQ_Q_2>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_Q_G_2_K_L: hipLaunchKernelGGL(encode_grp16_kernel<TFQ_Q_G_2_K_L>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_Q_G_3_K_L: hipLaunchKernelGGL(encode_grp16_kernel<TFQ_Q_G_3_K_L>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_Q_G_4_K_L: hipLaunchKernelGGL(encode_grp16_kernel<TFQ_Q_G_4_K_L>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_Q_6_5: hipLaunchKernelGGL(encode_grp16_kernel<TFQ_Q_6_5>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_Q_G_6:
+            // the _K_M / _K_H tiers re-run the search with more effort and keep the better candidate by decoded
+            // error (src/codec/block_codec.cpp:2733-2755); that selection is not on the device
+            hipLaunchKernelGGL(encode_q6k_kernel, grid, dim3(64), 0, s, w, dst, 4, 3, 3);
+            if (fmt == TFQ_Q_G_6_K_M || fmt == TFQ_Q_G_6_K_H) {
+                // longer searches, each kept only where it decodes strictly better (src/codec/block_codec.cpp:2733-2755)
+                uint8_t* cand = nullptr;
+                TFQ_HIP(hipMalloc(&cand, (size_t)nblocks * 210));
+                const int effort[2][3] = {{8, 5, 6}, {14, 8, 10}};
+                for (int c = 0; c < (fmt == TFQ_Q_G_6_K_H ? 2 : 1); ++c) {
+                    hipLaunchKernelGGL(encode_q6k_kernel, grid, dim3(64), 0, s, w, cand, effort[c][0], effort[c][1], effort[c][2]);
+                    hipLaunchKernelGGL(keep_better_q6k_kernel, grid, dim3(64), 0, s, w, dst, (const uint8_t*)cand);
+                }
+                const hipError_t e1 = hipStreamSynchronize(s);
+                (void)hipFree(cand);
+                if (e1 != hipSuccess) return hip_fail(e1, "hipStreamSynchronize");
+            }
+            break;
         case TFQ_Q_24: hipLaunchKernelGGL(encode_wide_kernel<TFQ_Q_24>, grid, block, 0, s, w, dst); break;
         case TFQ_Q_24_5: hipLaunchKernelGGL(encode_wide_kernel<TFQ_Q_24_5>, grid, block, 0, s, w, dst); break;
         case TFQ_Q_G_24: hipLaunchKernelGGL(encode_wide_kernel<TFQ_Q_G_24>, grid, block, 0, s, w, dst); break;
