@@ -25,7 +25,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes moved per algorithmic byte for the GEMV launches of this workload, from
 # rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy kernel (summary under profiles/)
-HBM_TRAFFIC_RATIO = 1.0075
+HBM_TRAFFIC_RATIO = 1.0073
 # (name, N, K, input) per decoder layer
 PROJ = [("q", 4096, 4096, "x"), ("k", 1024, 4096, "x"), ("v", 1024, 4096, "x"), ("o", 4096, 4096, "a"),
         ("gate", 14336, 4096, "x"), ("up", 14336, 4096, "x"), ("down", 4096, 14336, "h")]
@@ -46,6 +46,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM figure")
+    ap.add_argument("--no-moe", action="store_true", help="skip the mixture-of-experts layer figure")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one elementwise kernel that reads and writes 1 GiB (counter calibration)")
     args = ap.parse_args()
@@ -153,6 +154,10 @@ def main():
 
     if not args.no_prefill:
         res["prefill"] = prefill_gemm(tfq, torch, layers[0], gen)
+    if not args.no_moe:
+        del layers
+        torch.cuda.empty_cache()
+        res["moe"] = moe_layer(tfq, torch, fmt, bpw, gen)
     if not args.no_cpu:
         res["cpu_baseline"] = cpu_baseline(host_layer0, fmt, B, acts, bpw)
     print(json.dumps(res), flush=True)
@@ -183,6 +188,37 @@ def prefill_gemm(tfq, torch, layer, gen, M=2048, reps=10):
                      "frac": round(tf / MFMA_PEAK_TFLOPS, 4)}
         del x, y
     return out
+
+
+def moe_layer(tfq, torch, fmt, bpw, gen, E=8, top_k=2, T=16, D=4096, F=14336, reps=20):
+    """One mixture-of-experts FFN call (router top-k given on the host, like the reference's dispatch):
+    16 tokens, 8 experts, top-2, gate/up 14336x4096 and down 4096x14336 per expert.  Wall time per call
+    including the host-side routing lists; bytes = packed weights of the active experts.  A side figure."""
+    import numpy as np
+    gate, up, down = [], [], []
+    for _ in range(E):
+        for lst, n, k in ((gate, F, D), (up, F, D), (down, D, F)):
+            w = torch.randn(n * k, device="cuda", generator=gen) * 0.02
+            lst.append(tfq.Weight(fmt, n, k, tfq.encode(fmt, w)))
+            del w
+    logits = torch.randn(T, E, device="cuda", generator=gen)
+    _, idx, wts = tfq.moe_route(logits, top_k)
+    idx_h, w_h = idx.cpu().numpy().astype(np.int64), wts.cpu().numpy()
+    x = torch.randn(T, D, device="cuda", generator=gen).bfloat16()
+    for _ in range(3):
+        tfq.moe_ffn(gate, up, down, idx_h, w_h, x, mid_dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        tfq.moe_ffn(gate, up, down, idx_h, w_h, x, mid_dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / reps
+    active = len(set(idx_h.reshape(-1).tolist()))
+    nbytes = active * 3 * F * D * bpw / 8
+    return {"tokens": T, "experts": E, "top_k": top_k, "active_experts": active,
+            "tokens_per_expert": [int((idx_h == e).sum()) for e in range(E)],
+            "us_per_call": round(dt * 1e6, 1), "gbs": round(nbytes / dt / 1e9, 1),
+            "frac": round(nbytes / dt / 1e9 / HBM_PEAK_GBS, 4), "bound": "hbm"}
 
 
 def cpu_baseline(layer, fmt, B, acts, bpw, budget_s=12.0):
