@@ -14,6 +14,9 @@
 //   Q_4 / Q_8 lattice codec    src/codec/block_codec.cpp:182-203, 435-529
 //   8-bit companded grid       src/codec/block_codec.cpp:222-265, 306-358
 //   Q_G_8 compound codec       src/codec/block_codec.cpp:365-427
+//   fixed codebooks (Q_3/6/12) src/codec/block_codec.cpp:530-735
+//   12-bit compound (Q_G_12)   src/codec/block_codec.cpp:961-1040
+//   _K_M / _K_H tier searches  src/codec/block_codec.cpp:2378-2400, 2551-2665, 2756-2824
 //   affine grouped codec       src/codec/block_codec.cpp:1316-1521, 1620-1687
 //   format dispatch            src/codec/block_codec.cpp:2402-2867, 2869-3067
 //   seeded generator           src/core/random.cpp:45-81
@@ -67,9 +70,11 @@ enum : uint8_t {
     F_Q_2_5 = 74, F_Q_3_5 = 75, F_Q_4_5 = 76, F_Q_6_5 = 77, F_Q_8_5 = 78,
     F_Q_G_2_5 = 83, F_Q_G_3_5 = 84, F_Q_G_4_5 = 85, F_Q_G_6_5 = 86, F_Q_G_8_5 = 87,
     F_B32S4 = 105, F_B32S8 = 106, F_SB256A3 = 107, F_SB256A2 = 108,
+    F_Q_3 = 2, F_Q_6 = 4, F_Q_12 = 6, F_Q_2_K_L = 13, F_Q_3_K_L = 16, F_Q_4_K_L = 19, F_Q_6_K_L = 22, F_Q_8_K_L = 25,
+    F_Q_12_K_L = 28, F_Q_G_12 = 43, F_Q_G_8_K_L = 61, F_Q_G_12_K_L = 64, F_Q_12_5 = 79, F_Q_G_12_5 = 88,
 };
 
-enum class Codec { Raw32, Lattice, Affine, Grp8, Sym32, Q6K, Q1, Wide };
+enum class Codec { Raw32, Lattice, Affine, Grp8, Sym32, Q6K, Q1, Wide, Fixed, Grp12 };
 
 struct Spec {
     Codec codec;
@@ -103,6 +108,23 @@ bool spec_for(uint8_t fmt, Spec* s) {
         case F_Q_2:   *s = {Codec::Lattice, 2, 0, 0, 0, 2.0f}; return true;
         case F_Q_4:   *s = {Codec::Lattice, 4, 0, 0, 0, 4.0f}; return true;
         case F_Q_8:   *s = {Codec::Lattice, 8, 0, 0, 0, 8.0f}; return true;
+        // _K_L/_K_M/_K_H of the plain lattices: the base payload, then longer searches (:2551-2645)
+        case F_Q_2_K_L: case F_Q_2_K_L + 1: case F_Q_2_K_L + 2: *s = {Codec::Lattice, 2, 0, 0, 0, 2.0f, fmt - F_Q_2_K_L}; return true;
+        case F_Q_4_K_L: case F_Q_4_K_L + 1: case F_Q_4_K_L + 2: *s = {Codec::Lattice, 4, 0, 0, 0, 4.0f, fmt - F_Q_4_K_L}; return true;
+        case F_Q_8_K_L: case F_Q_8_K_L + 1: case F_Q_8_K_L + 2: *s = {Codec::Lattice, 8, 0, 0, 0, 8.0f, fmt - F_Q_8_K_L}; return true;
+        // fixed shared codebooks, no table on the wire (:530-735, :2570-2665)
+        case F_Q_3:  *s = {Codec::Fixed, 3, 0, 0, 0, 3.0f}; return true;
+        case F_Q_6:  *s = {Codec::Fixed, 6, 0, 0, 0, 6.0f}; return true;
+        case F_Q_12: *s = {Codec::Fixed, 12, 0, 0, 0, 12.0f}; return true;
+        case F_Q_3_K_L: case F_Q_3_K_L + 1: case F_Q_3_K_L + 2: *s = {Codec::Fixed, 3, 0, 0, 0, 3.0f, fmt - F_Q_3_K_L}; return true;
+        case F_Q_6_K_L: case F_Q_6_K_L + 1: case F_Q_6_K_L + 2: *s = {Codec::Fixed, 6, 0, 0, 0, 6.0f, fmt - F_Q_6_K_L}; return true;
+        case F_Q_12_K_L: case F_Q_12_K_L + 1: case F_Q_12_K_L + 2: *s = {Codec::Fixed, 12, 0, 0, 0, 12.0f, fmt - F_Q_12_K_L}; return true;
+        // 12-bit codes with one binary16 scale per 32 weights when the block is whole groups of 32;
+        // gsz names what other block sizes take: 0 the grouped-lattice fallback (:2494-2500), 1 the
+        // fixed 12-bit codebook (:2788-2824, :2835, :2845)
+        case F_Q_G_12: *s = {Codec::Grp12, 12, 0, 0, 0, 12.5f}; return true;
+        case F_Q_12_5: case F_Q_G_12_5: *s = {Codec::Grp12, 12, 1, 0, 0, 12.5f}; return true;
+        case F_Q_G_12_K_L: case F_Q_G_12_K_L + 1: case F_Q_G_12_K_L + 2: *s = {Codec::Grp12, 12, 1, 0, 0, 12.0f, fmt - F_Q_G_12_K_L}; return true;
         case F_Q_G_4: case F_Q_4_5: case F_Q_G_4_5:
             *s = {Codec::Affine, 4, 32, 6, 6, 4.5f}; return true;
         case F_Q_G_3: case F_Q_3_5: case F_Q_G_3_5:
@@ -110,6 +132,8 @@ bool spec_for(uint8_t fmt, Spec* s) {
         case F_Q_G_2: *s = {Codec::Affine, 2, 16, 4, 4, 2.625f}; return true;
         case F_Q_G_8: case F_Q_8_5: case F_Q_G_8_5:
             *s = {Codec::Grp8, 8, 32, 0, 0, 8.5f}; return true;
+        // :2756-2786: same compound payload; other block sizes go to the affine codec with a claim of 8.0
+        case F_Q_G_8_K_L: case F_Q_G_8_K_L + 1: case F_Q_G_8_K_L + 2: *s = {Codec::Grp8, 8, 32, 0, 0, 8.0f, fmt - F_Q_G_8_K_L}; return true;
         // Claims below the affine header's size: every block takes the grouped-lattice
         // fallback layout (src/codec/block_codec.cpp:1408-1411, :1622-1625), so the three
         // tiers of one width are byte-identical (:2676-2730).
@@ -358,7 +382,7 @@ size_t lattice_bytes(int bits, int n) {
     return (budget_bits + 7) / 8;
 }
 
-bool lattice_encode(int bits, const float* w, int n, uint8_t* out, size_t nbytes) {
+bool lattice_encode(int bits, const float* w, int n, uint8_t* out, size_t nbytes, int iters = 2, float smult = 1.0f) {
     std::memset(out, 0, nbytes);
     BitSink bs(out, nbytes);
     if (n < kSlots) {
@@ -367,7 +391,7 @@ bool lattice_encode(int bits, const float* w, int n, uint8_t* out, size_t nbytes
     }
     const int slots = std::min(kSlots, n);
     if (bits == 8) {
-        const float s = comp8_fit_scale(w, n) * 1.0f;
+        const float s = comp8_fit_scale(w, n) * smult;
         bs.put(half_from_float(s), 16);
         for (int i = 0; i < n; ++i) {
             const bool sl = slot_at(i, n, slots);
@@ -380,9 +404,9 @@ bool lattice_encode(int bits, const float* w, int n, uint8_t* out, size_t nbytes
     const float R = bits == 2 ? 1.5104f : bits == 4 ? 2.7178f : 8.0f;
     float maxa = 0.0f;
     for (int i = 0; i < n; ++i) maxa = std::max(maxa, std::fabs(w[i]));
-    float s = (maxa > 1e-30f) ? maxa / R * 1.0f : 0.0f;
+    float s = (maxa > 1e-30f) ? maxa / R * smult : 0.0f;
     if (s > 0.0f) {
-        for (int iter = 0; iter < 2; ++iter) {
+        for (int iter = 0; iter < iters; ++iter) {
             double num = 0.0, den = 0.0;
             for (int i = 0; i < n; ++i) {
                 const float l = grid_value(bits, grid_nearest(w[i] / s, bits));
@@ -423,12 +447,12 @@ void lattice_decode(int bits, const uint8_t* bytes, size_t size, int n, float* o
 // ------------------------------------------------------ Q_G_8 compound codec
 bool grp8_fits(int n) { return n >= 32 && n % 32 == 0; }
 
-void grp8_encode(const float* w, int n, uint8_t* out) {
+void grp8_encode(const float* w, int n, uint8_t* out, float smult = 1.0f) {
     const int ng = n / 32;
     uint8_t* code = out;
     uint8_t* sc = out + n;
     for (int g = 0; g < ng; ++g) {
-        const float s = comp8_fit_scale(w + g * 32, 32) * 1.0f;
+        const float s = comp8_fit_scale(w + g * 32, 32) * smult;
         for (int i = 0; i < 32; ++i)
             code[g * 32 + i] = (uint8_t)((s > 0.0f) ? comp8_nearest(w[g * 32 + i] / s) : 0u);
         const uint16_t h = half_from_float(s);
@@ -445,6 +469,175 @@ void grp8_decode(const uint8_t* bytes, size_t size, int n, float* out) {
         const int g = i >> 5;
         const uint16_t h = (uint16_t)(sc[2 * g] | ((uint16_t)sc[2 * g + 1] << 8));
         out[i] = half_to_float(h) * comp8().lv[bytes[i]];
+    }
+}
+
+// ------------------------------------------ fixed shared codebooks (Q_3/6/12)
+// src/codec/block_codec.cpp:530-735.  Q_3 takes eight Lloyd-Max levels of N(0,1);
+// Q_6 and Q_12 take the 64 / 4096 mid-quantiles of N(0,1), built once from a
+// rational erf approximation inverted by Newton steps, all in double and then
+// rounded to binary32.  No table travels with a block: a block is a binary16
+// scale and n codes, sixteen of which drop their low bit to pay for the scale.
+const float kFixed3[8] = {-3.0776f, -2.1479f, -1.2879f, -0.4240f, 0.4240f, 1.2879f, 2.1479f, 3.0776f};
+
+double erf_rational(double x) {  // :542-549
+    const double t = 1.0 / (1.0 + 0.5 * std::fabs(x));
+    const double tau = t * std::exp(-x * x - 1.26551223 +
+        t * (1.00002368 + t * (0.37409196 + t * (0.09678418 +
+        t * (-0.18628806 + t * (0.27886807 + t * (-1.13520398 +
+        t * (1.48851587 + t * (-0.82215223 + t * 0.17087277)))))))));
+    return (x >= 0.0) ? 1.0 - tau : tau - 1.0;
+}
+
+double erf_inverse(double y) {  // :551-561
+    if (y <= -0.999999) return -6.0;
+    if (y >= 0.999999) return 6.0;
+    double z = 0.0;
+    for (int it = 0; it < 24; ++it) {
+        const double e = erf_rational(z) - y;
+        z -= e / (1.1283791670955126 * std::exp(-z * z));
+        if (std::fabs(e) < 1e-13) break;
+    }
+    return z;
+}
+
+struct FixedTables {  // :563-588
+    std::vector<float> t6, t12;
+    static std::vector<float> build(int count) {
+        std::vector<float> t((size_t)count);
+        for (int j = 0; j < count / 2; ++j) {
+            const float q = (float)(erf_inverse(2.0 * ((double)j + 0.5) / (double)count - 1.0) * std::sqrt(2.0));
+            t[(size_t)j] = q;
+            t[(size_t)(count - 1 - j)] = -q;
+        }
+        return t;
+    }
+    FixedTables() : t6(build(64)), t12(build(4096)) {}
+};
+const FixedTables& fixed_tables() {
+    static const FixedTables t;
+    return t;
+}
+
+float fixed_value(int bits, uint32_t idx) {  // :590-594
+    if (bits == 3) return kFixed3[idx & 7u];
+    const std::vector<float>& t = bits == 6 ? fixed_tables().t6 : fixed_tables().t12;
+    return t[std::min<size_t>(idx, t.size() - 1)];
+}
+
+uint32_t fixed_nearest(int bits, float v) {  // :596-622
+    if (bits == 3) {
+        uint32_t best = 0;
+        float bd = std::fabs(v - kFixed3[0]);
+        for (int i = 1; i < 8; ++i) {
+            const float d = std::fabs(v - kFixed3[i]);
+            if (d < bd) { bd = d; best = (uint32_t)i; }
+        }
+        return best;
+    }
+    const std::vector<float>& t = bits == 6 ? fixed_tables().t6 : fixed_tables().t12;
+    const int half = (int)(t.size() / 2);
+    const float a = std::fabs(v);
+    int lo = half, hi = (int)t.size() - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi) / 2;
+        if (t[(size_t)mid] < a) lo = mid + 1; else hi = mid;
+    }
+    if (lo > half) {
+        const float d0 = a - t[(size_t)lo - 1];
+        const float d1 = t[(size_t)lo] - a;
+        if (d1 >= d0) --lo;
+    }
+    return (v >= 0.0f) ? (uint32_t)lo : (uint32_t)(half - 1 - (lo - half));
+}
+
+size_t fixed_bytes(int bits, int n) { return ((size_t)std::ceil((double)bits * (double)n) + 7) / 8; }
+
+// Least-squares scale of cnt weights against their nearest levels, `iters` rounds from max|w| / top * smult.
+float fixed_fit_scale(int bits, const float* w, int cnt, int iters, float smult) {
+    const float top = fixed_value(bits, (1u << bits) - 1u);
+    float maxa = 0.0f;
+    for (int i = 0; i < cnt; ++i) maxa = std::max(maxa, std::fabs(w[i]));
+    float s = (maxa > 1e-30f) ? maxa / top * smult : 0.0f;
+    if (s > 0.0f) {
+        for (int iter = 0; iter < iters; ++iter) {
+            double num = 0.0, den = 0.0;
+            for (int i = 0; i < cnt; ++i) {
+                const float l = fixed_value(bits, fixed_nearest(bits, w[i] / s));
+                num += (double)w[i] * (double)l;
+                den += (double)l * (double)l;
+            }
+            if (den > 1e-20) s = (float)(num / den);
+        }
+    }
+    return s;
+}
+
+bool fixed_encode(int bits, const float* w, int n, uint8_t* out, size_t nbytes, int iters = 3, float smult = 1.0f) {  // :624-663
+    std::memset(out, 0, nbytes);
+    BitSink bs(out, nbytes);
+    if (n < kSlots) {
+        for (int i = 0; i < n; ++i) bs.put(fixed_nearest(bits, w[i]), bits);
+        return !bs.overflow;
+    }
+    float s = fixed_fit_scale(bits, w, n, iters, smult);
+    if (!(s > 0.0f)) s = 0.0f;
+    bs.put(half_from_float(s), 16);
+    for (int i = 0; i < n; ++i) {
+        const bool sl = slot_at(i, n, kSlots);
+        uint32_t idx = fixed_nearest(bits, (s == 0.0f) ? 0.0f : w[i] / s);
+        if (sl) idx &= ~1u;
+        bs.put(sl ? (idx >> 1) : idx, bits - (sl ? 1 : 0));
+    }
+    return !bs.overflow;
+}
+
+void fixed_decode(int bits, const uint8_t* bytes, size_t size, int n, float* out) {  // :665-735
+    BitSource br(bytes, size);
+    if (n < kSlots) {
+        for (int i = 0; i < n; ++i) out[i] = fixed_value(bits, br.take(bits));
+        return;
+    }
+    const float scale = half_to_float((uint16_t)br.take(16));
+    for (int i = 0; i < n; ++i) {
+        const bool sl = slot_at(i, n, kSlots);
+        uint32_t idx = br.take(bits - (sl ? 1 : 0));
+        if (sl) idx <<= 1;
+        out[i] = fixed_value(bits, idx) * scale;
+    }
+}
+
+// 12-bit compound (:961-1040): n 12-bit codes of the fixed table, then one binary16 scale per 32 weights.
+bool grp12_fits(int n) {
+    return n >= 32 && n % 32 == 0 && (size_t)n * 12 + (size_t)(n / 32) * 16 == (size_t)std::ceil(12.5 * (double)n);
+}
+size_t grp12_bytes(int n) { return ((size_t)n * 12 + (size_t)(n / 32) * 16 + 7) / 8; }
+
+bool grp12_encode(const float* w, int n, uint8_t* out, size_t nbytes, int iters = 3, float smult = 1.0f) {
+    std::memset(out, 0, nbytes);
+    BitSink bs(out, nbytes);
+    const int ng = n / 32;
+    std::vector<float> sc((size_t)ng);
+    for (int g = 0; g < ng; ++g) {
+        const float s = fixed_fit_scale(12, w + g * 32, 32, iters, smult);
+        sc[(size_t)g] = (s > 0.0f) ? s : 0.0f;
+    }
+    for (int g = 0; g < ng; ++g)
+        for (int i = 0; i < 32; ++i)
+            bs.put(sc[(size_t)g] > 0.0f ? fixed_nearest(12, w[g * 32 + i] / sc[(size_t)g]) : 0u, 12);
+    for (int g = 0; g < ng; ++g) bs.put(half_from_float(sc[(size_t)g]), 16);
+    return !bs.overflow;
+}
+
+void grp12_decode(const uint8_t* bytes, size_t size, int n, float* out) {
+    const int ng = n / 32;
+    if (size * 8 < (size_t)n * 12 + (size_t)ng * 16) return;
+    BitSource codes(bytes, size), scales(bytes, size);
+    scales.pos = (size_t)n * 12;
+    float s = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        if ((i & 31) == 0) s = half_to_float((uint16_t)scales.take(16));
+        out[i] = s * fixed_value(12, codes.take(12));
     }
 }
 
@@ -1284,7 +1477,8 @@ bool sym32_decode(int bits, const uint8_t* bytes, size_t size, int n, float* out
 // ------------------------------------------------------------------ dispatch
 // A Q_G_8 block whose size is not a multiple of 32 is written by the affine codec
 // with 8-bit levels (src/codec/block_codec.cpp:2501-2510, :2957-2962).
-const Spec kGrp8Tail = {Codec::Affine, 8, 32, 6, 6, 8.5f};
+// The _K tiers pass a claim of 8.0 there (:2758, :3009).
+Spec grp8_tail(const Spec& sp) { return {Codec::Affine, 8, 32, 6, 6, sp.claimed}; }
 
 long affine_bytes(const Spec& sp, int n) {
     const AffineSizes z = affine_sizes(sp, n);
@@ -1316,15 +1510,76 @@ bool q6k_encode_tier(int tier, const float* w, int n, uint8_t* out, size_t nbyte
     return true;
 }
 
+// The _K_M / _K_H search shared by the lattice, fixed-codebook and compound ids
+// (:2551-2665, :2756-2824): the base payload first, then `count` further
+// candidates, each kept only when its decoded error is strictly smaller.
+template <class Enc, class Dec>
+bool keep_better(const float* w, int n, uint8_t* out, size_t nbytes, int count, Enc&& encode, Dec&& decode) {
+    std::vector<float> dec((size_t)n, 0.0f);
+    std::vector<uint8_t> cand(nbytes);
+    decode(out, dec.data());
+    double best = mean_sq_err(w, dec.data(), n);
+    for (int c = 0; c < count; ++c) {
+        if (!encode(c, cand.data())) return false;
+        std::fill(dec.begin(), dec.end(), 0.0f);
+        decode(cand.data(), dec.data());
+        const double e = mean_sq_err(w, dec.data(), n);
+        if (e < best) { best = e; std::memcpy(out, cand.data(), nbytes); }
+    }
+    return true;
+}
+
+const float kTierScale[6] = {1.0f, 1.0f, 0.9f, 1.1f, 0.7f, 1.3f};
+
+bool lattice_encode_tier(int bits, int tier, const float* w, int n, uint8_t* out, size_t nb) {
+    if (!lattice_encode(bits, w, n, out, nb)) return false;
+    if (tier <= 0) return true;
+    return keep_better(w, n, out, nb, tier >= 2 ? 6 : 1,
+        [&](int c, uint8_t* o) { return lattice_encode(bits, w, n, o, nb, c == 0 ? 6 : 14, kTierScale[c]); },
+        [&](const uint8_t* b, float* d) { lattice_decode(bits, b, nb, n, d); });
+}
+
+bool fixed_encode_tier(int bits, int tier, const float* w, int n, uint8_t* out, size_t nb) {
+    if (!fixed_encode(bits, w, n, out, nb)) return false;
+    if (tier <= 0) return true;
+    return keep_better(w, n, out, nb, tier >= 2 ? 6 : 1,
+        [&](int c, uint8_t* o) { return fixed_encode(bits, w, n, o, nb, c == 0 ? 10 : 24, kTierScale[c]); },
+        [&](const uint8_t* b, float* d) { fixed_decode(bits, b, nb, n, d); });
+}
+
+bool grp12_encode_tier(int tier, const float* w, int n, uint8_t* out, size_t nb) {
+    if (!grp12_encode(w, n, out, nb)) return false;
+    if (tier <= 0) return true;
+    static const int its[6] = {8, 8, 20, 20, 20, 20};
+    static const float sm[6] = {1.0f, 1.0f, 0.93f, 1.07f, 0.7f, 1.3f};
+    return keep_better(w, n, out, nb, tier >= 2 ? 6 : 1,
+        [&](int c, uint8_t* o) { return grp12_encode(w, n, o, nb, its[c], sm[c]); },
+        [&](const uint8_t* b, float* d) { grp12_decode(b, nb, n, d); });
+}
+
+bool grp8_encode_tier(int tier, const float* w, int n, uint8_t* out, size_t nb) {
+    grp8_encode(w, n, out);
+    if (tier <= 0) return true;
+    static const float ks[6] = {0.7f, 0.9f, 0.95f, 1.05f, 1.1f, 1.3f};
+    const int count = tier >= 2 ? 6 : 2;
+    return keep_better(w, n, out, nb, count,
+        [&](int c, uint8_t* o) { grp8_encode(w, n, o, ks[6 - count + c]); return true; },
+        [&](const uint8_t* b, float* d) { grp8_decode(b, nb, n, d); });
+}
+
 long block_bytes(uint8_t fmt, int n) {
     Spec sp;
     if (n <= 0 || !spec_for(fmt, &sp)) return -1;
     switch (sp.codec) {
         case Codec::Raw32: return (long)n * 4;
         case Codec::Lattice: return (long)lattice_bytes(sp.bits, n);
+        case Codec::Fixed: return (long)fixed_bytes(sp.bits, n);
+        case Codec::Grp12:
+            if (grp12_fits(n)) return (long)grp12_bytes(n);
+            return sp.gsz ? (long)fixed_bytes(12, n) : (long)grp16_sizes(12, n, 12.5f).total;
         case Codec::Grp8:
             if (grp8_fits(n)) return (long)n + (long)(n / 32) * 2;
-            return affine_bytes(kGrp8Tail, n);
+            return affine_bytes(grp8_tail(sp), n);
         case Codec::Affine: return affine_bytes(sp, n);
         case Codec::Q6K: return (long)q6k_sizes(n).total;
         case Codec::Q1: return (long)q1_bytes(n);
@@ -1342,10 +1597,23 @@ long encode_block(uint8_t fmt, const float* w, int n, uint8_t* out, size_t cap) 
     bool ok = true;
     switch (sp.codec) {
         case Codec::Raw32: std::memcpy(out, w, (size_t)n * 4); break;
-        case Codec::Lattice: ok = lattice_encode(sp.bits, w, n, out, (size_t)need); break;
+        case Codec::Lattice: ok = lattice_encode_tier(sp.bits, sp.tier, w, n, out, (size_t)need); break;
+        case Codec::Fixed: ok = fixed_encode_tier(sp.bits, sp.tier, w, n, out, (size_t)need); break;
+        case Codec::Grp12:
+            if (grp12_fits(n)) ok = grp12_encode_tier(sp.tier, w, n, out, (size_t)need);
+            else if (sp.gsz) ok = fixed_encode_tier(12, sp.tier, w, n, out, (size_t)need);
+            else ok = grp16_encode(12, w, n, 12.5f, out, (size_t)need);
+            break;
         case Codec::Grp8:
-            if (grp8_fits(n)) grp8_encode(w, n, out);
-            else ok = affine_encode(kGrp8Tail, w, n, out, (size_t)need);
+            if (grp8_fits(n)) ok = grp8_encode_tier(sp.tier, w, n, out, (size_t)need);
+            else {
+                // with a claim of 8.0 the affine header never fits, so the three tiers of a short
+                // block share the grouped-lattice fallback; an affine short block of a searched tier
+                // (:2775-2785) is not restated
+                const Spec tail = grp8_tail(sp);
+                if (sp.tier > 0 && affine_sizes(tail, n).ok) return -1;
+                ok = affine_encode(tail, w, n, out, (size_t)need);
+            }
             break;
         case Codec::Affine: ok = affine_encode(sp, w, n, out, (size_t)need); break;
         case Codec::Q6K: ok = q6k_encode_tier(sp.tier, w, n, out, (size_t)need); break;
@@ -1365,8 +1633,14 @@ int decode_block(uint8_t fmt, const uint8_t* bytes, size_t size, int n, float* o
     switch (sp.codec) {
         case Codec::Raw32: if (size >= (size_t)n * 4) std::memcpy(out, bytes, (size_t)n * 4); return 0;
         case Codec::Lattice: lattice_decode(sp.bits, bytes, size, n, out); return 0;
+        case Codec::Fixed: fixed_decode(sp.bits, bytes, size, n, out); return 0;
+        case Codec::Grp12:
+            if (grp12_fits(n)) grp12_decode(bytes, size, n, out);
+            else if (sp.gsz) fixed_decode(12, bytes, size, n, out);
+            else grp16_decode(12, bytes, size, n, out);
+            return 0;
         case Codec::Grp8:
-            if (!grp8_fits(n)) return affine_decode(kGrp8Tail, bytes, size, n, out) ? 0 : -1;
+            if (!grp8_fits(n)) return affine_decode(grp8_tail(sp), bytes, size, n, out) ? 0 : -1;
             grp8_decode(bytes, size, n, out);
             return 0;
         case Codec::Q6K: q6k_decode(bytes, size, n, out); return 0;
@@ -1434,6 +1708,11 @@ uint16_t orc_f32_to_f16(float v) { return half_from_float(v); }
 float orc_f16_to_f32(uint16_t h) { return half_to_float(h); }
 
 void orc_comp8_table(float* out256) { std::memcpy(out256, comp8().lv, sizeof(float) * 256); }
+
+// levels of the fixed 3-, 6- or 12-bit codebook (2^bits values)
+void orc_fixed_table(int bits, float* out) {
+    for (uint32_t i = 0; i < (1u << bits); ++i) out[i] = fixed_value(bits, i);
+}
 
 long orc_block_bytes(uint8_t fmt, int n) { return block_bytes(fmt, n); }
 

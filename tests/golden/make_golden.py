@@ -22,13 +22,17 @@ tails.npz
     reference codec, one row of `index` = (wire id, n, input, payload offset, payload
     bytes, decoded offset) into the flat `payloads` / `decoded` arrays: the short-block
     layouts (raw levels, one scale, grouped-lattice fallback), Q_2, Q_G_6, the ids
-    whose claim is below the affine header's size, the sign formats and the 16- and
-    24-bit formats
+    whose claim is below the affine header's size, the sign formats, the 16- and
+    24-bit formats, the fixed-codebook formats, the 12-bit compound and searched tiers
 sample.quant, sample_quant.npz
     a container written by the reference's QUANTWriter (header with a 5-byte config,
     format table, tensor table, block records): tensor "blk.0.ffn_gate" 4 x 512 in Q_G_4,
     "mixed" whose blocks alternate formats, "tail" of 300 weights in Q_G_8 and "raw" of 40
     weights in Q_32; the npz holds what QUANTReader::read_tensor returns for each name
+fixed_levels.npz, ../../transformers-fusion_amd/csrc/fixed{6,12}_levels.inc
+    the 64- and 4096-entry level tables of Q_6 / Q_12 as binary32 bit patterns, read off
+    the reference by decoding blocks of fewer than 16 weights (raw codes, implied scale 1)
+    that hold every code once; the .inc files carry the same words for the device build
 matmul.npz
     for Q_G_4 and Q_G_8: y = x.W^T with W 48x512 from the fixture generator,
     computed by the reference scalar_gemm_bt on the reference-decoded matrix
@@ -62,7 +66,9 @@ def inputs():
 
 TAIL_FORMATS = ["Q_2", "Q_4", "Q_8", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_6", "Q_G_8", "Q_G_2_K_H", "Q_G_3_K_L",
                 "Q_G_4_K_M", "Q_G_6_K_M", "Q_G_6_K_H", "Q_2_5", "Q_6_5",
-                "Q_1", "Q_G_1_K_H", "Q_1_5", "Q_16", "Q_G_16", "Q_24", "Q_G_24"]
+                "Q_1", "Q_G_1_K_H", "Q_1_5", "Q_16", "Q_G_16", "Q_24", "Q_G_24",
+                "Q_3", "Q_6", "Q_12", "Q_2_K_H", "Q_4_K_M", "Q_8_K_H", "Q_3_K_H", "Q_6_K_M", "Q_12_K_H", "Q_G_12",
+                "Q_G_8_K_H", "Q_G_12_K_H", "Q_12_5"]
 TAIL_SIZES = [1, 7, 8, 15, 16, 31, 32, 33, 100, 160, 250, 255, 256]
 
 
@@ -94,9 +100,43 @@ def container(w):
                         **{name: O.ref_container_read_tensor(path, name) for name, _ in tensors})
 
 
+def pack_lsb_first(codes, bits):
+    """Codes into a byte string, each `bits` wide, least significant bit first."""
+    out = np.zeros((len(codes) * bits + 7) // 8, np.uint8)
+    pos = 0
+    for c in codes:
+        for b in range(bits):
+            if (int(c) >> b) & 1:
+                out[pos >> 3] |= 1 << (pos & 7)
+            pos += 1
+    return out
+
+
+def fixed_levels():
+    tables = {}
+    for bits, fmt in ((6, "Q_6"), (12, "Q_12")):
+        count = 1 << bits
+        vals = np.empty(count, np.float32)
+        for c0 in range(0, count, 15):
+            codes = np.arange(c0, min(c0 + 15, count))
+            vals[c0:c0 + len(codes)] = O.ref_decode_block(fmt, pack_lsb_first(codes, bits), len(codes))
+        tables[f"t{bits}"] = vals.view(np.uint32)
+        inc = os.path.join(ROOT, "transformers-fusion_amd", "csrc", f"fixed{bits}_levels.inc")
+        with open(inc, "w") as f:
+            f.write(f"// {count} levels of the fixed {bits}-bit codebook as binary32 bit patterns: mid-quantiles of N(0,1),\n"
+                    f"// levels[j] = -levels[{count - 1} - j] = RN(sqrt(2) * erfinv(2 (j + 0.5) / {count} - 1)) for j < {count // 2}, with the\n"
+                    "// reference's own erf approximation and Newton inverse (src/codec/block_codec.cpp:542-588).\n"
+                    "// Shipped as data so that no transcendental is evaluated on the device.\n")
+            words = [f"0x{int(v):08x}u" for v in vals.view(np.uint32)]
+            for i in range(0, count, 8):
+                f.write("    " + ", ".join(words[i:i + 8]) + ",\n")
+    np.savez_compressed(os.path.join(HERE, "fixed_levels.npz"), **tables)
+
+
 def main():
     assert O.have_ref(), "build oracle/_ref first (make -C oracle)"
     w = inputs()
+    fixed_levels()
     tails(w)
     container(w)
     out = {"w": w}
