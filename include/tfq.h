@@ -54,6 +54,12 @@ enum {
     TFQ_Q_G_6_K_L = 58, TFQ_Q_G_6_K_M = 59, TFQ_Q_G_6_K_H = 60,
     TFQ_Q_2_5 = 74, TFQ_Q_3_5 = 75, TFQ_Q_4_5 = 76, TFQ_Q_6_5 = 77, TFQ_Q_8_5 = 78,
     TFQ_Q_G_2_5 = 83, TFQ_Q_G_3_5 = 84, TFQ_Q_G_4_5 = 85, TFQ_Q_G_6_5 = 86, TFQ_Q_G_8_5 = 87,
+    TFQ_Q_3 = 2, TFQ_Q_6 = 4, TFQ_Q_12 = 6,
+    TFQ_Q_2_K_L = 13, TFQ_Q_2_K_M = 14, TFQ_Q_2_K_H = 15, TFQ_Q_3_K_L = 16, TFQ_Q_3_K_M = 17, TFQ_Q_3_K_H = 18,
+    TFQ_Q_4_K_L = 19, TFQ_Q_4_K_M = 20, TFQ_Q_4_K_H = 21, TFQ_Q_6_K_L = 22, TFQ_Q_6_K_M = 23, TFQ_Q_6_K_H = 24,
+    TFQ_Q_8_K_L = 25, TFQ_Q_8_K_M = 26, TFQ_Q_8_K_H = 27, TFQ_Q_12_K_L = 28, TFQ_Q_12_K_M = 29, TFQ_Q_12_K_H = 30,
+    TFQ_Q_G_12 = 43, TFQ_Q_G_8_K_L = 61, TFQ_Q_G_8_K_M = 62, TFQ_Q_G_8_K_H = 63,
+    TFQ_Q_G_12_K_L = 64, TFQ_Q_G_12_K_M = 65, TFQ_Q_G_12_K_H = 66, TFQ_Q_12_5 = 79, TFQ_Q_G_12_5 = 88,
     TFQ_B32S4 = 105,   /* 32-group symmetric 4-bit, binary16 scale = absmax/7   */
     TFQ_B32S8 = 106,   /* 32-group symmetric 8-bit, binary16 scale = absmax/127 */
     TFQ_SB256A3 = 107, /* 256-superblock, 16x16 sub-blocks, 6-bit scale + min, 3-bit codes */

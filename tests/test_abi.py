@@ -32,16 +32,18 @@ def test_registry_mirror_without_gpu(tfq):
     assert L.tfq_format_name(40) == b"Q_G_4" and L.tfq_format_name(200) == b"unknown"
     # wire-truth bpw table (include/quant/types.h:197-230 of the reference)
     for fid, bpw in ((3, 4.0), (5, 8.0), (38, 2.625), (39, 3.5), (40, 4.5), (42, 8.5), (105, 4.5), (106, 8.5),
-                     (107, 3.875), (108, 2.875)):
+                     (107, 3.875), (108, 2.875), (2, 3.0), (6, 12.0), (43, 12.5), (74, 2.4375), (77, 6.4375), (61, 8.5),
+                     (64, 12.5), (83, 2.4375), (25, 8.0)):
         assert L.tfq_format_bpw(fid) == pytest.approx(bpw)
-    for fmt, nbytes in (("Q_4", 128), ("Q_8", 256), ("Q_G_2", 84), ("Q_G_3", 112), ("Q_G_4", 144), ("Q_G_8", 272)):
+    for fmt, nbytes in (("Q_4", 128), ("Q_8", 256), ("Q_G_2", 84), ("Q_G_3", 112), ("Q_G_4", 144), ("Q_G_8", 272),
+                        ("Q_3", 96), ("Q_6_K_H", 192), ("Q_12", 384), ("Q_G_12", 400), ("Q_G_12_K_M", 400), ("Q_G_8_K_L", 272)):
         assert tfq.block_bytes(fmt) == nbytes
 
 
 def test_errors_are_reported_not_swallowed(tfq):
     L = tfq.lib()
     out = C.c_size_t(0)
-    assert L.tfq_block_bytes(2, 256, C.byref(out)) == 2            # TFQ_ERR_FORMAT: Q_3 is not handled
+    assert L.tfq_block_bytes(91, 256, C.byref(out)) == 2           # TFQ_ERR_FORMAT: Q_MX_3_5 is not handled
     assert b"not handled" in L.tfq_last_error()
     assert L.tfq_block_bytes(40, 100, C.byref(out)) == 0 and out.value == 57   # short block: grouped-lattice fallback
     assert L.tfq_block_bytes(40, 257, C.byref(out)) == 3           # TFQ_ERR_SHAPE
@@ -63,3 +65,18 @@ def test_no_cpu_fallback_without_device(tfq):
     src = (C.c_float * 256)()
     dst = (C.c_uint8 * 144)()
     assert L.tfq_encode_blocks_host(105, src, 256, dst, 144, None) == 4   # TFQ_ERR_DEVICE
+
+
+def test_block_sizes_equal_the_oracle_for_every_id_and_length(O, tfq):
+    """The host-side layout rules (which short-block layout a length takes) against the oracle's, which is
+    pinned to the compiled reference: all handled wire ids, every n up to a full block."""
+    L = tfq.lib()
+    out = C.c_size_t(0)
+    for name, fid in sorted(tfq.FMT.items()):
+        for n in range(1, 257):
+            want = O.block_bytes(fid, n)
+            rc = L.tfq_block_bytes(fid, n, C.byref(out))
+            if want < 0:
+                assert rc != 0, (name, n)
+            else:
+                assert rc == 0 and out.value == want, (name, n, out.value, want)

@@ -11,7 +11,8 @@ G = os.path.join(os.path.dirname(__file__), "golden")
 DECODE_FORMATS = ["Q_2", "Q_4", "Q_8", "Q_32", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_6", "Q_G_8", "Q_4_5", "Q_G_8_5",
                   "Q_G_2_K_M", "Q_G_3_K_L", "Q_G_4_K_H", "Q_G_6_K_H", "Q_2_5", "Q_G_6_5",
                   "Q_1", "Q_G_1", "Q_G_1_K_H", "Q_1_5", "Q_16", "Q_16_5", "Q_G_16", "Q_G_16_K_M", "Q_24", "Q_G_24_5", "Q_G_24",
-                  "Q_G_24_K_L",
+                  "Q_G_24_K_L", "Q_3", "Q_6", "Q_12", "Q_3_K_M", "Q_4_K_H", "Q_12_K_L", "Q_G_12", "Q_G_12_K_H", "Q_12_5",
+                  "Q_G_8_K_M",
                   "B32S4", "B32S8", "SB256A3", "SB256A2"]
 
 
@@ -73,7 +74,7 @@ def test_decode_arbitrary_payload_bits(O, tfq, gpu, fmt):
 
 TAIL_FORMATS = ["Q_2", "Q_4", "Q_8", "Q_32", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_6", "Q_G_8", "Q_G_2_K_H", "Q_G_4_K_M",
                 "Q_G_6_K_L", "Q_6_5", "SB256A3", "Q_1", "Q_G_1_K_M", "Q_1_5", "Q_16", "Q_G_16", "Q_16_5", "Q_24", "Q_G_24",
-                "Q_G_24_K_H"]
+                "Q_G_24_K_H", "Q_3", "Q_6_K_M", "Q_12", "Q_G_12", "Q_G_12_K_L", "Q_G_12_5", "Q_G_8_K_H", "Q_2_K_L"]
 
 
 @pytest.mark.parametrize("fmt", TAIL_FORMATS)
@@ -124,7 +125,9 @@ def test_half_subnormal_scales_decode_exactly(O, tfq, gpu):
                                  "Q_G_4", "Q_4_5", "Q_G_3", "Q_G_2", "SB256A3", "SB256A2", "Q_1_5",
                                  "Q_G_8", "Q_8_5", "Q_8", "Q_4", "Q_2",
                                  "Q_G_2_K_L", "Q_G_3_K_M", "Q_G_4_K_H", "Q_2_5", "Q_G_6_5", "Q_G_6", "Q_G_6_K_L", "Q_G_6_K_M",
-                                 "Q_G_6_K_H"])
+                                 "Q_G_6_K_H", "Q_3", "Q_6", "Q_12", "Q_G_12", "Q_12_5", "Q_2_K_M", "Q_2_K_H", "Q_4_K_M", "Q_4_K_H",
+                                 "Q_8_K_M", "Q_8_K_H", "Q_3_K_M", "Q_3_K_H", "Q_6_K_M", "Q_6_K_H", "Q_12_K_M", "Q_12_K_H",
+                                 "Q_G_8_K_L", "Q_G_8_K_M", "Q_G_8_K_H", "Q_G_12_K_L", "Q_G_12_K_M", "Q_G_12_K_H"])
 def test_device_encoder_codes_bit_exact(O, tfq, gpu, fmt):
     import torch
     w = _inputs(O, 64)
@@ -136,7 +139,8 @@ def test_device_encoder_codes_bit_exact(O, tfq, gpu, fmt):
 
 
 @pytest.mark.parametrize("fmt", ["Q_G_4", "Q_G_3", "Q_G_2", "SB256A3", "SB256A2", "Q_G_8", "Q_8", "Q_4", "Q_2",
-                                 "Q_G_2_K_L", "Q_G_3_K_L", "Q_G_4_K_L", "Q_6_5", "Q_G_6", "Q_G_6_K_H"])
+                                 "Q_G_2_K_L", "Q_G_3_K_L", "Q_G_4_K_L", "Q_6_5", "Q_G_6", "Q_G_6_K_H",
+                                 "Q_3", "Q_6", "Q_12", "Q_G_12", "Q_4_K_H", "Q_6_K_H", "Q_G_12_K_H", "Q_G_8_K_H"])
 def test_iterative_encoders_many_blocks(O, tfq, gpu, fmt):
     """The iterative encoders (affine: per-group Lloyd fit + joint refinement; companded 8-bit: golden-section
     scale search; lattice: least-squares refits) on thousands of blocks of four distributions: every payload
@@ -144,7 +148,7 @@ def test_iterative_encoders_many_blocks(O, tfq, gpu, fmt):
     import torch
     print(f"encode many {fmt}", flush=True)
     rs = np.random.RandomState(11)
-    n = (512 if fmt in ("Q_G_8", "Q_8") else 2048) * 256
+    n = (512 if fmt in ("Q_G_8", "Q_8", "Q_G_8_K_H", "Q_12", "Q_G_12", "Q_G_12_K_H", "Q_6_K_H") else 2048) * 256
     w = np.concatenate([(rs.randn(n) * 0.02), rs.randn(n), rs.laplace(0, 0.015, n) + 0.01, np.abs(rs.randn(n)) * 0.3]).astype(np.float32)
     got = tfq.encode(fmt, torch.from_numpy(w).to(gpu)).cpu().numpy()
     want = O.encode_tensor(fmt, w)
@@ -167,4 +171,4 @@ def test_host_pointer_codec_entry_points(O, tfq, gpu):
     assert L.tfq_decode_blocks_host(40, pay.ctypes.data, pay.size, w.size, out.ctypes.data) == 0
     assert np.array_equal(out.view(np.uint32), O.decode_tensor("Q_G_4", pay, w.size).view(np.uint32))
     # a format this build does not handle must say so, not encode on the CPU
-    assert L.tfq_encode_blocks_host(4, w.ctypes.data, w.size, dst.ctypes.data, dst.size, None) in (2, 3)
+    assert L.tfq_encode_blocks_host(91, w.ctypes.data, w.size, dst.ctypes.data, dst.size, None) in (2, 3)

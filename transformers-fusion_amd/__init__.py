@@ -31,6 +31,11 @@ FMT = {
     "Q_2_5": 74, "Q_3_5": 75, "Q_4_5": 76, "Q_6_5": 77, "Q_8_5": 78,
     "Q_G_2_5": 83, "Q_G_3_5": 84, "Q_G_4_5": 85, "Q_G_6_5": 86, "Q_G_8_5": 87,
     "B32S4": 105, "B32S8": 106, "SB256A3": 107, "SB256A2": 108,
+    "Q_3": 2, "Q_6": 4, "Q_12": 6, "Q_2_K_L": 13, "Q_2_K_M": 14, "Q_2_K_H": 15, "Q_3_K_L": 16, "Q_3_K_M": 17,
+    "Q_3_K_H": 18, "Q_4_K_L": 19, "Q_4_K_M": 20, "Q_4_K_H": 21, "Q_6_K_L": 22, "Q_6_K_M": 23, "Q_6_K_H": 24,
+    "Q_8_K_L": 25, "Q_8_K_M": 26, "Q_8_K_H": 27, "Q_12_K_L": 28, "Q_12_K_M": 29, "Q_12_K_H": 30, "Q_G_12": 43,
+    "Q_G_8_K_L": 61, "Q_G_8_K_M": 62, "Q_G_8_K_H": 63, "Q_G_12_K_L": 64, "Q_G_12_K_M": 65, "Q_G_12_K_H": 66,
+    "Q_12_5": 79, "Q_G_12_5": 88,
 }
 
 

@@ -77,6 +77,16 @@ const NameRow kNames[] = {
     {"Q_G_2_5", TFQ_Q_G_2_5}, {"Q_G_3_5", TFQ_Q_G_3_5}, {"Q_G_4_5", TFQ_Q_G_4_5}, {"Q_G_6_5", TFQ_Q_G_6_5},
     {"Q_G_8_5", TFQ_Q_G_8_5},
     {"B32S4", TFQ_B32S4}, {"B32S8", TFQ_B32S8}, {"SB256A3", TFQ_SB256A3}, {"SB256A2", TFQ_SB256A2},
+    {"Q_3", TFQ_Q_3}, {"Q_6", TFQ_Q_6}, {"Q_12", TFQ_Q_12},
+    {"Q_2_K_L", TFQ_Q_2_K_L}, {"Q_2_K_M", TFQ_Q_2_K_M}, {"Q_2_K_H", TFQ_Q_2_K_H},
+    {"Q_3_K_L", TFQ_Q_3_K_L}, {"Q_3_K_M", TFQ_Q_3_K_M}, {"Q_3_K_H", TFQ_Q_3_K_H},
+    {"Q_4_K_L", TFQ_Q_4_K_L}, {"Q_4_K_M", TFQ_Q_4_K_M}, {"Q_4_K_H", TFQ_Q_4_K_H},
+    {"Q_6_K_L", TFQ_Q_6_K_L}, {"Q_6_K_M", TFQ_Q_6_K_M}, {"Q_6_K_H", TFQ_Q_6_K_H},
+    {"Q_8_K_L", TFQ_Q_8_K_L}, {"Q_8_K_M", TFQ_Q_8_K_M}, {"Q_8_K_H", TFQ_Q_8_K_H},
+    {"Q_12_K_L", TFQ_Q_12_K_L}, {"Q_12_K_M", TFQ_Q_12_K_M}, {"Q_12_K_H", TFQ_Q_12_K_H},
+    {"Q_G_12", TFQ_Q_G_12}, {"Q_G_8_K_L", TFQ_Q_G_8_K_L}, {"Q_G_8_K_M", TFQ_Q_G_8_K_M}, {"Q_G_8_K_H", TFQ_Q_G_8_K_H},
+    {"Q_G_12_K_L", TFQ_Q_G_12_K_L}, {"Q_G_12_K_M", TFQ_Q_G_12_K_M}, {"Q_G_12_K_H", TFQ_Q_G_12_K_H},
+    {"Q_12_5", TFQ_Q_12_5}, {"Q_G_12_5", TFQ_Q_G_12_5},
 };
 
 std::string normalise(const char* s) {
@@ -124,7 +134,7 @@ const char* tfq_format_name(uint8_t fmt) {
     return "unknown";
 }
 
-float tfq_format_bpw(uint8_t fmt) { return spec_of(fmt).bpw; }
+float tfq_format_bpw(uint8_t fmt) { return reported_bpw(fmt); }
 
 int tfq_format_supported(uint8_t fmt) { return spec_of(fmt).codec != Codec::None; }
 

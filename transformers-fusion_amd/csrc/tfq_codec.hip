@@ -532,7 +532,7 @@ struct Comp8Team {
 // FMT = Q_G_8: grid = 8 groups per block, a wavefront each (32 lanes hold a weight).  FMT = Q_8: a wavefront
 // per block, four weights per lane.
 template <int FMT>
-__global__ __launch_bounds__(64) void encode_comp8_kernel(const float* __restrict__ wg, uint8_t* __restrict__ dst) {
+__global__ __launch_bounds__(64) void encode_comp8_kernel(const float* __restrict__ wg, uint8_t* __restrict__ dst, float smult) {
     constexpr bool GROUPED = spec_of(FMT).codec == Codec::Grp8;
     constexpr int CNT = GROUPED ? 32 : 256;
     __shared__ float lv[256];
@@ -550,7 +550,7 @@ __global__ __launch_bounds__(64) void encode_comp8_kernel(const float* __restric
 #pragma unroll
     for (int sft = 32; sft >= 1; sft >>= 1) m = fmaxf(m, __shfl_xor(m, sft, 64));
     Comp8Team<CNT> team{lv, buf, res, w, lane};
-    const float s = team.fit((double)m);
+    const float s = team.fit((double)m) * smult;  // the _K tiers try scaled copies of the fitted scale
     for (int i = lane; i < CNT; i += 64) code[i] = (uint8_t)((s > 0.0f) ? team.nearest(w[i] / s) : 0u);
     __syncthreads();
     const uint32_t h = float_to_half_bits(s);
@@ -582,18 +582,26 @@ __global__ __launch_bounds__(64) void encode_comp8_kernel(const float* __restric
     }
 }
 
-// Plain lattice encoders Q_4 / Q_2 (quant_lattice, src/codec/block_codec.cpp:443-497): s = absmax / top level,
-// two least-squares refits over the nearest levels, binary16; codes are the nearest level of w / s, slots
-// (every 16th weight) keep the even index below.  A wavefront per block; sums in index order on lane 0.
+// Plain lattice encoders Q_4 / Q_2 (quant_lattice, src/codec/block_codec.cpp:443-497) and the fixed-codebook
+// encoders Q_3 / Q_6 / Q_12 (quant_fixed_codebook, :624-663), which differ in the level table only:
+// s = absmax / top level * smult, `iters` least-squares refits over the nearest levels, binary16; codes are the
+// nearest level of w / s, slots (every 16th weight) keep the even index below.  The base ids run 2 (lattice) or
+// 3 (fixed) refits with smult 1; the _K tiers try more.  A wavefront per block; sums in index order on lane 0.
 template <int FMT>
-__global__ __launch_bounds__(64) void encode_lattice_kernel(const float* __restrict__ wg, uint8_t* __restrict__ dst) {
-    constexpr int bits = spec_of(FMT).bits, BB = spec_of(FMT).block_bytes, CHUNK = 16 * bits - 1;
+__global__ __launch_bounds__(64) void encode_lattice_kernel(const float* __restrict__ wg, uint8_t* __restrict__ dst,
+                                                            int iters, float smult) {
+    constexpr Spec sp = spec_of(FMT);
+    constexpr int bits = sp.bits, BB = sp.block_bytes, CHUNK = 16 * bits - 1, NL = 1 << bits;
+    constexpr bool FIXED = sp.codec == Codec::Fixed;
+    constexpr bool SEARCH = FIXED && bits > 3;  // ascending quantile table: binary search on |v| (:596-622)
+    __shared__ float tab[NL];
     __shared__ float w[256];
     __shared__ float lev[256];
     __shared__ float sres;
-    __shared__ uint8_t code[256];
+    __shared__ uint16_t code[256];
     const int lane = threadIdx.x;
     const int64_t blk = blockIdx.x;
+    for (int i = lane; i < NL; i += 64) tab[i] = FIXED ? fixed_value(bits, (uint32_t)i) : grid_value(bits, (uint32_t)i);
     for (int i = lane; i < 256; i += 64) w[i] = wg[blk * 256 + i];
     __syncthreads();
     float m = 0.0f;
@@ -601,18 +609,34 @@ __global__ __launch_bounds__(64) void encode_lattice_kernel(const float* __restr
 #pragma unroll
     for (int sft = 32; sft >= 1; sft >>= 1) m = fmaxf(m, __shfl_xor(m, sft, 64));
     auto nearest = [&](float v) __attribute__((always_inline)) {
-        uint32_t best = 0;
-        float bd = fabsf(v - grid_value(bits, 0));
-        for (int i = 1; i < (1 << bits); ++i) {
-            const float d = fabsf(v - grid_value(bits, (uint32_t)i));
-            if (d < bd) { bd = d; best = (uint32_t)i; }
+        if constexpr (SEARCH) {
+            constexpr int half = NL / 2;
+            const float a = fabsf(v);
+            int lo = half, hi = NL - 1;
+            while (lo < hi) {
+                const int mid = (lo + hi) / 2;
+                if (tab[mid] < a) lo = mid + 1; else hi = mid;
+            }
+            if (lo > half) {
+                const float d0 = a - tab[lo - 1];
+                const float d1 = tab[lo] - a;
+                if (d1 >= d0) --lo;
+            }
+            return (v >= 0.0f) ? (uint32_t)lo : (uint32_t)(half - 1 - (lo - half));
+        } else {
+            uint32_t best = 0;
+            float bd = fabsf(v - tab[0]);
+            for (int i = 1; i < NL; ++i) {
+                const float d = fabsf(v - tab[i]);
+                if (d < bd) { bd = d; best = (uint32_t)i; }
+            }
+            return best;
         }
-        return best;
     };
-    float s = (m > 1e-30f) ? m / (bits == 2 ? 1.5104f : 2.7178f) : 0.0f;
+    float s = (m > 1e-30f) ? m / tab[NL - 1] * smult : 0.0f;
     if (s > 0.0f) {
-        for (int it = 0; it < 2; ++it) {
-            for (int i = lane; i < 256; i += 64) lev[i] = grid_value(bits, nearest(w[i] / s));
+        for (int it = 0; it < iters; ++it) {
+            for (int i = lane; i < 256; i += 64) lev[i] = tab[nearest(w[i] / s)];
             __syncthreads();
             if (lane == 0) {
                 double num = 0.0, den = 0.0;
@@ -628,7 +652,7 @@ __global__ __launch_bounds__(64) void encode_lattice_kernel(const float* __restr
         }
     }
     if (!(s > 0.0f)) s = 0.0f;
-    for (int i = lane; i < 256; i += 64) code[i] = (uint8_t)nearest((s == 0.0f) ? 0.0f : w[i] / s);
+    for (int i = lane; i < 256; i += 64) code[i] = (uint16_t)nearest((s == 0.0f) ? 0.0f : w[i] / s);
     __syncthreads();
     const uint32_t h = float_to_half_bits(s);
     uint8_t* p = dst + blk * BB;
@@ -648,6 +672,77 @@ __global__ __launch_bounds__(64) void encode_lattice_kernel(const float* __restr
             v |= bit << b;
         }
         p[byte] = (uint8_t)v;
+    }
+}
+
+// 12-bit compound encoder (quant_grp12_compound, src/codec/block_codec.cpp:969-1004): every group of 32 weights
+// gets its own least-squares scale against the 4096-level table (same fit as above on 32 weights), then 256
+// 12-bit codes and the eight binary16 scales.  A wavefront per block: eight lanes per group hold four weights
+// each, the first lane of a group sums it in index order.
+__global__ __launch_bounds__(64) void encode_grp12_kernel(const float* __restrict__ wg, uint8_t* __restrict__ dst,
+                                                          int iters, float smult) {
+    __shared__ float tab[4096];
+    __shared__ float w[256];
+    __shared__ float lev[256];
+    __shared__ float sg[8];
+    __shared__ uint16_t code[256];
+    const int lane = threadIdx.x, g = lane >> 3;
+    const int64_t blk = blockIdx.x;
+    for (int i = lane; i < 4096; i += 64) tab[i] = fixed_value(12, (uint32_t)i);
+    for (int i = lane; i < 256; i += 64) w[i] = wg[blk * 256 + i];
+    __syncthreads();
+    auto nearest = [&](float v) __attribute__((always_inline)) {
+        const float a = fabsf(v);
+        int lo = 2048, hi = 4095;
+        while (lo < hi) {
+            const int mid = (lo + hi) / 2;
+            if (tab[mid] < a) lo = mid + 1; else hi = mid;
+        }
+        if (lo > 2048) {
+            const float d0 = a - tab[lo - 1];
+            const float d1 = tab[lo] - a;
+            if (d1 >= d0) --lo;
+        }
+        return (v >= 0.0f) ? (uint32_t)lo : (uint32_t)(2047 - (lo - 2048));
+    };
+    // weights 4 (lane & 7) .. + 3 of group g: lanes of one group are consecutive, so an 8-lane max suffices
+    float m = 0.0f;
+    for (int t = 0; t < 4; ++t) m = fmaxf(m, fabsf(w[4 * lane + t]));
+#pragma unroll
+    for (int sft = 4; sft >= 1; sft >>= 1) m = fmaxf(m, __shfl_xor(m, sft, 64));
+    float s = (m > 1e-30f) ? m / tab[4095] * smult : 0.0f;
+    const bool live = s > 0.0f;  // per group; the refits run to the end once started, like the reference's
+    for (int it = 0; it < iters; ++it) {
+        if (live)
+            for (int t = 0; t < 4; ++t) lev[4 * lane + t] = tab[nearest(w[4 * lane + t] / s)];
+        __syncthreads();
+        if (live && (lane & 7) == 0) {
+            double num = 0.0, den = 0.0;
+            for (int i = 32 * g; i < 32 * g + 32; ++i) {
+                num = __builtin_fma((double)w[i], (double)lev[i], num);
+                den = __builtin_fma((double)lev[i], (double)lev[i], den);
+            }
+            sg[g] = (den > 1e-20) ? (float)(num / den) : s;
+        }
+        __syncthreads();
+        if (live) s = sg[g];
+        __syncthreads();
+    }
+    if (!(s > 0.0f)) s = 0.0f;
+    for (int t = 0; t < 4; ++t) code[4 * lane + t] = (uint16_t)((s > 0.0f) ? nearest(w[4 * lane + t] / s) : 0u);
+    if ((lane & 7) == 0) sg[g] = s;
+    __syncthreads();
+    uint8_t* p = dst + blk * 400;
+    for (int byte = lane; byte < 384; byte += 64) {
+        // two codes in three bytes
+        const int pair = byte / 3, part = byte - 3 * pair;
+        const uint32_t two = (uint32_t)code[2 * pair] | ((uint32_t)code[2 * pair + 1] << 12);
+        p[byte] = (uint8_t)(two >> (8 * part));
+    }
+    if (lane < 8) {
+        const uint32_t h = float_to_half_bits(sg[lane]);
+        p[384 + 2 * lane] = (uint8_t)(h & 0xFF);
+        p[385 + 2 * lane] = (uint8_t)(h >> 8);
     }
 }
 
@@ -908,20 +1003,22 @@ __global__ __launch_bounds__(64) void encode_q6k_kernel(const float* __restrict_
     }
 }
 
-// Q_G_6_K_M / _K_H (src/codec/block_codec.cpp:2733-2755): a candidate payload replaces the current one when
-// its decoded mean squared error (double, index order, fused like the reference's k_mse) is strictly smaller.
-// One wavefront per block: lanes decode both payloads, lane 0 compares, all lanes copy.
-__global__ __launch_bounds__(64) void keep_better_q6k_kernel(const float* __restrict__ wg, uint8_t* __restrict__ cur,
-                                                             const uint8_t* __restrict__ cand) {
+// _K_M / _K_H tiers (src/codec/block_codec.cpp:2378-2400, :2551-2665, :2733-2824): a candidate payload replaces
+// the current one when its decoded mean squared error (double, index order, fused like the reference's k_mse)
+// is strictly smaller.  One wavefront per block: lanes decode both payloads, lane 0 compares, all lanes copy.
+template <int FMT>
+__global__ __launch_bounds__(64) void keep_better_kernel(const float* __restrict__ wg, uint8_t* __restrict__ cur,
+                                                         const uint8_t* __restrict__ cand) {
+    constexpr int BB = spec_of(FMT).block_bytes;
     __shared__ float dc[256], dn[256];
     __shared__ int take;
     const int64_t blk = blockIdx.x;
     const int t = threadIdx.x;
-    uint8_t* pc = cur + blk * 210;
-    const uint8_t* pn = cand + blk * 210;
+    uint8_t* pc = cur + blk * BB;
+    const uint8_t* pn = cand + blk * BB;
     for (int i = t; i < 256; i += 64) {
-        dc[i] = decode_weight<TFQ_Q_G_6>(pc, i);
-        dn[i] = decode_weight<TFQ_Q_G_6>(pn, i);
+        dc[i] = decode_weight<FMT>(pc, i);
+        dn[i] = decode_weight<FMT>(pn, i);
     }
     __syncthreads();
     if (t == 0) {
@@ -936,7 +1033,7 @@ __global__ __launch_bounds__(64) void keep_better_q6k_kernel(const float* __rest
     }
     __syncthreads();
     if (take)
-        for (int i = t; i < 210; i += 64) pc[i] = pn[i];
+        for (int i = t; i < BB; i += 64) pc[i] = pn[i];
 }
 
 // Wire -> Tiled16: one lane per 16-byte piece of the tiled buffer.  Piece p of a unit: p < 64 code
@@ -1095,7 +1192,14 @@ bool block_layout(int fmt, int n, BlockLayout* L) {
             return affine_or_fallback(sp.bits, sp.gsz, sp.scb, sp.mb, (double)sp.bpw, n, L);
         case Codec::Grp8:
             if (n >= 32 && n % 32 == 0) { *L = {BK_GRP8, 8, n, n + (n / 32) * 2, 32, n / 32, 0, 0, 0}; return true; }
-            return affine_or_fallback(8, 32, 6, 6, 8.5, n, L);
+            return affine_or_fallback(8, 32, 6, 6, (double)sp.bpw, n, L);  // 8.5, or 8.0 for the _K tiers
+        case Codec::Fixed:
+            *L = {n < 16 ? BK_LEVELS : BK_LATTICE, sp.bits, n, (sp.bits * n + 7) / 8, 0, 0, 0, 0, 1};
+            return true;
+        case Codec::Grp12:
+            if (n >= 32 && n % 32 == 0) { *L = {BK_GRP12, 12, n, n * 3 / 2 + (n / 32) * 2, 32, n / 32, 0, 0, 0}; return true; }
+            if (sp.scb) { *L = {n < 16 ? BK_LEVELS : BK_LATTICE, 12, n, (12 * n + 7) / 8, 0, 0, 0, 0, 1}; return true; }
+            return affine_or_fallback(12, 512, 0, 0, 12.5, n, L);  // no affine layout: the grouped-lattice fallback
         case Codec::Q6K: {
             const int levels = (n * 6 + 7) / 8, sc_count = n >= 32 ? n / 16 : 0;
             const int budget = (int)std::ceil(6.5625 * (double)n / 8.0);
@@ -1141,6 +1245,10 @@ int launch_decode(int fmt, const uint8_t* src, int64_t nblocks, float* out, hipS
         case TFQ_Q_24_5: return run_decode<TFQ_Q_24_5>(src, nblocks, out, s);
         case TFQ_Q_G_24: return run_decode<TFQ_Q_G_24>(src, nblocks, out, s);
         case TFQ_Q_2: return run_decode<TFQ_Q_2>(src, nblocks, out, s);
+        case TFQ_Q_3: return run_decode<TFQ_Q_3>(src, nblocks, out, s);
+        case TFQ_Q_6: return run_decode<TFQ_Q_6>(src, nblocks, out, s);
+        case TFQ_Q_12: return run_decode<TFQ_Q_12>(src, nblocks, out, s);
+        case TFQ_Q_G_12: return run_decode<TFQ_Q_G_12>(src, nblocks, out, s);
         case TFQ_Q_G_6: return run_decode<TFQ_Q_G_6>(src, nblocks, out, s);
         case TFQ_Q_G_2_K_L: return run_decode<TFQ_Q_G_2_K_L>(src, nblocks, out, s);
         case TFQ_Q_G_3_K_L: return run_decode<TFQ_Q_G_3_K_L>(src, nblocks, out, s);
@@ -1212,6 +1320,43 @@ int launch_decode_tiled(int fmt, const uint8_t* tiled, int64_t N, int64_t K, flo
     }
 }
 
+// One more search per candidate (iters, smult), each kept only where it decodes strictly better than what
+// `dst` holds.  `launch(out, iters, smult)` enqueues the encoder of the family.
+struct TierTry { int iters; float smult; };
+
+template <int FMT, class Launch>
+static int encode_tiers(const TierTry* tries, int count, const float* w, int64_t nblocks, uint8_t* dst, hipStream_t s,
+                        Launch&& launch) {
+    if (count <= 0) return TFQ_OK;
+    constexpr size_t BB = spec_of(FMT).block_bytes;
+    uint8_t* cand = nullptr;
+    TFQ_HIP(hipMalloc(&cand, (size_t)nblocks * BB));
+    for (int c = 0; c < count; ++c) {
+        launch(cand, tries[c].iters, tries[c].smult);
+        hipLaunchKernelGGL(keep_better_kernel<FMT>, dim3((unsigned)nblocks), dim3(64), 0, s, w, dst, (const uint8_t*)cand);
+    }
+    const hipError_t e1 = hipStreamSynchronize(s);
+    (void)hipFree(cand);
+    if (e1 != hipSuccess) return hip_fail(e1, "hipStreamSynchronize");
+    return TFQ_OK;
+}
+
+// Lattice and fixed-codebook ids with their tiers: base (iters0, 1.0), _K_M one longer search, _K_H six
+// (src/codec/block_codec.cpp:2551-2665).
+template <int FMT>
+static int encode_lattice_family(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStream_t s) {
+    constexpr bool FIXED = spec_of(FMT).codec == Codec::Fixed;
+    const dim3 grid((unsigned)nblocks);
+    auto launch = [&](uint8_t* out, int iters, float smult) {
+        hipLaunchKernelGGL(encode_lattice_kernel<FMT>, grid, dim3(64), 0, s, w, out, iters, smult);
+    };
+    launch(dst, FIXED ? 3 : 2, 1.0f);
+    const int a = FIXED ? 10 : 6, b = FIXED ? 24 : 14;
+    const TierTry tries[6] = {{a, 1.0f}, {b, 1.0f}, {b, 0.9f}, {b, 1.1f}, {b, 0.7f}, {b, 1.3f}};
+    const int tier = tier_of(fmt);
+    return encode_tiers<FMT>(tries, tier >= 2 ? 6 : tier, w, nblocks, dst, s, launch);
+}
+
 int launch_encode(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStream_t s) {
     if (nblocks <= 0) return TFQ_OK;
     if (nblocks > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "encode: more than 2^31-1 blocks in one call");
@@ -1228,11 +1373,46 @@ int launch_encode(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStr
         case TFQ_Q_1_5: hipLaunchKernelGGL(encode_affine_kernel<TFQ_Q_1_5>, grid, dim3(64), 0, s, w, dst); break;
         case TFQ_Q_G_8:
             if (nblocks * 8 > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "encode: too many groups in one call");
-            hipLaunchKernelGGL(encode_comp8_kernel<TFQ_Q_G_8>, dim3((unsigned)(nblocks * 8)), dim3(64), 0, s, w, dst);
+            hipLaunchKernelGGL(encode_comp8_kernel<TFQ_Q_G_8>, dim3((unsigned)(nblocks * 8)), dim3(64), 0, s, w, dst, 1.0f);
+            if (const int tier = tier_of(fmt)) {
+                // :2756-2772: scaled copies of every group's fitted scale, the last two for _K_M, all six for _K_H
+                const TierTry tries[6] = {{0, 0.7f}, {0, 0.9f}, {0, 0.95f}, {0, 1.05f}, {0, 1.1f}, {0, 1.3f}};
+                const int count = tier >= 2 ? 6 : 2;
+                const int rc = encode_tiers<TFQ_Q_G_8>(tries + 6 - count, count, w, nblocks, dst, s, [&](uint8_t* out, int, float smult) {
+                    hipLaunchKernelGGL(encode_comp8_kernel<TFQ_Q_G_8>, dim3((unsigned)(nblocks * 8)), dim3(64), 0, s, w, out, smult);
+                });
+                if (rc != TFQ_OK) return rc;
+            }
             break;
-        case TFQ_Q_8: hipLaunchKernelGGL(encode_comp8_kernel<TFQ_Q_8>, grid, dim3(64), 0, s, w, dst); break;
-        case TFQ_Q_4: hipLaunchKernelGGL(encode_lattice_kernel<TFQ_Q_4>, grid, dim3(64), 0, s, w, dst); break;
-        case TFQ_Q_2: hipLaunchKernelGGL(encode_lattice_kernel<TFQ_Q_2>, grid, dim3(64), 0, s, w, dst); break;
+        case TFQ_Q_8:
+            hipLaunchKernelGGL(encode_comp8_kernel<TFQ_Q_8>, grid, dim3(64), 0, s, w, dst, 1.0f);
+            if (tier_of(fmt) >= 2) {
+                // :2627-2645: the tries with smult 1 repeat the base payload (the 8-bit fit takes no iteration
+                // count), so _K_M equals _K_L and _K_H has four scaled tries
+                const TierTry tries[4] = {{0, 0.9f}, {0, 1.1f}, {0, 0.7f}, {0, 1.3f}};
+                const int rc = encode_tiers<TFQ_Q_8>(tries, 4, w, nblocks, dst, s, [&](uint8_t* out, int, float smult) {
+                    hipLaunchKernelGGL(encode_comp8_kernel<TFQ_Q_8>, grid, dim3(64), 0, s, w, out, smult);
+                });
+                if (rc != TFQ_OK) return rc;
+            }
+            break;
+        case TFQ_Q_4: { const int rc = encode_lattice_family<TFQ_Q_4>(fmt, w, nblocks, dst, s); if (rc != TFQ_OK) return rc; break; }
+        case TFQ_Q_2: { const int rc = encode_lattice_family<TFQ_Q_2>(fmt, w, nblocks, dst, s); if (rc != TFQ_OK) return rc; break; }
+        case TFQ_Q_3: { const int rc = encode_lattice_family<TFQ_Q_3>(fmt, w, nblocks, dst, s); if (rc != TFQ_OK) return rc; break; }
+        case TFQ_Q_6: { const int rc = encode_lattice_family<TFQ_Q_6>(fmt, w, nblocks, dst, s); if (rc != TFQ_OK) return rc; break; }
+        case TFQ_Q_12: { const int rc = encode_lattice_family<TFQ_Q_12>(fmt, w, nblocks, dst, s); if (rc != TFQ_OK) return rc; break; }
+        case TFQ_Q_G_12: {
+            auto launch = [&](uint8_t* out, int iters, float smult) {
+                hipLaunchKernelGGL(encode_grp12_kernel, grid, dim3(64), 0, s, w, out, iters, smult);
+            };
+            launch(dst, 3, 1.0f);
+            // :2788-2810; the second try repeats the first
+            const TierTry tries[5] = {{8, 1.0f}, {20, 0.93f}, {20, 1.07f}, {20, 0.7f}, {20, 1.3f}};
+            const int tier = tier_of(fmt);
+            const int rc = encode_tiers<TFQ_Q_G_12>(tries, tier >= 2 ? 5 : tier, w, nblocks, dst, s, launch);
+            if (rc != TFQ_OK) return rc;
+            break;
+        }
         case TFQ_Q_G_2_K_L: hipLaunchKernelGGL(encode_grp16_kernel<TFQ_Q_G_2_K_L>, grid, dim3(64), 0, s, w, dst); break;
         case TFQ_Q_G_3_K_L: hipLaunchKernelGGL(encode_grp16_kernel<TFQ_Q_G_3_K_L>, grid, dim3(64), 0, s, w, dst); break;
         case TFQ_Q_G_4_K_L: hipLaunchKernelGGL(encode_grp16_kernel<TFQ_Q_G_4_K_L>, grid, dim3(64), 0, s, w, dst); break;
@@ -1248,7 +1428,7 @@ int launch_encode(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStr
                 const int effort[2][3] = {{8, 5, 6}, {14, 8, 10}};
                 for (int c = 0; c < (fmt == TFQ_Q_G_6_K_H ? 2 : 1); ++c) {
                     hipLaunchKernelGGL(encode_q6k_kernel, grid, dim3(64), 0, s, w, cand, effort[c][0], effort[c][1], effort[c][2]);
-                    hipLaunchKernelGGL(keep_better_q6k_kernel, grid, dim3(64), 0, s, w, dst, (const uint8_t*)cand);
+                    hipLaunchKernelGGL(keep_better_kernel<TFQ_Q_G_6>, grid, dim3(64), 0, s, w, dst, (const uint8_t*)cand);
                 }
                 const hipError_t e1 = hipStreamSynchronize(s);
                 (void)hipFree(cand);

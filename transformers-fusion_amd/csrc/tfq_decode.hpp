@@ -29,6 +29,22 @@ __device__ __constant__ static const float kGrid4[16] = {
 
 __device__ __constant__ static const float kGrid2[4] = {-1.5104f, -0.4528f, 0.4528f, 1.5104f};
 
+// fixed shared codebooks (src/codec/block_codec.cpp:530-594): eight Lloyd-Max levels of N(0,1)
+// for 3 bits, the 64 / 4096 mid-quantiles of N(0,1) for 6 and 12 bits
+__device__ __constant__ static const float kFixed3[8] = {-3.0776f, -2.1479f, -1.2879f, -0.4240f,
+                                                         0.4240f,  1.2879f,  2.1479f,  3.0776f};
+__device__ __constant__ static const uint32_t kFixed6Bits[64] = {
+#include "fixed6_levels.inc"
+};
+__device__ __constant__ static const uint32_t kFixed12Bits[4096] = {
+#include "fixed12_levels.inc"
+};
+__device__ __forceinline__ float fixed_value(int bits, uint32_t idx) {
+    if (bits == 3) return kFixed3[idx & 7u];
+    if (bits == 6) return __uint_as_float(kFixed6Bits[min(idx, 63u)]);
+    return __uint_as_float(kFixed12Bits[min(idx, 4095u)]);
+}
+
 // plain lattice grid (level_value, src/codec/block_codec.cpp:182-188): Lloyd-Max tables
 // for 2 and 4 bits, -8 + 16 i / (2^bits - 1) otherwise
 __device__ __forceinline__ float grid_value(int bits, uint32_t idx) {
@@ -58,7 +74,7 @@ __device__ __forceinline__ float decode_weight(const uint8_t* __restrict__ p, ui
     float v = 0.0f;
     if constexpr (sp.codec == Codec::Raw32) {
         v = __uint_as_float(stream_bits(p, BB, i * 32, 16) | (stream_bits(p, BB, i * 32 + 16, 16) << 16));
-    } else if constexpr (sp.codec == Codec::Lattice) {
+    } else if constexpr (sp.codec == Codec::Lattice || sp.codec == Codec::Fixed) {
         // [binary16 scale][256 codes]; every 16th weight (i % 16 == 15) is a
         // slot that stores one bit less and decodes as an even index.
         const float scale = half_bits_to_float(stream_bits(p, BB, 0, 16));
@@ -66,8 +82,14 @@ __device__ __forceinline__ float decode_weight(const uint8_t* __restrict__ p, ui
         const uint32_t pos = 16u + (uint32_t)sp.bits * i - (i >> 4);
         uint32_t idx = stream_bits(p, BB, pos, sp.bits - (slot ? 1 : 0));
         if (slot) idx <<= 1;
-        if constexpr (sp.bits == 8) v = scale * __uint_as_float(kComp8Bits[min(idx, 255u)]);
+        if constexpr (sp.codec == Codec::Fixed) v = fixed_value(sp.bits, idx) * scale;
+        else if constexpr (sp.bits == 8) v = scale * __uint_as_float(kComp8Bits[min(idx, 255u)]);
         else v = grid_value(sp.bits, idx) * scale;
+    } else if constexpr (sp.codec == Codec::Grp12) {
+        // [256 12-bit codes of the fixed table][8 binary16 scales]
+        const uint32_t idx = stream_bits(p, BB, i * 12u, 12);
+        const uint32_t h = (uint32_t)p[384 + 2 * (i >> 5)] | ((uint32_t)p[384 + 2 * (i >> 5) + 1] << 8);
+        v = half_bits_to_float(h) * fixed_value(12, idx);
     } else if constexpr (sp.codec == Codec::Grp8) {
         const uint32_t g = i >> 5;
         const uint32_t h = (uint32_t)p[256 + 2 * g] | ((uint32_t)p[256 + 2 * g + 1] << 8);
@@ -154,7 +176,8 @@ __device__ __forceinline__ uint32_t half_at(const uint8_t* p) { return *reinterp
 
 template <int FMT>
 constexpr bool kHasQuad = spec_of(FMT).codec == Codec::Raw32 || spec_of(FMT).codec == Codec::Lattice ||
-                          spec_of(FMT).codec == Codec::Grp16 || spec_of(FMT).codec == Codec::Q6K;
+                          spec_of(FMT).codec == Codec::Grp16 || spec_of(FMT).codec == Codec::Q6K ||
+                          spec_of(FMT).codec == Codec::Fixed || spec_of(FMT).codec == Codec::Grp12;
 
 // v[t] = decode_weight<FMT>(p, 4 * lane + t), the same arithmetic on the same operands
 template <int FMT>
@@ -165,18 +188,30 @@ __device__ __forceinline__ void decode_quad(const uint8_t* __restrict__ p, uint3
     if constexpr (sp.codec == Codec::Raw32) {
         const uint4 q = *reinterpret_cast<const uint4*>(p + 16 * lane);
         v[0] = __uint_as_float(q.x); v[1] = __uint_as_float(q.y); v[2] = __uint_as_float(q.z); v[3] = __uint_as_float(q.w);
-    } else if constexpr (sp.codec == Codec::Lattice) {
+    } else if constexpr (sp.codec == Codec::Lattice || sp.codec == Codec::Fixed) {
         const float scale = half_bits_to_float(half_at(p));
         const uint32_t i0 = 4 * lane;
-        const uint32_t w = window32(p, 16u + bits * i0 - (i0 >> 4), limit);
+        const uint32_t pos = 16u + bits * i0 - (i0 >> 4);
+        constexpr bool two = bits * 4 > 32;  // 12-bit codes: two windows of two codes each
+        const uint32_t w = window32(p, pos, limit);
+        uint32_t w2 = 0;
+        if constexpr (two) w2 = window32(p, pos + 2 * bits, limit);
 #pragma unroll
         for (uint32_t t = 0; t < 4; ++t) {
             const bool slot = t == 3 && (lane & 3u) == 3u;  // weight i is a slot when i % 16 == 15
-            uint32_t idx = (w >> (bits * t)) & ((1u << (bits - (slot ? 1 : 0))) - 1u);
+            const uint32_t src = (two && t >= 2) ? w2 >> (bits * (t & 1u)) : w >> (bits * t);
+            uint32_t idx = src & ((1u << (bits - (slot ? 1 : 0))) - 1u);
             if (slot) idx <<= 1;
-            if constexpr (bits == 8) v[t] = scale * __uint_as_float(kComp8Bits[min(idx, 255u)]);
+            if constexpr (sp.codec == Codec::Fixed) v[t] = fixed_value(bits, idx) * scale;
+            else if constexpr (bits == 8) v[t] = scale * __uint_as_float(kComp8Bits[min(idx, 255u)]);
             else v[t] = grid_value(bits, idx) * scale;
         }
+    } else if constexpr (sp.codec == Codec::Grp12) {
+        const uint32_t w = window32(p, 48u * lane, limit), w2 = window32(p, 48u * lane + 24u, limit);
+        const float sc = half_bits_to_float(half_at(p + 384 + 2 * (lane >> 3)));
+#pragma unroll
+        for (uint32_t t = 0; t < 4; ++t)
+            v[t] = sc * fixed_value(12, ((t >= 2 ? w2 : w) >> (12u * (t & 1u))) & 4095u);
     } else if constexpr (sp.codec == Codec::Grp16) {
         constexpr uint32_t lev_bits = 256u * bits;
         const uint32_t w = window32(p, 4u * bits * lane, limit);
@@ -201,8 +236,10 @@ __device__ __forceinline__ float decode_weight_short(const BlockLayout& L, const
     switch (L.kind) {
         case BK_RAW32:
             return __uint_as_float(stream_bits(p, size, i * 32, 16) | (stream_bits(p, size, i * 32 + 16, 16) << 16));
-        case BK_LEVELS:  // fewer than 16 weights: no header, implied scale 1 (:450-455, :508-511)
-            return grid_value(L.bits, stream_bits(p, size, i * bits, L.bits));
+        case BK_LEVELS: {  // fewer than 16 weights: no header, implied scale 1 (:450-455, :508-511, :629-633)
+            const uint32_t idx = stream_bits(p, size, i * bits, L.bits);
+            return L.aux ? fixed_value(L.bits, idx) : grid_value(L.bits, idx);
+        }
         case BK_LATTICE: {
             // 16 slots spread by is_slot (:176-180): weight i is one when floor(16 (i + 1) / n) steps
             const uint32_t before = (i * 16u) / n;
@@ -210,8 +247,14 @@ __device__ __forceinline__ float decode_weight_short(const BlockLayout& L, const
             const float scale = half_bits_to_float(stream_bits(p, size, 0, 16));
             uint32_t idx = stream_bits(p, size, 16u + bits * i - before, L.bits - (slot ? 1 : 0));
             if (slot) idx <<= 1;
+            if (L.aux) return fixed_value(L.bits, idx) * scale;
             if (L.bits == 8) return scale * __uint_as_float(kComp8Bits[min(idx, 255u)]);
             return grid_value(L.bits, idx) * scale;
+        }
+        case BK_GRP12: {  // whole groups of 32: n 12-bit codes, then a binary16 scale per group (byte aligned)
+            const uint32_t at = n * 3u / 2u + 2u * (i >> 5);
+            const uint32_t h = (uint32_t)p[at] | ((uint32_t)p[at + 1] << 8);
+            return half_bits_to_float(h) * fixed_value(12, stream_bits(p, size, i * 12u, 12));
         }
         case BK_AFFINE: {
             // the decoder reads n levels, then ng scale codes, ng min codes, d, dm; weights past

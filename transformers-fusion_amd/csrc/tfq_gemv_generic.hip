@@ -136,6 +136,10 @@ int launch_gemv_generic(const tfq_weight* w, const void* x, int x_dtype, int B, 
         case TFQ_Q_G_4_K_L: return batched<TFQ_Q_G_4_K_L>(w, x, x_dtype, B, y, y_dtype, s);
         case TFQ_Q_6_5: return batched<TFQ_Q_6_5>(w, x, x_dtype, B, y, y_dtype, s);
         case TFQ_Q_4: return batched<TFQ_Q_4>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_3: return batched<TFQ_Q_3>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_6: return batched<TFQ_Q_6>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_12: return batched<TFQ_Q_12>(w, x, x_dtype, B, y, y_dtype, s);
+        case TFQ_Q_G_12: return batched<TFQ_Q_G_12>(w, x, x_dtype, B, y, y_dtype, s);
         default:
             return fail(TFQ_ERR_FORMAT, std::string("gemv: no kernel for format ") + tfq_format_name(w->fmt));
     }

@@ -13,7 +13,7 @@
 namespace tfq {
 
 // ------------------------------------------------------------------ formats
-enum class Codec : int { None = 0, Raw32, Lattice, Affine, Grp8, Sym32, Grp16, Q6K, Q1, Q16, Q24 };
+enum class Codec : int { None = 0, Raw32, Lattice, Affine, Grp8, Sym32, Grp16, Q6K, Q1, Q16, Q24, Fixed, Grp12 };
 
 // Layout parameters of one wire format.  The affine family is the reference's
 // parametric codec quant_affine(bits, w, n, gsz, scb, mb, claimed)
@@ -52,13 +52,23 @@ __host__ __device__ constexpr Spec spec_of(int fmt) {
         case TFQ_Q_24_5: case TFQ_Q_G_24_5: return {Codec::Q24, 24, 0, 0, 0, 24.5f, 784};
         case TFQ_Q_G_24: return {Codec::Q24, 24, 0, 1, 0, 24.5f, 784};
         case TFQ_Q_G_24_K_L: case TFQ_Q_G_24_K_M: case TFQ_Q_G_24_K_H: return {Codec::Q24, 24, 0, 1, 0, 24.0f, 768};
-        case TFQ_Q_2: return {Codec::Lattice, 2, 0, 0, 0, 2.0f, 64};
-        case TFQ_Q_4: return {Codec::Lattice, 4, 0, 0, 0, 4.0f, 128};
-        case TFQ_Q_8: return {Codec::Lattice, 8, 0, 0, 0, 8.0f, 256};
+        case TFQ_Q_2: case TFQ_Q_2_K_L: case TFQ_Q_2_K_M: case TFQ_Q_2_K_H: return {Codec::Lattice, 2, 0, 0, 0, 2.0f, 64};
+        case TFQ_Q_4: case TFQ_Q_4_K_L: case TFQ_Q_4_K_M: case TFQ_Q_4_K_H: return {Codec::Lattice, 4, 0, 0, 0, 4.0f, 128};
+        case TFQ_Q_8: case TFQ_Q_8_K_L: case TFQ_Q_8_K_M: case TFQ_Q_8_K_H: return {Codec::Lattice, 8, 0, 0, 0, 8.0f, 256};
+        // fixed shared codebooks: the lattice layout with another level table
+        case TFQ_Q_3: case TFQ_Q_3_K_L: case TFQ_Q_3_K_M: case TFQ_Q_3_K_H: return {Codec::Fixed, 3, 0, 0, 0, 3.0f, 96};
+        case TFQ_Q_6: case TFQ_Q_6_K_L: case TFQ_Q_6_K_M: case TFQ_Q_6_K_H: return {Codec::Fixed, 6, 0, 0, 0, 6.0f, 192};
+        case TFQ_Q_12: case TFQ_Q_12_K_L: case TFQ_Q_12_K_M: case TFQ_Q_12_K_H: return {Codec::Fixed, 12, 0, 0, 0, 12.0f, 384};
+        // 12-bit compound: scb = 1 where blocks that are not whole groups of 32 take the fixed codebook
+        // instead of the grouped-lattice fallback; bpw is the claim the encoder budgets with
+        case TFQ_Q_G_12: return {Codec::Grp12, 12, 32, 0, 0, 12.5f, 400};
+        case TFQ_Q_12_5: case TFQ_Q_G_12_5: return {Codec::Grp12, 12, 32, 1, 0, 12.5f, 400};
+        case TFQ_Q_G_12_K_L: case TFQ_Q_G_12_K_M: case TFQ_Q_G_12_K_H: return {Codec::Grp12, 12, 32, 1, 0, 12.0f, 400};
         case TFQ_Q_G_4: case TFQ_Q_4_5: case TFQ_Q_G_4_5: return {Codec::Affine, 4, 32, 6, 6, 4.5f, 144};
         case TFQ_Q_G_3: case TFQ_Q_3_5: case TFQ_Q_G_3_5: return {Codec::Affine, 3, 32, 6, 6, 3.5f, 112};
         case TFQ_Q_G_2: return {Codec::Affine, 2, 16, 4, 4, 2.625f, 84};
         case TFQ_Q_G_8: case TFQ_Q_8_5: case TFQ_Q_G_8_5: return {Codec::Grp8, 8, 32, 0, 0, 8.5f, 272};
+        case TFQ_Q_G_8_K_L: case TFQ_Q_G_8_K_M: case TFQ_Q_G_8_K_H: return {Codec::Grp8, 8, 32, 0, 0, 8.0f, 272};  // short blocks budget with 8.0
         case TFQ_Q_G_6: case TFQ_Q_G_6_K_L: case TFQ_Q_G_6_K_M: case TFQ_Q_G_6_K_H:
             return {Codec::Q6K, 6, 16, 8, 0, 6.5625f, 210};
         // scb / mb keep the affine parameters: a short block of these ids may still fit the affine layout
@@ -81,7 +91,14 @@ __host__ __device__ constexpr int canonical(int fmt) {
     switch (fmt) {
         case TFQ_Q_4_5: case TFQ_Q_G_4_5: return TFQ_Q_G_4;
         case TFQ_Q_3_5: case TFQ_Q_G_3_5: return TFQ_Q_G_3;
-        case TFQ_Q_8_5: case TFQ_Q_G_8_5: return TFQ_Q_G_8;
+        case TFQ_Q_8_5: case TFQ_Q_G_8_5: case TFQ_Q_G_8_K_L: case TFQ_Q_G_8_K_M: case TFQ_Q_G_8_K_H: return TFQ_Q_G_8;
+        case TFQ_Q_2_K_L: case TFQ_Q_2_K_M: case TFQ_Q_2_K_H: return TFQ_Q_2;
+        case TFQ_Q_4_K_L: case TFQ_Q_4_K_M: case TFQ_Q_4_K_H: return TFQ_Q_4;
+        case TFQ_Q_8_K_L: case TFQ_Q_8_K_M: case TFQ_Q_8_K_H: return TFQ_Q_8;
+        case TFQ_Q_3_K_L: case TFQ_Q_3_K_M: case TFQ_Q_3_K_H: return TFQ_Q_3;
+        case TFQ_Q_6_K_L: case TFQ_Q_6_K_M: case TFQ_Q_6_K_H: return TFQ_Q_6;
+        case TFQ_Q_12_K_L: case TFQ_Q_12_K_M: case TFQ_Q_12_K_H: return TFQ_Q_12;
+        case TFQ_Q_12_5: case TFQ_Q_G_12_5: case TFQ_Q_G_12_K_L: case TFQ_Q_G_12_K_M: case TFQ_Q_G_12_K_H: return TFQ_Q_G_12;
         case TFQ_Q_G_6_K_L: case TFQ_Q_G_6_K_M: case TFQ_Q_G_6_K_H: return TFQ_Q_G_6;
         case TFQ_Q_G_2_K_M: case TFQ_Q_G_2_K_H: case TFQ_Q_2_5: case TFQ_Q_G_2_5: return TFQ_Q_G_2_K_L;
         case TFQ_Q_G_3_K_M: case TFQ_Q_G_3_K_H: return TFQ_Q_G_3_K_L;
@@ -97,6 +114,30 @@ __host__ __device__ constexpr int canonical(int fmt) {
         case TFQ_Q_G_24_K_L: case TFQ_Q_G_24_K_M: case TFQ_Q_G_24_K_H: return TFQ_Q_24;
         case TFQ_Q_G_24_5: return TFQ_Q_24_5;
         default: return fmt;
+    }
+}
+
+// Bits per weight the registry reports (format_bpw, include/quant/types.h:197-230): the measured
+// spend of a full block, which for a few ids is not the claim their encoder budgets with.
+__host__ __device__ constexpr float reported_bpw(int fmt) {
+    switch (fmt) {
+        case TFQ_Q_2_5: case TFQ_Q_G_2_5: return 2.4375f;
+        case TFQ_Q_6_5: case TFQ_Q_G_6_5: return 6.4375f;
+        case TFQ_Q_G_8_K_L: case TFQ_Q_G_8_K_M: case TFQ_Q_G_8_K_H: return 8.5f;
+        case TFQ_Q_G_12_K_L: case TFQ_Q_G_12_K_M: case TFQ_Q_G_12_K_H: return 12.5f;
+        default: return spec_of(fmt).bpw;
+    }
+}
+
+// K-tier search effort of an id: 0 for _K_L and plain ids, 1 for _K_M, 2 for _K_H
+// (k_tier, src/codec/block_codec.cpp:2389-2395).
+__host__ __device__ constexpr int tier_of(int fmt) {
+    switch (fmt) {
+        case TFQ_Q_2_K_M: case TFQ_Q_3_K_M: case TFQ_Q_4_K_M: case TFQ_Q_6_K_M: case TFQ_Q_8_K_M: case TFQ_Q_12_K_M:
+        case TFQ_Q_G_8_K_M: case TFQ_Q_G_12_K_M: return 1;
+        case TFQ_Q_2_K_H: case TFQ_Q_3_K_H: case TFQ_Q_4_K_H: case TFQ_Q_6_K_H: case TFQ_Q_8_K_H: case TFQ_Q_12_K_H:
+        case TFQ_Q_G_8_K_H: case TFQ_Q_G_12_K_H: return 2;
+        default: return 0;
     }
 }
 
@@ -134,10 +175,8 @@ enum : int { TFQ_LAYOUT_WIRE = 0, TFQ_LAYOUT_TILED16 = 1 };
 namespace tfq {
 // header bytes per row and block in the Tiled16 layout; 0 = the format stays in wire order
 __host__ __device__ constexpr int tiled_header_bytes(int fmt) {
-    switch (fmt) {
-        case TFQ_Q_G_4: case TFQ_Q_4_5: case TFQ_Q_G_4_5: case TFQ_B32S4: case TFQ_B32S8:
-        case TFQ_Q_G_3: case TFQ_Q_3_5: case TFQ_Q_G_3_5:
-        case TFQ_Q_G_8: case TFQ_Q_8_5: case TFQ_Q_G_8_5: case TFQ_Q_8: return 16;
+    switch (canonical(fmt)) {
+        case TFQ_Q_G_4: case TFQ_B32S4: case TFQ_B32S8: case TFQ_Q_G_3: case TFQ_Q_G_8: case TFQ_Q_8: return 16;
         case TFQ_Q_G_2: case TFQ_SB256A3: case TFQ_SB256A2: return 32;
         default: return 0;
     }
@@ -147,7 +186,7 @@ __host__ __device__ constexpr int tiled_header_bytes(int fmt) {
 // (the companded 8-bit formats store their code 0..255 the same way; plain Q_8 has its slot codes
 // widened to 8 bits and its one scale repeated for the eight groups)
 __host__ __device__ constexpr int tiled_planes(int fmt) {
-    return fmt == TFQ_B32S8 || fmt == TFQ_Q_G_8 || fmt == TFQ_Q_8_5 || fmt == TFQ_Q_G_8_5 || fmt == TFQ_Q_8 ? 2 : 1;
+    return canonical(fmt) == TFQ_B32S8 || canonical(fmt) == TFQ_Q_G_8 || canonical(fmt) == TFQ_Q_8 ? 2 : 1;
 }
 __host__ __device__ constexpr int tiled_unit_bytes(int fmt) { return 2048 * tiled_planes(fmt) + 16 * tiled_header_bytes(fmt); }
 }  // namespace tfq
@@ -167,14 +206,14 @@ namespace tfq {
 // Layout of one block of n <= 256 weights, as the reference's codecs choose it from
 // (format, n): short blocks drop or shrink their headers.  Filled on the host, passed
 // to the short-block decode kernel by value.
-enum : int { BK_RAW32 = 0, BK_LEVELS, BK_LATTICE, BK_AFFINE, BK_GRP16, BK_Q6K, BK_GRP8, BK_SYM32, BK_Q1, BK_WIDE };
+enum : int { BK_RAW32 = 0, BK_LEVELS, BK_LATTICE, BK_AFFINE, BK_GRP16, BK_Q6K, BK_GRP8, BK_SYM32, BK_Q1, BK_WIDE, BK_GRP12 };
 struct BlockLayout {
     int kind;
     int bits;   // code width
     int n;      // weights in the block
     int bytes;  // payload bytes
     int gsz, ng, scb, mb;  // affine: group size, group count, scale / min code widths
-    int aux;    // BK_GRP16: 0 raw levels, 1 one d, 2 group scales + d.  BK_Q6K: bit 0 d present, bits 8.. stored scale count.
+    int aux;    // BK_LEVELS / BK_LATTICE: 1 when the levels are the fixed codebook's.  BK_GRP16: 0 raw levels, 1 one d, 2 group scales + d.  BK_Q6K: bit 0 d present, bits 8.. stored scale count.
                 // BK_WIDE: bit 0 residual means follow the plain part, bit 1 packed 16-bit layout (else raw binary16 / 24-bit)
 };
 // false when the format cannot hold a block of n weights
