@@ -35,6 +35,8 @@ FMT = {
     "Q_8_K_L": 25, "Q_8_K_M": 26, "Q_8_K_H": 27, "Q_12_K_L": 28, "Q_12_K_M": 29, "Q_12_K_H": 30, "Q_G_12": 43,
     "Q_G_8_K_L": 61, "Q_G_8_K_M": 62, "Q_G_8_K_H": 63, "Q_G_12_K_L": 64, "Q_G_12_K_M": 65, "Q_G_12_K_H": 66,
     "Q_12_5": 79, "Q_G_12_5": 88,
+    "Q_MX_3_5": 91, "Q_MX_4_5": 92, "Q_MX_6_5": 93, "Q_MX_8_5": 94, "Q_MX_12_5": 95, "Q_MX_16_5": 96, "Q_MX_24_5": 97,
+    "Q_G_MX_3_5": 98, "Q_G_MX_4_5": 99, "Q_G_MX_6_5": 100, "Q_G_MX_8_5": 101, "Q_G_MX_12_5": 102, "Q_G_MX_16_5": 103, "Q_G_MX_24_5": 104,
 }
 # formats that exist in the reference (the compiled reference can run them)
 REF_FORMATS = [k for k, v in FMT.items() if v < 105]

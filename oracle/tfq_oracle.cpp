@@ -16,6 +16,7 @@
 //   Q_G_8 compound codec       src/codec/block_codec.cpp:365-427
 //   fixed codebooks (Q_3/6/12) src/codec/block_codec.cpp:530-735
 //   12-bit compound (Q_G_12)   src/codec/block_codec.cpp:961-1040
+//   four-tier mixes (Q_MX_*)   src/codec/block_codec.cpp:1875-2380
 //   _K_M / _K_H tier searches  src/codec/block_codec.cpp:2378-2400, 2551-2665, 2756-2824
 //   affine grouped codec       src/codec/block_codec.cpp:1316-1521, 1620-1687
 //   format dispatch            src/codec/block_codec.cpp:2402-2867, 2869-3067
@@ -72,9 +73,10 @@ enum : uint8_t {
     F_B32S4 = 105, F_B32S8 = 106, F_SB256A3 = 107, F_SB256A2 = 108,
     F_Q_3 = 2, F_Q_6 = 4, F_Q_12 = 6, F_Q_2_K_L = 13, F_Q_3_K_L = 16, F_Q_4_K_L = 19, F_Q_6_K_L = 22, F_Q_8_K_L = 25,
     F_Q_12_K_L = 28, F_Q_G_12 = 43, F_Q_G_8_K_L = 61, F_Q_G_12_K_L = 64, F_Q_12_5 = 79, F_Q_G_12_5 = 88,
+    F_Q_MX_3_5 = 91, F_Q_G_MX_3_5 = 98, F_Q_G_MX_24_5 = 104,
 };
 
-enum class Codec { Raw32, Lattice, Affine, Grp8, Sym32, Q6K, Q1, Wide, Fixed, Grp12 };
+enum class Codec { Raw32, Lattice, Affine, Grp8, Sym32, Q6K, Q1, Wide, Fixed, Grp12, Mix };
 
 struct Spec {
     Codec codec;
@@ -145,6 +147,17 @@ bool spec_for(uint8_t fmt, Spec* s) {
         case F_Q_G_6: case F_Q_G_6_K_L: *s = {Codec::Q6K, 6, 16, 8, 0, 6.5625f, 0}; return true;
         case F_Q_G_6_K_M: *s = {Codec::Q6K, 6, 16, 8, 0, 6.5625f, 1}; return true;
         case F_Q_G_6_K_H: *s = {Codec::Q6K, 6, 16, 8, 0, 6.5625f, 2}; return true;
+        // four-tier mixes (:1875-2380): bits = index into the tier table, gsz = 1 for the grouped ids
+        case 91: case 92: case 93: case 94: case 95: case 96: case 97: {
+            static const float claim[7] = {3.5f, 4.5f, 6.5f, 8.5f, 12.5f, 16.5f, 24.5f};
+            *s = {Codec::Mix, fmt - 91, 0, 0, 0, claim[fmt - 91]};
+            return true;
+        }
+        case 98: case 99: case 100: case 101: case 102: case 103: case 104: {
+            static const float claim[7] = {3.78125f, 4.5f, 6.5f, 8.5f, 12.5f, 16.5f, 24.5f};
+            *s = {Codec::Mix, 7 + fmt - 98, 1, 0, 0, claim[fmt - 98]};
+            return true;
+        }
         case F_SB256A3: *s = {Codec::Affine, 3, 16, 6, 6, 3.875f}; return true;
         case F_SB256A2: *s = {Codec::Affine, 2, 16, 6, 6, 2.875f}; return true;
         case F_B32S4: *s = {Codec::Sym32, 4, 32, 0, 0, 4.5f}; return true;
@@ -638,6 +651,231 @@ void grp12_decode(const uint8_t* bytes, size_t size, int n, float* out) {
     for (int i = 0; i < n; ++i) {
         if ((i & 31) == 0) s = half_to_float((uint16_t)scales.take(16));
         out[i] = s * fixed_value(12, codes.take(12));
+    }
+}
+
+// --------------------------------------------------- four-tier mixes (Q_MX_*)
+// src/codec/block_codec.cpp:1875-2380.  Every weight carries a 2-bit tier; the
+// tiers hold fixed shares of the block, the largest magnitudes in the widest
+// tier.  Layout: [n 2-bit tiers][tier 0 values][tier 1][tier 2][tier 3] as one
+// bit stream, then byte aligned binary16 scales: one per tier narrower than 16
+// bits, or one per 32 values of the most populated tier for the grouped ids.
+// Values: 1 bit = sign, 2/4/8 = plain lattice grid, 3/6/12 = fixed codebooks,
+// 16 = binary16, 24 = top three bytes of the binary32, 32 = the binary32.
+struct MixTier { int bits; float percent; };
+const MixTier kMix[14][4] = {  // :1950-1968, Q_MX_3_5 .. Q_MX_24_5 then Q_G_MX_3_5 .. Q_G_MX_24_5
+    {{1, 92.0f}, {2, 1.5f}, {4, 6.0f}, {32, 0.5f}},   {{1, 58.5f}, {2, 2.0f}, {4, 39.0f}, {32, 0.5f}},
+    {{1, 1.5f}, {2, 4.0f}, {4, 93.0f}, {32, 1.5f}},   {{1, 2.5f}, {2, 1.0f}, {4, 88.0f}, {32, 8.5f}},
+    {{1, 0.5f}, {3, 2.0f}, {8, 87.5f}, {32, 10.0f}},  {{1, 4.5f}, {2, 7.0f}, {16, 88.0f}, {32, 0.5f}},
+    {{1, 2.5f}, {2, 5.0f}, {24, 92.0f}, {32, 0.5f}},
+    {{1, 92.0f}, {2, 4.0f}, {4, 3.0f}, {32, 1.0f}},   {{1, 58.5f}, {2, 1.0f}, {4, 39.5f}, {32, 1.0f}},
+    {{1, 0.5f}, {3, 5.0f}, {4, 93.0f}, {32, 1.5f}},   {{1, 0.5f}, {3, 2.0f}, {4, 89.0f}, {32, 8.5f}},
+    {{1, 1.5f}, {2, 2.5f}, {8, 85.0f}, {32, 11.0f}},  {{1, 10.0f}, {2, 1.0f}, {16, 88.0f}, {32, 1.0f}},
+    {{1, 2.5f}, {2, 5.0f}, {24, 91.5f}, {32, 1.0f}},
+};
+
+struct MixLayout {
+    int c[4];      // weights per tier
+    int nsc[4];    // scales per tier
+    int dom;
+    bool collapsed;  // all weights as bare signs, no scales
+    size_t payload_bytes, total;
+};
+
+MixLayout mix_layout(const Spec& sp, int n) {
+    const MixTier* cfg = kMix[sp.bits];
+    const bool grp = sp.gsz != 0;
+    MixLayout L{};
+    int* c = L.c;
+    // :1974-1995
+    for (int i = 0; i < 3; ++i) c[i] = std::max(1, (int)std::lround(cfg[i].percent * 0.01 * (double)n));
+    c[3] = n - c[0] - c[1] - c[2];
+    if (c[3] < 1) {
+        c[3] = 1;
+        int excess = c[0] + c[1] + c[2] + 1 - n;
+        for (int i = 0; i < 3 && excess > 0; ++i) {
+            const int rem = std::min(c[i] - 1, excess);
+            c[i] -= rem;
+            excess -= rem;
+        }
+    }
+    for (int i = 0; i < 4; ++i) c[i] = std::max(0, std::min(n, c[i]));
+    int sum = c[0] + c[1] + c[2] + c[3];
+    for (int i = 0; i < 4 && sum > n; ++i) {
+        const int rem = std::min(c[i], sum - n);
+        c[i] -= rem;
+        sum -= rem;
+    }
+    // :1898-1923: demote boundary weights one tier at a time until the layout fits the claim
+    const size_t budget_bits = (size_t)std::ceil(sp.claimed * (double)n);
+    for (int guard = 0; guard < 4 * n; ++guard) {
+        size_t total = (size_t)2 * (size_t)n;
+        for (int t = 0; t < 4; ++t) total += (size_t)c[t] * (size_t)cfg[t].bits;
+        int dom = 0;
+        for (int t = 1; t < 4; ++t) if (c[t] > c[dom]) dom = t;
+        for (int t = 0; t < 4; ++t)
+            if (cfg[t].bits < 16) total += (grp && t == dom) ? (size_t)16 * ((size_t)(c[t] + 31) / 32) : 16;
+        if (total <= budget_bits) break;
+        bool moved = false;
+        for (int t = 3; t >= 1; --t) {
+            if (c[t] > 1 && cfg[t].bits > cfg[t - 1].bits) {
+                --c[t];
+                ++c[t - 1];
+                moved = true;
+                break;
+            }
+        }
+        if (!moved) break;
+    }
+    L.dom = 0;
+    for (int t = 1; t < 4; ++t) if (c[t] > c[L.dom]) L.dom = t;
+    // :1932-1945
+    {
+        size_t payload = (size_t)2 * (size_t)n;
+        for (int t = 0; t < 4; ++t) payload += (size_t)c[t] * (size_t)cfg[t].bits;
+        size_t scales = 0;
+        for (int t = 0; t < 4; ++t) {
+            if (cfg[t].bits >= 16 || c[t] == 0) continue;
+            scales += (size_t)((grp && t == L.dom) ? ((c[t] + 31) / 32) : 1) * 2;
+        }
+        L.collapsed = (payload + 7) / 8 + scales > (budget_bits + 7) / 8;
+    }
+    if (L.collapsed) { c[0] = n; c[1] = c[2] = c[3] = 0; }
+    size_t bits = (size_t)2 * (size_t)n, scale_bytes = 0;
+    for (int t = 0; t < 4; ++t) {
+        bits += (size_t)c[t] * (size_t)cfg[t].bits;
+        if (L.collapsed || cfg[t].bits >= 16 || c[t] == 0) continue;
+        L.nsc[t] = (grp && t == L.dom) ? ((c[t] + 31) / 32) : 1;
+        scale_bytes += (size_t)L.nsc[t] * 2;
+    }
+    L.payload_bytes = (bits + 7) / 8;
+    L.total = L.payload_bytes + scale_bytes;
+    return L;
+}
+
+float mix_top(int bits) {  // :1997-2008
+    switch (bits) {
+        case 2: return 1.5104f;
+        case 3: return kFixed3[7];
+        case 4: return 2.7178f;
+        case 6: return fixed_value(6, 63u);
+        case 8: return 8.0f;
+        case 12: return fixed_value(12, 4095u);
+        default: return 1.0f;
+    }
+}
+
+uint32_t mix_code(int bits, float nv) {
+    if (bits == 3 || bits == 6 || bits == 12) return fixed_nearest(bits, nv);
+    return grid_nearest(nv, bits);
+}
+float mix_level(int bits, uint32_t code) {
+    if (bits == 3 || bits == 6 || bits == 12) return fixed_value(bits, code);
+    return grid_value(bits, code);
+}
+
+bool mix_encode(const Spec& sp, const float* w, int n, uint8_t* out, size_t nbytes) {  // :2102-2205
+    const MixTier* cfg = kMix[sp.bits];
+    const MixLayout L = mix_layout(sp, n);
+    if (L.total != nbytes) return false;
+    std::memset(out, 0, nbytes);
+    // The largest magnitudes take the widest tier.  The reference sorts with an unstable
+    // std::sort, so which of several equal magnitudes crosses a tier boundary is whatever that
+    // library leaves; this restatement calls the same routine with the same comparator.
+    std::vector<std::pair<float, int>> mag((size_t)n);
+    for (int i = 0; i < n; ++i) mag[(size_t)i] = {std::fabs(w[i]), i};
+    std::sort(mag.begin(), mag.end(), [](const auto& a, const auto& b) { return a.first > b.first; });
+    std::vector<uint8_t> tier((size_t)n, 0);
+    int rank = 0;
+    for (int t = 3; t >= 0; --t)
+        for (int j = 0; j < L.c[t]; ++j, ++rank) tier[(size_t)mag[(size_t)rank].second] = (uint8_t)t;
+    std::vector<float> tv[4];
+    for (int i = 0; i < n; ++i) tv[tier[(size_t)i]].push_back(w[i]);
+    std::vector<float> sc[4];
+    for (int t = 0; t < 4; ++t) {
+        if (L.nsc[t] == 0) continue;
+        sc[t].assign((size_t)L.nsc[t], 0.0f);
+        const int bits = cfg[t].bits;
+        const float top = mix_top(bits);
+        for (int g = 0; g < L.nsc[t]; ++g) {
+            // values g*32 .. g*32+31 of the tier: a tier with a single scale is fitted on its
+            // first 32 values only (:2156-2160), and that scale then serves all of them (:2188-2190)
+            const int st = g * 32, last = std::min(L.c[t], st + 32);
+            float maxa = 0.0f;
+            for (int j = st; j < last; ++j) maxa = std::max(maxa, std::fabs(tv[t][(size_t)j]));
+            float s = (maxa > 1e-30f) ? maxa / top : 0.0f;
+            if (s > 0.0f) {
+                for (int iter = 0; iter < 2; ++iter) {
+                    double num = 0.0, den = 0.0;
+                    for (int j = st; j < last; ++j) {
+                        const float x = tv[t][(size_t)j];
+                        const float l = bits == 1 ? (x >= 0.0f ? 1.0f : -1.0f) : mix_level(bits, mix_code(bits, x / s));
+                        num += (double)x * (double)l;
+                        den += (double)l * (double)l;
+                    }
+                    if (den > 1e-20) s = (float)(num / den);
+                }
+            }
+            if (!(s > 0.0f)) s = 0.0f;
+            sc[t][(size_t)g] = s;
+        }
+    }
+    BitSink bs(out, L.payload_bytes);
+    for (int i = 0; i < n; ++i) bs.put(tier[(size_t)i], 2);
+    for (int t = 0; t < 4; ++t) {
+        const int bits = cfg[t].bits;
+        for (int j = 0; j < L.c[t]; ++j) {
+            const float v = tv[t][(size_t)j];
+            const float s = (bits < 16 && L.nsc[t] > 0) ? sc[t][(size_t)std::min(j / 32, L.nsc[t] - 1)] : 1.0f;
+            const float nv = (s == 0.0f) ? 0.0f : v / s;
+            uint32_t raw;
+            std::memcpy(&raw, &v, 4);
+            switch (bits) {
+                case 1: bs.put(v >= 0.0f ? 1u : 0u, 1); break;
+                case 16: bs.put(half_from_float(v), 16); break;
+                case 24: bs.put(raw >> 8, 24); break;
+                case 32: bs.put(raw & 0xFFFFu, 16); bs.put(raw >> 16, 16); break;
+                default: bs.put(mix_code(bits, nv), bits); break;
+            }
+        }
+    }
+    uint8_t* p = out + L.payload_bytes;
+    for (int t = 0; t < 4; ++t)
+        for (int g = 0; g < L.nsc[t]; ++g, p += 2) {
+            const uint16_t h = half_from_float(sc[t][(size_t)g]);
+            p[0] = (uint8_t)(h & 0xFF);
+            p[1] = (uint8_t)(h >> 8);
+        }
+    return !bs.overflow;
+}
+
+void mix_decode(const Spec& sp, const uint8_t* bytes, size_t size, int n, float* out) {  // :2207-2380
+    const MixTier* cfg = kMix[sp.bits];
+    const MixLayout L = mix_layout(sp, n);
+    if (size < L.total) return;
+    std::vector<float> sc[4];
+    const uint8_t* p = bytes + L.payload_bytes;
+    for (int t = 0; t < 4; ++t)
+        for (int g = 0; g < L.nsc[t]; ++g, p += 2) sc[t].push_back(half_to_float((uint16_t)(p[0] | ((uint16_t)p[1] << 8))));
+    BitSource br(bytes, L.payload_bytes);
+    std::vector<uint32_t> pos[4];
+    for (int i = 0; i < n; ++i) pos[br.take(2)].push_back((uint32_t)i);
+    for (int t = 0; t < 4; ++t) {
+        const int bits = cfg[t].bits;
+        const int cnt = std::min(L.c[t], (int)pos[t].size());  // surplus entries of a tier stay zero
+        for (int j = 0; j < cnt; ++j) {
+            const float s = L.nsc[t] > 0 ? sc[t][(size_t)std::min(j / 32, L.nsc[t] - 1)] : 1.0f;
+            float v;
+            uint32_t raw;
+            switch (bits) {
+                case 1: v = (br.take(1) == 0 ? -1.0f : 1.0f) * s; break;
+                case 16: v = half_to_float((uint16_t)br.take(16)); break;
+                case 24: raw = br.take(24) << 8; std::memcpy(&v, &raw, 4); break;
+                case 32: raw = br.take(16); raw |= br.take(16) << 16; std::memcpy(&v, &raw, 4); break;
+                default: v = mix_level(bits, br.take(bits)) * s; break;
+            }
+            out[pos[t][(size_t)j]] = v;
+        }
     }
 }
 
@@ -1574,6 +1812,7 @@ long block_bytes(uint8_t fmt, int n) {
         case Codec::Raw32: return (long)n * 4;
         case Codec::Lattice: return (long)lattice_bytes(sp.bits, n);
         case Codec::Fixed: return (long)fixed_bytes(sp.bits, n);
+        case Codec::Mix: return (long)mix_layout(sp, n).total;
         case Codec::Grp12:
             if (grp12_fits(n)) return (long)grp12_bytes(n);
             return sp.gsz ? (long)fixed_bytes(12, n) : (long)grp16_sizes(12, n, 12.5f).total;
@@ -1599,6 +1838,7 @@ long encode_block(uint8_t fmt, const float* w, int n, uint8_t* out, size_t cap) 
         case Codec::Raw32: std::memcpy(out, w, (size_t)n * 4); break;
         case Codec::Lattice: ok = lattice_encode_tier(sp.bits, sp.tier, w, n, out, (size_t)need); break;
         case Codec::Fixed: ok = fixed_encode_tier(sp.bits, sp.tier, w, n, out, (size_t)need); break;
+        case Codec::Mix: ok = mix_encode(sp, w, n, out, (size_t)need); break;
         case Codec::Grp12:
             if (grp12_fits(n)) ok = grp12_encode_tier(sp.tier, w, n, out, (size_t)need);
             else if (sp.gsz) ok = fixed_encode_tier(12, sp.tier, w, n, out, (size_t)need);
@@ -1634,6 +1874,7 @@ int decode_block(uint8_t fmt, const uint8_t* bytes, size_t size, int n, float* o
         case Codec::Raw32: if (size >= (size_t)n * 4) std::memcpy(out, bytes, (size_t)n * 4); return 0;
         case Codec::Lattice: lattice_decode(sp.bits, bytes, size, n, out); return 0;
         case Codec::Fixed: fixed_decode(sp.bits, bytes, size, n, out); return 0;
+        case Codec::Mix: mix_decode(sp, bytes, size, n, out); return 0;
         case Codec::Grp12:
             if (grp12_fits(n)) grp12_decode(bytes, size, n, out);
             else if (sp.gsz) fixed_decode(12, bytes, size, n, out);

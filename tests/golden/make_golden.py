@@ -23,7 +23,8 @@ tails.npz
     bytes, decoded offset) into the flat `payloads` / `decoded` arrays: the short-block
     layouts (raw levels, one scale, grouped-lattice fallback), Q_2, Q_G_6, the ids
     whose claim is below the affine header's size, the sign formats, the 16- and
-    24-bit formats, the fixed-codebook formats, the 12-bit compound and searched tiers
+    24-bit formats, the fixed-codebook formats, the 12-bit compound, searched tiers and
+    four-tier mixes
 sample.quant, sample_quant.npz
     a container written by the reference's QUANTWriter (header with a 5-byte config,
     format table, tensor table, block records): tensor "blk.0.ffn_gate" 4 x 512 in Q_G_4,
@@ -68,7 +69,8 @@ TAIL_FORMATS = ["Q_2", "Q_4", "Q_8", "Q_G_2", "Q_G_3", "Q_G_4", "Q_G_6", "Q_G_8"
                 "Q_G_4_K_M", "Q_G_6_K_M", "Q_G_6_K_H", "Q_2_5", "Q_6_5",
                 "Q_1", "Q_G_1_K_H", "Q_1_5", "Q_16", "Q_G_16", "Q_24", "Q_G_24",
                 "Q_3", "Q_6", "Q_12", "Q_2_K_H", "Q_4_K_M", "Q_8_K_H", "Q_3_K_H", "Q_6_K_M", "Q_12_K_H", "Q_G_12",
-                "Q_G_8_K_H", "Q_G_12_K_H", "Q_12_5"]
+                "Q_G_8_K_H", "Q_G_12_K_H", "Q_12_5", "Q_MX_3_5", "Q_MX_12_5", "Q_MX_24_5", "Q_G_MX_3_5", "Q_G_MX_6_5",
+                "Q_G_MX_8_5", "Q_G_MX_16_5"]
 TAIL_SIZES = [1, 7, 8, 15, 16, 31, 32, 33, 100, 160, 250, 255, 256]
 
 

@@ -134,3 +134,118 @@ def test_every_block_size_equals_the_compiled_reference(O):
             a, b = O.decode_block(fmt, rnd, n), O.ref_decode_block(fmt, rnd, n)
             keep = ~(np.isnan(a) & np.isnan(b))
             assert np.array_equal(a.view(np.uint32)[keep], b.view(np.uint32)[keep]), (fmt, n)
+
+
+# ---------------------------------------------------------------- four-tier mixes
+MIX = {"Q_MX_3_5": (3.5, [(1, 92.0), (2, 1.5), (4, 6.0), (32, 0.5)], False),
+       "Q_MX_12_5": (12.5, [(1, 0.5), (3, 2.0), (8, 87.5), (32, 10.0)], False),
+       "Q_G_MX_6_5": (6.5, [(1, 0.5), (3, 5.0), (4, 93.0), (32, 1.5)], True),
+       "Q_G_MX_16_5": (16.5, [(1, 10.0), (2, 1.0), (16, 88.0), (32, 1.0)], True)}
+GRID2 = np.array([-1.5104, -0.4528, 0.4528, 1.5104], np.float32)
+GRID4 = np.array([-2.7178, -2.0522, -1.5995, -1.2392, -0.9275, -0.6508, -0.3976, -0.1260,
+                  0.1260, 0.3976, 0.6508, 0.9275, 1.2392, 1.5995, 2.0522, 2.7178], np.float32)
+
+
+def mix_value(O, bits, code, s):
+    if bits == 1:
+        return np.float32(s) * np.float32(1.0 if code else -1.0)
+    if bits == 2:
+        return GRID2[code] * np.float32(s)
+    if bits == 4:
+        return GRID4[code] * np.float32(s)
+    if bits == 8:
+        return (np.float32(-8.0) + np.float32(16.0) * np.float32(code) / np.float32(255)) * np.float32(s)
+    if bits == 3:
+        return Q3[code] * np.float32(s)
+    if bits == 16:
+        return np.array([code], np.uint16).view(np.float16).astype(np.float32)[0]
+    return np.array([code], np.uint32).view(np.float32)[0]
+
+
+@pytest.mark.parametrize("fmt", sorted(MIX))
+def test_mix_layout_by_hand(O, fmt):
+    """Full block of a four-tier mix (src/codec/block_codec.cpp:1875-1995, :2207-2263): tier counts are the
+    rounded shares (the widest tier takes the rest), the stream is 256 2-bit tiers then the four value
+    runs, the scales follow byte aligned: one per tier narrower than 16 bits, one per 32 values for the
+    most populated tier of a grouped id.  A hand-built payload decodes to the values the layout implies."""
+    claim, tiers, grouped = MIX[fmt]
+    n = 256
+    c = [max(1, int(math.floor(p * 0.01 * n + 0.5))) for _, p in tiers[:3]]
+    c.append(n - sum(c))
+    bits = [b for b, _ in tiers]
+
+    def shape():
+        dom = int(np.argmax(c))
+        nsc = [0 if b >= 16 else ((c[t] + 31) // 32 if grouped and t == dom else 1) for t, b in enumerate(bits)]
+        return nsc, 2 * n + sum(ct * b for ct, b in zip(c, bits))
+
+    # while the layout is over the claim, one weight moves from the widest tier that can spare one to the next narrower
+    while shape()[1] + 16 * sum(shape()[0]) > math.ceil(claim * n):
+        t = max(t for t in (1, 2, 3) if c[t] > 1 and bits[t] > bits[t - 1])
+        c[t] -= 1
+        c[t - 1] += 1
+    nsc, payload_bits = shape()
+    total = (payload_bits + 7) // 8 + 2 * sum(nsc)
+    assert O.block_bytes(fmt, n) == total
+    rs = np.random.RandomState(len(fmt))
+    tier = np.repeat(np.arange(4), c)
+    rs.shuffle(tier)
+    buf = np.zeros(total, np.uint8)
+    pos = 0
+    for t in tier:
+        pos = put_bits(buf, pos, int(t), 2)
+    codes = [rs.randint(0, 1 << min(b, 31), ct).astype(np.uint64) for ct, b in zip(c, bits)]
+    for t in range(4):
+        if bits[t] == 32:
+            codes[t] = rs.randn(c[t]).astype(np.float32).view(np.uint32).astype(np.uint64)
+        for code in codes[t]:
+            pos = put_bits(buf, pos, int(code), bits[t])
+    assert pos == payload_bits
+    scales = [np.float16(2.0 ** -rs.randint(1, 6, k)) for k in nsc]
+    at = (payload_bits + 7) // 8
+    for t in range(4):
+        for s in scales[t]:
+            buf[at:at + 2] = np.array([s], np.float16).view(np.uint8)
+            at += 2
+    want = np.zeros(n, np.float32)
+    seen = [0, 0, 0, 0]
+    for i, t in enumerate(tier):
+        j = seen[t]
+        seen[t] += 1
+        s = float(scales[t][min(j // 32, nsc[t] - 1)]) if nsc[t] else 1.0
+        want[i] = mix_value(O, bits[t], int(codes[t][j]), s)
+    got = O.decode_block(fmt, buf)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_mix_round_trip_properties(O):
+    """The widest tier is lossless for the largest magnitudes (raw binary32), every payload is within
+    ceil(bpw n / 8) + 1 bytes for every n (tests/test_format_audit.cpp:52-77), and tails too small for the
+    map plus scales collapse to bare signs."""
+    rs = np.random.RandomState(9)
+    w = (rs.standard_t(3, 256) * 0.02).astype(np.float32)
+    order = np.argsort(-np.abs(w))
+    for fmt, claim in (("Q_MX_3_5", 3.5), ("Q_MX_8_5", 8.5), ("Q_G_MX_12_5", 12.5), ("Q_G_MX_24_5", 24.5), ("Q_G_MX_3_5", 3.78125)):
+        d = O.decode_block(fmt, O.encode_block(fmt, w))
+        assert np.array_equal(d[order[:1]], w[order[:1]])
+        for n in range(1, 257):
+            assert O.block_bytes(fmt, n) <= math.ceil(claim * n / 8) + 1, (fmt, n)
+    small = np.array([0.3, -0.2, 0.0, -5.0], np.float32)
+    pay = O.encode_block("Q_MX_3_5", small)
+    assert pay.size == 2 and np.array_equal(O.decode_block("Q_MX_3_5", pay, 4), np.array([1, -1, 1, -1], np.float32))
+
+
+def test_mix_equals_the_compiled_reference(O):
+    if not O.have_ref():
+        pytest.skip("compiled reference not built on this machine")
+    rs = np.random.RandomState(10)
+    for fid in range(91, 105):
+        for n in list(range(1, 70, 3)) + [96, 100, 128, 200, 250, 255, 256, 256]:
+            w = (rs.randn(n) * 0.02).astype(np.float32) if n % 2 else (rs.standard_t(3, n) * 0.5).astype(np.float32)
+            pay = O.ref_encode_block(fid, w)
+            assert O.block_bytes(fid, n) == pay.size, (fid, n)
+            assert np.array_equal(O.encode_block(fid, w), pay), (fid, n)
+            rnd = rs.randint(0, 256, pay.size).astype(np.uint8)
+            a, b = O.decode_block(fid, rnd, n), O.ref_decode_block(fid, rnd, n)
+            keep = ~(np.isnan(a) & np.isnan(b))
+            assert np.array_equal(a.view(np.uint32)[keep], b.view(np.uint32)[keep]), (fid, n)

@@ -36,7 +36,7 @@ def test_encode_and_decode_match_the_reference_for_every_block_size(O, tails):
         assert np.array_equal(O.encode_block(fmt, w), pay), (fmt, n, which)
         assert np.array_equal(O.decode_block(fmt, pay, n).view(np.uint32), dec.view(np.uint32)), (fmt, n, which)
         seen += 1
-    assert seen == 35 * 13 * 2
+    assert seen == 42 * 13 * 2
 
 
 @pytest.mark.parametrize("fmt", sorted(BPW))
