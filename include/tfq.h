@@ -60,6 +60,9 @@ enum {
     TFQ_Q_8_K_L = 25, TFQ_Q_8_K_M = 26, TFQ_Q_8_K_H = 27, TFQ_Q_12_K_L = 28, TFQ_Q_12_K_M = 29, TFQ_Q_12_K_H = 30,
     TFQ_Q_G_12 = 43, TFQ_Q_G_8_K_L = 61, TFQ_Q_G_8_K_M = 62, TFQ_Q_G_8_K_H = 63,
     TFQ_Q_G_12_K_L = 64, TFQ_Q_G_12_K_M = 65, TFQ_Q_G_12_K_H = 66, TFQ_Q_12_5 = 79, TFQ_Q_G_12_5 = 88,
+    TFQ_Q_MX_3_5 = 91, TFQ_Q_MX_4_5 = 92, TFQ_Q_MX_6_5 = 93, TFQ_Q_MX_8_5 = 94, TFQ_Q_MX_12_5 = 95, TFQ_Q_MX_16_5 = 96,
+    TFQ_Q_MX_24_5 = 97, TFQ_Q_G_MX_3_5 = 98, TFQ_Q_G_MX_4_5 = 99, TFQ_Q_G_MX_6_5 = 100, TFQ_Q_G_MX_8_5 = 101,
+    TFQ_Q_G_MX_12_5 = 102, TFQ_Q_G_MX_16_5 = 103, TFQ_Q_G_MX_24_5 = 104,
     TFQ_B32S4 = 105,   /* 32-group symmetric 4-bit, binary16 scale = absmax/7   */
     TFQ_B32S8 = 106,   /* 32-group symmetric 8-bit, binary16 scale = absmax/127 */
     TFQ_SB256A3 = 107, /* 256-superblock, 16x16 sub-blocks, 6-bit scale + min, 3-bit codes */

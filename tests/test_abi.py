@@ -33,7 +33,7 @@ def test_registry_mirror_without_gpu(tfq):
     # wire-truth bpw table (include/quant/types.h:197-230 of the reference)
     for fid, bpw in ((3, 4.0), (5, 8.0), (38, 2.625), (39, 3.5), (40, 4.5), (42, 8.5), (105, 4.5), (106, 8.5),
                      (107, 3.875), (108, 2.875), (2, 3.0), (6, 12.0), (43, 12.5), (74, 2.4375), (77, 6.4375), (61, 8.5),
-                     (64, 12.5), (83, 2.4375), (25, 8.0)):
+                     (64, 12.5), (83, 2.4375), (25, 8.0), (91, 3.5), (98, 3.78125), (104, 24.5)):
         assert L.tfq_format_bpw(fid) == pytest.approx(bpw)
     for fmt, nbytes in (("Q_4", 128), ("Q_8", 256), ("Q_G_2", 84), ("Q_G_3", 112), ("Q_G_4", 144), ("Q_G_8", 272),
                         ("Q_3", 96), ("Q_6_K_H", 192), ("Q_12", 384), ("Q_G_12", 400), ("Q_G_12_K_M", 400), ("Q_G_8_K_L", 272)):
@@ -43,7 +43,7 @@ def test_registry_mirror_without_gpu(tfq):
 def test_errors_are_reported_not_swallowed(tfq):
     L = tfq.lib()
     out = C.c_size_t(0)
-    assert L.tfq_block_bytes(91, 256, C.byref(out)) == 2           # TFQ_ERR_FORMAT: Q_MX_3_5 is not handled
+    assert L.tfq_block_bytes(19 + 100, 256, C.byref(out)) == 2     # TFQ_ERR_FORMAT: no such wire id
     assert b"not handled" in L.tfq_last_error()
     assert L.tfq_block_bytes(40, 100, C.byref(out)) == 0 and out.value == 57   # short block: grouped-lattice fallback
     assert L.tfq_block_bytes(40, 257, C.byref(out)) == 3           # TFQ_ERR_SHAPE

@@ -11,7 +11,8 @@ GEMV_FORMATS = ["Q_G_4", "B32S4"]
 OTHER_FORMATS = ["Q_G_8", "B32S8", "Q_G_3", "Q_G_2", "SB256A3", "SB256A2", "Q_4", "Q_8", "Q_32", "Q_4_5", "Q_G_8_5",
                  "Q_2", "Q_G_6", "Q_G_6_K_M", "Q_G_2_K_L", "Q_G_3_K_H", "Q_G_4_K_M", "Q_2_5", "Q_6_5",
                  "Q_1", "Q_G_1", "Q_1_5", "Q_16", "Q_G_16", "Q_24", "Q_G_24",
-                 "Q_3", "Q_6", "Q_12", "Q_G_12", "Q_G_12_K_M", "Q_G_8_K_M", "Q_4_K_H", "Q_8_K_L"]
+                 "Q_3", "Q_6", "Q_12", "Q_G_12", "Q_G_12_K_M", "Q_G_8_K_M", "Q_4_K_H", "Q_8_K_L",
+                 "Q_MX_3_5", "Q_MX_12_5", "Q_MX_16_5", "Q_G_MX_4_5", "Q_G_MX_8_5", "Q_G_MX_24_5"]
 
 
 def rel_err(y, ref):

@@ -87,6 +87,11 @@ const NameRow kNames[] = {
     {"Q_G_12", TFQ_Q_G_12}, {"Q_G_8_K_L", TFQ_Q_G_8_K_L}, {"Q_G_8_K_M", TFQ_Q_G_8_K_M}, {"Q_G_8_K_H", TFQ_Q_G_8_K_H},
     {"Q_G_12_K_L", TFQ_Q_G_12_K_L}, {"Q_G_12_K_M", TFQ_Q_G_12_K_M}, {"Q_G_12_K_H", TFQ_Q_G_12_K_H},
     {"Q_12_5", TFQ_Q_12_5}, {"Q_G_12_5", TFQ_Q_G_12_5},
+    {"Q_MX_3_5", TFQ_Q_MX_3_5}, {"Q_MX_4_5", TFQ_Q_MX_4_5}, {"Q_MX_6_5", TFQ_Q_MX_6_5}, {"Q_MX_8_5", TFQ_Q_MX_8_5},
+    {"Q_MX_12_5", TFQ_Q_MX_12_5}, {"Q_MX_16_5", TFQ_Q_MX_16_5}, {"Q_MX_24_5", TFQ_Q_MX_24_5},
+    {"Q_G_MX_3_5", TFQ_Q_G_MX_3_5}, {"Q_G_MX_4_5", TFQ_Q_G_MX_4_5}, {"Q_G_MX_6_5", TFQ_Q_G_MX_6_5},
+    {"Q_G_MX_8_5", TFQ_Q_G_MX_8_5}, {"Q_G_MX_12_5", TFQ_Q_G_MX_12_5}, {"Q_G_MX_16_5", TFQ_Q_G_MX_16_5},
+    {"Q_G_MX_24_5", TFQ_Q_G_MX_24_5},
 };
 
 std::string normalise(const char* s) {

@@ -1036,6 +1036,144 @@ __global__ __launch_bounds__(64) void keep_better_kernel(const float* __restrict
         for (int i = t; i < BB; i += 64) pc[i] = pn[i];
 }
 
+// ---- four-tier mixes (Q_MX_*, Q_G_MX_*): a wavefront per block of L.n <= 256 weights
+__global__ __launch_bounds__(64) void decode_mix_kernel(MixLayout L, const uint8_t* __restrict__ src, float* __restrict__ out) {
+    const uint32_t lane = threadIdx.x;
+    const int64_t blk = blockIdx.x;
+    float v[4];
+    mix_decode_wave(L, src + blk * L.bytes, lane, v);
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        if (4 * (int)lane + k < L.n) out[blk * L.n + 4 * lane + k] = v[k];
+}
+
+__device__ __forceinline__ float mix_level(int bits, uint32_t code) {
+    return bits == 3 ? fixed_value(3, code) : grid_value(bits, code);
+}
+// nearest_level / nearest_fixed_level for the widths the mixes use (src/codec/block_codec.cpp:190-203, :596-606)
+__device__ __forceinline__ uint32_t mix_nearest(int bits, float v) {
+    if (bits == 8) {
+        const float c = fmaxf(-8.0f, fminf(8.0f, v));
+        return (uint32_t)lroundf((c + 8.0f) * 255.0f / 16.0f);
+    }
+    uint32_t best = 0;
+    float bd = fabsf(v - mix_level(bits, 0));
+    for (int i = 1; i < (1 << bits); ++i) {
+        const float d = fabsf(v - mix_level(bits, (uint32_t)i));
+        if (d < bd) { bd = d; best = (uint32_t)i; }
+    }
+    return best;
+}
+
+// Encoder of a full block (quant_quad_mix, src/codec/block_codec.cpp:2102-2205): weights ranked by
+// magnitude, the c[3] largest into tier 3 and so on down; per tier (per 32 values of the most populated
+// tier of a grouped id) s = max / top level and two least-squares refits on the first 32 values the scale
+// covers; then tiers, values and scales as laid out in MixLayout.  Equal magnitudes rank by index here;
+// the reference leaves their order to an unstable sort, so a block with a tie across a tier boundary may
+// get the two weights' tiers the other way round.
+__global__ __launch_bounds__(64) void encode_mix_kernel(MixLayout L, const float* __restrict__ wg, uint8_t* __restrict__ dst) {
+    __shared__ float w[256], tv[256], lev[256];
+    __shared__ uint32_t mag[256];  // |w| as its bit pattern: the same order as the values, and total (NaN sorts above inf)
+    __shared__ float sc[4][8];
+    __shared__ int live[8];
+    __shared__ uint32_t words[200];  // the largest block is 784 bytes
+    const uint32_t lane = threadIdx.x;
+    const int64_t blk = blockIdx.x;
+    for (int i = lane; i < 256; i += 64) { const float x = wg[blk * 256 + i]; w[i] = x; mag[i] = __float_as_uint(x) & 0x7FFFFFFFu; }
+    for (int i = lane; i < 200; i += 64) words[i] = 0;
+    if (lane < 32) sc[lane >> 3][lane & 7] = 0.0f;
+    __syncthreads();
+    const int n3 = L.c[3], n2 = n3 + L.c[2], n1 = n2 + L.c[1];
+    uint32_t tiers = 0;
+    for (int k = 0; k < 4; ++k) {
+        const int i = 4 * lane + k;
+        const uint32_t m = mag[i];
+        int rank = 0;
+        for (int j = 0; j < 256; ++j) {
+            const uint32_t mj = mag[j];
+            rank += (mj > m || (mj == m && j < i)) ? 1 : 0;
+        }
+        const uint32_t t = rank < n3 ? 3u : rank < n2 ? 2u : rank < n1 ? 1u : 0u;
+        tiers |= t << (2 * k);
+    }
+    uint32_t before[4], total[4];
+    mix_scan(tiers, 4, lane, before, total);
+    const int first[4] = {0, L.c[0], L.c[0] + L.c[1], L.c[0] + L.c[1] + L.c[2]};  // tier runs inside tv
+    uint32_t rk[4];
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t t = (tiers >> (2 * k)) & 3u;
+        rk[k] = before[t]++;
+        tv[first[t] + rk[k]] = w[4 * lane + k];
+    }
+    __syncthreads();
+    for (int t = 0; t < 4; ++t) {
+        const int nsc = L.nsc[t];
+        if (nsc == 0) continue;
+        const int bits = L.bits[t], cnt = min(L.c[t], nsc * 32);
+        const float top = bits == 2 ? 1.5104f : bits == 3 ? 3.0776f : bits == 4 ? 2.7178f : bits == 8 ? 8.0f : 1.0f;
+        const float* x = tv + first[t];
+        if ((int)lane < nsc) {
+            float maxa = 0.0f;
+            for (int j = 32 * lane; j < min(cnt, 32 * (int)lane + 32); ++j) maxa = fmaxf(maxa, fabsf(x[j]));
+            const float s = (maxa > 1e-30f) ? maxa / top : 0.0f;
+            sc[t][lane] = s;
+            live[lane] = s > 0.0f;
+        }
+        __syncthreads();
+        for (int it = 0; it < 2; ++it) {
+            for (int j = lane; j < cnt; j += 64) {
+                if (!live[j >> 5]) continue;
+                lev[j] = bits == 1 ? (x[j] >= 0.0f ? 1.0f : -1.0f) : mix_level(bits, mix_nearest(bits, x[j] / sc[t][j >> 5]));
+            }
+            __syncthreads();
+            if ((int)lane < nsc && live[lane]) {
+                double num = 0.0, den = 0.0;
+                for (int j = 32 * lane; j < min(cnt, 32 * (int)lane + 32); ++j) {
+                    num = __builtin_fma((double)x[j], (double)lev[j], num);
+                    den = __builtin_fma((double)lev[j], (double)lev[j], den);
+                }
+                if (den > 1e-20) sc[t][lane] = (float)(num / den);
+            }
+            __syncthreads();
+        }
+        if ((int)lane < nsc && !(sc[t][lane] > 0.0f)) sc[t][lane] = 0.0f;
+        __syncthreads();
+    }
+    // the stream: byte l holds the tiers of lane l's weights, values at (start of the tier's run) + rank * width
+    atomicOr(&words[lane >> 2], tiers << (8 * (lane & 3u)));
+    uint32_t start[4];
+    uint32_t at = 512;
+    for (int t = 0; t < 4; ++t) { start[t] = at; at += (uint32_t)(L.c[t] * L.bits[t]); }
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t t = (tiers >> (2 * k)) & 3u;
+        const int bits = L.bits[t];
+        const float v = w[4 * lane + k];
+        const float s = L.nsc[t] > 0 ? sc[t][min((int)(rk[k] >> 5), L.nsc[t] - 1)] : 1.0f;
+        uint32_t code;
+        switch (bits) {
+            case 1: code = v >= 0.0f ? 1u : 0u; break;
+            case 16: code = float_to_half_bits(v); break;
+            case 24: code = __float_as_uint(v) >> 8; break;
+            case 32: code = __float_as_uint(v); break;
+            default: code = mix_nearest(bits, (s == 0.0f) ? 0.0f : v / s); break;
+        }
+        const uint32_t pos = start[t] + rk[k] * (uint32_t)bits, sh = pos & 31u;
+        atomicOr(&words[pos >> 5], code << sh);
+        if (sh + (uint32_t)bits > 32u) atomicOr(&words[(pos >> 5) + 1], code >> (32u - sh));
+    }
+    __syncthreads();
+    uint8_t* p = dst + blk * L.bytes;
+    for (int byte = lane; byte < L.payload_bytes; byte += 64) p[byte] = (uint8_t)(words[byte >> 2] >> (8 * (byte & 3)));
+    if (lane < 32) {
+        const int t = lane >> 3, g = lane & 7;
+        if (g < L.nsc[t]) {
+            const uint32_t h = float_to_half_bits(sc[t][g]);
+            p[L.sc_at[t] + 2 * g] = (uint8_t)(h & 0xFF);
+            p[L.sc_at[t] + 2 * g + 1] = (uint8_t)(h >> 8);
+        }
+    }
+}
+
 // Wire -> Tiled16: one lane per 16-byte piece of the tiled buffer.  Piece p of a unit: p < 64 code
 // slot of k-step 0, p < 128 of k-step 1, else a 16-byte part of a row header.  Codes narrower
 // than 4 bits are widened to nibbles.
@@ -1184,6 +1322,7 @@ bool block_layout(int fmt, int n, BlockLayout* L) {
     const Spec sp = spec_of(fmt);
     if (n <= 0 || n > 256) return false;
     switch (sp.codec) {
+        case Codec::Mix: *L = {BK_MIX, 0, n, mix_layout(fmt, n).bytes, 0, 0, 0, 0, fmt}; return true;
         case Codec::Raw32: *L = {BK_RAW32, 32, n, n * 4, 0, 0, 0, 0, 0}; return true;
         case Codec::Lattice:
             *L = {n < 16 ? BK_LEVELS : BK_LATTICE, sp.bits, n, ((int)std::ceil(sp.bpw * (double)n) + 7) / 8, 0, 0, 0, 0, 0};
@@ -1228,6 +1367,10 @@ bool block_layout(int fmt, int n, BlockLayout* L) {
 
 int launch_decode_short(const BlockLayout& L, const uint8_t* src, float* out, hipStream_t s) {
     if (L.n <= 0 || L.n > 256 || L.bytes <= 0) return fail(TFQ_ERR_SHAPE, "decode: bad short-block layout");
+    if (L.kind == BK_MIX) {
+        hipLaunchKernelGGL(decode_mix_kernel, dim3(1), dim3(64), 0, s, mix_layout(L.aux, L.n), src, out);
+        return hip_fail(hipGetLastError(), "decode launch");
+    }
     hipLaunchKernelGGL(decode_short_kernel, dim3(1), dim3(256), 0, s, L, src, out);
     return hip_fail(hipGetLastError(), "decode launch");
 }
@@ -1235,6 +1378,10 @@ int launch_decode_short(const BlockLayout& L, const uint8_t* src, float* out, hi
 int launch_decode(int fmt, const uint8_t* src, int64_t nblocks, float* out, hipStream_t s) {
     if (nblocks <= 0) return TFQ_OK;
     if (nblocks > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "decode: more than 2^31-1 blocks in one call");
+    if (is_mix(fmt)) {
+        hipLaunchKernelGGL(decode_mix_kernel, dim3((unsigned)nblocks), dim3(64), 0, s, mix_layout(fmt, 256), src, out);
+        return hip_fail(hipGetLastError(), "decode launch");
+    }
     switch (canonical(fmt)) {
         case TFQ_Q_1: return run_decode<TFQ_Q_1>(src, nblocks, out, s);
         case TFQ_Q_1_5: return run_decode<TFQ_Q_1_5>(src, nblocks, out, s);
@@ -1361,6 +1508,10 @@ int launch_encode(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStr
     if (nblocks <= 0) return TFQ_OK;
     if (nblocks > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "encode: more than 2^31-1 blocks in one call");
     const dim3 grid((unsigned)nblocks), block(256);
+    if (is_mix(fmt)) {
+        hipLaunchKernelGGL(encode_mix_kernel, grid, dim3(64), 0, s, mix_layout(fmt, 256), w, dst);
+        return hip_fail(hipGetLastError(), "encode launch");
+    }
     switch (canonical(fmt)) {
         case TFQ_Q_32: hipLaunchKernelGGL(encode_raw32_kernel, grid, block, 0, s, w, dst); break;
         case TFQ_B32S4: hipLaunchKernelGGL(encode_sym32_kernel<TFQ_B32S4>, grid, block, 0, s, w, dst); break;

@@ -228,6 +228,77 @@ __device__ __forceinline__ void decode_quad(const uint8_t* __restrict__ p, uint3
     }
 }
 
+// ---- four-tier mixes: one wavefront decodes one block, lane l its weights 4 l .. 4 l + 3
+// The position of a weight's value in the stream is its rank among the weights of its tier, so the
+// wavefront counts tiers per lane, scans the counts over the lanes and reads each value at
+// (start of the tier's run) + rank * width.  As in dequant_quad_mix (src/codec/block_codec.cpp:2207-2380),
+// a tier's run holds min(c[t], weights mapped to t) values, surplus weights of a tier stay zero, and the
+// stream ends at payload_bytes (bits past it read as zero).  All 64 lanes must call this together.
+__device__ __forceinline__ uint32_t mix_bits(const uint8_t* p, uint32_t size, uint32_t pos, int count) {
+    if (count <= 16) return stream_bits(p, size, pos, count);
+    return stream_bits(p, size, pos, 16) | (stream_bits(p, size, pos + 16, count - 16) << 16);
+}
+
+__device__ __forceinline__ float mix_value(int bits, uint32_t code, float s) {
+    switch (bits) {
+        case 1: return s * (code == 0 ? -1.0f : 1.0f);
+        case 3: return fixed_value(3, code) * s;
+        case 16: return half_bits_to_float(code);
+        case 24: return __uint_as_float(code << 8);
+        case 32: return __uint_as_float(code);
+        default: return grid_value(bits, code) * s;  // 2, 4: Lloyd-Max grids; 8: -8 + 16 i / 255
+    }
+}
+
+// per-lane tier counts -> exclusive prefix over lanes (lo: tiers 0 and 1, hi: tiers 2 and 3, 16 bits each)
+// and the block totals
+__device__ __forceinline__ void mix_scan(uint32_t tiers, int valid, uint32_t lane, uint32_t (&before)[4], uint32_t (&total)[4]) {
+    uint32_t lo = 0, hi = 0;
+    for (int k = 0; k < valid; ++k) {
+        const uint32_t t = (tiers >> (2 * k)) & 3u;
+        if (t < 2) lo += 1u << (16 * t); else hi += 1u << (16 * (t - 2));
+    }
+    uint32_t slo = lo, shi = hi;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t a = __shfl_up(slo, d, 64), b = __shfl_up(shi, d, 64);
+        if (lane >= (uint32_t)d) { slo += a; shi += b; }
+    }
+    const uint32_t tlo = __shfl(slo, 63, 64), thi = __shfl(shi, 63, 64);
+    slo -= lo; shi -= hi;
+    before[0] = slo & 0xFFFFu; before[1] = slo >> 16; before[2] = shi & 0xFFFFu; before[3] = shi >> 16;
+    total[0] = tlo & 0xFFFFu; total[1] = tlo >> 16; total[2] = thi & 0xFFFFu; total[3] = thi >> 16;
+}
+
+__device__ __forceinline__ void mix_decode_wave(const MixLayout& L, const uint8_t* __restrict__ p, uint32_t lane, float (&v)[4]) {
+    const int valid = max(0, min(4, L.n - 4 * (int)lane));
+    const uint32_t tiers = valid > 0 ? p[lane] : 0u;
+    uint32_t before[4], total[4];
+    mix_scan(tiers, valid, lane, before, total);
+    uint32_t start[4];
+    uint32_t at = 2u * (uint32_t)L.n;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        start[t] = at;
+        at += min((uint32_t)L.c[t], total[t]) * (uint32_t)L.bits[t];
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        v[k] = 0.0f;
+        if (k >= valid) continue;
+        const uint32_t t = (tiers >> (2 * k)) & 3u;
+        const uint32_t r = before[t]++;
+        if (r >= (uint32_t)L.c[t]) continue;
+        const uint32_t code = mix_bits(p, (uint32_t)L.payload_bytes, start[t] + r * (uint32_t)L.bits[t], L.bits[t]);
+        float s = 1.0f;
+        if (L.nsc[t] > 0) {
+            const uint8_t* q = p + L.sc_at[t] + 2 * min((int)(r >> 5), L.nsc[t] - 1);
+            s = half_bits_to_float((uint32_t)q[0] | ((uint32_t)q[1] << 8));
+        }
+        v[k] = mix_value(L.bits[t], code, s);
+    }
+}
+
 // Weight i of a block of L.n <= 256 weights.  Every part of such a block is one
 // LSB-first bit stream without byte alignment between the parts, except where the
 // reference's encoder places a trailer at a byte offset (noted below).

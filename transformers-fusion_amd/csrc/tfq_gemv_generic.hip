@@ -114,11 +114,80 @@ int batched(const tfq_weight* w, const void* x, int xd, int B, void* y, int yd, 
     return TFQ_OK;
 }
 
+// The four-tier mixes: same shape, the block decoded by the whole wavefront (mix_decode_wave), the
+// layout a kernel argument because it is a function of the wire id alone.
+template <int BT, bool XF32>
+__global__ __launch_bounds__(256) void gemv_mix_kernel(MixLayout L, const uint8_t* __restrict__ W, const void* __restrict__ xin,
+                                                       void* __restrict__ yout, int N, int K, int y_bf16) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nblk = K >> 8;
+    for (int row = blockIdx.x * 4 + wave; row < N; row += gridDim.x * 4) {
+        float acc[BT];
+#pragma unroll
+        for (int b = 0; b < BT; ++b) acc[b] = 0.0f;
+        const uint8_t* prow = W + (size_t)row * (size_t)nblk * L.bytes;
+        for (int blk = 0; blk < nblk; ++blk) {
+            float w[4];
+            mix_decode_wave(L, prow + (size_t)blk * L.bytes, (uint32_t)lane, w);
+            const size_t k0 = (size_t)blk * 256 + 4 * lane;
+#pragma unroll
+            for (int b = 0; b < BT; ++b) {
+                float xv[4];
+                if constexpr (XF32) {
+                    const float4 v = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(xin) + (size_t)b * K + k0);
+                    xv[0] = v.x; xv[1] = v.y; xv[2] = v.z; xv[3] = v.w;
+                } else {
+                    const uint2 v = *reinterpret_cast<const uint2*>(reinterpret_cast<const unsigned short*>(xin) + (size_t)b * K + k0);
+                    xv[0] = __uint_as_float(v.x << 16); xv[1] = __uint_as_float(v.x & 0xFFFF0000u);
+                    xv[2] = __uint_as_float(v.y << 16); xv[3] = __uint_as_float(v.y & 0xFFFF0000u);
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[b] = __builtin_fmaf(w[t], xv[t], acc[b]);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            const float v = wave_sum_lane63(acc[b]);
+            if (lane == 63) {
+                if (y_bf16) reinterpret_cast<unsigned short*>(yout)[(size_t)b * N + row] = (unsigned short)bf16_rne(v);
+                else reinterpret_cast<float*>(yout)[(size_t)b * N + row] = v;
+            }
+        }
+    }
+}
+
+template <int BT>
+int run_mix(const tfq_weight* w, const void* x, int xd, void* y, int yd, hipStream_t s) {
+    const int N = (int)w->N, K = (int)w->K;
+    const int grid = (N + 3) / 4 < 4096 ? (N + 3) / 4 : 4096;
+    const MixLayout L = mix_layout(w->fmt, 256);
+    if (xd == TFQ_F32)
+        hipLaunchKernelGGL((gemv_mix_kernel<BT, true>), dim3(grid), dim3(256), 0, s, L, w->dev, x, y, N, K, yd == TFQ_BF16);
+    else
+        hipLaunchKernelGGL((gemv_mix_kernel<BT, false>), dim3(grid), dim3(256), 0, s, L, w->dev, x, y, N, K, yd == TFQ_BF16);
+    return hip_fail(hipGetLastError(), "gemv launch");
+}
+
+int batched_mix(const tfq_weight* w, const void* x, int xd, int B, void* y, int yd, hipStream_t s) {
+    const size_t xe = xd == TFQ_F32 ? 4 : 2, ye = yd == TFQ_F32 ? 4 : 2;
+    for (int b0 = 0; b0 < B;) {
+        const int left = B - b0;
+        const int nb = left >= 4 ? 4 : left >= 2 ? 2 : 1;
+        const void* xb = (const uint8_t*)x + (size_t)b0 * w->K * xe;
+        void* yb = (uint8_t*)y + (size_t)b0 * w->N * ye;
+        const int rc = nb == 4 ? run_mix<4>(w, xb, xd, yb, yd, s) : nb == 2 ? run_mix<2>(w, xb, xd, yb, yd, s) : run_mix<1>(w, xb, xd, yb, yd, s);
+        if (rc) return rc;
+        b0 += nb;
+    }
+    return TFQ_OK;
+}
+
 }  // namespace
 
 int launch_gemv_generic(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype, hipStream_t s) {
     if (w->layout != TFQ_LAYOUT_WIRE) return fail(TFQ_ERR_FORMAT, "gemv: generic kernel expects the wire layout");
     if (w->N > 0x7FFFFFFF || w->K > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "gemv: shape too large");
+    if (is_mix(w->fmt)) return batched_mix(w, x, x_dtype, B, y, y_dtype, s);
     switch (canonical(w->fmt)) {
         case TFQ_Q_32: return batched<TFQ_Q_32>(w, x, x_dtype, B, y, y_dtype, s);
         case TFQ_Q_1: return batched<TFQ_Q_1>(w, x, x_dtype, B, y, y_dtype, s);

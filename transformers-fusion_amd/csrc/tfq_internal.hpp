@@ -13,7 +13,7 @@
 namespace tfq {
 
 // ------------------------------------------------------------------ formats
-enum class Codec : int { None = 0, Raw32, Lattice, Affine, Grp8, Sym32, Grp16, Q6K, Q1, Q16, Q24, Fixed, Grp12 };
+enum class Codec : int { None = 0, Raw32, Lattice, Affine, Grp8, Sym32, Grp16, Q6K, Q1, Q16, Q24, Fixed, Grp12, Mix };
 
 // Layout parameters of one wire format.  The affine family is the reference's
 // parametric codec quant_affine(bits, w, n, gsz, scb, mb, claimed)
@@ -38,7 +38,113 @@ struct Spec {
 // Q24: the top three bytes of the binary32 (:1809-1873).  For Q16 / Q24, scb = 1 marks the ids that
 // append a binary16 residual mean per 32 weights when the claimed size leaves room.
 
+// ---- four-tier mixes (Q_MX_*, Q_G_MX_*; src/codec/block_codec.cpp:1875-2380)
+// Every weight carries a 2-bit tier; the tiers hold fixed shares of a block, the largest magnitudes in
+// the widest tier.  One bit stream: n 2-bit tiers, then the values of tier 0, 1, 2, 3; then, byte
+// aligned, binary16 scales: one per tier narrower than 16 bits, or one per 32 values of the most
+// populated tier for the grouped ids.  Values: 1 bit = sign, 2/4/8 = plain lattice grid, 3 = fixed
+// codebook, 16 = binary16, 24 = top three bytes of the binary32, 32 = the binary32.  All sizes follow
+// from (id, n) alone.
+struct MixLayout {
+    int n;
+    int bits[4];     // value width per tier
+    int c[4];        // weights per tier
+    int nsc[4];      // scales per tier
+    int sc_at[4];    // byte offset of a tier's first scale
+    int payload_bytes, bytes;
+};
+
+__host__ __device__ constexpr bool is_mix(int fmt) { return fmt >= TFQ_Q_MX_3_5 && fmt <= TFQ_Q_G_MX_24_5; }
+
+__host__ __device__ constexpr MixLayout mix_layout(int fmt, int n) {
+    // tier widths and shares in percent (:1950-1968), bits per weight of the claim (include/quant/types.h:224-227)
+    constexpr int kBits[14][4] = {{1, 2, 4, 32}, {1, 2, 4, 32}, {1, 2, 4, 32}, {1, 2, 4, 32}, {1, 3, 8, 32}, {1, 2, 16, 32}, {1, 2, 24, 32},
+                                  {1, 2, 4, 32}, {1, 2, 4, 32}, {1, 3, 4, 32}, {1, 3, 4, 32}, {1, 2, 8, 32}, {1, 2, 16, 32}, {1, 2, 24, 32}};
+    constexpr float kShare[14][3] = {{92.0f, 1.5f, 6.0f}, {58.5f, 2.0f, 39.0f}, {1.5f, 4.0f, 93.0f}, {2.5f, 1.0f, 88.0f}, {0.5f, 2.0f, 87.5f},
+                                     {4.5f, 7.0f, 88.0f}, {2.5f, 5.0f, 92.0f},
+                                     {92.0f, 4.0f, 3.0f}, {58.5f, 1.0f, 39.5f}, {0.5f, 5.0f, 93.0f}, {0.5f, 2.0f, 89.0f}, {1.5f, 2.5f, 85.0f},
+                                     {10.0f, 1.0f, 88.0f}, {2.5f, 5.0f, 91.5f}};
+    constexpr float kClaim[14] = {3.5f, 4.5f, 6.5f, 8.5f, 12.5f, 16.5f, 24.5f, 3.78125f, 4.5f, 6.5f, 8.5f, 12.5f, 16.5f, 24.5f};
+    const int id = fmt - TFQ_Q_MX_3_5;
+    const bool grp = id >= 7;
+    MixLayout L{};
+    L.n = n;
+    int* c = L.c;
+    for (int t = 0; t < 4; ++t) L.bits[t] = kBits[id][t];
+    // :1974-1995: rounded shares (at least one weight each), the widest tier takes the rest
+    for (int i = 0; i < 3; ++i) {
+        const int r = (int)((double)kShare[id][i] * 0.01 * (double)n + 0.5);  // lround of a positive value
+        c[i] = r > 1 ? r : 1;
+    }
+    c[3] = n - c[0] - c[1] - c[2];
+    if (c[3] < 1) {
+        c[3] = 1;
+        int excess = c[0] + c[1] + c[2] + 1 - n;
+        for (int i = 0; i < 3 && excess > 0; ++i) {
+            const int rem = c[i] - 1 < excess ? c[i] - 1 : excess;
+            c[i] -= rem;
+            excess -= rem;
+        }
+    }
+    for (int i = 0; i < 4; ++i) c[i] = c[i] < 0 ? 0 : c[i] > n ? n : c[i];
+    int sum = c[0] + c[1] + c[2] + c[3];
+    for (int i = 0; i < 4 && sum > n; ++i) {
+        const int rem = c[i] < sum - n ? c[i] : sum - n;
+        c[i] -= rem;
+        sum -= rem;
+    }
+    // :1898-1923: while the layout is over the claim, a weight moves down one tier
+    const double claim_bits = (double)kClaim[id] * (double)n;
+    const long budget_bits = (long)claim_bits + ((double)(long)claim_bits < claim_bits ? 1 : 0);
+    for (int guard = 0; guard < 4 * n; ++guard) {
+        long total = 2L * n;
+        for (int t = 0; t < 4; ++t) total += (long)c[t] * L.bits[t];
+        int dom = 0;
+        for (int t = 1; t < 4; ++t) if (c[t] > c[dom]) dom = t;
+        for (int t = 0; t < 4; ++t)
+            if (L.bits[t] < 16) total += (grp && t == dom) ? 16L * ((c[t] + 31) / 32) : 16;
+        if (total <= budget_bits) break;
+        bool moved = false;
+        for (int t = 3; t >= 1; --t) {
+            if (c[t] > 1 && L.bits[t] > L.bits[t - 1]) {
+                --c[t];
+                ++c[t - 1];
+                moved = true;
+                break;
+            }
+        }
+        if (!moved) break;
+    }
+    int dom = 0;
+    for (int t = 1; t < 4; ++t) if (c[t] > c[dom]) dom = t;
+    // :1932-1945: a block too small for the map and the scales keeps bare signs only
+    long payload = 2L * n, scales = 0;
+    for (int t = 0; t < 4; ++t) {
+        payload += (long)c[t] * L.bits[t];
+        if (L.bits[t] >= 16 || c[t] == 0) continue;
+        scales += ((grp && t == dom) ? (c[t] + 31) / 32 : 1) * 2;
+    }
+    const bool collapsed = (payload + 7) / 8 + scales > (budget_bits + 7) / 8;
+    if (collapsed) { c[0] = n; c[1] = c[2] = c[3] = 0; }
+    long bits = 2L * n;
+    for (int t = 0; t < 4; ++t) bits += (long)c[t] * L.bits[t];
+    L.payload_bytes = (int)((bits + 7) / 8);
+    int at = L.payload_bytes;
+    for (int t = 0; t < 4; ++t) {
+        L.sc_at[t] = at;
+        if (collapsed || L.bits[t] >= 16 || c[t] == 0) continue;
+        L.nsc[t] = (grp && t == dom) ? (c[t] + 31) / 32 : 1;
+        at += 2 * L.nsc[t];
+    }
+    L.bytes = at;
+    return L;
+}
+
 __host__ __device__ constexpr Spec spec_of(int fmt) {
+    if (is_mix(fmt)) {
+        constexpr float kClaim[14] = {3.5f, 4.5f, 6.5f, 8.5f, 12.5f, 16.5f, 24.5f, 3.78125f, 4.5f, 6.5f, 8.5f, 12.5f, 16.5f, 24.5f};
+        return {Codec::Mix, 0, fmt >= TFQ_Q_G_MX_3_5 ? 1 : 0, 0, 0, kClaim[fmt - TFQ_Q_MX_3_5], mix_layout(fmt, 256).bytes};
+    }
     switch (fmt) {
         case TFQ_Q_32: return {Codec::Raw32, 32, 0, 0, 0, 32.0f, 1024};
         case TFQ_Q_1: case TFQ_Q_1_K_L: case TFQ_Q_1_K_M: case TFQ_Q_1_K_H:
@@ -206,14 +312,14 @@ namespace tfq {
 // Layout of one block of n <= 256 weights, as the reference's codecs choose it from
 // (format, n): short blocks drop or shrink their headers.  Filled on the host, passed
 // to the short-block decode kernel by value.
-enum : int { BK_RAW32 = 0, BK_LEVELS, BK_LATTICE, BK_AFFINE, BK_GRP16, BK_Q6K, BK_GRP8, BK_SYM32, BK_Q1, BK_WIDE, BK_GRP12 };
+enum : int { BK_RAW32 = 0, BK_LEVELS, BK_LATTICE, BK_AFFINE, BK_GRP16, BK_Q6K, BK_GRP8, BK_SYM32, BK_Q1, BK_WIDE, BK_GRP12, BK_MIX };
 struct BlockLayout {
     int kind;
     int bits;   // code width
     int n;      // weights in the block
     int bytes;  // payload bytes
     int gsz, ng, scb, mb;  // affine: group size, group count, scale / min code widths
-    int aux;    // BK_LEVELS / BK_LATTICE: 1 when the levels are the fixed codebook's.  BK_GRP16: 0 raw levels, 1 one d, 2 group scales + d.  BK_Q6K: bit 0 d present, bits 8.. stored scale count.
+    int aux;    // BK_MIX: the wire id.  BK_LEVELS / BK_LATTICE: 1 when the levels are the fixed codebook's.  BK_GRP16: 0 raw levels, 1 one d, 2 group scales + d.  BK_Q6K: bit 0 d present, bits 8.. stored scale count.
                 // BK_WIDE: bit 0 residual means follow the plain part, bit 1 packed 16-bit layout (else raw binary16 / 24-bit)
 };
 // false when the format cannot hold a block of n weights
