@@ -70,6 +70,15 @@ __device__ __forceinline__ uint4 pair_permute(uint4 v) {
     return p;
 }
 
+// 16 bytes of the weight stream: every packed byte is read once per launch, so the loads carry the
+// non-temporal hint (the lines are not kept in L2 for a reuse that never comes); measured on MI355X a
+// pure read of 66 MB with this access pattern takes 11.4 us with the hint and 12.4 us without.
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 stream_load16(const uint8_t* p) {
+    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+    return uint4{v.x, v.y, v.z, v.w};
+}
+
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float v) {
     const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false);
@@ -320,9 +329,9 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     const uint32_t off_c = 16u * lane, off_h = 1024u * NC + (uint32_t)F::HB * n;
     auto fetch = [&](uint4 (&cc)[NC], uint4 (&hd)[F::HV]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < NC; ++i) cc[i] = *reinterpret_cast<const uint4*>(f_ptr + off_c + 1024 * i);
+        for (int i = 0; i < NC; ++i) cc[i] = stream_load16(f_ptr + off_c + 1024 * i);
 #pragma unroll
-        for (int i = 0; i < F::HV; ++i) hd[i] = *reinterpret_cast<const uint4*>(f_ptr + off_h + 16 * i);
+        for (int i = 0; i < F::HV; ++i) hd[i] = stream_load16(f_ptr + off_h + 16 * i);
         if (--f_left > 0) {
             f_ptr += tile_stride;
             if (++f_t == tiles_here) {
