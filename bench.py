@@ -49,7 +49,16 @@ def main():
     ap.add_argument("--no-moe", action="store_true", help="skip the mixture-of-experts layer figure")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one elementwise kernel that reads and writes 1 GiB (counter calibration)")
+    ap.add_argument("--probe", action="store_true",
+                    help="run the machine probe instead (launch floor, pure-read stream, grid barrier) and print its lines")
     args = ap.parse_args()
+    if args.probe:
+        import subprocess
+        exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "transformers-fusion_amd", "tfq_probe")
+        if not os.path.exists(exe):
+            print(f"bench.py: {exe} is missing: run __graft_entry__.build() first", file=sys.stderr)
+            sys.exit(2)
+        sys.exit(subprocess.call([exe]))
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus above 1 is not supported "
               "(rows shard over GPUs without a collective, see DESIGN.md)", file=sys.stderr)
