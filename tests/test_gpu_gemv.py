@@ -242,3 +242,58 @@ def test_gemv_many_tiles_per_workgroup(O, tfq, gpu, fmt, N, K, B):
     err = float((y.double() - want).abs().max() / want.abs().max())
     assert err <= 1e-4, err
     W.close()
+
+
+@pytest.mark.parametrize("fmt", ["B32S4", "Q_G_4", "B32S8", "Q_G_8", "Q_8"])
+@pytest.mark.parametrize("N,K,B", [(16 * 256 * 3 + 40, 512, 16), (16 * 300, 4096, 9), (4096, 14336, 16), (1040, 4608, 5),
+                                   (16 * 256 * 9, 256, 13), (24, 7168, 8)])
+def test_gemv_five_to_sixteen_rows(O, tfq, gpu, fmt, N, K, B):
+    """Five or more bf16 rows take the tile-major kernel: several tiles per workgroup, K in chunks of 16 block
+    columns (one chunk, a partial last chunk, four chunks), rows not a multiple of four, more tiles than one
+    round of workgroups holds.  Checked against a dense product of the device-decoded matrix (bit-exact by the
+    codec tests), fp32 and bf16 outputs."""
+    import torch
+    print(f"gemv rows {fmt} N={N} K={K} B={B}", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(N + K + B)
+    if fmt in ("B32S4", "B32S8"):
+        pay = tfq.encode(fmt, torch.randn(N * K, device=gpu, generator=g) * 0.02)
+    else:
+        bb = tfq.block_bytes(fmt)
+        pay = torch.randint(0, 256, (N * K // 256, bb), device=gpu, dtype=torch.uint8, generator=g)
+        if fmt == "Q_G_4":
+            pay[:, -4:] = torch.tensor([0x00, 0x20, 0x00, 0x20], dtype=torch.uint8, device=gpu)
+        elif fmt == "Q_G_8":
+            pay[:, -16:] = torch.tensor([0x00, 0x20] * 8, dtype=torch.uint8, device=gpu)
+        else:
+            pay[:, :2] = torch.tensor([0x00, 0x20], dtype=torch.uint8, device=gpu)
+        pay = pay.reshape(-1)
+    W = tfq.Weight(fmt, N, K, pay)
+    x = torch.randn(B, K, device=gpu, generator=g).bfloat16()
+    want = x.double() @ W.decode().double().T
+    scale = float(want.abs().max())
+    y = W.gemv(x)
+    tol = 1e-4 if fmt in ("B32S4", "Q_G_4", "B32S8") else 1e-3  # the companded formats multiply through a line fit
+    assert float((y.double() - want).abs().max()) <= tol * scale
+    yb = W.gemv(x, out_dtype=torch.bfloat16)
+    assert float((yb.double() - want).abs().max()) <= 1e-2 * scale
+    # every row equals the single-row product of the same kernel family to rounding
+    one = W.gemv(x[B - 1:B])
+    assert float((y[B - 1] - one[0]).abs().max()) <= 2e-5 * scale
+    W.close()
+
+
+def test_gemv_multi_with_eight_rows(O, tfq, gpu):
+    """q/k/v style launch with more than four rows: three matrices, one launch of the tile-major kernel."""
+    import torch
+    K, B = 4096, 8
+    shapes = [4096, 1024, 1040]
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(B, K, device=gpu, generator=g).bfloat16()
+    Ws = [tfq.Weight("B32S4", N, K, tfq.encode("B32S4", torch.randn(N * K, device=gpu, generator=g) * 0.02)) for N in shapes]
+    outs = [torch.zeros(B, N, device=gpu) for N in shapes]
+    tfq.gemv_multi(Ws, x, outs)
+    for W, got in zip(Ws, outs):
+        want = x.double() @ W.decode().double().T
+        assert float((got.double() - want).abs().max()) <= 1e-4 * float(want.abs().max())
+        assert torch.equal(got, W.gemv(x))
+        W.close()

@@ -523,6 +523,277 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     TRACE(7);
 }
 
+// (a, off) of the four scale groups of k-step `khalf`: contribution of a group = a * D + off * X
+// (same fields and arithmetic as apply_groups; 32-weight groups only).
+template <int FMT>
+__device__ __forceinline__ void group_scales(const uint4* hv, int khalf, float (&a)[4], float (&off)[4]) {
+    constexpr Spec sp = spec_of(FMT);
+    if constexpr (FMT == TFQ_B32S4 || Fmt<FMT>::NP == 2) {
+        const f16x2_t s01 = __builtin_bit_cast(f16x2_t, khalf ? hv[0].z : hv[0].x);
+        const f16x2_t s23 = __builtin_bit_cast(f16x2_t, khalf ? hv[0].w : hv[0].y);
+        a[0] = (float)s01.x; a[1] = (float)s01.y; a[2] = (float)s23.x; a[3] = (float)s23.y;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) off[t] = 0.0f;
+    } else {
+        constexpr int NG = Fmt<FMT>::NG;
+        constexpr int sc_bits = ((NG * sp.scb + 7) / 8) * 8, mn_bits = ((NG * sp.mb + 7) / 8) * 8;
+        constexpr int mbias = (1 << sp.mb) / 2;
+        constexpr float inv_top = sp.bits == 4 ? 1.0f / 15.0f : sp.bits == 3 ? 1.0f / 7.0f : 1.0f / 3.0f;
+        const uint32_t w[4] = {hv[0].x, hv[0].y, hv[0].z, hv[0].w};
+        const uint32_t dd = field(w, sc_bits + mn_bits, 32);
+        const float dtop = half_fast(dd & 0xFFFFu) * inv_top;
+        const float dm = half_fast(dd >> 16);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int g = khalf * 4 + t;
+            a[t] = dtop * (float)field(w, g * sp.scb, sp.scb);
+            off[t] = dm * (float)(mbias - (int)field(w, sc_bits + g * sp.mb, sp.mb));
+        }
+    }
+}
+
+// 4 x 4 transpose of dwords across the four 16-lane rows of a wavefront: lane (n, q) gives v[j] = M[q][j]
+// and receives v[g] = M[g][q] (v_permlane32_swap exchanges rows 2, 3 of its first operand with rows 0, 1 of
+// the second, v_permlane16_swap the odd rows of the first with the even rows of the second).
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void transpose_rows(uint32_t (&v)[4]) {
+    u32x2_t p = __builtin_amdgcn_permlane32_swap(v[0], v[2], false, false); v[0] = p.x; v[2] = p.y;
+    p = __builtin_amdgcn_permlane32_swap(v[1], v[3], false, false); v[1] = p.x; v[3] = p.y;
+    p = __builtin_amdgcn_permlane16_swap(v[0], v[1], false, false); v[0] = p.x; v[1] = p.y;
+    p = __builtin_amdgcn_permlane16_swap(v[2], v[3], false, false); v[2] = p.x; v[3] = p.y;
+}
+
+// ---- five to sixteen bf16 activation rows: gemvb_kernel
+// With that many rows the activations are the operand that has to be reused (sixteen rows of K = 4096 are
+// 128 KB, more than the packed weights a workgroup streams per tile), so the walk is arranged around them:
+//   * K is cut into chunks of KC = 16 block columns.  A workgroup of eight wavefronts stages a chunk of the
+//     activations ONCE (all threads together, bf16 in the MFMA's A-fragment order, group sums beside them);
+//     wavefront w then takes the A fragments of ITS block columns w and w + 8 into registers and visits all
+//     the workgroup's T tiles for that chunk without touching LDS for operands again;
+//   * the MFMA is used densely: A holds up to sixteen activation rows of ONE scale group (lane (s, kq):
+//     elements 8 kq .. 8 kq + 7 of the group, row s), B the 32 weights of that group for sixteen weight rows,
+//     so a unit costs eight MFMAs whatever the row count.  A lane holds its code dwords group-major (group q,
+//     dwords 0..3); transpose_rows makes register g of lane (n, q) dword q of group g.  D[4 q + r][n] comes
+//     out in lane (n, q), register r;
+//   * every wavefront adds its partial sums into its own LDS cells per tile (no barrier while streaming);
+//     after the last chunk the eight partials of each output are added in wavefront order.  With a single K
+//     chunk (K <= 4096) the cells reuse the LDS of the staged activations, which are in registers by then,
+//     and a workgroup can hold many tiles; with several chunks they need room of their own (few tiles).
+// Unit fetches run four ahead (two tiles x two columns) with unconditional loads, as in gemv4_kernel.
+constexpr int kGemvbNW = 8, kGemvbKC = 16;
+constexpr int kGemvbMaxT1 = 16;  // tiles per workgroup, single chunk: 16 x 8 KB of cells inside the staging area
+constexpr int kGemvbMaxTn = 2;   // several chunks: cells behind the staging area
+
+template <int FMT>
+__global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const unsigned short* __restrict__ x) {
+    extern __shared__ uint4 smem[];
+    using F = Fmt<FMT>;
+    static_assert(F::GS == 32 && F::HV == 1, "32-weight groups and a 16-byte header");
+    constexpr int UB = tiled_unit_bytes(FMT), NC = 2 * F::NP, NW = kGemvbNW, KC = kGemvbKC;
+    // unit fetches in flight per wavefront: TW tiles x two columns (four tiles measured no faster)
+    constexpr int TW = 2, WD = 2 * TW;
+    const int K = args.K, T = args.tiles_per_wg, B = args.nslot;
+    const bool y_bf16 = args.y_bf16 != 0;
+    const int bid = blockIdx.x;
+    const int m = (bid >= args.g0) + (bid >= args.g1) + (bid >= args.g2);
+    const int wg_first = m == 0 ? 0 : m == 1 ? args.g0 : m == 2 ? args.g1 : args.g2;
+    const uint8_t* Wm = m == 0 ? args.W0 : m == 1 ? args.W1 : m == 2 ? args.W2 : args.W3;
+    void* ym = m == 0 ? args.y0 : m == 1 ? args.y1 : m == 2 ? args.y2 : args.y3;
+    const int nrm = m == 0 ? args.nr0 : m == 1 ? args.nr1 : m == 2 ? args.nr2 : args.nr3;
+
+    const int nblocks = K >> 8, nchunks = (nblocks + KC - 1) / KC;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, q = lane >> 4;
+    const int tile0 = (bid - wg_first) * T;
+    const int tiles_here = min(T, ((nrm + 15) >> 4) - tile0);
+    const int total_gt = nchunks * tiles_here;  // (chunk, tile) visits, chunk-major
+
+    uint4* const xa = smem;                                          // [KC][2 k-steps][4 groups][64 lanes]
+    float* const xsum = reinterpret_cast<float*>(smem + KC * 512);   // [KC][8 groups][16 rows]
+    // partial sums [T][NW][64 lanes][4]: inside xa when there is one chunk, behind xsum otherwise
+    float* const cells = nchunks == 1 ? reinterpret_cast<float*>(smem) : xsum + KC * 128;
+
+    // ---- unit fetch cursor in consumption order: chunk, tile, column slot (two per wavefront and chunk).
+    // A slot past the last block column re-reads the last one (never used); past the end the cursor parks.
+    int f_chunk = 0, f_t = 0, f_ci = 0;
+    const uint32_t off_c = 16u * lane, off_h = 1024u * NC + 16u * n;
+    auto fetch = [&](uint4 (&cc)[NC], uint4& hd) __attribute__((always_inline)) {
+        const int col = min(f_chunk * KC + wave + NW * f_ci, nblocks - 1);
+        const uint8_t* p = Wm + ((size_t)(tile0 + f_t) * nblocks + (size_t)col) * UB;
+#pragma unroll
+        for (int i = 0; i < NC; ++i) cc[i] = stream_load16(p + off_c + 1024 * i);
+        hd = stream_load16(p + off_h);
+        if (++f_ci == 2) {
+            f_ci = 0;
+            if (++f_t == tiles_here) {
+                f_t = 0;
+                if (f_chunk + 1 < nchunks) ++f_chunk; else f_t = tiles_here - 1, f_ci = 1;  // park on the last unit
+            }
+        }
+    };
+    uint4 cc[WD][NC], hd[WD];
+#pragma unroll
+    for (int u = 0; u < WD; ++u) fetch(cc[u], hd[u]);
+
+    const uint32_t ONES = 0x3F803F80u;
+    const uint32_t M = 0x000F000Fu;
+    uint32_t C = 0x43004300u;
+    asm volatile("" : "+v"(C));
+
+    // ---- activations of one K chunk -> LDS.  Item e = (column c, k-step h, group g, row s, slot kq), kq fastest:
+    // four adjacent lanes hold the four 8-element pieces of one group of one row, so their sums meet with two
+    // DPP adds; the entry lands where lane (s, kq) of a wavefront will read it with one 128-bit LDS load.
+    auto stage_chunk = [&](int chunk) __attribute__((always_inline)) {
+        const int cols_here = min(KC, nblocks - chunk * KC);
+        const unsigned short* xc = x + (size_t)chunk * KC * 256;
+        for (int e0 = 0; e0 < cols_here * 512; e0 += 512 * 4) {  // four loads of a thread in flight together
+            uint4 v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int e = e0 + 512 * i + tid;
+                const int kq = e & 3, s = (e >> 2) & 15, g = (e >> 6) & 3, h = (e >> 8) & 1, c = e >> 9;
+                v[i] = uint4{0, 0, 0, 0};
+                if (c < cols_here && s < B)
+                    v[i] = *reinterpret_cast<const uint4*>(xc + (size_t)s * K + c * 256 + h * 128 + g * 32 + kq * 8);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int e = e0 + 512 * i + tid;
+                const int kq = e & 3, s = (e >> 2) & 15, g = (e >> 6) & 3, h = (e >> 8) & 1, c = e >> 9;
+                const uint4 p = pair_permute(v[i]);
+                float sum = dot2(ONES, p.x, 0.0f);
+                sum = dot2(ONES, p.y, sum);
+                sum = dot2(ONES, p.z, sum);
+                sum = dot2(ONES, p.w, sum);
+                sum = dpp_add<0xB1>(sum);
+                sum = dpp_add<0x4E>(sum);
+                if (c < cols_here) {
+                    xa[((c * 2 + h) * 4 + g) * 64 + kq * 16 + s] = p;
+                    if (kq == 0) xsum[(c * 8 + h * 4 + g) * 16 + s] = sum;
+                }
+            }
+        }
+    };
+
+    // ---- the wavefront's A fragments of its two block columns of the chunk (64 registers), and the group sums
+    // too where the unit ring leaves room (one nibble plane); otherwise the sums are read from LDS per unit
+    constexpr bool XREG = false;  // keeping the sums in registers as well spills a few registers
+    uint4 avr[2][2][4];
+    float4 xr[XREG ? 2 : 1][2][4];
+    auto load_columns = [&](int chunk) __attribute__((always_inline)) {
+#pragma unroll
+        for (int ci = 0; ci < 2; ++ci) {
+            const int c_local = wave + NW * ci;
+            if (chunk * KC + c_local >= nblocks) continue;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    avr[ci][h][g] = xa[((c_local * 2 + h) * 4 + g) * 64 + lane];
+                    if constexpr (XREG) xr[ci][h][g] = *reinterpret_cast<const float4*>(xsum + (c_local * 8 + h * 4 + g) * 16 + 4 * q);
+                }
+        }
+    };
+
+    // ---- one unit: the lane's contribution to D[4 q + r][n], r = 0..3, added into res
+    auto compute = [&](int ci, int c_local, const uint4 (&cw_all)[NC], const uint4& hdr, float (&res)[4]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            f32x4_t D[4], D2[4];
+            float X[4][4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float4 xv;
+                if constexpr (XREG) xv = xr[ci][h][g];
+                else xv = *reinterpret_cast<const float4*>(xsum + (c_local * 8 + h * 4 + g) * 16 + 4 * q);
+                X[g][0] = xv.x; X[g][1] = xv.y; X[g][2] = xv.z; X[g][3] = xv.w;
+                D[g] = f32x4_t{-F::OFFS * xv.x, -F::OFFS * xv.y, -F::OFFS * xv.z, -F::OFFS * xv.w};
+                D2[g] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+#pragma unroll
+            for (int pl = 0; pl < F::NP; ++pl) {
+                const uint4 cw = cw_all[2 * pl + h];
+                uint32_t t[4] = {cw.x, cw.y, cw.z, cw.w};
+                transpose_rows(t);
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const uint32_t v = t[g];
+                    const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
+                    if (pl == 0)
+                        D[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, avr[ci][h][g]),
+                                                                       __builtin_bit_cast(bf16x8_t, wv), D[g], 0, 0, 0);
+                    else
+                        D2[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, avr[ci][h][g]),
+                                                                        __builtin_bit_cast(bf16x8_t, wv), D2[g], 0, 0, 0);
+                }
+            }
+            float a[4], off[4];
+            group_scales<FMT>(&hdr, h, a, off);
+            float ph[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float d = D[g][r];
+                    if constexpr (F::NP == 2) d = __builtin_fmaf(16.0f, D2[g][r], d);
+                    ph[r] = __builtin_fmaf(a[g], d, ph[r]);
+                    if constexpr (!(FMT == TFQ_B32S4 || F::NP == 2)) ph[r] = __builtin_fmaf(off[g], X[g][r], ph[r]);
+                }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) res[r] += F::COMP8 ? ph[r] * kComp8Gain : ph[r];
+        }
+    };
+
+    for (int gt0 = 0; gt0 < total_gt; gt0 += TW) {
+#pragma unroll
+        for (int dt = 0; dt < TW; ++dt) {
+            const int gt = gt0 + dt;
+            if (gt < total_gt) {  // uniform over the workgroup
+                const int chunk = gt / tiles_here, t = gt - chunk * tiles_here;
+                if (t == 0) {
+                    __syncthreads();  // every wavefront holds the previous chunk's fragments in registers, or is done with them
+                    stage_chunk(chunk);
+                    __syncthreads();
+                    load_columns(chunk);
+                    if (nchunks == 1) __syncthreads();  // the cells below overwrite the staged activations
+                }
+                float res[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int ci = 0; ci < 2; ++ci) {
+                    const int u = dt * 2 + ci;
+                    const int c_local = wave + NW * ci;
+                    if (chunk * KC + c_local < nblocks) compute(ci, c_local, cc[u], hd[u], res);
+                    fetch(cc[u], hd[u]);
+                }
+                float4* cell = reinterpret_cast<float4*>(cells) + (t * NW + wave) * 64 + lane;
+                if (chunk == 0) *cell = float4{res[0], res[1], res[2], res[3]};
+                else { const float4 o = *cell; *cell = float4{o.x + res[0], o.y + res[1], o.z + res[2], o.w + res[3]}; }
+            }
+        }
+    }
+    __syncthreads();
+    // ---- add the eight wavefronts' partials in order and store: thread tid < 256 owns D[4 q' + r][n'] with
+    // (n', q') = lane id tid % 64 and r = tid / 64, for every tile
+    if (tid < 256) {
+        const int nn = tid & 15, qq = (tid >> 4) & 3, r = tid >> 6;
+        const int slot = 4 * qq + r;
+        if (slot < B) {
+            for (int t = 0; t < tiles_here; ++t) {
+                const int row = (tile0 + t) * 16 + nn;
+                if (row >= nrm) continue;
+                const float* src = cells + ((size_t)t * NW * 64 + (tid & 63)) * 4 + r;
+                float v = 0.0f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) v += src[w * 256];
+                const size_t off = (size_t)slot * (size_t)nrm + (size_t)row;
+                if (y_bf16) reinterpret_cast<unsigned short*>(ym)[off] = (unsigned short)bf16_rne(v);
+                else reinterpret_cast<float*>(ym)[off] = v;
+            }
+        }
+    }
+}
+
 // Formats whose kernel is also built with several slot sets per pass (up to 16 bf16 rows).
 template <int FMT>
 constexpr bool kWide = FMT == TFQ_B32S4 || FMT == TFQ_B32S8 || FMT == TFQ_Q_G_4 || FMT == TFQ_Q_G_8 || FMT == TFQ_Q_8;
@@ -622,6 +893,46 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     return hip_fail(hipGetLastError(), "gemv launch");
 }
 
+// Launch of gemvb_kernel: nb = 5..16 bf16 activation rows in one pass.
+template <int FMT>
+int run_gemvb(GemvArgs a, const void* x, hipStream_t s) {
+    constexpr int num_cu = 256;
+    auto grid_for = [&](int T) {
+        int g = 0;
+        for (int m = 0; m < a.nmat; ++m) g += ((a.nrows[m] + 15) / 16 + T - 1) / T;
+        return g;
+    };
+    const int nchunks = ((a.K >> 8) + kGemvbKC - 1) / kGemvbKC;
+    const int max_t = nchunks == 1 ? kGemvbMaxT1 : kGemvbMaxTn;
+    int T = (a.ntiles + num_cu - 1) / num_cu;
+    while (grid_for(T) > num_cu && T < max_t) ++T;
+    if (T > max_t) T = max_t;
+    GemvKernArgs k{};
+    k.W0 = a.W[0]; k.W1 = a.W[1]; k.W2 = a.W[2]; k.W3 = a.W[3];
+    k.y0 = a.y[0]; k.y1 = a.y[1]; k.y2 = a.y[2]; k.y3 = a.y[3];
+    k.nr0 = a.nrows[0]; k.nr1 = a.nrows[1]; k.nr2 = a.nrows[2]; k.nr3 = a.nrows[3];
+    int ends[3], g = 0;
+    for (int m = 0; m < 3; ++m) {
+        if (m < a.nmat) g += ((a.nrows[m] + 15) / 16 + T - 1) / T;
+        ends[m] = m < a.nmat ? g : 0x7FFFFFFF;
+    }
+    k.g0 = ends[0]; k.g1 = ends[1]; k.g2 = ends[2];
+    int grid = g;
+    if (a.nmat == 4) grid += ((a.nrows[3] + 15) / 16 + T - 1) / T;
+    k.K = a.K; k.y_bf16 = a.y_bf16; k.nslot = a.nslot; k.tiles_per_wg = T;
+    // staged activations and group sums of a chunk; the cells are inside them (one chunk) or behind them
+    const size_t lds = (size_t)kGemvbKC * (8192 + 512) + (nchunks == 1 ? 0 : (size_t)T * kGemvbNW * 1024);
+    static bool lds_limit_raised = false;
+    if (!lds_limit_raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemvb_kernel<FMT>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
+        lds_limit_raised = true;
+    }
+    hipLaunchKernelGGL(gemvb_kernel<FMT>, dim3(grid), dim3(64 * kGemvbNW), lds, s, k, static_cast<const unsigned short*>(x));
+    return hip_fail(hipGetLastError(), "gemv launch");
+}
+
 template <int FMT>
 int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t s) {
     // One launch carries four bf16 activation rows (two fp32 rows); for the formats built with
@@ -629,6 +940,24 @@ int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t 
     const size_t xe = xd == TFQ_F32 ? 4 : 2, ye = yd == TFQ_F32 ? 4 : 2;
     a.y_bf16 = yd == TFQ_BF16;
     a.x_f32 = xd == TFQ_F32;
+    if constexpr (kWide<FMT>) {
+        // Five rows or more: the tile-major kernel carries sixteen rows per pass at any K.  Measured against the
+        // slot-set kernels below (B32S4): faster for more than eight rows (28672x4096 at 16 rows: 22 us against
+        // 41 us) and wherever those need several passes because their staged activations do not fit
+        // (4096x14336: 22 us against 24 / 47 us at 8 / 16 rows); slower for five to eight rows at K = 4096
+        // (21 us against 17 us), which therefore stay with the two-set kernel.
+        bool tile_major = !a.x_f32 && B > 8;
+        if (!a.x_f32 && B > 4 && B <= 8) tile_major = plan_gemv4<FMT>(a, 8).lds == 0;
+        if (tile_major) {
+            for (int b0 = 0; b0 < B; b0 += 16) {
+                GemvArgs ab = a;
+                ab.nslot = B - b0 < 16 ? B - b0 : 16;
+                for (int m = 0; m < a.nmat; ++m) ab.y[m] = (uint8_t*)a.y[m] + (size_t)b0 * (size_t)a.nrows[m] * ye;
+                if (int rc = run_gemvb<FMT>(ab, (const uint8_t*)x + (size_t)b0 * a.K * xe, s)) return rc;
+            }
+            return TFQ_OK;
+        }
+    }
     int step = a.x_f32 ? 2 : 4;
     if constexpr (kWide<FMT>) {
         if (!a.x_f32 && B > 4) {
