@@ -218,6 +218,20 @@ int tfq_gemv_multi(const tfq_weight_t* const* ws, int count, const void* x, int 
  * shape of Qwen35Engine::gemm(t, X, Y, B). */
 int tfq_matmul_host(const tfq_weight_t* w, const float* X, float* Y, int B);
 
+/* ---- dense SwiGLU feed-forward ----------------------------------------------------
+ * Qwen35Engine::mlp_step (src/adapters/tools/qwen35_engine.cpp:662-672) for B rows:
+ *   y[b] = down( silu(gate x[b]) * (up x[b]) ),  silu(v) = v / (1 + exp(-v))
+ * (src/math/math.cpp:117-126).  gate and up are F x D matrices of one format, down is D x F;
+ * x is [B][D], y is [B][D], device pointers.  Three launches: gate and up in one (they share x),
+ * the elementwise step, down.  mid_dtype is the type the SwiGLU product is rounded to before
+ * the down projection: TFQ_F32 keeps it in fp32 like the reference, TFQ_BF16 feeds the matrix
+ * cores.  workspace is device memory of at least tfq_mlp_workspace_bytes(B, F) bytes, 256-byte
+ * aligned (the gate and up products and the SwiGLU product live there). */
+size_t tfq_mlp_workspace_bytes(int B, int64_t F);
+int tfq_mlp_step(const tfq_weight_t* gate, const tfq_weight_t* up, const tfq_weight_t* down, const void* x,
+                 int x_dtype, int B, void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes,
+                 tfq_stream_t stream);
+
 /* ---- MoE expert path ------------------------------------------------------------
  * tfq_moe_route: router softmax + top-k on the device, softmax_with_topk
  * (src/model/moe_core.cpp:98-149): probs [T][E], idx [T][k] (descending

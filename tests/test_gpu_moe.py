@@ -153,3 +153,32 @@ def test_config5_mixtral_layer_full_size(tfq, gpu):
     assert torch.equal(y2, 2 * y)
     for wl in gate + up + down:
         wl.close()
+
+
+@pytest.mark.parametrize("fmt", ["B32S4", "Q_G_4", "Q_G_8", "Q_G_6"])
+@pytest.mark.parametrize("B,xdt,mid", [(1, "f32", "f32"), (3, "bf16", "bf16"), (16, "bf16", "bf16"), (20, "bf16", "f32")])
+def test_mlp_step_matches_the_oracle(O, tfq, gpu, fmt, B, xdt, mid):
+    """Dense SwiGLU feed-forward (Qwen35Engine::mlp_step): y = down(silu(gate x) * (up x)) against the oracle's
+    block-row matmuls and silu step; formats with and without the multi-matrix kernel, decode and prefill row counts."""
+    import torch
+    D, F = 512, 768
+    print(f"mlp_step {fmt} B={B} {xdt} mid={mid}", flush=True)
+    pays = [O.encode_tensor(fmt, O.rng_normal(70 + i, n * k, 0.02)) for i, (n, k) in enumerate(((F, D), (F, D), (D, F)))]
+    x = O.rng_normal(9, B * D, 1.0).reshape(B, D)
+    if xdt == "bf16":
+        x = O.bf16_round(x)
+    g = O.matmul(fmt, pays[0], F, D, x)
+    u = O.matmul(fmt, pays[1], F, D, x)
+    h = O.silu_mul(g.reshape(-1), u.reshape(-1)).reshape(B, F)
+    if mid == "bf16":
+        h = O.bf16_round(h)
+    want = O.matmul(fmt, pays[2], D, F, h)
+    Ws = [tfq.Weight(fmt, n, k, p) for p, (n, k) in zip(pays, ((F, D), (F, D), (D, F)))]
+    xt = torch.from_numpy(x).to(gpu)
+    if xdt == "bf16":
+        xt = xt.bfloat16()
+    y = tfq.mlp_step(Ws[0], Ws[1], Ws[2], xt, mid_dtype=torch.bfloat16 if mid == "bf16" else torch.float32).cpu().numpy()
+    tol = 1e-3 if xdt == "f32" and mid == "f32" else 1e-2
+    assert float(np.abs(y - want).max()) <= tol * float(np.abs(want).max())
+    for W in Ws:
+        W.close()

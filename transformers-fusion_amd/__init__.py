@@ -72,6 +72,8 @@ def _load():
         "tfq_gemm": (i32, [vp, vp, i32, i32, vp, i32, vp]),
         "tfq_gemv_multi": (i32, [vp, i32, vp, i32, i32, vp, i32, vp]),
         "tfq_matmul_host": (i32, [vp, vp, vp, i32]),
+        "tfq_mlp_workspace_bytes": (sz, [i32, i64]),
+        "tfq_mlp_step": (i32, [vp, vp, vp, vp, i32, i32, vp, i32, i32, vp, sz, vp]),
         "tfq_moe_route": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "tfq_moe_workspace_bytes": (sz, [i32, i32, i64, i64]),
         "tfq_moe_ffn": (i32, [vp, vp, vp, i32, vp, vp, i32, i32, vp, i32, vp, i32, i32, vp, sz, vp]),
@@ -339,6 +341,20 @@ def moe_route(logits, k: int):
     w = torch.empty((T, k), dtype=torch.float32, device=logits.device)
     _check(lib().tfq_moe_route(logits.data_ptr(), T, E, k, probs.data_ptr(), idx.data_ptr(), w.data_ptr(), _stream()))
     return probs, idx, w
+
+
+def mlp_step(gate, up, down, x, out_dtype=None, mid_dtype=None):
+    """Dense SwiGLU feed-forward y = down(silu(gate x) * (up x)) for x [B][D] on the device."""
+    import torch
+    x = x.contiguous()
+    B = x.numel() // gate.K
+    y = torch.empty((B, down.N), dtype=out_dtype or torch.float32, device=x.device)
+    mid = BF16 if (mid_dtype or x.dtype) == torch.bfloat16 else F32
+    nbytes = lib().tfq_mlp_workspace_bytes(B, gate.N)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    _check(lib().tfq_mlp_step(gate.handle, up.handle, down.handle, x.data_ptr(), _dtype_code(x), B, y.data_ptr(),
+                              _dtype_code(y), mid, ws.data_ptr(), nbytes, _stream()))
+    return y
 
 
 def moe_ffn(gate, up, down, topk_idx, topk_w, x, out_dtype=None, mid_dtype=None):

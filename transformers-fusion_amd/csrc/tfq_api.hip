@@ -374,6 +374,18 @@ int tfq_moe_ffn(const tfq_weight_t* const* gate, const tfq_weight_t* const* up, 
                           workspace_bytes, (hipStream_t)stream);
 }
 
+size_t tfq_mlp_workspace_bytes(int B, int64_t F) { return B > 0 && F > 0 ? mlp_workspace_bytes(B, F) : 0; }
+
+int tfq_mlp_step(const tfq_weight_t* gate, const tfq_weight_t* up, const tfq_weight_t* down, const void* x, int x_dtype,
+                 int B, void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes, tfq_stream_t stream) {
+    if (!gate || !up || !down || !workspace) return fail(TFQ_ERR_ARG, "tfq_mlp_step: null pointer");
+    if (mid_dtype != TFQ_F32 && mid_dtype != TFQ_BF16) return fail(TFQ_ERR_ARG, "tfq_mlp_step: dtype must be TFQ_F32 or TFQ_BF16");
+    if ((uintptr_t)workspace % 256) return fail(TFQ_ERR_ARG, "tfq_mlp_step: workspace must be 256-byte aligned");
+    if (int r = check_matmul("tfq_mlp_step", gate, x, x_dtype, B, workspace, TFQ_F32)) return r;
+    if (int r = check_matmul("tfq_mlp_step", down, workspace, mid_dtype, B, y, y_dtype)) return r;
+    return launch_mlp_step(gate, up, down, x, x_dtype, B, y, y_dtype, mid_dtype, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
 int tfq_matmul_host(const tfq_weight_t* w, const float* X, float* Y, int B) {
     if (!w || !X || !Y) return fail(TFQ_ERR_ARG, "tfq_matmul_host: null pointer");
     if (B <= 0) return fail(TFQ_ERR_ARG, "tfq_matmul_host: batch must be positive");

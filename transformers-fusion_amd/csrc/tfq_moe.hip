@@ -309,4 +309,36 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
     return hip_fail(hipGetLastError(), "moe launch");
 }
 
+// Dense SwiGLU feed-forward (Qwen35Engine::mlp_step, src/adapters/tools/qwen35_engine.cpp:662-672): gate and up
+// in one launch where the format has the multi-matrix kernel, the elementwise step, down.  Rows above sixteen go
+// through the prefill entry.
+size_t mlp_workspace_bytes(int B, int64_t F) { return 3 * align256((size_t)B * (size_t)F * 4); }
+
+int launch_mlp_step(const tfq_weight* gate, const tfq_weight* up, const tfq_weight* down, const void* x, int x_dtype, int B,
+                    void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes, hipStream_t s) {
+    const int64_t D = gate->K, F = gate->N;
+    if (up->K != D || up->N != F || down->K != F || down->N != D)
+        return fail(TFQ_ERR_SHAPE, "mlp_step: gate and up must be F x D and down D x F");
+    if (workspace_bytes < mlp_workspace_bytes(B, F)) return fail(TFQ_ERR_SHAPE, "mlp_step: workspace smaller than tfq_mlp_workspace_bytes");
+    const size_t part = align256((size_t)B * (size_t)F * 4);
+    float* g = reinterpret_cast<float*>(workspace);
+    float* u = reinterpret_cast<float*>((uint8_t*)workspace + part);
+    void* h = (uint8_t*)workspace + 2 * part;
+    if (B <= 16 && canonical(gate->fmt) == canonical(up->fmt)) {
+        const tfq_weight* gu[2] = {gate, up};
+        void* gy[2] = {g, u};
+        if (int rc = launch_gemv_multi(gu, 2, x, x_dtype, B, gy, TFQ_F32, s)) return rc;
+    } else {
+        if (int rc = launch_gemm(gate, x, x_dtype, B, g, TFQ_F32, s)) return rc;
+        if (int rc = launch_gemm(up, x, x_dtype, B, u, TFQ_F32, s)) return rc;
+    }
+    const int64_t nh = (int64_t)B * F;
+    if (mid_dtype == TFQ_BF16)
+        hipLaunchKernelGGL(silu_mul_kernel<true>, dim3((unsigned)((nh + 255) / 256)), dim3(256), 0, s, g, u, h, nh);
+    else
+        hipLaunchKernelGGL(silu_mul_kernel<false>, dim3((unsigned)((nh + 255) / 256)), dim3(256), 0, s, g, u, h, nh);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return hip_fail(e, "mlp_step launch");
+    return launch_gemm(down, h, mid_dtype, B, y, y_dtype, s);  // sixteen rows or fewer take the decode kernels inside
+}
+
 }  // namespace tfq

@@ -194,21 +194,16 @@ void BlockRowMatmul::mlp_step(const BlockRowMatmul& gate, const BlockRowMatmul& 
                               const float* x, float* out) {
     if (!gate.ok() || !up.ok() || !down.ok() || !x || !out) return;
     if (gate.rows() != up.rows() || gate.cols() != up.cols() || down.cols() != gate.rows()) return;
-    // One expert, one token, weight 1: the MoE entry point is exactly this chain on the device.
-    const tfq_weight_t* g = gate.handle();
-    const tfq_weight_t* u = up.handle();
-    const tfq_weight_t* dn = down.handle();
-    const int64_t idx = 0;
-    const float wt = 1.0f;
     const int64_t D = gate.cols(), F = gate.rows();
     if (down.rows() != D) return;
     DeviceBuffers d;
-    const size_t wsb = tfq_moe_workspace_bytes(1, 1, D, F);
+    const size_t wsb = tfq_mlp_workspace_bytes(1, F);
     void* ws = d.alloc(wsb);
     const float* dx = static_cast<const float*>(d.upload(x, (size_t)D * 4));
     float* dy = static_cast<float*>(d.alloc((size_t)D * 4));
     if (!ws || !dx || !dy) return;
-    if (tfq_moe_ffn(&g, &u, &dn, 1, &idx, &wt, 1, 1, dx, TFQ_F32, dy, TFQ_F32, TFQ_F32, ws, wsb, nullptr) != TFQ_OK) return;
+    // fp32 throughout, like the reference
+    if (tfq_mlp_step(gate.handle(), up.handle(), down.handle(), dx, TFQ_F32, 1, dy, TFQ_F32, TFQ_F32, ws, wsb, nullptr) != TFQ_OK) return;
     if (tfq_stream_sync(nullptr) != TFQ_OK) return;
     tfq_copy_to_host(out, dy, (size_t)D * 4);
 }
