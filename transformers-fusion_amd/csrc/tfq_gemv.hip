@@ -633,8 +633,10 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
         }
     };
     uint4 cc[WD][NC], hd[WD];
+    TRACE(0);
 #pragma unroll
     for (int u = 0; u < WD; ++u) fetch(cc[u], hd[u]);
+    TRACE(1);
 
     const uint32_t ONES = 0x3F803F80u;
     const uint32_t M = 0x000F000Fu;
@@ -753,10 +755,13 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
                 const int chunk = gt / tiles_here, t = gt - chunk * tiles_here;
                 if (t == 0) {
                     __syncthreads();  // every wavefront holds the previous chunk's fragments in registers, or is done with them
+                    if (chunk == 0) TRACE(2);
                     stage_chunk(chunk);
+                    if (chunk == 0) TRACE(3);
                     __syncthreads();
                     load_columns(chunk);
                     if (nchunks == 1) __syncthreads();  // the cells below overwrite the staged activations
+                    if (chunk == 0) TRACE(4);
                 }
                 float res[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -772,7 +777,9 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
             }
         }
     }
+    TRACE(5);
     __syncthreads();
+    TRACE(6);
     // ---- add the eight wavefronts' partials in order and store: thread tid < 256 owns D[4 q' + r][n'] with
     // (n', q') = lane id tid % 64 and r = tid / 64, for every tile
     if (tid < 256) {
@@ -792,6 +799,7 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
             }
         }
     }
+    TRACE(7);
 }
 
 // Formats whose kernel is also built with several slot sets per pass (up to 16 bf16 rows).
