@@ -45,15 +45,17 @@ def test_gemm_fp32_activations_take_the_exact_path(O, tfq, gpu):
     W.close()
 
 
+@pytest.mark.parametrize("fmt", ["B32S4", "Q_G_4"])
 @pytest.mark.parametrize("N,K", [(14336, 4096), (4096, 14336)])
-def test_config3_prefill_shapes(tfq, gpu, N, K):
+def test_config3_prefill_shapes(tfq, gpu, N, K, fmt):
     """M = 2048 tokens, bf16 activations N(0,1), 4-bit block-32 weights from N(0, 0.02), bf16 output:
     against a dense fp32 torch matmul of the decoded matrix."""
     import torch
     M = 2048
     g = torch.Generator(device="cuda").manual_seed(3)
     w = torch.randn(N * K, device=gpu, generator=g) * 0.02
-    W = tfq.Weight("B32S4", N, K, tfq.encode("B32S4", w))
+    print(f"prefill {fmt} M={M} N={N} K={K}", flush=True)
+    W = tfq.Weight(fmt, N, K, tfq.encode(fmt, w))
     del w
     x = torch.randn(M, K, device=gpu, generator=g).bfloat16()
     y = W.gemm(x, out_dtype=torch.bfloat16)

@@ -3,23 +3,28 @@
 // Replaces Qwen35Engine::gemm on the prefill path, which the reference runs in
 // chunks of 512 rows (src/adapters/tools/qwen35_engine.cpp:54-101, :681-686).
 //
-// A workgroup of 8 wavefronts owns a 256 x 256 output tile and walks K in steps
-// of 32 (one scale group per weight row).  Per step it
-//   * copies the 256 x 32 activation tile to LDS (bf16),
-//   * decodes the 256 x 32 weight tile: one lane takes two code dwords (8 weights each),
+// A workgroup of 8 wavefronts owns an output tile of 256 tokens x 256, 224 or 128 weight rows and walks K in
+// steps of 32 (one scale group per weight row).  Per step it
+//   * copies the 256 x 32 activation tile to LDS (bf16), global -> LDS without passing registers,
+//   * decodes the weight tile: one lane takes one or two code dwords (8 weights each),
 //     converts the nibbles with v_cvt_f32_ubyte, applies the group's scale and
 //     offset in fp32
 //         w = a * n + c,   (a, c) = (d, -8d) or (d*sc/15, -dm*mc)
 //     packs to bf16 (v_cvt_pk_bf16_f32) and stores the 8 weights to LDS,
-//   * runs 32 v_mfma_f32_16x16x32_bf16 per wavefront (a 128 x 64 sub-tile: LDS reads per MFMA
-//     are what bounds this kernel, and they shrink with the sub-tile's size).
-// Global loads run three steps ahead of their use in a ring of four register
-// sets (a step's loads have two full steps to arrive before they are written
-// to LDS), so HBM / L2 latency overlaps with arithmetic.  Weights are read from the
+//   * runs 32, 28 or 16 v_mfma_f32_16x16x32_bf16 per wavefront (sub-tiles of 128 x 64, 64 x 112, 64 x 64:
+//     LDS reads per MFMA are what bounds this kernel, and they shrink with the sub-tile's size).
+// Global loads are issued three steps ahead of the step that multiplies their data, into four LDS buffers
+// (activations) and a ring of four register sets (code dwords), and are waited for by exact counts, so
+// HBM / L2 latency overlaps with arithmetic.  Weights are read from the
 // Tiled16 layout, where the 16 rows of a tile hold a group as 256 contiguous bytes.
 // Workgroups are numbered so that the ones running together on an XCD share a
 // token tile: the activations, the larger operand by bytes, are then served from
 // that XCD's L2 and only the packed weights stream from HBM.
+// The matrix pipeline takes an MFMA every 16 cycles only while at most two other vector instructions are
+// issued per MFMA; two wavefronts per SIMD (512 threads) let one wavefront's decode and LDS traffic fill
+// the other's MFMA shadow without any hand scheduling.
+
+#include <algorithm>
 
 #include "tfq_internal.hpp"
 
@@ -32,8 +37,9 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 
-constexpr int BM = 256, BK = 32, THREADS = 512;  // the weight-strip width BN (256 or 128) is a template parameter
+constexpr int BM = 256, BK = 32;  // the weight-strip width BN (256, 224 or 128) and the workgroup size are template parameters
 
 __device__ __forceinline__ uint32_t bf16_rne(float f) {
     const uint32_t u = __float_as_uint(f);
@@ -93,14 +99,21 @@ __device__ __forceinline__ void group_coeffs(uint4 h, int g, float& a, float& c)
     }
 }
 
-template <int FMT, int BN>
-__global__ __launch_bounds__(THREADS) void gemm4_kernel(GemmArgs args) {
-    constexpr int WROWS = BN / 128;      // weight rows decoded per thread and step
-    constexpr int MI = BN == 256 ? 8 : 4;  // 16-row token fragments per wavefront: sub-tile 128 x 64 or 64 x 64
+template <int FMT, int BN, int NT>
+__global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
+    constexpr int XL = BM * 4 / NT;     // activation copies per thread and step (rows NT / 4 apart)
+    constexpr int BNA = BN > 128 ? 256 : 128;  // rows of the strip's LDS buffers and of the decode (224: the last 32 are spare)
+    constexpr int WROWS = BNA * 4 / NT;        // weight rows decoded per thread and step (rows NT / 4 apart)
+    constexpr int RSTRIDE = NT / 4;
+    // wavefront grid over the output tile and 16 x 16 fragments per wavefront:
+    //   BN 256: 2 x 4 wavefronts of 128 x 64;  BN 224: 4 x 2 of 64 x 112;  BN 128: 4 x 2 of 64 x 64
+    constexpr int WAVES_N = BN == 256 ? 4 : 2;
+    constexpr int WAVES_M = NT / 64 / WAVES_N;
+    constexpr int MI = BM / WAVES_M / 16, NJ = BN / WAVES_N / 16;
     // activations: four buffers of a 256 x 32 bf16 step (copied three steps ahead); weights: two buffers
     extern __shared__ uint4 smem[];
     uint4* const xs = smem;                 // [4][BM * 4]
-    uint4* const wsm = smem + 4 * BM * 4;   // [2][BN * 4]
+    uint4* const wsm = smem + 4 * BM * 4;   // [2][BNA * 4]
     const int M = args.M, N = args.N, K = args.K;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // workgroup -> (token tile, weight strip).  Workgroups are dealt to the 8 XCDs round robin, and the
@@ -119,106 +132,145 @@ __global__ __launch_bounds__(THREADS) void gemm4_kernel(GemmArgs args) {
     const int nblocks = K >> 8;
     const int ntiles16 = (N + 15) >> 4;
 
-    // ---- global -> register stage of one k-step
-    // activations: thread handles (row, 16-byte segment) pairs idx = tid and tid + 512
+    // ---- global -> LDS / register stage of one k-step
+    // A thread handles (row, 16-byte segment) pairs of the activation tile, rows RSTRIDE apart, and the
+    // code dword of the same (row, segment) of the weight strip.
     // LDS tiles are stored as [row / 8][16-byte segment][row % 8]: the 8 lanes that an LDS access
     // serves together (consecutive rows, same segment) then touch 128 consecutive bytes, all banks
     // once; with plain [row][segment] rows 64 bytes apart they would share banks four ways.
-    // Threads are matched to (row, segment) so that their writes follow the same rule.
+    // Threads are matched to (row, segment) so that their writes follow the same rule (slot = tid).
     auto lds_index = [](int row, int seg) { return ((row >> 3) << 5) + (seg << 3) + (row & 7); };
     const int xr0 = (tid & 7) + ((tid >> 5) << 3), xseg = (tid >> 3) & 3;
-    const unsigned short* xp0 = args.X + (size_t)min(m0 + xr0, M - 1) * K + xseg * 8;
-    const unsigned short* xp1 = args.X + (size_t)min(m0 + xr0 + 128, M - 1) * K + xseg * 8;
-    // weights: thread handles code dword j of rows wr and wr + 128 of the strip (same row inside their 16-row tiles)
     const int wr = xr0, wj = xseg;
-    const int wn = (n0 + wr) & 15;
-    const uint8_t* wbase0 = args.W + (size_t)min((n0 + wr) >> 4, ntiles16 - 1) * nblocks * 2304;
-    const uint8_t* wbase1 = args.W + (size_t)min((n0 + wr + (WROWS - 1) * 128) >> 4, ntiles16 - 1) * nblocks * 2304;
+    const int wn = (n0 + wr) & 15;  // RSTRIDE is a multiple of 16: the same row of a 16-row tile for all of a thread's rows
+    // Addresses are a scalar base (advanced per step / per block) plus a 32-bit offset per thread
+    // (the host side keeps both operands below 4 GiB).
+    uint32_t xoff[XL], woff[WROWS];
+#pragma unroll
+    for (int i = 0; i < XL; ++i) xoff[i] = (uint32_t)(((size_t)min(m0 + xr0 + i * RSTRIDE, M - 1) * K + xseg * 8) * 2);
+#pragma unroll
+    for (int i = 0; i < WROWS; ++i)
+        woff[i] = (uint32_t)((size_t)min((n0 + wr + i * RSTRIDE) >> 4, ntiles16 - 1) * nblocks * 2304 + 16 * wn + 4 * wj);
 
-    // ring of four register sets: set r holds the loads of a step with ks % 4 == r
-    uint32_t rw0[4], rw1[4];
-    uint4 hdr0 = {0, 0, 0, 0}, hdr1 = {0, 0, 0, 0}, hnext0 = {0, 0, 0, 0}, hnext1 = {0, 0, 0, 0};
+    // Every global load of the loop is written as an instruction and waited for by hand.  The copies
+    // of the activations go global -> LDS without passing registers (global_load_lds); the compiler
+    // cannot tell them from the LDS reads of the current step and would make each read wait for
+    // copies that are in flight on purpose.  Once they are outside its count, the weight loads must be
+    // too: it would wait for them with counts that leave the copies out, which are therefore too
+    // strict and, where it has moved a load, drain the whole queue in the middle of the loop.
+    // Loads return in the order of issue; step s issues, in this order, its XL copies, WROWS code
+    // dwords and (when it starts a block) WROWS headers for step s + 3.  A register that a load is
+    // still writing is named by no instruction until the wait that covers it.
+    uint32_t rw[WROWS][4];  // ring of four: set r holds the code dwords of a step with ks % 4 == r
+    u32x4_t hnext[WROWS];
+    uint4 hdr[WROWS];
     const int nsteps = K / BK;
-    // The activation copies go global -> LDS without passing registers (global_load_lds); they are
-    // written as instructions so that the compiler does not count them: it would make every LDS
-    // read wait for copies that are in flight on purpose.  They are waited for by hand (below).
     const uint32_t lds_x = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)xs;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const uint8_t* const xbytes = reinterpret_cast<const uint8_t*>(args.X);
     auto copy_x = [&](int ks_) __attribute__((always_inline)) {
         const int ks = min(ks_, nsteps - 1);  // past the end: the last step again, no branch
-        const uint32_t dst = lds_x + (uint32_t)(((ks_ & 3) * BM * 4 + 64 * wave_u) * 16);
-        const unsigned short* s0 = xp0 + (size_t)ks * BK;
-        const unsigned short* s1 = xp1 + (size_t)ks * BK;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(s0) : "memory");
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst + 512 * 16), "v"(s1) : "memory");
-    };
-    // g = ks % 8 is passed separately: a compile-time constant where the loop is unrolled over a block
-    auto load_step = [&](int ks_, int g, uint32_t& w0, uint32_t& w1) __attribute__((always_inline)) {  // ks = K offset / 32
-        const int ks = min(ks_, nsteps - 8 + g);  // past the end: the last block again, no branch
-        const int blk = ks >> 3;
-        const size_t off = (size_t)blk * 2304;
-        const int coff = (g >> 2) * 1024 + (wn + 16 * (g & 3)) * 16 + 4 * wj;
-        w0 = *reinterpret_cast<const uint32_t*>(wbase0 + off + coff);
-        if constexpr (WROWS == 2) w1 = *reinterpret_cast<const uint32_t*>(wbase1 + off + coff);
-        if (g == 0) {
-            hnext0 = *reinterpret_cast<const uint4*>(wbase0 + off + 2048 + 16 * wn);
-            if constexpr (WROWS == 2) hnext1 = *reinterpret_cast<const uint4*>(wbase1 + off + 2048 + 16 * wn);
+        const uint8_t* base = xbytes + (size_t)ks * (BK * 2);
+#pragma unroll
+        for (int i = 0; i < XL; ++i) {
+            const uint32_t dst = lds_x + (uint32_t)(((ks_ & 3) * BM * 4 + 64 * wave_u + i * NT) * 16);
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[i]), "s"(base) : "memory");
         }
     };
-    auto store_step = [&](int buf, int g, uint32_t w0, uint32_t w1) __attribute__((always_inline)) {
-        if (g == 0) { hdr0 = hnext0; hdr1 = hnext1; }
-        float a, c;
-        group_coeffs<FMT>(hdr0, g, a, c);
-        wsm[buf * BN * 4 + lds_index(wr, wj)] = decode8(w0, a, c);
-        if constexpr (WROWS == 2) {
-            group_coeffs<FMT>(hdr1, g, a, c);
-            wsm[buf * BN * 4 + lds_index(wr + 128, wj)] = decode8(w1, a, c);
+    // code dword of group G (static) of the block at `base` (W + 2304 * block); G == 0 also fetches the
+    // block's headers
+    auto load_step = [&]<int G, int R>(const uint8_t* base) __attribute__((always_inline)) {
+        constexpr int OFF = (G >> 2) * 1024 + (G & 3) * 256;
+#pragma unroll
+        for (int i = 0; i < WROWS; ++i) {
+            uint32_t& w = rw[i][R];
+            asm volatile("global_load_dword %0, %1, %2 offset:%3" : "=v"(w) : "v"(woff[i]), "s"(base), "n"(OFF) : "memory");
+        }
+        if constexpr (G == 0) {
+#pragma unroll
+            for (int i = 0; i < WROWS; ++i) {
+                u32x4_t& h = hnext[i];
+                const uint32_t ho = woff[i] - 4 * wj;
+                asm volatile("global_load_dwordx4 %0, %1, %2 offset:2048" : "=v"(h) : "v"(ho), "s"(base) : "memory");
+            }
+        }
+    };
+    // wait until at most PENDING loads are outstanding; the registers named become readable by it
+    // (naming them keeps their readers behind the wait)
+    auto arrive = [&]<int PENDING, int R, bool HDR>() __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PENDING));
+#pragma unroll
+        for (int i = 0; i < WROWS; ++i) {
+            uint32_t& w = rw[i][R];
+            asm volatile("" : "+v"(w));
+            if constexpr (HDR) {
+                u32x4_t& h = hnext[i];
+                asm volatile("" : "+v"(h));
+            }
+        }
+    };
+    auto store_step = [&]<int G, int R>(int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < WROWS; ++i) {
+            if constexpr (G == 0) hdr[i] = uint4{hnext[i][0], hnext[i][1], hnext[i][2], hnext[i][3]};
+            float a, c;
+            group_coeffs<FMT>(hdr[i], G, a, c);
+            wsm[buf * BNA * 4 + lds_index(wr + i * RSTRIDE, wj)] = decode8(rw[i][R], a, c);
         }
     };
 
-    // wavefront sub-tile: 2 (M) x 4 (N) wavefronts of 128 x 64, or 4 x 2 wavefronts of 64 x 64
-    const int wm = BN == 256 ? wave >> 2 : wave >> 1, wn_ = BN == 256 ? wave & 3 : wave & 1;
+    const int wm = wave / WAVES_N, wn_ = wave % WAVES_N;
     const int fr = lane & 15, fk = lane >> 4;
-    f32x4_t acc[MI][4];
+    f32x4_t acc[MI][NJ];
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int j = 0; j < NJ; ++j) acc[i][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    copy_x(0); load_step(0, 0, rw0[0], rw1[0]);
-    copy_x(1); load_step(1, 1, rw0[1], rw1[1]);
-    copy_x(2); load_step(2, 2, rw0[2], rw1[2]);
-    store_step(0, 0, rw0[0], rw1[0]);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    copy_x(0); load_step.template operator()<0, 0>(args.W);
+    copy_x(1); load_step.template operator()<1, 1>(args.W);
+    copy_x(2); load_step.template operator()<2, 2>(args.W);
+    arrive.template operator()<0, 0, true>();
+    store_step.template operator()<0, 0>(0);
     __syncthreads();
-    // The affine format's header fields are cheapest to extract at a static group index, so its loop
-    // is unrolled over a whole 256-wide block; the symmetric one keeps the shorter body.
-    constexpr int UNR = FMT == TFQ_Q_G_4 ? 8 : 4;
-    for (int ks0 = 0; ks0 < nsteps; ks0 += UNR) {
+    // One trip of the loop is a 256-wide block (eight steps), so a step's group index is static.
+    // Step U consumes the code dwords of step U + 1 (issued two steps earlier); behind them in the queue
+    // are the loads issued by the previous step and by this one.
+    auto step = [&]<int U>(int ks0, const uint8_t* cur, const uint8_t* nxt) __attribute__((always_inline)) {
+        const int ks = ks0 + U, buf = U & 1;
+        constexpr int PER_STEP = XL + WROWS;
+        constexpr int PENDING = 2 * PER_STEP + WROWS * (((U + 2) & 7) == 0) + WROWS * (((U + 3) & 7) == 0);
+        // buffer (ks + 3) % 4 was read during step ks - 1, which every wavefront has left
+        copy_x(ks + 3);
+        load_step.template operator()<(U + 3) & 7, (U + 3) & 3>(U + 3 < 8 ? cur : nxt);
+        uint4 af[MI], bfr[NJ];
 #pragma unroll
-        for (int u = 0; u < UNR; ++u) {
-            const int ks = ks0 + u, buf = u & 1;
-            const int gbase = UNR == 8 ? 0 : (ks0 & 4);
-            // buffer (ks + 3) % 4 was read during step ks - 1, which every wavefront has left
-            copy_x(ks + 3);
-            load_step(ks + 3, (gbase + u + 3) & 7, rw0[(u + 3) & 3], rw1[(u + 3) & 3]);
-            uint4 af[MI], bfr[4];
+        for (int j = 0; j < NJ; ++j) bfr[j] = wsm[buf * BNA * 4 + lds_index(wn_ * (NJ * 16) + j * 16 + fr, fk)];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) bfr[j] = wsm[buf * BN * 4 + lds_index(wn_ * 64 + j * 16 + fr, fk)];
+        for (int i = 0; i < MI; ++i) af[i] = xs[(U & 3) * BM * 4 + lds_index(wm * (MI * 16) + i * 16 + fr, fk)];
 #pragma unroll
-            for (int i = 0; i < MI; ++i) af[i] = xs[(u & 3) * BM * 4 + lds_index(wm * (MI * 16) + i * 16 + fr, fk)];
+        for (int i = 0; i < MI; ++i)
 #pragma unroll
-            for (int i = 0; i < MI; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[i]),
-                                                                        __builtin_bit_cast(bf16x8_t, bfr[j]), acc[i][j], 0, 0, 0);
-            store_step(buf ^ 1, (gbase + u + 1) & 7, rw0[(u + 1) & 3], rw1[(u + 1) & 3]);  // past the end: written, never read
-            // step ks + 1's activation copies were issued two steps ago; behind them at least the
-            // 2 + 4 + 4 = 10 loads of this and the previous step have been issued, 8 is a safe bound
-            asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-            __syncthreads();
-        }
+            for (int j = 0; j < NJ; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[i]),
+                                                                    __builtin_bit_cast(bf16x8_t, bfr[j]), acc[i][j], 0, 0, 0);
+        // the activation copies of step ks + 1 were issued before its code dwords: they have landed too
+        arrive.template operator()<PENDING, (U + 1) & 3, ((U + 1) & 7) == 0>();
+        store_step.template operator()<(U + 1) & 7, (U + 1) & 3>(buf ^ 1);  // past the end: written, never read
+        __syncthreads();
+    };
+    for (int ks0 = 0; ks0 < nsteps; ks0 += 8) {
+        const int blk = ks0 >> 3;
+        const uint8_t* cur = args.W + (size_t)blk * 2304;
+        const uint8_t* nxt = args.W + (size_t)min(blk + 1, nblocks - 1) * 2304;  // past the end: the last block again
+        step.template operator()<0>(ks0, cur, nxt);
+        step.template operator()<1>(ks0, cur, nxt);
+        step.template operator()<2>(ks0, cur, nxt);
+        step.template operator()<3>(ks0, cur, nxt);
+        step.template operator()<4>(ks0, cur, nxt);
+        step.template operator()<5>(ks0, cur, nxt);
+        step.template operator()<6>(ks0, cur, nxt);
+        step.template operator()<7>(ks0, cur, nxt);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may land in LDS after the workgroup is gone
 
@@ -226,8 +278,8 @@ __global__ __launch_bounds__(THREADS) void gemm4_kernel(GemmArgs args) {
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int col = n0 + wn_ * 64 + j * 16 + fr;
+        for (int j = 0; j < NJ; ++j) {
+            const int col = n0 + wn_ * (NJ * 16) + j * 16 + fr;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int row = m0 + wm * (MI * 16) + i * 16 + 4 * fk + r;
@@ -240,37 +292,54 @@ __global__ __launch_bounds__(THREADS) void gemm4_kernel(GemmArgs args) {
         }
 }
 
-template <int FMT, int BN>
+template <int FMT, int BN, int NT>
 int run_tiles(GemmArgs a, hipStream_t s) {
     a.tiles_n = (a.N + BN - 1) / BN;
     const int grid = 8 * ((a.tiles_m * a.tiles_n + 7) / 8);
-    constexpr size_t lds = (size_t)(4 * BM * 4 + 2 * BN * 4) * 16;  // 96 KB or 80 KB
+    constexpr size_t lds = (size_t)(4 * BM * 4 + 2 * (BN > 128 ? 256 : 128) * 4) * 16;  // 96 KB or 80 KB
     static bool lds_limit_raised = false;  // once: not allowed while a stream is being captured
     if (!lds_limit_raised) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm4_kernel<FMT, BN>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm4_kernel<FMT, BN, NT>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
         lds_limit_raised = true;
     }
-    hipLaunchKernelGGL((gemm4_kernel<FMT, BN>), dim3(grid), dim3(THREADS), lds, s, a);
+    hipLaunchKernelGGL((gemm4_kernel<FMT, BN, NT>), dim3(grid), dim3(NT), lds, s, a);
     return hip_fail(hipGetLastError(), "gemm launch");
 }
 
 template <int FMT>
 int run(const tfq_weight* w, const void* x, int M, void* y, int yd, hipStream_t s) {
-    GemmArgs a{};
-    a.W = w->dev;
-    a.X = (const unsigned short*)x;
-    a.Y = y;
-    a.M = M;
-    a.N = (int)w->N;
-    a.K = (int)w->K;
-    a.y_bf16 = yd == TFQ_BF16;
-    a.tiles_m = (M + BM - 1) / BM;
-    // 256-wide weight strips read LDS less per MFMA; they are used when they still give every
-    // compute unit a workgroup, otherwise the 128-wide ones double the number of workgroups
-    const int wide = a.tiles_m * ((a.N + 255) / 256);
-    return wide >= 256 ? run_tiles<FMT, 256>(a, s) : run_tiles<FMT, 128>(a, s);
+    // the kernel addresses X with 32-bit byte offsets: tall inputs go through in slices of whole tiles
+    const size_t row_bytes = (size_t)w->K * 2;
+    const int max_rows = (int)std::min<size_t>(((size_t)0xFFFFF000u / row_bytes) & ~(size_t)511, (size_t)1 << 30);
+    if (max_rows < 512) return fail(TFQ_ERR_SHAPE, "gemm: rows too long");
+    const size_t ye = yd == TFQ_BF16 ? 2 : 4;
+    for (int mb = 0; mb < M; mb += max_rows) {
+        GemmArgs a{};
+        a.W = w->dev;
+        a.X = (const unsigned short*)x + (size_t)mb * w->K;
+        a.Y = (uint8_t*)y + (size_t)mb * w->N * ye;
+        a.M = std::min(M - mb, max_rows);
+        a.N = (int)w->N;
+        a.K = (int)w->K;
+        a.y_bf16 = yd == TFQ_BF16;
+        a.tiles_m = (a.M + BM - 1) / BM;
+        // The strip width decides how many workgroups there are and how much LDS traffic an MFMA costs
+        // (wider is cheaper).  Workgroups run in rounds of one per compute unit, so the cost of a width is
+        // rounds x width, weighted by what a tile of that shape reaches; 224 (= 14 tiles of 16 rows) is there
+        // because it turns 1.75 rounds of 256-wide strips into two full ones at 14336 rows.
+        const auto cost = [&](int bn, double eff) {
+            const long tiles = (long)a.tiles_m * ((a.N + bn - 1) / bn);
+            return (double)((tiles + 255) / 256) * bn / eff;
+        };
+        const double c256 = cost(256, 1.0), c224 = cost(224, 0.97), c128 = cost(128, 0.8);
+        const int rc = c256 <= c224 && c256 <= c128 ? run_tiles<FMT, 256, 512>(a, s)
+                       : c224 <= c128               ? run_tiles<FMT, 224, 512>(a, s)
+                                                    : run_tiles<FMT, 128, 512>(a, s);
+        if (rc) return rc;
+    }
+    return TFQ_OK;
 }
 
 }  // namespace
@@ -278,7 +347,7 @@ int run(const tfq_weight* w, const void* x, int M, void* y, int yd, hipStream_t 
 int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype, hipStream_t s) {
     const bool mfma_path = w->layout == TFQ_LAYOUT_TILED16 && tiled_unit_bytes(w->fmt) == 2304 && x_dtype == TFQ_BF16 && M > 16;
     if (mfma_path) {
-        if (w->N > 0x7FFFFFF0 || w->K > 0x7FFFFFF0) return fail(TFQ_ERR_SHAPE, "gemm: shape too large");
+        if (w->N > 0x7FFFFFF0 || w->K > 0x7FFFFFF0 || w->dev_bytes >= 0xFFFFF000ull) return fail(TFQ_ERR_SHAPE, "gemm: matrix too large");
         switch (canonical(w->fmt)) {
             case TFQ_Q_G_4: return run<TFQ_Q_G_4>(w, x, M, y, y_dtype, s);
             case TFQ_B32S4: return run<TFQ_B32S4>(w, x, M, y, y_dtype, s);

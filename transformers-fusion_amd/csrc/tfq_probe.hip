@@ -6,6 +6,9 @@
 //            non-temporal hint, on 66 MB, 264 MB and 1 GB
 //   barrier  a grid-wide barrier over 256 resident workgroups (device-scope atomic counter, fences,
 //            spin bounded at 2^20 polls so that the kernel ends whatever happens)
+//   mfma     issue rate of v_mfma_f32_16x16x32_bf16 with 0, 2 or 4 independent vector instructions behind
+//            every MFMA, one and two wavefronts per SIMD: what a dequantising GEMM may spend on decode
+//            and LDS traffic per MFMA before the matrix pipeline starves
 // Not part of the library: built beside it, run by `python bench.py --probe`.
 #include <hip/hip_runtime.h>
 
@@ -88,6 +91,33 @@ __global__ __launch_bounds__(1024) void barrier_kernel(unsigned* counter, unsign
     if (passed == 0xFFFFFFFFu) sink[0] = passed;
 }
 
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+// 16 independent accumulators updated in place, VPER independent FMAs after every MFMA
+template <int VPER>
+__global__ __launch_bounds__(512) void mfma_issue_kernel(float* out, int iters) {
+    f32x4_t acc[16];
+    for (int i = 0; i < 16; ++i) acc[i] = f32x4_t{0, 0, 0, 0};
+    const u32x4_t a = {threadIdx.x, 1, 2, 3}, b = {4, 5, 6, threadIdx.x};
+    float v0 = (float)threadIdx.x, v1 = 1.0f;
+    const float v2 = 2.0f, v3 = 0.5f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i]) : "v"(a), "v"(b));
+#pragma unroll
+            for (int v = 0; v < VPER; ++v) {
+                if (v & 1) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(v0) : "v"(v2), "v"(v3));
+                else asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(v1) : "v"(v2), "v"(v3));
+            }
+        }
+    }
+    asm volatile("s_nop 15\n\ts_nop 15");
+    float sum = v0 + v1;
+    for (int i = 0; i < 16; ++i) sum += acc[i][0];
+    if (sum == 12345.0f) out[threadIdx.x] = sum;
+}
+
 int main() {
     unsigned *sink, *counter, *err;
     CK(hipMalloc(&sink, 4)); CK(hipMalloc(&counter, 4)); CK(hipMalloc(&err, 4));
@@ -135,6 +165,29 @@ int main() {
             std::printf("stream  %7.1f MB, %s loads: %8.2f us  %7.1f GB/s\n", bytes / 1e6, nt ? "non-temporal" : "plain       ", us, bytes / us / 1e3);
         }
         for (auto b : bufs) CK(hipFree(b));
+    }
+
+    // mfma: 256 workgroups of 4 or 8 wavefronts, 64000 MFMAs per wavefront
+    {
+        float* out = nullptr;
+        CK(hipMalloc(&out, 4096));
+        const int iters = 4000;
+        auto time_mfma = [&](auto kernel, int threads, int vper) {
+            hipLaunchKernelGGL(kernel, dim3(256), dim3(threads), 0, s, out, iters);
+            CK(hipEventRecord(e0, s));
+            hipLaunchKernelGGL(kernel, dim3(256), dim3(threads), 0, s, out, iters);
+            CK(hipEventRecord(e1, s)); CK(hipEventSynchronize(e1));
+            const double us = elapsed_us(), n = 16.0 * iters;
+            std::printf("mfma    %d wavefront(s) per SIMD, %d vector instructions per MFMA: %5.2f ns per MFMA and SIMD, %6.0f TFLOP/s\n",
+                        threads / 256, vper, us * 1e3 / n / (threads / 256), n * 16384.0 * (threads / 64) * 256 / us / 1e6);
+        };
+        for (int threads : {256, 512}) {
+            time_mfma(mfma_issue_kernel<0>, threads, 0);
+            time_mfma(mfma_issue_kernel<2>, threads, 2);
+            time_mfma(mfma_issue_kernel<3>, threads, 3);
+            time_mfma(mfma_issue_kernel<4>, threads, 4);
+        }
+        CK(hipFree(out));
     }
 
     // barrier: only if 256 workgroups of this kernel are resident together
