@@ -11,7 +11,7 @@ def rel_err(y, ref):
     return float(np.abs(y.astype(np.float64) - ref).max() / np.abs(ref).max())
 
 
-@pytest.mark.parametrize("fmt", ["Q_G_4", "B32S4"])
+@pytest.mark.parametrize("fmt", ["Q_G_4", "B32S4", "Q_G_3", "B32S8", "Q_G_8", "Q_8"])
 @pytest.mark.parametrize("M,N,K", [(17, 48, 256), (64, 128, 512), (300, 200, 1024), (512, 33, 2304), (256, 384, 4096)])
 def test_gemm_against_oracle(O, tfq, gpu, fmt, M, N, K):
     import torch
@@ -45,11 +45,12 @@ def test_gemm_fp32_activations_take_the_exact_path(O, tfq, gpu):
     W.close()
 
 
-@pytest.mark.parametrize("fmt", ["B32S4", "Q_G_4"])
+@pytest.mark.parametrize("fmt", ["B32S4", "Q_G_4", "Q_G_3", "B32S8", "Q_G_8"])
 @pytest.mark.parametrize("N,K", [(14336, 4096), (4096, 14336)])
 def test_config3_prefill_shapes(tfq, gpu, N, K, fmt):
-    """M = 2048 tokens, bf16 activations N(0,1), 4-bit block-32 weights from N(0, 0.02), bf16 output:
-    against a dense fp32 torch matmul of the decoded matrix."""
+    """M = 2048 tokens, bf16 activations N(0,1), block-32 weights from N(0, 0.02), bf16 output:
+    against a dense fp32 torch matmul of the decoded matrix (for the companded 8-bit grid that also
+    checks the line that stands for the grid in the matmul against the exact table of the decode)."""
     import torch
     M = 2048
     g = torch.Generator(device="cuda").manual_seed(3)

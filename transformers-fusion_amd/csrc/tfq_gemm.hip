@@ -1,4 +1,5 @@
-// Dequant-fused prefill GEMM:  Y[m][n] = sum_k X[m][k] * W[n][k]  for tall X
+// Dequant-fused prefill GEMM:  Y[m][n] = sum_k X[m][k] * W[n][k]  for tall X and the formats with
+// eight scale groups of 32 per block (Q_G_4, Q_G_3, B32S4; B32S8, Q_G_8, Q_8 as two nibble planes)
 // (M > 16), bf16 activations, fp32 accumulation on the matrix cores.
 // Replaces Qwen35Engine::gemm on the prefill path, which the reference runs in
 // chunks of 512 rows (src/adapters/tools/qwen35_engine.cpp:54-101, :681-686).
@@ -73,6 +74,24 @@ __device__ __forceinline__ uint4 decode8(uint32_t v, float a, float c) {
     return o;
 }
 
+// the same for an 8-bit code kept as two nibble planes (dword `lo`: low nibbles of codes 0..7, `hi`: high
+// nibbles): the planes are merged to bytes first, 6 + 8 + 8 + 4 operations
+__device__ __forceinline__ uint4 decode8x2(uint32_t lo, uint32_t hi, float a, float c) {
+    const uint32_t ev = ((hi & 0x0F0F0F0Fu) << 4) | (lo & 0x0F0F0F0Fu);  // codes 0,2,4,6 as bytes
+    const uint32_t od = (hi & 0xF0F0F0F0u) | ((lo >> 4) & 0x0F0F0F0Fu);  // codes 1,3,5,7
+    uint4 o;
+    o.x = pack_bf16(__builtin_fmaf(a, ubyte_to_float<0>(ev), c), __builtin_fmaf(a, ubyte_to_float<0>(od), c));
+    o.y = pack_bf16(__builtin_fmaf(a, ubyte_to_float<1>(ev), c), __builtin_fmaf(a, ubyte_to_float<1>(od), c));
+    o.z = pack_bf16(__builtin_fmaf(a, ubyte_to_float<2>(ev), c), __builtin_fmaf(a, ubyte_to_float<2>(od), c));
+    o.w = pack_bf16(__builtin_fmaf(a, ubyte_to_float<3>(ev), c), __builtin_fmaf(a, ubyte_to_float<3>(od), c));
+    return o;
+}
+
+// slope of the line that stands for the companded 8-bit grid in a matmul (level j ~ (j - 127.5) * gain,
+// within 7.5e-5 relative of tanh(0.02 t) / tanh(0.02), src/codec/block_codec.cpp:224-237); the decode
+// entry points use the exact table
+constexpr float kComp8Line = 1.0000742443371564f / 127.5f;
+
 struct GemmArgs {
     const uint8_t* W;  // Tiled16
     const unsigned short* X;  // bf16 [M][K]
@@ -85,17 +104,20 @@ struct GemmArgs {
 // (a, c) of group g (0..7) of a block from its 16-byte header: weight = a * code + c
 template <int FMT>
 __device__ __forceinline__ void group_coeffs(uint4 h, int g, float& a, float& c) {
-    if constexpr (FMT == TFQ_Q_G_4) {
+    if constexpr (FMT == TFQ_Q_G_4 || FMT == TFQ_Q_G_3) {
         const uint64_t scs = (uint64_t)h.x | ((uint64_t)(h.y & 0xFFFFu) << 32);
         const uint64_t mcs = (uint64_t)(h.y >> 16) | ((uint64_t)h.z << 16);
         const float sc = (float)(uint32_t)((scs >> (6 * g)) & 63u);
         const float mc = (float)((int)((mcs >> (6 * g)) & 63u) - 32);
-        a = half_fast(h.w & 0xFFFFu) * sc * (1.0f / 15.0f);
+        a = half_fast(h.w & 0xFFFFu) * sc * (FMT == TFQ_Q_G_4 ? 1.0f / 15.0f : 1.0f / 7.0f);
         c = -(half_fast(h.w >> 16) * mc);
     } else {
+        // eight fp16 scales; the code is stored with an offset: 8 (4-bit), 128 (8-bit), 127.5 (companded grid)
         const uint32_t hw[4] = {h.x, h.y, h.z, h.w};
         a = half_fast((hw[g >> 1] >> (16 * (g & 1))) & 0xFFFFu);
-        c = -8.0f * a;
+        if constexpr (FMT == TFQ_B32S4) c = -8.0f * a;
+        else if constexpr (FMT == TFQ_B32S8) c = -128.0f * a;
+        else { a *= kComp8Line; c = -127.5f * a; }
     }
 }
 
@@ -104,6 +126,8 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
     constexpr int XL = BM * 4 / NT;     // activation copies per thread and step (rows NT / 4 apart)
     constexpr int BNA = BN > 128 ? 256 : 128;  // rows of the strip's LDS buffers and of the decode (224: the last 32 are spare)
     constexpr int WROWS = BNA * 4 / NT;        // weight rows decoded per thread and step (rows NT / 4 apart)
+    constexpr int NP = tiled_planes(FMT);      // nibble planes of the codes: 2 for the 8-bit formats
+    constexpr int UB = tiled_unit_bytes(FMT);  // bytes of a unit (16 rows x one block): 2304 or 4352
     constexpr int RSTRIDE = NT / 4;
     // wavefront grid over the output tile and 16 x 16 fragments per wavefront:
     //   BN 256: 2 x 4 wavefronts of 128 x 64;  BN 224: 4 x 2 of 64 x 112;  BN 128: 4 x 2 of 64 x 64
@@ -150,7 +174,7 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
     for (int i = 0; i < XL; ++i) xoff[i] = (uint32_t)(((size_t)min(m0 + xr0 + i * RSTRIDE, M - 1) * K + xseg * 8) * 2);
 #pragma unroll
     for (int i = 0; i < WROWS; ++i)
-        woff[i] = (uint32_t)((size_t)min((n0 + wr + i * RSTRIDE) >> 4, ntiles16 - 1) * nblocks * 2304 + 16 * wn + 4 * wj);
+        woff[i] = (uint32_t)((size_t)min((n0 + wr + i * RSTRIDE) >> 4, ntiles16 - 1) * nblocks * UB + 16 * wn + 4 * wj);
 
     // Every global load of the loop is written as an instruction and waited for by hand.  The copies
     // of the activations go global -> LDS without passing registers (global_load_lds); the compiler
@@ -158,10 +182,10 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
     // copies that are in flight on purpose.  Once they are outside its count, the weight loads must be
     // too: it would wait for them with counts that leave the copies out, which are therefore too
     // strict and, where it has moved a load, drain the whole queue in the middle of the loop.
-    // Loads return in the order of issue; step s issues, in this order, its XL copies, WROWS code
+    // Loads return in the order of issue; step s issues, in this order, its XL copies, WROWS * NP code
     // dwords and (when it starts a block) WROWS headers for step s + 3.  A register that a load is
     // still writing is named by no instruction until the wait that covers it.
-    uint32_t rw[WROWS][4];  // ring of four: set r holds the code dwords of a step with ks % 4 == r
+    uint32_t rw[WROWS][NP][4];  // ring of four: set r holds the code dwords of a step with ks % 4 == r
     u32x4_t hnext[WROWS];
     uint4 hdr[WROWS];
     const int nsteps = K / BK;
@@ -183,14 +207,18 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
         constexpr int OFF = (G >> 2) * 1024 + (G & 3) * 256;
 #pragma unroll
         for (int i = 0; i < WROWS; ++i) {
-            uint32_t& w = rw[i][R];
+            uint32_t& w = rw[i][0][R];
             asm volatile("global_load_dword %0, %1, %2 offset:%3" : "=v"(w) : "v"(woff[i]), "s"(base), "n"(OFF) : "memory");
+            if constexpr (NP == 2) {
+                uint32_t& w2 = rw[i][NP - 1][R];
+                asm volatile("global_load_dword %0, %1, %2 offset:%3" : "=v"(w2) : "v"(woff[i]), "s"(base), "n"(OFF + 2048) : "memory");
+            }
         }
         if constexpr (G == 0) {
 #pragma unroll
             for (int i = 0; i < WROWS; ++i) {
                 u32x4_t& h = hnext[i];
-                const uint32_t ho = woff[i] - 4 * wj;
+                const uint32_t ho = woff[i] - 4 * wj + 2048 * (NP - 1);  // the headers follow the code planes
                 asm volatile("global_load_dwordx4 %0, %1, %2 offset:2048" : "=v"(h) : "v"(ho), "s"(base) : "memory");
             }
         }
@@ -201,8 +229,12 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PENDING));
 #pragma unroll
         for (int i = 0; i < WROWS; ++i) {
-            uint32_t& w = rw[i][R];
+            uint32_t& w = rw[i][0][R];
             asm volatile("" : "+v"(w));
+            if constexpr (NP == 2) {
+                uint32_t& w2 = rw[i][NP - 1][R];
+                asm volatile("" : "+v"(w2));
+            }
             if constexpr (HDR) {
                 u32x4_t& h = hnext[i];
                 asm volatile("" : "+v"(h));
@@ -215,7 +247,8 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
             if constexpr (G == 0) hdr[i] = uint4{hnext[i][0], hnext[i][1], hnext[i][2], hnext[i][3]};
             float a, c;
             group_coeffs<FMT>(hdr[i], G, a, c);
-            wsm[buf * BNA * 4 + lds_index(wr + i * RSTRIDE, wj)] = decode8(rw[i][R], a, c);
+            if constexpr (NP == 1) wsm[buf * BNA * 4 + lds_index(wr + i * RSTRIDE, wj)] = decode8(rw[i][0][R], a, c);
+            else wsm[buf * BNA * 4 + lds_index(wr + i * RSTRIDE, wj)] = decode8x2(rw[i][0][R], rw[i][NP - 1][R], a, c);
         }
     };
 
@@ -238,7 +271,7 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
     // are the loads issued by the previous step and by this one.
     auto step = [&]<int U>(int ks0, const uint8_t* cur, const uint8_t* nxt) __attribute__((always_inline)) {
         const int ks = ks0 + U, buf = U & 1;
-        constexpr int PER_STEP = XL + WROWS;
+        constexpr int PER_STEP = XL + WROWS * NP;
         constexpr int PENDING = 2 * PER_STEP + WROWS * (((U + 2) & 7) == 0) + WROWS * (((U + 3) & 7) == 0);
         // buffer (ks + 3) % 4 was read during step ks - 1, which every wavefront has left
         copy_x(ks + 3);
@@ -261,8 +294,8 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
     };
     for (int ks0 = 0; ks0 < nsteps; ks0 += 8) {
         const int blk = ks0 >> 3;
-        const uint8_t* cur = args.W + (size_t)blk * 2304;
-        const uint8_t* nxt = args.W + (size_t)min(blk + 1, nblocks - 1) * 2304;  // past the end: the last block again
+        const uint8_t* cur = args.W + (size_t)blk * UB;
+        const uint8_t* nxt = args.W + (size_t)min(blk + 1, nblocks - 1) * UB;  // past the end: the last block again
         step.template operator()<0>(ks0, cur, nxt);
         step.template operator()<1>(ks0, cur, nxt);
         step.template operator()<2>(ks0, cur, nxt);
@@ -333,10 +366,17 @@ int run(const tfq_weight* w, const void* x, int M, void* y, int yd, hipStream_t 
             const long tiles = (long)a.tiles_m * ((a.N + bn - 1) / bn);
             return (double)((tiles + 255) / 256) * bn / eff;
         };
-        const double c256 = cost(256, 1.0), c224 = cost(224, 0.97), c128 = cost(128, 0.8);
-        const int rc = c256 <= c224 && c256 <= c128 ? run_tiles<FMT, 256, 512>(a, s)
-                       : c224 <= c128               ? run_tiles<FMT, 224, 512>(a, s)
-                                                    : run_tiles<FMT, 128, 512>(a, s);
+        // (the 8-bit formats hold twice the code registers: no 256-wide kernel for them; the affine formats'
+        // longer decode gains nothing from the 64 x 112 sub-tiles: measured 254-261 us against 251 us)
+        constexpr bool kAffine = FMT == TFQ_Q_G_4 || FMT == TFQ_Q_G_3;
+        const double c256 = tiled_planes(FMT) == 1 ? cost(256, 1.0) : 1e30, c224 = cost(224, kAffine ? 0.86 : 0.97), c128 = cost(128, 0.8);
+        int rc;
+        if (c256 <= c224 && c256 <= c128) {
+            if constexpr (tiled_planes(FMT) == 1) rc = run_tiles<FMT, 256, 512>(a, s);
+            else rc = TFQ_ERR_SHAPE;
+        } else {
+            rc = c224 <= c128 ? run_tiles<FMT, 224, 512>(a, s) : run_tiles<FMT, 128, 512>(a, s);
+        }
         if (rc) return rc;
     }
     return TFQ_OK;
@@ -345,12 +385,16 @@ int run(const tfq_weight* w, const void* x, int M, void* y, int yd, hipStream_t 
 }  // namespace
 
 int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype, hipStream_t s) {
-    const bool mfma_path = w->layout == TFQ_LAYOUT_TILED16 && tiled_unit_bytes(w->fmt) == 2304 && x_dtype == TFQ_BF16 && M > 16;
+    const bool mfma_path = w->layout == TFQ_LAYOUT_TILED16 && tiled_header_bytes(w->fmt) == 16 && x_dtype == TFQ_BF16 && M > 16;
     if (mfma_path) {
         if (w->N > 0x7FFFFFF0 || w->K > 0x7FFFFFF0 || w->dev_bytes >= 0xFFFFF000ull) return fail(TFQ_ERR_SHAPE, "gemm: matrix too large");
         switch (canonical(w->fmt)) {
             case TFQ_Q_G_4: return run<TFQ_Q_G_4>(w, x, M, y, y_dtype, s);
             case TFQ_B32S4: return run<TFQ_B32S4>(w, x, M, y, y_dtype, s);
+            case TFQ_Q_G_3: return run<TFQ_Q_G_3>(w, x, M, y, y_dtype, s);
+            case TFQ_B32S8: return run<TFQ_B32S8>(w, x, M, y, y_dtype, s);
+            case TFQ_Q_G_8: return run<TFQ_Q_G_8>(w, x, M, y, y_dtype, s);
+            case TFQ_Q_8: return run<TFQ_Q_8>(w, x, M, y, y_dtype, s);
             default: break;
         }
     }
