@@ -97,6 +97,30 @@ def test_moe_ffn_skewed_routing(O, tfq, gpu, fmt):
         wl.close()
 
 
+@pytest.mark.parametrize("fmt,xdt,mid_bf16,tol", [("B32S4", "bf16", True, 1e-2), ("Q_G_8", "bf16", True, 1e-2),
+                                                  ("Q_G_4", "f32", False, 1e-3)])
+def test_moe_ffn_many_tokens_per_expert(O, tfq, gpu, fmt, xdt, mid_bf16, tol):
+    """A prefill-sized call: 200 tokens over 4 experts, top-2, so every expert holds far more than 16 rows and
+    the expert products go through the prefill entry (the matrix-core GEMM for bf16 rows)."""
+    import torch
+    E, Ktop, T, D, F = 4, 2, 200, 256, 512
+    gate, up, down, hg, hu, hd = _experts(O, tfq, fmt, E, D, F, 700)
+    logits = O.rng_normal(46, T * E, 1.0).reshape(T, E)
+    _, idx, w = O.softmax_topk(logits, Ktop)
+    assert min((idx == e).sum() for e in range(E)) > 32
+    x = O.rng_normal(47, T * D, 1.0).reshape(T, D)
+    if xdt == "bf16":
+        x = O.bf16_round(x)
+        xt = torch.from_numpy(x).to(gpu).bfloat16()
+    else:
+        xt = torch.from_numpy(x).to(gpu)
+    ref = O.moe_ffn(fmt, hg, hu, hd, D, F, idx, w, x, mid_bf16=mid_bf16)
+    y = tfq.moe_ffn(gate, up, down, idx, w, xt, mid_dtype=torch.bfloat16 if mid_bf16 else torch.float32).cpu().numpy()
+    assert rel_err(y, ref) <= tol
+    for W in gate + up + down:
+        W.close()
+
+
 def test_moe_single_token_equals_plain_mlp(O, tfq, gpu):
     """One token, one expert, weight 1: the MoE path reduces to the SwiGLU MLP step."""
     import torch

@@ -191,7 +191,12 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
 
     // Grouped launches: problems in expert order, an expert's rows cut into chunks of `cap` rows
     // (what one pass of the kernel carries at this K)
-    const bool grouped = P > 0 && gemv_grouped_supported(gate[0]->fmt) && gemv_grouped_supported(down[0]->fmt) &&
+    // With many tokens per expert (a prefill-sized call) every 16-row pass of the decode kernels would read
+    // the expert's weights again: those calls go expert by expert through the prefill GEMM instead.
+    int most_rows = 0;
+    for (int e = 0; e < E; ++e) most_rows = std::max(most_rows, first[e + 1] - first[e]);
+    const bool tall = most_rows > 32;
+    const bool grouped = P > 0 && !tall && gemv_grouped_supported(gate[0]->fmt) && gemv_grouped_supported(down[0]->fmt) &&
                          canonical(gate[0]->fmt) == canonical(up[0]->fmt);
     GemvGroupPlan planA{}, planB{};
     std::vector<const tfq_weight*> wA, wB;
@@ -278,6 +283,11 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
     }
     for (int e = 0; e < E && !grouped; ++e) {
         const int p0 = first[e], nt = first[e + 1] - first[e];
+        if (nt > 16) {  // the prefill entry: matrix cores for bf16 rows, 16-row slices otherwise
+            if (int rc = launch_gemm(gate[e], ws.xe + (size_t)p0 * D * xe_bytes, x_dtype, nt, ws.g + (size_t)p0 * F, TFQ_F32, s)) return rc;
+            if (int rc = launch_gemm(up[e], ws.xe + (size_t)p0 * D * xe_bytes, x_dtype, nt, ws.u + (size_t)p0 * F, TFQ_F32, s)) return rc;
+            continue;
+        }
         for (int b0 = 0; b0 < nt; b0 += 16) {  // the GEMV entry takes up to 16 rows
             const int nb = nt - b0 < 16 ? nt - b0 : 16;
             const tfq_weight* gu[2] = {gate[e], up[e]};
@@ -297,10 +307,9 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
     }
     for (int e = 0; e < E && !grouped; ++e) {
         const int p0 = first[e], nt = first[e + 1] - first[e];
-        for (int b0 = 0; b0 < nt; b0 += 16) {
-            const int nb = nt - b0 < 16 ? nt - b0 : 16;
-            if (int rc = launch_gemv(down[e], ws.h + (size_t)(p0 + b0) * F * he, mid_dtype, nb, ws.o + (size_t)(p0 + b0) * D, TFQ_F32, s)) return rc;
-        }
+        if (nt <= 0) continue;
+        // sixteen rows or fewer take the decode kernels inside
+        if (int rc = launch_gemm(down[e], ws.h + (size_t)p0 * F * he, mid_dtype, nt, ws.o + (size_t)p0 * D, TFQ_F32, s)) return rc;
     }
     if (y_dtype == TFQ_BF16)
         hipLaunchKernelGGL(combine_kernel<true>, dim3((unsigned)((nout + 255) / 256)), dim3(256), 0, s, y, ws.o, d_first, d_pairs, d_w, T, (int)D);
