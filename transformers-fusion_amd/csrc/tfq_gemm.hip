@@ -26,6 +26,7 @@
 // the other's MFMA shadow without any hand scheduling.
 
 #include <algorithm>
+#include <cmath>
 
 #include "tfq_internal.hpp"
 
@@ -384,9 +385,23 @@ int run(const tfq_weight* w, const void* x, int M, void* y, int yd, hipStream_t 
 
 }  // namespace
 
+// Few tokens make few workgroups for the tile kernel (one 256-token tile per 128 weight rows, each walking
+// all of K), while the batched decode kernel reads the matrix once per 16 rows with every compute unit busy.
+// Models of both from measurements on MI355X (us): a 16-row pass costs 2.5 + 3.2 per 4096 of K (activation
+// staging) + bytes / 6.5 TB/s, plus 15 %; the tile kernel 4 + rounds x (K / 32) x 0.44.  Measured crossovers:
+// 72 tokens at 14336x4096, 115 at 4096x4096, 125 at 4096x14336 (4-bit).
+static bool slices_cheaper(const tfq_weight* w, int M) {
+    if (!gemv_rows16_supported(w->fmt)) return false;
+    const double K = (double)w->K;
+    const double t16 = 1.15 * (2.5 + 3.2 * std::ceil(K / 4096.0) + (double)w->dev_bytes / 6.5e6);
+    const double tiles = (double)((M + 255) / 256) * (double)((w->N + 127) / 128);
+    const double t_gemm = 4.0 + std::ceil(tiles / 256.0) * (K / 32.0) * 0.44;
+    return (double)((M + 15) / 16) * t16 < t_gemm;
+}
+
 int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype, hipStream_t s) {
     const bool mfma_path = w->layout == TFQ_LAYOUT_TILED16 && tiled_header_bytes(w->fmt) == 16 && x_dtype == TFQ_BF16 && M > 16;
-    if (mfma_path) {
+    if (mfma_path && !slices_cheaper(w, M)) {
         if (w->N > 0x7FFFFFF0 || w->K > 0x7FFFFFF0 || w->dev_bytes >= 0xFFFFF000ull) return fail(TFQ_ERR_SHAPE, "gemm: matrix too large");
         switch (canonical(w->fmt)) {
             case TFQ_Q_G_4: return run<TFQ_Q_G_4>(w, x, M, y, y_dtype, s);

@@ -1042,6 +1042,14 @@ int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, 
 
 }  // namespace
 
+// formats whose 5..16-row calls take the tile-major batched kernel (one pass over the weights per 16 rows)
+bool gemv_rows16_supported(int fmt) {
+    switch (canonical(fmt)) {
+        case TFQ_Q_G_4: case TFQ_B32S4: case TFQ_B32S8: case TFQ_Q_G_8: case TFQ_Q_8: return true;
+        default: return false;
+    }
+}
+
 bool gemv_grouped_supported(int fmt) {
     switch (canonical(fmt)) {
         case TFQ_Q_G_4: case TFQ_B32S4: case TFQ_B32S8: case TFQ_Q_G_8: return true;

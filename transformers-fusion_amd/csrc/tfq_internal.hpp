@@ -347,6 +347,7 @@ struct GemvGroupPlan {
     size_t lds;
 };
 bool gemv_grouped_supported(int fmt);
+bool gemv_rows16_supported(int fmt);
 int plan_gemv_grouped(int fmt, int K, bool x_f32, const int* nrows, const int* nrows_x, int nprob, GemvGroupPlan* gp);
 size_t gemv_group_entry_bytes();
 void fill_gemv_group(const GemvGroupPlan& gp, const tfq_weight* const* ws, const void* const* xs, void* const* ys,
