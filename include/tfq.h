@@ -208,6 +208,16 @@ int tfq_gemv(const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, 
              tfq_stream_t stream);
 int tfq_gemm(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
              tfq_stream_t stream);
+/* tfq_gemm with scratch memory.  When M rows make fewer output tiles than the GPU has compute units
+ * (a tall K with few weight rows, or a few hundred tokens), the prefill kernel can split K over several
+ * workgroups per tile; the fp32 partial tiles go to `workspace` (device memory) and are added in a fixed
+ * order by a second kernel, so results do not depend on timing.  tfq_gemm_workspace_bytes returns what a
+ * call with these arguments would use (0 when it would not split); a smaller or null workspace is legal
+ * and only limits the split.  Same results as tfq_gemm to the stated tolerance.  The reference has no
+ * counterpart: its gemm (src/adapters/tools/qwen35_engine.cpp:54-101) partitions rows over CPU threads. */
+size_t tfq_gemm_workspace_bytes(const tfq_weight_t* w, int x_dtype, int M);
+int tfq_gemm_ws(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
+                void* workspace, size_t workspace_bytes, tfq_stream_t stream);
 /* Up to four matrices that share K, format and the activation rows in ONE launch:
  * ys[i][b][n] = sum_k x[b][k] * ws[i][n][k].  This is the q/k/v step and the
  * gate/up step of the reference engine, which issue one gemm per matrix on the

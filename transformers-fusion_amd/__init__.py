@@ -70,6 +70,8 @@ def _load():
         "tfq_weight_decode": (i32, [vp, vp, vp]),
         "tfq_gemv": (i32, [vp, vp, i32, i32, vp, i32, vp]),
         "tfq_gemm": (i32, [vp, vp, i32, i32, vp, i32, vp]),
+        "tfq_gemm_workspace_bytes": (sz, [vp, i32, i32]),
+        "tfq_gemm_ws": (i32, [vp, vp, i32, i32, vp, i32, vp, sz, vp]),
         "tfq_gemv_multi": (i32, [vp, i32, vp, i32, i32, vp, i32, vp]),
         "tfq_matmul_host": (i32, [vp, vp, vp, i32]),
         "tfq_mlp_workspace_bytes": (sz, [i32, i64]),
@@ -238,9 +240,21 @@ class Weight:
             return out
         return self._mm(lib().tfq_gemv, x, out_dtype)
 
-    def gemm(self, x, out_dtype=None):
-        """y[M][N] = x[M][K] . W^T for any M (prefill)."""
-        return self._mm(lib().tfq_gemm, x, out_dtype)
+    def gemm(self, x, out_dtype=None, workspace=True):
+        """y[M][N] = x[M][K] . W^T for any M (prefill).  With `workspace` the call goes through tfq_gemm_ws with
+        as much scratch memory as tfq_gemm_workspace_bytes asks for (the K split of the prefill kernel)."""
+        import torch
+        if not workspace:
+            return self._mm(lib().tfq_gemm, x, out_dtype)
+        x = x.contiguous()
+        assert x.is_cuda and x.shape[-1] == self.K
+        M = x.numel() // self.K
+        y = torch.empty((M, self.N), dtype=out_dtype or torch.float32, device=x.device)
+        need = int(lib().tfq_gemm_workspace_bytes(self.handle, _dtype_code(x), M))
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device=x.device)
+        _check(lib().tfq_gemm_ws(self.handle, x.data_ptr(), _dtype_code(x), M, y.data_ptr(), _dtype_code(y),
+                                 ws.data_ptr(), need, _stream()))
+        return y
 
 
 class Container:

@@ -100,6 +100,8 @@ struct GemmArgs {
     int M, N, K;
     int y_bf16;
     int tiles_m, tiles_n;
+    int ksplit;      // workgroups per output tile: each walks K / ksplit and writes an fp32 partial tile
+    float* partial;  // [ksplit][M][N] when ksplit > 1
 };
 
 // (a, c) of group g (0..7) of a block from its 16-byte header: weight = a * code + c
@@ -148,13 +150,18 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
     // the packed weight strips stream from HBM.
     const int wg = blockIdx.x;
     const int xcd = wg & 7, slot = wg >> 3;
-    const int items = args.tiles_m * args.tiles_n;
+    // (with K split over several workgroups per tile, a K range of a token tile counts as a tile of its own)
+    const int S = args.ksplit;
+    const int items = args.tiles_m * args.tiles_n * S;
     const int per_xcd = (items + 7) >> 3;
     const int item = xcd * per_xcd + slot;
     if (item >= items) return;
-    const int tm = item / args.tiles_n, strip = item - tm * args.tiles_n;
+    const int tms = item / args.tiles_n, strip = item - tms * args.tiles_n;
+    const int tm = tms / S;
+    const int split = __builtin_amdgcn_readfirstlane(tms - tm * S);  // integer division runs on the vector unit; these feed scalar bases
     const int m0 = tm * BM, n0 = strip * BN;
-    const int nblocks = K >> 8;
+    const int nblocks = K >> 8;            // blocks of a whole row: the stride between 16-row tiles
+    const int nb_walk = __builtin_amdgcn_readfirstlane(nblocks / S);  // blocks this workgroup walks, from block split * nb_walk
     const int ntiles16 = (N + 15) >> 4;
 
     // ---- global -> LDS / register stage of one k-step
@@ -189,10 +196,11 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
     uint32_t rw[WROWS][NP][4];  // ring of four: set r holds the code dwords of a step with ks % 4 == r
     u32x4_t hnext[WROWS];
     uint4 hdr[WROWS];
-    const int nsteps = K / BK;
+    const int nsteps = nb_walk * 8;
     const uint32_t lds_x = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)xs;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const uint8_t* const xbytes = reinterpret_cast<const uint8_t*>(args.X);
+    const uint8_t* const xbytes = reinterpret_cast<const uint8_t*>(args.X) + (size_t)split * nb_walk * 512;
+    const uint8_t* const wbytes = args.W + (size_t)split * nb_walk * UB;
     auto copy_x = [&](int ks_) __attribute__((always_inline)) {
         const int ks = min(ks_, nsteps - 1);  // past the end: the last step again, no branch
         const uint8_t* base = xbytes + (size_t)ks * (BK * 2);
@@ -261,9 +269,9 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
 #pragma unroll
         for (int j = 0; j < NJ; ++j) acc[i][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    copy_x(0); load_step.template operator()<0, 0>(args.W);
-    copy_x(1); load_step.template operator()<1, 1>(args.W);
-    copy_x(2); load_step.template operator()<2, 2>(args.W);
+    copy_x(0); load_step.template operator()<0, 0>(wbytes);
+    copy_x(1); load_step.template operator()<1, 1>(wbytes);
+    copy_x(2); load_step.template operator()<2, 2>(wbytes);
     arrive.template operator()<0, 0, true>();
     store_step.template operator()<0, 0>(0);
     __syncthreads();
@@ -295,8 +303,8 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
     };
     for (int ks0 = 0; ks0 < nsteps; ks0 += 8) {
         const int blk = ks0 >> 3;
-        const uint8_t* cur = args.W + (size_t)blk * UB;
-        const uint8_t* nxt = args.W + (size_t)min(blk + 1, nblocks - 1) * UB;  // past the end: the last block again
+        const uint8_t* cur = wbytes + (size_t)blk * UB;
+        const uint8_t* nxt = wbytes + (size_t)min(blk + 1, nb_walk - 1) * UB;  // past the end: the last block again
         step.template operator()<0>(ks0, cur, nxt);
         step.template operator()<1>(ks0, cur, nxt);
         step.template operator()<2>(ks0, cur, nxt);
@@ -319,17 +327,28 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
                 const int row = m0 + wm * (MI * 16) + i * 16 + 4 * fk + r;
                 if (row < M && col < N) {
                     const size_t o = (size_t)row * N + col;
-                    if (args.y_bf16) reinterpret_cast<unsigned short*>(args.Y)[o] = (unsigned short)bf16_rne(acc[i][j][r]);
+                    if (S > 1) args.partial[(size_t)split * M * N + o] = acc[i][j][r];
+                    else if (args.y_bf16) reinterpret_cast<unsigned short*>(args.Y)[o] = (unsigned short)bf16_rne(acc[i][j][r]);
                     else reinterpret_cast<float*>(args.Y)[o] = acc[i][j][r];
                 }
             }
         }
 }
 
+// y = sum over the K splits of their partial tiles, in split order
+__global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ partial, void* __restrict__ y, size_t n, int S, int y_bf16) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float v = partial[i];
+    for (int sp = 1; sp < S; ++sp) v += partial[(size_t)sp * n + i];
+    if (y_bf16) reinterpret_cast<unsigned short*>(y)[i] = (unsigned short)bf16_rne(v);
+    else reinterpret_cast<float*>(y)[i] = v;
+}
+
 template <int FMT, int BN, int NT>
 int run_tiles(GemmArgs a, hipStream_t s) {
     a.tiles_n = (a.N + BN - 1) / BN;
-    const int grid = 8 * ((a.tiles_m * a.tiles_n + 7) / 8);
+    const int grid = 8 * ((a.tiles_m * a.tiles_n * a.ksplit + 7) / 8);
     constexpr size_t lds = (size_t)(4 * BM * 4 + 2 * (BN > 128 ? 256 : 128) * 4) * 16;  // 96 KB or 80 KB
     static bool lds_limit_raised = false;  // once: not allowed while a stream is being captured
     if (!lds_limit_raised) {
@@ -339,11 +358,52 @@ int run_tiles(GemmArgs a, hipStream_t s) {
         lds_limit_raised = true;
     }
     hipLaunchKernelGGL((gemm4_kernel<FMT, BN, NT>), dim3(grid), dim3(NT), lds, s, a);
+    if (a.ksplit > 1) {
+        const size_t n = (size_t)a.M * a.N;
+        hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, a.partial, a.Y, n, a.ksplit, a.y_bf16);
+    }
     return hip_fail(hipGetLastError(), "gemm launch");
 }
 
+// What the tile kernel does with M rows and how long it takes by a model of measurements on MI355X.
+//   Strip width: decides how many workgroups there are and how much LDS traffic an MFMA costs (wider is
+//   cheaper); workgroups run in rounds of one per compute unit.  224 (= 14 tiles of 16 rows) is there because
+//   it turns 1.75 rounds of 256-wide strips into two full ones at 14336 rows.  The 8-bit formats hold twice
+//   the code registers (no 256-wide kernel); the affine formats' longer decode gains nothing from the
+//   64 x 112 sub-tiles (254-261 us against 251 us).
+//   K split: when the tiles do not fill the compute units, 2, 4 or 8 workgroups share a tile, each walks a
+//   part of K and writes an fp32 partial to the caller's scratch; a second kernel adds the partials in order.
+//   Time (us): 4 + rounds x steps x (0.98, 0.90, 0.60 us per step of a 256-, 224-, 128-wide strip with every
+//   compute unit busy, less when few are) + the partials' traffic at 5 TB/s.
+struct GemmPlan {
+    int bn, ksplit;
+    double us;
+};
 template <int FMT>
-int run(const tfq_weight* w, const void* x, int M, void* y, int yd, hipStream_t s) {
+GemmPlan plan_tiles(int M, int64_t N, int64_t K, size_t scratch_bytes) {
+    constexpr bool kAffine = FMT == TFQ_Q_G_4 || FMT == TFQ_Q_G_3;
+    constexpr bool kTwoPlanes = tiled_planes(FMT) == 2;
+    const struct { int bn; double step; } cand[3] = {{256, 0.98}, {224, kAffine ? 1.0 : 0.90}, {128, 0.60}};
+    const int tiles_m = (M + BM - 1) / BM, nblocks = (int)(K >> 8);
+    GemmPlan best{128, 1, 1e30};
+    for (const auto& c : cand) {
+        if (c.bn == 256 && kTwoPlanes) continue;
+        const long tiles = (long)tiles_m * (long)((N + c.bn - 1) / c.bn);
+        for (int S = 1; S <= 8; S *= 2) {
+            const double part_bytes = (double)S * (double)M * (double)N * 4.0;
+            if (S > 1 && (tiles * S > 256 || nblocks % S || nblocks / S < 2 || part_bytes > (double)scratch_bytes)) continue;
+            const long wgs = tiles * S;
+            const double occ = wgs >= 256 ? 1.0 : (double)wgs / 256.0;
+            double us = 4.0 + (double)((wgs + 255) / 256) * ((double)K / 32.0 / S) * c.step * (0.65 + 0.35 * occ) * (kTwoPlanes ? 1.1 : 1.0);
+            if (S > 1) us += 3.0 + part_bytes * (1.0 + 1.0 / S) / 5e6;
+            if (us < best.us) best = {c.bn, S, us};
+        }
+    }
+    return best;
+}
+
+template <int FMT>
+int run(const tfq_weight* w, const void* x, int M, void* y, int yd, void* scratch, size_t scratch_bytes, hipStream_t s) {
     // the kernel addresses X with 32-bit byte offsets: tall inputs go through in slices of whole tiles
     const size_t row_bytes = (size_t)w->K * 2;
     const int max_rows = (int)std::min<size_t>(((size_t)0xFFFFF000u / row_bytes) & ~(size_t)511, (size_t)1 << 30);
@@ -359,57 +419,66 @@ int run(const tfq_weight* w, const void* x, int M, void* y, int yd, hipStream_t 
         a.K = (int)w->K;
         a.y_bf16 = yd == TFQ_BF16;
         a.tiles_m = (a.M + BM - 1) / BM;
-        // The strip width decides how many workgroups there are and how much LDS traffic an MFMA costs
-        // (wider is cheaper).  Workgroups run in rounds of one per compute unit, so the cost of a width is
-        // rounds x width, weighted by what a tile of that shape reaches; 224 (= 14 tiles of 16 rows) is there
-        // because it turns 1.75 rounds of 256-wide strips into two full ones at 14336 rows.
-        const auto cost = [&](int bn, double eff) {
-            const long tiles = (long)a.tiles_m * ((a.N + bn - 1) / bn);
-            return (double)((tiles + 255) / 256) * bn / eff;
-        };
-        // (the 8-bit formats hold twice the code registers: no 256-wide kernel for them; the affine formats'
-        // longer decode gains nothing from the 64 x 112 sub-tiles: measured 254-261 us against 251 us)
-        constexpr bool kAffine = FMT == TFQ_Q_G_4 || FMT == TFQ_Q_G_3;
-        const double c256 = tiled_planes(FMT) == 1 ? cost(256, 1.0) : 1e30, c224 = cost(224, kAffine ? 0.86 : 0.97), c128 = cost(128, 0.8);
+        const GemmPlan p = plan_tiles<FMT>(a.M, w->N, w->K, scratch ? scratch_bytes : 0);
+        a.ksplit = p.ksplit;
+        a.partial = reinterpret_cast<float*>(scratch);
         int rc;
-        if (c256 <= c224 && c256 <= c128) {
+        if (p.bn == 256) {
             if constexpr (tiled_planes(FMT) == 1) rc = run_tiles<FMT, 256, 512>(a, s);
             else rc = TFQ_ERR_SHAPE;
         } else {
-            rc = c224 <= c128 ? run_tiles<FMT, 224, 512>(a, s) : run_tiles<FMT, 128, 512>(a, s);
+            rc = p.bn == 224 ? run_tiles<FMT, 224, 512>(a, s) : run_tiles<FMT, 128, 512>(a, s);
         }
         if (rc) return rc;
     }
     return TFQ_OK;
 }
 
-}  // namespace
-
-// Few tokens make few workgroups for the tile kernel (one 256-token tile per 128 weight rows, each walking
-// all of K), while the batched decode kernel reads the matrix once per 16 rows with every compute unit busy.
-// Models of both from measurements on MI355X (us): a 16-row pass costs 2.5 + 3.2 per 4096 of K (activation
-// staging) + bytes / 6.5 TB/s, plus 15 %; the tile kernel 4 + rounds x (K / 32) x 0.44.  Measured crossovers:
-// 72 tokens at 14336x4096, 115 at 4096x4096, 125 at 4096x14336 (4-bit).
-static bool slices_cheaper(const tfq_weight* w, int M) {
-    if (!gemv_rows16_supported(w->fmt)) return false;
-    const double K = (double)w->K;
-    const double t16 = 1.15 * (2.5 + 3.2 * std::ceil(K / 4096.0) + (double)w->dev_bytes / 6.5e6);
-    const double tiles = (double)((M + 255) / 256) * (double)((w->N + 127) / 128);
-    const double t_gemm = 4.0 + std::ceil(tiles / 256.0) * (K / 32.0) * 0.44;
-    return (double)((M + 15) / 16) * t16 < t_gemm;
+GemmPlan plan_for(const tfq_weight* w, int M, size_t scratch_bytes) {
+    switch (canonical(w->fmt)) {
+        case TFQ_Q_G_4: return plan_tiles<TFQ_Q_G_4>(M, w->N, w->K, scratch_bytes);
+        case TFQ_B32S4: return plan_tiles<TFQ_B32S4>(M, w->N, w->K, scratch_bytes);
+        case TFQ_Q_G_3: return plan_tiles<TFQ_Q_G_3>(M, w->N, w->K, scratch_bytes);
+        case TFQ_B32S8: return plan_tiles<TFQ_B32S8>(M, w->N, w->K, scratch_bytes);
+        case TFQ_Q_G_8: return plan_tiles<TFQ_Q_G_8>(M, w->N, w->K, scratch_bytes);
+        default: return plan_tiles<TFQ_Q_8>(M, w->N, w->K, scratch_bytes);
+    }
 }
 
-int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype, hipStream_t s) {
-    const bool mfma_path = w->layout == TFQ_LAYOUT_TILED16 && tiled_header_bytes(w->fmt) == 16 && x_dtype == TFQ_BF16 && M > 16;
-    if (mfma_path && !slices_cheaper(w, M)) {
+bool tile_kernel_serves(const tfq_weight* w, int x_dtype, int M) {
+    return w->layout == TFQ_LAYOUT_TILED16 && tiled_header_bytes(w->fmt) == 16 && x_dtype == TFQ_BF16 && M > 16;
+}
+
+}  // namespace
+
+// Few tokens make few workgroups for the tile kernel, while the batched decode kernel reads the matrix once
+// per 16 rows with every compute unit busy: a 16-row pass costs (us) 2.5 + 3.2 per 4096 of K (activation
+// staging) + bytes / 6.5 TB/s, plus 15 %.  Measured crossovers without a K split: 72 tokens at 14336x4096,
+// 115 at 4096x4096, 125 at 4096x14336 (4-bit).
+static bool slices_cheaper(const tfq_weight* w, int M, double tile_us) {
+    if (!gemv_rows16_supported(w->fmt)) return false;
+    const double t16 = 1.15 * (2.5 + 3.2 * std::ceil((double)w->K / 4096.0) + (double)w->dev_bytes / 6.5e6);
+    return (double)((M + 15) / 16) * t16 < tile_us;
+}
+
+size_t gemm_scratch_bytes(const tfq_weight* w, int x_dtype, int M) {
+    if (!tile_kernel_serves(w, x_dtype, M)) return 0;
+    const GemmPlan p = plan_for(w, M, ~(size_t)0);
+    if (p.ksplit == 1 || slices_cheaper(w, M, p.us)) return 0;
+    return (size_t)p.ksplit * (size_t)M * (size_t)w->N * 4;
+}
+
+int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype, hipStream_t s, void* scratch,
+                size_t scratch_bytes) {
+    if (tile_kernel_serves(w, x_dtype, M) && !slices_cheaper(w, M, plan_for(w, M, scratch ? scratch_bytes : 0).us)) {
         if (w->N > 0x7FFFFFF0 || w->K > 0x7FFFFFF0 || w->dev_bytes >= 0xFFFFF000ull) return fail(TFQ_ERR_SHAPE, "gemm: matrix too large");
         switch (canonical(w->fmt)) {
-            case TFQ_Q_G_4: return run<TFQ_Q_G_4>(w, x, M, y, y_dtype, s);
-            case TFQ_B32S4: return run<TFQ_B32S4>(w, x, M, y, y_dtype, s);
-            case TFQ_Q_G_3: return run<TFQ_Q_G_3>(w, x, M, y, y_dtype, s);
-            case TFQ_B32S8: return run<TFQ_B32S8>(w, x, M, y, y_dtype, s);
-            case TFQ_Q_G_8: return run<TFQ_Q_G_8>(w, x, M, y, y_dtype, s);
-            case TFQ_Q_8: return run<TFQ_Q_8>(w, x, M, y, y_dtype, s);
+            case TFQ_Q_G_4: return run<TFQ_Q_G_4>(w, x, M, y, y_dtype, scratch, scratch_bytes, s);
+            case TFQ_B32S4: return run<TFQ_B32S4>(w, x, M, y, y_dtype, scratch, scratch_bytes, s);
+            case TFQ_Q_G_3: return run<TFQ_Q_G_3>(w, x, M, y, y_dtype, scratch, scratch_bytes, s);
+            case TFQ_B32S8: return run<TFQ_B32S8>(w, x, M, y, y_dtype, scratch, scratch_bytes, s);
+            case TFQ_Q_G_8: return run<TFQ_Q_G_8>(w, x, M, y, y_dtype, scratch, scratch_bytes, s);
+            case TFQ_Q_8: return run<TFQ_Q_8>(w, x, M, y, y_dtype, scratch, scratch_bytes, s);
             default: break;
         }
     }

@@ -361,8 +361,16 @@ int launch_moe_route(const float* logits, int T, int E, int k, float* probs, int
 int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E,
                    const int64_t* topk_idx, const float* topk_w, int T, int Ktop, const void* x, int x_dtype,
                    void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes, hipStream_t s);
+// `scratch` (optional, device memory) lets the tile kernel split K over several workgroups per output tile when
+// the tiles alone do not fill the GPU; gemm_scratch_bytes says how much a call would use, gemm_scratch_bound is
+// an upper bound for any matrix with at most `rows` x `cols` outputs (a split never makes more than 256 tiles).
 int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
-                hipStream_t s);
+                hipStream_t s, void* scratch = nullptr, size_t scratch_bytes = 0);
+size_t gemm_scratch_bytes(const tfq_weight* w, int x_dtype, int M);
+inline size_t gemm_scratch_bound(size_t rows, size_t cols) {
+    const size_t by_split = 8 * rows * cols * 4, by_tiles = (size_t)256 * 256 * 256 * 4;
+    return by_split < by_tiles ? by_split : by_tiles;
+}
 int launch_lut4_gemm(const uint8_t* packed, const uint16_t* cb16, const float* act, float* out, int M, int N, int K,
                      hipStream_t s);
 int launch_lut8_gemm(const uint8_t* idx, const float* cb, const float* act, float* out, int M, int N, int K,

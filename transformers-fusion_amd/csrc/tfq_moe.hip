@@ -123,6 +123,8 @@ struct Workspace {
     float* o;      // [P][D]
     int* lists;    // rows[P] | tok_pairs[P] | tok_first[T + 1] | weights[P] (float bits) | grouped-launch tables
     size_t list_bytes;
+    uint8_t* scratch;  // K-split partials of the prefill kernel
+    size_t scratch_bytes;
     size_t total;
 };
 
@@ -141,6 +143,9 @@ Workspace carve(void* base, int T, int Ktop, int64_t D, int64_t F) {
     ws.list_bytes = (3 * P + (size_t)T + 1) * 4 + 64 + 3 * P * gemv_group_entry_bytes() +
                     (2 * P * (size_t)((F + 15) / 16) + P * (size_t)((D + 15) / 16)) * 4;
     ws.lists = (int*)take(ws.list_bytes);
+    // partial tiles of the prefill kernel's K split (calls with many tokens per expert)
+    ws.scratch_bytes = gemm_scratch_bound(P, (size_t)(F > D ? F : D));
+    ws.scratch = take(ws.scratch_bytes);
     ws.total = off;
     return ws;
 }
@@ -284,8 +289,8 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
     for (int e = 0; e < E && !grouped; ++e) {
         const int p0 = first[e], nt = first[e + 1] - first[e];
         if (nt > 16) {  // the prefill entry: matrix cores for bf16 rows, 16-row slices otherwise
-            if (int rc = launch_gemm(gate[e], ws.xe + (size_t)p0 * D * xe_bytes, x_dtype, nt, ws.g + (size_t)p0 * F, TFQ_F32, s)) return rc;
-            if (int rc = launch_gemm(up[e], ws.xe + (size_t)p0 * D * xe_bytes, x_dtype, nt, ws.u + (size_t)p0 * F, TFQ_F32, s)) return rc;
+            if (int rc = launch_gemm(gate[e], ws.xe + (size_t)p0 * D * xe_bytes, x_dtype, nt, ws.g + (size_t)p0 * F, TFQ_F32, s, ws.scratch, ws.scratch_bytes)) return rc;
+            if (int rc = launch_gemm(up[e], ws.xe + (size_t)p0 * D * xe_bytes, x_dtype, nt, ws.u + (size_t)p0 * F, TFQ_F32, s, ws.scratch, ws.scratch_bytes)) return rc;
             continue;
         }
         for (int b0 = 0; b0 < nt; b0 += 16) {  // the GEMV entry takes up to 16 rows
@@ -309,7 +314,7 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
         const int p0 = first[e], nt = first[e + 1] - first[e];
         if (nt <= 0) continue;
         // sixteen rows or fewer take the decode kernels inside
-        if (int rc = launch_gemm(down[e], ws.h + (size_t)p0 * F * he, mid_dtype, nt, ws.o + (size_t)p0 * D, TFQ_F32, s)) return rc;
+        if (int rc = launch_gemm(down[e], ws.h + (size_t)p0 * F * he, mid_dtype, nt, ws.o + (size_t)p0 * D, TFQ_F32, s, ws.scratch, ws.scratch_bytes)) return rc;
     }
     if (y_dtype == TFQ_BF16)
         hipLaunchKernelGGL(combine_kernel<true>, dim3((unsigned)((nout + 255) / 256)), dim3(256), 0, s, y, ws.o, d_first, d_pairs, d_w, T, (int)D);
@@ -321,7 +326,9 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
 // Dense SwiGLU feed-forward (Qwen35Engine::mlp_step, src/adapters/tools/qwen35_engine.cpp:662-672): gate and up
 // in one launch where the format has the multi-matrix kernel, the elementwise step, down.  Rows above sixteen go
 // through the prefill entry.
-size_t mlp_workspace_bytes(int B, int64_t F) { return 3 * align256((size_t)B * (size_t)F * 4); }
+size_t mlp_workspace_bytes(int B, int64_t F) {
+    return 3 * align256((size_t)B * (size_t)F * 4) + (B > 16 ? align256(gemm_scratch_bound((size_t)B, (size_t)F)) : 0);
+}
 
 int launch_mlp_step(const tfq_weight* gate, const tfq_weight* up, const tfq_weight* down, const void* x, int x_dtype, int B,
                     void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes, hipStream_t s) {
@@ -333,13 +340,15 @@ int launch_mlp_step(const tfq_weight* gate, const tfq_weight* up, const tfq_weig
     float* g = reinterpret_cast<float*>(workspace);
     float* u = reinterpret_cast<float*>((uint8_t*)workspace + part);
     void* h = (uint8_t*)workspace + 2 * part;
+    void* scratch = B > 16 ? (uint8_t*)workspace + 3 * part : nullptr;  // K-split partials of the prefill kernel
+    const size_t scratch_bytes = B > 16 ? gemm_scratch_bound((size_t)B, (size_t)F) : 0;
     if (B <= 16 && canonical(gate->fmt) == canonical(up->fmt)) {
         const tfq_weight* gu[2] = {gate, up};
         void* gy[2] = {g, u};
         if (int rc = launch_gemv_multi(gu, 2, x, x_dtype, B, gy, TFQ_F32, s)) return rc;
     } else {
-        if (int rc = launch_gemm(gate, x, x_dtype, B, g, TFQ_F32, s)) return rc;
-        if (int rc = launch_gemm(up, x, x_dtype, B, u, TFQ_F32, s)) return rc;
+        if (int rc = launch_gemm(gate, x, x_dtype, B, g, TFQ_F32, s, scratch, scratch_bytes)) return rc;
+        if (int rc = launch_gemm(up, x, x_dtype, B, u, TFQ_F32, s, scratch, scratch_bytes)) return rc;
     }
     const int64_t nh = (int64_t)B * F;
     if (mid_dtype == TFQ_BF16)
@@ -347,7 +356,7 @@ int launch_mlp_step(const tfq_weight* gate, const tfq_weight* up, const tfq_weig
     else
         hipLaunchKernelGGL(silu_mul_kernel<false>, dim3((unsigned)((nh + 255) / 256)), dim3(256), 0, s, g, u, h, nh);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return hip_fail(e, "mlp_step launch");
-    return launch_gemm(down, h, mid_dtype, B, y, y_dtype, s);  // sixteen rows or fewer take the decode kernels inside
+    return launch_gemm(down, h, mid_dtype, B, y, y_dtype, s, scratch, scratch_bytes);  // sixteen rows or fewer take the decode kernels inside
 }
 
 }  // namespace tfq
