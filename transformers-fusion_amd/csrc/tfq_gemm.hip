@@ -26,6 +26,7 @@
 // the other's MFMA shadow without any hand scheduling.
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 
 #include "tfq_internal.hpp"
@@ -350,7 +351,7 @@ int run_tiles(GemmArgs a, hipStream_t s) {
     a.tiles_n = (a.N + BN - 1) / BN;
     const int grid = 8 * ((a.tiles_m * a.tiles_n * a.ksplit + 7) / 8);
     constexpr size_t lds = (size_t)(4 * BM * 4 + 2 * (BN > 128 ? 256 : 128) * 4) * 16;  // 96 KB or 80 KB
-    static bool lds_limit_raised = false;  // once: not allowed while a stream is being captured
+    static std::atomic<bool> lds_limit_raised{false};  // once: not allowed while a stream is being captured
     if (!lds_limit_raised) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm4_kernel<FMT, BN, NT>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

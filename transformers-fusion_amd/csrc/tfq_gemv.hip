@@ -38,6 +38,8 @@
 // into a private LDS cell per (tile, lane); after the only barrier the NW
 // partials of each output are added in a fixed order (deterministic results).
 
+#include <atomic>
+
 #include "tfq_internal.hpp"
 
 
@@ -890,7 +892,7 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     }
     // Raise the dynamic-LDS limit once per kernel (not per launch: the call is
     // not allowed while a stream is being captured into a graph).
-    static bool lds_limit_raised[8] = {};
+    static std::atomic<bool> lds_limit_raised[8] = {};
     if (!lds_limit_raised[slot]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -930,7 +932,7 @@ int run_gemvb(GemvArgs a, const void* x, hipStream_t s) {
     k.K = a.K; k.y_bf16 = a.y_bf16; k.nslot = a.nslot; k.tiles_per_wg = T;
     // staged activations and group sums of a chunk; the cells are inside them (one chunk) or behind them
     const size_t lds = (size_t)kGemvbKC * (8192 + 512) + (nchunks == 1 ? 0 : (size_t)T * kGemvbNW * 1024);
-    static bool lds_limit_raised = false;
+    static std::atomic<bool> lds_limit_raised{false};
     if (!lds_limit_raised) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemvb_kernel<FMT>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -1030,7 +1032,7 @@ int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, 
         if (gp.sets == 2) { kern = gemv4_kernel<FMT, false, 2, 2, true>; slot = 2; }
         if (gp.sets == 4) { kern = gemv4_kernel<FMT, false, 1, 4, true>; slot = 3; }
     }
-    static bool lds_limit_raised[4] = {};
+    static std::atomic<bool> lds_limit_raised[4] = {};
     if (!lds_limit_raised[slot]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
