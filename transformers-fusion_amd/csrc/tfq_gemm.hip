@@ -316,6 +316,20 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
         step.template operator()<7>(ks0, cur, nxt);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may land in LDS after the workgroup is gone
+    // the last steps' loads (for steps past the end) are never read, but they still write their registers:
+    // naming every ring register here keeps the compiler from handing one out before the wait above
+#pragma unroll
+    for (int i = 0; i < WROWS; ++i) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                uint32_t& w = rw[i][p][r];
+                asm volatile("" : "+v"(w));
+            }
+        u32x4_t& h = hnext[i];
+        asm volatile("" : "+v"(h));
+    }
 
     // ---- store: lane holds column fr, rows 4 fk + r of each 16 x 16 tile
 #pragma unroll
