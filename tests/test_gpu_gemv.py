@@ -297,3 +297,44 @@ def test_gemv_multi_with_eight_rows(O, tfq, gpu):
         assert float((got.double() - want).abs().max()) <= 1e-4 * float(want.abs().max())
         assert torch.equal(got, W.gemv(x))
         W.close()
+
+
+@pytest.mark.parametrize("fmt", ["B32S4", "B32S8"])
+def test_gemv_rows_with_k_split_repeated_calls(O, tfq, gpu, fmt):
+    """K above 4096 with five or more rows: the workgroups of a row group split K and meet through partial sums
+    and an arrival counter kept with the handle.  The counter must be back at zero after every launch: calls in
+    a row on one handle (other activations, fewer rows, bf16 output, 40 rows through tfq_gemm) each match a dense
+    product of the decoded matrix, a repeated call gives the same bits (the parts are added in a fixed order),
+    and two matrices of such a K in one launch (no split there) agree with the single launches."""
+    import torch
+    N, K = 1000, 14336  # 63 tiles, the last one short; 56 block columns in 4 parts of 14
+    g = torch.Generator(device="cuda").manual_seed(77)
+    W = tfq.Weight(fmt, N, K, tfq.encode(fmt, torch.randn(N * K, device=gpu, generator=g) * 0.02))
+    dense = W.decode().double()
+    first = None
+    for i, B in enumerate((16, 16, 5, 12, 9)):
+        print(f"gemv k-split {fmt} call {i} B={B}", flush=True)
+        x = torch.randn(B, K, device=gpu, generator=torch.Generator(device="cuda").manual_seed(5 if i < 2 else 5 + i)).bfloat16()
+        want = x.double() @ dense.T
+        scale = float(want.abs().max())
+        y = W.gemv(x)
+        assert float((y.double() - want).abs().max()) <= 1e-4 * scale
+        if i == 0:
+            first = y.clone()
+        if i == 1:
+            assert torch.equal(y, first)
+        yb = W.gemv(x, out_dtype=torch.bfloat16)
+        assert float((yb.double() - want).abs().max()) <= 1e-2 * scale
+    x = torch.randn(40, K, device=gpu, generator=g).bfloat16()
+    want = x.double() @ dense.T
+    # (tfq_gemm may take the matrix-core tile kernel, which rounds the decoded weights to bf16: 1e-2 is the bar there)
+    assert float((W.gemm(x).double() - want).abs().max()) <= 1e-2 * float(want.abs().max())
+    W2 = tfq.Weight(fmt, 48, K, tfq.encode(fmt, torch.randn(48 * K, device=gpu, generator=g) * 0.02))
+    x = torch.randn(8, K, device=gpu, generator=g).bfloat16()
+    outs = [torch.zeros(8, N, device=gpu), torch.zeros(8, 48, device=gpu)]
+    tfq.gemv_multi([W, W2], x, outs)
+    for Wi, got in zip((W, W2), outs):
+        want = x.double() @ Wi.decode().double().T
+        assert float((got.double() - want).abs().max()) <= 1e-4 * float(want.abs().max())
+    W.close()
+    W2.close()

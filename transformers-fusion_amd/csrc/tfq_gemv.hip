@@ -102,6 +102,8 @@ struct GemvArgs {
     int nslot;         // bf16 activation rows held in LDS: B, or 2B for fp32 input (<= 4)
     int tiles_per_wg;  // T
     int cols_base, cols_rem;  // block columns per wavefront: cols_base + (wave < cols_rem)
+    float* split_partial;     // single matrix only: the handle's partial sums and arrival counters, or null
+    unsigned* split_counters;
 };
 
 // What the kernel receives, flattened.  No arrays on purpose: a chain of selects over array
@@ -114,6 +116,9 @@ struct GemvKernArgs {
     int g0, g1, g2;
     int nr0, nr1, nr2, nr3;
     int K, y_bf16, nslot, tiles_per_wg, cols_base, cols_rem;
+    int kparts, kcols;  // gemvb_kernel: workgroups per row group (K parts) and block columns per part
+    float* partial;
+    unsigned* counters;
 };
 
 // Grouped launch: many independent problems (matrix, activation rows, output) of one format and
@@ -586,7 +591,7 @@ constexpr int kGemvbNW = 8, kGemvbKC = 16;
 constexpr int kGemvbMaxT1 = 16;  // tiles per workgroup, single chunk: 16 x 8 KB of cells inside the staging area
 constexpr int kGemvbMaxTn = 2;   // several chunks: cells behind the staging area
 
-template <int FMT>
+template <int FMT, bool SPLIT>
 __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const unsigned short* __restrict__ x) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
@@ -603,11 +608,20 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
     void* ym = m == 0 ? args.y0 : m == 1 ? args.y1 : m == 2 ? args.y2 : args.y3;
     const int nrm = m == 0 ? args.nr0 : m == 1 ? args.nr1 : m == 2 ? args.nr2 : args.nr3;
 
-    const int nblocks = K >> 8, nchunks = (nblocks + KC - 1) / KC;
+    // K split over workgroups (single matrix): workgroup bid walks part bid % kparts, kcols <= KC block columns,
+    // of row group bid / kparts; the parts of a row group meet through the partial sums at the end.  Without
+    // the split a workgroup walks all the chunks of KC columns itself.
+    constexpr bool split = SPLIT;
+    const int kparts = split ? args.kparts : 1;
+    const int kcols = split ? args.kcols : KC;
+    const int nblocks = K >> 8;
+    const int chunk_first = split ? bid % kparts : 0;
+    const int nchunks = split ? 1 : (nblocks + KC - 1) / KC;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, q = lane >> 4;
-    const int tile0 = (bid - wg_first) * T;
+    const int rowgroup = split ? bid / kparts : bid - wg_first;
+    const int tile0 = rowgroup * T;
     const int tiles_here = min(T, ((nrm + 15) >> 4) - tile0);
     const int total_gt = nchunks * tiles_here;  // (chunk, tile) visits, chunk-major
 
@@ -621,7 +635,10 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
     int f_chunk = 0, f_t = 0, f_ci = 0;
     const uint32_t off_c = 16u * lane, off_h = 1024u * NC + 16u * n;
     auto fetch = [&](uint4 (&cc)[NC], uint4& hd) __attribute__((always_inline)) {
-        const int col = min(f_chunk * KC + wave + NW * f_ci, nblocks - 1);
+        // a slot with no column of its own in this chunk re-reads a column the wavefront does own (cache hit, never used)
+        const int col0 = (chunk_first + f_chunk) * kcols, cols_here = min(kcols, nblocks - col0);
+        const int c_slot = wave + NW * f_ci;
+        const int col = col0 + (c_slot < cols_here ? c_slot : min(wave, cols_here - 1));
         const uint8_t* p = Wm + ((size_t)(tile0 + f_t) * nblocks + (size_t)col) * UB;
 #pragma unroll
         for (int i = 0; i < NC; ++i) cc[i] = stream_load16(p + off_c + 1024 * i);
@@ -649,8 +666,8 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
     // four adjacent lanes hold the four 8-element pieces of one group of one row, so their sums meet with two
     // DPP adds; the entry lands where lane (s, kq) of a wavefront will read it with one 128-bit LDS load.
     auto stage_chunk = [&](int chunk) __attribute__((always_inline)) {
-        const int cols_here = min(KC, nblocks - chunk * KC);
-        const unsigned short* xc = x + (size_t)chunk * KC * 256;
+        const int cols_here = min(kcols, nblocks - chunk * kcols);
+        const unsigned short* xc = x + (size_t)chunk * kcols * 256;
         for (int e0 = 0; e0 < cols_here * 512; e0 += 512 * 4) {  // four loads of a thread in flight together
             uint4 v[4];
 #pragma unroll
@@ -689,7 +706,7 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
 #pragma unroll
         for (int ci = 0; ci < 2; ++ci) {
             const int c_local = wave + NW * ci;
-            if (chunk * KC + c_local >= nblocks) continue;
+            if (c_local >= kcols || chunk * kcols + c_local >= nblocks) continue;
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -754,27 +771,28 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
         for (int dt = 0; dt < TW; ++dt) {
             const int gt = gt0 + dt;
             if (gt < total_gt) {  // uniform over the workgroup
-                const int chunk = gt / tiles_here, t = gt - chunk * tiles_here;
+                const int lchunk = gt / tiles_here, t = gt - lchunk * tiles_here;
+                const int chunk = chunk_first + lchunk;
                 if (t == 0) {
                     __syncthreads();  // every wavefront holds the previous chunk's fragments in registers, or is done with them
-                    if (chunk == 0) TRACE(2);
+                    if (lchunk == 0) TRACE(2);
                     stage_chunk(chunk);
-                    if (chunk == 0) TRACE(3);
+                    if (lchunk == 0) TRACE(3);
                     __syncthreads();
                     load_columns(chunk);
                     if (nchunks == 1) __syncthreads();  // the cells below overwrite the staged activations
-                    if (chunk == 0) TRACE(4);
+                    if (lchunk == 0) TRACE(4);
                 }
                 float res[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int ci = 0; ci < 2; ++ci) {
                     const int u = dt * 2 + ci;
                     const int c_local = wave + NW * ci;
-                    if (chunk * KC + c_local < nblocks) compute(ci, c_local, cc[u], hd[u], res);
+                    if (c_local < kcols && chunk * kcols + c_local < nblocks) compute(ci, c_local, cc[u], hd[u], res);
                     fetch(cc[u], hd[u]);
                 }
                 float4* cell = reinterpret_cast<float4*>(cells) + (t * NW + wave) * 64 + lane;
-                if (chunk == 0) *cell = float4{res[0], res[1], res[2], res[3]};
+                if (lchunk == 0) *cell = float4{res[0], res[1], res[2], res[3]};
                 else { const float4 o = *cell; *cell = float4{o.x + res[0], o.y + res[1], o.z + res[2], o.w + res[3]}; }
             }
         }
@@ -784,20 +802,51 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
     TRACE(6);
     // ---- add the eight wavefronts' partials in order and store: thread tid < 256 owns D[4 q' + r][n'] with
     // (n', q') = lane id tid % 64 and r = tid / 64, for every tile
-    if (tid < 256) {
-        const int nn = tid & 15, qq = (tid >> 4) & 3, r = tid >> 6;
-        const int slot = 4 * qq + r;
-        if (slot < B) {
-            for (int t = 0; t < tiles_here; ++t) {
-                const int row = (tile0 + t) * 16 + nn;
-                if (row >= nrm) continue;
-                const float* src = cells + ((size_t)t * NW * 64 + (tid & 63)) * 4 + r;
-                float v = 0.0f;
+    const int nn = tid & 15, qq = (tid >> 4) & 3, r = tid >> 6;
+    const int slot = 4 * qq + r;
+    const bool owner = tid < 256 && slot < B;
+    if (owner) {
+        for (int t = 0; t < tiles_here; ++t) {
+            const int row = (tile0 + t) * 16 + nn;
+            if (row >= nrm) continue;
+            const float* src = cells + ((size_t)t * NW * 64 + (tid & 63)) * 4 + r;
+            float v = 0.0f;
 #pragma unroll
-                for (int w = 0; w < NW; ++w) v += src[w * 256];
-                const size_t off = (size_t)slot * (size_t)nrm + (size_t)row;
-                if (y_bf16) reinterpret_cast<unsigned short*>(ym)[off] = (unsigned short)bf16_rne(v);
-                else reinterpret_cast<float*>(ym)[off] = v;
+            for (int w = 0; w < NW; ++w) v += src[w * 256];
+            const size_t off = (size_t)slot * (size_t)nrm + (size_t)row;
+            if (split) __hip_atomic_store(args.partial + (size_t)chunk_first * 16 * (size_t)nrm + off, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else if (y_bf16) reinterpret_cast<unsigned short*>(ym)[off] = (unsigned short)bf16_rne(v);
+            else reinterpret_cast<float*>(ym)[off] = v;
+        }
+    }
+    if constexpr (split) {
+        // The last part of a row group to arrive adds the parts in part order (the same sum whichever part
+        // that is) and puts the counter back to zero for the next launch.  Every workgroup passes through
+        // here exactly once and waits for nobody.
+        int& last_arrival = *reinterpret_cast<int*>(xsum);  // the group sums are no longer needed; the cells are elsewhere
+        // The partial sums are device-scope stores (written through to where every compute unit sees them) and
+        // are read back with device-scope loads, so no cache write-back or invalidation is needed: it is enough
+        // that every store of the workgroup has completed before its arrival is counted.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned seen = __hip_atomic_fetch_add(args.counters + rowgroup, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_arrival = seen == (unsigned)kparts - 1u;
+            if (last_arrival) __hip_atomic_store(args.counters + rowgroup, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (last_arrival) {
+            if (owner) {
+                for (int t = 0; t < tiles_here; ++t) {
+                    const int row = (tile0 + t) * 16 + nn;
+                    if (row >= nrm) continue;
+                    const size_t off = (size_t)slot * (size_t)nrm + (size_t)row;
+                    float v = 0.0f;
+                    for (int c = 0; c < kparts; ++c)
+                        v += __hip_atomic_load(args.partial + (size_t)c * 16 * (size_t)nrm + off, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (y_bf16) reinterpret_cast<unsigned short*>(ym)[off] = (unsigned short)bf16_rne(v);
+                    else reinterpret_cast<float*>(ym)[off] = v;
+                }
             }
         }
     }
@@ -912,12 +961,22 @@ int run_gemvb(GemvArgs a, const void* x, hipStream_t s) {
         for (int m = 0; m < a.nmat; ++m) g += ((a.nrows[m] + 15) / 16 + T - 1) / T;
         return g;
     };
-    const int nchunks = ((a.K >> 8) + kGemvbKC - 1) / kGemvbKC;
+    int nchunks = ((a.K >> 8) + kGemvbKC - 1) / kGemvbKC;
+    // Several chunks and a handle with room for partial sums: one workgroup per (row group, K part).  Every
+    // workgroup then stages one part of the activations once and walks many tiles with it, instead of staging
+    // every chunk for one or two tiles (the staging is what such a launch otherwise spends most of its time on).
+    const bool split = nchunks > 1 && a.nmat == 1 && a.split_partial != nullptr;
+    const int kparts = split ? nchunks : 1;
+    if (split) nchunks = 1;
     const int max_t = nchunks == 1 ? kGemvbMaxT1 : kGemvbMaxTn;
-    int T = (a.ntiles + num_cu - 1) / num_cu;
-    while (grid_for(T) > num_cu && T < max_t) ++T;
+    int T = (a.ntiles * kparts + num_cu - 1) / num_cu;
+    while (grid_for(T) * kparts > num_cu && T < max_t) ++T;
     if (T > max_t) T = max_t;
     GemvKernArgs k{};
+    k.kparts = kparts;
+    k.kcols = split ? ((a.K >> 8) + kparts - 1) / kparts : kGemvbKC;
+    k.partial = a.split_partial;
+    k.counters = a.split_counters;
     k.W0 = a.W[0]; k.W1 = a.W[1]; k.W2 = a.W[2]; k.W3 = a.W[3];
     k.y0 = a.y[0]; k.y1 = a.y[1]; k.y2 = a.y[2]; k.y3 = a.y[3];
     k.nr0 = a.nrows[0]; k.nr1 = a.nrows[1]; k.nr2 = a.nrows[2]; k.nr3 = a.nrows[3];
@@ -929,17 +988,25 @@ int run_gemvb(GemvArgs a, const void* x, hipStream_t s) {
     k.g0 = ends[0]; k.g1 = ends[1]; k.g2 = ends[2];
     int grid = g;
     if (a.nmat == 4) grid += ((a.nrows[3] + 15) / 16 + T - 1) / T;
+    if (split) {  // one matrix: every workgroup is on matrix 0
+        k.g0 = k.g1 = k.g2 = 0x7FFFFFFF;
+        grid *= kparts;
+    }
     k.K = a.K; k.y_bf16 = a.y_bf16; k.nslot = a.nslot; k.tiles_per_wg = T;
     // staged activations and group sums of a chunk; the cells are inside them (one chunk) or behind them
     const size_t lds = (size_t)kGemvbKC * (8192 + 512) + (nchunks == 1 ? 0 : (size_t)T * kGemvbNW * 1024);
     static std::atomic<bool> lds_limit_raised{false};
     if (!lds_limit_raised) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemvb_kernel<FMT>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemvb_kernel<FMT, false>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemvb_kernel<FMT, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
         lds_limit_raised = true;
     }
-    hipLaunchKernelGGL(gemvb_kernel<FMT>, dim3(grid), dim3(64 * kGemvbNW), lds, s, k, static_cast<const unsigned short*>(x));
+    if (split) hipLaunchKernelGGL((gemvb_kernel<FMT, true>), dim3(grid), dim3(64 * kGemvbNW), lds, s, k, static_cast<const unsigned short*>(x));
+    else hipLaunchKernelGGL((gemvb_kernel<FMT, false>), dim3(grid), dim3(64 * kGemvbNW), lds, s, k, static_cast<const unsigned short*>(x));
     return hip_fail(hipGetLastError(), "gemv launch");
 }
 
@@ -1052,6 +1119,17 @@ bool gemv_rows16_supported(int fmt) {
     }
 }
 
+int gemv_rows16_parts(int fmt, int64_t K) {
+    if (!gemv_rows16_supported(fmt) || K <= 0 || K % 256) return 1;
+    return (int)(((K >> 8) + kGemvbKC - 1) / kGemvbKC);
+}
+
+size_t gemv_rows16_split_bytes(int fmt, int64_t N, int64_t K) {
+    const int parts = gemv_rows16_parts(fmt, K);
+    if (parts < 2) return 0;
+    return (size_t)parts * 16 * (size_t)N * 4 + (size_t)((N + 15) / 16) * 4;
+}
+
 bool gemv_grouped_supported(int fmt) {
     switch (canonical(fmt)) {
         case TFQ_Q_G_4: case TFQ_B32S4: case TFQ_B32S8: case TFQ_Q_G_8: return true;
@@ -1124,6 +1202,10 @@ int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int 
     a.ntiles = (int)tiles;
     a.nmat = nmat;
     a.K = (int)ws[0]->K;
+    if (nmat == 1) {
+        a.split_partial = ws[0]->split_partial;
+        a.split_counters = ws[0]->split_counters;
+    }
     switch (canonical(ws[0]->fmt)) {
         case TFQ_Q_G_4: return gemv4_batched<TFQ_Q_G_4>(a, x, x_dtype, B, y_dtype, s);
         case TFQ_B32S4: return gemv4_batched<TFQ_B32S4>(a, x, x_dtype, B, y_dtype, s);

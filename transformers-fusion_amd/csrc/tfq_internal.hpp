@@ -305,6 +305,11 @@ struct tfq_weight {
     size_t dev_bytes;
     int layout;
     bool owns;
+    // Behind the packed weights in the same allocation, for matrices whose K is cut into several parts by the
+    // 5..16-row decode kernel: fp32 partial sums [parts][16 rows][N] and one arrival counter per 16-row tile
+    // (zero between launches).  One call at a time per handle may use them.
+    float* split_partial;
+    unsigned* split_counters;
 };
 
 namespace tfq {
@@ -348,6 +353,9 @@ struct GemvGroupPlan {
 };
 bool gemv_grouped_supported(int fmt);
 bool gemv_rows16_supported(int fmt);
+// K parts of the 5..16-row decode kernel (1: no split) and the bytes of partial sums and counters they need
+int gemv_rows16_parts(int fmt, int64_t K);
+size_t gemv_rows16_split_bytes(int fmt, int64_t N, int64_t K);
 int plan_gemv_grouped(int fmt, int K, bool x_f32, const int* nrows, const int* nrows_x, int nprob, GemvGroupPlan* gp);
 size_t gemv_group_entry_bytes();
 void fill_gemv_group(const GemvGroupPlan& gp, const tfq_weight* const* ws, const void* const* xs, void* const* ys,
