@@ -691,7 +691,8 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
                 sum = dpp_add<0x4E>(sum);
                 if (c < cols_here) {
                     xa[((c * 2 + h) * 4 + g) * 64 + kq * 16 + s] = p;
-                    if (kq == 0) xsum[(c * 8 + h * 4 + g) * 16 + s] = sum;
+                    // kept as -OFFS * sum: the accumulators start from it (the codes ride on an offset of OFFS)
+                    if (kq == 0) xsum[(c * 8 + h * 4 + g) * 16 + s] = -F::OFFS * sum;
                 }
             }
         }
@@ -729,7 +730,7 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
                 if constexpr (XREG) xv = xr[ci][h][g];
                 else xv = *reinterpret_cast<const float4*>(xsum + (c_local * 8 + h * 4 + g) * 16 + 4 * q);
                 X[g][0] = xv.x; X[g][1] = xv.y; X[g][2] = xv.z; X[g][3] = xv.w;
-                D[g] = f32x4_t{-F::OFFS * xv.x, -F::OFFS * xv.y, -F::OFFS * xv.z, -F::OFFS * xv.w};
+                D[g] = f32x4_t{xv.x, xv.y, xv.z, xv.w};
                 D2[g] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
             }
 #pragma unroll
@@ -751,6 +752,10 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
             }
             float a[4], off[4];
             group_scales<FMT>(&hdr, h, a, off);
+            if constexpr (!(FMT == TFQ_B32S4 || F::NP == 2)) {  // X holds -OFFS * (group sum)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) off[g] *= -1.0f / F::OFFS;
+            }
             float ph[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int g = 0; g < 4; ++g)
