@@ -27,6 +27,7 @@
 #include "tfq_internal.hpp"
 
 #include <algorithm>
+#include <mutex>
 #include <vector>
 
 namespace tfq {
@@ -150,6 +151,47 @@ Workspace carve(void* base, int T, int Ktop, int64_t D, int64_t F) {
     return ws;
 }
 
+// Pinned host buffers for the routing lists of a call, so that their upload is a true asynchronous copy and
+// the host can prepare the next call while the GPU still works on this one.  A ring of four; a slot is reused
+// only after the copy that last read it has completed (its event), which in a steady loop it long has.
+struct ListSlot {
+    void* host = nullptr;
+    size_t cap = 0;
+    hipEvent_t done = nullptr;
+    int device = -1;
+    bool recorded = false;
+};
+std::mutex g_list_mutex;
+ListSlot g_list_slots[4];
+unsigned g_list_next = 0;
+
+// Called with g_list_mutex held; the caller records slot->done behind the copy before it lets go.
+int acquire_list_slot(size_t bytes, ListSlot** out) {
+    int dev = 0;
+    TFQ_HIP(hipGetDevice(&dev));
+    ListSlot& sl = g_list_slots[g_list_next++ & 3u];
+    if (sl.recorded) {
+        TFQ_HIP(hipEventSynchronize(sl.done));
+        sl.recorded = false;
+    }
+    if (sl.device != dev && sl.done) {
+        (void)hipEventDestroy(sl.done);
+        sl.done = nullptr;
+    }
+    if (!sl.done) TFQ_HIP(hipEventCreateWithFlags(&sl.done, hipEventDisableTiming));
+    sl.device = dev;
+    if (sl.cap < bytes) {
+        if (sl.host) (void)hipHostFree(sl.host);
+        sl.host = nullptr;
+        sl.cap = 0;
+        const size_t want = (bytes + 65535) & ~(size_t)65535;
+        TFQ_HIP(hipHostMalloc(&sl.host, want, hipHostMallocDefault));
+        sl.cap = want;
+    }
+    *out = &sl;
+    return TFQ_OK;
+}
+
 }  // namespace
 
 size_t moe_workspace_bytes(int T, int Ktop, int64_t D, int64_t F) { return carve(nullptr, T, Ktop, D, F).total; }
@@ -253,13 +295,16 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
     const size_t mapA = tabB + wB.size() * eb, mapB = mapA + (size_t)planA.grid * 4;
     const size_t list_bytes = grouped ? mapB + (size_t)planB.grid * 4 : base_ints * 4;
     if (list_bytes > ws.list_bytes) return fail(TFQ_ERR_SHAPE, "moe: routing tables exceed the workspace");
-    std::vector<int> lists(list_bytes / 4 + 2);
+    std::lock_guard<std::mutex> list_lock(g_list_mutex);
+    ListSlot* slot = nullptr;
+    if (int rc = acquire_list_slot(list_bytes + 8, &slot)) return rc;
+    int* const lists = static_cast<int*>(slot->host);
     if (grouped) {
-        uint8_t* lb = reinterpret_cast<uint8_t*>(lists.data());
+        uint8_t* lb = reinterpret_cast<uint8_t*>(lists);
         fill_gemv_group(planA, wA.data(), xA.data(), yA.data(), rA.data(), (int)wA.size(), lb + tabA, reinterpret_cast<int*>(lb + mapA));
         fill_gemv_group(planB, wB.data(), xB.data(), yB.data(), rB.data(), (int)wB.size(), lb + tabB, reinterpret_cast<int*>(lb + mapB));
     }
-    int* h_rows = lists.data();
+    int* h_rows = lists;
     int* h_pairs = h_rows + P;
     int* h_first = h_pairs + P;
     float* h_w = reinterpret_cast<float*>(h_first + T + 1);
@@ -272,9 +317,10 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
     int* d_pairs = d_rows + P;
     int* d_first = d_pairs + P;
     float* d_w = reinterpret_cast<float*>(d_first + T + 1);
-    // The source is pageable host memory: wait for the copy before the vectors go out of scope.
-    TFQ_HIP(hipMemcpyAsync(ws.lists, lists.data(), list_bytes, hipMemcpyHostToDevice, s));
-    TFQ_HIP(hipStreamSynchronize(s));
+    // The source is pinned: the copy is asynchronous, and the event tells when the slot may be filled again.
+    TFQ_HIP(hipMemcpyAsync(ws.lists, lists, list_bytes, hipMemcpyHostToDevice, s));
+    TFQ_HIP(hipEventRecord(slot->done, s));
+    slot->recorded = true;
 
     if (P) {
         const int row_u4 = (int)(D * xe_bytes / 16);
