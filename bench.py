@@ -47,6 +47,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM figure")
     ap.add_argument("--no-moe", action="store_true", help="skip the mixture-of-experts layer figure")
+    ap.add_argument("--no-sweep", action="store_true",
+                    help="skip the batch / format sweep (batch 4, 8, 16; the 8-bit format; the low-bit superblock formats)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one elementwise kernel that reads and writes 1 GiB (counter calibration)")
     ap.add_argument("--probe", action="store_true",
@@ -163,13 +165,107 @@ def main():
 
     if not args.no_prefill:
         res["prefill"] = prefill_gemm(tfq, torch, layers[0], gen)
+    if not args.no_sweep:
+        res["sweep"] = decode_sweep(tfq, torch, layers, fmt, gen)
     if not args.no_moe:
         del layers
         torch.cuda.empty_cache()
-        res["moe"] = moe_layer(tfq, torch, fmt, bpw, gen)
+        # a generator of its own: the routing does not depend on which other figures ran before
+        res["moe"] = moe_layer(tfq, torch, fmt, bpw, torch.Generator(device=dev).manual_seed(45))
     if not args.no_cpu:
         res["cpu_baseline"] = cpu_baseline(host_layer0, fmt, B, acts, bpw)
     print(json.dumps(res), flush=True)
+
+
+def time_graph(torch, fn, reps=10):
+    """us per call of fn (launches on the current stream), from graph replays when capture works."""
+    fn()
+    torch.cuda.synchronize()
+    run = fn
+    try:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        g.replay()
+        run = g.replay
+    except Exception:
+        pass
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / reps
+
+
+def decode_sweep(tfq, torch, layers, fmt, gen):
+    """Side figures, never `value`: the decode layer of the main workload at batch 4, 8 and 16 (same weights,
+    same four launches per layer), the 8-bit block-32 format at batch 1 and 16 on eight layers, and the low-bit
+    superblock formats (Laplace(0, 0.015) weights, 14336x4096, twelve rotated copies) at batch 1 and 8.
+    GB/s = algorithmic bytes / time, as for `value`."""
+    dev = "cuda"
+    out = {}
+
+    def layer_step(ls, B):
+        acts = {k: torch.randn(B, n, device=dev, generator=gen).bfloat16() for k, n in (("x", 4096), ("a", 4096), ("h", 14336))}
+        outs = {name: torch.empty(B, N, device=dev, dtype=torch.float32) for name, N, _, _ in PROJ}
+
+        def step():
+            for ws in ls:
+                tfq.gemv_multi([ws["q"], ws["k"], ws["v"]], acts["x"], [outs["q"], outs["k"], outs["v"]])
+                ws["o"].gemv(acts["a"], out=outs["o"])
+                tfq.gemv_multi([ws["gate"], ws["up"]], acts["x"], [outs["gate"], outs["up"]])
+                ws["down"].gemv(acts["h"], out=outs["down"])
+        return step
+
+    def layer_figures(ls, f, B):
+        bpw = float(tfq.lib().tfq_format_bpw(tfq.fmt_id(f)))
+        us = time_graph(torch, layer_step(ls, B)) / len(ls)
+        nbytes = sum(alg_bytes(N, K, B, bpw) for _, N, K, _ in PROJ)
+        return {"us_per_layer": round(us, 2), "gbs": round(nbytes / us / 1e3, 1),
+                "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "tok_s": round(B * 1e6 / (us * 32.0), 1)}
+
+    out[fmt] = {str(B): layer_figures(layers, fmt, B) for B in (4, 8, 16)}
+    ls8 = []
+    for _ in range(8):
+        ws = {}
+        for name, N, K, _ in PROJ:
+            w = torch.randn(N * K, device=dev, generator=gen) * 0.02
+            ws[name] = tfq.Weight("B32S8", N, K, tfq.encode("B32S8", w))
+            del w
+        ls8.append(ws)
+    out["B32S8"] = {str(B): layer_figures(ls8, "B32S8", B) for B in (1, 16)}
+    for ws in ls8:
+        for W in ws.values():
+            W.close()
+    del ls8
+    N, K = 14336, 4096
+    for f in ("SB256A3", "SB256A2"):
+        bpw = float(tfq.lib().tfq_format_bpw(tfq.fmt_id(f)))
+        Ws = []
+        for _ in range(12):
+            u = torch.rand(N * K, device=dev, generator=gen) - 0.5
+            w = -0.015 * torch.sign(u) * torch.log1p(-2.0 * u.abs())
+            Ws.append(tfq.Weight(f, N, K, tfq.encode(f, w)))
+            del u, w
+        out[f] = {}
+        for B in (1, 8):
+            x = torch.randn(B, K, device=dev, generator=gen).bfloat16()
+            y = torch.empty(B, N, device=dev, dtype=torch.float32)
+
+            def step():
+                for W in Ws:
+                    W.gemv(x, out=y)
+            us = time_graph(torch, step) / len(Ws)
+            nbytes = alg_bytes(N, K, B, bpw)
+            out[f][str(B)] = {"shape": "%dx%d" % (N, K), "us": round(us, 2), "gbs": round(nbytes / us / 1e3, 1),
+                              "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        for W in Ws:
+            W.close()
+        del Ws
+    return out
 
 
 MFMA_PEAK_TFLOPS = 2500.0

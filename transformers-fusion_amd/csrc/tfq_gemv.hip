@@ -861,6 +861,9 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
 // Formats whose kernel is also built with several slot sets per pass (up to 16 bf16 rows).
 template <int FMT>
 constexpr bool kWide = FMT == TFQ_B32S4 || FMT == TFQ_B32S8 || FMT == TFQ_Q_G_4 || FMT == TFQ_Q_G_8 || FMT == TFQ_Q_8;
+// Formats built with two slot sets only (eight bf16 rows per pass): the affine low-bit formats.
+template <int FMT>
+constexpr bool kTwoSets = kWide<FMT> || FMT == TFQ_Q_G_3 || FMT == TFQ_Q_G_2 || FMT == TFQ_SB256A3 || FMT == TFQ_SB256A2;
 
 struct GemvPlan {
     int NW, T, sets;
@@ -943,6 +946,15 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
             kern = p.sets == 2 ? gemv4_kernel<FMT, false, 2, 2> : gemv4_kernel<FMT, false, 1, 4>;
             slot = p.sets == 2 ? 6 : 7;
         }
+    } else if constexpr (kTwoSets<FMT>) {
+        if (p.sets == 2) {
+            kern = gemv4_kernel<FMT, false, 2, 2>;
+            slot = 6;
+        } else if (p.sets > 2) {
+            return fail(TFQ_ERR_SHAPE, "gemv: more than eight rows in one pass for this format");
+        }
+    } else if (p.sets > 1) {
+        return fail(TFQ_ERR_SHAPE, "gemv: more than four rows in one pass for this format");
     }
     // Raise the dynamic-LDS limit once per kernel (not per launch: the call is
     // not allowed while a stream is being captured into a graph).
@@ -1041,9 +1053,9 @@ int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t 
         }
     }
     int step = a.x_f32 ? 2 : 4;
-    if constexpr (kWide<FMT>) {
+    if constexpr (kTwoSets<FMT>) {
         if (!a.x_f32 && B > 4) {
-            for (int rows = 16; rows > 4; rows >>= 1)
+            for (int rows = kWide<FMT> ? 16 : 8; rows > 4; rows >>= 1)
                 if (plan_gemv4<FMT>(a, rows).lds != 0) { step = rows; break; }
         }
     }
