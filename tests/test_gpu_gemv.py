@@ -338,3 +338,30 @@ def test_gemv_rows_with_k_split_repeated_calls(O, tfq, gpu, fmt):
         assert float((got.double() - want).abs().max()) <= 1e-4 * float(want.abs().max())
     W.close()
     W2.close()
+
+
+def test_gemv_k_split_in_graph_replays(O, tfq, gpu):
+    """The K-split launch inside a captured graph: its arrival counters reset themselves, so every replay
+    (with eager launches on the same handle between replays) gives the bits of the eager result."""
+    import torch
+    N, K, B = 4096, 14336, 16
+    g = torch.Generator(device="cuda").manual_seed(11)
+    W = tfq.Weight("B32S4", N, K, tfq.encode("B32S4", torch.randn(N * K, device=gpu, generator=g) * 0.02))
+    xs = [torch.randn(B, K, device=gpu, generator=g).bfloat16() for _ in range(3)]
+    eager = [W.gemv(x).clone() for x in xs]
+    outs = [torch.empty(B, N, device=gpu) for _ in xs]
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for x, y in zip(xs, outs):
+            W.gemv(x, out=y)
+    for rep in range(5):
+        print(f"gemv k-split graph replay {rep}", flush=True)
+        for y in outs:
+            y.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for want, got in zip(eager, outs):
+            assert torch.equal(want, got)
+        assert torch.equal(W.gemv(xs[rep % 3]), eager[rep % 3])  # eager work between the replays
+    W.close()
