@@ -877,11 +877,14 @@ GemvPlan plan_gemv4(const GemvArgs& a, int nslot) {
     const int nblocks = a.K >> 8;
     GemvPlan p{};
     p.sets = nslot <= 4 ? 1 : nslot <= 8 ? 2 : 4;
-    // wavefronts per workgroup: the count in max/2..max that splits the block columns most evenly;
-    // several slot sets need the registers of two wavefronts, so at most 8 then
+    // wavefronts per workgroup.  One slot set: as many as there are (16); more wavefronts keep more fetches in
+    // flight, which counts for more than an even split of the block columns (measured, B32S4 4096x14336: 8.8 us
+    // with 16 wavefronts of 3 or 4 columns against 9.7-10.5 us with 14 of 4; 4096x7168 5.25 against 5.9 us).
+    // Several slot sets need the registers of two wavefronts, so at most 8 then: the count in 4..8 that splits
+    // the block columns most evenly.
     const int max_nw = p.sets == 1 ? 16 : 8;
     p.NW = nblocks < max_nw ? nblocks : max_nw;
-    if (nblocks > max_nw) {
+    if (nblocks > max_nw && p.sets > 1) {
         int best_waste = 1 << 30;
         for (int w = max_nw; w >= max_nw / 2; --w) {
             const int waste = (nblocks + w - 1) / w * w - nblocks;
