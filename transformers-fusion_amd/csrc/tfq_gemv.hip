@@ -934,9 +934,12 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     k.K = a.K; k.y_bf16 = a.y_bf16; k.nslot = a.nslot; k.tiles_per_wg = T;
     k.cols_base = a.cols_base; k.cols_rem = a.cols_rem;
     const int full_items = a.cols_base * T;  // units of a wavefront with the fewest block columns in a full workgroup
-    // formats with a 32-byte header or two nibble planes hold more registers per unit in flight: at most two units
-    constexpr int WDMAX = Fmt<FMT>::HV == 1 && Fmt<FMT>::NP == 1 ? 4 : 2;
-    const int wd = full_items >= 4 && WDMAX == 4 ? 4 : full_items >= 2 ? 2 : 1;
+    // Two unit fetches in flight per wavefront at most.  Sixteen wavefronts already keep 32 units (74 KB) per
+    // compute unit on their way; four per wavefront (which only the one-plane formats with a 16-byte header
+    // have the registers for) measured slower: B32S4 28672x4096 14.8 us against 14.0-14.2 us, 14336x4096 8.6
+    // against 8.2 us, at four rows 15.3 against 14.2 us.
+    constexpr int WDMAX = 2;
+    const int wd = full_items >= 2 ? 2 : 1;
     using Kernel = void (*)(GemvKernArgs, const void*);
     static const Kernel kernels[2][3] = {
         {gemv4_kernel<FMT, false, 1>, gemv4_kernel<FMT, false, 2>, gemv4_kernel<FMT, false, WDMAX>},
