@@ -586,7 +586,7 @@ __device__ __forceinline__ void transpose_rows(uint32_t (&v)[4]) {
 //     after the last chunk the eight partials of each output are added in wavefront order.  With a single K
 //     chunk (K <= 4096) the cells reuse the LDS of the staged activations, which are in registers by then,
 //     and a workgroup can hold many tiles; with several chunks they need room of their own (few tiles).
-// Unit fetches run four ahead (two tiles x two columns) with unconditional loads, as in gemv4_kernel.
+// Unit fetches run two ahead (one tile x two columns) with unconditional loads, as in gemv4_kernel.
 constexpr int kGemvbNW = 8, kGemvbKC = 16;
 constexpr int kGemvbMaxT1 = 16;  // tiles per workgroup, single chunk: 16 x 8 KB of cells inside the staging area
 constexpr int kGemvbMaxTn = 2;   // several chunks: cells behind the staging area
@@ -597,8 +597,10 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
     using F = Fmt<FMT>;
     static_assert(F::GS == 32 && F::HV == 1, "32-weight groups and a 16-byte header");
     constexpr int UB = tiled_unit_bytes(FMT), NC = 2 * F::NP, NW = kGemvbNW, KC = kGemvbKC;
-    // unit fetches in flight per wavefront: TW tiles x two columns (four tiles measured no faster)
-    constexpr int TW = 2, WD = 2 * TW;
+    // unit fetches in flight per wavefront: TW tiles x two columns.  One tile (two fetches) measured faster than
+    // two at sixteen rows: B32S4 4096x14336 17.6 against 18.5 us, 6144x4096 9.6 / 10.3 us, 4096x4096 8.3 / 8.6 us,
+    // 28672x4096 equal; B32S8 28672x4096 32.5 / 35.9 us, 4096x14336 22.8 / 24.5 us (four tiles no faster than two)
+    constexpr int TW = 1, WD = 2 * TW;
     const int K = args.K, T = args.tiles_per_wg, B = args.nslot;
     const bool y_bf16 = args.y_bf16 != 0;
     const int bid = blockIdx.x;
