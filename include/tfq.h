@@ -247,6 +247,58 @@ int tfq_mlp_step(const tfq_weight_t* gate, const tfq_weight_t* up, const tfq_wei
                  int x_dtype, int B, void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes,
                  tfq_stream_t stream);
 
+/* ---- a chain of dependent matrix-vector products in one launch -----------------------
+ * The decode step of the reference engine is a sequence of B = 1 gemm calls, each on the result
+ * of the one before, with elementwise steps between them:
+ *   rmsnorm -> q, k, v | o -> h += o | rmsnorm -> gate, up -> silu(gate) * up -> down -> h += down
+ * (Qwen35Engine::append_token, src/adapters/tools/qwen35_engine.cpp:807-835; mlp_step :662-672;
+ * rmsnorm :46-51: x * 1/sqrt(mean(x^2) + eps) * (1 + w)).  A chain runs such a sequence
+ * ("phases") in ONE persistent launch: the packed weights of every phase stream without a gap
+ * while the arithmetic of a phase waits for the phase before it.
+ *
+ * A phase multiplies up to four matrices (one format per chain: B32S4 or Q_G_4; equal K inside
+ * a phase, K <= 14336) with the same B <= 2 activation rows.
+ *   x          device pointer [B][K] (x_dtype), or NULL: the result of the previous phase, which
+ *              is the concatenation of its outputs [B][N0 + N1 + ...] (its first K columns are
+ *              used), the SwiGLU product [B][N], or the updated residual rows
+ *   x_depends  set when a non-NULL x is written by an earlier phase of the same chain (for
+ *              example the residual buffer): the phase then waits for the phase before it
+ *   x_op       TFQ_CHAIN_X_PLAIN, or TFQ_CHAIN_X_RMSNORM: x * rsqrt(mean(x^2) + eps) * gamma
+ *              (gamma_plus_one: * (1 + gamma), the reference's form) before the product
+ *   y_op       TFQ_CHAIN_Y_PLAIN; TFQ_CHAIN_Y_SWIGLU: two matrices (gate, up), result =
+ *              silu(gate x) * (up x); TFQ_CHAIN_Y_RESIDUAL: one matrix, residual[B][N] += W x in
+ *              place, and the sum is the phase's result
+ *   y[i]       device output [B][N_i] of matrix i (y_dtype; fp32 for SwiGLU), or NULL when only
+ *              the next phase reads the result
+ * Activations are rounded to bf16 before every product (accumulation and elementwise steps in
+ * fp32), as in tfq_gemv with bf16 x.  The chain owns device memory for its tables, counters and
+ * intermediate results: runs of ONE chain must not overlap in time (one stream).  The handles and
+ * buffers named at creation must stay alive.  tfq_chain_check, called after the stream has been
+ * synchronised, reports a run whose internal waits ran out (TFQ_ERR_DEVICE) and clears that state. */
+enum { TFQ_CHAIN_X_PLAIN = 0, TFQ_CHAIN_X_RMSNORM = 1 };
+enum { TFQ_CHAIN_Y_PLAIN = 0, TFQ_CHAIN_Y_SWIGLU = 1, TFQ_CHAIN_Y_RESIDUAL = 2 };
+typedef struct tfq_chain_phase {
+    const tfq_weight_t* w[4];
+    int count;
+    const void* x;
+    int x_dtype;
+    int x_depends;
+    int x_op;
+    const float* gamma;
+    float eps;
+    int gamma_plus_one;
+    int y_op;
+    void* y[4];
+    int y_dtype;
+    float* residual;
+} tfq_chain_phase_t;
+typedef struct tfq_chain tfq_chain_t;
+tfq_chain_t* tfq_chain_create(const tfq_chain_phase_t* phases, int nphase, int B);
+int tfq_chain_run(const tfq_chain_t* chain, tfq_stream_t stream);
+int tfq_chain_check(const tfq_chain_t* chain);
+size_t tfq_chain_weight_bytes(const tfq_chain_t* chain); /* packed bytes one run streams */
+void tfq_chain_free(tfq_chain_t* chain);
+
 /* ---- MoE expert path ------------------------------------------------------------
  * tfq_moe_route: router softmax + top-k on the device, softmax_with_topk
  * (src/model/moe_core.cpp:98-149): probs [T][E], idx [T][k] (descending

@@ -1,0 +1,127 @@
+"""The persistent chain of dependent matrix-vector products (tfq_chain_*) against the oracle.
+
+The oracle side is a composition of pinned pieces: O.matmul (block-row GEMV in the reference's loop order),
+O.silu_mul (src/math/math.cpp:117-126) and the rmsnorm of Qwen35Engine::rmsnorm
+(src/adapters/tools/qwen35_engine.cpp:46-51) restated in numpy below; activations are rounded to bf16 before
+every product, as the chain does.  Tolerance: max |y - y_ref| / max |y_ref| <= 1e-2 (bf16 activations).
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_err(y, ref):
+    return float(np.abs(y.astype(np.float64) - ref).max() / np.abs(ref).max())
+
+
+def rmsnorm_ref(x, w, eps=1e-6, plus_one=True):
+    """Qwen35Engine::rmsnorm: out = x * 1/sqrt(sum(x^2)/n + eps) * (1 + w), fp32."""
+    x = x.astype(np.float32)
+    s = np.float32(0)
+    for v in x:  # the reference's sequential fp32 sum
+        s = np.float32(s + v * v)
+    r = np.float32(1.0) / np.sqrt(np.float32(s / np.float32(x.size) + np.float32(eps)), dtype=np.float32)
+    g = (np.float32(1) + w) if plus_one else w
+    return ((x * r) * g).astype(np.float32)
+
+
+def _weights(O, tfq, fmt, shapes, seed):
+    out = {}
+    for i, (name, N, K) in enumerate(shapes):
+        pay = O.encode_tensor(fmt, O.rng_normal(seed + i, N * K, 0.02))
+        out[name] = (tfq.Weight(fmt, N, K, pay), pay, N, K)
+    return out
+
+
+@pytest.mark.parametrize("fmt", ["B32S4", "Q_G_4"])
+@pytest.mark.parametrize("D,F,B", [(1024, 2048, 1), (4096, 14336, 1), (2048, 3584, 2)])
+def test_chain_mlp_step_matches_oracle(O, tfq, gpu, fmt, D, F, B):
+    """Qwen35Engine::mlp_step as one launch: [gate, up] -> silu(gate) * up -> down."""
+    import torch
+    W = _weights(O, tfq, fmt, [("gate", F, D), ("up", F, D), ("down", D, F)], 300)
+    x = O.bf16_round(O.rng_normal(43, B * D, 1.0)).reshape(B, D)
+    xd = torch.from_numpy(x).to(gpu).bfloat16()
+    g_d = torch.zeros(B, F, device=gpu)
+    u_d = torch.zeros(B, F, device=gpu)
+    y_d = torch.zeros(B, D, device=gpu)
+    chain = tfq.Chain([
+        {"w": [W["gate"][0], W["up"][0]], "x": xd, "y_op": tfq.Y_SWIGLU, "y": [g_d, u_d]},
+        {"w": [W["down"][0]], "y": [y_d]},
+    ], B=B)
+    chain.run()
+    torch.cuda.synchronize()
+    chain.check()
+    g = O.matmul(fmt, W["gate"][1], F, D, x)
+    u = O.matmul(fmt, W["up"][1], F, D, x)
+    h = O.bf16_round(O.silu_mul(g, u))
+    y = O.matmul(fmt, W["down"][1], D, F, h)
+    assert rel_err(g_d.cpu().numpy(), g) <= 1e-2
+    assert rel_err(u_d.cpu().numpy(), u) <= 1e-2
+    assert rel_err(y_d.cpu().numpy(), y) <= 1e-2
+    # a second run gives the same bits (fixed summation order, counters back at zero)
+    first = y_d.clone()
+    y_d.zero_()
+    chain.run()
+    torch.cuda.synchronize()
+    chain.check()
+    assert torch.equal(first, y_d)
+    chain.close()
+
+
+@pytest.mark.parametrize("fmt", ["B32S4"])
+def test_chain_decoder_layer_matches_oracle(O, tfq, gpu, fmt):
+    """rmsnorm -> q, k, v | o(q) -> h += . | rmsnorm -> gate, up -> silu * up -> down -> h += .
+    (append_token's projections; the attention between q/k/v and o is outside the path, o takes q)."""
+    import torch
+    D, F, KV = 2048, 4096, 512
+    W = _weights(O, tfq, fmt, [("q", D, D), ("k", KV, D), ("v", KV, D), ("o", D, D), ("gate", F, D), ("up", F, D), ("down", D, F)], 500)
+    h0 = O.rng_normal(7, D, 1.0)
+    g1 = O.rng_normal(8, D, 0.1)
+    g2 = O.rng_normal(9, D, 0.1)
+    h_d = torch.from_numpy(h0.copy()).to(gpu).reshape(1, D)
+    g1_d, g2_d = torch.from_numpy(g1).to(gpu), torch.from_numpy(g2).to(gpu)
+    q_d, k_d, v_d = (torch.zeros(1, n, device=gpu) for n in (D, KV, KV))
+    chain = tfq.Chain([
+        {"w": [W["q"][0], W["k"][0], W["v"][0]], "x": h_d, "x_op": tfq.X_RMSNORM, "gamma": g1_d, "gamma_plus_one": True,
+         "y": [q_d, k_d, v_d]},
+        {"w": [W["o"][0]], "y_op": tfq.Y_RESIDUAL, "residual": h_d},
+        {"w": [W["gate"][0], W["up"][0]], "x_op": tfq.X_RMSNORM, "gamma": g2_d, "gamma_plus_one": True, "y_op": tfq.Y_SWIGLU},
+        {"w": [W["down"][0]], "y_op": tfq.Y_RESIDUAL, "residual": h_d},
+    ], B=1)
+    chain.run()
+    torch.cuda.synchronize()
+    chain.check()
+
+    xn = O.bf16_round(rmsnorm_ref(h0, g1))
+    q = O.matmul(fmt, W["q"][1], D, D, xn)
+    k = O.matmul(fmt, W["k"][1], KV, D, xn)
+    v = O.matmul(fmt, W["v"][1], KV, D, xn)
+    o = O.matmul(fmt, W["o"][1], D, D, O.bf16_round(q.reshape(-1)))
+    h1 = (h0 + o.reshape(-1)).astype(np.float32)
+    xn2 = O.bf16_round(rmsnorm_ref(h1, g2))
+    g = O.matmul(fmt, W["gate"][1], F, D, xn2)
+    u = O.matmul(fmt, W["up"][1], F, D, xn2)
+    hh = O.bf16_round(O.silu_mul(g, u))
+    dn = O.matmul(fmt, W["down"][1], D, F, hh)
+    h2 = (h1 + dn.reshape(-1)).astype(np.float32)
+    assert rel_err(q_d.cpu().numpy(), q) <= 1e-2
+    assert rel_err(k_d.cpu().numpy(), k) <= 1e-2
+    assert rel_err(v_d.cpu().numpy(), v) <= 1e-2
+    assert rel_err(h_d.cpu().numpy().reshape(-1), h2) <= 1e-2
+    chain.close()
+
+
+def test_chain_rejects_what_it_cannot_run(O, tfq, gpu):
+    import torch
+    pay = O.encode_tensor("Q_G_8", O.rng_normal(1, 256 * 256, 0.02))
+    w8 = tfq.Weight("Q_G_8", 256, 256, pay)
+    x = torch.zeros(1, 256, device=gpu).bfloat16()
+    with pytest.raises(tfq.TfqError):
+        tfq.Chain([{"w": [w8], "x": x, "y": [torch.zeros(1, 256, device=gpu)]}])
+    pay4 = O.encode_tensor("B32S4", O.rng_normal(2, 256 * 256, 0.02))
+    w4 = tfq.Weight("B32S4", 256, 256, pay4)
+    with pytest.raises(tfq.TfqError):  # the first phase has no input
+        tfq.Chain([{"w": [w4], "y": [torch.zeros(1, 256, device=gpu)]}])
+    with pytest.raises(tfq.TfqError):  # three rows
+        tfq.Chain([{"w": [w4], "x": torch.zeros(3, 256, device=gpu).bfloat16(), "y": [torch.zeros(3, 256, device=gpu)]}], B=3)

@@ -109,6 +109,11 @@ def _load():
         "tfq_container_read_tensor": (i32, [vp, C.c_char_p, vp, i64, vp]),
         "tfq_container_read_tensor_host": (i32, [vp, C.c_char_p, vp, i64]),
         "tfq_container_weight": (vp, [vp, C.c_char_p, i64, i64]),
+        "tfq_chain_create": (vp, [vp, i32, i32]),
+        "tfq_chain_run": (i32, [vp, vp]),
+        "tfq_chain_check": (i32, [vp]),
+        "tfq_chain_weight_bytes": (sz, [vp]),
+        "tfq_chain_free": (None, [vp]),
         "tfq_malloc": (vp, [sz]),
         "tfq_free": (None, [vp]),
         "tfq_copy_to_device": (i32, [vp, vp, sz]),
@@ -255,6 +260,90 @@ class Weight:
         _check(lib().tfq_gemm_ws(self.handle, x.data_ptr(), _dtype_code(x), M, y.data_ptr(), _dtype_code(y),
                                  ws.data_ptr(), need, _stream()))
         return y
+
+
+class _ChainPhase(C.Structure):
+    """tfq_chain_phase_t (include/tfq.h)."""
+    _fields_ = [("w", C.c_void_p * 4), ("count", C.c_int), ("x", C.c_void_p), ("x_dtype", C.c_int),
+                ("x_depends", C.c_int), ("x_op", C.c_int), ("gamma", C.c_void_p), ("eps", C.c_float),
+                ("gamma_plus_one", C.c_int), ("y_op", C.c_int), ("y", C.c_void_p * 4), ("y_dtype", C.c_int),
+                ("residual", C.c_void_p)]
+
+
+X_PLAIN, X_RMSNORM = 0, 1
+Y_PLAIN, Y_SWIGLU, Y_RESIDUAL = 0, 1, 2
+
+
+class Chain:
+    """A sequence of dependent matrix-vector products in one persistent launch (tfq_chain_*).
+
+    phases: list of dicts with keys
+      w (list of Weight), x (tensor [B][K] or None = the previous phase's result), x_depends (bool),
+      x_op (X_PLAIN / X_RMSNORM), gamma (fp32 tensor), eps, gamma_plus_one,
+      y_op (Y_PLAIN / Y_SWIGLU / Y_RESIDUAL), y (list of tensors or None), residual (fp32 tensor [B][N]).
+    The tensors and Weight objects are kept alive by the chain."""
+
+    def __init__(self, phases, B: int = 1):
+        arr = (_ChainPhase * len(phases))()
+        self._keep = []
+        for i, ph in enumerate(phases):
+            d = arr[i]
+            ws = ph["w"]
+            d.count = len(ws)
+            for m, w in enumerate(ws):
+                d.w[m] = w.handle
+                self._keep.append(w)
+            x = ph.get("x")
+            if x is not None:
+                d.x = x.data_ptr()
+                d.x_dtype = _dtype_code(x)
+                self._keep.append(x)
+            d.x_depends = 1 if ph.get("x_depends") else 0
+            d.x_op = ph.get("x_op", X_PLAIN)
+            g = ph.get("gamma")
+            if g is not None:
+                d.gamma = g.data_ptr()
+                self._keep.append(g)
+            d.eps = float(ph.get("eps", 1e-6))
+            d.gamma_plus_one = 1 if ph.get("gamma_plus_one") else 0
+            d.y_op = ph.get("y_op", Y_PLAIN)
+            ys = ph.get("y") or []
+            d.y_dtype = F32
+            for m, y in enumerate(ys):
+                if y is not None:
+                    d.y[m] = y.data_ptr()
+                    d.y_dtype = _dtype_code(y)
+                    self._keep.append(y)
+            r = ph.get("residual")
+            if r is not None:
+                d.residual = r.data_ptr()
+                self._keep.append(r)
+        h = lib().tfq_chain_create(C.cast(arr, C.c_void_p), len(phases), B)
+        if not h:
+            raise TfqError(lib().tfq_last_error().decode())
+        self.handle = C.c_void_p(h)
+
+    @property
+    def weight_bytes(self) -> int:
+        return int(lib().tfq_chain_weight_bytes(self.handle))
+
+    def run(self):
+        _check(lib().tfq_chain_run(self.handle, _stream()))
+
+    def check(self):
+        """Call after synchronising: raises if a wait inside the last runs ran out."""
+        _check(lib().tfq_chain_check(self.handle))
+
+    def close(self):
+        if getattr(self, "handle", None):
+            lib().tfq_chain_free(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class Container:
