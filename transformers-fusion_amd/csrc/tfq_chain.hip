@@ -29,6 +29,7 @@
 
 #include "tfq_gemv_common.hpp"
 
+
 namespace tfq {
 
 namespace {
@@ -37,6 +38,7 @@ using namespace gemv_detail;
 
 constexpr int kWG = 256;         // workgroups of a launch = compute units of an MI355X
 constexpr int kWaves = 16;       // wavefronts per workgroup
+constexpr int kLoaders = 2;      // of which loaders (one is not enough: 47 against 40 us per Llama-3-8B layer)
 constexpr int kMaxPhases = 128;  // phases per launch
 constexpr int kMaxSlot = 2;      // activation rows (bf16) per chain
 constexpr int kMaxTiles = 8;     // 16-row tiles of one workgroup in one phase (both segments)
@@ -112,6 +114,53 @@ __device__ __forceinline__ void lds_copy16(uint32_t lds_base, uint32_t lane_off,
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3 nt" ::"s"(lds_base), "v"(lane_off), "s"(base), "n"(OFF) : "memory");
 }
 
+// One unit (NCODE pieces of 1 KB and a header piece of 16 * HV lanes) into a ring slot, M0 written once; the
+// header copy runs with the upper lanes switched off, so that it writes 256 (512) bytes of LDS only.
+template <int NCODE, int HV>
+__device__ __forceinline__ void lds_copy_unit(uint32_t lds_base, uint32_t lane_off, const uint8_t* base) {
+    unsigned long long saved;
+    if constexpr (NCODE == 2 && HV == 1) {
+        asm volatile(
+            "s_mov_b32 m0, %1\n\ts_nop 0\n\t"
+            "global_load_lds_dwordx4 %2, %3 offset:0 nt\n\t"
+            "global_load_lds_dwordx4 %2, %3 offset:1024 nt\n\t"
+            "s_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffff\n\t"
+            "global_load_lds_dwordx4 %2, %3 offset:2048 nt\n\t"
+            "s_mov_b64 exec, %0"
+            : "=&s"(saved) : "s"(lds_base), "v"(lane_off), "s"(base) : "memory");
+    } else if constexpr (NCODE == 2 && HV == 2) {
+        asm volatile(
+            "s_mov_b32 m0, %1\n\ts_nop 0\n\t"
+            "global_load_lds_dwordx4 %2, %3 offset:0 nt\n\t"
+            "global_load_lds_dwordx4 %2, %3 offset:1024 nt\n\t"
+            "s_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffffffff\n\t"
+            "global_load_lds_dwordx4 %2, %3 offset:2048 nt\n\t"
+            "s_mov_b64 exec, %0"
+            : "=&s"(saved) : "s"(lds_base), "v"(lane_off), "s"(base) : "memory");
+    } else {
+        static_assert(NCODE == 4 && HV == 1, "unit shapes of the Tiled16 layout");
+        asm volatile(
+            "s_mov_b32 m0, %1\n\ts_nop 0\n\t"
+            "global_load_lds_dwordx4 %2, %3 offset:0 nt\n\t"
+            "global_load_lds_dwordx4 %2, %3 offset:1024 nt\n\t"
+            "global_load_lds_dwordx4 %2, %3 offset:2048 nt\n\t"
+            "global_load_lds_dwordx4 %2, %3 offset:3072 nt\n\t"
+            "s_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffff\n\t"
+            "global_load_lds_dwordx4 %2, %3 offset:4096 nt\n\t"
+            "s_mov_b64 exec, %0"
+            : "=&s"(saved) : "s"(lds_base), "v"(lane_off), "s"(base) : "memory");
+    }
+}
+
+// waits until the oldest of `outstanding` (1..K) units in flight, LOADS copies each, has landed
+template <int LOADS, int K>
+__device__ __forceinline__ void wait_oldest(int outstanding) {
+    if constexpr (K >= 1) {
+        if (outstanding == K) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS * (K - 1)) : "memory");
+        else wait_oldest<LOADS, K - 1>(outstanding);
+    }
+}
+
 // LDS words of control state
 enum : int { C_ABORT = 0, C_SYNC = 1, C_DEP = 2, C_SUMSQ = 4 /* .. +2*15 */, C_WORDS = 40 };
 
@@ -122,7 +171,10 @@ __global__ __launch_bounds__(1024) void chain_kernel(ChainArgs a) {
     constexpr int UB = tiled_unit_bytes(FMT);
     constexpr int NCODE = 2 * F::NP;         // 1 KB code pieces of a unit
     constexpr int LOADS = NCODE + 1;         // copies per unit (the header piece is 16 * HB = 256 or 512 bytes)
-    constexpr int Q = 63 / LOADS;            // copies in flight per loader: the hardware counter holds 63
+    // units in flight per loader (the hardware counter holds 63 copies).  One wavefront with 8 units in flight
+    // streams 6.2 TB/s on MI355X, two with 8 each 6.8 TB/s; more in flight gains nothing and makes every other
+    // memory access of the compute unit wait longer.
+    constexpr int Q = 63 / LOADS < 8 ? 63 / LOADS : 8;
     constexpr int NC = kWaves - NL;          // consumer wavefronts
     constexpr int NG = F::NG, PER = NG / 2;
     static_assert(F::HV == 1 || F::HV == 2, "header of one or two 16-byte pieces per row");
@@ -196,47 +248,63 @@ __global__ __launch_bounds__(1024) void chain_kernel(ChainArgs a) {
         bool stop = false;
         for (int p = 0; p < nph && !stop; ++p) {
             const int* e = lph + p * 8;
-            const unsigned long long w0 = ((unsigned long long)uni((unsigned)e[1]) << 32) | uni((unsigned)e[0]);
-            const unsigned long long w1 = ((unsigned long long)uni((unsigned)e[3]) << 32) | uni((unsigned)e[2]);
-            const int T0 = uni(e[4]), T1 = uni(e[5]), nb = uni(e[6]), seq0 = uni(e[7]);
-            const int T2 = T0 + T1, U = T2 * nb;
-            int j = ((lid - seq0) % NL + NL) % NL;  // first unit of this phase that is this loader's
-            int col = j / (T2 > 0 ? T2 : 1), t = j - col * T2;
-            int slot = (seq0 + j) % R;
-            for (; j < U; j += NL) {
-                const unsigned g = (unsigned)(seq0 + j);
-                const uint8_t* ptr = t < T0 ? (const uint8_t*)w0 + ((size_t)t * nb + col) * UB
-                                            : (const uint8_t*)w1 + ((size_t)(t - T0) * nb + col) * UB;
-                if (g >= (unsigned)R) {  // the slot's previous unit must have been taken
-                    const unsigned need = g - (unsigned)R + 1u;
-                    if ((int)(lds_get(free_seq + slot) - need) < 0) {
-                        drain();
+            const unsigned long long wseg[2] = {((unsigned long long)uni((unsigned)e[1]) << 32) | uni((unsigned)e[0]),
+                                                ((unsigned long long)uni((unsigned)e[3]) << 32) | uni((unsigned)e[2])};
+            const int nb = uni(e[6]), seq0 = uni(e[7]);
+            const int useg[2] = {uni(e[4]) * nb, uni(e[5]) * nb};  // units of the two segments
+            // units in memory order: segment by segment, tile by tile, block columns inside (contiguous bytes)
+            for (int sg = 0; sg < 2 && !stop; ++sg) {
+                const int first = sg ? useg[0] : 0;  // unit index inside the phase
+                int j = first + (((lid - seq0 - first) % NL + NL) % NL);  // this loader's first unit of the segment
+                int count = j < first + useg[sg] ? (first + useg[sg] - j + NL - 1) / NL : 0;
+                const uint8_t* ptr = (const uint8_t*)wseg[sg] + (size_t)(j - first) * UB;
+                unsigned g = (unsigned)(seq0 + j);
+                int slot = (int)(g % (unsigned)R);
+                while (count > 0) {
+                    // how many of the next units have a free slot?  Lane i looks at the i-th one.
+                    int nfree;
+                    {
+                        const unsigned gi = g + (unsigned)(lane * NL);
+                        const int si = (int)(gi % (unsigned)R);
+                        bool fr = lane < count && lane < 32;
+                        if (fr && gi >= (unsigned)R)
+                            fr = (int)(__hip_atomic_load(free_seq + si, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) - (gi - (unsigned)R + 1u)) >= 0;
+                        const unsigned long long m = __builtin_amdgcn_ballot_w64(fr);
+                        nfree = (int)__builtin_ctzll(~m);
+                    }
+                    if (nfree == 0) {
+                        // The ring is full.  Copies already in flight are published one by one while there is
+                        // nothing else to do, but not at once: where the consumers set the pace a slot comes
+                        // free within a few polls, and waiting for the youngest copy would leave one unit in flight.
+                        const unsigned need = g - (unsigned)R + 1u;
                         unsigned polls = 0;
                         while ((int)(lds_get(free_seq + slot) - need) < 0) {
-                            __builtin_amdgcn_s_sleep(1);
-                            if ((++polls & 63u) == 0 && (aborted() || polls > spin_limit)) { stop = true; break; }
+                            ++polls;
+                            if ((polls & 15u) == 0 && outstanding > 0) {
+                                wait_oldest<LOADS, Q>(outstanding);
+                                publish_oldest();
+                            } else {
+                                __builtin_amdgcn_s_sleep(1);
+                            }
+                            if ((polls & 63u) == 0 && (aborted() || polls > spin_limit)) { stop = true; break; }
                         }
                         if (stop) { if (!aborted()) give_up(1u); break; }
+                        nfree = 1;
+                    }
+                    count -= nfree;
+                    for (; nfree > 0; --nfree) {
+                        lds_copy_unit<NCODE, F::HV>(uni(ring_lds + (uint32_t)slot * UB), off_c, uni_ptr(ptr));
+                        ptr += (size_t)NL * UB;
+                        g += NL;
+                        slot += NL;
+                        if (slot >= R) slot -= R;
+                        ++outstanding;
+                        if (outstanding == Q) {
+                            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS * (Q - 1)) : "memory");
+                            publish_oldest();
+                        }
                     }
                 }
-                const uint8_t* p8 = uni_ptr(ptr);
-                const uint32_t dst = uni(ring_lds + (uint32_t)slot * UB);
-                lds_copy16<0>(dst, off_c, p8);
-                lds_copy16<1024>(dst, off_c, p8);
-                if constexpr (NCODE == 4) {
-                    lds_copy16<2048>(dst, off_c, p8);
-                    lds_copy16<3072>(dst, off_c, p8);
-                }
-                if (lane < 16 * F::HV) lds_copy16<1024 * NCODE>(dst, off_c, p8);
-                ++outstanding;
-                if (outstanding > Q) {
-                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS * Q) : "memory");
-                    publish_oldest();
-                }
-                t += NL;
-                while (t >= T2) { t -= T2; ++col; }
-                slot += NL;
-                if (slot >= R) slot -= R;
             }
         }
         drain();
@@ -271,7 +339,6 @@ __global__ __launch_bounds__(1024) void chain_kernel(ChainArgs a) {
         const int* e = lph + p * 8;
         const int T0 = uni(e[4]), T1 = uni(e[5]), nb = uni(e[6]), seq0 = uni(e[7]);
         const int T2 = T0 + T1, U = T2 * nb;
-
         // ---- the previous phase must be complete everywhere (wave 0 asks, the others wait for its word)
         if (p > 0) {
             if (wave == 0) {
@@ -296,7 +363,6 @@ __global__ __launch_bounds__(1024) void chain_kernel(ChainArgs a) {
             }
             if (!ok || aborted()) { ok = false; break; }
         }
-
         // ---- stage the activations: wavefront w takes block columns w, w + NC, ...; lanes 0..31 carry slot 0,
         // lanes 32..63 slot 1; a lane holds 8 consecutive elements
         {
@@ -397,17 +463,16 @@ __global__ __launch_bounds__(1024) void chain_kernel(ChainArgs a) {
             }
             if (!meet()) { ok = false; break; }
         }
-
         // ---- the units: consumer w takes units w, w + NC, ... of the phase, in the loader's order
-        // (block-column major, tiles inside)
         {
             int j = wave;
-            int col = j / (T2 > 0 ? T2 : 1), t = j - col * T2;
+            int t = j / nb, col = j - t * nb;  // tile by tile, block columns inside
             int slot = (seq0 + j) % R;
             for (; j < U; j += NC) {
                 const unsigned g = (unsigned)(seq0 + j);
                 unsigned polls = 0;
                 while (lds_get(ready_seq + slot) != g + 1u) {
+                    __builtin_amdgcn_s_sleep(1);
                     if ((++polls & 63u) == 0 && (aborted() || polls > spin_limit)) { if (!aborted()) give_up(16u); ok = false; break; }
                 }
                 if (!ok) break;
@@ -467,8 +532,8 @@ __global__ __launch_bounds__(1024) void chain_kernel(ChainArgs a) {
                 }
                 if (q < nslot) mycells[(t * nslot + q) * 16 + n] += res;
 
-                t += NC;
-                while (t >= T2) { t -= T2; ++col; }
+                col += NC;
+                while (col >= nb) { col -= nb; ++t; }
                 slot += NC;
                 while (slot >= R) slot -= R;
             }
@@ -562,7 +627,7 @@ int chain_occupancy(size_t lds) {
 using namespace tfq;
 
 struct tfq_chain {
-    int fmt = 0, nph = 0, B = 0, loaders = 2;
+    int fmt = 0, nph = 0, B = 0;
     int ring = 0, ncols_max = 0, tmax = 0;
     size_t lds = 0;
     ChainPhase* d_phases = nullptr;
@@ -604,8 +669,7 @@ tfq_chain_t* tfq_chain_create(const tfq_chain_phase_t* phases, int nphase, int B
     tfq_chain* c = new tfq_chain();
     c->nph = nphase;
     c->B = B;
-    if (const char* env = std::getenv("TFQ_CHAIN_LOADERS")) c->loaders = std::atoi(env) == 1 ? 1 : 2;
-    const int NC = kWaves - c->loaders;
+    const int NC = kWaves - kLoaders;
     std::vector<ChainPhase> hp((size_t)nphase);
     std::vector<ChainWg> hw((size_t)nphase * kWG);
     std::vector<long long> load(kWG, 0);  // units handed to each workgroup so far
@@ -736,8 +800,7 @@ tfq_chain_t* tfq_chain_create(const tfq_chain_phase_t* phases, int nphase, int B
     if (ring > 4096) ring = 4096;
     c->ring = ring;
     c->lds = fixed + (size_t)ring * (UB + 8);
-    const int occ = c->loaders == 1 ? (fmt == TFQ_B32S4 ? chain_occupancy<TFQ_B32S4, 1>(c->lds) : chain_occupancy<TFQ_Q_G_4, 1>(c->lds))
-                                    : (fmt == TFQ_B32S4 ? chain_occupancy<TFQ_B32S4, 2>(c->lds) : chain_occupancy<TFQ_Q_G_4, 2>(c->lds));
+    const int occ = fmt == TFQ_B32S4 ? chain_occupancy<TFQ_B32S4, kLoaders>(c->lds) : chain_occupancy<TFQ_Q_G_4, kLoaders>(c->lds);
     if (occ < 1) { chain_fail(c, TFQ_ERR_DEVICE, "tfq_chain_create: the chain kernel does not fit a compute unit"); return nullptr; }
     if (hipMalloc(&c->d_phases, hp.size() * sizeof(ChainPhase)) != hipSuccess || hipMalloc(&c->d_wgs, hw.size() * sizeof(ChainWg)) != hipSuccess ||
         hipMemcpy(c->d_phases, hp.data(), hp.size() * sizeof(ChainPhase), hipMemcpyHostToDevice) != hipSuccess ||
@@ -756,8 +819,7 @@ int tfq_chain_run(const tfq_chain_t* c, tfq_stream_t stream) {
     a.spin_limit = kSpinLimit;
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;
-    if (c->loaders == 1) e = c->fmt == TFQ_B32S4 ? launch_chain<TFQ_B32S4, 1>(a, c->lds, s) : launch_chain<TFQ_Q_G_4, 1>(a, c->lds, s);
-    else e = c->fmt == TFQ_B32S4 ? launch_chain<TFQ_B32S4, 2>(a, c->lds, s) : launch_chain<TFQ_Q_G_4, 2>(a, c->lds, s);
+    e = c->fmt == TFQ_B32S4 ? launch_chain<TFQ_B32S4, kLoaders>(a, c->lds, s) : launch_chain<TFQ_Q_G_4, kLoaders>(a, c->lds, s);
     return hip_fail(e, "chain launch");
 }
 
@@ -771,6 +833,7 @@ int tfq_chain_check(const tfq_chain_t* c) {
     }
     return TFQ_OK;
 }
+
 
 size_t tfq_chain_weight_bytes(const tfq_chain_t* c) { return c ? c->weight_bytes : 0; }
 
