@@ -223,6 +223,16 @@ int tfq_gemm(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, 
 size_t tfq_gemm_workspace_bytes(const tfq_weight_t* w, int x_dtype, int M);
 int tfq_gemm_ws(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
                 void* workspace, size_t workspace_bytes, tfq_stream_t stream);
+/* tfq_gemm_ws for callers that cannot allocate or bring a workspace: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  The K-split scratch is a fixed array of
+ * tfq_gemm_static_scratch_bytes() = 32 MiB in the library's device image (every GPU the library runs on holds
+ * its copy until the process ends); the call itself allocates nothing.  A product whose split would use more
+ * (tfq_gemm_workspace_bytes above that size) is refused with TFQ_ERR_SHAPE.  Same results as tfq_gemm_ws with
+ * a workspace of tfq_gemm_workspace_bytes.  All calls on one GPU share the array: calls that overlap in time
+ * on one GPU race (issue them on one stream).  No counterpart in the reference. */
+int tfq_gemm_static(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
+                    tfq_stream_t stream);
+size_t tfq_gemm_static_scratch_bytes(void);
 /* Up to four matrices that share K, format and the activation rows in ONE launch:
  * ys[i][b][n] = sum_k x[b][k] * ws[i][n][k].  This is the q/k/v step and the
  * gate/up step of the reference engine, which issue one gemm per matrix on the

@@ -72,6 +72,8 @@ def _load():
         "tfq_gemm": (i32, [vp, vp, i32, i32, vp, i32, vp]),
         "tfq_gemm_workspace_bytes": (sz, [vp, i32, i32]),
         "tfq_gemm_ws": (i32, [vp, vp, i32, i32, vp, i32, vp, sz, vp]),
+        "tfq_gemm_static": (i32, [vp, vp, i32, i32, vp, i32, vp]),
+        "tfq_gemm_static_scratch_bytes": (sz, []),
         "tfq_gemv_multi": (i32, [vp, i32, vp, i32, i32, vp, i32, vp]),
         "tfq_matmul_host": (i32, [vp, vp, vp, i32]),
         "tfq_mlp_workspace_bytes": (sz, [i32, i64]),

@@ -363,6 +363,13 @@ int tfq_gemm_ws(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* 
     return launch_gemm(w, x, x_dtype, M, y, y_dtype, (hipStream_t)stream, workspace, workspace ? workspace_bytes : 0);
 }
 
+int tfq_gemm_static(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, int y_dtype, tfq_stream_t stream) {
+    if (int r = check_matmul("tfq_gemm_static", w, x, x_dtype, M, y, y_dtype)) return r;
+    return launch_gemm_static(w, x, x_dtype, M, y, y_dtype, (hipStream_t)stream);
+}
+
+size_t tfq_gemm_static_scratch_bytes(void) { return gemm_static_scratch_bytes(); }
+
 int tfq_moe_route(const float* logits, int T, int E, int k, float* probs, int32_t* idx, float* weights, tfq_stream_t stream) {
     if (!logits || !probs || !idx || !weights) return fail(TFQ_ERR_ARG, "tfq_moe_route: null pointer");
     if (T <= 0 || E <= 0) return fail(TFQ_ERR_ARG, "tfq_moe_route: T and E must be positive");

@@ -511,4 +511,41 @@ int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y,
     return TFQ_OK;
 }
 
+// ---- the prefill product for callers that cannot allocate
+// The K split of the tile kernel keeps its fp32 partial tiles in scratch memory.  tfq_gemm_ws takes that memory
+// from the caller; here it is a fixed array in the library's device image, so a call allocates nothing (no
+// hipMalloc, no hipFree, no allocating library routine).  Each GPU has its own copy of the array at its own
+// address: the name below is only the host-side handle of the symbol, the address a kernel can use comes from
+// hipGetSymbolAddress with that GPU current, once per GPU.
+constexpr size_t kStaticScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_static_scratch_ptr[kMaxDevices] = {};
+}  // namespace
+
+int launch_gemm_static(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype, hipStream_t s) {
+    int dev = -1;
+    TFQ_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(TFQ_ERR_DEVICE, "tfq_gemm_static: device index out of range");
+    void* scratch = g_static_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!scratch) {
+        void* p = nullptr;
+        TFQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_scratch)));
+        if (!p) return fail(TFQ_ERR_DEVICE, "tfq_gemm_static: the scratch array has no device address");
+        g_static_scratch_ptr[dev].store(p, std::memory_order_release);  // the same address whichever thread resolves it
+        scratch = p;
+    }
+    const size_t need = gemm_scratch_bytes(w, x_dtype, M);
+    if (need > kStaticScratchBytes)
+        return fail(TFQ_ERR_SHAPE, "tfq_gemm_static: this product would use " + std::to_string(need) +
+                                       " bytes of scratch memory, the static area holds " + std::to_string(kStaticScratchBytes) +
+                                       "; use tfq_gemm_ws with a workspace of your own");
+    // every partial tile is written before it is read, so nothing has to start at zero
+    return launch_gemm(w, x, x_dtype, M, y, y_dtype, s, scratch, kStaticScratchBytes);
+}
+
+size_t gemm_static_scratch_bytes() { return kStaticScratchBytes; }
+
 }  // namespace tfq

@@ -375,6 +375,9 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
 int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
                 hipStream_t s, void* scratch = nullptr, size_t scratch_bytes = 0);
 size_t gemm_scratch_bytes(const tfq_weight* w, int x_dtype, int M);
+// launch_gemm with the K-split scratch in a fixed device array of the library (no allocation in the call)
+int launch_gemm_static(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype, hipStream_t s);
+size_t gemm_static_scratch_bytes();
 inline size_t gemm_scratch_bound(size_t rows, size_t cols) {
     const size_t by_split = 8 * rows * cols * 4, by_tiles = (size_t)256 * 256 * 256 * 4;
     return by_split < by_tiles ? by_split : by_tiles;
