@@ -333,6 +333,27 @@ int tfq_moe_ffn(const tfq_weight_t* const* gate, const tfq_weight_t* const* up,
                 int T, int k, const void* x, int x_dtype, void* y, int y_dtype, int mid_dtype,
                 void* workspace, size_t workspace_bytes, tfq_stream_t stream);
 
+/* Capacity-limited dispatch, moe_engine::plan_dispatch / gather_expert_inputs / combine_expert_outputs
+ * (engines/trainer/moe/dispatch.cpp:9-78): the slots (t, j) are walked in token order, j inside; a slot joins
+ * the list of its expert while that list has fewer than slots_per_expert items and is dropped otherwise; an
+ * expert id outside 0..E-1 is an error (the reference throws).  Every kept slot contributes
+ * out[t] += w(t, j) * FFN_e(x_t), experts ascending and items in list order, whatever the sign of the weight.
+ *   tfq_moe_plan_dispatch  the plan alone, host arrays: expert_first [E + 1] (items of expert e are
+ *                          expert_first[e] .. expert_first[e + 1]), item_token / item_weight [T * k],
+ *                          dropped_slot [T * k] (t * k + j of the dropped slots in order; may be NULL),
+ *                          *dropped = their count
+ *   tfq_moe_ffn_capacity   plan + gather + expert FFNs + combine; topk_idx is int32 like the reference's
+ *                          index tensor; *dropped (host, may be NULL) receives the dropped count that
+ *                          combine_expert_outputs returns.  Other arguments as tfq_moe_ffn. */
+int tfq_moe_plan_dispatch(const int32_t* topk_idx, const float* topk_w, int T, int k, int E,
+                          int64_t slots_per_expert, int32_t* expert_first, int32_t* item_token,
+                          float* item_weight, int32_t* dropped_slot, int64_t* dropped);
+int tfq_moe_ffn_capacity(const tfq_weight_t* const* gate, const tfq_weight_t* const* up,
+                         const tfq_weight_t* const* down, int E, const int32_t* topk_idx, const float* topk_w,
+                         int T, int k, int64_t slots_per_expert, const void* x, int x_dtype, void* y,
+                         int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes,
+                         int64_t* dropped, tfq_stream_t stream);
+
 /* ---- codebook-lookup operators ----------------------------------------------------
  * Weights are BITS-wide indices into one small table of centroids.  packed / idx,
  * act / X and out / Y are device pointers; the codebook is a HOST pointer (it is

@@ -272,6 +272,49 @@ def moe_ffn(fmt, gate, up, down, D: int, F: int, topk_idx, topk_w, x, mid_bf16: 
     return out
 
 
+def moe_plan_dispatch(topk_idx, topk_w, E: int, slots: int):
+    """plan_dispatch (engines/trainer/moe/dispatch.cpp:9-38): (expert_first [E + 1], item_token, item_weight, dropped slots)."""
+    idx = np.ascontiguousarray(topk_idx, np.int32)
+    w = _f32(topk_w)
+    T, Kk = idx.shape
+    first = np.zeros(E + 1, np.int32)
+    tok = np.zeros(T * Kk, np.int32)
+    wt = np.zeros(T * Kk, np.float32)
+    dr = np.zeros(T * Kk, np.int32)
+    i32p = C.POINTER(C.c_int32)
+    lib.orc_moe_plan_dispatch.restype = C.c_int64
+    lib.orc_moe_plan_dispatch.argtypes = [i32p, _f32p, C.c_int64, C.c_int64, C.c_int64, C.c_int64, i32p, i32p, _f32p, i32p]
+    nd = lib.orc_moe_plan_dispatch(idx.ctypes.data_as(i32p), _ptr(w, _f32p), T, Kk, E, slots, first.ctypes.data_as(i32p),
+                                   tok.ctypes.data_as(i32p), _ptr(wt, _f32p), dr.ctypes.data_as(i32p))
+    if nd < 0:
+        raise RuntimeError("oracle plan_dispatch: expert id out of range")
+    n = int(first[E])
+    return first, tok[:n], wt[:n], dr[:nd]
+
+
+def moe_ffn_capacity(fmt, gate, up, down, D: int, F: int, topk_idx, topk_w, slots: int, x, mid_bf16: bool = False,
+                     threads: int = THREADS):
+    """(out [T][D], dropped count): plan_dispatch + gather + expert FFN + combine_expert_outputs (dispatch.cpp:9-78)."""
+    E = len(gate)
+    keep = [np.ascontiguousarray(a, np.uint8) for a in list(gate) + list(up) + list(down)]
+    arr = lambda xs: (_u8p * E)(*[_ptr(a, _u8p) for a in xs])
+    idx = np.ascontiguousarray(topk_idx, np.int32)
+    topk_w = _f32(topk_w)
+    x = _f32(x)
+    T, Kk = idx.shape
+    out = np.empty((T, D), np.float32)
+    i32p = C.POINTER(C.c_int32)
+    lib.orc_moe_ffn_capacity.restype = C.c_int64
+    lib.orc_moe_ffn_capacity.argtypes = [C.c_uint8, C.POINTER(_u8p), C.POINTER(_u8p), C.POINTER(_u8p), C.c_int, C.c_int64, C.c_int64,
+                                         i32p, _f32p, C.c_int64, C.c_int64, C.c_int64, _f32p, _f32p, C.c_int, C.c_int]
+    nd = lib.orc_moe_ffn_capacity(fmt_id(fmt), arr(keep[:E]), arr(keep[E:2 * E]), arr(keep[2 * E:]), E, D, F,
+                                  idx.ctypes.data_as(i32p), _ptr(topk_w, _f32p), T, Kk, slots, _ptr(x, _f32p), _ptr(out, _f32p),
+                                  int(mid_bf16), threads)
+    if nd < 0:
+        raise RuntimeError("oracle moe_ffn_capacity failed")
+    return out, int(nd)
+
+
 def quant4_gemm(w, cb16, act, M: int, N: int, K: int) -> np.ndarray:
     w = np.ascontiguousarray(w, np.uint8)
     cb16 = np.ascontiguousarray(cb16, np.uint16)

@@ -2175,6 +2175,60 @@ int orc_moe_ffn(uint8_t fmt, const uint8_t* const* gate, const uint8_t* const* u
     return 0;
 }
 
+// Capacity-limited dispatch (engines/trainer/moe/dispatch.cpp:9-78).  plan_dispatch (:9-38): slots in (t, k)
+// order join their expert's list while it has fewer than `slots` items, the rest are dropped; gather (:40-60):
+// an expert's rows in list order; combine (:60-78): h[t] += w * y_e[i], experts ascending, items in list order,
+// no test on the sign of w.  expert_first has E + 1 entries; returns the dropped count, or -1 for an expert id
+// outside 0..E-1 (the reference throws).
+int64_t orc_moe_plan_dispatch(const int32_t* idx, const float* w, int64_t T, int64_t Kk, int64_t E, int64_t slots,
+                              int32_t* expert_first, int32_t* item_token, float* item_weight, int32_t* dropped_slot) {
+    std::vector<std::vector<int32_t>> tok((size_t)E);
+    std::vector<std::vector<float>> wt((size_t)E);
+    int64_t nd = 0;
+    for (int64_t t = 0; t < T; ++t)
+        for (int64_t k = 0; k < Kk; ++k) {
+            const int32_t e = idx[t * Kk + k];
+            if (e < 0 || e >= E) return -1;
+            if ((int64_t)tok[(size_t)e].size() < slots) { tok[(size_t)e].push_back((int32_t)t); wt[(size_t)e].push_back(w[t * Kk + k]); }
+            else { if (dropped_slot) dropped_slot[nd] = (int32_t)(t * Kk + k); ++nd; }
+        }
+    int32_t n = 0;
+    for (int64_t e = 0; e < E; ++e) {
+        expert_first[e] = n;
+        for (size_t i = 0; i < tok[(size_t)e].size(); ++i, ++n) { item_token[n] = tok[(size_t)e][i]; item_weight[n] = wt[(size_t)e][i]; }
+    }
+    expert_first[E] = n;
+    return nd;
+}
+
+int64_t orc_moe_ffn_capacity(uint8_t fmt, const uint8_t* const* gate, const uint8_t* const* up, const uint8_t* const* down,
+                             int E, int64_t D, int64_t F, const int32_t* topk_idx, const float* topk_w, int64_t T, int64_t Kk,
+                             int64_t slots, const float* x, float* out, int mid_bf16, int threads) {
+    if (E <= 0 || T <= 0 || Kk <= 0 || slots <= 0 || D % 256 || F % 256) return -1;
+    std::vector<int32_t> first((size_t)E + 1), tok((size_t)(T * Kk));
+    std::vector<float> wts((size_t)(T * Kk));
+    const int64_t nd = orc_moe_plan_dispatch(topk_idx, topk_w, T, Kk, E, slots, first.data(), tok.data(), wts.data(), nullptr);
+    if (nd < 0) return -1;
+    std::fill(out, out + T * D, 0.0f);
+    for (int e = 0; e < E; ++e) {
+        const int64_t p0 = first[(size_t)e], nt = first[(size_t)e + 1] - p0;
+        if (!nt) continue;
+        std::vector<float> bi((size_t)(nt * D)), g((size_t)(nt * F)), u((size_t)(nt * F)), h((size_t)(nt * F)), bo((size_t)(nt * D));
+        for (int64_t i = 0; i < nt; ++i) std::memcpy(&bi[(size_t)(i * D)], x + (int64_t)tok[(size_t)(p0 + i)] * D, (size_t)D * 4);
+        if (orc_matmul(fmt, gate[e], F, D, bi.data(), (int)nt, g.data(), threads)) return -1;
+        if (orc_matmul(fmt, up[e], F, D, bi.data(), (int)nt, u.data(), threads)) return -1;
+        orc_silu_mul(g.data(), u.data(), nt * F, h.data());
+        if (mid_bf16) for (auto& v : h) v = bf16_round(v);
+        if (orc_matmul(fmt, down[e], D, F, h.data(), (int)nt, bo.data(), threads)) return -1;
+        for (int64_t i = 0; i < nt; ++i) {
+            const int64_t t = tok[(size_t)(p0 + i)];
+            const float wgt = wts[(size_t)(p0 + i)];
+            for (int64_t dd = 0; dd < D; ++dd) out[t * D + dd] += wgt * bo[(size_t)(i * D + dd)];
+        }
+    }
+    return nd;
+}
+
 // ---- codebook-LUT GEMM operators, scalar semantics
 // quant4: one packed row per (m, n) pair, activation row indexed by n;
 // nibble k even -> low, odd -> high; codebook = 16 binary16 values.

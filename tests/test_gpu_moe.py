@@ -206,3 +206,31 @@ def test_mlp_step_matches_the_oracle(O, tfq, gpu, fmt, B, xdt, mid):
     assert float(np.abs(y - want).max()) <= tol * float(np.abs(want).max())
     for W in Ws:
         W.close()
+
+
+def test_capacity_dispatch_matches_oracle(O, tfq, gpu):
+    """moe_engine::plan_dispatch / gather / combine (engines/trainer/moe/dispatch.cpp:9-78) through the C ABI."""
+    import torch
+    fmt, E, D, F, T, K, slots = "B32S4", 4, 1024, 2048, 16, 2, 5
+    gate, up, down, hg, hu, hd = _experts(O, tfq, fmt, E, D, F, 900)
+    x = O.rng_normal(11, T * D, 1.0).reshape(T, D)
+    rng = np.random.default_rng(12)
+    idx = rng.integers(0, E, size=(T, K)).astype(np.int32)
+    w = rng.standard_normal((T, K)).astype(np.float32)
+    # the plan alone: the library's host-side lists equal the oracle's
+    for a, b in zip(tfq.moe_plan_dispatch(idx, w, E, slots), O.moe_plan_dispatch(idx, w, E, slots)):
+        assert np.array_equal(a, b)
+    ref, nd_ref = O.moe_ffn_capacity(fmt, hg, hu, hd, D, F, idx, w, slots, x)
+    y, nd = tfq.moe_ffn_capacity(gate, up, down, idx, w, slots, torch.from_numpy(x).to(gpu), mid_dtype=torch.float32)
+    assert nd == nd_ref and nd > 0
+    assert rel_err(y.cpu().numpy(), ref) <= 1e-3
+    # bf16 activations and intermediate
+    xb = O.bf16_round(x)
+    refb, _ = O.moe_ffn_capacity(fmt, hg, hu, hd, D, F, idx, w, slots, xb, mid_bf16=True)
+    yb, _ = tfq.moe_ffn_capacity(gate, up, down, idx, w, slots, torch.from_numpy(xb).to(gpu).bfloat16(), out_dtype=torch.float32)
+    assert rel_err(yb.cpu().numpy(), refb) <= 1e-2
+    # an expert id outside 0..E-1 is an error, as in the reference
+    bad = idx.copy()
+    bad[0, 0] = E
+    with pytest.raises(tfq.TfqError):
+        tfq.moe_ffn_capacity(gate, up, down, bad, w, slots, torch.from_numpy(x).to(gpu))

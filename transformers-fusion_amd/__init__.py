@@ -81,6 +81,8 @@ def _load():
         "tfq_moe_route": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "tfq_moe_workspace_bytes": (sz, [i32, i32, i64, i64]),
         "tfq_moe_ffn": (i32, [vp, vp, vp, i32, vp, vp, i32, i32, vp, i32, vp, i32, i32, vp, sz, vp]),
+        "tfq_moe_plan_dispatch": (i32, [vp, vp, i32, i32, i32, i64, vp, vp, vp, vp, vp]),
+        "tfq_moe_ffn_capacity": (i32, [vp, vp, vp, i32, vp, vp, i32, i32, i64, vp, i32, vp, i32, i32, vp, sz, vp, vp]),
         "tfq_lut4_gemm": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
         "tfq_lut8_gemm": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
         "tfq_lut_gemv_batch": (i32, [i32, vp, vp, C.c_float, vp, vp, i32, i32, i32, vp]),
@@ -481,6 +483,45 @@ def moe_ffn(gate, up, down, topk_idx, topk_w, x, out_dtype=None, mid_dtype=None)
                              x.data_ptr(), _dtype_code(x), y.data_ptr(), _dtype_code(y), mid,
                              ws.data_ptr(), nbytes, _stream()))
     return y
+
+
+def moe_plan_dispatch(topk_idx, topk_w, E: int, slots_per_expert: int):
+    """moe_engine::plan_dispatch on the host side of the library: (expert_first, item_token, item_weight, dropped slots)."""
+    import numpy as np
+    idx = np.ascontiguousarray(topk_idx, np.int32)
+    wts = np.ascontiguousarray(topk_w, np.float32)
+    T, k = idx.shape
+    first = np.zeros(E + 1, np.int32)
+    tok = np.zeros(T * k, np.int32)
+    wt = np.zeros(T * k, np.float32)
+    dr = np.zeros(T * k, np.int32)
+    nd = C.c_int64(0)
+    _check(lib().tfq_moe_plan_dispatch(idx.ctypes.data, wts.ctypes.data, T, k, E, slots_per_expert, first.ctypes.data,
+                                       tok.ctypes.data, wt.ctypes.data, dr.ctypes.data, C.addressof(nd)))
+    n = int(first[E])
+    return first, tok[:n], wt[:n], dr[:nd.value]
+
+
+def moe_ffn_capacity(gate, up, down, topk_idx, topk_w, slots_per_expert: int, x, out_dtype=None, mid_dtype=None):
+    """Capacity-limited MoE FFN (tfq_moe_ffn_capacity): returns (y [T][D], dropped count)."""
+    import numpy as np
+    import torch
+    E = len(gate)
+    idx = np.ascontiguousarray(topk_idx, np.int32)
+    wts = np.ascontiguousarray(topk_w, np.float32)
+    T, k = idx.shape
+    D, F = gate[0].K, gate[0].N
+    x = x.contiguous()
+    y = torch.empty((T, D), dtype=out_dtype or torch.float32, device=x.device)
+    mid = BF16 if (mid_dtype or x.dtype) == torch.bfloat16 else F32
+    nbytes = lib().tfq_moe_workspace_bytes(T, k, D, F)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    arr = lambda ws_: (C.c_void_p * E)(*[w.handle for w in ws_])
+    nd = C.c_int64(0)
+    _check(lib().tfq_moe_ffn_capacity(arr(gate), arr(up), arr(down), E, idx.ctypes.data, wts.ctypes.data, T, k,
+                                      slots_per_expert, x.data_ptr(), _dtype_code(x), y.data_ptr(), _dtype_code(y), mid,
+                                      ws.data_ptr(), nbytes, C.addressof(nd), _stream()))
+    return y, int(nd.value)
 
 
 def lut4_gemm(packed, codebook16, act, M: int, N: int, K: int):

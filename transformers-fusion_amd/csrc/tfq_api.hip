@@ -401,6 +401,49 @@ int tfq_moe_ffn(const tfq_weight_t* const* gate, const tfq_weight_t* const* up, 
                           workspace_bytes, (hipStream_t)stream);
 }
 
+int tfq_moe_plan_dispatch(const int32_t* topk_idx, const float* topk_w, int T, int k, int E, int64_t slots_per_expert,
+                          int32_t* expert_first, int32_t* item_token, float* item_weight, int32_t* dropped_slot,
+                          int64_t* dropped) {
+    if (!topk_idx || !topk_w || !expert_first || !item_token || !item_weight)
+        return fail(TFQ_ERR_ARG, "tfq_moe_plan_dispatch: null pointer");
+    if (T <= 0 || k <= 0) return fail(TFQ_ERR_ARG, "tfq_moe_plan_dispatch: T and k must be positive");
+    std::vector<std::vector<int>> tok;
+    std::vector<std::vector<float>> wt;
+    std::vector<int> dropped_slots;
+    if (int r = moe_plan_dispatch(topk_idx, topk_w, T, k, E, slots_per_expert, tok, wt, &dropped_slots)) return r;
+    int n = 0;
+    for (int e = 0; e < E; ++e) {
+        expert_first[e] = n;
+        for (size_t i = 0; i < tok[(size_t)e].size(); ++i, ++n) {
+            item_token[n] = tok[(size_t)e][i];
+            item_weight[n] = wt[(size_t)e][i];
+        }
+    }
+    expert_first[E] = n;
+    if (dropped_slot)
+        for (size_t i = 0; i < dropped_slots.size(); ++i) dropped_slot[i] = dropped_slots[i];
+    if (dropped) *dropped = (int64_t)dropped_slots.size();
+    return TFQ_OK;
+}
+
+int tfq_moe_ffn_capacity(const tfq_weight_t* const* gate, const tfq_weight_t* const* up, const tfq_weight_t* const* down,
+                         int E, const int32_t* topk_idx, const float* topk_w, int T, int k, int64_t slots_per_expert,
+                         const void* x, int x_dtype, void* y, int y_dtype, int mid_dtype, void* workspace,
+                         size_t workspace_bytes, int64_t* dropped, tfq_stream_t stream) {
+    if (!gate || !up || !down || !topk_idx || !topk_w || !x || !y || !workspace)
+        return fail(TFQ_ERR_ARG, "tfq_moe_ffn_capacity: null pointer");
+    if (E <= 0 || T <= 0 || k <= 0) return fail(TFQ_ERR_ARG, "tfq_moe_ffn_capacity: E, T and k must be positive");
+    if ((x_dtype != TFQ_F32 && x_dtype != TFQ_BF16) || (y_dtype != TFQ_F32 && y_dtype != TFQ_BF16) ||
+        (mid_dtype != TFQ_F32 && mid_dtype != TFQ_BF16))
+        return fail(TFQ_ERR_ARG, "tfq_moe_ffn_capacity: dtype must be TFQ_F32 or TFQ_BF16");
+    for (int e = 0; e < E; ++e)
+        if (!gate[e] || !up[e] || !down[e]) return fail(TFQ_ERR_ARG, "tfq_moe_ffn_capacity: null expert handle");
+    if ((uintptr_t)x % 16 || (uintptr_t)workspace % 256) return fail(TFQ_ERR_ARG, "tfq_moe_ffn_capacity: x must be 16-byte, workspace 256-byte aligned");
+    if (int r = ensure_device()) return r;
+    return launch_moe_ffn_capacity(gate, up, down, E, topk_idx, topk_w, T, k, slots_per_expert, x, x_dtype, y, y_dtype,
+                                   mid_dtype, workspace, workspace_bytes, dropped, (hipStream_t)stream);
+}
+
 size_t tfq_mlp_workspace_bytes(int B, int64_t F) { return B > 0 && F > 0 ? mlp_workspace_bytes(B, F) : 0; }
 
 int tfq_mlp_step(const tfq_weight_t* gate, const tfq_weight_t* up, const tfq_weight_t* down, const void* x, int x_dtype,

@@ -7,6 +7,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <string>
+#include <vector>
 
 #include "../../include/tfq.h"
 
@@ -369,6 +370,12 @@ int launch_moe_route(const float* logits, int T, int E, int k, float* probs, int
 int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E,
                    const int64_t* topk_idx, const float* topk_w, int T, int Ktop, const void* x, int x_dtype,
                    void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes, hipStream_t s);
+int moe_plan_dispatch(const int32_t* topk_idx, const float* topk_w, int T, int Ktop, int E, int64_t slots_per_expert,
+                      std::vector<std::vector<int>>& tok, std::vector<std::vector<float>>& wt, std::vector<int>* dropped_slots);
+int launch_moe_ffn_capacity(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E,
+                            const int32_t* topk_idx, const float* topk_w, int T, int Ktop, int64_t slots_per_expert,
+                            const void* x, int x_dtype, void* y, int y_dtype, int mid_dtype, void* workspace,
+                            size_t workspace_bytes, int64_t* dropped, hipStream_t s);
 // `scratch` (optional, device memory) lets the tile kernel split K over several workgroups per output tile when
 // the tiles alone do not fill the GPU; gemm_scratch_bytes says how much a call would use, gemm_scratch_bound is
 // an upper bound for any matrix with at most `rows` x `cols` outputs (a split never makes more than 256 tiles).

@@ -61,10 +61,11 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__
 
 // out[t][d] = sum over the pairs of token t, in ascending pair (= expert) order, of w[p] * o[p][d];
 // tok_pairs[tok_first[t] .. tok_first[t + 1]) lists them
+// (keep_all: the capacity form adds every kept pair whatever the sign of its weight)
 template <bool OUT_BF16>
 __global__ __launch_bounds__(256) void combine_kernel(void* __restrict__ out, const float* __restrict__ o,
                                                       const int* __restrict__ tok_first, const int* __restrict__ tok_pairs,
-                                                      const float* __restrict__ w, int T, int D) {
+                                                      const float* __restrict__ w, int T, int D, int keep_all) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= (int64_t)T * D) return;
     const int t = (int)(i / D), d = (int)(i - (int64_t)t * D);
@@ -72,7 +73,7 @@ __global__ __launch_bounds__(256) void combine_kernel(void* __restrict__ out, co
     for (int j = tok_first[t]; j < tok_first[t + 1]; ++j) {
         const int p = tok_pairs[j];
         const float wt = w[p];
-        if (wt > 0.0f) acc += wt * o[(int64_t)p * D + d];
+        if (wt > 0.0f || keep_all) acc += wt * o[(int64_t)p * D + d];
     }
     if (OUT_BF16) reinterpret_cast<unsigned short*>(out)[i] = (unsigned short)bf16_rne(acc);
     else reinterpret_cast<float*>(out)[i] = acc;
@@ -201,20 +202,57 @@ int launch_moe_route(const float* logits, int T, int E, int k, float* probs, int
     return hip_fail(hipGetLastError(), "route launch");
 }
 
+namespace {
+int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E,
+            const std::vector<int>& rows, const std::vector<float>& wts, const std::vector<int>& first, bool keep_all,
+            int T, int Ktop, const void* x, int x_dtype, void* y, int y_dtype, int mid_dtype, void* workspace,
+            size_t workspace_bytes, hipStream_t s);
+}  // namespace
+
+// plan_dispatch (engines/trainer/moe/dispatch.cpp:9-38): slots in (token, k) order; a slot joins its expert's
+// list while that list has fewer than slots_per_expert items, otherwise it is dropped.
+int moe_plan_dispatch(const int32_t* topk_idx, const float* topk_w, int T, int Ktop, int E, int64_t slots_per_expert,
+                      std::vector<std::vector<int>>& tok, std::vector<std::vector<float>>& wt,
+                      std::vector<int>* dropped_slots) {
+    if (E <= 0 || slots_per_expert <= 0) return fail(TFQ_ERR_ARG, "moe dispatch: experts and slots per expert must be positive");
+    tok.assign((size_t)E, {});
+    wt.assign((size_t)E, {});
+    for (int t = 0; t < T; ++t)
+        for (int k = 0; k < Ktop; ++k) {
+            const int e = topk_idx[(int64_t)t * Ktop + k];
+            if (e < 0 || e >= E) return fail(TFQ_ERR_ARG, "moe dispatch: expert id outside 0..E-1");
+            if ((int64_t)tok[(size_t)e].size() < slots_per_expert) {
+                tok[(size_t)e].push_back(t);
+                wt[(size_t)e].push_back(topk_w[(int64_t)t * Ktop + k]);
+            } else if (dropped_slots) {
+                dropped_slots->push_back(t * Ktop + k);
+            }
+        }
+    return TFQ_OK;
+}
+
+int launch_moe_ffn_capacity(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E,
+                            const int32_t* topk_idx, const float* topk_w, int T, int Ktop, int64_t slots_per_expert,
+                            const void* x, int x_dtype, void* y, int y_dtype, int mid_dtype, void* workspace,
+                            size_t workspace_bytes, int64_t* dropped, hipStream_t s) {
+    std::vector<std::vector<int>> tok;
+    std::vector<std::vector<float>> wt;
+    std::vector<int> dropped_slots;
+    if (int rc = moe_plan_dispatch(topk_idx, topk_w, T, Ktop, E, slots_per_expert, tok, wt, &dropped_slots)) return rc;
+    std::vector<int> rows, first((size_t)E + 1, 0);
+    std::vector<float> wts;
+    for (int e = 0; e < E; ++e) {
+        rows.insert(rows.end(), tok[(size_t)e].begin(), tok[(size_t)e].end());
+        wts.insert(wts.end(), wt[(size_t)e].begin(), wt[(size_t)e].end());
+        first[(size_t)e + 1] = (int)rows.size();
+    }
+    if (dropped) *dropped = (int64_t)dropped_slots.size();
+    return moe_run(gate, up, down, E, rows, wts, first, true, T, Ktop, x, x_dtype, y, y_dtype, mid_dtype, workspace, workspace_bytes, s);
+}
+
 int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E,
                    const int64_t* topk_idx, const float* topk_w, int T, int Ktop, const void* x, int x_dtype,
                    void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes, hipStream_t s) {
-    const int64_t D = gate[0]->K, F = gate[0]->N;
-    for (int e = 0; e < E; ++e) {
-        if (gate[e]->K != D || gate[e]->N != F || up[e]->K != D || up[e]->N != F || down[e]->K != F || down[e]->N != D)
-            return fail(TFQ_ERR_SHAPE, "moe: expert shapes must be gate/up F x D and down D x F");
-    }
-    if (T > 4096) return fail(TFQ_ERR_SHAPE, "moe: at most 4096 tokens per call");
-    const Workspace ws = carve(workspace, T, Ktop, D, F);
-    if (workspace_bytes < ws.total) return fail(TFQ_ERR_SHAPE, "moe: workspace smaller than tfq_moe_workspace_bytes");
-    const size_t xe_bytes = x_dtype == TFQ_F32 ? 4 : 2;
-    const int64_t nout = (int64_t)T * D;
-
     // Pair lists, built on the host from the caller's routing arrays and uploaded once: per expert
     // the tokens routed to it in ascending token order (one entry per (token, slot), like the
     // reference), and per token its pairs in ascending pair order.
@@ -233,6 +271,24 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
                 }
         first[e + 1] = (int)rows.size();
     }
+    return moe_run(gate, up, down, E, rows, wts, first, false, T, Ktop, x, x_dtype, y, y_dtype, mid_dtype, workspace, workspace_bytes, s);
+}
+
+namespace {
+int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E,
+            const std::vector<int>& rows, const std::vector<float>& wts, const std::vector<int>& first, bool keep_all,
+            int T, int Ktop, const void* x, int x_dtype, void* y, int y_dtype, int mid_dtype, void* workspace,
+            size_t workspace_bytes, hipStream_t s) {
+    const int64_t D = gate[0]->K, F = gate[0]->N;
+    for (int e = 0; e < E; ++e) {
+        if (gate[e]->K != D || gate[e]->N != F || up[e]->K != D || up[e]->N != F || down[e]->K != F || down[e]->N != D)
+            return fail(TFQ_ERR_SHAPE, "moe: expert shapes must be gate/up F x D and down D x F");
+    }
+    if (T > 4096) return fail(TFQ_ERR_SHAPE, "moe: at most 4096 tokens per call");
+    const Workspace ws = carve(workspace, T, Ktop, D, F);
+    if (workspace_bytes < ws.total) return fail(TFQ_ERR_SHAPE, "moe: workspace smaller than tfq_moe_workspace_bytes");
+    const size_t xe_bytes = x_dtype == TFQ_F32 ? 4 : 2;
+    const int64_t nout = (int64_t)T * D;
     const int P = (int)rows.size();  // <= T * Ktop; slots naming an expert outside 0..E-1 are dropped
     const size_t he = mid_dtype == TFQ_BF16 ? 2 : 4;
 
@@ -363,11 +419,12 @@ int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, c
         if (int rc = launch_gemm(down[e], ws.h + (size_t)p0 * F * he, mid_dtype, nt, ws.o + (size_t)p0 * D, TFQ_F32, s, ws.scratch, ws.scratch_bytes)) return rc;
     }
     if (y_dtype == TFQ_BF16)
-        hipLaunchKernelGGL(combine_kernel<true>, dim3((unsigned)((nout + 255) / 256)), dim3(256), 0, s, y, ws.o, d_first, d_pairs, d_w, T, (int)D);
+        hipLaunchKernelGGL(combine_kernel<true>, dim3((unsigned)((nout + 255) / 256)), dim3(256), 0, s, y, ws.o, d_first, d_pairs, d_w, T, (int)D, keep_all ? 1 : 0);
     else
-        hipLaunchKernelGGL(combine_kernel<false>, dim3((unsigned)((nout + 255) / 256)), dim3(256), 0, s, y, ws.o, d_first, d_pairs, d_w, T, (int)D);
+        hipLaunchKernelGGL(combine_kernel<false>, dim3((unsigned)((nout + 255) / 256)), dim3(256), 0, s, y, ws.o, d_first, d_pairs, d_w, T, (int)D, keep_all ? 1 : 0);
     return hip_fail(hipGetLastError(), "moe launch");
 }
+}  // namespace
 
 // Dense SwiGLU feed-forward (Qwen35Engine::mlp_step, src/adapters/tools/qwen35_engine.cpp:662-672): gate and up
 // in one launch where the format has the multi-matrix kernel, the elementwise step, down.  Rows above sixteen go
