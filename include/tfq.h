@@ -161,8 +161,8 @@ int tfq_container_read_tensor(const tfq_container_t* c, const char* name, float*
                               tfq_stream_t stream);
 int tfq_container_read_tensor_host(const tfq_container_t* c, const char* name, float* out, int64_t cap);
 /* Qwen35Engine::resolve (src/adapters/tools/qwen35_engine.cpp:116-150) + upload: the tensor's
- * first rows * cols / 256 blocks as a device-resident matrix.  All of them must be full blocks
- * of one format. */
+ * first rows * cols / 256 blocks as a device-resident matrix.  All of them must be full blocks;
+ * a tensor that mixes formats becomes a mixed-format handle (tfq_weight_upload_mixed). */
 tfq_weight_t* tfq_container_weight(const tfq_container_t* c, const char* name, int64_t rows, int64_t cols);
 
 /* ---- block codec ------------------------------------------------------------
@@ -194,6 +194,14 @@ tfq_weight_t* tfq_weight_upload(uint8_t fmt, int64_t N, int64_t K, const uint8_t
                                 size_t bytes);
 tfq_weight_t* tfq_weight_wrap(uint8_t fmt, int64_t N, int64_t K, const uint8_t* packed_dev,
                               size_t bytes);
+/* A matrix whose blocks carry their own wire ids, as the reference's containers store them (a format byte per
+ * block, include/quant/quant_format.h:15-34) and its engine reads them (decode_block takes the format per block,
+ * src/adapters/tools/qwen35_engine.cpp:19-35).  block_formats has N * K/256 entries in block order, packed_host the
+ * payloads one behind the other, each tfq_block_bytes(format, 256) long.  The handle serves tfq_gemv, tfq_gemm,
+ * tfq_matmul_host and tfq_weight_decode (a general kernel that decodes each block from its own layout; the
+ * single-format handles are the fast path).  tfq_weight_info reports the first block's id. */
+tfq_weight_t* tfq_weight_upload_mixed(int64_t N, int64_t K, const uint8_t* block_formats,
+                                      const uint8_t* packed_host, size_t bytes);
 void tfq_weight_free(tfq_weight_t* w);
 int tfq_weight_info(const tfq_weight_t* w, uint8_t* fmt, int64_t* N, int64_t* K, size_t* bytes);
 /* decoded fp32 matrix [N][K] (device) */

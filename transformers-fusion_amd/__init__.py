@@ -65,6 +65,7 @@ def _load():
         "tfq_decode_blocks_host": (i32, [u8, vp, sz, i64, vp]),
         "tfq_weight_upload": (vp, [u8, i64, i64, vp, sz]),
         "tfq_weight_wrap": (vp, [u8, i64, i64, vp, sz]),
+        "tfq_weight_upload_mixed": (vp, [i64, i64, vp, vp, sz]),
         "tfq_weight_free": (None, [vp]),
         "tfq_weight_info": (i32, [vp, C.POINTER(u8), C.POINTER(i64), C.POINTER(i64), C.POINTER(sz)]),
         "tfq_weight_decode": (i32, [vp, vp, vp]),
@@ -213,6 +214,18 @@ class Weight:
         if not h:
             raise TfqError(lib().tfq_last_error().decode())
         self.handle = C.c_void_p(h)
+
+    @classmethod
+    def mixed(cls, N: int, K: int, block_formats, packed):
+        """A matrix whose blocks carry their own wire ids (tfq_weight_upload_mixed): block_formats uint8 [N * K / 256]
+        (names or ids), packed the concatenated payloads (host array)."""
+        import numpy as np
+        fm = np.ascontiguousarray([fmt_id(f) for f in block_formats], dtype=np.uint8)
+        arr = np.ascontiguousarray(packed, dtype=np.uint8)
+        h = lib().tfq_weight_upload_mixed(N, K, fm.ctypes.data, arr.ctypes.data, arr.size)
+        if not h:
+            raise TfqError(lib().tfq_last_error().decode())
+        return cls(int(fm[0]), N, K, None, handle=h)
 
     def close(self):
         if getattr(self, "handle", None):

@@ -301,6 +301,59 @@ tfq_weight_t* tfq_weight_wrap(uint8_t fmt, int64_t N, int64_t K, const uint8_t* 
     return make_weight("tfq_weight_wrap", fmt, N, K, packed_dev, bytes, false);
 }
 
+tfq_weight_t* tfq_weight_upload_mixed(int64_t N, int64_t K, const uint8_t* block_formats, const uint8_t* packed_host, size_t bytes) {
+    const char* who = "tfq_weight_upload_mixed";
+    if (!block_formats || !packed_host || N <= 0 || K <= 0) { fail(TFQ_ERR_ARG, std::string(who) + ": null pointer or non-positive shape"); return nullptr; }
+    if (K % 256) { fail(TFQ_ERR_SHAPE, std::string(who) + ": K must be a multiple of 256"); return nullptr; }
+    const size_t nblocks = (size_t)N * (size_t)(K / 256);
+    std::vector<uint32_t> off(nblocks);
+    std::vector<BlockLayout> layouts((size_t)kMixedIds);
+    std::vector<MixLayout> tiers(14);
+    std::vector<char> have((size_t)kMixedIds, 0);
+    size_t at = 0;
+    for (size_t b = 0; b < nblocks; ++b) {
+        const int f = block_formats[b];
+        if (f >= kMixedIds) { fail(TFQ_ERR_FORMAT, std::string(who) + ": wire id " + std::to_string(f) + " is not handled"); return nullptr; }
+        if (!have[(size_t)f]) {
+            BlockLayout L{};
+            if (spec_of(f).codec == Codec::None || !block_layout(f, 256, &L)) { fail(TFQ_ERR_FORMAT, std::string(who) + ": wire id " + std::to_string(f) + " is not handled"); return nullptr; }
+            layouts[(size_t)f] = L;
+            if (is_mix(f)) tiers[(size_t)(f - TFQ_Q_MX_3_5)] = mix_layout(f, 256);
+            have[(size_t)f] = 1;
+        }
+        if (at > 0xFFFFFFFFull) { fail(TFQ_ERR_SHAPE, std::string(who) + ": more than 4 GiB of payload"); return nullptr; }
+        off[b] = (uint32_t)at;
+        at += (size_t)layouts[(size_t)f].bytes;
+    }
+    if (at != bytes) { fail(TFQ_ERR_SHAPE, std::string(who) + ": payload is " + std::to_string(bytes) + " bytes, the blocks need " + std::to_string(at)); return nullptr; }
+    if (ensure_device()) return nullptr;
+    tfq_weight_t* w = new (std::nothrow) tfq_weight_t{block_formats[0], N, K, bytes, nullptr, 0, TFQ_LAYOUT_MIXED, true, nullptr, nullptr};
+    if (!w) { fail(TFQ_ERR_NOMEM, std::string(who) + ": out of host memory"); return nullptr; }
+    // one allocation: payloads (+ 16 bytes the decoders' window reads may touch) | offsets | wire ids | layouts
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t o_off = up(bytes + 16), o_fmt = o_off + up(nblocks * 4), o_lay = o_fmt + up(nblocks);
+    const size_t o_tier = o_lay + up(layouts.size() * sizeof(BlockLayout)), total = o_tier + up(tiers.size() * sizeof(MixLayout));
+    w->dev_bytes = total;
+    hipError_t e = hipMalloc(&w->dev, total);
+    if (e == hipSuccess) e = hipMemset(w->dev + bytes, 0, 16);
+    if (e == hipSuccess) e = hipMemcpy(w->dev, packed_host, bytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(w->dev + o_off, off.data(), nblocks * 4, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(w->dev + o_fmt, block_formats, nblocks, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(w->dev + o_lay, layouts.data(), layouts.size() * sizeof(BlockLayout), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(w->dev + o_tier, tiers.data(), tiers.size() * sizeof(MixLayout), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        hip_fail(e, who);
+        if (w->dev) (void)hipFree(w->dev);
+        delete w;
+        return nullptr;
+    }
+    w->mix_off = reinterpret_cast<const uint32_t*>(w->dev + o_off);
+    w->mix_fmt = w->dev + o_fmt;
+    w->mix_layouts = w->dev + o_lay;
+    w->mix_tier_layouts = w->dev + o_tier;
+    return w;
+}
+
 void tfq_weight_free(tfq_weight_t* w) {
     if (!w) return;
     if (w->owns && w->dev) (void)hipFree(w->dev);
@@ -319,6 +372,7 @@ int tfq_weight_info(const tfq_weight_t* w, uint8_t* fmt, int64_t* N, int64_t* K,
 int tfq_weight_decode(const tfq_weight_t* w, float* out, tfq_stream_t stream) {
     if (!w || !out) return fail(TFQ_ERR_ARG, "tfq_weight_decode: null pointer");
     if (int r = ensure_device()) return r;
+    if (w->layout == TFQ_LAYOUT_MIXED) return launch_decode_mixed(w, out, (hipStream_t)stream);
     if (w->layout == TFQ_LAYOUT_WIRE) return launch_decode(w->fmt, w->dev, w->N * (w->K / 256), out, (hipStream_t)stream);
     return launch_decode_tiled(w->fmt, w->dev, w->N, w->K, out, (hipStream_t)stream);
 }

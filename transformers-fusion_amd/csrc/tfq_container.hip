@@ -366,6 +366,28 @@ tfq_weight_t* tfq_container_weight(const tfq_container_t* c, const char* name, i
         fail(TFQ_ERR_SHAPE, std::string("tfq_container_weight: tensor ") + name + " has " + std::to_string(pl.rec.size()) + " blocks, the shape needs " + std::to_string(need));
         return nullptr;
     }
+    bool uniform = true;
+    for (uint64_t b = 1; b < need && uniform; ++b) uniform = pl.fmt[b] == pl.fmt[0];
+    if (!uniform) {
+        // a format byte per block, as decode_block reads it (src/adapters/tools/qwen35_engine.cpp:19-35)
+        std::vector<uint8_t> packed, fmts((size_t)need);
+        try {
+            size_t total = 0;
+            for (uint64_t b = 0; b < need; ++b) total += pl.rec[b].idx_bytes;
+            packed.reserve(total);
+        } catch (const std::bad_alloc&) { fail(TFQ_ERR_NOMEM, "tfq_container_weight: out of host memory"); return nullptr; }
+        for (uint64_t b = 0; b < need; ++b) {
+            const Record& r = pl.rec[b];
+            BlockLayout L{};
+            if (r.weights != 256 || spec_of(pl.fmt[b]).codec == Codec::None || !block_layout(pl.fmt[b], 256, &L) || r.idx_bytes != (uint32_t)L.bytes) {
+                fail(TFQ_ERR_SHAPE, std::string("tfq_container_weight: block ") + std::to_string(b) + " of " + name + " is not a full block of its format");
+                return nullptr;
+            }
+            fmts[(size_t)b] = pl.fmt[b];
+            packed.insert(packed.end(), r.idx, r.idx + r.idx_bytes);
+        }
+        return tfq_weight_upload_mixed(rows, cols, fmts.data(), packed.data(), packed.size());
+    }
     const uint8_t fmt = pl.fmt[0];
     const Spec sp = spec_of(fmt);
     if (sp.codec == Codec::None) { fail(TFQ_ERR_FORMAT, "tfq_container_weight: wire id " + std::to_string(fmt) + " is not handled"); return nullptr; }
@@ -375,7 +397,6 @@ tfq_weight_t* tfq_container_weight(const tfq_container_t* c, const char* name, i
     } catch (const std::bad_alloc&) { fail(TFQ_ERR_NOMEM, "tfq_container_weight: out of host memory"); return nullptr; }
     for (uint64_t b = 0; b < need; ++b) {
         const Record& r = pl.rec[b];
-        if (pl.fmt[b] != fmt) { fail(TFQ_ERR_FORMAT, std::string("tfq_container_weight: tensor ") + name + " mixes wire ids " + std::to_string(fmt) + " and " + std::to_string(pl.fmt[b])); return nullptr; }
         if (r.weights != 256 || r.idx_bytes != (uint32_t)sp.block_bytes) {
             fail(TFQ_ERR_SHAPE, std::string("tfq_container_weight: block ") + std::to_string(b) + " of " + name + " is not a full block of its format");
             return nullptr;

@@ -1053,6 +1053,13 @@ int launch_gemv_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, c
 
 int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
                       void* const* ys, int y_dtype, hipStream_t s) {
+    if (ws[0]->layout == TFQ_LAYOUT_MIXED) {  // blocks of several formats: one launch per matrix
+        for (int m = 0; m < nmat; ++m) {
+            if (ws[m]->layout != TFQ_LAYOUT_MIXED) return fail(TFQ_ERR_SHAPE, "gemv: matrices of one launch must share their layout");
+            if (int rc = launch_gemv_mixed(ws[m], x, x_dtype, B, ys[m], y_dtype, s)) return rc;
+        }
+        return TFQ_OK;
+    }
     if (ws[0]->layout == TFQ_LAYOUT_WIRE) {  // formats without a tiled kernel: one launch per matrix
         for (int m = 0; m < nmat; ++m)
             if (int rc = launch_gemv_generic(ws[m], x, x_dtype, B, ys[m], y_dtype, s)) return rc;

@@ -182,7 +182,113 @@ int batched_mix(const tfq_weight* w, const void* x, int xd, int B, void* y, int 
     return TFQ_OK;
 }
 
+// A matrix whose blocks carry their own wire ids, as a container tensor written with a format byte per block
+// (decode_block takes the format per block: src/adapters/tools/qwen35_engine.cpp:19-35).  Same shape as the
+// kernels above; the block is decoded from its run-time layout.
+__device__ __forceinline__ void decode_mixed_quad(const BlockLayout* layouts, const MixLayout* tiers, int fmt, const uint8_t* p,
+                                                  int lane, float (&w)[4]) {
+    if (is_mix(fmt)) {
+        mix_decode_wave(tiers[fmt - TFQ_Q_MX_3_5], p, (uint32_t)lane, w);
+    } else {
+        const BlockLayout L = layouts[fmt];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) w[t] = decode_weight_short(L, p, (uint32_t)(4 * lane + t));
+    }
+}
+
+template <int BT, bool XF32>
+__global__ __launch_bounds__(256) void gemv_mixed_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ off,
+                                                         const uint8_t* __restrict__ fmts, const BlockLayout* __restrict__ layouts,
+                                                         const MixLayout* __restrict__ tiers, const void* __restrict__ xin,
+                                                         void* __restrict__ yout, int N, int K, int y_bf16) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nblk = K >> 8;
+    for (int row = blockIdx.x * 4 + wave; row < N; row += gridDim.x * 4) {
+        float acc[BT];
+#pragma unroll
+        for (int b = 0; b < BT; ++b) acc[b] = 0.0f;
+        for (int blk = 0; blk < nblk; ++blk) {
+            const size_t bi = (size_t)row * nblk + blk;
+            const int fmt = __builtin_amdgcn_readfirstlane((int)fmts[bi]);
+            float w[4];
+            decode_mixed_quad(layouts, tiers, fmt, W + off[bi], lane, w);
+            const size_t k0 = (size_t)blk * 256 + 4 * lane;
+#pragma unroll
+            for (int b = 0; b < BT; ++b) {
+                float xv[4];
+                if constexpr (XF32) {
+                    const float4 v = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(xin) + (size_t)b * K + k0);
+                    xv[0] = v.x; xv[1] = v.y; xv[2] = v.z; xv[3] = v.w;
+                } else {
+                    const uint2 v = *reinterpret_cast<const uint2*>(reinterpret_cast<const unsigned short*>(xin) + (size_t)b * K + k0);
+                    xv[0] = __uint_as_float(v.x << 16); xv[1] = __uint_as_float(v.x & 0xFFFF0000u);
+                    xv[2] = __uint_as_float(v.y << 16); xv[3] = __uint_as_float(v.y & 0xFFFF0000u);
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[b] = __builtin_fmaf(w[t], xv[t], acc[b]);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            const float v = wave_sum_lane63(acc[b]);
+            if (lane == 63) {
+                if (y_bf16) reinterpret_cast<unsigned short*>(yout)[(size_t)b * N + row] = (unsigned short)bf16_rne(v);
+                else reinterpret_cast<float*>(yout)[(size_t)b * N + row] = v;
+            }
+        }
+    }
+}
+
+// one wavefront per block
+__global__ __launch_bounds__(64) void decode_mixed_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ off,
+                                                          const uint8_t* __restrict__ fmts, const BlockLayout* __restrict__ layouts,
+                                                          const MixLayout* __restrict__ tiers, float* __restrict__ out) {
+    const size_t bi = blockIdx.x;
+    const int lane = threadIdx.x;
+    const int fmt = __builtin_amdgcn_readfirstlane((int)fmts[bi]);
+    float w[4];
+    decode_mixed_quad(layouts, tiers, fmt, W + off[bi], lane, w);
+    *reinterpret_cast<float4*>(out + bi * 256 + 4 * lane) = float4{w[0], w[1], w[2], w[3]};
+}
+
+template <int BT>
+int run_mixed(const tfq_weight* w, const void* x, int xd, void* y, int yd, hipStream_t s) {
+    const int N = (int)w->N, K = (int)w->K;
+    const int grid = (N + 3) / 4 < 4096 ? (N + 3) / 4 : 4096;
+    const BlockLayout* lay = static_cast<const BlockLayout*>(w->mix_layouts);
+    const MixLayout* tiers = static_cast<const MixLayout*>(w->mix_tier_layouts);
+    if (xd == TFQ_F32)
+        hipLaunchKernelGGL((gemv_mixed_kernel<BT, true>), dim3(grid), dim3(256), 0, s, w->dev, w->mix_off, w->mix_fmt, lay, tiers, x, y, N, K, yd == TFQ_BF16);
+    else
+        hipLaunchKernelGGL((gemv_mixed_kernel<BT, false>), dim3(grid), dim3(256), 0, s, w->dev, w->mix_off, w->mix_fmt, lay, tiers, x, y, N, K, yd == TFQ_BF16);
+    return hip_fail(hipGetLastError(), "gemv launch");
+}
+
 }  // namespace
+
+int launch_gemv_mixed(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype, hipStream_t s) {
+    if (w->layout != TFQ_LAYOUT_MIXED) return fail(TFQ_ERR_FORMAT, "gemv: not a mixed-format matrix");
+    const size_t xe = x_dtype == TFQ_F32 ? 4 : 2, ye = y_dtype == TFQ_F32 ? 4 : 2;
+    for (int b0 = 0; b0 < B;) {
+        const int left = B - b0;
+        const int nb = left >= 4 ? 4 : left >= 2 ? 2 : 1;
+        const void* xb = (const uint8_t*)x + (size_t)b0 * w->K * xe;
+        void* yb = (uint8_t*)y + (size_t)b0 * w->N * ye;
+        const int rc = nb == 4 ? run_mixed<4>(w, xb, x_dtype, yb, y_dtype, s) : nb == 2 ? run_mixed<2>(w, xb, x_dtype, yb, y_dtype, s)
+                                                                                        : run_mixed<1>(w, xb, x_dtype, yb, y_dtype, s);
+        if (rc) return rc;
+        b0 += nb;
+    }
+    return TFQ_OK;
+}
+
+int launch_decode_mixed(const tfq_weight* w, float* out, hipStream_t s) {
+    const int64_t nblocks = w->N * (w->K / 256);
+    if (nblocks > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "decode: more than 2^31-1 blocks in one call");
+    hipLaunchKernelGGL(decode_mixed_kernel, dim3((unsigned)nblocks), dim3(64), 0, s, w->dev, w->mix_off, w->mix_fmt,
+                       static_cast<const BlockLayout*>(w->mix_layouts), static_cast<const MixLayout*>(w->mix_tier_layouts), out);
+    return hip_fail(hipGetLastError(), "decode launch");
+}
 
 int launch_gemv_generic(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype, hipStream_t s) {
     if (w->layout != TFQ_LAYOUT_WIRE) return fail(TFQ_ERR_FORMAT, "gemv: generic kernel expects the wire layout");

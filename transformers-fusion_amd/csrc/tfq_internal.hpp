@@ -277,7 +277,7 @@ int ensure_device();  // TFQ_OK once a gfx950 device is current and tables are l
 //            Units are ordered tile-major, so one wavefront reads one unit as a
 //            contiguous run.  For the 4-bit formats this is a permutation of the
 //            wire bytes.
-enum : int { TFQ_LAYOUT_WIRE = 0, TFQ_LAYOUT_TILED16 = 1 };
+enum : int { TFQ_LAYOUT_WIRE = 0, TFQ_LAYOUT_TILED16 = 1, TFQ_LAYOUT_MIXED = 2 };
 
 namespace tfq {
 // header bytes per row and block in the Tiled16 layout; 0 = the format stays in wire order
@@ -311,6 +311,13 @@ struct tfq_weight {
     // (zero between launches).  One call at a time per handle may use them.
     float* split_partial;
     unsigned* split_counters;
+    // TFQ_LAYOUT_MIXED: every block carries its own wire id (the container's per-block format byte).  dev holds
+    // the payloads one behind the other; these device arrays (behind them in the same allocation) give each
+    // block's byte offset and wire id, and the block layout of every wire id.
+    const uint32_t* mix_off = nullptr;
+    const uint8_t* mix_fmt = nullptr;
+    const void* mix_layouts = nullptr;     // BlockLayout[kMixedIds]
+    const void* mix_tier_layouts = nullptr;  // MixLayout[14] of the four-tier ids
 };
 
 namespace tfq {
@@ -344,6 +351,10 @@ int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int 
                       void* const* ys, int y_dtype, hipStream_t s);
 int launch_gemv_generic(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype,
                         hipStream_t s);
+// a matrix whose blocks mix wire ids (TFQ_LAYOUT_MIXED)
+constexpr int kMixedIds = 112;
+int launch_gemv_mixed(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype, hipStream_t s);
+int launch_decode_mixed(const tfq_weight* w, float* out, hipStream_t s);
 // Grouped GEMV: many (matrix, activation rows, output) problems of one format and K in one launch.
 // plan -> fill the host images of the problem table and the workgroup map -> copy both to the
 // device -> launch.  nrows[i] = weight rows of problem i, nrows_x[i] = its activation rows.
