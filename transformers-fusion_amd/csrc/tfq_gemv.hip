@@ -912,6 +912,9 @@ int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t 
         }
     }
     int step = a.x_f32 ? 2 : 4;
+    // A long K leaves LDS room for fewer staged rows: halve the rows per pass until the plan fits
+    // (K = 16640..20480 takes three or two bf16 rows, one fp32 row up to 32768, one bf16 row up to 61440).
+    while (step > 1 && plan_gemv4<FMT>(a, a.x_f32 ? 2 * step : step).lds == 0) step >>= 1;
     if constexpr (kTwoSets<FMT>) {
         if (!a.x_f32 && B > 4) {
             for (int rows = kWide<FMT> ? 16 : 8; rows > 4; rows >>= 1)

@@ -187,7 +187,8 @@ BlockRowMatmul::~BlockRowMatmul() { tfq_weight_free(handle_); }
 
 void BlockRowMatmul::gemm(const float* X, float* Y, int B) const {
     if (!handle_ || !X || !Y || B <= 0 || B > MAX_BATCH) return;
-    tfq_matmul_host(handle_, X, Y, B);
+    // the reference's gemm has no error channel; a product that could not run leaves zeros, not stale memory
+    if (tfq_matmul_host(handle_, X, Y, B) != TFQ_OK) std::memset(Y, 0, (size_t)B * (size_t)rows_ * sizeof(float));
 }
 
 void BlockRowMatmul::mlp_step(const BlockRowMatmul& gate, const BlockRowMatmul& up, const BlockRowMatmul& down,
