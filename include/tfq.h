@@ -276,23 +276,26 @@ int tfq_mlp_step(const tfq_weight_t* gate, const tfq_weight_t* up, const tfq_wei
  *
  * A phase multiplies up to four matrices (one format per chain: B32S4 or Q_G_4; equal K inside
  * a phase, K <= 14336) with the same B <= 2 activation rows.
- *   x          device pointer [B][K] (x_dtype), or NULL: the result of the previous phase, which
- *              is the concatenation of its outputs [B][N0 + N1 + ...] (its first K columns are
- *              used), the SwiGLU product [B][N], or the updated residual rows
- *   x_depends  set when a non-NULL x is written by an earlier phase of the same chain (for
- *              example the residual buffer): the phase then waits for the phase before it
+ *   x          first phase: device pointer [B][K] (x_dtype).  Every later phase: NULL; it reads the
+ *              result of the phase before it, which is the concatenation of that phase's outputs
+ *              [B][N0 + N1 + ...] (its first K columns are used), the SwiGLU product [B][N], or the
+ *              updated residual rows.  (Results travel between workgroups as values that carry the
+ *              launch and phase they belong to, so a reader needs no barrier; a buffer of the
+ *              caller's cannot carry such marks, hence no external x after the first phase.)
  *   x_op       TFQ_CHAIN_X_PLAIN, or TFQ_CHAIN_X_RMSNORM: x * rsqrt(mean(x^2) + eps) * gamma
  *              (gamma_plus_one: * (1 + gamma), the reference's form) before the product
  *   y_op       TFQ_CHAIN_Y_PLAIN; TFQ_CHAIN_Y_SWIGLU: two matrices (gate, up), result =
  *              silu(gate x) * (up x); TFQ_CHAIN_Y_RESIDUAL: one matrix, residual[B][N] += W x in
- *              place, and the sum is the phase's result
+ *              place, and the sum is the phase's result (one residual buffer per chain)
  *   y[i]       device output [B][N_i] of matrix i (y_dtype; fp32 for SwiGLU), or NULL when only
  *              the next phase reads the result
  * Activations are rounded to bf16 before every product (accumulation and elementwise steps in
- * fp32), as in tfq_gemv with bf16 x.  The chain owns device memory for its tables, counters and
- * intermediate results: runs of ONE chain must not overlap in time (one stream).  The handles and
- * buffers named at creation must stay alive.  tfq_chain_check, called after the stream has been
- * synchronised, reports a run whose internal waits ran out (TFQ_ERR_DEVICE) and clears that state. */
+ * fp32), as in tfq_gemv with bf16 x; with RMSNorm the rounding is of x * gamma and the factor
+ * rsqrt(...) multiplies the finished sums.  The chain owns device memory for its tables, counters
+ * and intermediate results: runs of ONE chain must not overlap in time (one stream).  The handles
+ * and buffers named at creation must stay alive.  At most 128 phases.  tfq_chain_check, called
+ * after the stream has been synchronised, reports a run whose internal waits ran out
+ * (TFQ_ERR_DEVICE; every wait in the kernel is bounded) and clears that state. */
 enum { TFQ_CHAIN_X_PLAIN = 0, TFQ_CHAIN_X_RMSNORM = 1 };
 enum { TFQ_CHAIN_Y_PLAIN = 0, TFQ_CHAIN_Y_SWIGLU = 1, TFQ_CHAIN_Y_RESIDUAL = 2 };
 typedef struct tfq_chain_phase {
@@ -300,7 +303,6 @@ typedef struct tfq_chain_phase {
     int count;
     const void* x;
     int x_dtype;
-    int x_depends;
     int x_op;
     const float* gamma;
     float eps;

@@ -282,7 +282,7 @@ class Weight:
 class _ChainPhase(C.Structure):
     """tfq_chain_phase_t (include/tfq.h)."""
     _fields_ = [("w", C.c_void_p * 4), ("count", C.c_int), ("x", C.c_void_p), ("x_dtype", C.c_int),
-                ("x_depends", C.c_int), ("x_op", C.c_int), ("gamma", C.c_void_p), ("eps", C.c_float),
+                ("x_op", C.c_int), ("gamma", C.c_void_p), ("eps", C.c_float),
                 ("gamma_plus_one", C.c_int), ("y_op", C.c_int), ("y", C.c_void_p * 4), ("y_dtype", C.c_int),
                 ("residual", C.c_void_p)]
 
@@ -295,7 +295,7 @@ class Chain:
     """A sequence of dependent matrix-vector products in one persistent launch (tfq_chain_*).
 
     phases: list of dicts with keys
-      w (list of Weight), x (tensor [B][K] or None = the previous phase's result), x_depends (bool),
+      w (list of Weight), x (tensor [B][K] for the first phase; None afterwards = the previous phase's result),
       x_op (X_PLAIN / X_RMSNORM), gamma (fp32 tensor), eps, gamma_plus_one,
       y_op (Y_PLAIN / Y_SWIGLU / Y_RESIDUAL), y (list of tensors or None), residual (fp32 tensor [B][N]).
     The tensors and Weight objects are kept alive by the chain."""
@@ -315,7 +315,6 @@ class Chain:
                 d.x = x.data_ptr()
                 d.x_dtype = _dtype_code(x)
                 self._keep.append(x)
-            d.x_depends = 1 if ph.get("x_depends") else 0
             d.x_op = ph.get("x_op", X_PLAIN)
             g = ph.get("gamma")
             if g is not None:

@@ -4,31 +4,37 @@
 // rmsnorm -> q/k/v -> ... -> o -> residual -> rmsnorm -> gate/up -> silu*up -> down -> residual
 // (Qwen35Engine::append_token, src/adapters/tools/qwen35_engine.cpp:807-835; mlp_step :662-672; rmsnorm :46-51).
 // Launched one by one, every product pays a launch boundary and a cold start of the weight stream.  Here the
-// whole sequence ("phases") runs in one launch of 256 resident workgroups, one per compute unit:
+// whole sequence ("phases") runs in one launch of 256 resident workgroups of 16 wavefronts, one per compute unit:
 //
-//   * weights do not depend on activations, so each workgroup streams ITS share of every phase's packed
-//     weights, in phase order, through a ring of unit slots in LDS (global -> LDS copies that bypass the
-//     registers), and keeps doing so while the arithmetic waits for a dependency;
-//   * one or two LOADER wavefronts per workgroup issue those copies and publish a slot once its copy has
-//     landed; the other CONSUMER wavefronts never touch global memory while they multiply: they take units from
-//     the ring in a fixed round-robin order (deterministic results), with the arithmetic of gemv4_kernel
-//     (block-diagonal bf16 MFMA, scales applied to group sums in fp32);
-//   * a phase's result is written with device-scope stores; when every store of a workgroup has completed it
-//     counts its arrival on one of 16 counters (256 bytes apart, so that 256 arrivals do not queue on one
-//     memory channel), and the next phase's activations are read with device-scope loads once all counters
-//     show the phase complete.  No fence, no cache write-back or invalidation.
-//   * the elementwise steps between the products ride in the staging and the epilogue: RMSNorm while the
-//     activations are staged, silu(gate) * up and the residual addition where the outputs are written.
+//   * Weights do not depend on activations.  Wavefront w of a workgroup owns the block columns w, w + 16, ... of
+//     the workgroup's 16-row tiles in every phase and streams those units, in phase order, through a private ring
+//     of LDS slots with global -> LDS copies that bypass the registers.  The copies run a few units ahead of
+//     the arithmetic and keep running across phase boundaries, so the stream does not stop while a phase waits
+//     for its input.  A wavefront's own wait counter says when a slot has landed: no flags, no barrier.
+//   * Owning block columns means owning a slice of the activations: a wavefront builds the MFMA A fragments of
+//     its column once per phase, in registers, and multiplies them with every tile (the arithmetic of
+//     gemv4_kernel: block-diagonal bf16 MFMA, scales applied to group sums in fp32).
+//   * Results travel between phases as TAGGED values: every element of an intermediate vector is stored with the
+//     tag of its phase and launch beside it in one naturally aligned store ((bf16, tag16) in four bytes or
+//     (fp32, tag32) in eight), with device scope.  A consumer simply loads its slice with device-scope loads
+//     until every tag is the expected one.  There is no arrival counter, no fence, no wait for store
+//     acknowledgements and no grid-wide barrier; a wavefront starts a phase as soon as ITS 256 inputs exist.
+//   * The wavefront that finishes a phase last in its workgroup adds the sixteen partial sums per output in
+//     wavefront order (deterministic), applies the epilogue (silu(gate) * up, residual addition, the RMSNorm
+//     factor of the input), and stores.  RMSNorm is applied as x * (1 + gamma) before the product and
+//     1 / sqrt(mean(x^2) + eps) after it: the factor is a scalar per row, so no wavefront waits for the others'
+//     slices of x before it starts.
 //
 // Every wait is bounded: a wait that runs out sets an error word and an abort flag that every loop tests, so
-// the grid always drains.  The last workgroup to finish puts the counters back to zero for the next launch.
+// the grid always drains.  The tag carries a launch counter that the last workgroup to finish advances, so
+// values left by an earlier launch are never taken for new ones.
 
+#include <algorithm>
 #include <atomic>
-#include <mutex>
+#include <cstddef>
 #include <vector>
 
 #include "tfq_gemv_common.hpp"
-
 
 namespace tfq {
 
@@ -38,50 +44,39 @@ using namespace gemv_detail;
 
 constexpr int kWG = 256;         // workgroups of a launch = compute units of an MI355X
 constexpr int kWaves = 16;       // wavefronts per workgroup
-constexpr int kLoaders = 2;      // of which loaders (one is not enough: 47 against 40 us per Llama-3-8B layer)
 constexpr int kMaxPhases = 128;  // phases per launch
 constexpr int kMaxSlot = 2;      // activation rows (bf16) per chain
 constexpr int kMaxTiles = 8;     // 16-row tiles of one workgroup in one phase (both segments)
-constexpr int kCounters = 16, kCounterStride = 64;  // arrival counters, dwords apart
-constexpr unsigned kSpinLimit = 1u << 22;
+constexpr unsigned kSpinLimit = 1u << 20;
 
 enum : int { XOP_NONE = 0, XOP_RMSNORM = 1 };
 enum : int { YOP_NONE = 0, YOP_SWIGLU = 1, YOP_RESIDUAL = 2 };
+// how a phase's input is stored
+enum : int { XK_PLAIN_BF16 = 0, XK_PLAIN_F32 = 1, XK_TAGGED_BF16 = 2, XK_TAGGED_F32 = 3 };
 
-// What every workgroup needs to know about a phase.
-struct ChainPhase {
-    const void* x;       // activations [nslot][x_stride]
-    const float* gamma;  // RMSNorm gain, or null
-    float* residual;     // YOP_RESIDUAL: [nslot][n_result], updated in place
-    void* link;          // the phase's result for a later phase ([nslot][n_result], link_dtype), or null
-    int K, nslot, x_dtype, x_stride;
-    int x_op, y_op, y_dtype, link_dtype;
-    int n_result, dep, gamma_plus_one, pad;
-    float eps, pad2;
+// One phase as a workgroup sees it: 40 dwords, copied to LDS when the kernel starts.
+struct ChainEntry {
+    const uint8_t* w[2];   // first unit of each segment's first tile (segment: a run of tiles of one matrix)
+    void* y[2];            // the segment's matrix output, element (0, 0), or null
+    const void* x;         // input vector [nslot][x_stride]
+    const float* gamma;    // RMSNorm gain or null
+    void* link;            // tagged result for the next phase, or null
+    float* residual;       // YOP_RESIDUAL: the caller's residual rows [nslot][n_result] (plain fp32, updated)
+    const void* hprev;     // YOP_RESIDUAL: tagged (fp32, tag) copy of the residual rows as the previous residual phase left them, or null (then `residual` is read)
+    int T[2], row0[2], nrows[2], res0[2];
+    int nb, x_kind, x_stride, x_op;
+    int y_op, y_dtype, link_kind, n_result;
+    int x_tag_phase, hprev_tag_phase, gamma_plus_one;
+    float eps;
+    int pad[2];
 };
-static_assert(sizeof(ChainPhase) == 88, "ChainPhase layout");
-
-// The share of one workgroup in one phase: up to two runs of 16-row tiles ("segments"; two matrices of a fused
-// launch, or the gate and up tiles of the same rows for SwiGLU).
-struct ChainWg {
-    const uint8_t* w[2];  // first unit of the segment's first tile
-    void* y[2];           // the segment's matrix output, element (0, 0), or null
-    int T[2];             // tiles
-    int row0[2];          // first row inside the matrix
-    int nrows[2];         // rows of the matrix
-    int res0[2];          // index of the segment's first row inside the phase result
-};
-static_assert(sizeof(ChainWg) == 64, "ChainWg layout");
+constexpr int kEntryWords = 40;
+static_assert(sizeof(ChainEntry) == kEntryWords * 4, "ChainEntry layout");
 
 struct ChainArgs {
-    const ChainPhase* phases;
-    const ChainWg* wgs;   // [nph][kWG]
-    unsigned* sync;       // kCounters counters kCounterStride dwords apart, then [1024] finish, [1025] error
-    int nph;
-    int ring;             // unit slots in the LDS ring
-    int ncols_max;        // block columns of the widest phase
-    int nslot;            // activation rows of the chain (1 or 2)
-    int tmax;             // most tiles (both segments) any workgroup has in any phase
+    const ChainEntry* entries;  // [nph][kWG]
+    unsigned* sync;             // [0] launch counter, [1] finished workgroups, [2] error bits
+    int nph, depth, nslot, tmax;
     unsigned spin_limit;
 };
 
@@ -96,30 +91,14 @@ __device__ __forceinline__ unsigned lds_get(const unsigned* p) {
 }
 __device__ __forceinline__ void lds_set(unsigned* p, unsigned v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
 
-// device-scope accesses: they go past the caches that are private to a part of the chip
-__device__ __forceinline__ u32x4_t load_dev16(const void* p) {
-    u32x4_t v;
-    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
-    return v;
-}
-__device__ __forceinline__ float load_dev_f32(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ void store_dev_f32(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ void store_dev_u16(unsigned short* p, unsigned short v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-
-// 16 bytes per lane, global memory -> LDS without passing the registers: lane l's piece lands at LDS byte
-// lds_base + OFF + 16 l, read from base + OFF + lane_off (the instruction's offset field moves both addresses).
-// lds_base and base are wave-uniform.
-template <int OFF>
-__device__ __forceinline__ void lds_copy16(uint32_t lds_base, uint32_t lane_off, const uint8_t* base) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3 nt" ::"s"(lds_base), "v"(lane_off), "s"(base), "n"(OFF) : "memory");
-}
-
-// One unit (NCODE pieces of 1 KB and a header piece of 16 * HV lanes) into a ring slot, M0 written once; the
-// header copy runs with the upper lanes switched off, so that it writes 256 (512) bytes of LDS only.
-template <int NCODE, int HV>
+// One unit (two pieces of 1 KB and a header piece of 16 * HV lanes) global -> LDS without passing the registers:
+// lane l's 16 bytes of a piece land at LDS byte lds_base + piece offset + 16 l (the instruction's offset field
+// moves both addresses); the header copy runs with the upper lanes switched off, so it writes 256 (512) bytes.
+template <int HV>
 __device__ __forceinline__ void lds_copy_unit(uint32_t lds_base, uint32_t lane_off, const uint8_t* base) {
     unsigned long long saved;
-    if constexpr (NCODE == 2 && HV == 1) {
+    static_assert(HV == 1 || HV == 2, "unit shapes served here");
+    if constexpr (HV == 1) {
         asm volatile(
             "s_mov_b32 m0, %1\n\ts_nop 0\n\t"
             "global_load_lds_dwordx4 %2, %3 offset:0 nt\n\t"
@@ -128,7 +107,7 @@ __device__ __forceinline__ void lds_copy_unit(uint32_t lds_base, uint32_t lane_o
             "global_load_lds_dwordx4 %2, %3 offset:2048 nt\n\t"
             "s_mov_b64 exec, %0"
             : "=&s"(saved) : "s"(lds_base), "v"(lane_off), "s"(base) : "memory");
-    } else if constexpr (NCODE == 2 && HV == 2) {
+    } else {
         asm volatile(
             "s_mov_b32 m0, %1\n\ts_nop 0\n\t"
             "global_load_lds_dwordx4 %2, %3 offset:0 nt\n\t"
@@ -137,486 +116,383 @@ __device__ __forceinline__ void lds_copy_unit(uint32_t lds_base, uint32_t lane_o
             "global_load_lds_dwordx4 %2, %3 offset:2048 nt\n\t"
             "s_mov_b64 exec, %0"
             : "=&s"(saved) : "s"(lds_base), "v"(lane_off), "s"(base) : "memory");
-    } else {
-        static_assert(NCODE == 4 && HV == 1, "unit shapes of the Tiled16 layout");
-        asm volatile(
-            "s_mov_b32 m0, %1\n\ts_nop 0\n\t"
-            "global_load_lds_dwordx4 %2, %3 offset:0 nt\n\t"
-            "global_load_lds_dwordx4 %2, %3 offset:1024 nt\n\t"
-            "global_load_lds_dwordx4 %2, %3 offset:2048 nt\n\t"
-            "global_load_lds_dwordx4 %2, %3 offset:3072 nt\n\t"
-            "s_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffff\n\t"
-            "global_load_lds_dwordx4 %2, %3 offset:4096 nt\n\t"
-            "s_mov_b64 exec, %0"
-            : "=&s"(saved) : "s"(lds_base), "v"(lane_off), "s"(base) : "memory");
     }
 }
 
-// waits until the oldest of `outstanding` (1..K) units in flight, LOADS copies each, has landed
-template <int LOADS, int K>
-__device__ __forceinline__ void wait_oldest(int outstanding) {
-    if constexpr (K >= 1) {
-        if (outstanding == K) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS * (K - 1)) : "memory");
-        else wait_oldest<LOADS, K - 1>(outstanding);
-    }
-}
+__device__ __forceinline__ unsigned make_tag(unsigned epoch, int phase) { return 0x8000u | ((epoch & 0x7Fu) << 8) | (unsigned)(phase + 1); }
 
-// LDS words of control state
-enum : int { C_ABORT = 0, C_SYNC = 1, C_DEP = 2, C_SUMSQ = 4 /* .. +2*15 */, C_WORDS = 40 };
+// LDS control words
+// (a wavefront without work in a phase runs ahead, so arrivals are counted per phase: word C_WORDS + p)
+enum : int { C_ABORT = 0, C_FINISHED = 2, C_WORDS = 8 };
 
-template <int FMT, int NL>
+template <int FMT, int D>
 __global__ __launch_bounds__(1024) void chain_kernel(ChainArgs a) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
+    static_assert(F::GS == 32 && F::NP == 1, "one nibble plane, groups of 32");
     constexpr int UB = tiled_unit_bytes(FMT);
-    constexpr int NCODE = 2 * F::NP;         // 1 KB code pieces of a unit
-    constexpr int LOADS = NCODE + 1;         // copies per unit (the header piece is 16 * HB = 256 or 512 bytes)
-    // units in flight per loader (the hardware counter holds 63 copies).  One wavefront with 8 units in flight
-    // streams 6.2 TB/s on MI355X, two with 8 each 6.8 TB/s; more in flight gains nothing and makes every other
-    // memory access of the compute unit wait longer.
-    constexpr int Q = 63 / LOADS < 8 ? 63 / LOADS : 8;
-    constexpr int NC = kWaves - NL;          // consumer wavefronts
-    constexpr int NG = F::NG, PER = NG / 2;
-    static_assert(F::HV == 1 || F::HV == 2, "header of one or two 16-byte pieces per row");
+    constexpr int LOADS = 3;  // copies per unit
+    constexpr int NG = 8, PER = 4;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = uni(tid >> 6);
     const int b = blockIdx.x;
-    const int nph = a.nph, R = a.ring;
+    const int nph = a.nph, nslot = a.nslot, tmax = a.tmax;
 
-    // ---- LDS: ring | activations | cells | slot states | phase table | control
-    uint8_t* const ring = reinterpret_cast<uint8_t*>(smem);
-    const int nslot = a.nslot, tmax = a.tmax;
-    const int col_stride = nslot * 32 + NG;  // uint4 per block column: A entries [slot][32] + sums [4][NG] floats
-    uint4* const xreg = reinterpret_cast<uint4*>(ring + (size_t)R * UB);
-    uint4* const zero4 = xreg + (size_t)a.ncols_max * col_stride;   // four zero entries
-    float* const cells = reinterpret_cast<float*>(zero4 + 4);       // [NC][tmax][nslot][16]
-    unsigned* const ready_seq = reinterpret_cast<unsigned*>(cells + NC * tmax * nslot * 16);
-    unsigned* const free_seq = ready_seq + R;
-    int* const lph = reinterpret_cast<int*>(free_seq + R);          // [nph][8]: w0 lo, hi, w1 lo, hi, T0, T1, nb, first sequence number
-    unsigned* const ctl = reinterpret_cast<unsigned*>(lph + nph * 8);
+    // ---- LDS: rings [16][D][UB] | bounce [16][nslot * 512 + 128 bytes] | cells [2][16][tmax][nslot][16] f32 |
+    //          sums of squares [2][16][2] f32 | phase table [nph][40] | control
+    uint8_t* const rings = reinterpret_cast<uint8_t*>(smem);
+    const int bounce_bytes = nslot * 512 + 128;
+    uint8_t* const bounce = rings + (size_t)kWaves * D * UB + (size_t)wave * bounce_bytes;
+    float* const cells = reinterpret_cast<float*>(rings + (size_t)kWaves * D * UB + (size_t)kWaves * bounce_bytes);
+    const int cells_per_phase = kWaves * tmax * nslot * 16;
+    float* const ssq = cells + 2 * cells_per_phase;
+    int* const table = reinterpret_cast<int*>(ssq + 2 * kWaves * 2);
+    unsigned* const ctl = reinterpret_cast<unsigned*>(table + nph * kEntryWords);
 
-    for (int i = tid; i < 2 * R; i += 1024) ready_seq[i] = 0;
-    for (int i = tid; i < C_WORDS; i += 1024) ctl[i] = 0;
-    if (tid < 4) zero4[tid] = uint4{0, 0, 0, 0};
-    if (tid < nph) {
-        const ChainWg g = a.wgs[(size_t)tid * kWG + b];
-        int* e = lph + tid * 8;
-        e[0] = (int)(unsigned)(unsigned long long)g.w[0]; e[1] = (int)(unsigned)((unsigned long long)g.w[0] >> 32);
-        e[2] = (int)(unsigned)(unsigned long long)g.w[1]; e[3] = (int)(unsigned)((unsigned long long)g.w[1] >> 32);
-        e[4] = g.T[0]; e[5] = g.T[1];
-        e[6] = a.phases[tid].K >> 8;
-        e[7] = 0;
+    for (int i = tid; i < nph * kEntryWords; i += 1024) {
+        const int ph = i / kEntryWords, word = i - ph * kEntryWords;
+        table[i] = reinterpret_cast<const int*>(a.entries + ((size_t)ph * kWG + b))[word];
     }
-    __syncthreads();
-    if (tid == 0) {  // first sequence number of every phase
-        int seq = 0;
-        for (int p = 0; p < nph; ++p) {
-            lph[p * 8 + 7] = seq;
-            seq += (lph[p * 8 + 4] + lph[p * 8 + 5]) * lph[p * 8 + 6];
-        }
-    }
-    __syncthreads();
+    if (tid < C_WORDS + nph) ctl[tid] = 0;
+    __syncthreads();  // the only workgroup barrier of the kernel
+
     const unsigned spin_limit = a.spin_limit;
+    const unsigned epoch = uni(__hip_atomic_load(a.sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
     auto aborted = [&]() __attribute__((always_inline)) { return lds_get(ctl + C_ABORT) != 0u; };
     auto give_up = [&](unsigned code) __attribute__((always_inline)) {
         if (lane == 0) {
             lds_set(ctl + C_ABORT, 1u);
-            __hip_atomic_fetch_or(a.sync + 1025, code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_fetch_or(a.sync + 2, code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     };
+    auto entry = [&](int p) __attribute__((always_inline)) { return reinterpret_cast<const ChainEntry*>(table + p * kEntryWords); };
+    auto tget = [&](int p, int word) __attribute__((always_inline)) { return uni(table[p * kEntryWords + word]); };
+    // dword offsets inside a ChainEntry
+    constexpr int E_W0 = 0, E_W1 = 2, E_T0 = 18, E_T1 = 19, E_NB = 26;
+    static_assert(offsetof(ChainEntry, T) == E_T0 * 4 && offsetof(ChainEntry, nb) == E_NB * 4 && offsetof(ChainEntry, w) == 0, "entry offsets");
 
-    if (wave >= NC) {
-        // =================================================================== loader
-        const int lid = wave - NC;
-        const uint32_t ring_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)ring;
-        const uint32_t off_c = 16u * lane;
-        int outstanding = 0;
-        int m_slot = lid % R;             // slot and sequence number of the oldest copy not yet published
-        unsigned m_seq = (unsigned)lid;
-        auto publish_oldest = [&]() __attribute__((always_inline)) {
-            if (lane == 0) lds_set(ready_seq + m_slot, m_seq + 1u);
-            m_seq += NL;
-            m_slot += NL;
-            if (m_slot >= R) m_slot -= R;
-            --outstanding;
-        };
-        auto drain = [&]() __attribute__((always_inline)) {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            while (outstanding > 0) publish_oldest();
-        };
-        bool stop = false;
-        for (int p = 0; p < nph && !stop; ++p) {
-            const int* e = lph + p * 8;
-            const unsigned long long wseg[2] = {((unsigned long long)uni((unsigned)e[1]) << 32) | uni((unsigned)e[0]),
-                                                ((unsigned long long)uni((unsigned)e[3]) << 32) | uni((unsigned)e[2])};
-            const int nb = uni(e[6]), seq0 = uni(e[7]);
-            const int useg[2] = {uni(e[4]) * nb, uni(e[5]) * nb};  // units of the two segments
-            // units in memory order: segment by segment, tile by tile, block columns inside (contiguous bytes)
-            for (int sg = 0; sg < 2 && !stop; ++sg) {
-                const int first = sg ? useg[0] : 0;  // unit index inside the phase
-                int j = first + (((lid - seq0 - first) % NL + NL) % NL);  // this loader's first unit of the segment
-                int count = j < first + useg[sg] ? (first + useg[sg] - j + NL - 1) / NL : 0;
-                const uint8_t* ptr = (const uint8_t*)wseg[sg] + (size_t)(j - first) * UB;
-                unsigned g = (unsigned)(seq0 + j);
-                int slot = (int)(g % (unsigned)R);
-                while (count > 0) {
-                    // how many of the next units have a free slot?  Lane i looks at the i-th one.
-                    int nfree;
-                    {
-                        const unsigned gi = g + (unsigned)(lane * NL);
-                        const int si = (int)(gi % (unsigned)R);
-                        bool fr = lane < count && lane < 32;
-                        if (fr && gi >= (unsigned)R)
-                            fr = (int)(__hip_atomic_load(free_seq + si, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) - (gi - (unsigned)R + 1u)) >= 0;
-                        const unsigned long long m = __builtin_amdgcn_ballot_w64(fr);
-                        nfree = (int)__builtin_ctzll(~m);
-                    }
-                    if (nfree == 0) {
-                        // The ring is full.  Copies already in flight are published one by one while there is
-                        // nothing else to do, but not at once: where the consumers set the pace a slot comes
-                        // free within a few polls, and waiting for the youngest copy would leave one unit in flight.
-                        const unsigned need = g - (unsigned)R + 1u;
-                        unsigned polls = 0;
-                        while ((int)(lds_get(free_seq + slot) - need) < 0) {
-                            ++polls;
-                            if ((polls & 15u) == 0 && outstanding > 0) {
-                                wait_oldest<LOADS, Q>(outstanding);
-                                publish_oldest();
-                            } else {
-                                __builtin_amdgcn_s_sleep(1);
-                            }
-                            if ((polls & 63u) == 0 && (aborted() || polls > spin_limit)) { stop = true; break; }
-                        }
-                        if (stop) { if (!aborted()) give_up(1u); break; }
-                        nfree = 1;
-                    }
-                    count -= nfree;
-                    for (; nfree > 0; --nfree) {
-                        lds_copy_unit<NCODE, F::HV>(uni(ring_lds + (uint32_t)slot * UB), off_c, uni_ptr(ptr));
-                        ptr += (size_t)NL * UB;
-                        g += NL;
-                        slot += NL;
-                        if (slot >= R) slot -= R;
-                        ++outstanding;
-                        if (outstanding == Q) {
-                            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS * (Q - 1)) : "memory");
-                            publish_oldest();
-                        }
-                    }
-                }
+    // ---- the copy cursor: this wavefront's units in the order it will use them (phase, block column, tile)
+    const uint32_t ring_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)(rings + (size_t)wave * D * UB);
+    const uint32_t off_c = 16u * lane;
+    int f_p = -1, f_col = 0, f_t = 0, f_T0 = 0, f_T2 = 0, f_nb = 0;
+    unsigned long long f_w0 = 0, f_w1 = 0;
+    // something valid to read again once the cursor has run past the end
+    const uint8_t* f_last = (const uint8_t*)(((unsigned long long)(unsigned)tget(0, E_W0 + 1) << 32) | (unsigned)tget(0, E_W0));
+    bool f_end = false;
+    auto f_next_phase = [&]() __attribute__((always_inline)) {
+        // moves to the first unit of the next phase in which this wavefront has one
+        for (;;) {
+            ++f_p;
+            if (f_p >= nph) { f_end = true; return; }
+            f_T0 = tget(f_p, E_T0);
+            f_T2 = f_T0 + tget(f_p, E_T1);
+            f_nb = tget(f_p, E_NB);
+            if (f_T2 > 0 && wave < f_nb) break;
+        }
+        f_w0 = ((unsigned long long)(unsigned)tget(f_p, E_W0 + 1) << 32) | (unsigned)tget(f_p, E_W0);
+        f_w1 = ((unsigned long long)(unsigned)tget(f_p, E_W1 + 1) << 32) | (unsigned)tget(f_p, E_W1);
+        f_col = wave;
+        f_t = 0;
+    };
+    auto issue = [&](int slot) __attribute__((always_inline)) {
+        const uint8_t* ptr = f_last;
+        if (!f_end) {
+            ptr = f_t < f_T0 ? (const uint8_t*)f_w0 + ((size_t)f_t * f_nb + f_col) * UB
+                             : (const uint8_t*)f_w1 + ((size_t)(f_t - f_T0) * f_nb + f_col) * UB;
+            ptr = uni_ptr(ptr);
+            f_last = ptr;
+            if (++f_t == f_T2) {
+                f_t = 0;
+                f_col += kWaves;
+                if (f_col >= f_nb) f_next_phase();
             }
         }
-        drain();
-        return;
-    }
-
-    // ======================================================================= consumers
-    // workgroup-level meeting of the NC consumer wavefronts
-    unsigned sync_target = 0;
-    auto meet = [&]() __attribute__((always_inline)) {
-        sync_target += NC;
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        if (lane == 0) __hip_atomic_fetch_add(ctl + C_SYNC, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        unsigned polls = 0;
-        while ((int)(lds_get(ctl + C_SYNC) - sync_target) < 0) {
-            if ((++polls & 63u) == 0 && (aborted() || polls > spin_limit)) { if (!aborted()) give_up(2u); return false; }
-        }
-        return true;
+        lds_copy_unit<F::HV>(uni(ring_lds + (uint32_t)slot * UB), off_c, ptr);
     };
+    f_next_phase();
+#pragma unroll
+    for (int s = 0; s < D; ++s) issue(s);
 
     const int n = lane & 15, q = lane >> 4;
     const int s_a = n >> 2, c_a = n & 3;
+    const bool live = (c_a == q) && (s_a < nslot);
     const uint32_t M = 0x000F000Fu;
     uint32_t C = 0x43004300u;
     asm volatile("" : "+v"(C));
     const uint32_t ONES = 0x3F803F80u;
-    float* const mycells = cells + (size_t)wave * tmax * nslot * 16;
+    int slot = 0;
     bool ok = true;
 
     for (int p = 0; p < nph && ok; ++p) {
-        const ChainPhase ph = a.phases[p];
-        const int* e = lph + p * 8;
-        const int T0 = uni(e[4]), T1 = uni(e[5]), nb = uni(e[6]), seq0 = uni(e[7]);
-        const int T2 = T0 + T1, U = T2 * nb;
-        // ---- the previous phase must be complete everywhere (wave 0 asks, the others wait for its word)
-        if (p > 0) {
-            if (wave == 0) {
-                if (ph.dep) {
-                    const unsigned target = (unsigned)p * (kWG / kCounters);
+        const ChainEntry* e = entry(p);
+        const int T0 = uni(e->T[0]), T2 = T0 + uni(e->T[1]), nb = uni(e->nb);
+        const int x_kind = uni(e->x_kind), x_op = uni(e->x_op), x_stride = uni(e->x_stride);
+        const int par = p & 1;
+        float* const mycells = cells + (size_t)par * cells_per_phase + (size_t)wave * tmax * nslot * 16;
+        // the cells of this parity were read by the finisher of phase p - 2
+        if (p >= 2) {
+            unsigned polls = 0;
+            while (lds_get(ctl + C_FINISHED) < (unsigned)(p - 1)) {
+                __builtin_amdgcn_s_sleep(1);
+                if ((++polls & 63u) == 0 && (aborted() || polls > spin_limit)) { if (!aborted()) give_up(1u); ok = false; break; }
+            }
+            if (!ok) break;
+        }
+        float sumsq[2] = {0.0f, 0.0f};
+
+        for (int col = wave; col < nb && ok; col += kWaves) {
+            // ---- this block column's 256 activations per row: lane l takes elements 4 l .. 4 l + 3
+            const unsigned want = make_tag(epoch, uni(e->x_tag_phase));
+            for (int s = 0; s < nslot && ok; ++s) {
+                float f[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                const size_t el = (size_t)s * x_stride + (size_t)col * 256 + 4 * lane;
+                if (x_kind == XK_PLAIN_BF16) {
+                    const uint2 v = *reinterpret_cast<const uint2*>(static_cast<const unsigned short*>(e->x) + el);
+                    f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xFFFF0000u);
+                    f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xFFFF0000u);
+                } else if (x_kind == XK_PLAIN_F32) {
+                    const float4 v = *reinterpret_cast<const float4*>(static_cast<const float*>(e->x) + el);
+                    f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+                } else if (x_kind == XK_TAGGED_BF16) {
+                    const uint8_t* src = static_cast<const uint8_t*>(e->x) + el * 4;
                     unsigned polls = 0;
                     for (;;) {
-                        unsigned v;
-                        const unsigned* cp = a.sync + kCounterStride * (lane & (kCounters - 1));
-                        asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(cp) : "memory");
-                        if (__builtin_amdgcn_ballot_w64((int)(v - target) < 0) == 0) break;
-                        if ((++polls & 15u) == 0 && (aborted() || polls > spin_limit)) { if (!aborted()) give_up(4u); ok = false; break; }
+                        u32x4_t v;
+                        asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(src) : "memory");
+                        const bool good = (v.x >> 16) == want && (v.y >> 16) == want && (v.z >> 16) == want && (v.w >> 16) == want;
+                        if (__builtin_amdgcn_ballot_w64(!good) == 0) {
+                            f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.y << 16);
+                            f[2] = __uint_as_float(v.z << 16); f[3] = __uint_as_float(v.w << 16);
+                            break;
+                        }
+                        __builtin_amdgcn_s_sleep(4);
+                        if ((++polls & 15u) == 0 && (aborted() || polls > spin_limit)) { if (!aborted()) give_up(2u); ok = false; break; }
                     }
-                }
-                if (lane == 0) lds_set(ctl + C_DEP, (unsigned)p);
-            } else {
-                unsigned polls = 0;
-                while (lds_get(ctl + C_DEP) < (unsigned)p) {
-                    __builtin_amdgcn_s_sleep(1);
-                    if ((++polls & 63u) == 0 && (aborted() || polls > spin_limit)) { if (!aborted()) give_up(8u); ok = false; break; }
-                }
-            }
-            if (!ok || aborted()) { ok = false; break; }
-        }
-        // ---- stage the activations: wavefront w takes block columns w, w + NC, ...; lanes 0..31 carry slot 0,
-        // lanes 32..63 slot 1; a lane holds 8 consecutive elements
-        {
-            constexpr int MAXC = 4;  // columns per wavefront: K <= 256 * NC * MAXC
-            const int quad = lane & 31, s = lane >> 5;
-            const bool live = s < nslot;
-            float f[MAXC][8];
-            float sumsq = 0.0f;
-            u32x4_t lo[MAXC], hi[MAXC];
-#pragma unroll
-            for (int ci = 0; ci < MAXC; ++ci) {
-                const int c = wave + NC * ci;
-                lo[ci] = u32x4_t{0, 0, 0, 0};
-                hi[ci] = u32x4_t{0, 0, 0, 0};
-                if (c < nb && live) {
-                    const size_t el = (size_t)s * ph.x_stride + (size_t)c * 256 + quad * 8;
-                    const uint8_t* src = static_cast<const uint8_t*>(ph.x) + el * (ph.x_dtype == TFQ_F32 ? 4 : 2);
-                    if (ph.dep) {
-                        asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(lo[ci]) : "v"(src) : "memory");
-                        if (ph.x_dtype == TFQ_F32) asm volatile("global_load_dwordx4 %0, %1, off offset:16 sc1" : "=v"(hi[ci]) : "v"(src) : "memory");
-                    } else {
-                        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(lo[ci]) : "v"(src) : "memory");
-                        if (ph.x_dtype == TFQ_F32) asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=v"(hi[ci]) : "v"(src) : "memory");
-                    }
-                }
-            }
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#pragma unroll
-            for (int ci = 0; ci < MAXC; ++ci) {
-                asm volatile("" : "+v"(lo[ci]), "+v"(hi[ci]));
-                if (ph.x_dtype == TFQ_F32) {
-                    f[ci][0] = __uint_as_float(lo[ci].x); f[ci][1] = __uint_as_float(lo[ci].y); f[ci][2] = __uint_as_float(lo[ci].z); f[ci][3] = __uint_as_float(lo[ci].w);
-                    f[ci][4] = __uint_as_float(hi[ci].x); f[ci][5] = __uint_as_float(hi[ci].y); f[ci][6] = __uint_as_float(hi[ci].z); f[ci][7] = __uint_as_float(hi[ci].w);
                 } else {
-                    const uint32_t d[4] = {lo[ci].x, lo[ci].y, lo[ci].z, lo[ci].w};
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) { f[ci][2 * i] = __uint_as_float(d[i] << 16); f[ci][2 * i + 1] = __uint_as_float(d[i] & 0xFFFF0000u); }
-                }
-#pragma unroll
-                for (int i = 0; i < 8; ++i) sumsq = __builtin_fmaf(f[ci][i], f[ci][i], sumsq);
-            }
-            // this wavefront's cells start at zero (they were read before the previous phase was announced complete)
-            for (int i = lane; i < T2 * nslot * 16; i += 64) mycells[i] = 0.0f;
-            float rs[2] = {1.0f, 1.0f};
-            if (ph.x_op == XOP_RMSNORM) {
-                // sum of squares of each activation row over the whole workgroup, added in wavefront order
-                sumsq = dpp_add<0xB1>(sumsq);
-                sumsq = dpp_add<0x4E>(sumsq);
-                sumsq += __shfl_xor(sumsq, 4);
-                sumsq += __shfl_xor(sumsq, 8);
-                sumsq += __shfl_xor(sumsq, 16);
-                if (quad == 0) reinterpret_cast<float*>(ctl + C_SUMSQ)[wave * 2 + s] = sumsq;
-                if (!meet()) { ok = false; break; }
-#pragma unroll
-                for (int r = 0; r < 2; ++r) {
-                    float tot = 0.0f;
-                    for (int w = 0; w < NC; ++w) tot += reinterpret_cast<const float*>(ctl + C_SUMSQ)[w * 2 + r];
-                    rs[r] = 1.0f / sqrtf(tot / (float)ph.K + ph.eps);
-                }
-            }
-            const float r_me = s == 0 ? rs[0] : rs[1];
-#pragma unroll
-            for (int ci = 0; ci < MAXC; ++ci) {
-                const int c = wave + NC * ci;
-                if (c >= nb) continue;  // uniform
-                uint4* col = xreg + (size_t)c * col_stride;
-                float* colX = reinterpret_cast<float*>(col + nslot * 32);
-                float sum = 0.0f;
-                if (live) {
-                    float g8[8];
-                    if (ph.x_op == XOP_RMSNORM) {
-                        const float* gp = ph.gamma + (size_t)c * 256 + quad * 8;
-                        const float4 g0 = *reinterpret_cast<const float4*>(gp), g1 = *reinterpret_cast<const float4*>(gp + 4);
-                        g8[0] = g0.x; g8[1] = g0.y; g8[2] = g0.z; g8[3] = g0.w; g8[4] = g1.x; g8[5] = g1.y; g8[6] = g1.z; g8[7] = g1.w;
+                    const uint8_t* src = static_cast<const uint8_t*>(e->x) + el * 8;
+                    unsigned polls = 0;
+                    for (;;) {
+                        u32x4_t v0, v1;
+                        asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:16 sc1\n\ts_waitcnt vmcnt(0)"
+                                     : "=&v"(v0), "=&v"(v1) : "v"(src) : "memory");
+                        const bool good = v0.y == want && v0.w == want && v1.y == want && v1.w == want;
+                        if (__builtin_amdgcn_ballot_w64(!good) == 0) {
+                            f[0] = __uint_as_float(v0.x); f[1] = __uint_as_float(v0.z);
+                            f[2] = __uint_as_float(v1.x); f[3] = __uint_as_float(v1.z);
+                            break;
+                        }
+                        __builtin_amdgcn_s_sleep(4);
+                        if ((++polls & 15u) == 0 && (aborted() || polls > spin_limit)) { if (!aborted()) give_up(2u); ok = false; break; }
                     }
-                    uint32_t ebits[8];
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        float v = f[ci][i];
-                        if (ph.x_op == XOP_RMSNORM) v = (v * r_me) * (ph.gamma_plus_one ? 1.0f + g8[i] : g8[i]);
-                        ebits[i] = bf16_rne(v);
-                    }
-                    uint4 v4;
-                    v4.x = ebits[0] | (ebits[1] << 16); v4.y = ebits[2] | (ebits[3] << 16);
-                    v4.z = ebits[4] | (ebits[5] << 16); v4.w = ebits[6] | (ebits[7] << 16);
-                    const uint4 pp = pair_permute(v4);
-                    col[s * 32 + quad] = pp;
-                    sum = dot2(ONES, pp.x, 0.0f);
-                    sum = dot2(ONES, pp.y, sum);
-                    sum = dot2(ONES, pp.z, sum);
-                    sum = dot2(ONES, pp.w, sum);
-                }
-                sum = dpp_add<0xB1>(sum);
-                if constexpr (F::GS == 32) sum = dpp_add<0x4E>(sum);
-                constexpr int LPG = F::GS / 8;
-                if (live && (quad & (LPG - 1)) == 0) colX[s * NG + quad / LPG] = sum;
-                if (lane < (4 - nslot) * NG) colX[nslot * NG + lane] = 0.0f;  // the slots that do not exist
-            }
-            if (!meet()) { ok = false; break; }
-        }
-        // ---- the units: consumer w takes units w, w + NC, ... of the phase, in the loader's order
-        {
-            int j = wave;
-            int t = j / nb, col = j - t * nb;  // tile by tile, block columns inside
-            int slot = (seq0 + j) % R;
-            for (; j < U; j += NC) {
-                const unsigned g = (unsigned)(seq0 + j);
-                unsigned polls = 0;
-                while (lds_get(ready_seq + slot) != g + 1u) {
-                    __builtin_amdgcn_s_sleep(1);
-                    if ((++polls & 63u) == 0 && (aborted() || polls > spin_limit)) { if (!aborted()) give_up(16u); ok = false; break; }
                 }
                 if (!ok) break;
-                const uint8_t* sp = ring + (size_t)slot * UB;
-                uint4 cc[NCODE], hd[F::HV];
+                if (x_op == XOP_RMSNORM) {
+                    float ss = 0.0f;
 #pragma unroll
-                for (int i = 0; i < NCODE; ++i) cc[i] = *reinterpret_cast<const uint4*>(sp + 1024 * i + 16 * lane);
+                    for (int i = 0; i < 4; ++i) ss = __builtin_fmaf(f[i], f[i], ss);
+                    sumsq[s] += ss;
+                    const float4 g = *reinterpret_cast<const float4*>(e->gamma + (size_t)col * 256 + 4 * lane);
+                    const float gg[4] = {g.x, g.y, g.z, g.w};
+                    const bool plus = uni(e->gamma_plus_one) != 0;
 #pragma unroll
-                for (int i = 0; i < F::HV; ++i) hd[i] = *reinterpret_cast<const uint4*>(sp + 1024 * NCODE + F::HB * n + 16 * i);
-                // A fragments and group sums of this block column
-                const uint4* colp = xreg + (size_t)col * col_stride;
-                const float* colX = reinterpret_cast<const float*>(colp + nslot * 32);
-                const bool live = (c_a == q) && (s_a < nslot);
-                uint4 av[2][4];
-                float xv[2][PER];
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const uint4* src = live ? colp + s_a * 32 + h * 16 + q * 4 : zero4;
-#pragma unroll
-                    for (int jj = 0; jj < 4; ++jj) av[h][jj] = src[jj];
-#pragma unroll
-                    for (int tt = 0; tt < PER; tt += 4) {
-                        const float4 fx = *reinterpret_cast<const float4*>(colX + q * NG + h * PER + tt);
-                        xv[h][tt] = fx.x; xv[h][tt + 1] = fx.y; xv[h][tt + 2] = fx.z; xv[h][tt + 3] = fx.w;
-                    }
+                    for (int i = 0; i < 4; ++i) f[i] *= plus ? 1.0f + gg[i] : gg[i];
                 }
+                // bf16, in element order, into this wavefront's bounce area; the group sums (of the rounded
+                // values) beside them
+                const uint32_t e0 = bf16_rne(f[0]) | (bf16_rne(f[1]) << 16), e1 = bf16_rne(f[2]) | (bf16_rne(f[3]) << 16);
+                *reinterpret_cast<uint2*>(bounce + s * 512 + 8 * lane) = uint2{e0, e1};
+                float sum = dot2(ONES, e0, 0.0f);
+                sum = dot2(ONES, e1, sum);
+                sum += __shfl_xor(sum, 1);
+                sum += __shfl_xor(sum, 2);
+                sum += __shfl_xor(sum, 4);  // 8 lanes = 32 elements = one group
+                if ((lane & 7) == 0) reinterpret_cast<float*>(bounce + nslot * 512)[s * NG + (lane >> 3)] = sum;
+            }
+            if (!ok) break;
+            if (lane < (4 - nslot) * NG) reinterpret_cast<float*>(bounce + nslot * 512)[nslot * NG + lane] = 0.0f;
+            // A fragments: lane (n, q) is non-zero on the diagonal c == q of activation row s
+            uint4 av[2][4];
+            float xv[2][PER];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) {
+                    uint4 v = {0, 0, 0, 0};
+                    if (live) v = pair_permute(*reinterpret_cast<const uint4*>(bounce + s_a * 512 + (h * 128 + q * 32 + jj * 8) * 2));
+                    av[h][jj] = v;
+                }
+                const float4 fx = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(bounce + nslot * 512) + q * NG + h * PER);
+                xv[h][0] = fx.x; xv[h][1] = fx.y; xv[h][2] = fx.z; xv[h][3] = fx.w;
+            }
+
+            // ---- this block column's units, tile by tile
+            for (int t = 0; t < T2; ++t) {
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS * (D - 1)) : "memory");
+                const uint8_t* sp = rings + ((size_t)wave * D + slot) * UB;
+                uint4 cc[2], hd[F::HV];
+                cc[0] = *reinterpret_cast<const uint4*>(sp + 16 * lane);
+                cc[1] = *reinterpret_cast<const uint4*>(sp + 1024 + 16 * lane);
+#pragma unroll
+                for (int i = 0; i < F::HV; ++i) hd[i] = *reinterpret_cast<const uint4*>(sp + 2048 + F::HB * n + 16 * i);
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                if (lane == 0) lds_set(free_seq + slot, g + 1u);  // the slot's bytes are in registers
+                issue(slot);
+                slot = slot + 1 == D ? 0 : slot + 1;
 
                 float res = 0.0f;
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
-                    f32x4_t DA, DB = {0.0f, 0.0f, 0.0f, 0.0f};
-                    const float* X = xv[h];
-                    if constexpr (F::GS == 32) {
-                        DA = f32x4_t{-F::OFFS * X[0], -F::OFFS * X[1], -F::OFFS * X[2], -F::OFFS * X[3]};
-                    } else {
-                        DA = f32x4_t{-F::OFFS * X[0], -F::OFFS * X[2], -F::OFFS * X[4], -F::OFFS * X[6]};
-                        DB = f32x4_t{-F::OFFS * X[1], -F::OFFS * X[3], -F::OFFS * X[5], -F::OFFS * X[7]};
-                    }
+                    f32x4_t DA = {-F::OFFS * xv[h][0], -F::OFFS * xv[h][1], -F::OFFS * xv[h][2], -F::OFFS * xv[h][3]};
+                    const f32x4_t DB = {0.0f, 0.0f, 0.0f, 0.0f};
+                    const uint32_t qq[4] = {cc[h].x, cc[h].y, cc[h].z, cc[h].w};
 #pragma unroll
-                    for (int pl = 0; pl < F::NP; ++pl) {
-                        const uint4 cw = cc[2 * pl + h];
-                        const uint32_t qq[4] = {cw.x, cw.y, cw.z, cw.w};
-#pragma unroll
-                        for (int jj = 0; jj < 4; ++jj) {
-                            const uint32_t v = qq[jj];
-                            const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
-                            const bool second = pl == 1 || (F::GS == 16 && jj >= 2);
-                            if (!second)
-                                DA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[h][jj]), __builtin_bit_cast(bf16x8_t, wv), DA, 0, 0, 0);
-                            else
-                                DB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[h][jj]), __builtin_bit_cast(bf16x8_t, wv), DB, 0, 0, 0);
-                        }
+                    for (int jj = 0; jj < 4; ++jj) {
+                        const uint32_t v = qq[jj];
+                        const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
+                        DA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[h][jj]), __builtin_bit_cast(bf16x8_t, wv), DA, 0, 0, 0);
                     }
                     res += apply_groups<FMT>(hd, h, DA, DB, xv[h]);
                 }
-                if (q < nslot) mycells[(t * nslot + q) * 16 + n] += res;
+                if (q < nslot) {
+                    float* cell = mycells + (t * nslot + q) * 16 + n;
+                    if (col == wave) *cell = res;
+                    else *cell += res;
+                }
+            }
+        }
+        if (!ok) break;
+        // a wavefront without a block column in this phase still owns cells: they must read as zero
+        if (wave >= nb) for (int i = lane; i < T2 * nslot * 16; i += 64) mycells[i] = 0.0f;
+        if (x_op == XOP_RMSNORM) {
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                float v = sumsq[s];
+                v += __shfl_xor(v, 1); v += __shfl_xor(v, 2); v += __shfl_xor(v, 4);
+                v += __shfl_xor(v, 8); v += __shfl_xor(v, 16); v += __shfl_xor(v, 32);
+                if (lane == 0) ssq[(par * kWaves + wave) * 2 + s] = v;
+            }
+        }
 
-                col += NC;
-                while (col >= nb) { col -= nb; ++t; }
-                slot += NC;
-                while (slot >= R) slot -= R;
+        // ---- the wavefront that arrives last finishes the phase for the workgroup
+        unsigned arrived = 0;
+        if (lane == 0) arrived = __hip_atomic_fetch_add(ctl + C_WORDS + p, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        arrived = uni(arrived);
+        if (arrived != (unsigned)(kWaves - 1)) continue;
+
+        const bool swiglu = uni(e->y_op) == YOP_SWIGLU, resid = uni(e->y_op) == YOP_RESIDUAL;
+        const int Tout = swiglu ? T0 : T2;
+        const int nout = Tout * nslot * 16;
+        const float* pc = cells + (size_t)par * cells_per_phase;
+        float rs[2] = {1.0f, 1.0f};
+        if (x_op == XOP_RMSNORM) {
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                float tot = 0.0f;
+                for (int w = 0; w < kWaves; ++w) tot += ssq[(par * kWaves + w) * 2 + s];
+                rs[s] = 1.0f / sqrtf(tot / (float)(nb * 256) + e->eps);
+            }
+        }
+        const unsigned tag = make_tag(epoch, p);
+        const int n_result = uni(e->n_result), link_kind = uni(e->link_kind), y_dtype = uni(e->y_dtype);
+        bool fin_ok = true;
+        for (int o = lane; o < nout; o += 64) {
+            const int nn = o & 15, s = (o >> 4) % nslot, t = (o >> 4) / nslot;
+            const int seg = t < T0 ? 0 : 1, tt = seg ? t - T0 : t;
+            const int row = e->row0[seg] + tt * 16 + nn;
+            if (row >= e->nrows[seg]) continue;
+            float v = 0.0f;
+            for (int w = 0; w < kWaves; ++w) v += pc[((size_t)(w * tmax + t) * nslot + s) * 16 + nn];
+            v *= s == 0 ? rs[0] : rs[1];
+            const size_t ri = (size_t)s * n_result + e->res0[seg] + tt * 16 + nn;
+            if (swiglu) {
+                float u = 0.0f;
+                for (int w = 0; w < kWaves; ++w) u += pc[((size_t)(w * tmax + t + T0) * nslot + s) * 16 + nn];
+                u *= s == 0 ? rs[0] : rs[1];
+                if (e->y[0]) static_cast<float*>(e->y[0])[(size_t)s * e->nrows[0] + row] = v;
+                if (e->y[1]) static_cast<float*>(e->y[1])[(size_t)s * e->nrows[1] + row] = u;
+                v = v / (1.0f + expf(-v)) * u;
+            }
+            if (resid) {
+                float h = 0.0f;
+                if (e->hprev) {
+                    const unsigned hwant = make_tag(epoch, e->hprev_tag_phase);
+                    const unsigned long long* src = static_cast<const unsigned long long*>(e->hprev) + ri;
+                    unsigned polls = 0;
+                    for (;;) {
+                        const unsigned long long hv = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if ((unsigned)(hv >> 32) == hwant) { h = __uint_as_float((unsigned)hv); break; }
+                        if (++polls > spin_limit) { fin_ok = false; break; }
+                    }
+                } else {
+                    h = e->residual[ri];
+                }
+                v += h;
+                e->residual[ri] = v;
+            }
+            if (!swiglu && e->y[seg]) {
+                const size_t off = (size_t)s * e->nrows[seg] + row;
+                if (y_dtype == TFQ_BF16) static_cast<unsigned short*>(e->y[seg])[off] = (unsigned short)bf16_rne(v);
+                else static_cast<float*>(e->y[seg])[off] = v;
+            }
+            if (e->link) {
+                if (link_kind == XK_TAGGED_BF16)
+                    __hip_atomic_store(static_cast<unsigned*>(e->link) + ri, bf16_rne(v) | (tag << 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                else
+                    __hip_atomic_store(static_cast<unsigned long long*>(e->link) + ri, (unsigned long long)__float_as_uint(v) | ((unsigned long long)tag << 32),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        if (__builtin_amdgcn_ballot_w64(!fin_ok) != 0) { give_up(4u); ok = false; break; }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        {   // finishers of consecutive phases may be different wavefronts: they publish in phase order
+            unsigned polls = 0;
+            while (lds_get(ctl + C_FINISHED) < (unsigned)p) {
+                __builtin_amdgcn_s_sleep(1);
+                if ((++polls & 63u) == 0 && (aborted() || polls > spin_limit)) { if (!aborted()) give_up(8u); ok = false; break; }
             }
             if (!ok) break;
         }
-        if (!meet()) { ok = false; break; }
-
-        // ---- wave 0 adds the wavefronts' partial sums in order, applies the epilogue, stores and announces
-        if (wave == 0) {
-            const ChainWg wg = a.wgs[(size_t)p * kWG + b];
-            const bool swiglu = ph.y_op == YOP_SWIGLU;
-            const int Tout = swiglu ? T0 : T2;  // result tiles
-            const int nout = Tout * nslot * 16;
-            for (int o = lane; o < nout; o += 64) {
-                const int nn = o & 15, s = (o >> 4) % nslot, t = (o >> 4) / nslot;
-                const int seg = t < T0 ? 0 : 1, tt = seg ? t - T0 : t;
-                const int row = wg.row0[seg] + tt * 16 + nn;
-                if (row >= wg.nrows[seg]) continue;
-                float v = 0.0f;
-                for (int w = 0; w < NC; ++w) v += cells[((size_t)(w * tmax + t) * nslot + s) * 16 + nn];
-                if (swiglu) {
-                    float u = 0.0f;
-                    for (int w = 0; w < NC; ++w) u += cells[((size_t)(w * tmax + t + T0) * nslot + s) * 16 + nn];
-                    if (wg.y[0]) store_dev_f32(static_cast<float*>(wg.y[0]) + (size_t)s * wg.nrows[0] + row, v);  // fp32 only (host checks)
-                    if (wg.y[1]) store_dev_f32(static_cast<float*>(wg.y[1]) + (size_t)s * wg.nrows[1] + row, u);
-                    v = v / (1.0f + expf(-v)) * u;
-                } else if (wg.y[seg] && ph.y_op != YOP_RESIDUAL) {
-                    const size_t off = (size_t)s * wg.nrows[seg] + row;
-                    if (ph.y_dtype == TFQ_BF16) store_dev_u16(static_cast<unsigned short*>(wg.y[seg]) + off, (unsigned short)bf16_rne(v));
-                    else store_dev_f32(static_cast<float*>(wg.y[seg]) + off, v);
-                }
-                const size_t ri = (size_t)s * ph.n_result + wg.res0[seg] + tt * 16 + nn;
-                if (ph.y_op == YOP_RESIDUAL) {
-                    v += load_dev_f32(ph.residual + ri);
-                    store_dev_f32(ph.residual + ri, v);
-                    if (wg.y[seg]) {
-                        const size_t off = (size_t)s * wg.nrows[seg] + row;
-                        if (ph.y_dtype == TFQ_BF16) store_dev_u16(static_cast<unsigned short*>(wg.y[seg]) + off, (unsigned short)bf16_rne(v));
-                        else store_dev_f32(static_cast<float*>(wg.y[seg]) + off, v);
-                    }
-                }
-                if (ph.link) {
-                    if (ph.link_dtype == TFQ_BF16) store_dev_u16(static_cast<unsigned short*>(ph.link) + ri, (unsigned short)bf16_rne(v));
-                    else store_dev_f32(static_cast<float*>(ph.link) + ri, v);
-                }
-            }
-            // every store of this workgroup has completed before its arrival is counted
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            if (lane == 0) __hip_atomic_fetch_add(a.sync + kCounterStride * (b & (kCounters - 1)), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+        if (lane == 0) lds_set(ctl + C_FINISHED, (unsigned)(p + 1));
     }
 
-    // ---- the last workgroup to get here puts the counters back to zero for the next launch.  Every workgroup
-    // comes through (all waits are bounded), after its last look at the counters.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this workgroup's last arrival has been counted
-    if (wave == 0 && lane == 0) {
-        const unsigned seen = __hip_atomic_fetch_add(a.sync + 1024, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (seen == kWG - 1) {
-            for (int i = 0; i < kCounters; ++i) __hip_atomic_store(a.sync + kCounterStride * i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(a.sync + 1024, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // no copy may land in LDS after the workgroup is gone; plain result stores complete with the kernel
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // The last workgroup to get here advances the launch counter.  Every workgroup comes through (all waits are
+    // bounded); one wavefront per workgroup counts, after the workgroup's last phase has been finished or given up.
+    if (wave == 0) {
+        unsigned polls = 0;
+        while (lds_get(ctl + C_FINISHED) < (unsigned)nph && !aborted()) {
+            __builtin_amdgcn_s_sleep(2);
+            if (++polls > spin_limit) break;
+        }
+        if (lane == 0) {
+            const unsigned seen = __hip_atomic_fetch_add(a.sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (seen == kWG - 1) {
+                __hip_atomic_store(a.sync + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_fetch_add(a.sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
     }
 }
 
-
 // ---------------------------------------------------------------------------------------- host side
-template <int FMT, int NL>
+template <int FMT, int D>
 hipError_t launch_chain(const ChainArgs& a, size_t lds, hipStream_t s) {
     static std::atomic<bool> raised{false};
     if (!raised) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(chain_kernel<FMT, NL>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(chain_kernel<FMT, D>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         raised = true;
     }
-    hipLaunchKernelGGL((chain_kernel<FMT, NL>), dim3(kWG), dim3(64 * kWaves), lds, s, a);
+    hipLaunchKernelGGL((chain_kernel<FMT, D>), dim3(kWG), dim3(64 * kWaves), lds, s, a);
     return hipGetLastError();
 }
 
-template <int FMT, int NL>
+template <int FMT, int D>
 int chain_occupancy(size_t lds) {
     int per_cu = 0;
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(chain_kernel<FMT, NL>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, chain_kernel<FMT, NL>, 64 * kWaves, lds) != hipSuccess) return 0;
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(chain_kernel<FMT, D>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, chain_kernel<FMT, D>, 64 * kWaves, lds) != hipSuccess) return 0;
     return per_cu;
 }
 
@@ -628,10 +504,9 @@ using namespace tfq;
 
 struct tfq_chain {
     int fmt = 0, nph = 0, B = 0;
-    int ring = 0, ncols_max = 0, tmax = 0;
+    int depth = 0, tmax = 0;
     size_t lds = 0;
-    ChainPhase* d_phases = nullptr;
-    ChainWg* d_wgs = nullptr;
+    ChainEntry* d_entries = nullptr;
     unsigned* d_sync = nullptr;
     uint8_t* d_links = nullptr;
     size_t weight_bytes = 0;  // packed bytes one run streams
@@ -639,7 +514,7 @@ struct tfq_chain {
 
 namespace {
 
-constexpr int kSyncWords = 1026;
+constexpr int kSyncWords = 64;
 
 int chain_fail(tfq_chain* c, int code, const std::string& msg) {
     if (c) tfq_chain_free(c);
@@ -651,6 +526,11 @@ bool chain_format(int fmt) {
         case TFQ_B32S4: case TFQ_Q_G_4: return true;
         default: return false;
     }
+}
+
+size_t chain_lds_bytes(int depth, int fmt, int B, int tmax, int nph) {
+    return (size_t)kWaves * depth * tiled_unit_bytes(fmt) + (size_t)kWaves * (B * 512 + 128) + (size_t)2 * kWaves * tmax * B * 64 +
+           (size_t)2 * kWaves * 2 * 4 + (size_t)nph * kEntryWords * 4 + (size_t)(C_WORDS + nph) * 4;
 }
 
 }  // namespace
@@ -669,29 +549,29 @@ tfq_chain_t* tfq_chain_create(const tfq_chain_phase_t* phases, int nphase, int B
     tfq_chain* c = new tfq_chain();
     c->nph = nphase;
     c->B = B;
-    const int NC = kWaves - kLoaders;
-    std::vector<ChainPhase> hp((size_t)nphase);
-    std::vector<ChainWg> hw((size_t)nphase * kWG);
+    std::vector<ChainEntry> he((size_t)nphase * kWG);
     std::vector<long long> load(kWG, 0);  // units handed to each workgroup so far
-    // results that a later phase reads through x == NULL live in two alternating link buffers
-    size_t link_bytes = 0;
-    for (int p = 0; p + 1 < nphase; ++p) {
-        if (phases[p + 1].x == nullptr && phases[p].y_op != TFQ_CHAIN_Y_RESIDUAL) {
-            size_t n = 0;
-            for (int m = 0; m < phases[p].count; ++m) n += phases[p].w[m] ? (size_t)phases[p].w[m]->N : 0;
-            link_bytes = std::max(link_bytes, (size_t)B * n * 4);
-        }
+    // Intermediate vectors: two alternating link buffers for results read through x == NULL and two for the
+    // tagged copy of the residual rows; elements of 8 bytes (fp32, tag) at most.
+    size_t link_elems = 0;
+    for (int p = 0; p < nphase; ++p) {
+        size_t n = 0;
+        for (int m = 0; m < phases[p].count && m < 4; ++m) n += phases[p].w[m] ? (size_t)phases[p].w[m]->N : 0;
+        link_elems = std::max(link_elems, (size_t)B * n);
     }
-    link_bytes = (link_bytes + 255) & ~(size_t)255;
+    const size_t link_bytes = (link_elems * 8 + 255) & ~(size_t)255;
     if (hipMalloc(&c->d_sync, kSyncWords * 4) != hipSuccess || hipMemset(c->d_sync, 0, kSyncWords * 4) != hipSuccess ||
-        (link_bytes && hipMalloc(&c->d_links, 2 * link_bytes) != hipSuccess)) {
+        hipMalloc(&c->d_links, 4 * link_bytes) != hipSuccess || hipMemset(c->d_links, 0, 4 * link_bytes) != hipSuccess) {
         chain_fail(c, TFQ_ERR_NOMEM, "tfq_chain_create: device allocation failed");
         return nullptr;
     }
     int fmt = -1;
+    float* residual_buf = nullptr;
+    int resid_count = 0;           // residual phases so far
+    int last_resid_phase = -1;
+    struct Prev { int n_result = 0, link_kind = 0; void* link = nullptr; } prev;
     for (int p = 0; p < nphase; ++p) {
         const tfq_chain_phase_t& ph = phases[p];
-        ChainPhase& d = hp[(size_t)p];
         if (ph.count < 1 || ph.count > 4) { chain_fail(c, TFQ_ERR_ARG, "tfq_chain_create: 1 to 4 matrices per phase"); return nullptr; }
         int64_t K = 0, ntot = 0;
         for (int m = 0; m < ph.count; ++m) {
@@ -705,61 +585,75 @@ tfq_chain_t* tfq_chain_create(const tfq_chain_phase_t* phases, int nphase, int B
             ntot += w->N;
             c->weight_bytes += (size_t)((w->N + 15) / 16) * (size_t)(w->K / 256) * tiled_unit_bytes(fmt);
         }
-        if (K % 256 || K > 256LL * NC * 4) { chain_fail(c, TFQ_ERR_SHAPE, "tfq_chain_create: K must be a multiple of 256, at most 14336"); return nullptr; }
-        const bool swiglu = ph.y_op == TFQ_CHAIN_Y_SWIGLU;
+        if (K % 256 || K > 0x7FFFFF00) { chain_fail(c, TFQ_ERR_SHAPE, "tfq_chain_create: K must be a multiple of 256"); return nullptr; }
+        const bool swiglu = ph.y_op == TFQ_CHAIN_Y_SWIGLU, resid = ph.y_op == TFQ_CHAIN_Y_RESIDUAL;
         if (swiglu && (ph.count != 2 || ph.w[0]->N != ph.w[1]->N || ph.y_dtype != TFQ_F32)) { chain_fail(c, TFQ_ERR_SHAPE, "tfq_chain_create: SwiGLU takes gate and up of equal shape and fp32 outputs"); return nullptr; }
-        if (ph.y_op == TFQ_CHAIN_Y_RESIDUAL && (!ph.residual || ph.count != 1)) { chain_fail(c, TFQ_ERR_ARG, "tfq_chain_create: the residual form takes one matrix and a residual buffer"); return nullptr; }
+        if (resid && (!ph.residual || ph.count != 1)) { chain_fail(c, TFQ_ERR_ARG, "tfq_chain_create: the residual form takes one matrix and a residual buffer"); return nullptr; }
+        if (resid && residual_buf && residual_buf != ph.residual) { chain_fail(c, TFQ_ERR_ARG, "tfq_chain_create: one residual buffer per chain"); return nullptr; }
         if (ph.x_op == TFQ_CHAIN_X_RMSNORM && !ph.gamma) { chain_fail(c, TFQ_ERR_ARG, "tfq_chain_create: RMSNorm needs a gain vector"); return nullptr; }
+        if (ph.x_op != TFQ_CHAIN_X_PLAIN && ph.x_op != TFQ_CHAIN_X_RMSNORM) { chain_fail(c, TFQ_ERR_ARG, "tfq_chain_create: unknown x_op"); return nullptr; }
         const int64_t n_result = swiglu ? ph.w[0]->N : ntot;
-        d = ChainPhase{};
-        d.K = (int)K;
-        d.nslot = B;
-        d.x_op = ph.x_op; d.y_op = ph.y_op; d.y_dtype = ph.y_dtype;
-        d.gamma = ph.gamma; d.eps = ph.eps; d.gamma_plus_one = ph.gamma_plus_one;
-        d.residual = ph.residual;
-        d.n_result = (int)n_result;
-        if (ph.x) {
-            d.x = ph.x; d.x_dtype = ph.x_dtype; d.x_stride = (int)K; d.dep = ph.x_depends ? 1 : 0;
+        ChainEntry base{};
+        base.nb = (int)(K / 256);
+        base.x_op = ph.x_op; base.y_op = ph.y_op; base.y_dtype = ph.y_dtype;
+        base.gamma = ph.gamma; base.eps = ph.eps; base.gamma_plus_one = ph.gamma_plus_one;
+        base.n_result = (int)n_result;
+        if (p == 0) {
+            if (!ph.x) { chain_fail(c, TFQ_ERR_ARG, "tfq_chain_create: the first phase needs x"); return nullptr; }
+            if ((uintptr_t)ph.x % 16) { chain_fail(c, TFQ_ERR_ARG, "tfq_chain_create: x must be 16-byte aligned"); return nullptr; }
+            base.x = ph.x;
+            base.x_kind = ph.x_dtype == TFQ_F32 ? XK_PLAIN_F32 : XK_PLAIN_BF16;
+            base.x_stride = (int)K;
         } else {
-            if (p == 0) { chain_fail(c, TFQ_ERR_ARG, "tfq_chain_create: the first phase needs x"); return nullptr; }
-            const ChainPhase& prev = hp[(size_t)p - 1];
+            // Every later phase reads the result of the phase before it.  (An input from outside, or one written
+            // by an earlier phase into a caller's buffer, would need a grid-wide wait that this kernel does not have.)
+            if (ph.x) { chain_fail(c, TFQ_ERR_ARG, "tfq_chain_create: only the first phase takes x; later phases read the previous result (x = NULL)"); return nullptr; }
             if (prev.n_result < K) { chain_fail(c, TFQ_ERR_SHAPE, "tfq_chain_create: the previous phase's result is shorter than K"); return nullptr; }
-            d.dep = 1;
-            d.x_stride = prev.n_result;
-            if (prev.y_op == YOP_RESIDUAL) { d.x = prev.residual; d.x_dtype = TFQ_F32; }
-            else { d.x = prev.link; d.x_dtype = prev.link_dtype; }
+            base.x = prev.link;
+            base.x_kind = prev.link_kind;
+            base.x_stride = prev.n_result;
+            base.x_tag_phase = p - 1;
         }
-        if (p + 1 < nphase && phases[p + 1].x == nullptr && ph.y_op != TFQ_CHAIN_Y_RESIDUAL) {
-            d.link = c->d_links + (size_t)(p & 1) * link_bytes;
-            // RMSNorm reads the unrounded values; a plain product rounds to bf16 anyway
-            d.link_dtype = phases[p + 1].x_op == TFQ_CHAIN_X_RMSNORM ? TFQ_F32 : TFQ_BF16;
+        if (resid) {
+            residual_buf = ph.residual;
+            base.residual = ph.residual;
+            base.hprev = resid_count ? c->d_links + (size_t)(2 + ((resid_count - 1) & 1)) * link_bytes : nullptr;
+            base.hprev_tag_phase = last_resid_phase;
         }
-        c->ncols_max = std::max(c->ncols_max, (int)(K / 256));
+        // The phase's own tagged result: the residual rows keep their precision (the next RMSNorm and the next
+        // residual phase read them), a product that will be rounded to bf16 anyway travels as bf16.
+        if (resid) {
+            base.link = c->d_links + (size_t)(2 + (resid_count & 1)) * link_bytes;
+            base.link_kind = XK_TAGGED_F32;
+        } else if (p + 1 < nphase) {
+            base.link = c->d_links + (size_t)(p & 1) * link_bytes;
+            base.link_kind = phases[p + 1].x_op == TFQ_CHAIN_X_RMSNORM ? XK_TAGGED_F32 : XK_TAGGED_BF16;
+        }
+        if (resid) { ++resid_count; last_resid_phase = p; }
+        prev.n_result = (int)n_result; prev.link = base.link; prev.link_kind = base.link_kind;
 
         // ---- tiles -> workgroups.  SwiGLU: a workgroup takes the same tiles of gate and up.
         const int nb = (int)(K / 256);
-        std::vector<int> tiles_of;  // concatenated tile list: matrix of every tile
         const int nmat_split = swiglu ? 1 : ph.count;
         int64_t total_tiles = 0;
         for (int m = 0; m < nmat_split; ++m) total_tiles += (ph.w[m]->N + 15) / 16;
         const int per_tile_units = swiglu ? 2 * nb : nb;
-        const int base = (int)(total_tiles / kWG), extra = (int)(total_tiles % kWG);
-        if ((base + (extra ? 1 : 0)) * (swiglu ? 2 : 1) > kMaxTiles) { chain_fail(c, TFQ_ERR_SHAPE, "tfq_chain_create: a phase has more rows than one launch covers"); return nullptr; }
-        std::vector<int> order(kWG), count(kWG, base);
+        const int basecnt = (int)(total_tiles / kWG), extra = (int)(total_tiles % kWG);
+        if ((basecnt + (extra ? 1 : 0)) * (swiglu ? 2 : 1) > kMaxTiles) { chain_fail(c, TFQ_ERR_SHAPE, "tfq_chain_create: a phase has more rows than one launch covers"); return nullptr; }
+        std::vector<int> order(kWG), count(kWG, basecnt);
         for (int i = 0; i < kWG; ++i) order[(size_t)i] = i;
         std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return load[(size_t)x] < load[(size_t)y]; });
         for (int i = 0; i < extra; ++i) ++count[(size_t)order[(size_t)i]];
         int64_t next = 0;  // next tile in the concatenated list
         for (int b = 0; b < kWG; ++b) {
-            ChainWg& g = hw[(size_t)p * kWG + b];
-            g = ChainWg{};
+            ChainEntry& g = he[(size_t)p * kWG + b];
+            g = base;
             int left = count[(size_t)b], seg = 0;
             load[(size_t)b] += (long long)left * per_tile_units;
             c->tmax = std::max(c->tmax, left * (swiglu ? 2 : 1));
             int64_t t = next;
             next += left;
             while (left > 0) {
-                // matrix of tile t
                 int m = 0;
                 int64_t first = 0, res0 = 0;
                 while (t >= first + (ph.w[m]->N + 15) / 16) { first += (ph.w[m]->N + 15) / 16; res0 += ph.w[m]->N; ++m; }
@@ -784,27 +678,21 @@ tfq_chain_t* tfq_chain_create(const tfq_chain_phase_t* phases, int nphase, int B
                 t += take;
                 left -= take;
             }
-            if (g.T[0] == 0) { g.w[0] = ph.w[0]->dev; g.w[1] = ph.w[0]->dev; }
-            if (g.T[1] == 0 && !g.w[1]) g.w[1] = g.w[0];
+            if (!g.w[0]) g.w[0] = ph.w[0]->dev;
+            if (!g.w[1]) g.w[1] = g.w[0];
         }
     }
     c->fmt = fmt;
     if (c->tmax < 1) c->tmax = 1;
-    // LDS budget: everything but the ring is fixed; the ring takes the rest
-    const int NG = spec_of(fmt).gsz == 16 ? 16 : 8;
-    const size_t fixed = ((size_t)c->ncols_max * (B * 32 + NG) + 4) * 16 + (size_t)NC * c->tmax * B * 64 + (size_t)nphase * 32 + C_WORDS * 4 + 64;
-    const size_t UB = (size_t)tiled_unit_bytes(fmt);
-    const size_t budget = 160 * 1024;
-    if (fixed + 8 * UB + 64 > budget) { chain_fail(c, TFQ_ERR_SHAPE, "tfq_chain_create: the activations leave no room for the weight ring in LDS"); return nullptr; }
-    int ring = (int)((budget - fixed) / (UB + 8));
-    if (ring > 4096) ring = 4096;
-    c->ring = ring;
-    c->lds = fixed + (size_t)ring * (UB + 8);
-    const int occ = fmt == TFQ_B32S4 ? chain_occupancy<TFQ_B32S4, kLoaders>(c->lds) : chain_occupancy<TFQ_Q_G_4, kLoaders>(c->lds);
+    // ring depth: three units per wavefront where LDS allows it, else two
+    c->depth = chain_lds_bytes(3, fmt, B, c->tmax, nphase) <= 160 * 1024 ? 3 : 2;
+    c->lds = chain_lds_bytes(c->depth, fmt, B, c->tmax, nphase);
+    if (c->lds > 160 * 1024) { chain_fail(c, TFQ_ERR_SHAPE, "tfq_chain_create: the phases do not fit in LDS"); return nullptr; }
+    const int occ = c->depth == 3 ? (fmt == TFQ_B32S4 ? chain_occupancy<TFQ_B32S4, 3>(c->lds) : chain_occupancy<TFQ_Q_G_4, 3>(c->lds))
+                                  : (fmt == TFQ_B32S4 ? chain_occupancy<TFQ_B32S4, 2>(c->lds) : chain_occupancy<TFQ_Q_G_4, 2>(c->lds));
     if (occ < 1) { chain_fail(c, TFQ_ERR_DEVICE, "tfq_chain_create: the chain kernel does not fit a compute unit"); return nullptr; }
-    if (hipMalloc(&c->d_phases, hp.size() * sizeof(ChainPhase)) != hipSuccess || hipMalloc(&c->d_wgs, hw.size() * sizeof(ChainWg)) != hipSuccess ||
-        hipMemcpy(c->d_phases, hp.data(), hp.size() * sizeof(ChainPhase), hipMemcpyHostToDevice) != hipSuccess ||
-        hipMemcpy(c->d_wgs, hw.data(), hw.size() * sizeof(ChainWg), hipMemcpyHostToDevice) != hipSuccess) {
+    if (hipMalloc(&c->d_entries, he.size() * sizeof(ChainEntry)) != hipSuccess ||
+        hipMemcpy(c->d_entries, he.data(), he.size() * sizeof(ChainEntry), hipMemcpyHostToDevice) != hipSuccess) {
         chain_fail(c, TFQ_ERR_NOMEM, "tfq_chain_create: device allocation failed");
         return nullptr;
     }
@@ -814,33 +702,33 @@ tfq_chain_t* tfq_chain_create(const tfq_chain_phase_t* phases, int nphase, int B
 int tfq_chain_run(const tfq_chain_t* c, tfq_stream_t stream) {
     if (!c) return fail(TFQ_ERR_ARG, "tfq_chain_run: null chain");
     ChainArgs a{};
-    a.phases = c->d_phases; a.wgs = c->d_wgs; a.sync = c->d_sync;
-    a.nph = c->nph; a.ring = c->ring; a.ncols_max = c->ncols_max; a.nslot = c->B; a.tmax = c->tmax;
+    a.entries = c->d_entries; a.sync = c->d_sync;
+    a.nph = c->nph; a.depth = c->depth; a.nslot = c->B; a.tmax = c->tmax;
     a.spin_limit = kSpinLimit;
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;
-    e = c->fmt == TFQ_B32S4 ? launch_chain<TFQ_B32S4, kLoaders>(a, c->lds, s) : launch_chain<TFQ_Q_G_4, kLoaders>(a, c->lds, s);
+    if (c->depth == 3) e = c->fmt == TFQ_B32S4 ? launch_chain<TFQ_B32S4, 3>(a, c->lds, s) : launch_chain<TFQ_Q_G_4, 3>(a, c->lds, s);
+    else e = c->fmt == TFQ_B32S4 ? launch_chain<TFQ_B32S4, 2>(a, c->lds, s) : launch_chain<TFQ_Q_G_4, 2>(a, c->lds, s);
     return hip_fail(e, "chain launch");
 }
 
 int tfq_chain_check(const tfq_chain_t* c) {
     if (!c) return fail(TFQ_ERR_ARG, "tfq_chain_check: null chain");
-    unsigned err = 0;
-    TFQ_HIP(hipMemcpy(&err, c->d_sync + 1025, 4, hipMemcpyDeviceToHost));
-    if (err) {
-        (void)hipMemset(c->d_sync, 0, kSyncWords * 4);
-        return fail(TFQ_ERR_DEVICE, "tfq_chain_check: a wait inside the chain kernel ran out (code " + std::to_string(err) + "); the results of that run are incomplete");
+    unsigned w[3] = {0, 0, 0};
+    TFQ_HIP(hipMemcpy(w, c->d_sync, 12, hipMemcpyDeviceToHost));
+    if (w[2]) {
+        const unsigned zero[2] = {0, 0};
+        (void)hipMemcpy(c->d_sync + 1, zero, 8, hipMemcpyHostToDevice);  // finished count and error bits; the launch counter stays
+        return fail(TFQ_ERR_DEVICE, "tfq_chain_check: a wait inside the chain kernel ran out (code " + std::to_string(w[2]) + "); the results of that run are incomplete");
     }
     return TFQ_OK;
 }
-
 
 size_t tfq_chain_weight_bytes(const tfq_chain_t* c) { return c ? c->weight_bytes : 0; }
 
 void tfq_chain_free(tfq_chain_t* c) {
     if (!c) return;
-    (void)hipFree(c->d_phases);
-    (void)hipFree(c->d_wgs);
+    (void)hipFree(c->d_entries);
     (void)hipFree(c->d_sync);
     (void)hipFree(c->d_links);
     delete c;
