@@ -169,10 +169,10 @@ tfq_weight_t* tfq_container_weight(const tfq_container_t* c, const char* name, i
  * quantize_block_all / dequantize_block_all (include/quant/block_codec.h:69-77),
  * applied to a tensor cut into 256-weight blocks the way
  * FormatRegistry::quantize / dequantize do (src/codec/format_registry.cpp:168-207,
- * 241-290): payloads are concatenated in block order.  Encoding needs n to be a
- * multiple of 256; decoding also takes a short last block of n % 256 weights in
- * the layout the reference's codec chooses for that size (tfq_block_bytes gives
- * its byte count).  dst/src and w/out are device pointers. */
+ * 241-290): payloads are concatenated in block order.  A last block of n % 256
+ * weights is written and read in the layout the reference's codec chooses for that
+ * size (tfq_block_bytes gives its byte count; TFQ_ERR_SHAPE for the two literal
+ * block-32 formats when n % 32 != 0).  dst/src and w/out are device pointers. */
 int tfq_encode_blocks(uint8_t fmt, const float* w, int64_t n, uint8_t* dst, size_t cap,
                       tfq_stream_t stream);
 int tfq_decode_blocks(uint8_t fmt, const uint8_t* src, size_t bytes, int64_t n, float* out,

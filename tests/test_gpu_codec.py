@@ -111,6 +111,27 @@ def test_decode_short_blocks_golden(tfq, gpu):
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (fmt, n, which)
 
 
+def test_encode_short_blocks_golden(O, tfq, gpu):
+    """The device encoder of a short block against the payloads the compiled reference wrote
+    (tests/golden/tails.npz: 42 ids x 13 block sizes x 2 inputs), and a tensor of full blocks plus a
+    short one against the oracle."""
+    import torch
+    t = np.load(os.path.join(G, "tails.npz"))
+    for fmt, n, which, poff, plen, doff in t["index"]:
+        w = np.ascontiguousarray(t["src"][which][:n])
+        want = t["payloads"][poff:poff + plen]
+        got = tfq.encode(int(fmt), torch.from_numpy(w).to(gpu)).cpu().numpy()
+        assert np.array_equal(got, want), (fmt, n, which)
+    for fmt in ("Q_G_4", "Q_4", "Q_G_8", "Q_G_6_K_H", "Q_8_K_H", "Q_G_12", "Q_MX_4_5", "B32S4"):
+        n = 3 * 256 + 160
+        w = O.rng_normal(77, n, 0.05)
+        want = O.encode_tensor(fmt, w)
+        got = tfq.encode(fmt, torch.from_numpy(w).to(gpu)).cpu().numpy()
+        assert np.array_equal(got, want), fmt
+        back = tfq.decode(fmt, torch.from_numpy(want).to(gpu), n).cpu().numpy()
+        assert np.array_equal(back.view(np.uint32), O.decode_tensor(fmt, want, n).view(np.uint32)), fmt
+
+
 def test_half_subnormal_scales_decode_exactly(O, tfq, gpu):
     import torch
     pay = np.zeros((128, 272), np.uint8)

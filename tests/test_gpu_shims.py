@@ -211,3 +211,20 @@ def test_tensor_codec_round_trip(O, drv):
     assert np.array_equal(pay[:got], want)
     assert (sizes == 144).all()
     assert np.array_equal(dec.view(np.uint32), O.decode_tensor(fmt, want, n).view(np.uint32))
+
+
+@pytest.mark.parametrize("fmt,tail", [("Q_G_4", 100), ("Q_4", 33), ("Q_G_8", 160), ("B32S4", 96)])
+def test_tensor_codec_short_last_block(O, drv, fmt, tail):
+    """A tensor whose size is not a multiple of 256: the last block is short
+    (FormatRegistry::quantize, src/codec/format_registry.cpp:168-207)."""
+    n = 256 * 5 + tail
+    w = O.rng_normal(11, n, 0.02)
+    want = O.encode_tensor(fmt, w)
+    pay = np.zeros(want.size + 16, np.uint8)
+    sizes = np.zeros(6, np.uint32)
+    dec = np.zeros(n, np.float32)
+    got = drv.drv_tensor_round_trip(O.FMT[fmt], pf(w), n, p8(pay), pay.size, sizes.ctypes.data_as(C.POINTER(C.c_uint32)), pf(dec))
+    assert got == want.size
+    assert np.array_equal(pay[:got], want)
+    assert (sizes[:5] == O.block_bytes(fmt, 256)).all() and sizes[5] == O.block_bytes(fmt, tail)
+    assert np.array_equal(dec.view(np.uint32), O.decode_tensor(fmt, want, n).view(np.uint32))

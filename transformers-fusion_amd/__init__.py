@@ -176,12 +176,13 @@ def init(device: int = 0):
 
 
 def encode(fmt, w):
-    """fp32 device tensor (numel multiple of 256) -> uint8 device tensor of payloads."""
+    """fp32 device tensor -> uint8 device tensor of payloads (256-weight blocks, the last one possibly short)."""
     import torch
     w = w.contiguous()
     assert w.is_cuda and w.dtype == torch.float32
     n = w.numel()
-    out = torch.empty((n // 256) * block_bytes(fmt), dtype=torch.uint8, device=w.device)
+    nbytes = (n // 256) * block_bytes(fmt) + (block_bytes(fmt, n % 256) if n % 256 else 0)
+    out = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
     _check(lib().tfq_encode_blocks(fmt_id(fmt), w.data_ptr(), n, out.data_ptr(), out.numel(), _stream()))
     return out
 

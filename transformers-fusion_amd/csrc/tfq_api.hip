@@ -170,21 +170,16 @@ static int check_tensor(const char* who, uint8_t fmt, int64_t n, size_t* need, B
     return TFQ_OK;
 }
 
-static int check_blocks(const char* who, uint8_t fmt, int64_t n, size_t* need) {
-    const Spec sp = spec_of(fmt);
-    if (sp.codec == Codec::None) return fail(TFQ_ERR_FORMAT, std::string(who) + ": wire id " + std::to_string(fmt) + " is not handled");
-    if (n <= 0 || n % 256) return fail(TFQ_ERR_SHAPE, std::string(who) + ": n must be a positive multiple of 256");
-    *need = (size_t)(n / 256) * (size_t)sp.block_bytes;
-    return TFQ_OK;
-}
-
 int tfq_encode_blocks(uint8_t fmt, const float* w, int64_t n, uint8_t* dst, size_t cap, tfq_stream_t stream) {
     size_t need = 0;
+    BlockLayout tail;
     if (!w || !dst) return fail(TFQ_ERR_ARG, "tfq_encode_blocks: null pointer");
-    if (int r = check_blocks("tfq_encode_blocks", fmt, n, &need)) return r;
+    if (int r = check_tensor("tfq_encode_blocks", fmt, n, &need, &tail)) return r;
     if (cap < need) return fail(TFQ_ERR_SHAPE, "tfq_encode_blocks: destination too small");
     if (int r = ensure_device()) return r;
-    return launch_encode(fmt, w, n / 256, dst, (hipStream_t)stream);
+    if (int r = launch_encode(fmt, w, n / 256, dst, (hipStream_t)stream)) return r;
+    if (!tail.n) return TFQ_OK;
+    return launch_encode_short(fmt, tail, w + (n / 256) * 256, dst + need - (size_t)tail.bytes, (hipStream_t)stream);
 }
 
 int tfq_decode_blocks(uint8_t fmt, const uint8_t* src, size_t bytes, int64_t n, float* out, tfq_stream_t stream) {
@@ -201,8 +196,9 @@ int tfq_decode_blocks(uint8_t fmt, const uint8_t* src, size_t bytes, int64_t n, 
 
 int tfq_encode_blocks_host(uint8_t fmt, const float* w, int64_t n, uint8_t* dst, size_t cap, uint32_t* per_block_bytes) {
     size_t need = 0;
+    BlockLayout tail;
     if (!w || !dst) return fail(TFQ_ERR_ARG, "tfq_encode_blocks_host: null pointer");
-    if (int r = check_blocks("tfq_encode_blocks_host", fmt, n, &need)) return r;
+    if (int r = check_tensor("tfq_encode_blocks_host", fmt, n, &need, &tail)) return r;
     if (cap < need) return fail(TFQ_ERR_SHAPE, "tfq_encode_blocks_host: destination too small");
     if (int r = ensure_device()) return r;
     float* dw = nullptr;
@@ -212,11 +208,15 @@ int tfq_encode_blocks_host(uint8_t fmt, const float* w, int64_t n, uint8_t* dst,
     if (e != hipSuccess) { (void)hipFree(dw); return hip_fail(e, "hipMalloc"); }
     int rc = hip_fail(hipMemcpy(dw, w, (size_t)n * 4, hipMemcpyHostToDevice), "hipMemcpy H2D");
     if (!rc) rc = launch_encode(fmt, dw, n / 256, dd, nullptr);
+    if (!rc && tail.n) rc = launch_encode_short(fmt, tail, dw + (n / 256) * 256, dd + need - (size_t)tail.bytes, nullptr);
     if (!rc) rc = hip_fail(hipMemcpy(dst, dd, need, hipMemcpyDeviceToHost), "hipMemcpy D2H");
     (void)hipFree(dw);
     (void)hipFree(dd);
     if (!rc && per_block_bytes)
+    {
         for (int64_t b = 0; b < n / 256; ++b) per_block_bytes[b] = (uint32_t)spec_of(fmt).block_bytes;
+        if (tail.n) per_block_bytes[n / 256] = (uint32_t)tail.bytes;
+    }
     return rc;
 }
 

@@ -345,6 +345,8 @@ int launch_decode_short(const BlockLayout& L, const uint8_t* src, float* out, hi
 int launch_tile16(int fmt, const uint8_t* wire, uint8_t* tiled, int64_t N, int64_t K, hipStream_t s);
 int launch_decode_tiled(int fmt, const uint8_t* tiled, int64_t N, int64_t K, float* out, hipStream_t s);
 int launch_encode(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStream_t s);
+// one block of L.n < 256 weights (the last block of a tensor) in the layout L = block_layout(fmt, L.n)
+int launch_encode_short(int fmt, const BlockLayout& L, const float* w, uint8_t* dst, hipStream_t s);
 int launch_gemv(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype,
                 hipStream_t s);
 int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,

@@ -212,11 +212,13 @@ void BlockRowMatmul::mlp_step(const BlockRowMatmul& gate, const BlockRowMatmul& 
 TensorPayload TensorCodec::quantize(uint8_t wire_format, const float* data, int64_t n) {
     TensorPayload p;
     p.num_elements = n;
-    size_t per = 0;
-    if (!data || n <= 0 || n % 256 || tfq_block_bytes(wire_format, 256, &per) != TFQ_OK) return p;
+    size_t per = 0, tail = 0;
+    if (!data || n <= 0 || tfq_block_bytes(wire_format, 256, &per) != TFQ_OK) return p;
+    // the last block may be short (src/codec/format_registry.cpp:168-207)
+    if (n % 256 && tfq_block_bytes(wire_format, (uint32_t)(n % 256), &tail) != TFQ_OK) return p;
     const size_t blocks = (size_t)(n / 256);
-    p.indices.resize(blocks * per);
-    p.block_idx_bytes.resize(blocks);
+    p.indices.resize(blocks * per + tail);
+    p.block_idx_bytes.resize(blocks + (n % 256 ? 1 : 0));
     if (tfq_encode_blocks_host(wire_format, data, n, p.indices.data(), p.indices.size(), p.block_idx_bytes.data()) != TFQ_OK) {
         p.indices.clear();
         p.block_idx_bytes.clear();
@@ -229,7 +231,7 @@ TensorPayload TensorCodec::quantize(uint8_t wire_format, const float* data, int6
 void TensorCodec::dequantize(uint8_t wire_format, const TensorPayload& p, float* output, int64_t n) {
     if (!output || n <= 0) return;
     std::memset(output, 0, (size_t)n * sizeof(float));
-    if (!p.success || n % 256 || n > p.num_elements) return;
+    if (!p.success || n > p.num_elements || (n % 256 && n != p.num_elements)) return;
     tfq_decode_blocks_host(wire_format, p.indices.data(), p.indices.size(), n, output);
 }
 
