@@ -4,9 +4,14 @@
 One step = the projection GEMVs of one decode token: for each of 32 decoder
 layers (distinct weights, 3.9 GB packed in total, so nothing is served from
 cache) q 4096x4096, k/v 1024x4096, o 4096x4096, gate/up 14336x4096 and down
-4096x14336, batch 1, bf16 activations, fp32 outputs.  Weights are synthetic
-N(0, 0.02) quantized on the device to the 4-bit block-32 binary16-scale format
-(B32S4, 4.5 bits per weight); inputs are resident in HBM before timing starts.
+4096x14336, batch 1, bf16 activations, fp32 outputs.  Inputs are the seeded
+streams of the reference's generator (quant::RNG, src/core/random.cpp:45-81,
+through the library's own RNG mirror): weights RNG(42).normal() * 0.02 for one
+decoder layer, rotated by a different offset for every further layer, quantized
+on the device to the 4-bit block-32 binary16-scale format (B32S4, 4.5 bits per
+weight); activations RNG(43).normal() rounded to bf16; Laplace weights from
+RNG(44); router logits from RNG(45).  Everything is resident in HBM before
+timing starts.
 
 Prints one JSON line.  value = algorithmic bytes per step / wall time per step.
 """
@@ -51,16 +56,7 @@ def main():
                     help="skip the batch / format sweep (batch 4, 8, 16; the 8-bit format; the low-bit superblock formats)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one elementwise kernel that reads and writes 1 GiB (counter calibration)")
-    ap.add_argument("--probe", action="store_true",
-                    help="run the machine probe instead (launch floor, pure-read stream, grid barrier) and print its lines")
     args = ap.parse_args()
-    if args.probe:
-        import subprocess
-        exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "transformers-fusion_amd", "tfq_probe")
-        if not os.path.exists(exe):
-            print(f"bench.py: {exe} is missing: run __graft_entry__.build() first", file=sys.stderr)
-            sys.exit(2)
-        sys.exit(subprocess.call([exe]))
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus above 1 is not supported "
               "(rows shard over GPUs without a collective, see DESIGN.md)", file=sys.stderr)
@@ -73,21 +69,28 @@ def main():
     B, fmt = args.batch, args.fmt
     bpw = float(tfq.lib().tfq_format_bpw(tfq.fmt_id(fmt)))
 
-    gen = torch.Generator(device=dev).manual_seed(42)
+    # one decoder layer from RNG(42), the projections in PROJ order on one stream
+    total = sum(N * K for _, N, K, _ in PROJ)
+    w_all = torch.from_numpy(tfq.rng_normal(42, total, 0.02)).to(dev)
+    base, at = {}, 0
+    for name, N, K, _ in PROJ:
+        base[name] = w_all[at:at + N * K]
+        at += N * K
     layers, host_layer0 = [], {}
     for li in range(args.layers):
         ws = {}
         for name, N, K, _ in PROJ:
-            w = torch.randn(N * K, device=dev, generator=gen) * 0.02
+            w = base[name] if li == 0 else torch.roll(base[name], li * 1000003)
             packed = tfq.encode(fmt, w)
             ws[name] = tfq.Weight(fmt, N, K, packed)
             if li == 0 and not args.no_cpu:
                 host_layer0[name] = packed.cpu().numpy()  # wire payload for the CPU baseline
             del w, packed
         layers.append(ws)
-    acts = {"x": torch.randn(B, 4096, device=dev, generator=gen).bfloat16(),
-            "a": torch.randn(B, 4096, device=dev, generator=gen).bfloat16(),
-            "h": torch.randn(B, 14336, device=dev, generator=gen).bfloat16()}
+    a_all = torch.from_numpy(tfq.rng_normal(43, B * (4096 + 4096 + 14336))).to(dev)
+    acts = {"x": a_all[:B * 4096].reshape(B, 4096).bfloat16(),
+            "a": a_all[B * 4096:2 * B * 4096].reshape(B, 4096).bfloat16(),
+            "h": a_all[2 * B * 4096:].reshape(B, 14336).bfloat16()}
     outs = {name: torch.empty(B, N, device=dev, dtype=torch.float32) for name, N, _, _ in PROJ}
     torch.cuda.synchronize()
 
@@ -149,7 +152,9 @@ def main():
         "metric": "4-bit block GEMV achieved HBM GB/s, Llama-3-8B layer shapes, batch %d" % B,
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic: quant::RNG streams (seed 42 weights N(0, 0.02), one layer, rotated per layer; seed 43 "
+                "activations N(0, 1) as bf16; 44 Laplace; 45 router logits)",
         "config": {"workload": "llama3-8b decode projections (q,k,v,o,gate,up,down) x %d layers, batch %d, "
                                "%s weights, bf16 activations, fp32 outputs" % (args.layers, B, fmt),
                    "format": fmt, "layers": args.layers, "batch": B, "launch": "hipGraph" if graph else "stream"},
@@ -164,16 +169,18 @@ def main():
     }
 
     if not args.no_prefill:
-        res["prefill"] = prefill_gemm(tfq, torch, layers[0], gen)
+        res["prefill"] = prefill_gemm(tfq, torch, layers[0])
     if not args.no_sweep:
-        res["sweep"] = decode_sweep(tfq, torch, layers, fmt, gen)
+        res["sweep"] = decode_sweep(tfq, torch, layers, fmt, base)
     if not args.no_moe:
         del layers
         torch.cuda.empty_cache()
-        # a generator of its own: the routing does not depend on which other figures ran before
-        res["moe"] = moe_layer(tfq, torch, fmt, bpw, torch.Generator(device=dev).manual_seed(45))
+        res["moe"] = moe_layer(tfq, torch, fmt, bpw, base)
     if not args.no_cpu:
-        res["cpu_baseline"] = cpu_baseline(host_layer0, fmt, B, acts, bpw)
+        # the reference caps its matmul at 8 threads (src/adapters/tools/qwen35_engine.cpp:60); the second
+        # figure uses every core this process may use
+        res["cpu_baseline"] = cpu_baseline(host_layer0, fmt, B, acts, bpw, threads=min(8, usable_cores()))
+        res["cpu_baseline_all_cores"] = cpu_baseline(host_layer0, fmt, B, acts, bpw, threads=usable_cores(), budget_s=8.0)
     print(json.dumps(res), flush=True)
 
 
@@ -200,7 +207,7 @@ def time_graph(torch, fn, reps=10):
     return e0.elapsed_time(e1) * 1e3 / reps
 
 
-def decode_sweep(tfq, torch, layers, fmt, gen):
+def decode_sweep(tfq, torch, layers, fmt, base):
     """Side figures, never `value`: the decode layer of the main workload at batch 4, 8 and 16 (same weights,
     same four launches per layer), the 8-bit block-32 format at batch 1 and 16 on eight layers, and the low-bit
     superblock formats (Laplace(0, 0.015) weights, 14336x4096, twelve rotated copies) at batch 1 and 8.
@@ -209,7 +216,9 @@ def decode_sweep(tfq, torch, layers, fmt, gen):
     out = {}
 
     def layer_step(ls, B):
-        acts = {k: torch.randn(B, n, device=dev, generator=gen).bfloat16() for k, n in (("x", 4096), ("a", 4096), ("h", 14336))}
+        a_all = torch.from_numpy(tfq.rng_normal(43, B * (4096 + 4096 + 14336))).to(dev)
+        acts = {"x": a_all[:B * 4096].reshape(B, 4096).bfloat16(), "a": a_all[B * 4096:2 * B * 4096].reshape(B, 4096).bfloat16(),
+                "h": a_all[2 * B * 4096:].reshape(B, 14336).bfloat16()}
         outs = {name: torch.empty(B, N, device=dev, dtype=torch.float32) for name, N, _, _ in PROJ}
 
         def step():
@@ -229,10 +238,10 @@ def decode_sweep(tfq, torch, layers, fmt, gen):
 
     out[fmt] = {str(B): layer_figures(layers, fmt, B) for B in (4, 8, 16)}
     ls8 = []
-    for _ in range(8):
+    for li in range(8):
         ws = {}
         for name, N, K, _ in PROJ:
-            w = torch.randn(N * K, device=dev, generator=gen) * 0.02
+            w = base[name] if li == 0 else torch.roll(base[name], li * 1000003)
             ws[name] = tfq.Weight("B32S8", N, K, tfq.encode("B32S8", w))
             del w
         ls8.append(ws)
@@ -242,17 +251,19 @@ def decode_sweep(tfq, torch, layers, fmt, gen):
             W.close()
     del ls8
     N, K = 14336, 4096
+    u = torch.from_numpy(tfq.rng_uniform(44, N * K)).to(dev) - 0.5
+    lap = -0.015 * torch.sign(u) * torch.log1p(-2.0 * u.abs())  # Laplace(0, 0.015) by inverse CDF
+    del u
     for f in ("SB256A3", "SB256A2"):
         bpw = float(tfq.lib().tfq_format_bpw(tfq.fmt_id(f)))
         Ws = []
-        for _ in range(12):
-            u = torch.rand(N * K, device=dev, generator=gen) - 0.5
-            w = -0.015 * torch.sign(u) * torch.log1p(-2.0 * u.abs())
+        for c in range(12):
+            w = lap if c == 0 else torch.roll(lap, c * 1000003)
             Ws.append(tfq.Weight(f, N, K, tfq.encode(f, w)))
-            del u, w
+            del w
         out[f] = {}
         for B in (1, 8):
-            x = torch.randn(B, K, device=dev, generator=gen).bfloat16()
+            x = torch.from_numpy(tfq.rng_normal(43, B * K)).to(dev).reshape(B, K).bfloat16()
             y = torch.empty(B, N, device=dev, dtype=torch.float32)
 
             def step():
@@ -271,13 +282,13 @@ def decode_sweep(tfq, torch, layers, fmt, gen):
 MFMA_PEAK_TFLOPS = 2500.0
 
 
-def prefill_gemm(tfq, torch, layer, gen, M=2048, reps=10):
+def prefill_gemm(tfq, torch, layer, M=2048, reps=10):
     """The prefill GEMM on the same weights: M = 2048 bf16 tokens through gate (14336x4096) and down
     (4096x14336), bf16 output, fp32 accumulation on the matrix cores.  A side figure, not `value`."""
     out = {"tokens": M, "peak_tflops": MFMA_PEAK_TFLOPS, "bound": "mfma"}
     for name in ("gate", "down"):
         W = layer[name]
-        x = torch.randn(M, W.K, device="cuda", generator=gen).bfloat16()
+        x = torch.from_numpy(tfq.rng_normal(43, M * W.K)).to("cuda").reshape(M, W.K).bfloat16()
         for _ in range(3):
             y = W.gemm(x, out_dtype=torch.bfloat16)
         torch.cuda.synchronize()
@@ -295,21 +306,21 @@ def prefill_gemm(tfq, torch, layer, gen, M=2048, reps=10):
     return out
 
 
-def moe_layer(tfq, torch, fmt, bpw, gen, E=8, top_k=2, T=16, D=4096, F=14336, reps=20):
+def moe_layer(tfq, torch, fmt, bpw, base, E=8, top_k=2, T=16, D=4096, F=14336, reps=20):
     """One mixture-of-experts FFN call (router top-k given on the host, like the reference's dispatch):
     16 tokens, 8 experts, top-2, gate/up 14336x4096 and down 4096x14336 per expert.  Wall time per call
     including the host-side routing lists; bytes = packed weights of the active experts.  A side figure."""
     import numpy as np
     gate, up, down = [], [], []
-    for _ in range(E):
-        for lst, n, k in ((gate, F, D), (up, F, D), (down, D, F)):
-            w = torch.randn(n * k, device="cuda", generator=gen) * 0.02
+    for e in range(E):  # expert e = the layer's gate / up / down stream rotated by e * 1000003 elements
+        for lst, name, n, k in ((gate, "gate", F, D), (up, "up", F, D), (down, "down", D, F)):
+            w = base[name] if e == 0 else torch.roll(base[name], e * 1000003)
             lst.append(tfq.Weight(fmt, n, k, tfq.encode(fmt, w)))
             del w
-    logits = torch.randn(T, E, device="cuda", generator=gen)
+    logits = torch.from_numpy(tfq.rng_normal(45, T * E)).to("cuda").reshape(T, E)
     _, idx, wts = tfq.moe_route(logits, top_k)
     idx_h, w_h = idx.cpu().numpy().astype(np.int64), wts.cpu().numpy()
-    x = torch.randn(T, D, device="cuda", generator=gen).bfloat16()
+    x = torch.from_numpy(tfq.rng_normal(43, T * D)).to("cuda").reshape(T, D).bfloat16()
     for _ in range(3):
         tfq.moe_ffn(gate, up, down, idx_h, w_h, x, mid_dtype=torch.bfloat16)
     torch.cuda.synchronize()
@@ -326,13 +337,21 @@ def moe_layer(tfq, torch, fmt, bpw, gen, E=8, top_k=2, T=16, D=4096, F=14336, re
             "frac": round(nbytes / dt / 1e9 / HBM_PEAK_GBS, 4), "bound": "hbm"}
 
 
-def cpu_baseline(layer, fmt, B, acts, bpw, budget_s=12.0):
+def usable_cores():
+    """Cores this process may run on (the scheduler affinity), at most 16: a one-GPU box gives a job that share."""
+    try:
+        n = len(os.sched_getaffinity(0))
+    except AttributeError:
+        n = os.cpu_count() or 1
+    return max(1, min(16, n))
+
+
+def cpu_baseline(layer, fmt, B, acts, bpw, threads, budget_s=12.0):
     """The oracle's block-row matmul (reference loop structure: rows split over threads,
     decode 256 weights, 256-long fp32 dot per activation row) on the host cores, on a
     bounded sample: the seven projections of ONE decoder layer, repeated until about
-    `budget_s` seconds of CPU work have been timed.  Threads = the reference's own cap of 8."""
+    `budget_s` seconds of CPU work have been timed, on `threads` threads."""
     import oracle as O
-    threads = min(8, os.cpu_count() or 1)
     xs = {k: v.float().cpu().numpy() for k, v in acts.items()}
     total_b, total_t, passes = 0.0, 0.0, 0
     while total_t < budget_s and passes < 400:

@@ -124,4 +124,28 @@ struct TensorCodec {
     static void dequantize(uint8_t wire_format, const TensorPayload& p, float* output, int64_t n);
 };
 
+// The generator of seeded synthetic inputs, quant::RNG (include/quant/random.h:27-46,
+// src/core/random.cpp:45-81): splitmix64 of the seed fills the two words of a xoroshiro128+
+// state; uniform() = (next >> 11) * 2^-53 as a float; normal() = Box-Muller on two uniform
+// draws in binary32 with the first floored at 1e-10.  Host arithmetic, as in the reference:
+// benchmarks and tests draw weights and activations from it so that both sides of a comparison
+// see the same numbers.
+class RNG {
+public:
+    explicit RNG(uint64_t seed = 42);
+    void seed(uint64_t s);
+    float uniform();
+    float normal();
+    uint64_t next_u64();
+
+private:
+    uint64_t s[2];
+};
+
 }  // namespace tfq
+
+extern "C" {
+/* n draws of RNG(seed): normal() * scale, or uniform(), into a host buffer. */
+void tfq_rng_normal(uint64_t seed, int64_t n, float scale, float* out);
+void tfq_rng_uniform(uint64_t seed, int64_t n, float* out);
+}

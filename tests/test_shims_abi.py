@@ -53,3 +53,18 @@ def test_the_compiled_reference_defines_the_same_names():
     have = defined(REF)
     missing = [s for s in EXPECTED if s not in have]
     assert not missing, missing
+
+
+def test_library_generator_matches_the_reference_streams():
+    """tfq::RNG (the library's mirror of quant::RNG, src/core/random.cpp:45-81) against the streams the
+    compiled reference wrote (tests/golden/rng.npz).  Host arithmetic: no GPU needed."""
+    import importlib
+
+    import numpy as np
+    if not os.path.exists(SHIMS):
+        pytest.skip("libtfq_shims.so not built")
+    tfq = importlib.import_module("transformers-fusion_amd")
+    r = np.load(os.path.join(ROOT, "tests", "golden", "rng.npz"))
+    assert np.array_equal(tfq.rng_uniform(42, 4096).view(np.uint32), r["uniform_42"].view(np.uint32))
+    assert np.array_equal(tfq.rng_normal(42, 4096, 0.02).view(np.uint32), r["normal_42_002"].view(np.uint32))
+    assert np.array_equal(tfq.rng_normal(43, 4096, 1.0).view(np.uint32), r["normal_43"].view(np.uint32))

@@ -142,6 +142,41 @@ def lib():
     return _lib
 
 
+SHIMS_PATH = os.path.join(_HERE, "libtfq_shims.so")
+_shims = None
+
+
+def shims():
+    """libtfq_shims.so: the reference-named host C++ entry points and the seeded generator."""
+    global _shims
+    if _shims is None:
+        lib()  # libtfq.so first: the shim library links against it
+        if not os.path.exists(SHIMS_PATH):
+            raise TfqError(f"{SHIMS_PATH} is missing: run __graft_entry__.build() first")
+        s = C.CDLL(SHIMS_PATH)
+        s.tfq_rng_normal.argtypes = [C.c_uint64, C.c_int64, C.c_float, C.c_void_p]
+        s.tfq_rng_normal.restype = None
+        s.tfq_rng_uniform.argtypes = [C.c_uint64, C.c_int64, C.c_void_p]
+        s.tfq_rng_uniform.restype = None
+        _shims = s
+    return _shims
+
+
+def rng_normal(seed: int, n: int, scale: float = 1.0):
+    """n draws of quant::RNG(seed).normal() * scale as a float32 numpy array (src/core/random.cpp:45-81)."""
+    import numpy as np
+    out = np.empty(n, np.float32)
+    shims().tfq_rng_normal(seed, n, scale, out.ctypes.data)
+    return out
+
+
+def rng_uniform(seed: int, n: int):
+    import numpy as np
+    out = np.empty(n, np.float32)
+    shims().tfq_rng_uniform(seed, n, out.ctypes.data)
+    return out
+
+
 def _check(rc: int):
     if rc != 0:
         raise TfqError(f"tfq error {rc}: {lib().tfq_last_error().decode()}")

@@ -72,25 +72,6 @@ def build_shims(verbose: bool = False) -> str:
     return SHIMS
 
 
-PROBE = os.path.join(HERE, "tfq_probe")
-
-
-def build_probe(verbose: bool = False) -> str:
-    """The machine probe bench.py --probe runs (launch floor, read stream, grid barrier); not part of the library."""
-    cmd = [hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++20", "-Xclang", "-target-feature", "-Xclang",
-           "-packed-fp32-ops", os.path.join(CSRC, "tfq_probe.hip"), "-o", PROBE]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    text = "\n".join(l for l in out.stdout.splitlines() if "packed-fp32-ops" not in l)
-    if text.strip():
-        print(text, flush=True)
-    if out.returncode:
-        raise RuntimeError("hipcc failed on the probe")
-    return PROBE
-
-
 if __name__ == "__main__":
     print(build_library(verbose=True))
     print(build_shims(verbose=True))
-    print(build_probe(verbose=True))

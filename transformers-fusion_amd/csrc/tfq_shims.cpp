@@ -1,7 +1,8 @@
 // Definitions of the reference-named entry points declared in include/tfq_shims.hpp.
 // Host C++ only (built with g++, linked against libtfq.so): each function moves the
 // caller's host buffers to the device through the C ABI, runs the HIP path and
-// moves the result back.  There is no CPU computation in this file.
+// moves the result back.  The only arithmetic on the host is the generator of seeded
+// synthetic inputs (tfq::RNG), which is host code in the reference too.
 
 #include "../../include/tfq_shims.hpp"
 
@@ -235,4 +236,54 @@ void TensorCodec::dequantize(uint8_t wire_format, const TensorPayload& p, float*
     tfq_decode_blocks_host(wire_format, p.indices.data(), p.indices.size(), n, output);
 }
 
+namespace {
+uint64_t splitmix64(uint64_t& st) {
+    uint64_t z = (st += 0x9e3779b97f4a7c15ULL);
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ULL;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebULL;
+    return z ^ (z >> 31);
+}
+inline uint64_t rotl64(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
+}  // namespace
+
+RNG::RNG(uint64_t sd) { seed(sd); }
+
+void RNG::seed(uint64_t sd) {
+    s[0] = splitmix64(sd);
+    s[1] = splitmix64(sd);
+}
+
+uint64_t RNG::next_u64() {
+    const uint64_t a = s[0];
+    uint64_t b = s[1];
+    const uint64_t r = a + b;
+    b ^= a;
+    s[0] = rotl64(a, 24) ^ b ^ (b << 16);
+    s[1] = rotl64(b, 37);
+    return r;
+}
+
+float RNG::uniform() { return (float)(next_u64() >> 11) * (1.0f / 9007199254740992.0f); }
+
+float RNG::normal() {
+    float u1 = uniform();
+    const float u2 = uniform();
+    if (u1 < 1e-10f) u1 = 1e-10f;
+    return std::sqrt(-2.0f * std::log(u1)) * std::cos(6.283185307179586f * u2);
+}
+
 }  // namespace tfq
+
+extern "C" {
+
+void tfq_rng_normal(uint64_t seed, int64_t n, float scale, float* out) {
+    tfq::RNG r(seed);
+    for (int64_t i = 0; i < n; ++i) out[i] = r.normal() * scale;
+}
+
+void tfq_rng_uniform(uint64_t seed, int64_t n, float* out) {
+    tfq::RNG r(seed);
+    for (int64_t i = 0; i < n; ++i) out[i] = r.uniform();
+}
+
+}  // extern "C"
