@@ -247,6 +247,27 @@ size_t tfq_gemm_static_scratch_bytes(void);
  * same input (src/adapters/tools/qwen35_engine.cpp:662-672 for gate/up). */
 int tfq_gemv_multi(const tfq_weight_t* const* ws, int count, const void* x, int x_dtype, int B,
                    void* const* ys, int y_dtype, tfq_stream_t stream);
+/* tfq_gemv_multi with an elementwise step of the reference engine applied to the activations while the
+ * kernel stages them, so the step costs no launch and no round trip through memory.  x is fp32 [B][K],
+ * B <= 16 (two rows ride in one pass over the weights, like every fp32 input).
+ *   TFQ_PRO_RMSNORM  x * rsqrt(mean(x^2) + eps) * gamma, or * (1 + gamma) with gamma_plus_one, the form of
+ *                    Qwen35Engine::rmsnorm (src/adapters/tools/qwen35_engine.cpp:46-51), in front of the
+ *                    q/k/v and the gate/up products
+ *   TFQ_PRO_SWIGLU   x is the gate product and `up` the up product, both fp32 [B][K]: silu(x) * up
+ *                    (Qwen35Engine::mlp_step :662-672, math::silu src/math/math.cpp:117-126) in front of the
+ *                    down product; mid_dtype TFQ_BF16 rounds the product to bf16 first, TFQ_F32 keeps it
+ * Formats with a tiled matrix-core kernel only (TFQ_ERR_FORMAT otherwise). */
+enum { TFQ_PRO_NONE = 0, TFQ_PRO_RMSNORM = 1, TFQ_PRO_SWIGLU = 2 };
+typedef struct tfq_prologue {
+    int op;
+    const float* gamma; /* RMSNORM: [K] */
+    float eps;
+    int gamma_plus_one;
+    const float* up;    /* SWIGLU: [B][K] */
+    int mid_dtype;      /* SWIGLU: TFQ_F32 or TFQ_BF16 */
+} tfq_prologue_t;
+int tfq_gemv_multi_fused(const tfq_weight_t* const* ws, int count, const float* x, int B, void* const* ys,
+                         int y_dtype, const tfq_prologue_t* prologue, tfq_stream_t stream);
 /* host-pointer form of tfq_gemv/tfq_gemm with fp32 x and y: the exact call
  * shape of Qwen35Engine::gemm(t, X, Y, B). */
 int tfq_matmul_host(const tfq_weight_t* w, const float* X, float* Y, int B);
@@ -255,8 +276,10 @@ int tfq_matmul_host(const tfq_weight_t* w, const float* X, float* Y, int B);
  * Qwen35Engine::mlp_step (src/adapters/tools/qwen35_engine.cpp:662-672) for B rows:
  *   y[b] = down( silu(gate x[b]) * (up x[b]) ),  silu(v) = v / (1 + exp(-v))
  * (src/math/math.cpp:117-126).  gate and up are F x D matrices of one format, down is D x F;
- * x is [B][D], y is [B][D], device pointers.  Three launches: gate and up in one (they share x),
- * the elementwise step, down.  mid_dtype is the type the SwiGLU product is rounded to before
+ * x is [B][D], y is [B][D], device pointers.  Up to 16 rows and a format with a tiled kernel: two
+ * launches, gate and up in one (they share x) and down with silu(gate) * up applied while it stages
+ * its activations; otherwise gate / up, the elementwise step and down are launches of their own.
+ * mid_dtype is the type the SwiGLU product is rounded to before
  * the down projection: TFQ_F32 keeps it in fp32 like the reference, TFQ_BF16 feeds the matrix
  * cores.  workspace is device memory of at least tfq_mlp_workspace_bytes(B, F) bytes, 256-byte
  * aligned (the gate and up products and the SwiGLU product live there). */

@@ -389,3 +389,66 @@ def test_long_k_takes_fewer_rows_per_pass(O, tfq, gpu, K, B, xdt):
         ym = W.gemm(torch.from_numpy(np.concatenate([x, x])).to(gpu), workspace=False).cpu().numpy()
         assert float(np.abs(ym[:B] - ref).max() / np.abs(ref).max()) <= tol
     W.close()
+
+
+def _rmsnorm_ref(x, w, eps=1e-6, plus_one=True):
+    """Qwen35Engine::rmsnorm (src/adapters/tools/qwen35_engine.cpp:46-51): x * 1/sqrt(sum(x^2)/n + eps) * (1 + w),
+    fp32 with the reference's sequential sum."""
+    x = x.astype(np.float32)
+    s = np.float32(0)
+    for v in x:
+        s = np.float32(s + v * v)
+    r = np.float32(1.0) / np.sqrt(np.float32(s / np.float32(x.size) + np.float32(eps)), dtype=np.float32)
+    g = (np.float32(1) + w) if plus_one else w
+    return ((x * r) * g).astype(np.float32)
+
+
+@pytest.mark.parametrize("fmt", ["B32S4", "Q_G_4", "B32S8", "SB256A3"])
+@pytest.mark.parametrize("B,plus_one", [(1, True), (2, False), (5, True)])
+def test_rmsnorm_prologue_matches_oracle(O, tfq, gpu, fmt, B, plus_one):
+    """rmsnorm -> q, k, v in one launch against the oracle's rmsnorm + fp32 matmul; fp32 activations, 1e-3."""
+    import torch
+    K = 2048
+    shapes = [("q", 1024, K), ("k", 256, K), ("v", 272, K)]
+    pays = {n: O.encode_tensor(fmt, O.rng_normal(60 + i, N * K, 0.02)) for i, (n, N, _) in enumerate(shapes)}
+    Ws = [tfq.Weight(fmt, N, K, pays[n]) for n, N, _ in shapes]
+    x = O.rng_normal(43, B * K, 1.5).reshape(B, K)
+    gamma = O.rng_normal(44, K, 0.2)
+    outs = [torch.zeros(B, N, device=gpu) for _, N, _ in shapes]
+    tfq.gemv_multi_fused(Ws, torch.from_numpy(x).to(gpu), outs, rmsnorm=torch.from_numpy(gamma).to(gpu), eps=1e-6,
+                         gamma_plus_one=plus_one)
+    xn = np.stack([_rmsnorm_ref(x[b], gamma, 1e-6, plus_one) for b in range(B)])
+    for (n, N, _), o in zip(shapes, outs):
+        ref = O.matmul(fmt, pays[n], N, K, xn)
+        got = o.cpu().numpy()
+        assert np.abs(got - ref).max() / np.abs(ref).max() <= 1e-3, (n, fmt)
+
+
+@pytest.mark.parametrize("fmt", ["B32S4", "Q_G_4"])
+@pytest.mark.parametrize("B,mid", [(1, "f32"), (2, "bf16"), (3, "f32")])
+def test_swiglu_prologue_matches_oracle(O, tfq, gpu, fmt, B, mid):
+    """down(silu(g) * u) with the elementwise step inside the down launch (Qwen35Engine::mlp_step)."""
+    import torch
+    F, D = 3584, 1024
+    pay = O.encode_tensor(fmt, O.rng_normal(70, D * F, 0.02))
+    W = tfq.Weight(fmt, D, F, pay)
+    g = O.rng_normal(71, B * F, 1.0).reshape(B, F)
+    u = O.rng_normal(72, B * F, 1.0).reshape(B, F)
+    y = torch.zeros(B, D, device=gpu)
+    tfq.gemv_multi_fused([W], torch.from_numpy(g).to(gpu), [y], swiglu_up=torch.from_numpy(u).to(gpu),
+                         mid_dtype=torch.bfloat16 if mid == "bf16" else torch.float32)
+    h = O.silu_mul(g.reshape(-1), u.reshape(-1)).reshape(B, F)
+    if mid == "bf16":
+        h = O.bf16_round(h)
+    ref = O.matmul(fmt, pay, D, F, h)
+    tol = 1e-2 if mid == "bf16" else 1e-3
+    assert np.abs(y.cpu().numpy() - ref).max() / np.abs(ref).max() <= tol
+
+
+def test_prologue_rejects_untiled_formats(O, tfq, gpu):
+    import torch
+    pay = O.encode_tensor("Q_4", O.rng_normal(1, 256 * 256, 0.02))
+    W = tfq.Weight("Q_4", 256, 256, pay)
+    with pytest.raises(tfq.TfqError):
+        tfq.gemv_multi_fused([W], torch.zeros(1, 256, device=gpu), [torch.zeros(1, 256, device=gpu)],
+                             rmsnorm=torch.zeros(256, device=gpu))

@@ -66,7 +66,16 @@ struct GemvArgs {
     int cols_base, cols_rem;  // block columns per wavefront: cols_base + (wave < cols_rem)
     float* split_partial;     // single matrix only: the handle's partial sums and arrival counters, or null
     unsigned* split_counters;
+    // prologue fused into the activation staging (fp32 input only): XOP_RMSNORM takes gamma / eps /
+    // gamma_plus_one, XOP_SWIGLU takes x2 (the up product; x is the gate product) and mid_bf16
+    int xop;
+    const float* gamma;
+    const float* x2;
+    float eps;
+    int gamma_plus_one, mid_bf16;
 };
+
+enum : int { XOP_NONE = 0, XOP_RMSNORM = 1, XOP_SWIGLU = 2 };
 
 // What the kernel receives, flattened.  No arrays on purpose: a chain of selects over array
 // elements is folded by the optimizer into an indexed read of the argument block, which costs a
@@ -81,6 +90,10 @@ struct GemvKernArgs {
     int kparts, kcols;  // gemvb_kernel: workgroups per row group (K parts) and block columns per part
     float* partial;
     unsigned* counters;
+    const float* gamma;  // XOP_RMSNORM
+    const float* x2;     // XOP_SWIGLU: the second factor, same shape as x
+    float eps;
+    int gamma_plus_one, mid_bf16;
 };
 
 // Grouped launch: many independent problems (matrix, activation rows, output) of one format and
@@ -101,10 +114,19 @@ struct GemvProb {
 // chooses WD <= the number of units of a full wavefront (a short one re-reads a unit it never uses).
 // SETS = sets of four activation slots that ride in one pass (1, 2 or 4: up to 16 bf16 rows).  More
 // than one set keeps that many A fragments in registers, which fits at 8 wavefronts per workgroup.
-template <int FMT, bool XF32, int WD, int SETS = 1, bool GROUPED = false>
+// XOP = a prologue applied while the activations are staged (fp32 input, one slot set):
+//   XOP_RMSNORM  x * (1 + gamma) (or * gamma) is staged, every wavefront adds the squares of its slice, and the
+//                outputs are multiplied by 1 / sqrt(mean(x^2) + eps) when the partial sums are added: the factor
+//                is a scalar per activation row, so it commutes with the product (Qwen35Engine::rmsnorm,
+//                src/adapters/tools/qwen35_engine.cpp:46-51, in front of the q/k/v and gate/up products)
+//   XOP_SWIGLU   x is the gate product and x2 the up product: silu(x) * x2 is staged (math::silu and the
+//                elementwise product of Qwen35Engine::mlp_step, qwen35_engine.cpp:662-672), in fp32 (split into
+//                a bf16 high and low part like every fp32 input) or rounded to bf16 (mid_bf16)
+template <int FMT, bool XF32, int WD, int SETS = 1, bool GROUPED = false, int XOP = XOP_NONE>
 __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin_arg) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
+    static_assert(XOP == XOP_NONE || (XF32 && SETS == 1 && !GROUPED), "prologues take fp32 input in the plain launch");
     constexpr int UB = tiled_unit_bytes(FMT);  // bytes of a unit
     constexpr int NC = 2 * F::NP;              // 1 KB code pieces of a unit: [plane][k-step]
     constexpr int NG = F::NG, PER = NG / 2;  // scale groups per block / per k-step
@@ -160,7 +182,7 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     // A pass covers two activation slots of one block column: lane l < 32 owns the 8-element quad l
     // of slot s0, lane l + 32 the same quad of slot s0 + 1 (clamped to the last slot: the load is
     // unconditional and staging drops what it does not need).
-    constexpr int XP = 4;  // passes whose loads are issued before the weight stream
+    constexpr int XP = XOP == XOP_NONE ? 4 : 2;  // passes whose loads are issued before the weight stream
     const int quad = lane & 31, sl_in_pass = lane >> 5;
     // passes per block column: a power of two, so that a pass index splits with shifts
     const int npc = SETS == 1 ? (nslot + 1) >> 1 : 2 * SETS;
@@ -169,23 +191,35 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     constexpr int XE = XF32 ? 4 : 2;   // bytes per activation element
     const uint8_t* xbytes = static_cast<const uint8_t*>(xin);
     // per-lane byte offset inside a pass, and the per-pass scalar offset
-    auto x_load = [&](int pass, uint4& lo, uint4& hi) __attribute__((always_inline)) {
+    // (lo2, hi2): the second operand of a prologue, the same eight elements of x2, or of gamma (which has one row)
+    auto x_load = [&](int pass, uint4& lo, uint4& hi, uint4& lo2, uint4& hi2) __attribute__((always_inline)) {
         const int ci = pass >> npc_shift;
         const int s0 = (pass & (npc - 1)) * 2;
         const int s = min(s0 + sl_in_pass, nslot - 1);
         const int row = XF32 ? s >> 1 : s;
         const uint32_t lane_off = ((uint32_t)row * (uint32_t)K + (uint32_t)quad * 8u) * XE;
-        const uint8_t* base = xbytes + (size_t)(wave + NW * ci) * (256 * XE);
-        const uint4* src = reinterpret_cast<const uint4*>(base + lane_off);
+        const size_t col_off = (size_t)(wave + NW * ci) * (256 * XE);
+        const uint4* src = reinterpret_cast<const uint4*>(xbytes + col_off + lane_off);
         lo = src[0];
         if constexpr (XF32) hi = src[1];
+        if constexpr (XOP == XOP_SWIGLU) {
+            const uint4* src2 = reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(args.x2) + col_off + lane_off);
+            lo2 = src2[0];
+            hi2 = src2[1];
+        } else if constexpr (XOP == XOP_RMSNORM) {
+            const uint4* src2 = reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(args.gamma) + col_off + (size_t)quad * 32u);
+            lo2 = src2[0];
+            hi2 = src2[1];
+        }
     };
-    uint4 pxlo[XP], pxhi[XP];
+    constexpr int XP2 = XOP == XOP_NONE ? 1 : XP;
+    uint4 pxlo[XP], pxhi[XP], px2lo[XP2], px2hi[XP2];
 #pragma unroll
     for (int p = 0; p < XP; ++p) {
         pxlo[p] = uint4{0, 0, 0, 0};
         pxhi[p] = uint4{0, 0, 0, 0};
-        if (p < npass) x_load(p, pxlo[p], pxhi[p]);
+        if constexpr (XOP != XOP_NONE) { px2lo[p] = uint4{0, 0, 0, 0}; px2hi[p] = uint4{0, 0, 0, 0}; }
+        if (p < npass) x_load(p, pxlo[p], pxhi[p], px2lo[XOP == XOP_NONE ? 0 : p], px2hi[XOP == XOP_NONE ? 0 : p]);
     }
 
     // ---- unit fetch cursor: a pointer that walks the tiles of a block column, then moves to the
@@ -221,7 +255,10 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     // ---- stage this wavefront's activations: bf16 in nibble-pair order, group sums beside them
     const uint32_t ONES = 0x3F803F80u;
     if (lane < 4) zero4[lane] = uint4{0, 0, 0, 0};
-    auto stage = [&](int pass, uint4 xlo, uint4 xhi) __attribute__((always_inline)) {
+    float ssq0 = 0.0f, ssq1 = 0.0f;  // XOP_RMSNORM: this lane's share of sum(x^2) of activation rows 0 and 1
+    const bool mid_bf16 = XOP == XOP_SWIGLU && args.mid_bf16 != 0;
+    const bool plus_one = XOP == XOP_RMSNORM && args.gamma_plus_one != 0;
+    auto stage = [&](int pass, uint4 xlo, uint4 xhi, uint4 x2lo, uint4 x2hi) __attribute__((always_inline)) {
         const int ci = pass >> npc_shift;
         const int s = (pass & (npc - 1)) * 2 + sl_in_pass;
         uint4* col = my + (size_t)ci * col_stride;
@@ -230,14 +267,32 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
         if (s < nslot) {
             uint4 v = xlo;
             if constexpr (XF32) {
-                const float f[8] = {__uint_as_float(xlo.x), __uint_as_float(xlo.y), __uint_as_float(xlo.z),
-                                    __uint_as_float(xlo.w), __uint_as_float(xhi.x), __uint_as_float(xhi.y),
-                                    __uint_as_float(xhi.z), __uint_as_float(xhi.w)};
+                float f[8] = {__uint_as_float(xlo.x), __uint_as_float(xlo.y), __uint_as_float(xlo.z),
+                              __uint_as_float(xlo.w), __uint_as_float(xhi.x), __uint_as_float(xhi.y),
+                              __uint_as_float(xhi.z), __uint_as_float(xhi.w)};
+                if constexpr (XOP != XOP_NONE) {
+                    const float f2[8] = {__uint_as_float(x2lo.x), __uint_as_float(x2lo.y), __uint_as_float(x2lo.z),
+                                         __uint_as_float(x2lo.w), __uint_as_float(x2hi.x), __uint_as_float(x2hi.y),
+                                         __uint_as_float(x2hi.z), __uint_as_float(x2hi.w)};
+                    if constexpr (XOP == XOP_SWIGLU) {
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) f[t] = f[t] / (1.0f + expf(-f[t])) * f2[t];
+                    } else {
+                        float ss = 0.0f;
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) {
+                            ss = __builtin_fmaf(f[t], f[t], ss);
+                            f[t] *= plus_one ? 1.0f + f2[t] : f2[t];
+                        }
+                        // the high and the low slot of a row see the same elements: the high slot counts them
+                        if (!(s & 1)) { if ((pass & (npc - 1)) == 0) ssq0 += ss; else ssq1 += ss; }
+                    }
+                }
                 uint32_t e[8];
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
                     const uint32_t hb = bf16_rne(f[t]);
-                    e[t] = (s & 1) ? bf16_rne(f[t] - __uint_as_float(hb << 16)) : hb;
+                    e[t] = (s & 1) ? (mid_bf16 ? 0u : bf16_rne(f[t] - __uint_as_float(hb << 16))) : hb;
                 }
                 v.x = e[0] | (e[1] << 16); v.y = e[2] | (e[3] << 16);
                 v.z = e[4] | (e[5] << 16); v.w = e[6] | (e[7] << 16);
@@ -260,11 +315,22 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     };
 #pragma unroll
     for (int p = 0; p < XP; ++p)
-        if (p < npass) stage(p, pxlo[p], pxhi[p]);
+        if (p < npass) stage(p, pxlo[p], pxhi[p], px2lo[XOP == XOP_NONE ? 0 : p], px2hi[XOP == XOP_NONE ? 0 : p]);
     for (int p = XP; p < npass; ++p) {
-        uint4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
-        x_load(p, lo, hi);
-        stage(p, lo, hi);
+        uint4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0}, lo2 = {0, 0, 0, 0}, hi2 = {0, 0, 0, 0};
+        x_load(p, lo, hi, lo2, hi2);
+        stage(p, lo, hi, lo2, hi2);
+    }
+    // sums of squares of this wavefront's slices, behind the partial sums
+    float* ssq_lds = part + (size_t)T * NW * SETS * 64;
+    if constexpr (XOP == XOP_RMSNORM) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            float v = b ? ssq1 : ssq0;
+            v += __shfl_xor(v, 1); v += __shfl_xor(v, 2); v += __shfl_xor(v, 4);
+            v += __shfl_xor(v, 8); v += __shfl_xor(v, 16); v += __shfl_xor(v, 32);
+            if (lane == 0) ssq_lds[wave * 2 + b] = v;
+        }
     }
 
     // ---- per-lane operand addressing
@@ -382,6 +448,11 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
         for (int w = 0; w < NW; ++w) {
 #pragma unroll
             for (int h = 0; h < rows_per_out; ++h) v += src[w * SETS * 64 + h * 16];
+        }
+        if constexpr (XOP == XOP_RMSNORM) {
+            float tot = 0.0f;
+            for (int w = 0; w < NW; ++w) tot += ssq_lds[w * 2 + b];
+            v *= 1.0f / sqrtf(tot / (float)K + args.eps);
         }
         const size_t off = (size_t)b * (size_t)nrm + (size_t)row;
         if (y_bf16) reinterpret_cast<unsigned short*>(ym)[off] = (unsigned short)bf16_rne(v);
@@ -755,10 +826,10 @@ GemvPlan plan_gemv4(const GemvArgs& a, int nslot) {
         return g;
     };
     int T = (a.ntiles + num_cu - 1) / num_cu;
-    while (grid_for(T) > num_cu && x_bytes + (size_t)(T + 1) * per_tile <= 160 * 1024) ++T;
-    while (T > 1 && x_bytes + (size_t)T * per_tile > 160 * 1024) --T;
+    while (grid_for(T) > num_cu && x_bytes + (size_t)(T + 1) * per_tile + 128 <= 160 * 1024) ++T;
+    while (T > 1 && x_bytes + (size_t)T * per_tile + 128 > 160 * 1024) --T;
     p.T = T;
-    p.lds = x_bytes + (size_t)T * per_tile;
+    p.lds = x_bytes + (size_t)T * per_tile + 128;  // + the wavefronts' sums of squares (RMSNorm prologue)
     if (p.lds > 160 * 1024) p.lds = 0;
     return p;
 }
@@ -786,6 +857,7 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     if (a.nmat == 4) grid += ((a.nrows[3] + 15) / 16 + T - 1) / T;
     k.K = a.K; k.y_bf16 = a.y_bf16; k.nslot = a.nslot; k.tiles_per_wg = T;
     k.cols_base = a.cols_base; k.cols_rem = a.cols_rem;
+    k.gamma = a.gamma; k.x2 = a.x2; k.eps = a.eps; k.gamma_plus_one = a.gamma_plus_one; k.mid_bf16 = a.mid_bf16;
     const int full_items = a.cols_base * T;  // units of a wavefront with the fewest block columns in a full workgroup
     // Two unit fetches in flight per wavefront at most.  Sixteen wavefronts already keep 32 units (74 KB) per
     // compute unit on their way; four per wavefront (which only the one-plane formats with a 16-byte header
@@ -800,6 +872,14 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     const int xi = a.x_f32 ? 1 : 0, wi = wd == 4 ? 2 : wd == 2 ? 1 : 0;
     Kernel kern = kernels[xi][wi];
     int slot = xi * 3 + wi;  // which kernel's LDS limit is being raised
+    if (a.xop != XOP_NONE) {
+        static const Kernel fused[2][2] = {
+            {gemv4_kernel<FMT, true, 1, 1, false, XOP_RMSNORM>, gemv4_kernel<FMT, true, 2, 1, false, XOP_RMSNORM>},
+            {gemv4_kernel<FMT, true, 1, 1, false, XOP_SWIGLU>, gemv4_kernel<FMT, true, 2, 1, false, XOP_SWIGLU>}};
+        if (!a.x_f32 || p.sets != 1) return fail(TFQ_ERR_SHAPE, "gemv: a prologue takes fp32 input, two rows per pass");
+        kern = fused[a.xop - 1][wd == 2 ? 1 : 0];
+        slot = 8 + (a.xop - 1) * 2 + (wd == 2 ? 1 : 0);
+    } else
     if constexpr (kWide<FMT>) {
         if (p.sets > 1) {
             kern = p.sets == 2 ? gemv4_kernel<FMT, false, 2, 2> : gemv4_kernel<FMT, false, 1, 4>;
@@ -817,7 +897,7 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     }
     // Raise the dynamic-LDS limit once per kernel (not per launch: the call is
     // not allowed while a stream is being captured into a graph).
-    static std::atomic<bool> lds_limit_raised[8] = {};
+    static std::atomic<bool> lds_limit_raised[12] = {};
     if (!lds_limit_raised[slot]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -927,6 +1007,7 @@ int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t 
         ab.nslot = a.x_f32 ? 2 * nb : nb;
         for (int m = 0; m < a.nmat; ++m) ab.y[m] = (uint8_t*)a.y[m] + (size_t)b0 * (size_t)a.nrows[m] * ye;
         const void* xb = (const uint8_t*)x + (size_t)b0 * a.K * xe;
+        if (a.x2) ab.x2 = a.x2 + (size_t)b0 * a.K;
         if (int rc = run_gemv4<FMT>(ab, xb, s)) return rc;
     }
     return TFQ_OK;
@@ -1056,6 +1137,19 @@ int launch_gemv_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, c
 
 int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
                       void* const* ys, int y_dtype, hipStream_t s) {
+    return launch_gemv_multi_fused(ws, nmat, x, x_dtype, B, ys, y_dtype, nullptr, s);
+}
+
+bool gemv_prologue_supported(const tfq_weight* w) { return w->layout == TFQ_LAYOUT_TILED16; }
+
+int launch_gemv_multi_fused(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
+                            void* const* ys, int y_dtype, const tfq_prologue_t* pro, hipStream_t s) {
+    const bool fused = pro && pro->op != TFQ_PRO_NONE;
+    if (fused) {
+        if (x_dtype != TFQ_F32) return fail(TFQ_ERR_ARG, "gemv: a prologue takes fp32 activations");
+        if (ws[0]->layout != TFQ_LAYOUT_TILED16)
+            return fail(TFQ_ERR_FORMAT, std::string("gemv: no fused prologue for format ") + tfq_format_name(ws[0]->fmt));
+    }
     if (ws[0]->layout == TFQ_LAYOUT_MIXED) {  // blocks of several formats: one launch per matrix
         for (int m = 0; m < nmat; ++m) {
             if (ws[m]->layout != TFQ_LAYOUT_MIXED) return fail(TFQ_ERR_SHAPE, "gemv: matrices of one launch must share their layout");
@@ -1091,6 +1185,11 @@ int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int 
     if (nmat == 1) {
         a.split_partial = ws[0]->split_partial;
         a.split_counters = ws[0]->split_counters;
+    }
+    if (fused) {
+        a.xop = pro->op == TFQ_PRO_RMSNORM ? XOP_RMSNORM : XOP_SWIGLU;
+        a.gamma = pro->gamma; a.x2 = pro->up; a.eps = pro->eps;
+        a.gamma_plus_one = pro->gamma_plus_one; a.mid_bf16 = pro->mid_dtype == TFQ_BF16;
     }
     switch (canonical(ws[0]->fmt)) {
         case TFQ_Q_G_4: return gemv4_batched<TFQ_Q_G_4>(a, x, x_dtype, B, y_dtype, s);

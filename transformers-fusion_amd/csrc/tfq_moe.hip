@@ -453,6 +453,14 @@ int launch_mlp_step(const tfq_weight* gate, const tfq_weight* up, const tfq_weig
         if (int rc = launch_gemm(gate, x, x_dtype, B, g, TFQ_F32, s, scratch, scratch_bytes)) return rc;
         if (int rc = launch_gemm(up, x, x_dtype, B, u, TFQ_F32, s, scratch, scratch_bytes)) return rc;
     }
+    if (B <= 16 && gemv_prologue_supported(down)) {
+        // silu(gate) * up happens while the down kernel stages its activations
+        tfq_prologue_t pro{};
+        pro.op = TFQ_PRO_SWIGLU;
+        pro.up = u;
+        pro.mid_dtype = mid_dtype;
+        return launch_gemv_multi_fused(&down, 1, g, TFQ_F32, B, &y, y_dtype, &pro, s);
+    }
     const int64_t nh = (int64_t)B * F;
     if (mid_dtype == TFQ_BF16)
         hipLaunchKernelGGL(silu_mul_kernel<true>, dim3((unsigned)((nh + 255) / 256)), dim3(256), 0, s, g, u, h, nh);
