@@ -342,6 +342,37 @@ int tfq_chain_check(const tfq_chain_t* chain);
 size_t tfq_chain_weight_bytes(const tfq_chain_t* chain); /* packed bytes one run streams */
 void tfq_chain_free(tfq_chain_t* chain);
 
+/* ---- dense fp32 operators -------------------------------------------------------------
+ * The operator set of backend::ComputeBackend (include/quant/backend.h:77-108) on device-resident
+ * row-major fp32 arrays, with the arithmetic of the routines the reference's CPU backend forwards to
+ * (src/math/math.cpp:50-309): what a GPU_HIP subclass of that interface calls (tfq::HipBackend in
+ * include/tfq_shims.hpp is that subclass without the reference's Tensor type).
+ *   gemm        C[M][N] = alpha A[M][K] B[K][N] + beta C        (math.cpp:72-95; fp32 matrix cores)
+ *   gemv        y[M] = alpha A[M][N] x[N] + beta y                (:50-70)
+ *   softmax     over `dim` entries spaced `inner` apart, `outer` times (:232-274): the reference's axis
+ *               form, outer = product of the extents before the axis, inner = after it
+ *   layer_norm  (x - mean) / sqrt(var + eps) * gamma + beta over the last dimension n (:173-205)
+ *   rms_norm    x / sqrt(mean(x^2) + eps) * gamma (:207-230)
+ *   unary       relu, gelu = 0.5 x (1 + erf(x / sqrt 2)), silu = x / (1 + exp(-x)), scale = s x,
+ *               copy, fill = s (x may be NULL)     (:97-126, :303-309)
+ *   binary      add, mul (:276-301)
+ * In-place use (y == x) is allowed for unary, binary and the norms. */
+enum { TFQ_DENSE_RELU = 0, TFQ_DENSE_GELU = 1, TFQ_DENSE_SILU = 2, TFQ_DENSE_SCALE = 3, TFQ_DENSE_COPY = 4,
+       TFQ_DENSE_FILL = 5, TFQ_DENSE_ADD = 6, TFQ_DENSE_MUL = 7 };
+int tfq_dense_gemm(float alpha, const float* A, const float* B, float beta, float* C, int64_t M, int64_t N,
+                   int64_t K, tfq_stream_t stream);
+int tfq_dense_gemv(float alpha, const float* A, const float* x, float beta, float* y, int64_t M, int64_t N,
+                   tfq_stream_t stream);
+int tfq_dense_softmax(const float* x, float* y, int64_t outer, int64_t dim, int64_t inner, tfq_stream_t stream);
+int tfq_dense_layer_norm(const float* x, const float* gamma, const float* beta, float eps, float* y,
+                         int64_t rows, int64_t n, tfq_stream_t stream);
+int tfq_dense_rms_norm(const float* x, const float* gamma, float eps, float* y, int64_t rows, int64_t n,
+                       tfq_stream_t stream);
+int tfq_dense_unary(int op, const float* x, float s, float* y, int64_t n, tfq_stream_t stream);
+int tfq_dense_binary(int op, const float* a, const float* b, float* y, int64_t n, tfq_stream_t stream);
+/* free and total device memory in bytes (ComputeBackend::memory_free / memory_total) */
+int tfq_device_memory(int64_t* free_bytes, int64_t* total_bytes);
+
 /* ---- MoE expert path ------------------------------------------------------------
  * tfq_moe_route: router softmax + top-k on the device, softmax_with_topk
  * (src/model/moe_core.cpp:98-149): probs [T][E], idx [T][k] (descending

@@ -124,6 +124,31 @@ struct TensorCodec {
     static void dequantize(uint8_t wire_format, const TensorPayload& p, float* output, int64_t n);
 };
 
+// backend::ComputeBackend for GPU_HIP (include/quant/backend.h:77-108) without the reference's Tensor
+// type: the same operators on host row-major fp32 buffers and explicit extents.  Every call moves its
+// operands to the device, runs the HIP kernel and moves the result back, which is how the reference's
+// GPU backends behave (src/backend/gpu_compute_hip.cpp:528-553).  An operator that cannot run leaves its
+// output untouched and returns false; is_available() is false without a gfx950 device.
+class HipBackend {
+public:
+    static const char* name() { return "GPU_HIP"; }
+    static bool is_available();
+    static int64_t memory_free();
+    static int64_t memory_total();
+    static void synchronize();
+    static bool gemm(float alpha, const float* A, const float* B, float beta, float* C, int64_t M, int64_t N, int64_t K);
+    static bool gemv(float alpha, const float* A, const float* x, float beta, float* y, int64_t M, int64_t N);
+    static bool softmax(const float* x, float* y, int64_t outer, int64_t dim, int64_t inner);
+    static bool layer_norm(const float* x, const float* gamma, const float* beta, float eps, float* y, int64_t rows, int64_t n);
+    static bool rms_norm(const float* x, const float* gamma, float eps, float* y, int64_t rows, int64_t n);
+    static bool relu(const float* x, float* y, int64_t n);
+    static bool gelu(const float* x, float* y, int64_t n);
+    static bool silu(const float* x, float* y, int64_t n);
+    static bool add(const float* a, const float* b, float* c, int64_t n);
+    static bool mul(const float* a, const float* b, float* c, int64_t n);
+    static bool scale(float s, const float* x, float* y, int64_t n);
+};
+
 // The generator of seeded synthetic inputs, quant::RNG (include/quant/random.h:27-46,
 // src/core/random.cpp:45-81): splitmix64 of the seed fills the two words of a xoroshiro128+
 // state; uniform() = (next >> 11) * 2^-53 as a float; normal() = Box-Muller on two uniform

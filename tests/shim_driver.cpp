@@ -83,4 +83,31 @@ long drv_tensor_round_trip(uint8_t fmt, const float* data, int64_t n, uint8_t* p
     return (long)p.indices.size();
 }
 
+// ---- tfq::HipBackend (ComputeBackend for GPU_HIP on host buffers)
+int drv_backend_available() { return tfq::HipBackend::is_available() ? 1 : 0; }
+long long drv_backend_memory_total() { return tfq::HipBackend::memory_total(); }
+int drv_backend_gemm(float alpha, const float* A, const float* B, float beta, float* C, long long M, long long N, long long K) {
+    return tfq::HipBackend::gemm(alpha, A, B, beta, C, M, N, K) ? 1 : 0;
+}
+int drv_backend_gemv(float alpha, const float* A, const float* x, float beta, float* y, long long M, long long N) {
+    return tfq::HipBackend::gemv(alpha, A, x, beta, y, M, N) ? 1 : 0;
+}
+int drv_backend_softmax(const float* x, float* y, long long outer, long long dim, long long inner) {
+    return tfq::HipBackend::softmax(x, y, outer, dim, inner) ? 1 : 0;
+}
+int drv_backend_norm(int layer, const float* x, const float* gamma, const float* beta, float eps, float* y, long long rows, long long n) {
+    return (layer ? tfq::HipBackend::layer_norm(x, gamma, beta, eps, y, rows, n) : tfq::HipBackend::rms_norm(x, gamma, eps, y, rows, n)) ? 1 : 0;
+}
+int drv_backend_unary(int op, float s, const float* x, float* y, long long n) {
+    switch (op) {
+        case 0: return tfq::HipBackend::relu(x, y, n);
+        case 1: return tfq::HipBackend::gelu(x, y, n);
+        case 2: return tfq::HipBackend::silu(x, y, n);
+        default: return tfq::HipBackend::scale(s, x, y, n);
+    }
+}
+int drv_backend_binary(int op, const float* a, const float* b, float* c, long long n) {
+    return (op == 0 ? tfq::HipBackend::add(a, b, c, n) : tfq::HipBackend::mul(a, b, c, n)) ? 1 : 0;
+}
+
 }  // extern "C"

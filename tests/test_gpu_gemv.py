@@ -367,6 +367,35 @@ def test_gemv_k_split_in_graph_replays(O, tfq, gpu):
     W.close()
 
 
+def test_gemv_k_split_soak(O, tfq, gpu):
+    """A bounded soak of the K-split rendezvous: 3000 replays of a graph holding three K-split launches, each
+    compared bit for bit with the eager result on the device; the loop stops at the first block of replays
+    that holds a mismatch.  (The rendezvous passes partial sums between workgroups on different XCDs through
+    device-scope stores, a wait for their acknowledgement and a device-scope counter; a lost or late partial
+    sum would change bits.)"""
+    import torch
+    N, K, B = 4096, 14336, 16
+    g = torch.Generator(device="cuda").manual_seed(12)
+    W = tfq.Weight("B32S4", N, K, tfq.encode("B32S4", torch.randn(N * K, device=gpu, generator=g) * 0.02))
+    xs = [torch.randn(B, K, device=gpu, generator=g).bfloat16() for _ in range(3)]
+    eager = [W.gemv(x).clone() for x in xs]
+    outs = [torch.empty(B, N, device=gpu) for _ in xs]
+    bad = torch.zeros((), device=gpu, dtype=torch.int64)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for x, y in zip(xs, outs):
+            W.gemv(x, out=y)
+    for block in range(30):
+        for _ in range(100):
+            graph.replay()
+            for want, got in zip(eager, outs):
+                bad += (want != got).sum()
+        torch.cuda.synchronize()
+        assert int(bad.item()) == 0, f"mismatch within replays {block * 100}..{block * 100 + 99}"
+    W.close()
+
+
 @pytest.mark.parametrize("K,B,xdt", [(28672, 4, "bf16"), (28672, 2, "f32"), (20480, 4, "bf16"), (32768, 3, "f32")])
 def test_long_k_takes_fewer_rows_per_pass(O, tfq, gpu, K, B, xdt):
     """K above 16384 leaves LDS room for fewer staged rows per pass; the product must still run (and match)."""

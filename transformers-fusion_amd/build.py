@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtfq.so")
 
-SOURCES = ["tfq_api.hip", "tfq_codec.hip", "tfq_codec_short.hip", "tfq_gemv.hip", "tfq_chain.hip", "tfq_gemv_generic.hip", "tfq_moe.hip", "tfq_gemm.hip",
+SOURCES = ["tfq_api.hip", "tfq_codec.hip", "tfq_codec_short.hip", "tfq_gemv.hip", "tfq_chain.hip", "tfq_dense.hip", "tfq_gemv_generic.hip", "tfq_moe.hip", "tfq_gemm.hip",
            "tfq_lut.hip", "tfq_container.hip", "tfq_engines.hip"]
 
 # -ffp-contract=off: the decode arithmetic is ordered to match the reference

@@ -7,6 +7,9 @@
 #include "../../include/tfq_shims.hpp"
 
 #include <cmath>
+#include <initializer_list>
+#include <utility>
+#include <vector>
 #include <cstring>
 
 namespace {
@@ -234,6 +237,65 @@ void TensorCodec::dequantize(uint8_t wire_format, const TensorPayload& p, float*
     std::memset(output, 0, (size_t)n * sizeof(float));
     if (!p.success || n > p.num_elements || (n % 256 && n != p.num_elements)) return;
     tfq_decode_blocks_host(wire_format, p.indices.data(), p.indices.size(), n, output);
+}
+
+// ---- HipBackend: host buffers in, device operator, host buffers out
+bool HipBackend::is_available() { int64_t f = 0; return tfq_device_memory(&f, nullptr) == TFQ_OK; }
+int64_t HipBackend::memory_free() { int64_t f = 0; return tfq_device_memory(&f, nullptr) == TFQ_OK ? f : 0; }
+int64_t HipBackend::memory_total() { int64_t t = 0; return tfq_device_memory(nullptr, &t) == TFQ_OK ? t : 0; }
+void HipBackend::synchronize() { (void)tfq_stream_sync(nullptr); }
+
+namespace {
+template <class Run>
+bool on_device(std::initializer_list<std::pair<const float*, int64_t>> inputs, float* out, int64_t out_n, bool out_is_input, Run&& run) {
+    DeviceBuffers d;
+    std::vector<const float*> dev;
+    for (const auto& in : inputs) {
+        if (!in.first || in.second <= 0) return false;
+        const float* p = static_cast<const float*>(d.upload(in.first, (size_t)in.second * 4));
+        if (!p) return false;
+        dev.push_back(p);
+    }
+    if (!out || out_n <= 0) return false;
+    float* dy = static_cast<float*>(out_is_input ? d.upload(out, (size_t)out_n * 4) : d.alloc((size_t)out_n * 4));
+    if (!dy) return false;
+    if (run(dev, dy) != TFQ_OK || tfq_stream_sync(nullptr) != TFQ_OK) return false;
+    return tfq_copy_to_host(out, dy, (size_t)out_n * 4) == TFQ_OK;
+}
+}  // namespace
+
+bool HipBackend::gemm(float alpha, const float* A, const float* B, float beta, float* C, int64_t M, int64_t N, int64_t K) {
+    return on_device({{A, M * K}, {B, K * N}}, C, M * N, beta != 0.0f,
+                     [&](const std::vector<const float*>& in, float* dc) { return tfq_dense_gemm(alpha, in[0], in[1], beta, dc, M, N, K, nullptr); });
+}
+bool HipBackend::gemv(float alpha, const float* A, const float* x, float beta, float* y, int64_t M, int64_t N) {
+    return on_device({{A, M * N}, {x, N}}, y, M, beta != 0.0f,
+                     [&](const std::vector<const float*>& in, float* dy) { return tfq_dense_gemv(alpha, in[0], in[1], beta, dy, M, N, nullptr); });
+}
+bool HipBackend::softmax(const float* x, float* y, int64_t outer, int64_t dim, int64_t inner) {
+    return on_device({{x, outer * dim * inner}}, y, outer * dim * inner, false,
+                     [&](const std::vector<const float*>& in, float* dy) { return tfq_dense_softmax(in[0], dy, outer, dim, inner, nullptr); });
+}
+bool HipBackend::layer_norm(const float* x, const float* gamma, const float* beta, float eps, float* y, int64_t rows, int64_t n) {
+    return on_device({{x, rows * n}, {gamma, n}, {beta, n}}, y, rows * n, false,
+                     [&](const std::vector<const float*>& in, float* dy) { return tfq_dense_layer_norm(in[0], in[1], in[2], eps, dy, rows, n, nullptr); });
+}
+bool HipBackend::rms_norm(const float* x, const float* gamma, float eps, float* y, int64_t rows, int64_t n) {
+    return on_device({{x, rows * n}, {gamma, n}}, y, rows * n, false,
+                     [&](const std::vector<const float*>& in, float* dy) { return tfq_dense_rms_norm(in[0], in[1], eps, dy, rows, n, nullptr); });
+}
+static bool unary_host(int op, const float* x, float s, float* y, int64_t n) {
+    return on_device({{x, n}}, y, n, false, [&](const std::vector<const float*>& in, float* dy) { return tfq_dense_unary(op, in[0], s, dy, n, nullptr); });
+}
+bool HipBackend::relu(const float* x, float* y, int64_t n) { return unary_host(TFQ_DENSE_RELU, x, 0.0f, y, n); }
+bool HipBackend::gelu(const float* x, float* y, int64_t n) { return unary_host(TFQ_DENSE_GELU, x, 0.0f, y, n); }
+bool HipBackend::silu(const float* x, float* y, int64_t n) { return unary_host(TFQ_DENSE_SILU, x, 0.0f, y, n); }
+bool HipBackend::scale(float s, const float* x, float* y, int64_t n) { return unary_host(TFQ_DENSE_SCALE, x, s, y, n); }
+bool HipBackend::add(const float* a, const float* b, float* c, int64_t n) {
+    return on_device({{a, n}, {b, n}}, c, n, false, [&](const std::vector<const float*>& in, float* dy) { return tfq_dense_binary(TFQ_DENSE_ADD, in[0], in[1], dy, n, nullptr); });
+}
+bool HipBackend::mul(const float* a, const float* b, float* c, int64_t n) {
+    return on_device({{a, n}, {b, n}}, c, n, false, [&](const std::vector<const float*>& in, float* dy) { return tfq_dense_binary(TFQ_DENSE_MUL, in[0], in[1], dy, n, nullptr); });
 }
 
 namespace {
