@@ -1181,8 +1181,8 @@ template <int FMT>
 __global__ __launch_bounds__(256) void tile16_kernel(const uint8_t* __restrict__ wire, uint4* __restrict__ tiled,
                                                      int64_t N, int nblocks, int64_t npieces) {
     constexpr Spec sp = spec_of(FMT);
-    constexpr int HB = tiled_header_bytes(FMT), HP = HB / 16, NP = tiled_planes(FMT);
-    constexpr int CP = 128 * NP, PIECES = CP + 16 * HP;  // code pieces, all pieces of a unit
+    constexpr int HB = tiled_header_bytes(FMT), HP = HB / 16, NP = tiled_planes(FMT), CW = tiled_code_width(FMT);
+    constexpr int CP = tiled_code_bytes(FMT) / 16, PIECES = CP + 16 * HP;  // code pieces, all pieces of a unit
     constexpr uint32_t BB = sp.block_bytes, code_bytes = 256u * sp.bits / 8;
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= npieces) return;
@@ -1191,7 +1191,20 @@ __global__ __launch_bounds__(256) void tile16_kernel(const uint8_t* __restrict__
     const int64_t tile = unit / nblocks;
     const int blk = (int)(unit - tile * nblocks);
     uint32_t o[4] = {0, 0, 0, 0};
-    if (p < CP) {
+    if (CW < 4 && p < CP) {
+        // true-width code area: piece p = the 2-bit fields of lane p
+        const int l = p, n = l & 15, c = l >> 4;
+        const int64_t row = tile * 16 + n;
+        if (row < N) {
+            const uint8_t* src = wire + (row * nblocks + blk) * (int64_t)BB;
+            for (int h = 0; h < 2; ++h)
+                for (int e = 0; e < 32; ++e) {  // element e of the lane's 32-slot of k-step h
+                    const uint32_t code = stream_bits(src, code_bytes, (uint32_t)(128 * h + 32 * c + e) * sp.bits, sp.bits);
+                    const int j = e >> 3, t = e & 3, upper = (e >> 2) & 1;  // MFMA j, pair t, low / high half-word
+                    o[2 * h + (j >> 1)] |= code << (16 * upper + 2 * (t + 4 * (j & 1)));
+                }
+        }
+    } else if (p < CP) {
         const int plane = p >> 7, l = p & 63, n = l & 15, g32 = (l >> 4) + 4 * ((p >> 6) & 1);
         const int64_t row = tile * 16 + n;
         if (row < N) {
@@ -1226,6 +1239,21 @@ __global__ __launch_bounds__(256) void tile16_kernel(const uint8_t* __restrict__
             if constexpr (sp.codec == Codec::Lattice) {  // the block's one binary16 scale, for each of the 8 groups
                 const uint32_t s2 = (uint32_t)src[0] | ((uint32_t)src[1] << 8);
                 o[0] = o[1] = o[2] = o[3] = s2 | (s2 << 16);
+            } else if constexpr (tiled_header_in_bytes(FMT)) {
+                // part 0: the 16 scale codes, one per byte; part 1: the 16 offset codes (still biased); part 2: d, dm
+                constexpr uint32_t ng = 256 / sp.gsz, sc_bits = ((ng * sp.scb + 7) / 8) * 8, mn_bits = ((ng * sp.mb + 7) / 8) * 8;
+                const uint8_t* hsrc = src + code_bytes;
+                const uint32_t hbytes = BB - code_bytes;
+                if (part < 2) {
+#pragma unroll
+                    for (int g = 0; g < 16; ++g) {
+                        const uint32_t code = part == 0 ? stream_bits(hsrc, hbytes, (uint32_t)g * sp.scb, sp.scb)
+                                                        : stream_bits(hsrc, hbytes, sc_bits + (uint32_t)g * sp.mb, sp.mb);
+                        o[g >> 2] |= code << (8 * (g & 3));
+                    }
+                } else {
+                    o[0] = stream_bits(hsrc, hbytes, sc_bits + mn_bits, 16) | (stream_bits(hsrc, hbytes, sc_bits + mn_bits + 16, 16) << 16);
+                }
             } else {
 #pragma unroll
                 for (int j = 0; j < 16; ++j) {
@@ -1253,8 +1281,15 @@ __global__ __launch_bounds__(256) void decode_tiled_kernel(const uint8_t* __rest
     const int n = (int)(row & 15);
     const uint32_t g32 = i >> 5, j = i & 31;
     const uint8_t* codes = unit + (g32 >> 2) * 1024 + (n + 16 * (g32 & 3)) * 16;
-    const uint32_t idx = (codes[j >> 1] >> ((j & 1u) * 4)) & 15u;
-    const uint8_t* h = unit + 2048 * tiled_planes(FMT) + n * HB;
+    uint32_t idx;
+    if constexpr (tiled_code_width(FMT) < 4) {
+        const uint32_t ks = g32 >> 2, lane = (uint32_t)n + 16 * (g32 & 3), mj = j >> 3, t = j & 3, upper = (j >> 2) & 1;
+        const uint32_t* lo = reinterpret_cast<const uint32_t*>(unit + 16 * lane);
+        idx = (lo[2 * ks + (mj >> 1)] >> (16 * upper + 2 * (t + 4 * (mj & 1)))) & 3u;
+    } else {
+        idx = (codes[j >> 1] >> ((j & 1u) * 4)) & 15u;
+    }
+    const uint8_t* h = unit + tiled_code_bytes(FMT) + n * HB;
     float v;
     if constexpr (sp.codec == Codec::Grp8 || sp.codec == Codec::Lattice) {
         const float d = half_bits_to_float((uint32_t)h[2 * g32] | ((uint32_t)h[2 * g32 + 1] << 8));
@@ -1271,10 +1306,18 @@ __global__ __launch_bounds__(256) void decode_tiled_kernel(const uint8_t* __rest
         constexpr uint32_t mn_bits = ((ng * sp.mb + 7) / 8) * 8;
         constexpr int bias = (1 << sp.mb) / 2;
         const uint32_t g = i / sp.gsz;
-        const float sc = (float)stream_bits(h, HB, g * sp.scb, sp.scb);
-        const float mc = (float)stream_bits(h, HB, sc_bits + g * sp.mb, sp.mb) - (float)bias;
-        const float d = half_bits_to_float(stream_bits(h, HB, sc_bits + mn_bits, 16));
-        const float dm = half_bits_to_float(stream_bits(h, HB, sc_bits + mn_bits + 16, 16));
+        float sc, mc, d, dm;
+        if constexpr (tiled_header_in_bytes(FMT)) {
+            sc = (float)h[g];
+            mc = (float)h[16 + g] - (float)bias;
+            d = half_bits_to_float((uint32_t)h[32] | ((uint32_t)h[33] << 8));
+            dm = half_bits_to_float((uint32_t)h[34] | ((uint32_t)h[35] << 8));
+        } else {
+            sc = (float)stream_bits(h, HB, g * sp.scb, sp.scb);
+            mc = (float)stream_bits(h, HB, sc_bits + g * sp.mb, sp.mb) - (float)bias;
+            d = half_bits_to_float(stream_bits(h, HB, sc_bits + mn_bits, 16));
+            dm = half_bits_to_float(stream_bits(h, HB, sc_bits + mn_bits + 16, 16));
+        }
         const float es = d * sc;
         const float neg = -(dm * mc);
         v = __builtin_fmaf(es, unit_level(sp.bits, idx), neg);

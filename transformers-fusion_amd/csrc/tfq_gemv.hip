@@ -128,7 +128,9 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     using F = Fmt<FMT>;
     static_assert(XOP == XOP_NONE || (XF32 && SETS == 1 && !GROUPED), "prologues take fp32 input in the plain launch");
     constexpr int UB = tiled_unit_bytes(FMT);  // bytes of a unit
-    constexpr int NC = 2 * F::NP;              // 1 KB code pieces of a unit: [plane][k-step]
+    // code registers (uint4) of a unit per lane: nibble formats [plane][k-step] from 1 KB pieces; the 2-bit
+    // formats one register of 2-bit fields for both k-steps
+    constexpr int NC = F::CW == 4 ? 2 * F::NP : 1;
     constexpr int NG = F::NG, PER = NG / 2;  // scale groups per block / per k-step
     const int K = args.K, T = args.tiles_per_wg;
     const int cols_base = args.cols_base, cols_rem = args.cols_rem;
@@ -232,10 +234,14 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     const uint8_t* col_ptr = Wm + ((size_t)tile0 * nblocks + (size_t)wave) * UB;
     const uint8_t* f_ptr = col_ptr;
     int f_t = 0, f_left = nitems;
-    const uint32_t off_c = 16u * lane, off_h = 1024u * NC + (uint32_t)F::HB * n;
+    const uint32_t off_c = 16u * lane, off_h = (uint32_t)F::CODE_BYTES + (uint32_t)F::HB * n;
     auto fetch = [&](uint4 (&cc)[NC], uint4 (&hd)[F::HV]) __attribute__((always_inline)) {
+        if constexpr (F::CW == 4) {
 #pragma unroll
-        for (int i = 0; i < NC; ++i) cc[i] = stream_load16(f_ptr + off_c + 1024 * i);
+            for (int i = 0; i < NC; ++i) cc[i] = stream_load16(f_ptr + off_c + 1024 * i);
+        } else {
+            cc[0] = stream_load16(f_ptr + off_c);
+        }
 #pragma unroll
         for (int i = 0; i < F::HV; ++i) hd[i] = stream_load16(f_ptr + off_h + 16 * i);
         if (--f_left > 0) {
@@ -385,12 +391,21 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
             }
 #pragma unroll
             for (int pl = 0; pl < F::NP; ++pl) {  // nibble planes: the second one accumulates into DB
-                const uint4 cw = cc[u][2 * pl + h];
+                const uint4 cw = cc[u][F::CW == 4 ? 2 * pl + h : 0];
                 const uint32_t qq[4] = {cw.x, cw.y, cw.z, cw.w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const uint32_t v = qq[j];
-                    const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
+                    uint4 wv;
+                    if constexpr (F::CW == 4) {
+                        const uint32_t v = qq[j];
+                        wv = uint4{(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
+                    } else {
+                        // 2-bit fields: dword 2h + j / 2 of the lane holds the pairs of two MFMAs
+                        constexpr uint32_t M2 = 0x00030003u;
+                        const uint32_t v = qq[2 * h + (j >> 1)];
+                        const int s = 8 * (j & 1);
+                        wv = uint4{((v >> s) & M2) | C, ((v >> (s + 2)) & M2) | C, ((v >> (s + 4)) & M2) | C, ((v >> (s + 6)) & M2) | C};
+                    }
                     const bool second = pl == 1 || (F::GS == 16 && j >= 2);
 #pragma unroll
                     for (int st = 0; st < SETS; ++st) {

@@ -60,6 +60,8 @@ struct Fmt {
     static constexpr int GS = spec_of(FMT).gsz == 16 ? 16 : 32;
     static constexpr int NG = 256 / GS;  // groups per block: 8 or 16
     static constexpr int NP = tiled_planes(FMT);  // nibble planes of the codes (2: low and high nibble of code + 128)
+    static constexpr int CW = tiled_code_width(FMT);  // 4: nibbles; 2: true-width 2-bit fields (tfq_internal.hpp)
+    static constexpr int CODE_BYTES = tiled_code_bytes(FMT);
     // 4-bit symmetric: 128 + 8; 8-bit symmetric: code = 16 hi + lo - 128 with both nibbles carrying
     // +128, so 16 * 128 + 128 + 128; affine: 128
     // companded 8-bit (Q_G_8, Q_8): code j = 16 hi + lo stands for the level (j - 127.5) * kComp8Gain, so
@@ -74,6 +76,17 @@ struct Fmt {
 // to 7.5e-5 relative; the matmul uses that line (codes as integers on the matrix cores, the slope
 // in the scale), which costs under a tenth of the 1e-3 output tolerance.  Decode keeps the table.
 constexpr float kComp8Gain = 1.0000742443371564f / 127.5f;
+
+// byte B of a dword as a float (v_cvt_f32_ubyteB)
+template <int B>
+__device__ __forceinline__ float byte_to_float(uint32_t v) {
+    float f;
+    if constexpr (B == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(v));
+    else if constexpr (B == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(v));
+    else if constexpr (B == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(v));
+    else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(v));
+    return f;
+}
 
 // `count` bits at bit `pos` (both compile-time after unrolling) of the little-endian bit string w[0], w[1], ...
 __device__ __forceinline__ uint32_t field(const uint32_t* w, int pos, int count) {
@@ -109,6 +122,29 @@ __device__ __forceinline__ float apply_groups(const uint4* hv, int khalf, f32x4_
         res = __builtin_fmaf((float)s23.x, DA[2], res);
         res = __builtin_fmaf((float)s23.y, DA[3], res);
         if constexpr (Fmt<FMT>::COMP8) res *= kComp8Gain;
+    } else if constexpr (tiled_header_in_bytes(FMT)) {
+        // header: 16 scale codes, one per byte | 16 offset codes (biased), one per byte | binary16 d, dm.
+        // sum_g (d sc_g / top) D_g - dm (mc_g - bias) X_g with d / top and dm taken out of the sums: a code
+        // becomes a float with one v_cvt_f32_ubyteN, and a group costs two multiply-adds.
+        constexpr int mbias = (1 << sp.mb) / 2;
+        constexpr float inv_top = sp.bits == 4 ? 1.0f / 15.0f : sp.bits == 3 ? 1.0f / 7.0f : 1.0f / 3.0f;
+        const uint32_t sc_lo = khalf ? hv[0].z : hv[0].x, sc_hi = khalf ? hv[0].w : hv[0].y;
+        const uint32_t mc_lo = khalf ? hv[1].z : hv[1].x, mc_hi = khalf ? hv[1].w : hv[1].y;
+        const float dtop = half_fast(hv[2].x & 0xFFFFu) * inv_top;
+        const float dm = half_fast(hv[2].x >> 16);
+        const float sc[8] = {byte_to_float<0>(sc_lo), byte_to_float<1>(sc_lo), byte_to_float<2>(sc_lo), byte_to_float<3>(sc_lo),
+                             byte_to_float<0>(sc_hi), byte_to_float<1>(sc_hi), byte_to_float<2>(sc_hi), byte_to_float<3>(sc_hi)};
+        const float mc[8] = {byte_to_float<0>(mc_lo), byte_to_float<1>(mc_lo), byte_to_float<2>(mc_lo), byte_to_float<3>(mc_lo),
+                             byte_to_float<0>(mc_hi), byte_to_float<1>(mc_hi), byte_to_float<2>(mc_hi), byte_to_float<3>(mc_hi)};
+        float sa = 0.0f, sm = 0.0f, sx = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const float D = (t & 1) ? DB[t >> 1] : DA[t >> 1];
+            sa = __builtin_fmaf(sc[t], D, sa);
+            sm = __builtin_fmaf(mc[t], X[t], sm);
+            sx += X[t];
+        }
+        res = __builtin_fmaf(dtop, sa, dm * __builtin_fmaf((float)mbias, sx, -sm));
     } else {
         // header: NG scale codes of scb bits | NG offset codes of mb bits (biased) | binary16 d | binary16 dm
         constexpr int NG = Fmt<FMT>::NG, PER = NG / 2;  // groups per k-step

@@ -284,10 +284,13 @@ namespace tfq {
 __host__ __device__ constexpr int tiled_header_bytes(int fmt) {
     switch (canonical(fmt)) {
         case TFQ_Q_G_4: case TFQ_B32S4: case TFQ_B32S8: case TFQ_Q_G_3: case TFQ_Q_G_8: case TFQ_Q_8: return 16;
-        case TFQ_Q_G_2: case TFQ_SB256A3: case TFQ_SB256A2: return 32;
+        // sixteen groups of 16: the scale and offset codes are kept one per byte (16 + 16 bytes), then d and dm,
+        // so that the kernel turns a code into a float with one byte-convert instead of a bit-field extract
+        case TFQ_Q_G_2: case TFQ_SB256A3: case TFQ_SB256A2: return 48;
         default: return 0;
     }
 }
+__host__ __device__ constexpr bool tiled_header_in_bytes(int fmt) { return tiled_header_bytes(fmt) == 48; }
 // nibble planes of the code area: the 8-bit symmetric format is stored as two, the low and the
 // high nibble of (code + 128), each laid out like a 4-bit format's codes
 // (the companded 8-bit formats store their code 0..255 the same way; plain Q_8 has its slot codes
@@ -295,7 +298,23 @@ __host__ __device__ constexpr int tiled_header_bytes(int fmt) {
 __host__ __device__ constexpr int tiled_planes(int fmt) {
     return canonical(fmt) == TFQ_B32S8 || canonical(fmt) == TFQ_Q_G_8 || canonical(fmt) == TFQ_Q_8 ? 2 : 1;
 }
-__host__ __device__ constexpr int tiled_unit_bytes(int fmt) { return 2048 * tiled_planes(fmt) + 16 * tiled_header_bytes(fmt); }
+// Width of a code in the Tiled16 code area.  4: nibbles (codes narrower than four bits are widened, wider ones
+// are split into nibble planes).  2: the 2-bit formats keep their true width: one 1 KB piece of 2-bit fields for
+// both k-steps (lane l owns 16 bytes: dword 2h + m holds the codes 16m..16m+15 of its 32-slot of k-step h; inside a
+// dword the low half-word carries, at bit 2 (t + 4 j'), code 8 j' + t and the high half-word code 8 j' + t + 4, so
+// that (v >> 2 (t + 4 j')) & 0x00030003 is the pair an MFMA operand dword needs).  The 3-bit superblock format
+// stays with nibbles: as a 2-bit plane plus a plane of high bits it read 18 % fewer bytes and ran 8 % slower
+// (14336 x 4096, one row: 12.7 us against 11.8 us), because its kernel is bound by instruction issue, not bytes.
+__host__ __device__ constexpr int tiled_code_width(int fmt) {
+    switch (canonical(fmt)) {
+        case TFQ_SB256A2: case TFQ_Q_G_2: return 2;
+        default: return 4;
+    }
+}
+__host__ __device__ constexpr int tiled_code_bytes(int fmt) {
+    return tiled_code_width(fmt) == 2 ? 1024 : 2048 * tiled_planes(fmt);
+}
+__host__ __device__ constexpr int tiled_unit_bytes(int fmt) { return tiled_code_bytes(fmt) + 16 * tiled_header_bytes(fmt); }
 }  // namespace tfq
 
 struct tfq_weight {
