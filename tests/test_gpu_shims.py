@@ -167,8 +167,9 @@ def test_production_gemvs(O, drv):
 
 
 @pytest.mark.parametrize("fmt", ["Q_G_4", "B32S4", "Q_G_8"])
-@pytest.mark.parametrize("B", [1, 5, 40])
+@pytest.mark.parametrize("B", [1, 5, 40, 512])
 def test_block_row_matmul_like_the_engine_gemm(O, drv, fmt, B):
+    """B = 40 and 512 (the engine's MAX_BATCH): fp32 rows go through the 16-row decode kernel as a bf16 high and low part."""
     N, K = 96, 1024
     w = O.rng_normal(42, N * K, 0.02)
     X = O.rng_normal(43, B * K, 1.0).reshape(B, K)
