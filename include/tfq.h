@@ -391,6 +391,12 @@ int tfq_device_memory(int64_t* free_bytes, int64_t* total_bytes);
  * least tfq_moe_workspace_bytes(T, k, D, F) bytes, 256-byte aligned. */
 int tfq_moe_route(const float* logits, int T, int E, int k, float* probs, int32_t* idx, float* weights,
                   tfq_stream_t stream);
+/* The router in front of it: logits[t][e] = x[t] . router_w[e] (+ router_bias[e], may be NULL), the Linear the
+ * reference's model applies to the normalised hidden state (block.moe->router_weight.forward,
+ * src/model/moe_model.cpp:582), then tfq_moe_route on those logits.  x is [T][D] (x_dtype), router_w fp32
+ * [E][D]; logits [T][E] is written too (the load-balance loss reads it, src/model/moe_core.cpp:155-190). */
+int tfq_moe_router(const void* x, int x_dtype, const float* router_w, const float* router_bias, int T, int D,
+                   int E, int k, float* logits, float* probs, int32_t* idx, float* weights, tfq_stream_t stream);
 size_t tfq_moe_workspace_bytes(int T, int k, int64_t D, int64_t F);
 int tfq_moe_ffn(const tfq_weight_t* const* gate, const tfq_weight_t* const* up,
                 const tfq_weight_t* const* down, int E, const int64_t* topk_idx, const float* topk_w,

@@ -26,6 +26,30 @@ def test_route_matches_reference_softmax_topk(O, tfq, gpu):
     assert tfq.moe_route(torch.from_numpy(logits).to(gpu), 99)[1].shape == (T, E)
 
 
+@pytest.mark.parametrize("xdt", ["f32", "bf16"])
+def test_router_linear_then_route(O, tfq, gpu, xdt):
+    """tfq_moe_router: logits = x . Wr^T + b (float64 numpy as the check, 1e-5 of the largest logit), then the
+    route of those very logits equals the oracle's softmax_topk of them."""
+    import torch
+    T, D, E, K = 16, 4096, 8, 2
+    x = O.rng_normal(43, T * D, 1.0).reshape(T, D)
+    if xdt == "bf16":
+        x = O.bf16_round(x)
+    Wr = O.rng_normal(46, E * D, 0.05).reshape(E, D)
+    b = O.rng_normal(47, E, 0.1)
+    xd = torch.from_numpy(x).to(gpu)
+    if xdt == "bf16":
+        xd = xd.bfloat16()
+    logits, probs, idx, w = tfq.moe_router(xd, torch.from_numpy(Wr).to(gpu), K, bias=torch.from_numpy(b).to(gpu))
+    ref = x.astype(np.float64) @ Wr.astype(np.float64).T + b
+    got = logits.cpu().numpy()
+    assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max()
+    p_ref, i_ref, w_ref = O.softmax_topk(got, K)
+    assert np.array_equal(idx.cpu().numpy().astype(np.int64), i_ref)
+    assert np.abs(probs.cpu().numpy() - p_ref).max() <= 2e-7
+    assert np.abs(w.cpu().numpy() - w_ref).max() <= 2e-7
+
+
 def _experts(O, tfq, fmt, E, D, F, seed):
     gate, up, down, hg, hu, hd = [], [], [], [], [], []
     for e in range(E):

@@ -516,6 +516,26 @@ def gemv_multi_fused(ws, x, outs, *, rmsnorm=None, swiglu_up=None, eps=1e-6, gam
     return outs
 
 
+def moe_router(x, router_w, k: int, bias=None):
+    """Router Linear + softmax + top-k on the device: returns (logits, probs, idx int32, weights)."""
+    import torch
+    T, D = x.shape
+    E = router_w.shape[0]
+    assert router_w.dtype == torch.float32 and router_w.is_contiguous() and x.is_contiguous()
+    logits = torch.empty(T, E, device=x.device)
+    probs = torch.empty(T, E, device=x.device)
+    kk = max(1, min(k, E))
+    idx = torch.empty(T, kk, device=x.device, dtype=torch.int32)
+    w = torch.empty(T, kk, device=x.device)
+    L = lib()
+    L.tfq_moe_router.restype = C.c_int
+    L.tfq_moe_router.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
+                                 C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    _check(L.tfq_moe_router(x.data_ptr(), _dtype_code(x), router_w.data_ptr(), bias.data_ptr() if bias is not None else None,
+                            T, D, E, k, logits.data_ptr(), probs.data_ptr(), idx.data_ptr(), w.data_ptr(), _stream()))
+    return logits, probs, idx, w
+
+
 def moe_route(logits, k: int):
     """Device softmax + top-k: returns (probs [T][E], idx [T][k] int32, weights [T][k])."""
     import torch

@@ -424,6 +424,18 @@ int tfq_gemm_static(const tfq_weight_t* w, const void* x, int x_dtype, int M, vo
 
 size_t tfq_gemm_static_scratch_bytes(void) { return gemm_static_scratch_bytes(); }
 
+int tfq_moe_router(const void* x, int x_dtype, const float* router_w, const float* router_bias, int T, int D, int E, int k,
+                   float* logits, float* probs, int32_t* idx, float* weights, tfq_stream_t stream) {
+    if (!x || !router_w || !logits || !probs || !idx || !weights) return fail(TFQ_ERR_ARG, "tfq_moe_router: null pointer");
+    if (T <= 0 || E <= 0 || D <= 0) return fail(TFQ_ERR_ARG, "tfq_moe_router: T, D and E must be positive");
+    if (x_dtype != TFQ_F32 && x_dtype != TFQ_BF16) return fail(TFQ_ERR_ARG, "tfq_moe_router: x_dtype must be TFQ_F32 or TFQ_BF16");
+    if (k < 1) k = 1;
+    if (k > E) k = E;
+    if (int r = ensure_device()) return r;
+    if (int r = launch_moe_router_logits(x, x_dtype, router_w, router_bias, logits, T, E, D, (hipStream_t)stream)) return r;
+    return launch_moe_route(logits, T, E, k, probs, idx, weights, (hipStream_t)stream);
+}
+
 int tfq_moe_route(const float* logits, int T, int E, int k, float* probs, int32_t* idx, float* weights, tfq_stream_t stream) {
     if (!logits || !probs || !idx || !weights) return fail(TFQ_ERR_ARG, "tfq_moe_route: null pointer");
     if (T <= 0 || E <= 0) return fail(TFQ_ERR_ARG, "tfq_moe_route: T and E must be positive");

@@ -403,6 +403,7 @@ size_t mlp_workspace_bytes(int B, int64_t F);
 int launch_mlp_step(const tfq_weight* gate, const tfq_weight* up, const tfq_weight* down, const void* x, int x_dtype, int B,
                     void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes, hipStream_t s);
 int launch_moe_route(const float* logits, int T, int E, int k, float* probs, int* idx, float* wts, hipStream_t s);
+int launch_moe_router_logits(const void* x, int x_dtype, const float* Wr, const float* bias, float* logits, int T, int E, int D, hipStream_t s);
 int launch_moe_ffn(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E,
                    const int64_t* topk_idx, const float* topk_w, int T, int Ktop, const void* x, int x_dtype,
                    void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes, hipStream_t s);

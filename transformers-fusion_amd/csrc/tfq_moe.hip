@@ -197,6 +197,38 @@ int acquire_list_slot(size_t bytes, ListSlot** out) {
 
 size_t moe_workspace_bytes(int T, int Ktop, int64_t D, int64_t F) { return carve(nullptr, T, Ktop, D, F).total; }
 
+namespace {
+// router logits[t][e] = x[t] . Wr[e] (+ bias[e]): one wavefront per (token, expert)
+template <bool XBF16>
+__global__ __launch_bounds__(256) void router_logits_kernel(const void* __restrict__ xv, const float* __restrict__ Wr, const float* __restrict__ bias,
+                                                            float* __restrict__ logits, int T, int E, int D) {
+    const int lane = threadIdx.x & 63;
+    const long long pair = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (pair >= (long long)T * E) return;
+    const int t = (int)(pair / E), e = (int)(pair - (long long)t * E);
+    const float* w = Wr + (size_t)e * D;
+    float s = 0.0f;
+    for (int d = lane; d < D; d += 64) {
+        float xd;
+        if constexpr (XBF16) xd = __uint_as_float((uint32_t)static_cast<const unsigned short*>(xv)[(size_t)t * D + d] << 16);
+        else xd = static_cast<const float*>(xv)[(size_t)t * D + d];
+        s = __builtin_fmaf(xd, w[d], s);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+    if (lane == 0) logits[pair] = bias ? s + bias[e] : s;
+}
+}  // namespace
+
+int launch_moe_router_logits(const void* x, int x_dtype, const float* Wr, const float* bias, float* logits, int T, int E, int D, hipStream_t s) {
+    const long long pairs = (long long)T * E;
+    if ((pairs + 3) / 4 > 0x7FFFFFFF) return fail(TFQ_ERR_SHAPE, "router: too many (token, expert) pairs");
+    const dim3 grid((unsigned)((pairs + 3) / 4));
+    if (x_dtype == TFQ_BF16) hipLaunchKernelGGL(router_logits_kernel<true>, grid, dim3(256), 0, s, x, Wr, bias, logits, T, E, D);
+    else hipLaunchKernelGGL(router_logits_kernel<false>, grid, dim3(256), 0, s, x, Wr, bias, logits, T, E, D);
+    return hip_fail(hipGetLastError(), "router launch");
+}
+
 int launch_moe_route(const float* logits, int T, int E, int k, float* probs, int* idx, float* wts, hipStream_t s) {
     hipLaunchKernelGGL(route_kernel, dim3((T + 63) / 64), dim3(64), 0, s, logits, T, E, k, probs, idx, wts);
     return hip_fail(hipGetLastError(), "route launch");
