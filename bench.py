@@ -52,6 +52,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM figure")
     ap.add_argument("--no-moe", action="store_true", help="skip the mixture-of-experts layer figure")
+    ap.add_argument("--no-chain", action="store_true",
+                    help="skip the figure of the same step as one persistent launch (tfq_chain_*: true data dependencies)")
     ap.add_argument("--no-sweep", action="store_true",
                     help="skip the batch / format sweep (batch 4, 8, 16; the 8-bit format; the low-bit superblock formats)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -168,6 +170,9 @@ def main():
                      "alg_bytes_per_launch": int(bytes_per_step / launches_per_step)},
     }
 
+    if not args.no_chain and B <= 2 and fmt in ("B32S4", "Q_G_4"):
+        res["chain"] = chain_step(tfq, torch, layers, bytes_per_step)
+        res["fused_launches"] = fused_launch_step(tfq, torch, layers, bytes_per_step)
     if not args.no_prefill:
         res["prefill"] = prefill_gemm(tfq, torch, layers[0])
     if not args.no_sweep:
@@ -182,6 +187,63 @@ def main():
         res["cpu_baseline"] = cpu_baseline(host_layer0, fmt, B, acts, bpw, threads=min(8, usable_cores()))
         res["cpu_baseline_all_cores"] = cpu_baseline(host_layer0, fmt, B, acts, bpw, threads=usable_cores(), budget_s=8.0)
     print(json.dumps(res), flush=True)
+
+
+def chain_step(tfq, torch, layers, bytes_per_step, reps=20):
+    """The same projections as ONE persistent launch with the data dependencies of a decoder layer kept inside
+    the kernel (rmsnorm -> q, k, v | o(q) -> h += . | rmsnorm -> gate, up -> silu * up -> down -> h += ., attention
+    itself is outside the path, so o takes q): a side figure, never `value`."""
+    dev = "cuda"
+    h = torch.from_numpy(tfq.rng_normal(43, 4096)).to(dev).reshape(1, 4096)
+    gamma = torch.zeros(4096, device=dev)
+    phases = []
+    for li, ws in enumerate(layers):
+        phases += [
+            {"w": [ws["q"], ws["k"], ws["v"]], "x": h if li == 0 else None, "x_op": tfq.X_RMSNORM, "gamma": gamma, "gamma_plus_one": True},
+            {"w": [ws["o"]], "y_op": tfq.Y_RESIDUAL, "residual": h},
+            {"w": [ws["gate"], ws["up"]], "x_op": tfq.X_RMSNORM, "gamma": gamma, "gamma_plus_one": True, "y_op": tfq.Y_SWIGLU},
+            {"w": [ws["down"]], "y_op": tfq.Y_RESIDUAL, "residual": h},
+        ]
+    if len(phases) > 128:
+        return {"skipped": "more than 128 phases"}
+    chain = tfq.Chain(phases, B=1)
+    chain.run()
+    torch.cuda.synchronize()
+    chain.check()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        chain.run()
+    e1.record()
+    torch.cuda.synchronize()
+    chain.check()
+    us = e0.elapsed_time(e1) * 1e3 / reps
+    chain.close()
+    return {"launches_per_step": 1, "phases": len(phases), "us_per_step": round(us, 1), "us_per_layer": round(us / len(layers), 2),
+            "gbs": round(bytes_per_step / us / 1e3, 1), "frac": round(bytes_per_step / us / 1e3 / HBM_PEAK_GBS, 4),
+            "note": "dependent phases inside one launch, RMSNorm / SwiGLU / residual fused"}
+
+
+def fused_launch_step(tfq, torch, layers, bytes_per_step):
+    """The same dependent decoder-layer sequence as four launches per layer with every elementwise step inside the
+    launches (tfq_gemv_multi_fused: RMSNorm in front of q/k/v and gate/up, SwiGLU in front of down, the residual
+    additions in the epilogues of o and down), fp32 hidden state.  A side figure, never `value`."""
+    dev = "cuda"
+    h = torch.from_numpy(tfq.rng_normal(43, 4096)).to(dev).reshape(1, 4096)
+    gamma = torch.zeros(4096, device=dev)
+    q, k, v = (torch.empty(1, n, device=dev) for n in (4096, 1024, 1024))
+    g, u = torch.empty(1, 14336, device=dev), torch.empty(1, 14336, device=dev)
+
+    def step():
+        for ws in layers:
+            tfq.gemv_multi_fused([ws["q"], ws["k"], ws["v"]], h, [q, k, v], rmsnorm=gamma)
+            tfq.gemv_multi_fused([ws["o"]], q, [h], accumulate=True)
+            tfq.gemv_multi_fused([ws["gate"], ws["up"]], h, [g, u], rmsnorm=gamma)
+            tfq.gemv_multi_fused([ws["down"]], g, [h], swiglu_up=u, accumulate=True)
+    us = time_graph(torch, step)
+    return {"launches_per_layer": 4, "us_per_layer": round(us / len(layers), 2), "gbs": round(bytes_per_step / us / 1e3, 1),
+            "frac": round(bytes_per_step / us / 1e3 / HBM_PEAK_GBS, 4),
+            "note": "fp32 hidden state; RMSNorm, SwiGLU and the residual additions fused into the 4 GEMV launches of a layer"}
 
 
 def time_graph(torch, fn, reps=10):

@@ -248,8 +248,9 @@ size_t tfq_gemm_static_scratch_bytes(void);
 int tfq_gemv_multi(const tfq_weight_t* const* ws, int count, const void* x, int x_dtype, int B,
                    void* const* ys, int y_dtype, tfq_stream_t stream);
 /* tfq_gemv_multi with an elementwise step of the reference engine applied to the activations while the
- * kernel stages them, so the step costs no launch and no round trip through memory.  x is fp32 [B][K],
- * B <= 16 (two rows ride in one pass over the weights, like every fp32 input).
+ * kernel stages them, so the step costs no launch and no round trip through memory.  With RMSNORM or SWIGLU
+ * x is fp32 [B][K], B <= 16 (two rows ride in one pass over the weights, like every fp32 input); with
+ * TFQ_PRO_NONE (only `accumulate` set) x may be bf16 too.
  *   TFQ_PRO_RMSNORM  x * rsqrt(mean(x^2) + eps) * gamma, or * (1 + gamma) with gamma_plus_one, the form of
  *                    Qwen35Engine::rmsnorm (src/adapters/tools/qwen35_engine.cpp:46-51), in front of the
  *                    q/k/v and the gate/up products
@@ -265,9 +266,12 @@ typedef struct tfq_prologue {
     int gamma_plus_one;
     const float* up;    /* SWIGLU: [B][K] */
     int mid_dtype;      /* SWIGLU: TFQ_F32 or TFQ_BF16 */
+    int accumulate;     /* ys[i] += product instead of ys[i] = product: the residual addition h += o(...), h += down(...)
+                           of a decoder layer (Qwen35Engine::append_token, qwen35_engine.cpp:807-835); any op, x of
+                           either type, up to four bf16 or two fp32 rows */
 } tfq_prologue_t;
-int tfq_gemv_multi_fused(const tfq_weight_t* const* ws, int count, const float* x, int B, void* const* ys,
-                         int y_dtype, const tfq_prologue_t* prologue, tfq_stream_t stream);
+int tfq_gemv_multi_fused(const tfq_weight_t* const* ws, int count, const void* x, int x_dtype, int B,
+                         void* const* ys, int y_dtype, const tfq_prologue_t* prologue, tfq_stream_t stream);
 /* host-pointer form of tfq_gemv/tfq_gemm with fp32 x and y: the exact call
  * shape of Qwen35Engine::gemm(t, X, Y, B). */
 int tfq_matmul_host(const tfq_weight_t* w, const float* X, float* Y, int B);

@@ -481,3 +481,25 @@ def test_prologue_rejects_untiled_formats(O, tfq, gpu):
     with pytest.raises(tfq.TfqError):
         tfq.gemv_multi_fused([W], torch.zeros(1, 256, device=gpu), [torch.zeros(1, 256, device=gpu)],
                              rmsnorm=torch.zeros(256, device=gpu))
+
+
+@pytest.mark.parametrize("xdt,B", [("bf16", 1), ("bf16", 4), ("f32", 2)])
+def test_accumulate_epilogue_adds_into_y(O, tfq, gpu, xdt, B):
+    """ys += W x (the residual addition of a decoder layer) in the launch's epilogue."""
+    import torch
+    fmt, N, K = "B32S4", 1040, 2048
+    pay = O.encode_tensor(fmt, O.rng_normal(80, N * K, 0.02))
+    W = tfq.Weight(fmt, N, K, pay)
+    x = O.rng_normal(81, B * K, 1.0).reshape(B, K)
+    y0 = O.rng_normal(82, B * N, 1.0).reshape(B, N)
+    if xdt == "bf16":
+        x = O.bf16_round(x)
+        xd = torch.from_numpy(x).to(gpu).bfloat16()
+    else:
+        xd = torch.from_numpy(x).to(gpu)
+    y = torch.from_numpy(y0.copy()).to(gpu)
+    tfq.gemv_multi_fused([W], xd, [y], accumulate=True)
+    ref = y0 + O.matmul(fmt, pay, N, K, x)
+    assert np.abs(y.cpu().numpy() - ref).max() / np.abs(ref).max() <= (1e-2 if xdt == "bf16" else 1e-3)
+    with pytest.raises(tfq.TfqError):  # more rows than one pass carries
+        tfq.gemv_multi_fused([W], torch.zeros(8, K, device=gpu).bfloat16(), [torch.zeros(8, N, device=gpu)], accumulate=True)

@@ -124,7 +124,7 @@ def _load():
         "tfq_copy_to_device": (i32, [vp, vp, sz]),
         "tfq_copy_to_host": (i32, [vp, vp, sz]),
         "tfq_stream_sync": (i32, [vp]),
-        "tfq_gemv_multi_fused": (i32, [vp, i32, vp, i32, vp, i32, vp, vp]),
+        "tfq_gemv_multi_fused": (i32, [vp, i32, vp, i32, i32, vp, i32, vp, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -489,22 +489,23 @@ def gemv_multi(weights, x, outs):
 class _Prologue(C.Structure):
     """tfq_prologue_t (include/tfq.h)."""
     _fields_ = [("op", C.c_int), ("gamma", C.c_void_p), ("eps", C.c_float), ("gamma_plus_one", C.c_int),
-                ("up", C.c_void_p), ("mid_dtype", C.c_int)]
+                ("up", C.c_void_p), ("mid_dtype", C.c_int), ("accumulate", C.c_int)]
 
 
 PRO_NONE, PRO_RMSNORM, PRO_SWIGLU = 0, 1, 2
 
 
-def gemv_multi_fused(ws, x, outs, *, rmsnorm=None, swiglu_up=None, eps=1e-6, gamma_plus_one=True, mid_dtype=None):
+def gemv_multi_fused(ws, x, outs, *, rmsnorm=None, swiglu_up=None, eps=1e-6, gamma_plus_one=True, mid_dtype=None, accumulate=False):
     """tfq_gemv_multi_fused: up to four matrices on fp32 x [B][K] with RMSNorm (rmsnorm = the fp32 gain vector)
     or SwiGLU (x = the gate product, swiglu_up = the up product) applied while the activations are staged."""
     import torch
     n = len(ws)
-    assert x.dtype == torch.float32 and x.is_contiguous()
+    assert x.is_contiguous()
     B = x.shape[0]
     hs = (C.c_void_p * n)(*[w.handle for w in ws])
     ys = (C.c_void_p * n)(*[o.data_ptr() for o in outs])
     pro = _Prologue()
+    pro.accumulate = 1 if accumulate else 0
     if rmsnorm is not None:
         assert rmsnorm.dtype == torch.float32
         pro.op, pro.gamma, pro.eps, pro.gamma_plus_one = PRO_RMSNORM, rmsnorm.data_ptr(), eps, 1 if gamma_plus_one else 0
@@ -512,7 +513,7 @@ def gemv_multi_fused(ws, x, outs, *, rmsnorm=None, swiglu_up=None, eps=1e-6, gam
         assert swiglu_up.dtype == torch.float32 and swiglu_up.shape == x.shape and swiglu_up.is_contiguous()
         pro.op, pro.up = PRO_SWIGLU, swiglu_up.data_ptr()
         pro.mid_dtype = BF16 if mid_dtype == torch.bfloat16 else F32
-    _check(lib().tfq_gemv_multi_fused(hs, n, x.data_ptr(), B, ys, _dtype_code(outs[0]), C.byref(pro), _stream()))
+    _check(lib().tfq_gemv_multi_fused(hs, n, x.data_ptr(), _dtype_code(x), B, ys, _dtype_code(outs[0]), C.byref(pro), _stream()))
     return outs
 
 

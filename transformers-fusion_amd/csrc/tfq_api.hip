@@ -512,12 +512,13 @@ int tfq_moe_ffn_capacity(const tfq_weight_t* const* gate, const tfq_weight_t* co
 
 size_t tfq_mlp_workspace_bytes(int B, int64_t F) { return B > 0 && F > 0 ? mlp_workspace_bytes(B, F) : 0; }
 
-int tfq_gemv_multi_fused(const tfq_weight_t* const* ws, int count, const float* x, int B, void* const* ys, int y_dtype,
+int tfq_gemv_multi_fused(const tfq_weight_t* const* ws, int count, const void* x, int x_dtype, int B, void* const* ys, int y_dtype,
                          const tfq_prologue_t* pro, tfq_stream_t stream) {
     if (!ws || !ys || count < 1 || count > 4) return fail(TFQ_ERR_ARG, "tfq_gemv_multi_fused: one to four matrices");
     if (B < 1 || B > 16) return fail(TFQ_ERR_SHAPE, "tfq_gemv_multi_fused: 1 to 16 activation rows");
     for (int m = 0; m < count; ++m)
-        if (int r = check_matmul("tfq_gemv_multi_fused", ws[m], x, TFQ_F32, B, ys[m], y_dtype)) return r;
+        if (int r = check_matmul("tfq_gemv_multi_fused", ws[m], x, x_dtype, B, ys[m], y_dtype)) return r;
+    if (pro && pro->op != TFQ_PRO_NONE && x_dtype != TFQ_F32) return fail(TFQ_ERR_ARG, "tfq_gemv_multi_fused: a prologue takes fp32 activations");
     if (pro && pro->op != TFQ_PRO_NONE) {
         if (pro->op == TFQ_PRO_RMSNORM) {
             if (!pro->gamma || (uintptr_t)pro->gamma % 16) return fail(TFQ_ERR_ARG, "tfq_gemv_multi_fused: RMSNorm needs a 16-byte aligned gain vector");
@@ -528,7 +529,7 @@ int tfq_gemv_multi_fused(const tfq_weight_t* const* ws, int count, const float* 
             return fail(TFQ_ERR_ARG, "tfq_gemv_multi_fused: unknown prologue");
         }
     }
-    return launch_gemv_multi_fused(ws, count, x, TFQ_F32, B, ys, y_dtype, pro, (hipStream_t)stream);
+    return launch_gemv_multi_fused(ws, count, x, x_dtype, B, ys, y_dtype, pro, (hipStream_t)stream);
 }
 
 int tfq_mlp_step(const tfq_weight_t* gate, const tfq_weight_t* up, const tfq_weight_t* down, const void* x, int x_dtype,

@@ -73,6 +73,7 @@ struct GemvArgs {
     const float* x2;
     float eps;
     int gamma_plus_one, mid_bf16;
+    int accumulate;  // y += product (the residual addition of a decoder layer) instead of y = product
 };
 
 enum : int { XOP_NONE = 0, XOP_RMSNORM = 1, XOP_SWIGLU = 2 };
@@ -94,6 +95,7 @@ struct GemvKernArgs {
     const float* x2;     // XOP_SWIGLU: the second factor, same shape as x
     float eps;
     int gamma_plus_one, mid_bf16;
+    int accumulate;
 };
 
 // Grouped launch: many independent problems (matrix, activation rows, output) of one format and
@@ -470,6 +472,10 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
             v *= 1.0f / sqrtf(tot / (float)K + args.eps);
         }
         const size_t off = (size_t)b * (size_t)nrm + (size_t)row;
+        if (args.accumulate) {  // every output element belongs to one workgroup, so the update needs no atomic
+            if (y_bf16) v += __uint_as_float((uint32_t)reinterpret_cast<const unsigned short*>(ym)[off] << 16);
+            else v += reinterpret_cast<const float*>(ym)[off];
+        }
         if (y_bf16) reinterpret_cast<unsigned short*>(ym)[off] = (unsigned short)bf16_rne(v);
         else reinterpret_cast<float*>(ym)[off] = v;
     }
@@ -873,6 +879,7 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     k.K = a.K; k.y_bf16 = a.y_bf16; k.nslot = a.nslot; k.tiles_per_wg = T;
     k.cols_base = a.cols_base; k.cols_rem = a.cols_rem;
     k.gamma = a.gamma; k.x2 = a.x2; k.eps = a.eps; k.gamma_plus_one = a.gamma_plus_one; k.mid_bf16 = a.mid_bf16;
+    k.accumulate = a.accumulate;
     const int full_items = a.cols_base * T;  // units of a wavefront with the fewest block columns in a full workgroup
     // Two unit fetches in flight per wavefront at most.  Sixteen wavefronts already keep 32 units (74 KB) per
     // compute unit on their way; four per wavefront (which only the one-plane formats with a 16-byte header
@@ -1160,6 +1167,9 @@ bool gemv_prologue_supported(const tfq_weight* w) { return w->layout == TFQ_LAYO
 int launch_gemv_multi_fused(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
                             void* const* ys, int y_dtype, const tfq_prologue_t* pro, hipStream_t s) {
     const bool fused = pro && pro->op != TFQ_PRO_NONE;
+    const bool accumulate = pro && pro->accumulate;
+    if (accumulate && (ws[0]->layout != TFQ_LAYOUT_TILED16 || B > (x_dtype == TFQ_F32 ? 2 : 4)))
+        return fail(TFQ_ERR_SHAPE, "gemv: accumulation into y takes a tiled format and one pass (four bf16 or two fp32 rows)");
     if (fused) {
         if (x_dtype != TFQ_F32) return fail(TFQ_ERR_ARG, "gemv: a prologue takes fp32 activations");
         if (ws[0]->layout != TFQ_LAYOUT_TILED16)
@@ -1201,6 +1211,8 @@ int launch_gemv_multi_fused(const tfq_weight* const* ws, int nmat, const void* x
         a.split_partial = ws[0]->split_partial;
         a.split_counters = ws[0]->split_counters;
     }
+    a.accumulate = accumulate ? 1 : 0;
+    if (accumulate) { a.split_partial = nullptr; a.split_counters = nullptr; }
     if (fused) {
         a.xop = pro->op == TFQ_PRO_RMSNORM ? XOP_RMSNORM : XOP_SWIGLU;
         a.gamma = pro->gamma; a.x2 = pro->up; a.eps = pro->eps;
