@@ -30,7 +30,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes moved per algorithmic byte for the GEMV launches of this workload, from
 # rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy kernel (summary under profiles/)
-HBM_TRAFFIC_RATIO = 1.0240
+HBM_TRAFFIC_RATIO = 1.0245
 # (name, N, K, input) per decoder layer
 PROJ = [("q", 4096, 4096, "x"), ("k", 1024, 4096, "x"), ("v", 1024, 4096, "x"), ("o", 4096, 4096, "a"),
         ("gate", 14336, 4096, "x"), ("up", 14336, 4096, "x"), ("down", 4096, 14336, "h")]
