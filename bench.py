@@ -226,20 +226,21 @@ def chain_step(tfq, torch, layers, bytes_per_step, reps=20):
 
 def fused_launch_step(tfq, torch, layers, bytes_per_step):
     """The same dependent decoder-layer sequence as four launches per layer with every elementwise step inside the
-    launches (tfq_gemv_multi_fused: RMSNorm in front of q/k/v and gate/up, SwiGLU in front of down, the residual
-    additions in the epilogues of o and down), fp32 hidden state.  A side figure, never `value`."""
+    launches (tfq_gemv_multi_fused: RMSNorm in front of q/k/v and gate/up, SwiGLU in the epilogue of the paired
+    gate/up launch, the residual additions in the epilogues of o and down), fp32 hidden state, bf16 SwiGLU product.
+    A side figure, never `value`."""
     dev = "cuda"
     h = torch.from_numpy(tfq.rng_normal(43, 4096)).to(dev).reshape(1, 4096)
     gamma = torch.zeros(4096, device=dev)
     q, k, v = (torch.empty(1, n, device=dev) for n in (4096, 1024, 1024))
-    g, u = torch.empty(1, 14336, device=dev), torch.empty(1, 14336, device=dev)
+    mid = torch.empty(1, 14336, device=dev, dtype=torch.bfloat16)
 
     def step():
         for ws in layers:
             tfq.gemv_multi_fused([ws["q"], ws["k"], ws["v"]], h, [q, k, v], rmsnorm=gamma)
             tfq.gemv_multi_fused([ws["o"]], q, [h], accumulate=True)
-            tfq.gemv_multi_fused([ws["gate"], ws["up"]], h, [g, u], rmsnorm=gamma)
-            tfq.gemv_multi_fused([ws["down"]], g, [h], swiglu_up=u, accumulate=True)
+            tfq.gemv_multi_fused([ws["gate"], ws["up"]], h, [mid], rmsnorm=gamma, pair_swiglu=True)
+            tfq.gemv_multi_fused([ws["down"]], mid, [h], accumulate=True)
     us = time_graph(torch, step)
     return {"launches_per_layer": 4, "us_per_layer": round(us / len(layers), 2), "gbs": round(bytes_per_step / us / 1e3, 1),
             "frac": round(bytes_per_step / us / 1e3 / HBM_PEAK_GBS, 4),

@@ -266,6 +266,9 @@ typedef struct tfq_prologue {
     int gamma_plus_one;
     const float* up;    /* SWIGLU: [B][K] */
     int mid_dtype;      /* SWIGLU: TFQ_F32 or TFQ_BF16 */
+    int pair_swiglu;    /* ws = {gate, up} of equal shape: ys[0] = silu(gate x) * (up x) [B][N] in y_dtype, written by
+                           the launch's epilogue (ys[1] is not written); op TFQ_PRO_NONE or TFQ_PRO_RMSNORM; up to four
+                           bf16 or two fp32 rows; formats B32S4, B32S8, Q_G_4, Q_G_8 */
     int accumulate;     /* ys[i] += product instead of ys[i] = product: the residual addition h += o(...), h += down(...)
                            of a decoder layer (Qwen35Engine::append_token, qwen35_engine.cpp:807-835); any op, x of
                            either type, up to four bf16 or two fp32 rows */
@@ -281,7 +284,8 @@ int tfq_matmul_host(const tfq_weight_t* w, const float* X, float* Y, int B);
  *   y[b] = down( silu(gate x[b]) * (up x[b]) ),  silu(v) = v / (1 + exp(-v))
  * (src/math/math.cpp:117-126).  gate and up are F x D matrices of one format, down is D x F;
  * x is [B][D], y is [B][D], device pointers.  Up to 16 rows and a format with a tiled kernel: two
- * launches, gate and up in one (they share x) and down with silu(gate) * up applied while it stages
+ * launches: gate and up in one whose epilogue writes silu(gate x) * (up x) (up to four bf16 / two fp32 rows,
+ * formats B32S4, B32S8, Q_G_4, Q_G_8) or, failing that, down with the elementwise step applied while it stages
  * its activations; otherwise gate / up, the elementwise step and down are launches of their own.
  * mid_dtype is the type the SwiGLU product is rounded to before
  * the down projection: TFQ_F32 keeps it in fp32 like the reference, TFQ_BF16 feeds the matrix

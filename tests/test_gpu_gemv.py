@@ -503,3 +503,29 @@ def test_accumulate_epilogue_adds_into_y(O, tfq, gpu, xdt, B):
     assert np.abs(y.cpu().numpy() - ref).max() / np.abs(ref).max() <= (1e-2 if xdt == "bf16" else 1e-3)
     with pytest.raises(tfq.TfqError):  # more rows than one pass carries
         tfq.gemv_multi_fused([W], torch.zeros(8, K, device=gpu).bfloat16(), [torch.zeros(8, N, device=gpu)], accumulate=True)
+
+
+@pytest.mark.parametrize("fmt", ["B32S4", "Q_G_4", "B32S8"])
+@pytest.mark.parametrize("xdt,B,norm,ydt", [("bf16", 1, False, "f32"), ("bf16", 4, False, "bf16"), ("f32", 2, False, "f32"),
+                                          ("f32", 1, True, "bf16")])
+def test_paired_gate_up_with_swiglu_epilogue(O, tfq, gpu, fmt, xdt, B, norm, ydt):
+    """gate and up in one launch, silu(gate x) * (up x) written by its epilogue (Qwen35Engine::mlp_step), with and
+    without RMSNorm in front; F = 1040 leaves a partial last tile."""
+    import torch
+    F, D = 1040, 2048
+    pg = O.encode_tensor(fmt, O.rng_normal(90, F * D, 0.02))
+    pu = O.encode_tensor(fmt, O.rng_normal(91, F * D, 0.02))
+    Wg, Wu = tfq.Weight(fmt, F, D, pg), tfq.Weight(fmt, F, D, pu)
+    x = O.rng_normal(92, B * D, 1.0).reshape(B, D)
+    gamma = O.rng_normal(93, D, 0.2)
+    if xdt == "bf16":
+        x = O.bf16_round(x)
+        xd = torch.from_numpy(x).to(gpu).bfloat16()
+    else:
+        xd = torch.from_numpy(x).to(gpu)
+    xin = np.stack([_rmsnorm_ref(x[b], gamma) for b in range(B)]) if norm else x
+    h = torch.zeros(B, F, device=gpu, dtype=torch.bfloat16 if ydt == "bf16" else torch.float32)
+    tfq.gemv_multi_fused([Wg, Wu], xd, [h], pair_swiglu=True, rmsnorm=torch.from_numpy(gamma).to(gpu) if norm else None)
+    ref = O.silu_mul(O.matmul(fmt, pg, F, D, xin).reshape(-1), O.matmul(fmt, pu, F, D, xin).reshape(-1)).reshape(B, F)
+    tol = 1e-2 if (xdt == "bf16" or ydt == "bf16") else 1e-3
+    assert np.abs(h.float().cpu().numpy() - ref).max() / np.abs(ref).max() <= tol

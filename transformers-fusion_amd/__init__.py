@@ -489,13 +489,14 @@ def gemv_multi(weights, x, outs):
 class _Prologue(C.Structure):
     """tfq_prologue_t (include/tfq.h)."""
     _fields_ = [("op", C.c_int), ("gamma", C.c_void_p), ("eps", C.c_float), ("gamma_plus_one", C.c_int),
-                ("up", C.c_void_p), ("mid_dtype", C.c_int), ("accumulate", C.c_int)]
+                ("up", C.c_void_p), ("mid_dtype", C.c_int), ("pair_swiglu", C.c_int), ("accumulate", C.c_int)]
 
 
 PRO_NONE, PRO_RMSNORM, PRO_SWIGLU = 0, 1, 2
 
 
-def gemv_multi_fused(ws, x, outs, *, rmsnorm=None, swiglu_up=None, eps=1e-6, gamma_plus_one=True, mid_dtype=None, accumulate=False):
+def gemv_multi_fused(ws, x, outs, *, rmsnorm=None, swiglu_up=None, eps=1e-6, gamma_plus_one=True, mid_dtype=None, accumulate=False,
+                     pair_swiglu=False):
     """tfq_gemv_multi_fused: up to four matrices on fp32 x [B][K] with RMSNorm (rmsnorm = the fp32 gain vector)
     or SwiGLU (x = the gate product, swiglu_up = the up product) applied while the activations are staged."""
     import torch
@@ -506,6 +507,9 @@ def gemv_multi_fused(ws, x, outs, *, rmsnorm=None, swiglu_up=None, eps=1e-6, gam
     ys = (C.c_void_p * n)(*[o.data_ptr() for o in outs])
     pro = _Prologue()
     pro.accumulate = 1 if accumulate else 0
+    pro.pair_swiglu = 1 if pair_swiglu else 0
+    if pair_swiglu and len(outs) == 1:  # ys[1] is not written; the C call still wants two pointers
+        ys = (C.c_void_p * n)(outs[0].data_ptr(), outs[0].data_ptr())
     if rmsnorm is not None:
         assert rmsnorm.dtype == torch.float32
         pro.op, pro.gamma, pro.eps, pro.gamma_plus_one = PRO_RMSNORM, rmsnorm.data_ptr(), eps, 1 if gamma_plus_one else 0

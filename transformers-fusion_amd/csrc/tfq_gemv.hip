@@ -74,6 +74,7 @@ struct GemvArgs {
     float eps;
     int gamma_plus_one, mid_bf16;
     int accumulate;  // y += product (the residual addition of a decoder layer) instead of y = product
+    int pair;        // W[0] = gate, W[1] = up of equal shape: y[0] = silu(gate x) * (up x), one launch (gemv4_kernel, PAIR)
 };
 
 enum : int { XOP_NONE = 0, XOP_RMSNORM = 1, XOP_SWIGLU = 2 };
@@ -124,11 +125,18 @@ struct GemvProb {
 //   XOP_SWIGLU   x is the gate product and x2 the up product: silu(x) * x2 is staged (math::silu and the
 //                elementwise product of Qwen35Engine::mlp_step, qwen35_engine.cpp:662-672), in fp32 (split into
 //                a bf16 high and low part like every fp32 input) or rounded to bf16 (mid_bf16)
-template <int FMT, bool XF32, int WD, int SETS = 1, bool GROUPED = false, int XOP = XOP_NONE>
+//
+// PAIR = the gate and up products of a SwiGLU feed-forward in one launch with the elementwise step in its
+// epilogue (Qwen35Engine::mlp_step, src/adapters/tools/qwen35_engine.cpp:662-672): W0 is gate, W1 is up (same
+// shape and format); a workgroup walks its T tiles of gate and then the same T tiles of up for every block
+// column (2 T partial-sum cells), and the epilogue writes silu(gate x) * (up x) to y0.  The down product then
+// reads that vector like any other activation, instead of evaluating the exponentials in every workgroup.
+template <int FMT, bool XF32, int WD, int SETS = 1, bool GROUPED = false, int XOP = XOP_NONE, bool PAIR = false>
 __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin_arg) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
     static_assert(XOP == XOP_NONE || (XF32 && SETS == 1 && !GROUPED), "prologues take fp32 input in the plain launch");
+    static_assert(!PAIR || (SETS == 1 && !GROUPED && XOP != XOP_SWIGLU), "the paired launch: one slot set, plain launch");
     constexpr int UB = tiled_unit_bytes(FMT);  // bytes of a unit
     // code registers (uint4) of a unit per lane: nibble formats [plane][k-step] from 1 KB pieces; the 2-bit
     // formats one register of 2-bit fields for both k-steps
@@ -166,7 +174,8 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, q = lane >> 4;
     const int tile0 = (bid - wg_first) * T;              // inside the matrix
-    const int tiles_here = min(T, ((nrm + 15) >> 4) - tile0);
+    const int tiles_real = min(T, ((nrm + 15) >> 4) - tile0);
+    const int tiles_here = PAIR ? 2 * tiles_real : tiles_real;  // PAIR: the tiles of gate, then the same tiles of up
     const int ncols = cols_base + (wave < cols_rem ? 1 : 0);  // block columns wave, wave + NW, ...
     const int ncols_max = cols_base + (cols_rem ? 1 : 0);
     const int nitems = ncols * tiles_here;  // block-column major, tiles inside
@@ -233,6 +242,7 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     // activations alone and a unit is consumed as soon as IT has arrived (behind a conditional
     // fetch the compiler waits for everything in flight).
     const size_t tile_stride = (size_t)nblocks * UB;
+    const ptrdiff_t pair_delta = PAIR ? args.W1 - args.W0 : 0;
     const uint8_t* col_ptr = Wm + ((size_t)tile0 * nblocks + (size_t)wave) * UB;
     const uint8_t* f_ptr = col_ptr;
     int f_t = 0, f_left = nitems;
@@ -248,7 +258,11 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
         for (int i = 0; i < F::HV; ++i) hd[i] = stream_load16(f_ptr + off_h + 16 * i);
         if (--f_left > 0) {
             f_ptr += tile_stride;
-            if (++f_t == tiles_here) {
+            ++f_t;
+            if constexpr (PAIR) {
+                if (f_t == tiles_real) f_ptr = col_ptr + pair_delta;  // the same tiles of the second matrix
+            }
+            if (f_t == tiles_here) {
                 f_t = 0;
                 col_ptr += (size_t)NW * UB;
                 f_ptr = col_ptr;
@@ -330,7 +344,7 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
         stage(p, lo, hi, lo2, hi2);
     }
     // sums of squares of this wavefront's slices, behind the partial sums
-    float* ssq_lds = part + (size_t)T * NW * SETS * 64;
+    float* ssq_lds = part + (size_t)(PAIR ? 2 * T : T) * NW * SETS * 64;
     if constexpr (XOP == XOP_RMSNORM) {
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
@@ -453,7 +467,7 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     constexpr int rows_per_out = XF32 ? 2 : 1;  // fp32 input: high and low part live in adjacent activation rows
     const int nb = nslot / rows_per_out;
     const int bshift = nb > 8 ? 4 : nb > 4 ? 3 : nb > 2 ? 2 : nb - 1;  // log2 of nb rounded up to a power of two
-    const int nout = tiles_here << (4 + bshift);
+    const int nout = tiles_real << (4 + bshift);
     __syncthreads();
     for (int o = tid; o < nout; o += blockDim.x) {
         const int t = o >> (4 + bshift), b = (o >> 4) & ((1 << bshift) - 1), nn = o & 15;
@@ -466,11 +480,22 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
 #pragma unroll
             for (int h = 0; h < rows_per_out; ++h) v += src[w * SETS * 64 + h * 16];
         }
+        float v2 = 0.0f;  // PAIR: the up product of the same output
+        if constexpr (PAIR) {
+            const float* src2 = src + (size_t)tiles_real * NW * SETS * 64;
+            for (int w = 0; w < NW; ++w) {
+#pragma unroll
+                for (int h = 0; h < rows_per_out; ++h) v2 += src2[w * SETS * 64 + h * 16];
+            }
+        }
         if constexpr (XOP == XOP_RMSNORM) {
             float tot = 0.0f;
             for (int w = 0; w < NW; ++w) tot += ssq_lds[w * 2 + b];
-            v *= 1.0f / sqrtf(tot / (float)K + args.eps);
+            const float r = 1.0f / sqrtf(tot / (float)K + args.eps);
+            v *= r;
+            v2 *= r;
         }
+        if constexpr (PAIR) v = v / (1.0f + expf(-v)) * v2;
         const size_t off = (size_t)b * (size_t)nrm + (size_t)row;
         if (args.accumulate) {  // every output element belongs to one workgroup, so the update needs no atomic
             if (y_bf16) v += __uint_as_float((uint32_t)reinterpret_cast<const unsigned short*>(ym)[off] << 16);
@@ -807,6 +832,9 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
 template <int FMT>
 constexpr bool kWide = FMT == TFQ_B32S4 || FMT == TFQ_B32S8 || FMT == TFQ_Q_G_4 || FMT == TFQ_Q_G_8 || FMT == TFQ_Q_8;
 // Formats built with two slot sets only (eight bf16 rows per pass): the affine low-bit formats.
+// Formats whose kernel is also built as the paired gate / up launch with the SwiGLU epilogue.
+template <int FMT>
+constexpr bool kPaired = FMT == TFQ_B32S4 || FMT == TFQ_B32S8 || FMT == TFQ_Q_G_4 || FMT == TFQ_Q_G_8;
 template <int FMT>
 constexpr bool kTwoSets = kWide<FMT> || FMT == TFQ_Q_G_3 || FMT == TFQ_Q_G_2 || FMT == TFQ_SB256A3 || FMT == TFQ_SB256A2;
 
@@ -838,7 +866,7 @@ GemvPlan plan_gemv4(const GemvArgs& a, int nslot) {
     }
     const int ncols_max = (nblocks + p.NW - 1) / p.NW;
     const size_t x_bytes = ((size_t)p.NW * ncols_max * (nslot * 32 + p.sets * Fmt<FMT>::NG) + 4 * p.NW) * 16;
-    const size_t per_tile = (size_t)p.NW * p.sets * 256;
+    const size_t per_tile = (size_t)p.NW * p.sets * 256 * (a.pair ? 2 : 1);  // the paired launch keeps two cells per tile
     // tiles per workgroup: one round of workgroups over the compute units where LDS allows it;
     // every workgroup stays inside one matrix
     auto grid_for = [&](int T) {
@@ -894,6 +922,22 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     const int xi = a.x_f32 ? 1 : 0, wi = wd == 4 ? 2 : wd == 2 ? 1 : 0;
     Kernel kern = kernels[xi][wi];
     int slot = xi * 3 + wi;  // which kernel's LDS limit is being raised
+    if (a.pair) {
+        if constexpr (kPaired<FMT>) {
+            static const Kernel paired[3][2] = {
+                {gemv4_kernel<FMT, false, 1, 1, false, XOP_NONE, true>, gemv4_kernel<FMT, false, 2, 1, false, XOP_NONE, true>},
+                {gemv4_kernel<FMT, true, 1, 1, false, XOP_NONE, true>, gemv4_kernel<FMT, true, 2, 1, false, XOP_NONE, true>},
+                {gemv4_kernel<FMT, true, 1, 1, false, XOP_RMSNORM, true>, gemv4_kernel<FMT, true, 2, 1, false, XOP_RMSNORM, true>}};
+            if (p.sets != 1 || a.xop == XOP_SWIGLU || (a.xop == XOP_RMSNORM && !a.x_f32))
+                return fail(TFQ_ERR_SHAPE, "gemv: the paired gate / up launch takes one pass of rows and at most the RMSNorm prologue");
+            const int ki = !a.x_f32 ? 0 : a.xop == XOP_RMSNORM ? 2 : 1;
+            const int wdp = 2 * full_items >= 2 ? 2 : 1;  // a wavefront walks gate and up: twice the units
+            kern = paired[ki][wdp == 2 ? 1 : 0];
+            slot = 12 + ki * 2 + (wdp == 2 ? 1 : 0);
+        } else {
+            return fail(TFQ_ERR_FORMAT, "gemv: no paired gate / up kernel for this format");
+        }
+    } else
     if (a.xop != XOP_NONE) {
         static const Kernel fused[2][2] = {
             {gemv4_kernel<FMT, true, 1, 1, false, XOP_RMSNORM>, gemv4_kernel<FMT, true, 2, 1, false, XOP_RMSNORM>},
@@ -919,7 +963,7 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     }
     // Raise the dynamic-LDS limit once per kernel (not per launch: the call is
     // not allowed while a stream is being captured into a graph).
-    static std::atomic<bool> lds_limit_raised[12] = {};
+    static std::atomic<bool> lds_limit_raised[20] = {};
     if (!lds_limit_raised[slot]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -1164,10 +1208,22 @@ int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int 
 
 bool gemv_prologue_supported(const tfq_weight* w) { return w->layout == TFQ_LAYOUT_TILED16; }
 
+bool gemv_pair_supported(const tfq_weight* w) {
+    if (w->layout != TFQ_LAYOUT_TILED16) return false;
+    const int f = canonical(w->fmt);
+    return f == TFQ_B32S4 || f == TFQ_B32S8 || f == TFQ_Q_G_4 || f == TFQ_Q_G_8;
+}
+
 int launch_gemv_multi_fused(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
                             void* const* ys, int y_dtype, const tfq_prologue_t* pro, hipStream_t s) {
     const bool fused = pro && pro->op != TFQ_PRO_NONE;
     const bool accumulate = pro && pro->accumulate;
+    const bool pair = pro && pro->pair_swiglu;
+    if (pair) {
+        if (nmat != 2 || ws[0]->N != ws[1]->N || ws[0]->layout != TFQ_LAYOUT_TILED16 || ws[1]->layout != TFQ_LAYOUT_TILED16 ||
+            B > (x_dtype == TFQ_F32 ? 2 : 4) || accumulate || (pro->op != TFQ_PRO_NONE && pro->op != TFQ_PRO_RMSNORM))
+            return fail(TFQ_ERR_SHAPE, "gemv: pair_swiglu takes gate and up of equal shape in a tiled format, one pass of rows, no accumulation");
+    }
     if (accumulate && (ws[0]->layout != TFQ_LAYOUT_TILED16 || B > (x_dtype == TFQ_F32 ? 2 : 4)))
         return fail(TFQ_ERR_SHAPE, "gemv: accumulation into y takes a tiled format and one pass (four bf16 or two fp32 rows)");
     if (fused) {
@@ -1210,6 +1266,12 @@ int launch_gemv_multi_fused(const tfq_weight* const* ws, int nmat, const void* x
     if (nmat == 1) {
         a.split_partial = ws[0]->split_partial;
         a.split_counters = ws[0]->split_counters;
+    }
+    if (pair) {  // one grid over the tiles of gate; the kernel walks the same tiles of up (W[1]) behind them
+        a.pair = 1;
+        a.nmat = 1;
+        a.ntiles = (int)((ws[0]->N + 15) / 16);
+        a.split_partial = nullptr; a.split_counters = nullptr;
     }
     a.accumulate = accumulate ? 1 : 0;
     if (accumulate) { a.split_partial = nullptr; a.split_counters = nullptr; }

@@ -374,6 +374,7 @@ int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int 
 int launch_gemv_multi_fused(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
                             void* const* ys, int y_dtype, const tfq_prologue_t* pro, hipStream_t s);
 bool gemv_prologue_supported(const tfq_weight* w);
+bool gemv_pair_supported(const tfq_weight* w);  // the paired gate / up launch with the SwiGLU epilogue
 int launch_gemv_generic(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype,
                         hipStream_t s);
 // a matrix whose blocks mix wire ids (TFQ_LAYOUT_MIXED)

@@ -477,6 +477,15 @@ int launch_mlp_step(const tfq_weight* gate, const tfq_weight* up, const tfq_weig
     void* h = (uint8_t*)workspace + 2 * part;
     void* scratch = B > 16 ? (uint8_t*)workspace + 3 * part : nullptr;  // K-split partials of the prefill kernel
     const size_t scratch_bytes = B > 16 ? gemm_scratch_bound((size_t)B, (size_t)F) : 0;
+    if (B <= (x_dtype == TFQ_F32 ? 2 : 4) && canonical(gate->fmt) == canonical(up->fmt) && gemv_pair_supported(gate) && gemv_pair_supported(up)) {
+        // gate and up in one launch whose epilogue writes silu(gate x) * (up x); down reads it like any activation
+        const tfq_weight* gu[2] = {gate, up};
+        void* gy[2] = {h, h};
+        tfq_prologue_t pro{};
+        pro.pair_swiglu = 1;
+        if (int rc = launch_gemv_multi_fused(gu, 2, x, x_dtype, B, gy, mid_dtype, &pro, s)) return rc;
+        return launch_gemv(down, h, mid_dtype, B, y, y_dtype, s);
+    }
     if (B <= 16 && canonical(gate->fmt) == canonical(up->fmt)) {
         const tfq_weight* gu[2] = {gate, up};
         void* gy[2] = {g, u};
