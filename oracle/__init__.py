@@ -225,6 +225,20 @@ def rng_laplace(seed: int, n: int, b: float) -> np.ndarray:
     return out
 
 
+def rmsnorm(x, w, eps: float = 1e-6, plus_one: bool = True) -> np.ndarray:
+    """Qwen35Engine::rmsnorm (src/adapters/tools/qwen35_engine.cpp:46-51) for one row:
+    s = sum x_i^2 accumulated in fp32 in index order, r = 1 / sqrt(s / n + eps), out_i = x_i * r * (1 + w_i),
+    every operation in fp32 (plus_one=False: * w_i, the plain form of math::rms_norm)."""
+    x = _f32(x).reshape(-1)
+    w = _f32(w).reshape(-1)
+    s = np.float32(0)
+    for v in x:
+        s = np.float32(s + np.float32(v * v))
+    r = np.float32(1.0) / np.sqrt(np.float32(np.float32(s / np.float32(x.size)) + np.float32(eps)), dtype=np.float32)
+    g = (np.float32(1) + w) if plus_one else w
+    return (np.float32(1) * (x * r) * g).astype(np.float32)
+
+
 def bf16_round(a) -> np.ndarray:
     """fp32 -> nearest-even bf16 -> fp32 (the reference has no bf16 type; this is
     how 'bf16 activations' enter its fp32 matmul)."""

@@ -1,8 +1,8 @@
 """The persistent chain of dependent matrix-vector products (tfq_chain_*) against the oracle.
 
 The oracle side is a composition of pinned pieces: O.matmul (block-row GEMV in the reference's loop order),
-O.silu_mul (src/math/math.cpp:117-126) and the rmsnorm of Qwen35Engine::rmsnorm
-(src/adapters/tools/qwen35_engine.cpp:46-51) restated in numpy below; activations are rounded to bf16 before
+O.silu_mul (src/math/math.cpp:117-126) and O.rmsnorm (Qwen35Engine::rmsnorm,
+src/adapters/tools/qwen35_engine.cpp:46-51); activations are rounded to bf16 before
 every product, as the chain does.  Tolerance: max |y - y_ref| / max |y_ref| <= 1e-2 (bf16 activations).
 """
 import numpy as np
@@ -13,17 +13,6 @@ pytestmark = pytest.mark.gpu
 
 def rel_err(y, ref):
     return float(np.abs(y.astype(np.float64) - ref).max() / np.abs(ref).max())
-
-
-def rmsnorm_ref(x, w, eps=1e-6, plus_one=True):
-    """Qwen35Engine::rmsnorm: out = x * 1/sqrt(sum(x^2)/n + eps) * (1 + w), fp32."""
-    x = x.astype(np.float32)
-    s = np.float32(0)
-    for v in x:  # the reference's sequential fp32 sum
-        s = np.float32(s + v * v)
-    r = np.float32(1.0) / np.sqrt(np.float32(s / np.float32(x.size) + np.float32(eps)), dtype=np.float32)
-    g = (np.float32(1) + w) if plus_one else w
-    return ((x * r) * g).astype(np.float32)
 
 
 def _weights(O, tfq, fmt, shapes, seed):
@@ -93,13 +82,13 @@ def test_chain_decoder_layer_matches_oracle(O, tfq, gpu, fmt):
     torch.cuda.synchronize()
     chain.check()
 
-    xn = O.bf16_round(rmsnorm_ref(h0, g1))
+    xn = O.bf16_round(O.rmsnorm(h0, g1))
     q = O.matmul(fmt, W["q"][1], D, D, xn)
     k = O.matmul(fmt, W["k"][1], KV, D, xn)
     v = O.matmul(fmt, W["v"][1], KV, D, xn)
     o = O.matmul(fmt, W["o"][1], D, D, O.bf16_round(q.reshape(-1)))
     h1 = (h0 + o.reshape(-1)).astype(np.float32)
-    xn2 = O.bf16_round(rmsnorm_ref(h1, g2))
+    xn2 = O.bf16_round(O.rmsnorm(h1, g2))
     g = O.matmul(fmt, W["gate"][1], F, D, xn2)
     u = O.matmul(fmt, W["up"][1], F, D, xn2)
     hh = O.bf16_round(O.silu_mul(g, u))

@@ -420,18 +420,6 @@ def test_long_k_takes_fewer_rows_per_pass(O, tfq, gpu, K, B, xdt):
     W.close()
 
 
-def _rmsnorm_ref(x, w, eps=1e-6, plus_one=True):
-    """Qwen35Engine::rmsnorm (src/adapters/tools/qwen35_engine.cpp:46-51): x * 1/sqrt(sum(x^2)/n + eps) * (1 + w),
-    fp32 with the reference's sequential sum."""
-    x = x.astype(np.float32)
-    s = np.float32(0)
-    for v in x:
-        s = np.float32(s + v * v)
-    r = np.float32(1.0) / np.sqrt(np.float32(s / np.float32(x.size) + np.float32(eps)), dtype=np.float32)
-    g = (np.float32(1) + w) if plus_one else w
-    return ((x * r) * g).astype(np.float32)
-
-
 @pytest.mark.parametrize("fmt", ["B32S4", "Q_G_4", "B32S8", "SB256A3"])
 @pytest.mark.parametrize("B,plus_one", [(1, True), (2, False), (5, True)])
 def test_rmsnorm_prologue_matches_oracle(O, tfq, gpu, fmt, B, plus_one):
@@ -446,7 +434,7 @@ def test_rmsnorm_prologue_matches_oracle(O, tfq, gpu, fmt, B, plus_one):
     outs = [torch.zeros(B, N, device=gpu) for _, N, _ in shapes]
     tfq.gemv_multi_fused(Ws, torch.from_numpy(x).to(gpu), outs, rmsnorm=torch.from_numpy(gamma).to(gpu), eps=1e-6,
                          gamma_plus_one=plus_one)
-    xn = np.stack([_rmsnorm_ref(x[b], gamma, 1e-6, plus_one) for b in range(B)])
+    xn = np.stack([O.rmsnorm(x[b], gamma, 1e-6, plus_one) for b in range(B)])
     for (n, N, _), o in zip(shapes, outs):
         ref = O.matmul(fmt, pays[n], N, K, xn)
         got = o.cpu().numpy()
@@ -523,7 +511,7 @@ def test_paired_gate_up_with_swiglu_epilogue(O, tfq, gpu, fmt, xdt, B, norm, ydt
         xd = torch.from_numpy(x).to(gpu).bfloat16()
     else:
         xd = torch.from_numpy(x).to(gpu)
-    xin = np.stack([_rmsnorm_ref(x[b], gamma) for b in range(B)]) if norm else x
+    xin = np.stack([O.rmsnorm(x[b], gamma) for b in range(B)]) if norm else x
     h = torch.zeros(B, F, device=gpu, dtype=torch.bfloat16 if ydt == "bf16" else torch.float32)
     tfq.gemv_multi_fused([Wg, Wu], xd, [h], pair_swiglu=True, rmsnorm=torch.from_numpy(gamma).to(gpu) if norm else None)
     ref = O.silu_mul(O.matmul(fmt, pg, F, D, xin).reshape(-1), O.matmul(fmt, pu, F, D, xin).reshape(-1)).reshape(B, F)

@@ -107,3 +107,25 @@ def test_moe_ffn_capacity_against_dense_float64(O):
                 drop += 1
     assert nd == drop and drop > 0
     assert np.abs(out - ref).max() / np.abs(ref).max() < 2e-5
+
+
+def test_rmsnorm_closed_forms(O):
+    """O.rmsnorm (Qwen35Engine::rmsnorm, src/adapters/tools/qwen35_engine.cpp:46-51) against what the formula fixes:
+    a constant row, unit root-mean-square of the output for zero gains, scale invariance, the (1 + w) gain (not w),
+    and float64 numpy on a random row."""
+    n = 384
+    c = np.full(n, 3.0, np.float32)
+    out = O.rmsnorm(c, np.zeros(n, np.float32))
+    assert np.allclose(out, 3.0 / np.sqrt(9.0 + 1e-6), rtol=1e-6)
+    x = O.rng_normal(5, n, 2.0)
+    out = O.rmsnorm(x, np.zeros(n, np.float32))
+    assert abs(np.sqrt(np.mean(out.astype(np.float64) ** 2)) - 1.0) < 1e-5  # eps is 1e-6 against mean(x^2) of 4
+    assert np.allclose(O.rmsnorm(8.0 * x, np.zeros(n, np.float32)), out, rtol=1e-5, atol=1e-6)
+    w = O.rng_normal(6, n, 0.3)
+    x64 = x.astype(np.float64)
+    ref = x64 / np.sqrt(np.mean(x64 ** 2) + 1e-6) * (1.0 + w.astype(np.float64))
+    assert np.abs(O.rmsnorm(x, w) - ref).max() <= 2e-6 * np.abs(ref).max()
+    ref_plain = x64 / np.sqrt(np.mean(x64 ** 2) + 1e-6) * w.astype(np.float64)
+    assert np.abs(O.rmsnorm(x, w, plus_one=False) - ref_plain).max() <= 2e-6 * np.abs(ref).max()
+    # a dropped eps would turn a zero row into NaN
+    assert np.array_equal(O.rmsnorm(np.zeros(n, np.float32), w), np.zeros(n, np.float32))
