@@ -61,7 +61,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus above 1 is not supported "
-              "(rows shard over GPUs without a collective, see DESIGN.md)", file=sys.stderr)
+              "(rows of a matrix would shard over GPUs without a collective; that is not built)", file=sys.stderr)
         sys.exit(2)
 
     import torch
