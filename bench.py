@@ -272,7 +272,7 @@ def time_graph(torch, fn, reps=10):
 
 def decode_sweep(tfq, torch, layers, fmt, base):
     """Side figures, never `value`: the decode layer of the main workload at batch 4, 8 and 16 (same weights,
-    same four launches per layer), the 8-bit block-32 format at batch 1 and 16 on eight layers, and the low-bit
+    same four launches per layer), the 8-bit block-32 format at batch 1, 4, 8 and 16 on eight layers, and the low-bit
     superblock formats (Laplace(0, 0.015) weights, 14336x4096, twelve rotated copies) at batch 1 and 8.
     GB/s = algorithmic bytes / time, as for `value`."""
     dev = "cuda"
@@ -308,7 +308,7 @@ def decode_sweep(tfq, torch, layers, fmt, base):
             ws[name] = tfq.Weight("B32S8", N, K, tfq.encode("B32S8", w))
             del w
         ls8.append(ws)
-    out["B32S8"] = {str(B): layer_figures(ls8, "B32S8", B) for B in (1, 16)}
+    out["B32S8"] = {str(B): layer_figures(ls8, "B32S8", B) for B in (1, 4, 8, 16)}
     for ws in ls8:
         for W in ws.values():
             W.close()
