@@ -248,10 +248,10 @@ def test_gemv_many_tiles_per_workgroup(O, tfq, gpu, fmt, N, K, B):
 @pytest.mark.parametrize("N,K,B", [(16 * 256 * 3 + 40, 512, 16), (16 * 300, 4096, 9), (4096, 14336, 16), (1040, 4608, 5),
                                    (16 * 256 * 9, 256, 13), (24, 7168, 8)])
 def test_gemv_five_to_sixteen_rows(O, tfq, gpu, fmt, N, K, B):
-    """Five or more bf16 rows take the tile-major kernel: several tiles per workgroup, K in chunks of 16 block
-    columns (one chunk, a partial last chunk, four chunks), rows not a multiple of four, more tiles than one
-    round of workgroups holds.  Checked against a dense product of the device-decoded matrix (bit-exact by the
-    codec tests), fp32 and bf16 outputs."""
+    """Five or more bf16 rows take the sixteen-row kernel (one block column per wavefront, K parts over workgroups
+    above sixteen block columns): a single block column, sixteen, a partial last part, four parts, rows not a
+    multiple of four, more tiles than one round of workgroups holds.  Checked against a dense product of the
+    device-decoded matrix (bit-exact by the codec tests), fp32 and bf16 outputs."""
     import torch
     print(f"gemv rows {fmt} N={N} K={K} B={B}", flush=True)
     g = torch.Generator(device="cuda").manual_seed(N + K + B)
@@ -283,7 +283,7 @@ def test_gemv_five_to_sixteen_rows(O, tfq, gpu, fmt, N, K, B):
 
 
 def test_gemv_multi_with_eight_rows(O, tfq, gpu):
-    """q/k/v style launch with more than four rows: three matrices, one launch of the tile-major kernel."""
+    """q/k/v style launch with more than four rows: three matrices, one launch of the sixteen-row kernel."""
     import torch
     K, B = 4096, 8
     shapes = [4096, 1024, 1040]

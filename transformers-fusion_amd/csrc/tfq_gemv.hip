@@ -547,36 +547,33 @@ __device__ __forceinline__ void transpose_rows(uint32_t (&v)[4]) {
 }
 
 // ---- five to sixteen bf16 activation rows: gemvb_kernel
-// With that many rows the activations are the operand that has to be reused (sixteen rows of K = 4096 are
-// 128 KB, more than the packed weights a workgroup streams per tile), so the walk is arranged around them:
-//   * K is cut into chunks of KC = 16 block columns.  A workgroup of eight wavefronts stages a chunk of the
-//     activations ONCE (all threads together, bf16 in the MFMA's A-fragment order, group sums beside them);
-//     wavefront w then takes the A fragments of ITS block columns w and w + 8 into registers and visits all
-//     the workgroup's T tiles for that chunk without touching LDS for operands again;
-//   * the MFMA is used densely: A holds up to sixteen activation rows of ONE scale group (lane (s, kq):
-//     elements 8 kq .. 8 kq + 7 of the group, row s), B the 32 weights of that group for sixteen weight rows,
-//     so a unit costs eight MFMAs whatever the row count.  A lane holds its code dwords group-major (group q,
-//     dwords 0..3); transpose_rows makes register g of lane (n, q) dword q of group g.  D[4 q + r][n] comes
-//     out in lane (n, q), register r;
-//   * every wavefront adds its partial sums into its own LDS cells per tile (no barrier while streaming);
-//     after the last chunk the eight partials of each output are added in wavefront order.  With a single K
-//     chunk (K <= 4096) the cells reuse the LDS of the staged activations, which are in registers by then,
-//     and a workgroup can hold many tiles; with several chunks they need room of their own (few tiles).
-// Unit fetches run two ahead (one tile x two columns) with unconditional loads, as in gemv4_kernel.
-constexpr int kGemvbNW = 8, kGemvbKC = 16;
-constexpr int kGemvbMaxT1 = 16;  // tiles per workgroup, single chunk: 16 x 8 KB of cells inside the staging area
-constexpr int kGemvbMaxTn = 2;   // several chunks: cells behind the staging area
-
+// The MFMA is used densely: A holds up to sixteen activation rows of ONE scale group (lane (s, kq): elements
+// 8 kq .. 8 kq + 7 of the group, row s), B the 32 weights of that group for sixteen weight rows, so a unit costs
+// eight MFMAs whatever the row count.  A lane holds its code dwords group-major (group q, dwords 0..3);
+// transpose_rows makes register g of lane (n, q) dword q of group g.  D[4 q + r][n] comes out in lane (n, q),
+// register r.
+// The walk: a wavefront owns block columns wave, wave + NW, ... of its workgroup's K part and takes the A
+// fragments of a column from global memory itself, so no wavefront waits for another before the end.  The group
+// sums come from the matrix cores as well: A times a B operand of ones leaves sum_k A[4 q + r][k] in register r
+// of every lane of row q.  They are kept (times -OFFS) in 512 bytes of LDS of the wavefront's own and read back
+// per unit as the start value of the accumulators.  A workgroup covers T tiles x one K part; the wavefronts'
+// partial sums meet in LDS cells at the end, and the K parts of a row group (SPLIT: single matrix, K above
+// sixteen block columns) through the handle's partial buffer.  Unit fetches run two ahead with unconditional
+// loads, as in gemv4_kernel.
+// Measured at sixteen rows on the Llama-3-8B decoder shapes (B32S4, kernel trace medians): 8.0 / 8.0 / 16.2 /
+// 16.8 us for q+k+v, o, gate+up, down, against 9.6 / 8.4 / 20.5 / 17.5 us for a walk that staged sixteen block
+// columns of activations per workgroup behind two barriers.  With the A loads and the arithmetic taken out the
+// same launches take 6.2 / 6.2 / 14.0 / 14.5 us: what is left above the single-row kernel (5.6 / 4.6 / 13.3 /
+// 9.0 us) is mostly the K-part rendezvous of the down launch (two dependent device-scope round trips).  Three
+// or four unit fetches in flight, eight wavefronts of two columns, and fewer tiles per workgroup measured equal
+// or slower.
+constexpr int kGemvbKC = 16;  // block columns per K part
 template <int FMT, bool SPLIT>
-__global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const unsigned short* __restrict__ x) {
+__global__ __launch_bounds__(1024) void gemvb_kernel(GemvKernArgs args, const unsigned short* __restrict__ x) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
     static_assert(F::GS == 32 && F::HV == 1, "32-weight groups and a 16-byte header");
-    constexpr int UB = tiled_unit_bytes(FMT), NC = 2 * F::NP, NW = kGemvbNW, KC = kGemvbKC;
-    // unit fetches in flight per wavefront: TW tiles x two columns.  One tile (two fetches) measured faster than
-    // two at sixteen rows: B32S4 4096x14336 17.6 against 18.5 us, 6144x4096 9.6 / 10.3 us, 4096x4096 8.3 / 8.6 us,
-    // 28672x4096 equal; B32S8 28672x4096 32.5 / 35.9 us, 4096x14336 22.8 / 24.5 us (four tiles no faster than two)
-    constexpr int TW = 1, WD = 2 * TW;
+    constexpr int UB = tiled_unit_bytes(FMT), NC = 2 * F::NP, WD = 2;
     const int K = args.K, T = args.tiles_per_wg, B = args.nslot;
     const bool y_bf16 = args.y_bf16 != 0;
     const int bid = blockIdx.x;
@@ -586,223 +583,233 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
     void* ym = m == 0 ? args.y0 : m == 1 ? args.y1 : m == 2 ? args.y2 : args.y3;
     const int nrm = m == 0 ? args.nr0 : m == 1 ? args.nr1 : m == 2 ? args.nr2 : args.nr3;
 
-    // K split over workgroups (single matrix): workgroup bid walks part bid % kparts, kcols <= KC block columns,
-    // of row group bid / kparts; the parts of a row group meet through the partial sums at the end.  Without
-    // the split a workgroup walks all the chunks of KC columns itself.
-    constexpr bool split = SPLIT;
-    const int kparts = split ? args.kparts : 1;
-    const int kcols = split ? args.kcols : KC;
+    const int kparts = SPLIT ? args.kparts : 1;
     const int nblocks = K >> 8;
-    const int chunk_first = split ? bid % kparts : 0;
-    const int nchunks = split ? 1 : (nblocks + KC - 1) / KC;
+    const int kcols = SPLIT ? args.kcols : nblocks;
+    const int part = SPLIT ? bid % kparts : 0;
+    const int rowgroup = SPLIT ? bid / kparts : bid - wg_first;
+    const int col0 = part * kcols;
+    const int cols_here = min(kcols, nblocks - col0);
+    const int NW = blockDim.x >> 6;
+    const int nw_live = min(NW, cols_here);  // wavefronts that own a block column
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, q = lane >> 4;
-    const int rowgroup = split ? bid / kparts : bid - wg_first;
     const int tile0 = rowgroup * T;
     const int tiles_here = min(T, ((nrm + 15) >> 4) - tile0);
-    const int total_gt = nchunks * tiles_here;  // (chunk, tile) visits, chunk-major
+    const int ncols = wave < cols_here ? (cols_here - wave + NW - 1) / NW : 0;
+    const int nitems = ncols * tiles_here;  // block-column major, tiles inside
 
-    uint4* const xa = smem;                                          // [KC][2 k-steps][4 groups][64 lanes]
-    float* const xsum = reinterpret_cast<float*>(smem + KC * 512);   // [KC][8 groups][16 rows]
-    // partial sums [T][NW][64 lanes][4]: inside xa when there is one chunk, behind xsum otherwise
-    float* const cells = nchunks == 1 ? reinterpret_cast<float*>(smem) : xsum + KC * 128;
+    float* const xs = reinterpret_cast<float*>(smem) + wave * 128;  // this wavefront's group sums [2 k-steps][4 groups][16 rows]
+    uint4* const stg = smem + NW * 32 + wave * 128;                 // this wavefront's 2 KB for turning loaded rows into A fragments
+    float4* const cells = reinterpret_cast<float4*>(smem + NW * 160);  // [T][NW][64 lanes]
 
-    // ---- unit fetch cursor in consumption order: chunk, tile, column slot (two per wavefront and chunk).
-    // A slot past the last block column re-reads the last one (never used); past the end the cursor parks.
-    int f_chunk = 0, f_t = 0, f_ci = 0;
-    const uint32_t off_c = 16u * lane, off_h = 1024u * NC + 16u * n;
-    auto fetch = [&](uint4 (&cc)[NC], uint4& hd) __attribute__((always_inline)) {
-        // a slot with no column of its own in this chunk re-reads a column the wavefront does own (cache hit, never used)
-        const int col0 = (chunk_first + f_chunk) * kcols, cols_here = min(kcols, nblocks - col0);
-        const int c_slot = wave + NW * f_ci;
-        const int col = col0 + (c_slot < cols_here ? c_slot : min(wave, cols_here - 1));
-        const uint8_t* p = Wm + ((size_t)(tile0 + f_t) * nblocks + (size_t)col) * UB;
+    if (nitems > 0) {
+        // ---- A fragments of one block column: lane (s = n, kq = q) holds elements 8 kq .. 8 kq + 7 of every group of
+        // row s.  Loaded that way a quarter wavefront would touch sixteen rows (sixteen cache lines for 256 bytes);
+        // instead a load covers eight rows x 128 bytes (lane: row lane / 8, 16-byte piece lane % 8 = (group of a
+        // pair, kq)), two full lines per quarter, and the pieces change lanes through the wavefront's own LDS: a
+        // pair of groups is written (two loads: rows 0..7, 8..15) and read back in fragment order.  The row index
+        // is xor-ed with twice the piece index so that the sixteen lanes of a quarter hit sixteen different
+        // 16-byte bank groups on the way in and on the way out.
+        uint4 avr[2][4];
+        const int piece = lane & 7, lrow = lane >> 3;
+        const unsigned short* xrow0 = x + (size_t)min(lrow, B - 1) * K + piece * 8;
+        const unsigned short* xrow1 = x + (size_t)min(8 + lrow, B - 1) * K + piece * 8;
+        const int w_slot0 = (piece >> 2) * 64 + (piece & 3) * 16 + (lrow ^ (piece * 2));
+        const int w_slot1 = (piece >> 2) * 64 + (piece & 3) * 16 + ((8 + lrow) ^ (piece * 2));
+        const int r_slot0 = q * 16 + (n ^ (q * 2));
+        const int r_slot1 = 64 + q * 16 + (n ^ ((4 + q) * 2));
+        auto load_a = [&](int col) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < NC; ++i) cc[i] = stream_load16(p + off_c + 1024 * i);
-        hd = stream_load16(p + off_h);
-        if (++f_ci == 2) {
-            f_ci = 0;
-            if (++f_t == tiles_here) {
-                f_t = 0;
-                if (f_chunk + 1 < nchunks) ++f_chunk; else f_t = tiles_here - 1, f_ci = 1;  // park on the last unit
-            }
-        }
-    };
-    uint4 cc[WD][NC], hd[WD];
+            for (int h = 0; h < 2; ++h)
 #pragma unroll
-    for (int u = 0; u < WD; ++u) fetch(cc[u], hd[u]);
-
-    const uint32_t ONES = 0x3F803F80u;
-    const uint32_t M = 0x000F000Fu;
-    uint32_t C = 0x43004300u;
-    asm volatile("" : "+v"(C));
-
-    // ---- activations of one K chunk -> LDS.  Item e = (column c, k-step h, group g, row s, slot kq), kq fastest:
-    // four adjacent lanes hold the four 8-element pieces of one group of one row, so their sums meet with two
-    // DPP adds; the entry lands where lane (s, kq) of a wavefront will read it with one 128-bit LDS load.
-    auto stage_chunk = [&](int chunk) __attribute__((always_inline)) {
-        const int cols_here = min(kcols, nblocks - chunk * kcols);
-        const unsigned short* xc = x + (size_t)chunk * kcols * 256;
-        for (int e0 = 0; e0 < cols_here * 512; e0 += 512 * 4) {  // four loads of a thread in flight together
-            uint4 v[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int e = e0 + 512 * i + tid;
-                const int kq = e & 3, s = (e >> 2) & 15, g = (e >> 6) & 3, h = (e >> 8) & 1, c = e >> 9;
-                v[i] = uint4{0, 0, 0, 0};
-                if (c < cols_here && s < B)
-                    v[i] = *reinterpret_cast<const uint4*>(xc + (size_t)s * K + c * 256 + h * 128 + g * 32 + kq * 8);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int e = e0 + 512 * i + tid;
-                const int kq = e & 3, s = (e >> 2) & 15, g = (e >> 6) & 3, h = (e >> 8) & 1, c = e >> 9;
-                const uint4 p = pair_permute(v[i]);
-                float sum = dot2(ONES, p.x, 0.0f);
-                sum = dot2(ONES, p.y, sum);
-                sum = dot2(ONES, p.z, sum);
-                sum = dot2(ONES, p.w, sum);
-                sum = dpp_add<0xB1>(sum);
-                sum = dpp_add<0x4E>(sum);
-                if (c < cols_here) {
-                    xa[((c * 2 + h) * 4 + g) * 64 + kq * 16 + s] = p;
-                    // kept as -OFFS * sum: the accumulators start from it (the codes ride on an offset of OFFS)
-                    if (kq == 0) xsum[(c * 8 + h * 4 + g) * 16 + s] = -F::OFFS * sum;
+                for (int gp = 0; gp < 2; ++gp) {
+                    const int o = col * 256 + h * 128 + gp * 64;
+                    avr[h][2 * gp] = *reinterpret_cast<const uint4*>(xrow0 + o);
+                    avr[h][2 * gp + 1] = *reinterpret_cast<const uint4*>(xrow1 + o);
                 }
-            }
-        }
-    };
-
-    // ---- the wavefront's A fragments of its two block columns of the chunk (64 registers), and the group sums
-    // too where the unit ring leaves room (one nibble plane); otherwise the sums are read from LDS per unit
-    constexpr bool XREG = false;  // keeping the sums in registers as well spills a few registers
-    uint4 avr[2][2][4];
-    float4 xr[XREG ? 2 : 1][2][4];
-    auto load_columns = [&](int chunk) __attribute__((always_inline)) {
+        };
+        auto finish_a = [&]() __attribute__((always_inline)) {
+            const uint4 ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
 #pragma unroll
-        for (int ci = 0; ci < 2; ++ci) {
-            const int c_local = wave + NW * ci;
-            if (c_local >= kcols || chunk * kcols + c_local >= nblocks) continue;
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int gp = 0; gp < 2; ++gp) {
+                    stg[w_slot0] = avr[h][2 * gp];
+                    stg[w_slot1] = avr[h][2 * gp + 1];
+                    avr[h][2 * gp] = stg[r_slot0];
+                    avr[h][2 * gp + 1] = stg[r_slot1];
+                }
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    avr[ci][h][g] = xa[((c_local * 2 + h) * 4 + g) * 64 + lane];
-                    if constexpr (XREG) xr[ci][h][g] = *reinterpret_cast<const float4*>(xsum + (c_local * 8 + h * 4 + g) * 16 + 4 * q);
+                    uint4 v = avr[h][g];
+                    if (n >= B) v = uint4{0, 0, 0, 0};
+                    v = pair_permute(v);
+                    avr[h][g] = v;
+                    const f32x4_t S = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, v), __builtin_bit_cast(bf16x8_t, ones),
+                                                                              f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+                    if (n == 0)
+                        *reinterpret_cast<float4*>(xs + (h * 4 + g) * 16 + 4 * q) =
+                            float4{-F::OFFS * S[0], -F::OFFS * S[1], -F::OFFS * S[2], -F::OFFS * S[3]};
                 }
-        }
-    };
+        };
+        load_a(col0 + wave);
 
-    // ---- one unit: the lane's contribution to D[4 q + r][n], r = 0..3, added into res
-    auto compute = [&](int ci, int c_local, const uint4 (&cw_all)[NC], const uint4& hdr, float (&res)[4]) __attribute__((always_inline)) {
+        // ---- unit fetch cursor in consumption order; past the end it stays on the last unit (never used)
+        const size_t tile_stride = (size_t)nblocks * UB;
+        const uint8_t* col_ptr = Wm + ((size_t)tile0 * nblocks + (size_t)(col0 + wave)) * UB;
+        const uint8_t* f_ptr = col_ptr;
+        int f_t = 0, f_left = nitems;
+        const uint32_t off_c = 16u * lane, off_h = 1024u * NC + 16u * n;
+        auto fetch = [&](uint4 (&cc)[NC], uint4& hd) __attribute__((always_inline)) {
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            f32x4_t D[4], D2[4];
-            float X[4][4];
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                float4 xv;
-                if constexpr (XREG) xv = xr[ci][h][g];
-                else xv = *reinterpret_cast<const float4*>(xsum + (c_local * 8 + h * 4 + g) * 16 + 4 * q);
-                X[g][0] = xv.x; X[g][1] = xv.y; X[g][2] = xv.z; X[g][3] = xv.w;
-                D[g] = f32x4_t{xv.x, xv.y, xv.z, xv.w};
-                D2[g] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int i = 0; i < NC; ++i) cc[i] = stream_load16(f_ptr + off_c + 1024 * i);
+            hd = stream_load16(f_ptr + off_h);
+            if (--f_left > 0) {
+                f_ptr += tile_stride;
+                if (++f_t == tiles_here) {
+                    f_t = 0;
+                    col_ptr += (size_t)NW * UB;
+                    f_ptr = col_ptr;
+                }
             }
+        };
+        uint4 cc[WD][NC], hd[WD];
 #pragma unroll
-            for (int pl = 0; pl < F::NP; ++pl) {
-                const uint4 cw = cw_all[2 * pl + h];
-                uint32_t t[4] = {cw.x, cw.y, cw.z, cw.w};
-                transpose_rows(t);
+        for (int u = 0; u < WD; ++u) fetch(cc[u], hd[u]);
+        finish_a();
+
+        const uint32_t M = 0x000F000Fu;
+        uint32_t C = 0x43004300u;
+        asm volatile("" : "+v"(C));
+        int c_ci = 0, c_t = 0;
+        auto consume = [&](const uint4 (&cw_all)[NC], const uint4& hdr) __attribute__((always_inline)) {
+            if (c_t == 0 && c_ci > 0) {
+                load_a(col0 + wave + NW * c_ci);
+                finish_a();
+            }
+            float res[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                f32x4_t D[4], D2[4];
+                float X[4][4];
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const uint32_t v = t[g];
-                    const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
-                    if (pl == 0)
-                        D[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, avr[ci][h][g]),
-                                                                       __builtin_bit_cast(bf16x8_t, wv), D[g], 0, 0, 0);
-                    else
-                        D2[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, avr[ci][h][g]),
-                                                                        __builtin_bit_cast(bf16x8_t, wv), D2[g], 0, 0, 0);
+                    const float4 xv = *reinterpret_cast<const float4*>(xs + (h * 4 + g) * 16 + 4 * q);
+                    X[g][0] = xv.x; X[g][1] = xv.y; X[g][2] = xv.z; X[g][3] = xv.w;
+                    D[g] = f32x4_t{xv.x, xv.y, xv.z, xv.w};
+                    D2[g] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
                 }
+#pragma unroll
+                for (int pl = 0; pl < F::NP; ++pl) {
+                    const uint4 cw = cw_all[2 * pl + h];
+                    uint32_t t[4] = {cw.x, cw.y, cw.z, cw.w};
+                    transpose_rows(t);
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const uint32_t v = t[g];
+                        const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
+                        if (pl == 0)
+                            D[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, avr[h][g]),
+                                                                           __builtin_bit_cast(bf16x8_t, wv), D[g], 0, 0, 0);
+                        else
+                            D2[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, avr[h][g]),
+                                                                            __builtin_bit_cast(bf16x8_t, wv), D2[g], 0, 0, 0);
+                    }
+                }
+                float a[4], off[4];
+                group_scales<FMT>(&hdr, h, a, off);
+                if constexpr (!(FMT == TFQ_B32S4 || F::NP == 2)) {  // X holds -OFFS * (group sum)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) off[g] *= -1.0f / F::OFFS;
+                }
+                float ph[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        float d = D[g][r];
+                        if constexpr (F::NP == 2) d = __builtin_fmaf(16.0f, D2[g][r], d);
+                        ph[r] = __builtin_fmaf(a[g], d, ph[r]);
+                        if constexpr (!(FMT == TFQ_B32S4 || F::NP == 2)) ph[r] = __builtin_fmaf(off[g], X[g][r], ph[r]);
+                    }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) res[r] += F::COMP8 ? ph[r] * kComp8Gain : ph[r];
             }
-            float a[4], off[4];
-            group_scales<FMT>(&hdr, h, a, off);
-            if constexpr (!(FMT == TFQ_B32S4 || F::NP == 2)) {  // X holds -OFFS * (group sum)
+            float4* cell = cells + (c_t * NW + wave) * 64 + lane;
+            if (c_ci == 0) *cell = float4{res[0], res[1], res[2], res[3]};
+            else { const float4 o = *cell; *cell = float4{o.x + res[0], o.y + res[1], o.z + res[2], o.w + res[3]}; }
+            if (++c_t == tiles_here) { c_t = 0; ++c_ci; }
+        };
+        const int groups = (nitems + WD - 1) / WD;
+        for (int g = 1; g < groups; ++g) {
 #pragma unroll
-                for (int g = 0; g < 4; ++g) off[g] *= -1.0f / F::OFFS;
-            }
-            float ph[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-            for (int g = 0; g < 4; ++g)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    float d = D[g][r];
-                    if constexpr (F::NP == 2) d = __builtin_fmaf(16.0f, D2[g][r], d);
-                    ph[r] = __builtin_fmaf(a[g], d, ph[r]);
-                    if constexpr (!(FMT == TFQ_B32S4 || F::NP == 2)) ph[r] = __builtin_fmaf(off[g], X[g][r], ph[r]);
-                }
-#pragma unroll
-            for (int r = 0; r < 4; ++r) res[r] += F::COMP8 ? ph[r] * kComp8Gain : ph[r];
-        }
-    };
-
-    for (int gt0 = 0; gt0 < total_gt; gt0 += TW) {
-#pragma unroll
-        for (int dt = 0; dt < TW; ++dt) {
-            const int gt = gt0 + dt;
-            if (gt < total_gt) {  // uniform over the workgroup
-                const int lchunk = gt / tiles_here, t = gt - lchunk * tiles_here;
-                const int chunk = chunk_first + lchunk;
-                if (t == 0) {
-                    __syncthreads();  // every wavefront holds the previous chunk's fragments in registers, or is done with them
-                    stage_chunk(chunk);
-                    __syncthreads();
-                    load_columns(chunk);
-                    if (nchunks == 1) __syncthreads();  // the cells below overwrite the staged activations
-                }
-                float res[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                for (int ci = 0; ci < 2; ++ci) {
-                    const int u = dt * 2 + ci;
-                    const int c_local = wave + NW * ci;
-                    if (c_local < kcols && chunk * kcols + c_local < nblocks) compute(ci, c_local, cc[u], hd[u], res);
-                    fetch(cc[u], hd[u]);
-                }
-                float4* cell = reinterpret_cast<float4*>(cells) + (t * NW + wave) * 64 + lane;
-                if (lchunk == 0) *cell = float4{res[0], res[1], res[2], res[3]};
-                else { const float4 o = *cell; *cell = float4{o.x + res[0], o.y + res[1], o.z + res[2], o.w + res[3]}; }
+            for (int u = 0; u < WD; ++u) {
+                consume(cc[u], hd[u]);
+                fetch(cc[u], hd[u]);
             }
         }
+        const int last0 = (groups - 1) * WD;
+#pragma unroll
+        for (int u = 0; u < WD; ++u)
+            if (last0 + u < nitems) consume(cc[u], hd[u]);
     }
     __syncthreads();
-    // ---- add the eight wavefronts' partials in order and store: thread tid < 256 owns D[4 q' + r][n'] with
-    // (n', q') = lane id tid % 64 and r = tid / 64, for every tile
-    const int nn = tid & 15, qq = (tid >> 4) & 3, r = tid >> 6;
-    const int slot = 4 * qq + r;
-    const bool owner = tid < 256 && slot < B;
-    if (owner) {
-        for (int t = 0; t < tiles_here; ++t) {
-            const int row = (tile0 + t) * 16 + nn;
-            if (row >= nrm) continue;
-            const float* src = cells + ((size_t)t * NW * 64 + (tid & 63)) * 4 + r;
-            float v = 0.0f;
+    // ---- add the wavefronts' partials in wavefront order and store.  Wavefront w takes tiles w, w + NW, ...; its lane
+    // (n, q) holds D[4 q + r][n], r = 0..3, of the tile: the same cell layout the streaming loop wrote, so every read
+    // is one 128-bit LDS load, four of them in flight at a time.
+    auto sum_cells = [&](int t) __attribute__((always_inline)) {
+        const float4* src = cells + (size_t)t * NW * 64 + lane;
+        float4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int w0 = 0; w0 < nw_live; w0 += 4) {
+            float4 v[4];
 #pragma unroll
-            for (int w = 0; w < NW; ++w) v += src[w * 256];
+            for (int j = 0; j < 4; ++j) v[j] = w0 + j < nw_live ? src[(w0 + j) * 64] : float4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) { acc.x += v[j].x; acc.y += v[j].y; acc.z += v[j].z; acc.w += v[j].w; }
+        }
+        return acc;
+    };
+    auto store_out = [&](int t, const float4& v) __attribute__((always_inline)) {
+        const int row = (tile0 + t) * 16 + n;
+        if (row >= nrm) return;
+        const float o[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int slot = 4 * q + r;
+            if (slot >= B) continue;
             const size_t off = (size_t)slot * (size_t)nrm + (size_t)row;
-            if (split) __hip_atomic_store(args.partial + (size_t)chunk_first * 16 * (size_t)nrm + off, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            else if (y_bf16) reinterpret_cast<unsigned short*>(ym)[off] = (unsigned short)bf16_rne(v);
-            else reinterpret_cast<float*>(ym)[off] = v;
+            if (y_bf16) reinterpret_cast<unsigned short*>(ym)[off] = (unsigned short)bf16_rne(o[r]);
+            else reinterpret_cast<float*>(ym)[off] = o[r];
+        }
+    };
+    for (int t = wave; t < tiles_here; t += NW) {
+        const float4 v = sum_cells(t);
+        if constexpr (SPLIT) {
+            const int row = (tile0 + t) * 16 + n;
+            if (row >= nrm) continue;
+            const float o[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int slot = 4 * q + r;
+                if (slot < B)
+                    __hip_atomic_store(args.partial + (size_t)part * 16 * (size_t)nrm + (size_t)slot * (size_t)nrm + (size_t)row, o[r],
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        } else {
+            store_out(t, v);
         }
     }
-    if constexpr (split) {
+    if constexpr (SPLIT) {
         // The last part of a row group to arrive adds the parts in part order (the same sum whichever part
         // that is) and puts the counter back to zero for the next launch.  Every workgroup passes through
-        // here exactly once and waits for nobody.
-        int& last_arrival = *reinterpret_cast<int*>(xsum);  // the group sums are no longer needed; the cells are elsewhere
-        // The partial sums are device-scope stores (written through to where every compute unit sees them) and
-        // are read back with device-scope loads, so no cache write-back or invalidation is needed: it is enough
-        // that every store of the workgroup has completed before its arrival is counted.
+        // here exactly once and waits for nobody.  The partial sums are device-scope stores and are read back
+        // with device-scope loads: it is enough that every store of the workgroup has completed before its
+        // arrival is counted.
+        int& last_arrival = *reinterpret_cast<int*>(smem);  // the group sums are no longer needed
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (tid == 0) {
@@ -812,17 +819,20 @@ __global__ __launch_bounds__(512) void gemvb_kernel(GemvKernArgs args, const uns
         }
         __syncthreads();
         if (last_arrival) {
-            if (owner) {
-                for (int t = 0; t < tiles_here; ++t) {
-                    const int row = (tile0 + t) * 16 + nn;
-                    if (row >= nrm) continue;
-                    const size_t off = (size_t)slot * (size_t)nrm + (size_t)row;
-                    float v = 0.0f;
-                    for (int c = 0; c < kparts; ++c)
-                        v += __hip_atomic_load(args.partial + (size_t)c * 16 * (size_t)nrm + off, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (y_bf16) reinterpret_cast<unsigned short*>(ym)[off] = (unsigned short)bf16_rne(v);
-                    else reinterpret_cast<float*>(ym)[off] = v;
+            for (int t = wave; t < tiles_here; t += NW) {
+                const int row = (tile0 + t) * 16 + n;
+                if (row >= nrm) continue;
+                float o[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                for (int c = 0; c < kparts; ++c) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int slot = 4 * q + r;
+                        if (slot < B)
+                            o[r] += __hip_atomic_load(args.partial + (size_t)c * 16 * (size_t)nrm + (size_t)slot * (size_t)nrm + (size_t)row,
+                                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
                 }
+                store_out(t, float4{o[0], o[1], o[2], o[3]});
             }
         }
     }
@@ -978,25 +988,25 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
 template <int FMT>
 int run_gemvb(GemvArgs a, const void* x, hipStream_t s) {
     constexpr int num_cu = 256;
+    const int nblocks = a.K >> 8;
     auto grid_for = [&](int T) {
         int g = 0;
         for (int m = 0; m < a.nmat; ++m) g += ((a.nrows[m] + 15) / 16 + T - 1) / T;
         return g;
     };
-    int nchunks = ((a.K >> 8) + kGemvbKC - 1) / kGemvbKC;
-    // Several chunks and a handle with room for partial sums: one workgroup per (row group, K part).  Every
-    // workgroup then stages one part of the activations once and walks many tiles with it, instead of staging
-    // every chunk for one or two tiles (the staging is what such a launch otherwise spends most of its time on).
-    const bool split = nchunks > 1 && a.nmat == 1 && a.split_partial != nullptr;
-    const int kparts = split ? nchunks : 1;
-    if (split) nchunks = 1;
-    const int max_t = nchunks == 1 ? kGemvbMaxT1 : kGemvbMaxTn;
+    // K parts over workgroups (single matrix with a partial buffer on its handle): parts of at most sixteen
+    // block columns, one per wavefront
+    const bool split = nblocks > kGemvbKC && a.nmat == 1 && a.split_partial != nullptr;
+    const int kparts = split ? (nblocks + kGemvbKC - 1) / kGemvbKC : 1;
+    const int kcols = split ? (nblocks + kparts - 1) / kparts : nblocks;
+    const int NW = kcols < 16 ? kcols : 16;  // a wavefront per block column of the part, at most sixteen
+    const int max_t = (int)((160 * 1024 - (size_t)NW * 2560) / ((size_t)NW * 1024));
     int T = (a.ntiles * kparts + num_cu - 1) / num_cu;
     while (grid_for(T) * kparts > num_cu && T < max_t) ++T;
     if (T > max_t) T = max_t;
     GemvKernArgs k{};
     k.kparts = kparts;
-    k.kcols = split ? ((a.K >> 8) + kparts - 1) / kparts : kGemvbKC;
+    k.kcols = kcols;
     k.partial = a.split_partial;
     k.counters = a.split_counters;
     k.W0 = a.W[0]; k.W1 = a.W[1]; k.W2 = a.W[2]; k.W3 = a.W[3];
@@ -1015,20 +1025,16 @@ int run_gemvb(GemvArgs a, const void* x, hipStream_t s) {
         grid *= kparts;
     }
     k.K = a.K; k.y_bf16 = a.y_bf16; k.nslot = a.nslot; k.tiles_per_wg = T;
-    // staged activations and group sums of a chunk; the cells are inside them (one chunk) or behind them
-    const size_t lds = (size_t)kGemvbKC * (8192 + 512) + (nchunks == 1 ? 0 : (size_t)T * kGemvbNW * 1024);
-    static std::atomic<bool> lds_limit_raised{false};
-    if (!lds_limit_raised) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemvb_kernel<FMT, false>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemvb_kernel<FMT, true>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    const size_t lds = (size_t)NW * 2560 + (size_t)T * NW * 1024;
+    using Kernel = void (*)(GemvKernArgs, const unsigned short*);
+    const Kernel kern = split ? gemvb_kernel<FMT, true> : gemvb_kernel<FMT, false>;
+    static std::atomic<bool> lds_limit_raised[2] = {};
+    if (!lds_limit_raised[split ? 1 : 0]) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
-        lds_limit_raised = true;
+        lds_limit_raised[split ? 1 : 0] = true;
     }
-    if (split) hipLaunchKernelGGL((gemvb_kernel<FMT, true>), dim3(grid), dim3(64 * kGemvbNW), lds, s, k, static_cast<const unsigned short*>(x));
-    else hipLaunchKernelGGL((gemvb_kernel<FMT, false>), dim3(grid), dim3(64 * kGemvbNW), lds, s, k, static_cast<const unsigned short*>(x));
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, s, k, static_cast<const unsigned short*>(x));
     return hip_fail(hipGetLastError(), "gemv launch");
 }
 
@@ -1040,14 +1046,14 @@ int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t 
     a.y_bf16 = yd == TFQ_BF16;
     a.x_f32 = xd == TFQ_F32;
     if constexpr (kWide<FMT>) {
-        // Five rows or more: the tile-major kernel carries sixteen rows per pass at any K.  Measured against the
-        // slot-set kernels below (B32S4): faster for more than eight rows (28672x4096 at 16 rows: 22 us against
-        // 41 us) and wherever those need several passes because their staged activations do not fit
-        // (4096x14336: 22 us against 24 / 47 us at 8 / 16 rows); slower for five to eight rows at K = 4096
-        // (21 us against 17 us), which therefore stay with the two-set kernel.
-        bool tile_major = !a.x_f32 && B > 8;
-        if (!a.x_f32 && B > 4 && B <= 8) tile_major = plan_gemv4<FMT>(a, 8).lds == 0;
-        if (tile_major) {
+        // Five rows or more: gemvb_kernel carries sixteen rows per pass at any K.  Measured against the slot-set
+        // kernels below (B32S4, kernel trace medians): faster for more than eight rows (28672x4096 at 16 rows:
+        // 16 us against 41 us) and wherever those need several passes because their staged activations do not
+        // fit (4096x14336: 17 us against 24 / 47 us at 8 / 16 rows); equal for five to eight rows at K = 4096
+        // (q+k+v 8.1 / 8.0, o 7.6 / 7.2, gate+up 15.6 / 15.7 us), which stay with the two-set kernel.
+        bool dense_rows = !a.x_f32 && B > 8;
+        if (!a.x_f32 && B > 4 && B <= 8) dense_rows = plan_gemv4<FMT>(a, 8).lds == 0;
+        if (dense_rows) {
             for (int b0 = 0; b0 < B; b0 += 16) {
                 GemvArgs ab = a;
                 ab.nslot = B - b0 < 16 ? B - b0 : 16;
@@ -1137,7 +1143,7 @@ int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, 
 
 }  // namespace
 
-// formats whose 5..16-row calls take the tile-major batched kernel (one pass over the weights per 16 rows)
+// formats whose 5..16-row calls take gemvb_kernel (one pass over the weights per 16 rows)
 bool gemv_rows16_supported(int fmt) {
     switch (canonical(fmt)) {
         case TFQ_Q_G_4: case TFQ_B32S4: case TFQ_B32S8: case TFQ_Q_G_8: case TFQ_Q_8: return true;
