@@ -6,7 +6,9 @@
 //
 // A workgroup of 8 wavefronts owns an output tile of 256 tokens x 256, 224 or 128 weight rows and walks K in
 // steps of 32 (one scale group per weight row).  Per step it
-//   * copies the 256 x 32 activation tile to LDS (bf16), global -> LDS without passing registers,
+//   * copies half of a 256 x 64 activation chunk to LDS (bf16), global -> LDS without passing registers, a whole
+//     128-byte line per row (64 bytes per row, one step's worth, left L2 at half the rate: a loop of nothing
+//     but the copies and the barriers took 140 us for 14336x4096 x 2048 tokens against 85 us with whole lines),
 //   * decodes the weight tile: one lane takes one or two code dwords (8 weights each),
 //     converts the nibbles with v_cvt_f32_ubyte, applies the group's scale and
 //     offset in fp32
@@ -14,16 +16,21 @@
 //     packs to bf16 (v_cvt_pk_bf16_f32) and stores the 8 weights to LDS,
 //   * runs 32, 28 or 16 v_mfma_f32_16x16x32_bf16 per wavefront (sub-tiles of 128 x 64, 64 x 112, 64 x 64:
 //     LDS reads per MFMA are what bounds this kernel, and they shrink with the sub-tile's size).
-// Global loads are issued three steps ahead of the step that multiplies their data, into four LDS buffers
-// (activations) and a ring of four register sets (code dwords), and are waited for by exact counts, so
-// HBM / L2 latency overlaps with arithmetic.  Weights are read from the
+// Global loads are issued ahead of the step that multiplies their data (activation chunks two chunks, into four
+// LDS buffers; code dwords three steps, into a ring of four register sets) and are waited for by exact counts,
+// so HBM / L2 latency overlaps with arithmetic.  Weights are read from the
 // Tiled16 layout, where the 16 rows of a tile hold a group as 256 contiguous bytes.
 // Workgroups are numbered so that the ones running together on an XCD share a
 // token tile: the activations, the larger operand by bytes, are then served from
 // that XCD's L2 and only the packed weights stream from HBM.
 // The matrix pipeline takes an MFMA every 16 cycles only while at most two other vector instructions are
 // issued per MFMA; two wavefronts per SIMD (512 threads) let one wavefront's decode and LDS traffic fill
-// the other's MFMA shadow without any hand scheduling.
+// the other's MFMA shadow.  On a full grid the step is cut in two phases with a barrier each (loads, fragment
+// reads, decode | MFMAs) and the two wavefronts of a SIMD are kept in opposite phases (PP below).
+// Where the time of a step goes (14336x4096 x 2048 tokens, B32S4, 253 us; parts taken out at compile time):
+// without the decode and its LDS stores 175 us, without the fragment reads 188 us, without the MFMAs 218 us,
+// loads and barriers alone 100 us: the decode's vector instructions (about 58 per wavefront and step beside 28
+// MFMAs) are the largest part, and they are already at one decode per weight and workgroup.
 
 #include <algorithm>
 #include <atomic>
@@ -125,7 +132,7 @@ __device__ __forceinline__ void group_coeffs(uint4 h, int g, float& a, float& c)
     }
 }
 
-template <int FMT, int BN, int NT>
+template <int FMT, int BN, int NT, bool PP>
 __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
     constexpr int XL = BM * 4 / NT;     // activation copies per thread and step (rows NT / 4 apart)
     constexpr int BNA = BN > 128 ? 256 : 128;  // rows of the strip's LDS buffers and of the decode (224: the last 32 are spare)
@@ -138,10 +145,12 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
     constexpr int WAVES_N = BN == 256 ? 4 : 2;
     constexpr int WAVES_M = NT / 64 / WAVES_N;
     constexpr int MI = BM / WAVES_M / 16, NJ = BN / WAVES_N / 16;
-    // activations: four buffers of a 256 x 32 bf16 step (copied three steps ahead); weights: two buffers
+    // activations: four buffers of a 256 x 64 bf16 chunk (two steps; copied two chunks ahead, whole 128-byte
+    // lines per row; four, so that a step's buffer is known at compile time: a block is four chunks); weights:
+    // two buffers of a step
     extern __shared__ uint4 smem[];
-    uint4* const xs = smem;                 // [4][BM * 4]
-    uint4* const wsm = smem + 4 * BM * 4;   // [2][BNA * 4]
+    uint4* const xs = smem;                 // [4][BM * 8]
+    uint4* const wsm = smem + 4 * BM * 8;   // [2][BNA * 4]
     const int M = args.M, N = args.N, K = args.K;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // workgroup -> (token tile, weight strip).  Workgroups are dealt to the 8 XCDs round robin, and the
@@ -173,14 +182,23 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
     // once; with plain [row][segment] rows 64 bytes apart they would share banks four ways.
     // Threads are matched to (row, segment) so that their writes follow the same rule (slot = tid).
     auto lds_index = [](int row, int seg) { return ((row >> 3) << 5) + (seg << 3) + (row & 7); };
-    const int xr0 = (tid & 7) + ((tid >> 5) << 3), xseg = (tid >> 3) & 3;
-    const int wr = xr0, wj = xseg;
+    // Activation chunks are copied a whole cache line per row: eight adjacent lanes take the eight 16-byte pieces
+    // of a row's 128 bytes (copies of 64 bytes per row, one step's worth, moved half as many bytes per second
+    // out of L2).  global -> LDS copies land at consecutive 16-byte slots in lane order, so the chunk is stored
+    // [row][8 pieces]; which piece a lane takes is xor-ed with the row (mod 8), and so is the piece index of a
+    // fragment read: the eight lanes an LDS access serves together (consecutive rows, same piece) then touch
+    // eight different 16-byte bank groups.
+    const int wr = (tid & 7) + ((tid >> 5) << 3), wj = (tid >> 3) & 3;
+    const int xpiece = (tid & 7) ^ ((tid >> 3) & 7);
     const int wn = (n0 + wr) & 15;  // RSTRIDE is a multiple of 16: the same row of a 16-row tile for all of a thread's rows
     // Addresses are a scalar base (advanced per step / per block) plus a 32-bit offset per thread
     // (the host side keeps both operands below 4 GiB).
-    uint32_t xoff[XL], woff[WROWS];
+    uint32_t xoff0[XL], xoff1[XL], woff[WROWS];  // activations: the halves of a chunk, rows 0..127 / 128..255
 #pragma unroll
-    for (int i = 0; i < XL; ++i) xoff[i] = (uint32_t)(((size_t)min(m0 + xr0 + i * RSTRIDE, M - 1) * K + xseg * 8) * 2);
+    for (int i = 0; i < XL; ++i) {
+        xoff0[i] = (uint32_t)(((size_t)min(m0 + i * (NT / 8) + (tid >> 3), M - 1) * K + xpiece * 8) * 2);
+        xoff1[i] = (uint32_t)(((size_t)min(m0 + 128 + i * (NT / 8) + (tid >> 3), M - 1) * K + xpiece * 8) * 2);
+    }
 #pragma unroll
     for (int i = 0; i < WROWS; ++i)
         woff[i] = (uint32_t)((size_t)min((n0 + wr + i * RSTRIDE) >> 4, ntiles16 - 1) * nblocks * UB + 16 * wn + 4 * wj);
@@ -202,13 +220,15 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const uint8_t* const xbytes = reinterpret_cast<const uint8_t*>(args.X) + (size_t)split * nb_walk * 512;
     const uint8_t* const wbytes = args.W + (size_t)split * nb_walk * UB;
-    auto copy_x = [&](int ks_) __attribute__((always_inline)) {
-        const int ks = min(ks_, nsteps - 1);  // past the end: the last step again, no branch
-        const uint8_t* base = xbytes + (size_t)ks * (BK * 2);
+    // half H (static) of chunk `chunk` into chunk buffer `cbuf`
+    const int nchunks = nsteps >> 1;
+    auto copy_x = [&]<int H>(int chunk, int cbuf) __attribute__((always_inline)) {
+        const uint8_t* base = xbytes + (size_t)min(chunk, nchunks - 1) * 128;  // past the end: the last chunk again, no branch
 #pragma unroll
         for (int i = 0; i < XL; ++i) {
-            const uint32_t dst = lds_x + (uint32_t)(((ks_ & 3) * BM * 4 + 64 * wave_u + i * NT) * 16);
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(xoff[i]), "s"(base) : "memory");
+            const uint32_t dst = lds_x + (uint32_t)((cbuf * BM + H * 128 + i * (NT / 8) + 8 * wave_u) * 128);
+            const uint32_t off = H ? xoff1[i] : xoff0[i];
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(base) : "memory");
         }
     };
     // code dword of group G (static) of the block at `base` (W + 2304 * block); G == 0 also fetches the
@@ -270,38 +290,69 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
 #pragma unroll
         for (int j = 0; j < NJ; ++j) acc[i][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    copy_x(0); load_step.template operator()<0, 0>(wbytes);
-    copy_x(1); load_step.template operator()<1, 1>(wbytes);
-    copy_x(2); load_step.template operator()<2, 2>(wbytes);
+    // chunks 0 and 1 whole, the code dwords of steps 0..2; from then on step ks issues half ks % 2 of chunk
+    // ks / 2 + 2 and the code dwords of step ks + 3
+    copy_x.template operator()<0>(0, 0); copy_x.template operator()<1>(0, 0);
+    copy_x.template operator()<0>(1, 1); copy_x.template operator()<1>(1, 1);
+    load_step.template operator()<0, 0>(wbytes);
+    load_step.template operator()<1, 1>(wbytes);
+    load_step.template operator()<2, 2>(wbytes);
     arrive.template operator()<0, 0, true>();
     store_step.template operator()<0, 0>(0);
     __syncthreads();
-    // One trip of the loop is a 256-wide block (eight steps), so a step's group index is static.
-    // Step U consumes the code dwords of step U + 1 (issued two steps earlier); behind them in the queue
-    // are the loads issued by the previous step and by this one.
+    // fragment reads of the activations: row wm * (MI * 16) + i * 16 + fr, piece (step parity * 4 + fk) ^ (row % 8)
+    const int xfrag0 = (wm * (MI * 16) + fr) * 8 + (fk ^ (fr & 7)), xfrag1 = (wm * (MI * 16) + fr) * 8 + ((4 + fk) ^ (fr & 7));
+    // One trip of the loop is a 256-wide block (eight steps, four chunks), so a step's group index and buffers
+    // are static.  Step U consumes the code dwords of step U + 1 (issued two steps earlier); behind them in the
+    // queue are the loads issued by the previous step and by this one.  A chunk's halves were issued four and
+    // three steps before its first step, so they have landed (for every wavefront: there is a barrier per step)
+    // by then; the buffer a step copies into was last read two steps ago.
     auto step = [&]<int U>(int ks0, const uint8_t* cur, const uint8_t* nxt) __attribute__((always_inline)) {
         const int ks = ks0 + U, buf = U & 1;
         constexpr int PER_STEP = XL + WROWS * NP;
         constexpr int PENDING = 2 * PER_STEP + WROWS * (((U + 2) & 7) == 0) + WROWS * (((U + 3) & 7) == 0);
-        // buffer (ks + 3) % 4 was read during step ks - 1, which every wavefront has left
-        copy_x(ks + 3);
+        copy_x.template operator()<U & 1>((ks >> 1) + 2, ((U >> 1) + 2) & 3);
         load_step.template operator()<(U + 3) & 7, (U + 3) & 3>(U + 3 < 8 ? cur : nxt);
         uint4 af[MI], bfr[NJ];
 #pragma unroll
         for (int j = 0; j < NJ; ++j) bfr[j] = wsm[buf * BNA * 4 + lds_index(wn_ * (NJ * 16) + j * 16 + fr, fk)];
 #pragma unroll
-        for (int i = 0; i < MI; ++i) af[i] = xs[(U & 3) * BM * 4 + lds_index(wm * (MI * 16) + i * 16 + fr, fk)];
+        for (int i = 0; i < MI; ++i) af[i] = xs[(U >> 1) * BM * 8 + ((U & 1) ? xfrag1 : xfrag0) + i * 128];
+        if constexpr (PP) {
+            // Two phases with a barrier after each: L (the loads above, decode and LDS store of the next step's
+            // weights) and C (the MFMAs, on registers only).  The second half of the wavefronts runs one barrier
+            // behind the first (see below), so on every SIMD one wavefront is in its C phase while the other is
+            // in its L phase.
+            arrive.template operator()<PENDING, (U + 1) & 3, ((U + 1) & 7) == 0>();
+            store_step.template operator()<(U + 1) & 7, (U + 1) & 3>(buf ^ 1);  // past the end: written, never read
+            // every LDS read of this phase has returned and every store is done before the others move on
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(1);
+        }
 #pragma unroll
         for (int i = 0; i < MI; ++i)
 #pragma unroll
             for (int j = 0; j < NJ; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[i]),
                                                                     __builtin_bit_cast(bf16x8_t, bfr[j]), acc[i][j], 0, 0, 0);
-        // the activation copies of step ks + 1 were issued before its code dwords: they have landed too
-        arrive.template operator()<PENDING, (U + 1) & 3, ((U + 1) & 7) == 0>();
-        store_step.template operator()<(U + 1) & 7, (U + 1) & 3>(buf ^ 1);  // past the end: written, never read
-        __syncthreads();
+        if constexpr (PP) {
+            __builtin_amdgcn_s_setprio(0);
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+        } else {
+            // the activation copies of step ks + 1 were issued before its code dwords: they have landed too
+            arrive.template operator()<PENDING, (U + 1) & 3, ((U + 1) & 7) == 0>();
+            store_step.template operator()<(U + 1) & 7, (U + 1) & 3>(buf ^ 1);  // past the end: written, never read
+            __syncthreads();
+        }
     };
+    if constexpr (PP) {
+        if (wave_u >= NT / 128) __builtin_amdgcn_s_barrier();  // the second half of the wavefronts: one phase behind
+    }
     for (int ks0 = 0; ks0 < nsteps; ks0 += 8) {
         const int blk = ks0 >> 3;
         const uint8_t* cur = wbytes + (size_t)blk * UB;
@@ -314,6 +365,9 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
         step.template operator()<5>(ks0, cur, nxt);
         step.template operator()<6>(ks0, cur, nxt);
         step.template operator()<7>(ks0, cur, nxt);
+    }
+    if constexpr (PP) {
+        if (wave_u < NT / 128) __builtin_amdgcn_s_barrier();  // the first half passes the barrier the second half started with
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may land in LDS after the workgroup is gone
     // the last steps' loads (for steps past the end) are never read, but they still write their registers:
@@ -364,15 +418,20 @@ template <int FMT, int BN, int NT>
 int run_tiles(GemmArgs a, hipStream_t s) {
     a.tiles_n = (a.N + BN - 1) / BN;
     const int grid = 8 * ((a.tiles_m * a.tiles_n * a.ksplit + 7) / 8);
-    constexpr size_t lds = (size_t)(4 * BM * 4 + 2 * (BN > 128 ? 256 : 128) * 4) * 16;  // 96 KB or 80 KB
-    static std::atomic<bool> lds_limit_raised{false};  // once: not allowed while a stream is being captured
-    if (!lds_limit_raised) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm4_kernel<FMT, BN, NT>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    // The two-phase form (see the kernel) when there is at least a workgroup per compute unit: measured 2-5 %
+    // faster there (B32S4 14336x4096 x 2048 tokens 259 -> 253 us, 4096x14336 239 -> 233 us; B32S8 253 -> 240 us),
+    // equal or slower on smaller grids.
+    const bool pp = a.tiles_m * a.tiles_n * a.ksplit >= 256;
+    constexpr size_t lds = (size_t)(4 * BM * 8 + 2 * (BN > 128 ? 256 : 128) * 4) * 16;  // 160 KB or 144 KB
+    using Kernel = void (*)(GemmArgs);
+    const Kernel kern = pp ? gemm4_kernel<FMT, BN, NT, true> : gemm4_kernel<FMT, BN, NT, false>;
+    static std::atomic<bool> lds_limit_raised[2] = {};  // once: not allowed while a stream is being captured
+    if (!lds_limit_raised[pp]) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
-        lds_limit_raised = true;
+        lds_limit_raised[pp] = true;
     }
-    hipLaunchKernelGGL((gemm4_kernel<FMT, BN, NT>), dim3(grid), dim3(NT), lds, s, a);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), lds, s, a);
     if (a.ksplit > 1) {
         const size_t n = (size_t)a.M * a.N;
         hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, a.partial, a.Y, n, a.ksplit, a.y_bf16);
