@@ -107,6 +107,7 @@ struct GemvProb {
     const uint8_t* W;
     void* y;
     const void* x;
+    const uint8_t* W2;  // paired plan: the up matrix (W is gate)
     int nrows;
     int nslot;
     int wg_first;  // first workgroup of this problem
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
     static_assert(XOP == XOP_NONE || (XF32 && SETS == 1 && !GROUPED), "prologues take fp32 input in the plain launch");
-    static_assert(!PAIR || (SETS == 1 && !GROUPED && XOP != XOP_SWIGLU), "the paired launch: one slot set, plain launch");
+    static_assert(!PAIR || ((GROUPED || SETS == 1) && XOP != XOP_SWIGLU), "the paired launch: one slot set unless grouped");
     constexpr int UB = tiled_unit_bytes(FMT);  // bytes of a unit
     // code registers (uint4) of a unit per lane: nibble formats [plane][k-step] from 1 KB pieces; the 2-bit
     // formats one register of 2-bit fields for both k-steps
@@ -150,6 +151,7 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     const int bid = blockIdx.x;
     int wg_first, nrm, nslot;
     const uint8_t* Wm;
+    const uint8_t* Wm2 = nullptr;  // PAIR: the second matrix
     void* ym;
     const void* xin;
     if constexpr (GROUPED) {
@@ -158,6 +160,7 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
         const GemvProb pr = table[wg_map[bid]];
         wg_first = pr.wg_first; nrm = pr.nrows; nslot = pr.nslot;
         Wm = pr.W; ym = pr.y; xin = pr.x;
+        Wm2 = pr.W2;
     } else {
         const int m = (bid >= args.g0) + (bid >= args.g1) + (bid >= args.g2);
         wg_first = m == 0 ? 0 : m == 1 ? args.g0 : m == 2 ? args.g1 : args.g2;
@@ -166,6 +169,7 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
         nrm = m == 0 ? args.nr0 : m == 1 ? args.nr1 : m == 2 ? args.nr2 : args.nr3;
         nslot = args.nslot;
         xin = xin_arg;
+        Wm2 = args.W1;
     }
 
     const int nblocks = K >> 8;
@@ -242,7 +246,7 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     // activations alone and a unit is consumed as soon as IT has arrived (behind a conditional
     // fetch the compiler waits for everything in flight).
     const size_t tile_stride = (size_t)nblocks * UB;
-    const ptrdiff_t pair_delta = PAIR ? args.W1 - args.W0 : 0;
+    const ptrdiff_t pair_delta = PAIR ? Wm2 - Wm : 0;
     const uint8_t* col_ptr = Wm + ((size_t)tile0 * nblocks + (size_t)wave) * UB;
     const uint8_t* f_ptr = col_ptr;
     int f_t = 0, f_left = nitems;
@@ -1087,7 +1091,7 @@ int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t 
 
 // ---- grouped launch
 template <int FMT>
-int plan_grouped(int K, bool x_f32, const int* nrows, const int* nrows_x, int nprob, GemvGroupPlan* gp) {
+int plan_grouped(int K, bool x_f32, const int* nrows, const int* nrows_x, int nprob, GemvGroupPlan* gp, bool pair) {
     const int nblocks = K >> 8;
     int max_rows = 1;
     for (int i = 0; i < nprob; ++i) max_rows = nrows_x[i] > max_rows ? nrows_x[i] : max_rows;
@@ -1098,16 +1102,19 @@ int plan_grouped(int K, bool x_f32, const int* nrows, const int* nrows_x, int np
     a.nmat = 1;
     a.nrows[0] = nrows[0];
     a.ntiles = (nrows[0] + 15) / 16;
+    a.pair = pair ? 1 : 0;
     GemvPlan p = plan_gemv4<FMT>(a, nslot);
     if (p.lds == 0) return fail(TFQ_ERR_SHAPE, "gemv group: the activation rows of one problem do not fit in LDS");
     // tiles per workgroup: about 512 KB of packed weights each (a workgroup stages its activations before it
     // streams, and that start-up is paid per workgroup: 512 KB measured 4 % faster than 256 KB on the
     // mixture layer), within what LDS leaves for the partial sums
-    const size_t per_tile = (size_t)p.NW * p.sets * 256, x_bytes = p.lds - (size_t)p.T * per_tile;
+    const size_t per_tile = (size_t)p.NW * p.sets * 256 * (pair ? 2 : 1), x_bytes = p.lds - (size_t)p.T * per_tile;
     int T = (int)((512 * 1024 + (size_t)nblocks * tiled_unit_bytes(FMT) - 1) / ((size_t)nblocks * tiled_unit_bytes(FMT)));
+    if (pair) T = (T + 1) / 2;  // a workgroup walks its tiles of both matrices
     while (T > 1 && x_bytes + (size_t)T * per_tile > 160 * 1024) --T;
     gp->NW = p.NW; gp->T = T; gp->sets = p.sets; gp->lds = x_bytes + (size_t)T * per_tile;
     gp->x_f32 = x_f32;
+    gp->pair = pair;
     gp->K = K;
     int grid = 0;
     for (int i = 0; i < nprob; ++i) grid += ((nrows[i] + 15) / 16 + T - 1) / T;
@@ -1125,13 +1132,27 @@ int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, 
     k.cols_base = nblocks / gp.NW; k.cols_rem = nblocks % gp.NW;
     using Kernel = void (*)(GemvKernArgs, const void*);
     constexpr int WDG = 2;  // two unit fetches in flight: every format's kernel holds that many without spilling
+    // The two-set kernel (eight wavefronts per workgroup) takes four here: with two, a compute unit has 37 KB on
+    // its way and the grouped gate / up launch of a mixture layer streams at 4.45 TB/s (118.6 us); with four,
+    // 110.3 us.  The plain launch of the same kernel is slower with four (gate + up at eight rows 16.8 against
+    // 15.7 us) and keeps two.
     Kernel kern = gp.x_f32 ? gemv4_kernel<FMT, true, WDG, 1, true> : gemv4_kernel<FMT, false, WDG, 1, true>;
     int slot = gp.x_f32 ? 1 : 0;
     if constexpr (kWide<FMT>) {
-        if (gp.sets == 2) { kern = gemv4_kernel<FMT, false, 2, 2, true>; slot = 2; }
+        if (gp.sets == 2) { kern = gemv4_kernel<FMT, false, 4, 2, true>; slot = 2; }
         if (gp.sets == 4) { kern = gemv4_kernel<FMT, false, 1, 4, true>; slot = 3; }
     }
-    static std::atomic<bool> lds_limit_raised[4] = {};
+    if (gp.pair) {
+        if constexpr (kPaired<FMT>) {
+            kern = gp.x_f32 ? gemv4_kernel<FMT, true, WDG, 1, true, XOP_NONE, true> : gemv4_kernel<FMT, false, WDG, 1, true, XOP_NONE, true>;
+            slot = gp.x_f32 ? 5 : 4;
+            if (gp.sets == 2) { kern = gemv4_kernel<FMT, false, 4, 2, true, XOP_NONE, true>; slot = 6; }
+            if (gp.sets == 4) { kern = gemv4_kernel<FMT, false, 1, 4, true, XOP_NONE, true>; slot = 7; }
+        } else {
+            return fail(TFQ_ERR_FORMAT, "gemv group: no paired kernel for this format");
+        }
+    }
+    static std::atomic<bool> lds_limit_raised[8] = {};
     if (!lds_limit_raised[slot]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
@@ -1169,13 +1190,13 @@ bool gemv_grouped_supported(int fmt) {
     }
 }
 
-int plan_gemv_grouped(int fmt, int K, bool x_f32, const int* nrows, const int* nrows_x, int nprob, GemvGroupPlan* gp) {
+int plan_gemv_grouped(int fmt, int K, bool x_f32, const int* nrows, const int* nrows_x, int nprob, GemvGroupPlan* gp, bool pair) {
     if (nprob <= 0) return fail(TFQ_ERR_ARG, "gemv group: no problems");
     switch (canonical(fmt)) {
-        case TFQ_Q_G_4: return plan_grouped<TFQ_Q_G_4>(K, x_f32, nrows, nrows_x, nprob, gp);
-        case TFQ_B32S4: return plan_grouped<TFQ_B32S4>(K, x_f32, nrows, nrows_x, nprob, gp);
-        case TFQ_B32S8: return plan_grouped<TFQ_B32S8>(K, x_f32, nrows, nrows_x, nprob, gp);
-        case TFQ_Q_G_8: return plan_grouped<TFQ_Q_G_8>(K, x_f32, nrows, nrows_x, nprob, gp);
+        case TFQ_Q_G_4: return plan_grouped<TFQ_Q_G_4>(K, x_f32, nrows, nrows_x, nprob, gp, pair);
+        case TFQ_B32S4: return plan_grouped<TFQ_B32S4>(K, x_f32, nrows, nrows_x, nprob, gp, pair);
+        case TFQ_B32S8: return plan_grouped<TFQ_B32S8>(K, x_f32, nrows, nrows_x, nprob, gp, pair);
+        case TFQ_Q_G_8: return plan_grouped<TFQ_Q_G_8>(K, x_f32, nrows, nrows_x, nprob, gp, pair);
         default: return fail(TFQ_ERR_FORMAT, "gemv group: no grouped kernel for this format");
     }
 }
@@ -1183,12 +1204,12 @@ int plan_gemv_grouped(int fmt, int K, bool x_f32, const int* nrows, const int* n
 // Fills the host images of the problem table (nprob entries of gemv_group_entry_bytes() each) and of the
 // workgroup map (gp.grid ints).
 void fill_gemv_group(const GemvGroupPlan& gp, const tfq_weight* const* ws, const void* const* xs, void* const* ys,
-                     const int* nrows_x, int nprob, void* table_host, int* map_host) {
+                     const int* nrows_x, int nprob, void* table_host, int* map_host, const tfq_weight* const* ws2) {
     GemvProb* t = static_cast<GemvProb*>(table_host);
     int wg = 0;
     for (int i = 0; i < nprob; ++i) {
         const int n = ((int)((ws[i]->N + 15) / 16) + gp.T - 1) / gp.T;
-        t[i] = GemvProb{ws[i]->dev, ys[i], xs[i], (int)ws[i]->N, gp.x_f32 ? 2 * nrows_x[i] : nrows_x[i], wg, 0};
+        t[i] = GemvProb{ws[i]->dev, ys[i], xs[i], ws2 ? ws2[i]->dev : nullptr, (int)ws[i]->N, gp.x_f32 ? 2 * nrows_x[i] : nrows_x[i], wg, 0};
         for (int j = 0; j < n; ++j) map_host[wg + j] = i;
         wg += n;
     }

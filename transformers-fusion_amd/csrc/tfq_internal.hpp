@@ -387,6 +387,7 @@ int launch_decode_mixed(const tfq_weight* w, float* out, hipStream_t s);
 struct GemvGroupPlan {
     int NW, T, sets, grid, K;
     bool x_f32;
+    bool pair;  // every problem is a gate / up pair: y = silu(gate x) * (up x)
     size_t lds;
 };
 bool gemv_grouped_supported(int fmt);
@@ -394,10 +395,11 @@ bool gemv_rows16_supported(int fmt);
 // K parts of the 5..16-row decode kernel (1: no split) and the bytes of partial sums and counters they need
 int gemv_rows16_parts(int fmt, int64_t K);
 size_t gemv_rows16_split_bytes(int fmt, int64_t N, int64_t K);
-int plan_gemv_grouped(int fmt, int K, bool x_f32, const int* nrows, const int* nrows_x, int nprob, GemvGroupPlan* gp);
+int plan_gemv_grouped(int fmt, int K, bool x_f32, const int* nrows, const int* nrows_x, int nprob, GemvGroupPlan* gp, bool pair = false);
 size_t gemv_group_entry_bytes();
+// ws2: the second matrix of every problem (the up matrices of a paired plan), or null
 void fill_gemv_group(const GemvGroupPlan& gp, const tfq_weight* const* ws, const void* const* xs, void* const* ys,
-                     const int* nrows_x, int nprob, void* table_host, int* map_host);
+                     const int* nrows_x, int nprob, void* table_host, int* map_host, const tfq_weight* const* ws2 = nullptr);
 int launch_gemv_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s);
 size_t moe_workspace_bytes(int T, int Ktop, int64_t D, int64_t F);
 size_t mlp_workspace_bytes(int B, int64_t F);

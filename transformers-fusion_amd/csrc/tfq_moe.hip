@@ -12,7 +12,7 @@
 // A (token, expert) pair is one row of every intermediate buffer, pairs in expert-major
 // order.  One launch gathers the activation rows of all pairs, the experts' gate/up and
 // down GEMVs run one after the other on their slices of those buffers, SwiGLU is one
-// launch over all pairs, and one launch combines: the lane that owns out[t][d] adds its
+// launch over all pairs (or the epilogue of the grouped gate / up launch), and one launch combines: the lane that owns out[t][d] adds its
 // token's pairs in ascending expert order, which is the reference's accumulation order
 // (expert-major), without atomics, so results are deterministic.  For the formats with a
 // grouped GEMV kernel all experts' gate/up products are ONE launch and all down products
@@ -334,36 +334,38 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
     const bool grouped = P > 0 && !tall && gemv_grouped_supported(gate[0]->fmt) && gemv_grouped_supported(down[0]->fmt) &&
                          canonical(gate[0]->fmt) == canonical(up[0]->fmt);
     GemvGroupPlan planA{}, planB{};
-    std::vector<const tfq_weight*> wA, wB;
+    std::vector<const tfq_weight*> wA, wA2, wB;
     std::vector<const void*> xA, xB;
     std::vector<void*> yA, yB;
     std::vector<int> nA, nB, rA, rB;
     if (grouped) {
         int max_nt = 1;
         for (int e = 0; e < E; ++e) max_nt = std::max(max_nt, first[e + 1] - first[e]);
-        auto chunk_cap = [&](int fmt, int K, bool f32, int nrows) {
+        auto chunk_cap = [&](int fmt, int K, bool f32, int nrows, bool pair) {
             if (f32) return 2;
             for (int cap = 16; cap > 4; cap >>= 1) {
                 if (cap / 2 >= max_nt) continue;  // a smaller pass already holds every expert's rows
                 GemvGroupPlan probe{};
                 const int one = cap;
-                if (plan_gemv_grouped(fmt, K, false, &nrows, &one, 1, &probe) == TFQ_OK) return cap;
+                if (plan_gemv_grouped(fmt, K, false, &nrows, &one, 1, &probe, pair) == TFQ_OK) return cap;
             }
             return 4;
         };
-        const int capA = chunk_cap(gate[0]->fmt, (int)D, x_dtype == TFQ_F32, (int)F);
-        const int capB = chunk_cap(down[0]->fmt, (int)F, mid_dtype == TFQ_F32, (int)D);
+        // gate and up of an expert are one problem: the kernel walks the same tiles of both and its epilogue writes
+        // silu(gate x) * (up x) in the mid dtype (ExpertFFN::forward, src/model/moe_core.cpp:78-92), so the two
+        // products never go to memory and no elementwise launch follows
+        const int capA = chunk_cap(gate[0]->fmt, (int)D, x_dtype == TFQ_F32, (int)F, true);
+        const int capB = chunk_cap(down[0]->fmt, (int)F, mid_dtype == TFQ_F32, (int)D, false);
         for (int e = 0; e < E; ++e) {
             const int p0 = first[e], nt = first[e + 1] - first[e];
             for (int b0 = 0; b0 < nt; b0 += capA) {
                 const int nb = std::min(capA, nt - b0);
-                for (int m = 0; m < 2; ++m) {
-                    wA.push_back(m ? up[e] : gate[e]);
-                    xA.push_back(ws.xe + (size_t)(p0 + b0) * D * xe_bytes);
-                    yA.push_back((m ? ws.u : ws.g) + (size_t)(p0 + b0) * F);
-                    nA.push_back((int)F);
-                    rA.push_back(nb);
-                }
+                wA.push_back(gate[e]);
+                wA2.push_back(up[e]);
+                xA.push_back(ws.xe + (size_t)(p0 + b0) * D * xe_bytes);
+                yA.push_back(ws.h + (size_t)(p0 + b0) * F * he);
+                nA.push_back((int)F);
+                rA.push_back(nb);
             }
             for (int b0 = 0; b0 < nt; b0 += capB) {
                 const int nb = std::min(capB, nt - b0);
@@ -374,7 +376,7 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
                 rB.push_back(nb);
             }
         }
-        if (int rc = plan_gemv_grouped(gate[0]->fmt, (int)D, x_dtype == TFQ_F32, nA.data(), rA.data(), (int)nA.size(), &planA)) return rc;
+        if (int rc = plan_gemv_grouped(gate[0]->fmt, (int)D, x_dtype == TFQ_F32, nA.data(), rA.data(), (int)nA.size(), &planA, true)) return rc;
         if (int rc = plan_gemv_grouped(down[0]->fmt, (int)F, mid_dtype == TFQ_F32, nB.data(), rB.data(), (int)nB.size(), &planB)) return rc;
     }
     const size_t eb = gemv_group_entry_bytes();
@@ -389,7 +391,7 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
     int* const lists = static_cast<int*>(slot->host);
     if (grouped) {
         uint8_t* lb = reinterpret_cast<uint8_t*>(lists);
-        fill_gemv_group(planA, wA.data(), xA.data(), yA.data(), rA.data(), (int)wA.size(), lb + tabA, reinterpret_cast<int*>(lb + mapA));
+        fill_gemv_group(planA, wA.data(), xA.data(), yA.data(), rA.data(), (int)wA.size(), lb + tabA, reinterpret_cast<int*>(lb + mapA), wA2.data());
         fill_gemv_group(planB, wB.data(), xB.data(), yB.data(), rB.data(), (int)wB.size(), lb + tabB, reinterpret_cast<int*>(lb + mapB));
     }
     int* h_rows = lists;
@@ -418,7 +420,7 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
     }
     const uint8_t* d_lists = reinterpret_cast<const uint8_t*>(ws.lists);
     if (grouped) {
-        if (int rc = launch_gemv_grouped(gate[0]->fmt, planA, d_lists + tabA, reinterpret_cast<const int*>(d_lists + mapA), TFQ_F32, s)) return rc;
+        if (int rc = launch_gemv_grouped(gate[0]->fmt, planA, d_lists + tabA, reinterpret_cast<const int*>(d_lists + mapA), mid_dtype, s)) return rc;
     }
     for (int e = 0; e < E && !grouped; ++e) {
         const int p0 = first[e], nt = first[e + 1] - first[e];
@@ -435,7 +437,7 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
         }
     }
     const int64_t nh = (int64_t)P * F;
-    if (P) {
+    if (P && !grouped) {
         if (mid_dtype == TFQ_BF16)
             hipLaunchKernelGGL(silu_mul_kernel<true>, dim3((unsigned)((nh + 255) / 256)), dim3(256), 0, s, ws.g, ws.u, (void*)ws.h, nh);
         else
