@@ -145,6 +145,30 @@ def test_moe_ffn_many_tokens_per_expert(O, tfq, gpu, fmt, xdt, mid_bf16, tol):
         W.close()
 
 
+@pytest.mark.parametrize("fmt", ["B32S4", "B32S8"])
+def test_moe_ffn_long_down_rows_five_to_sixteen(O, tfq, gpu, fmt):
+    """Experts with five to sixteen tokens and a down product too long for their staged rows (K = 5120: twenty
+    block columns, so some wavefronts of the sixteen-row kernel own two): bf16 mid activations take the grouped
+    sixteen-row launch, which reads every down matrix once; fp32 mid activations keep the two-row passes."""
+    import torch
+    E, Ktop, T, D, F = 4, 2, 18, 256, 5120
+    gate, up, down, hg, hu, hd = _experts(O, tfq, fmt, E, D, F, 900)
+    logits = O.rng_normal(48, T * E, 1.0).reshape(T, E)
+    logits[:, 3] -= 20.0  # three experts share the tokens: twelve each
+    _, idx, w = O.softmax_topk(logits, Ktop)
+    counts = [int((idx == e).sum()) for e in range(E)]
+    assert counts[3] == 0 and min(counts[:3]) > 4 and max(counts) <= 16, counts
+    x = O.bf16_round(O.rng_normal(49, T * D, 1.0).reshape(T, D))
+    ref = O.moe_ffn(fmt, hg, hu, hd, D, F, idx, w, x, mid_bf16=True)
+    y = tfq.moe_ffn(gate, up, down, idx, w, torch.from_numpy(x).to(gpu).bfloat16(), mid_dtype=torch.bfloat16).cpu().numpy()
+    assert rel_err(y, ref) <= 1e-2
+    ref32 = O.moe_ffn(fmt, hg, hu, hd, D, F, idx, w, x, mid_bf16=False)
+    y32 = tfq.moe_ffn(gate, up, down, idx, w, torch.from_numpy(x).to(gpu).bfloat16(), mid_dtype=torch.float32).cpu().numpy()
+    assert rel_err(y32, ref32) <= 1e-3
+    for wl in gate + up + down:
+        wl.close()
+
+
 def test_moe_single_token_equals_plain_mlp(O, tfq, gpu):
     """One token, one expert, weight 1: the MoE path reduces to the SwiGLU MLP step."""
     import torch

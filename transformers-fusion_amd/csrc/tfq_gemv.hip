@@ -572,20 +572,37 @@ __device__ __forceinline__ void transpose_rows(uint32_t (&v)[4]) {
 // or four unit fetches in flight, eight wavefronts of two columns, and fewer tiles per workgroup measured equal
 // or slower.
 constexpr int kGemvbKC = 16;  // block columns per K part
-template <int FMT, bool SPLIT>
-__global__ __launch_bounds__(1024) void gemvb_kernel(GemvKernArgs args, const unsigned short* __restrict__ x) {
+template <int FMT, bool SPLIT, bool GROUPED = false>
+__global__ __launch_bounds__(1024) void gemvb_kernel(GemvKernArgs args, const unsigned short* __restrict__ x_arg) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
     static_assert(F::GS == 32 && F::HV == 1, "32-weight groups and a 16-byte header");
+    static_assert(!(SPLIT && GROUPED), "a grouped launch has no K parts");
     constexpr int UB = tiled_unit_bytes(FMT), NC = 2 * F::NP, WD = 2;
-    const int K = args.K, T = args.tiles_per_wg, B = args.nslot;
+    const int K = args.K, T = args.tiles_per_wg;
     const bool y_bf16 = args.y_bf16 != 0;
     const int bid = blockIdx.x;
-    const int m = (bid >= args.g0) + (bid >= args.g1) + (bid >= args.g2);
-    const int wg_first = m == 0 ? 0 : m == 1 ? args.g0 : m == 2 ? args.g1 : args.g2;
-    const uint8_t* Wm = m == 0 ? args.W0 : m == 1 ? args.W1 : m == 2 ? args.W2 : args.W3;
-    void* ym = m == 0 ? args.y0 : m == 1 ? args.y1 : m == 2 ? args.y2 : args.y3;
-    const int nrm = m == 0 ? args.nr0 : m == 1 ? args.nr1 : m == 2 ? args.nr2 : args.nr3;
+    // this workgroup's matrix: selected with compares, or read from the problem table of a grouped launch
+    // (W0 = table of GemvProb, W1 = map workgroup -> problem; both reads are uniform)
+    int wg_first, nrm, B;
+    const uint8_t* Wm;
+    void* ym;
+    const unsigned short* x;
+    if constexpr (GROUPED) {
+        const GemvProb* table = reinterpret_cast<const GemvProb*>(args.W0);
+        const int* wg_map = reinterpret_cast<const int*>(args.W1);
+        const GemvProb pr = table[wg_map[bid]];
+        wg_first = pr.wg_first; nrm = pr.nrows; B = pr.nslot;
+        Wm = pr.W; ym = pr.y; x = static_cast<const unsigned short*>(pr.x);
+    } else {
+        const int m = (bid >= args.g0) + (bid >= args.g1) + (bid >= args.g2);
+        wg_first = m == 0 ? 0 : m == 1 ? args.g0 : m == 2 ? args.g1 : args.g2;
+        Wm = m == 0 ? args.W0 : m == 1 ? args.W1 : m == 2 ? args.W2 : args.W3;
+        ym = m == 0 ? args.y0 : m == 1 ? args.y1 : m == 2 ? args.y2 : args.y3;
+        nrm = m == 0 ? args.nr0 : m == 1 ? args.nr1 : m == 2 ? args.nr2 : args.nr3;
+        B = args.nslot;
+        x = x_arg;
+    }
 
     const int kparts = SPLIT ? args.kparts : 1;
     const int nblocks = K >> 8;
@@ -1163,6 +1180,71 @@ int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, 
 }
 
 }  // namespace
+
+// ---- grouped launch of gemvb_kernel: problems of up to sixteen bf16 activation rows at any K, each matrix read once
+namespace {
+template <int FMT>
+int plan_rows16_grouped(int K, const int* nrows, int nprob, GemvGroupPlan* gp) {
+    const int nblocks = K >> 8;
+    const int NW = nblocks < 16 ? nblocks : 16;
+    const int max_t = (int)((160 * 1024 - (size_t)NW * 2560) / ((size_t)NW * 1024));
+    // tiles per workgroup: the fewest rounds of 256 workgroups, counting a workgroup's start-up (its wavefronts'
+    // first A fragments) as two tiles' worth
+    int best_t = 1;
+    long best_cost = -1;
+    for (int T = max_t; T >= 1; --T) {
+        long wgs = 0;
+        for (int i = 0; i < nprob; ++i) wgs += ((nrows[i] + 15) / 16 + T - 1) / T;
+        const long cost = (wgs + 255) / 256 * (T + 2);
+        if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_t = T; }
+    }
+    gp->NW = NW; gp->T = best_t; gp->sets = 4; gp->K = K; gp->x_f32 = false; gp->pair = false;
+    gp->lds = (size_t)NW * 2560 + (size_t)best_t * NW * 1024;
+    int grid = 0;
+    for (int i = 0; i < nprob; ++i) grid += ((nrows[i] + 15) / 16 + best_t - 1) / best_t;
+    gp->grid = grid;
+    return TFQ_OK;
+}
+
+template <int FMT>
+int run_rows16_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_bf16, hipStream_t s) {
+    GemvKernArgs k{};
+    k.W0 = static_cast<const uint8_t*>(d_table);
+    k.W1 = reinterpret_cast<const uint8_t*>(d_map);
+    k.K = gp.K; k.y_bf16 = y_bf16; k.tiles_per_wg = gp.T;
+    k.kparts = 1; k.kcols = gp.K >> 8;
+    static std::atomic<bool> lds_limit_raised{false};
+    if (!lds_limit_raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemvb_kernel<FMT, false, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
+        lds_limit_raised = true;
+    }
+    hipLaunchKernelGGL((gemvb_kernel<FMT, false, true>), dim3(gp.grid), dim3(64 * gp.NW), gp.lds, s, k, nullptr);
+    return hip_fail(hipGetLastError(), "gemv group launch");
+}
+}  // namespace
+
+int plan_gemv_rows16_grouped(int fmt, int K, const int* nrows, int nprob, GemvGroupPlan* gp) {
+    if (nprob <= 0) return fail(TFQ_ERR_ARG, "gemv group: no problems");
+    switch (canonical(fmt)) {
+        case TFQ_Q_G_4: return plan_rows16_grouped<TFQ_Q_G_4>(K, nrows, nprob, gp);
+        case TFQ_B32S4: return plan_rows16_grouped<TFQ_B32S4>(K, nrows, nprob, gp);
+        case TFQ_B32S8: return plan_rows16_grouped<TFQ_B32S8>(K, nrows, nprob, gp);
+        case TFQ_Q_G_8: return plan_rows16_grouped<TFQ_Q_G_8>(K, nrows, nprob, gp);
+        default: return fail(TFQ_ERR_FORMAT, "gemv group: no sixteen-row kernel for this format");
+    }
+}
+
+int launch_gemv_rows16_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s) {
+    const int yb = y_dtype == TFQ_BF16;
+    switch (canonical(fmt)) {
+        case TFQ_Q_G_4: return run_rows16_grouped<TFQ_Q_G_4>(gp, d_table, d_map, yb, s);
+        case TFQ_B32S4: return run_rows16_grouped<TFQ_B32S4>(gp, d_table, d_map, yb, s);
+        case TFQ_B32S8: return run_rows16_grouped<TFQ_B32S8>(gp, d_table, d_map, yb, s);
+        case TFQ_Q_G_8: return run_rows16_grouped<TFQ_Q_G_8>(gp, d_table, d_map, yb, s);
+        default: return fail(TFQ_ERR_FORMAT, "gemv group: no sixteen-row kernel for this format");
+    }
+}
 
 // formats whose 5..16-row calls take gemvb_kernel (one pass over the weights per 16 rows)
 bool gemv_rows16_supported(int fmt) {

@@ -401,6 +401,9 @@ size_t gemv_group_entry_bytes();
 void fill_gemv_group(const GemvGroupPlan& gp, const tfq_weight* const* ws, const void* const* xs, void* const* ys,
                      const int* nrows_x, int nprob, void* table_host, int* map_host, const tfq_weight* const* ws2 = nullptr);
 int launch_gemv_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s);
+// the same for problems of up to sixteen bf16 activation rows at any K (gemvb_kernel; tables from fill_gemv_group)
+int plan_gemv_rows16_grouped(int fmt, int K, const int* nrows, int nprob, GemvGroupPlan* gp);
+int launch_gemv_rows16_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s);
 size_t moe_workspace_bytes(int T, int Ktop, int64_t D, int64_t F);
 size_t mlp_workspace_bytes(int B, int64_t F);
 int launch_mlp_step(const tfq_weight* gate, const tfq_weight* up, const tfq_weight* down, const void* x, int x_dtype, int B,

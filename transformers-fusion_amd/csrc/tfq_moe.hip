@@ -334,6 +334,7 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
     const bool grouped = P > 0 && !tall && gemv_grouped_supported(gate[0]->fmt) && gemv_grouped_supported(down[0]->fmt) &&
                          canonical(gate[0]->fmt) == canonical(up[0]->fmt);
     GemvGroupPlan planA{}, planB{};
+    bool down16 = false;  // the down stage through the sixteen-row kernel
     std::vector<const tfq_weight*> wA, wA2, wB;
     std::vector<const void*> xA, xB;
     std::vector<void*> yA, yB;
@@ -355,7 +356,12 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
         // silu(gate x) * (up x) in the mid dtype (ExpertFFN::forward, src/model/moe_core.cpp:78-92), so the two
         // products never go to memory and no elementwise launch follows
         const int capA = chunk_cap(gate[0]->fmt, (int)D, x_dtype == TFQ_F32, (int)F, true);
-        const int capB = chunk_cap(down[0]->fmt, (int)F, mid_dtype == TFQ_F32, (int)D, false);
+        int capB = chunk_cap(down[0]->fmt, (int)F, mid_dtype == TFQ_F32, (int)D, false);
+        // Down at a long K: the staged activations of more than four rows do not fit, and an expert with more
+        // tokens would read its matrix once per four.  With bf16 mid activations the sixteen-row kernel (A
+        // fragments in registers, any K) reads every matrix once instead.
+        down16 = mid_dtype == TFQ_BF16 && max_nt > capB && gemv_rows16_supported(down[0]->fmt);
+        if (down16) capB = 16;
         for (int e = 0; e < E; ++e) {
             const int p0 = first[e], nt = first[e + 1] - first[e];
             for (int b0 = 0; b0 < nt; b0 += capA) {
@@ -377,7 +383,11 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
             }
         }
         if (int rc = plan_gemv_grouped(gate[0]->fmt, (int)D, x_dtype == TFQ_F32, nA.data(), rA.data(), (int)nA.size(), &planA, true)) return rc;
-        if (int rc = plan_gemv_grouped(down[0]->fmt, (int)F, mid_dtype == TFQ_F32, nB.data(), rB.data(), (int)nB.size(), &planB)) return rc;
+        if (down16) {
+            if (int rc = plan_gemv_rows16_grouped(down[0]->fmt, (int)F, nB.data(), (int)nB.size(), &planB)) return rc;
+        } else if (int rc = plan_gemv_grouped(down[0]->fmt, (int)F, mid_dtype == TFQ_F32, nB.data(), rB.data(), (int)nB.size(), &planB)) {
+            return rc;
+        }
     }
     const size_t eb = gemv_group_entry_bytes();
     const size_t base_ints = ((size_t)3 * P + T + 1 + 1) & ~(size_t)1;  // tables start 8-byte aligned
@@ -444,7 +454,11 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
             hipLaunchKernelGGL(silu_mul_kernel<false>, dim3((unsigned)((nh + 255) / 256)), dim3(256), 0, s, ws.g, ws.u, (void*)ws.h, nh);
     }
     if (grouped) {
-        if (int rc = launch_gemv_grouped(down[0]->fmt, planB, d_lists + tabB, reinterpret_cast<const int*>(d_lists + mapB), TFQ_F32, s)) return rc;
+        if (down16) {
+            if (int rc = launch_gemv_rows16_grouped(down[0]->fmt, planB, d_lists + tabB, reinterpret_cast<const int*>(d_lists + mapB), TFQ_F32, s)) return rc;
+        } else if (int rc = launch_gemv_grouped(down[0]->fmt, planB, d_lists + tabB, reinterpret_cast<const int*>(d_lists + mapB), TFQ_F32, s)) {
+            return rc;
+        }
     }
     for (int e = 0; e < E && !grouped; ++e) {
         const int p0 = first[e], nt = first[e + 1] - first[e];
