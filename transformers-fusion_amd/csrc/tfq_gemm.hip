@@ -72,14 +72,22 @@ __device__ __forceinline__ float ubyte_to_float(uint32_t v) {
     return f;
 }
 
-// one code dword (nibble t = weight t) -> eight bf16 weights in k order: 3 + 8 + 8 + 4 operations
-__device__ __forceinline__ uint4 decode8(uint32_t v, float a, float c) {
-    const uint32_t ev = v & 0x0F0F0F0Fu, od = (v >> 4) & 0x0F0F0F0Fu;  // nibbles 0,2,4,6 / 1,3,5,7 as bytes
+// one code dword (nibble t = weight t) -> eight bf16 weights in k order: 7 + 8 + 4 operations.
+// (v >> 4 t) & 0x000F000F | 0x64006400 is the pair of binary16 numbers 1024 + n_t, 1024 + n_(t+4), exactly; the
+// multiply-add reads either half as binary16 (v_fma_mix_f32) and takes c - 1024 a as its addend.  For the
+// symmetric formats (a binary16 scale, c = -8 a or -128 a) that addend is exact in fp32 and a n + c is rounded
+// once, to the same bits as a (float) n + c; for the affine formats it carries one rounding of its own, 2^-14
+// of a, far below the bf16 rounding of the weight that follows.
+// (M = 0x000F000F and C = 0x64006400 come in registers, so that (x & M) | C is one v_and_or_b32.)
+__device__ __forceinline__ uint4 decode8(uint32_t v, float a, float c, uint32_t M, uint32_t C) {
+    const float c2 = __builtin_fmaf(-1024.0f, a, c);
+    const f16x2_t p0 = __builtin_bit_cast(f16x2_t, (v & M) | C), p1 = __builtin_bit_cast(f16x2_t, ((v >> 4) & M) | C);
+    const f16x2_t p2 = __builtin_bit_cast(f16x2_t, ((v >> 8) & M) | C), p3 = __builtin_bit_cast(f16x2_t, ((v >> 12) & M) | C);
     uint4 o;
-    o.x = pack_bf16(__builtin_fmaf(a, ubyte_to_float<0>(ev), c), __builtin_fmaf(a, ubyte_to_float<0>(od), c));
-    o.y = pack_bf16(__builtin_fmaf(a, ubyte_to_float<1>(ev), c), __builtin_fmaf(a, ubyte_to_float<1>(od), c));
-    o.z = pack_bf16(__builtin_fmaf(a, ubyte_to_float<2>(ev), c), __builtin_fmaf(a, ubyte_to_float<2>(od), c));
-    o.w = pack_bf16(__builtin_fmaf(a, ubyte_to_float<3>(ev), c), __builtin_fmaf(a, ubyte_to_float<3>(od), c));
+    o.x = pack_bf16(__builtin_fmaf(a, (float)p0.x, c2), __builtin_fmaf(a, (float)p1.x, c2));
+    o.y = pack_bf16(__builtin_fmaf(a, (float)p2.x, c2), __builtin_fmaf(a, (float)p3.x, c2));
+    o.z = pack_bf16(__builtin_fmaf(a, (float)p0.y, c2), __builtin_fmaf(a, (float)p1.y, c2));
+    o.w = pack_bf16(__builtin_fmaf(a, (float)p2.y, c2), __builtin_fmaf(a, (float)p3.y, c2));
     return o;
 }
 
@@ -271,13 +279,15 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
             }
         }
     };
+    uint32_t nib_mask = 0x000F000Fu, f16_bias = 0x64006400u;
+    asm volatile("" : "+v"(nib_mask), "+v"(f16_bias));  // kept in registers (see decode8)
     auto store_step = [&]<int G, int R>(int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < WROWS; ++i) {
             if constexpr (G == 0) hdr[i] = uint4{hnext[i][0], hnext[i][1], hnext[i][2], hnext[i][3]};
             float a, c;
             group_coeffs<FMT>(hdr[i], G, a, c);
-            if constexpr (NP == 1) wsm[buf * BNA * 4 + lds_index(wr + i * RSTRIDE, wj)] = decode8(rw[i][0][R], a, c);
+            if constexpr (NP == 1) wsm[buf * BNA * 4 + lds_index(wr + i * RSTRIDE, wj)] = decode8(rw[i][0][R], a, c, nib_mask, f16_bias);
             else wsm[buf * BNA * 4 + lds_index(wr + i * RSTRIDE, wj)] = decode8x2(rw[i][0][R], rw[i][NP - 1][R], a, c);
         }
     };
