@@ -394,10 +394,37 @@ def moe_layer(tfq, torch, fmt, bpw, base, E=8, top_k=2, T=16, D=4096, F=14336, r
     dt = (time.perf_counter() - t0) / reps
     active = len(set(idx_h.reshape(-1).tolist()))
     nbytes = active * 3 * F * D * bpw / 8
-    return {"tokens": T, "experts": E, "top_k": top_k, "active_experts": active,
-            "tokens_per_expert": [int((idx_h == e).sum()) for e in range(E)],
-            "us_per_call": round(dt * 1e6, 1), "gbs": round(nbytes / dt / 1e9, 1),
-            "frac": round(nbytes / dt / 1e9 / HBM_PEAK_GBS, 4), "bound": "hbm"}
+    out = {"tokens": T, "experts": E, "top_k": top_k, "active_experts": active,
+           "tokens_per_expert": [int((idx_h == e).sum()) for e in range(E)],
+           "us_per_call": round(dt * 1e6, 1), "gbs": round(nbytes / dt / 1e9, 1),
+           "frac": round(nbytes / dt / 1e9 / HBM_PEAK_GBS, 4), "bound": "hbm"}
+    # the same call with the routing arrays left on the device (lists and launch tables built there), as graph replays
+    routed = tfq.RoutedMoe(gate, up, down, T, top_k)
+    y = torch.empty(T, D, device="cuda")
+    for _ in range(3):
+        routed(idx, wts, x, y)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        routed(idx, wts, x, y)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        routed(idx, wts, x, y)
+    for _ in range(3):
+        g.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        g.replay()
+    torch.cuda.synchronize()
+    dtr = (time.perf_counter() - t0) / reps
+    out["routed_on_device"] = {"us_per_call": round(dtr * 1e6, 1), "gbs": round(nbytes / dtr / 1e9, 1),
+                               "frac": round(nbytes / dtr / 1e9 / HBM_PEAK_GBS, 4),
+                               "note": "routing arrays on the device, lists built there, graph replays"}
+    return out
 
 
 def usable_cores():

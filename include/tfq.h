@@ -411,6 +411,26 @@ int tfq_moe_ffn(const tfq_weight_t* const* gate, const tfq_weight_t* const* up,
                 int T, int k, const void* x, int x_dtype, void* y, int y_dtype, int mid_dtype,
                 void* workspace, size_t workspace_bytes, tfq_stream_t stream);
 
+/* tfq_moe_ffn with the routing arrays on the device, as tfq_moe_route / tfq_moe_router leave them (topk_idx
+ * int32 [T][k], topk_w [T][k], device pointers): nothing is read back to the host, the per-expert lists are built
+ * on the device (count, scan, ordered scatter: the same expert-major, ascending-token order), and every launch has
+ * a grid that follows from (T, k, E) alone, so the call can be captured into a graph and replayed with other
+ * routing.  Same results as tfq_moe_ffn to rounding (the rows of an expert may be cut into passes differently).
+ * bf16 x and bf16 mid activations, experts of one tiled format per stage that has the grouped kernels (Q_G_4,
+ * B32S4, B32S8, Q_G_8), T * k <= 1024, E <= 256; anything else is refused (use tfq_moe_ffn).
+ *   tfq_moe_expert_table           writes the experts' device addresses to expert_table (device memory of
+ *                                  3 * E * 8 bytes), once per set of experts (a synchronous copy)
+ *   tfq_moe_routed_workspace_bytes the workspace the call needs (0: this configuration is refused) */
+int tfq_moe_expert_table(const tfq_weight_t* const* gate, const tfq_weight_t* const* up,
+                         const tfq_weight_t* const* down, int E, void* expert_table);
+size_t tfq_moe_routed_workspace_bytes(const tfq_weight_t* const* gate, const tfq_weight_t* const* up,
+                                      const tfq_weight_t* const* down, int E, int T, int k);
+int tfq_moe_ffn_routed(const tfq_weight_t* const* gate, const tfq_weight_t* const* up,
+                       const tfq_weight_t* const* down, int E, const void* expert_table,
+                       const int32_t* topk_idx, const float* topk_w, int T, int k, const void* x, int x_dtype,
+                       void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes,
+                       tfq_stream_t stream);
+
 /* Capacity-limited dispatch, moe_engine::plan_dispatch / gather_expert_inputs / combine_expert_outputs
  * (engines/trainer/moe/dispatch.cpp:9-78): the slots (t, j) are walked in token order, j inside; a slot joins
  * the list of its expert while that list has fewer than slots_per_expert items and is dropped otherwise; an

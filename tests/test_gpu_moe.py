@@ -169,6 +169,77 @@ def test_moe_ffn_long_down_rows_five_to_sixteen(O, tfq, gpu, fmt):
         wl.close()
 
 
+@pytest.mark.parametrize("fmt", ["B32S4", "Q_G_8"])
+def test_moe_ffn_routed_builds_its_lists_on_the_device(O, tfq, gpu, fmt):
+    """tfq_moe_ffn_routed: routing arrays stay on the device, lists and launch tables are built there.  Skewed
+    routing (an expert with more rows than one pass, an expert with none, a slot whose id is out of range) against
+    the oracle and against tfq_moe_ffn with the same routing on the host."""
+    import torch
+    E, Ktop, T, D, F = 6, 2, 24, 512, 1024
+    gate, up, down, hg, hu, hd = _experts(O, tfq, fmt, E, D, F, 800)
+    logits = O.rng_normal(50, T * E, 1.0).reshape(T, E)
+    logits[:, 2] += 6.0      # every token picks expert 2 first: 24 rows, three passes of eight
+    logits[:, 4] -= 20.0     # nobody picks expert 4
+    _, idx, w = O.softmax_topk(logits, Ktop)
+    idx = idx.copy()
+    idx[5, 1] = E + 3        # an id outside 0..E-1: the slot is skipped
+    x = O.bf16_round(O.rng_normal(51, T * D, 1.0).reshape(T, D))
+    ref = O.moe_ffn(fmt, hg, hu, hd, D, F, idx, w, x, mid_bf16=True)
+    xt = torch.from_numpy(x).to(gpu).bfloat16()
+    host = tfq.moe_ffn(gate, up, down, idx, w, xt, mid_dtype=torch.bfloat16)
+    routed = tfq.RoutedMoe(gate, up, down, T, Ktop)
+    y = torch.empty(T, D, device=gpu)
+    routed(torch.from_numpy(idx.astype(np.int32)).to(gpu), torch.from_numpy(w.astype(np.float32)).to(gpu), xt, y)
+    assert rel_err(y.cpu().numpy(), ref) <= 1e-2
+    assert float((y - host).abs().max()) <= 1e-5 * float(host.abs().max())
+    for wl in gate + up + down:
+        wl.close()
+
+
+def test_moe_ffn_routed_in_a_graph(O, tfq, gpu):
+    """The routed call captured into a graph together with the router: replays with other activations (hence other
+    routing) equal the eager calls bit for bit, with eager work and synchronizations between the replays."""
+    import torch
+    fmt, E, Ktop, T, D, F = "B32S4", 8, 2, 16, 512, 1536
+    gate, up, down, _, _, _ = _experts(O, tfq, fmt, E, D, F, 820)
+    Wr = torch.from_numpy(O.rng_normal(52, E * D, 0.05).reshape(E, D).astype(np.float32)).to(gpu)
+    routed = tfq.RoutedMoe(gate, up, down, T, Ktop)
+    xs = [torch.from_numpy(O.rng_normal(60 + i, T * D, 1.0).reshape(T, D).astype(np.float32)).to(gpu).bfloat16() for i in range(4)]
+    x = xs[0].clone()
+    y = torch.zeros(T, D, device=gpu)
+
+    def step():
+        _, _, idx, wts = tfq.moe_router(x, Wr, Ktop)
+        routed(idx, wts, x, y)
+        return idx
+
+    step()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step()
+    seen = set()
+    for i in (1, 2, 3, 0, 2):
+        x.copy_(xs[i])
+        g.replay()
+        torch.cuda.synchronize()
+        got = y.clone()
+        y.zero_()
+        idx = step()
+        torch.cuda.synchronize()
+        seen.add(tuple(idx.cpu().numpy().reshape(-1).tolist()))
+        assert torch.equal(got, y), i
+    assert len(seen) >= 3  # the replays really saw different routing
+    for wl in gate + up + down:
+        wl.close()
+
+
 def test_moe_single_token_equals_plain_mlp(O, tfq, gpu):
     """One token, one expert, weight 1: the MoE path reduces to the SwiGLU MLP step."""
     import torch

@@ -82,6 +82,9 @@ def _load():
         "tfq_moe_route": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "tfq_moe_workspace_bytes": (sz, [i32, i32, i64, i64]),
         "tfq_moe_ffn": (i32, [vp, vp, vp, i32, vp, vp, i32, i32, vp, i32, vp, i32, i32, vp, sz, vp]),
+        "tfq_moe_expert_table": (i32, [vp, vp, vp, i32, vp]),
+        "tfq_moe_routed_workspace_bytes": (sz, [vp, vp, vp, i32, i32, i32]),
+        "tfq_moe_ffn_routed": (i32, [vp, vp, vp, i32, vp, vp, vp, i32, i32, vp, i32, vp, i32, i32, vp, sz, vp]),
         "tfq_moe_plan_dispatch": (i32, [vp, vp, i32, i32, i32, i64, vp, vp, vp, vp, vp]),
         "tfq_moe_ffn_capacity": (i32, [vp, vp, vp, i32, vp, vp, i32, i32, i64, vp, i32, vp, i32, i32, vp, sz, vp, vp]),
         "tfq_lut4_gemm": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
@@ -587,6 +590,33 @@ def moe_ffn(gate, up, down, topk_idx, topk_w, x, out_dtype=None, mid_dtype=None)
                              x.data_ptr(), _dtype_code(x), y.data_ptr(), _dtype_code(y), mid,
                              ws.data_ptr(), nbytes, _stream()))
     return y
+
+
+class RoutedMoe:
+    """tfq_moe_ffn_routed for one set of experts and one call shape: the experts' address table and the workspace
+    are made once, so a call allocates nothing and can be captured into a graph.  idx (int32) and weights are device
+    tensors [T][k] as moe_route returns them."""
+
+    def __init__(self, gate, up, down, T: int, k: int, device="cuda"):
+        import torch
+        self.E = len(gate)
+        self.gate, self.up, self.down = list(gate), list(up), list(down)
+        self.T, self.k, self.D, self.F = T, k, gate[0].K, gate[0].N
+        arr = lambda ws_: (C.c_void_p * self.E)(*[w.handle for w in ws_])
+        self._g, self._u, self._d = arr(gate), arr(up), arr(down)
+        self.table = torch.empty(3 * self.E * 8, dtype=torch.uint8, device=device)
+        _check(lib().tfq_moe_expert_table(self._g, self._u, self._d, self.E, self.table.data_ptr()))
+        self.nbytes = int(lib().tfq_moe_routed_workspace_bytes(self._g, self._u, self._d, self.E, T, k))
+        if self.nbytes == 0:
+            raise TfqError("tfq_moe_ffn_routed does not take this configuration")
+        self.ws = torch.empty(self.nbytes, dtype=torch.uint8, device=device)
+
+    def __call__(self, idx, wts, x, y):
+        assert idx.is_cuda and wts.is_cuda and idx.dtype.itemsize == 4 and x.is_contiguous() and y.is_contiguous()
+        _check(lib().tfq_moe_ffn_routed(self._g, self._u, self._d, self.E, self.table.data_ptr(), idx.data_ptr(), wts.data_ptr(),
+                                        self.T, self.k, x.data_ptr(), _dtype_code(x), y.data_ptr(), _dtype_code(y), BF16,
+                                        self.ws.data_ptr(), self.nbytes, _stream()))
+        return y
 
 
 def moe_plan_dispatch(topk_idx, topk_w, E: int, slots_per_expert: int):

@@ -467,6 +467,39 @@ int tfq_moe_ffn(const tfq_weight_t* const* gate, const tfq_weight_t* const* up, 
                           workspace_bytes, (hipStream_t)stream);
 }
 
+int tfq_moe_expert_table(const tfq_weight_t* const* gate, const tfq_weight_t* const* up, const tfq_weight_t* const* down, int E,
+                         void* expert_table) {
+    if (!gate || !up || !down || !expert_table || E <= 0) return fail(TFQ_ERR_ARG, "tfq_moe_expert_table: null pointer or no experts");
+    for (int e = 0; e < E; ++e)
+        if (!gate[e] || !up[e] || !down[e]) return fail(TFQ_ERR_ARG, "tfq_moe_expert_table: null expert handle");
+    if (int r = ensure_device()) return r;
+    return moe_expert_table(gate, up, down, E, expert_table);
+}
+
+size_t tfq_moe_routed_workspace_bytes(const tfq_weight_t* const* gate, const tfq_weight_t* const* up, const tfq_weight_t* const* down,
+                                      int E, int T, int k) {
+    if (!gate || !up || !down || E <= 0 || T <= 0 || k <= 0) return 0;
+    for (int e = 0; e < E; ++e)
+        if (!gate[e] || !up[e] || !down[e]) return 0;
+    return moe_routed_workspace_bytes(gate, up, down, E, T, k);
+}
+
+int tfq_moe_ffn_routed(const tfq_weight_t* const* gate, const tfq_weight_t* const* up, const tfq_weight_t* const* down, int E,
+                       const void* expert_table, const int32_t* topk_idx, const float* topk_w, int T, int k, const void* x,
+                       int x_dtype, void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes,
+                       tfq_stream_t stream) {
+    if (!gate || !up || !down || !expert_table || !topk_idx || !topk_w || !x || !y || !workspace)
+        return fail(TFQ_ERR_ARG, "tfq_moe_ffn_routed: null pointer");
+    if (E <= 0 || T <= 0 || k <= 0) return fail(TFQ_ERR_ARG, "tfq_moe_ffn_routed: E, T and k must be positive");
+    if (y_dtype != TFQ_F32 && y_dtype != TFQ_BF16) return fail(TFQ_ERR_ARG, "tfq_moe_ffn_routed: y dtype must be TFQ_F32 or TFQ_BF16");
+    for (int e = 0; e < E; ++e)
+        if (!gate[e] || !up[e] || !down[e]) return fail(TFQ_ERR_ARG, "tfq_moe_ffn_routed: null expert handle");
+    if ((uintptr_t)x % 16 || (uintptr_t)workspace % 256) return fail(TFQ_ERR_ARG, "tfq_moe_ffn_routed: x must be 16-byte, workspace 256-byte aligned");
+    if (int r = ensure_device()) return r;
+    return launch_moe_ffn_routed(gate, up, down, E, expert_table, topk_idx, topk_w, T, k, x, x_dtype, y, y_dtype, mid_dtype, workspace,
+                                 workspace_bytes, (hipStream_t)stream);
+}
+
 int tfq_moe_plan_dispatch(const int32_t* topk_idx, const float* topk_w, int T, int k, int E, int64_t slots_per_expert,
                           int32_t* expert_first, int32_t* item_token, float* item_weight, int32_t* dropped_slot,
                           int64_t* dropped) {

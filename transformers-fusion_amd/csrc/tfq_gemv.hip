@@ -99,21 +99,6 @@ struct GemvKernArgs {
     int accumulate;
 };
 
-// Grouped launch: many independent problems (matrix, activation rows, output) of one format and
-// K in one grid, e.g. all experts of a mixture layer.  The kernel then receives a device table of
-// problems and a map workgroup -> problem instead of the flattened arguments (W0 = table,
-// W1 = map); both reads are uniform per workgroup.
-struct GemvProb {
-    const uint8_t* W;
-    void* y;
-    const void* x;
-    const uint8_t* W2;  // paired plan: the up matrix (W is gate)
-    int nrows;
-    int nslot;
-    int wg_first;  // first workgroup of this problem
-    int pad;
-};
-
 // WD = unit fetches in flight per wavefront; the first WD are requested unconditionally, so the host
 // chooses WD <= the number of units of a full wavefront (a short one re-reads a unit it never uses).
 // SETS = sets of four activation slots that ride in one pass (1, 2 or 4: up to 16 bf16 rows).  More
@@ -157,7 +142,9 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     if constexpr (GROUPED) {
         const GemvProb* table = reinterpret_cast<const GemvProb*>(args.W0);
         const int* wg_map = reinterpret_cast<const int*>(args.W1);
-        const GemvProb pr = table[wg_map[bid]];
+        const int prob = wg_map[bid];
+        if (prob < 0) return;  // a workgroup beyond the problems of this call (tables built on the device)
+        const GemvProb pr = table[prob];
         wg_first = pr.wg_first; nrm = pr.nrows; nslot = pr.nslot;
         Wm = pr.W; ym = pr.y; xin = pr.x;
         Wm2 = pr.W2;
@@ -591,7 +578,9 @@ __global__ __launch_bounds__(1024) void gemvb_kernel(GemvKernArgs args, const un
     if constexpr (GROUPED) {
         const GemvProb* table = reinterpret_cast<const GemvProb*>(args.W0);
         const int* wg_map = reinterpret_cast<const int*>(args.W1);
-        const GemvProb pr = table[wg_map[bid]];
+        const int prob = wg_map[bid];
+        if (prob < 0) return;  // a workgroup beyond the problems of this call (tables built on the device)
+        const GemvProb pr = table[prob];
         wg_first = pr.wg_first; nrm = pr.nrows; B = pr.nslot;
         Wm = pr.W; ym = pr.y; x = static_cast<const unsigned short*>(pr.x);
     } else {

@@ -384,6 +384,21 @@ int launch_decode_mixed(const tfq_weight* w, float* out, hipStream_t s);
 // Grouped GEMV: many (matrix, activation rows, output) problems of one format and K in one launch.
 // plan -> fill the host images of the problem table and the workgroup map -> copy both to the
 // device -> launch.  nrows[i] = weight rows of problem i, nrows_x[i] = its activation rows.
+// Grouped launch: many independent problems (matrix, activation rows, output) of one format and
+// K in one grid, e.g. all experts of a mixture layer.  The kernel then receives a device table of
+// problems and a map workgroup -> problem instead of the flattened arguments (W0 = table,
+// W1 = map); both reads are uniform per workgroup.
+struct GemvProb {
+    const uint8_t* W;
+    void* y;
+    const void* x;
+    const uint8_t* W2;  // paired plan: the up matrix (W is gate)
+    int nrows;
+    int nslot;
+    int wg_first;  // first workgroup of this problem
+    int pad;
+};
+
 struct GemvGroupPlan {
     int NW, T, sets, grid, K;
     bool x_f32;
@@ -405,6 +420,13 @@ int launch_gemv_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, c
 int plan_gemv_rows16_grouped(int fmt, int K, const int* nrows, int nprob, GemvGroupPlan* gp);
 int launch_gemv_rows16_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s);
 size_t moe_workspace_bytes(int T, int Ktop, int64_t D, int64_t F);
+// the same call with the routing arrays on the device (see tfq_moe.hip)
+size_t moe_routed_workspace_bytes(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E, int T, int Ktop);
+int moe_expert_table(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E, void* d_table);
+int launch_moe_ffn_routed(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E,
+                          const void* d_expert_table, const int32_t* d_topk_idx, const float* d_topk_w, int T, int Ktop,
+                          const void* x, int x_dtype, void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes,
+                          hipStream_t s);
 size_t mlp_workspace_bytes(int B, int64_t F);
 int launch_mlp_step(const tfq_weight* gate, const tfq_weight* up, const tfq_weight* down, const void* x, int x_dtype, int B,
                     void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes, hipStream_t s);

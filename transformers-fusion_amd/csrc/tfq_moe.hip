@@ -474,6 +474,236 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
 }
 }  // namespace
 
+// ---- the same call with the routing arrays on the device (tfq_moe_route's outputs): nothing is read back, the
+// lists and the tables of the grouped launches are built by a small kernel, and every launch has a grid the
+// host fixes from (T, k, E) alone, so the call can be captured into a graph.  Workgroups beyond the problems a
+// call turns out to have find -1 in their map and leave.  (Lists and tables come from one kernel of one workgroup.)
+namespace {
+constexpr int kRoutedMaxPairs = 1024;  // T * k of a routed call (one workgroup builds the lists in LDS)
+
+struct RoutedShape {
+    int E, T, Ktop;
+    int capA, capB;      // activation rows per problem of the gate / up and of the down launch
+    int wgA, wgB;        // workgroups per problem
+    int maxA, maxB;      // problems at most
+    int nrowsA, nrowsB;  // F, D
+    size_t strideXA, strideYA, strideXB, strideYB;  // bytes per activation row in the gathered / mid / output buffers
+};
+
+// Lists of a call, by one workgroup.  Pairs are the slots (t, j) whose expert id is inside 0..E-1, expert-major,
+// ascending (t, j) inside an expert (moe_dispatch_batched, src/model/moe_core.cpp:289-343); the weight of a pair
+// is that of the first slot of its token that names the expert.
+//   first[E + 1], rows[P] (token of a pair; 0 behind the last pair), wts[P + 1] (wts[P] = 0: the pair a slot
+//   without an expert points at), tok_first[T + 1] = t * Ktop, tok_pairs[T * Ktop] (ascending per token)
+__global__ __launch_bounds__(1024) void routed_lists_kernel(const int32_t* __restrict__ idx, const float* __restrict__ w, int T, int Ktop, int E,
+                                                            int* __restrict__ first, int* __restrict__ rows, float* __restrict__ wts,
+                                                            int* __restrict__ tok_first, int* __restrict__ tok_pairs,
+                                                            RoutedShape sh, const uint8_t* const* __restrict__ ptrs, const uint8_t* xe, uint8_t* h, uint8_t* o,
+                                                            GemvProb* __restrict__ tabA, int* __restrict__ mapA,
+                                                            GemvProb* __restrict__ tabB, int* __restrict__ mapB) {
+    __shared__ int s_idx[kRoutedMaxPairs];
+    __shared__ int s_first[257];
+    __shared__ int s_cnt[256];
+    __shared__ int s_pair[kRoutedMaxPairs];
+    const int P = T * Ktop, tid = threadIdx.x;
+    for (int e = tid; e < E; e += blockDim.x) s_cnt[e] = 0;
+    for (int sl = tid; sl < P; sl += blockDim.x) {
+        const int e = idx[sl];
+        s_idx[sl] = e >= 0 && e < E ? e : -1;
+    }
+    __syncthreads();
+    // rank of a slot among the slots of its expert, in slot order
+    for (int sl = tid; sl < P; sl += blockDim.x) {
+        const int e = s_idx[sl];
+        int rank = 0;
+        if (e >= 0) {
+            for (int q = 0; q < sl; ++q) rank += s_idx[q] == e;
+            atomicAdd(&s_cnt[e], 1);
+        }
+        s_pair[sl] = rank;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int acc = 0;
+        for (int e = 0; e < E; ++e) { s_first[e] = acc; acc += s_cnt[e]; }
+        s_first[E] = acc;
+    }
+    __syncthreads();
+    for (int e = tid; e <= E; e += blockDim.x) first[e] = s_first[e];
+    const int total = s_first[E];
+    for (int p = total + tid; p < P; p += blockDim.x) rows[p] = 0;
+    if (tid == 0) wts[P] = 0.0f;
+    for (int sl = tid; sl < P; sl += blockDim.x) {
+        const int e = s_idx[sl];
+        if (e < 0) { s_pair[sl] = P; continue; }
+        const int p = s_first[e] + s_pair[sl];
+        const int t = sl / Ktop;
+        float wt = 0.0f;
+        for (int j = 0; j < Ktop; ++j)
+            if (s_idx[t * Ktop + j] == e) { wt = w[t * Ktop + j]; break; }
+        rows[p] = t;
+        wts[p] = wt;
+        s_pair[sl] = p;
+    }
+    __syncthreads();
+    for (int t = tid; t <= T; t += blockDim.x) tok_first[t] = t * Ktop;
+    for (int t = tid; t < T; t += blockDim.x) {  // the pairs of a token in ascending order (selection, Ktop is small)
+        int prev = -1;
+        for (int j = 0; j < Ktop; ++j) {
+            int best = 0x7FFFFFFF;
+            for (int q = 0; q < Ktop; ++q) {
+                const int p = s_pair[t * Ktop + q];
+                if (p > prev && p < best) best = p;
+            }
+            // equal pair indices cannot occur among real pairs; slots without an expert all point at P
+            tok_pairs[t * Ktop + j] = best == 0x7FFFFFFF ? P : best;
+            if (best != 0x7FFFFFFF && best != P) prev = best; else prev = P;
+        }
+    }
+    // Problem tables and workgroup maps of the two grouped launches: an expert's rows in chunks of capA / capB.
+    // ptrs = device addresses of the experts' packed matrices, [gate | up | down][E].
+    __shared__ int s_nA, s_nB;
+    if (tid == 0) {
+        int nA = 0, nB = 0;
+        for (int e = 0; e < E; ++e) {
+            const int p0 = s_first[e], nt = s_first[e + 1] - p0;
+            for (int b0 = 0; b0 < nt; b0 += sh.capA) {
+                const int nb = min(sh.capA, nt - b0);
+                tabA[nA] = GemvProb{ptrs[e], h + (size_t)(p0 + b0) * sh.strideYA, xe + (size_t)(p0 + b0) * sh.strideXA, ptrs[E + e],
+                                    sh.nrowsA, nb, nA * sh.wgA, 0};
+                ++nA;
+            }
+            for (int b0 = 0; b0 < nt; b0 += sh.capB) {
+                const int nb = min(sh.capB, nt - b0);
+                tabB[nB] = GemvProb{ptrs[2 * E + e], o + (size_t)(p0 + b0) * sh.strideYB, h + (size_t)(p0 + b0) * sh.strideXB, nullptr,
+                                    sh.nrowsB, nb, nB * sh.wgB, 0};
+                ++nB;
+            }
+        }
+        s_nA = nA;
+        s_nB = nB;
+    }
+    __syncthreads();
+    const int nA = s_nA, nB = s_nB;
+    for (int i = tid; i < sh.maxA * sh.wgA; i += blockDim.x) mapA[i] = i / sh.wgA < nA ? i / sh.wgA : -1;
+    for (int i = tid; i < sh.maxB * sh.wgB; i += blockDim.x) mapB[i] = i / sh.wgB < nB ? i / sh.wgB : -1;
+}
+
+struct RoutedPlan {
+    RoutedShape sh;
+    GemvGroupPlan planA, planB;
+    size_t off_first, off_rows, off_wts, off_tokf, off_tokp, off_tabA, off_tabB, off_mapA, off_mapB, list_bytes;
+};
+
+int plan_routed(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E, int T, int Ktop,
+                int x_dtype, int mid_dtype, RoutedPlan* rp) {
+    const int64_t D = gate[0]->K, F = gate[0]->N;
+    const long P = (long)T * Ktop;
+    if (P > kRoutedMaxPairs || E > 256) return fail(TFQ_ERR_SHAPE, "moe routed: at most 1024 (token, slot) pairs and 256 experts; larger calls take tfq_moe_ffn");
+    if (x_dtype != TFQ_BF16 || mid_dtype != TFQ_BF16) return fail(TFQ_ERR_ARG, "moe routed: bf16 activations and bf16 mid activations");
+    for (int e = 0; e < E; ++e) {
+        if (gate[e]->K != D || gate[e]->N != F || up[e]->K != D || up[e]->N != F || down[e]->K != F || down[e]->N != D)
+            return fail(TFQ_ERR_SHAPE, "moe: expert shapes must be gate/up F x D and down D x F");
+        if (canonical(gate[e]->fmt) != canonical(gate[0]->fmt) || canonical(up[e]->fmt) != canonical(gate[0]->fmt) ||
+            canonical(down[e]->fmt) != canonical(down[0]->fmt) || gate[e]->layout != TFQ_LAYOUT_TILED16 || up[e]->layout != TFQ_LAYOUT_TILED16 ||
+            down[e]->layout != TFQ_LAYOUT_TILED16)
+            return fail(TFQ_ERR_FORMAT, "moe routed: every expert in one tiled format per stage");
+    }
+    if (!gemv_grouped_supported(gate[0]->fmt) || !gemv_rows16_supported(down[0]->fmt))
+        return fail(TFQ_ERR_FORMAT, "moe routed: no grouped kernels for this format; use tfq_moe_ffn");
+    RoutedShape& sh = rp->sh;
+    sh = RoutedShape{};
+    sh.E = E; sh.T = T; sh.Ktop = Ktop;
+    sh.nrowsA = (int)F; sh.nrowsB = (int)D;
+    // gate / up: the paired eight-row form where its staged rows fit, else four rows; down: sixteen rows at any K
+    sh.capA = 8;
+    const int nrA = (int)F, nrB = (int)D;
+    if (plan_gemv_grouped(gate[0]->fmt, (int)D, false, &nrA, &sh.capA, 1, &rp->planA, true) != TFQ_OK) {
+        sh.capA = 4;
+        if (int rc = plan_gemv_grouped(gate[0]->fmt, (int)D, false, &nrA, &sh.capA, 1, &rp->planA, true)) return rc;
+    }
+    sh.capB = 16;
+    {   // tiles per workgroup as for one problem per expert (what a decode-sized call usually has)
+        const std::vector<int> nrs((size_t)std::min<long>(E, P), nrB);
+        if (int rc = plan_gemv_rows16_grouped(down[0]->fmt, (int)F, nrs.data(), (int)nrs.size(), &rp->planB)) return rc;
+    }
+    sh.wgA = rp->planA.grid;  // workgroups of one problem
+    sh.wgB = (((int)D + 15) / 16 + rp->planB.T - 1) / rp->planB.T;
+    // an expert's last chunk may be short: at most one more problem per expert that has pairs than P / cap
+    sh.maxA = (int)std::min<long>(P, (long)std::min<long>(E, P) + P / sh.capA);
+    sh.maxB = (int)std::min<long>(P, (long)std::min<long>(E, P) + P / sh.capB);
+    rp->planA.grid = sh.maxA * sh.wgA;
+    rp->planB.grid = sh.maxB * sh.wgB;
+    sh.strideXA = (size_t)D * 2; sh.strideYA = (size_t)F * 2; sh.strideXB = (size_t)F * 2; sh.strideYB = (size_t)D * 4;
+    size_t off = 0;
+    auto take = [&](size_t bytes) { const size_t at = off; off += (bytes + 15) & ~(size_t)15; return at; };
+    rp->off_first = take((size_t)(E + 1) * 4);
+    rp->off_rows = take((size_t)P * 4);
+    rp->off_wts = take((size_t)(P + 1) * 4);
+    rp->off_tokf = take((size_t)(T + 1) * 4);
+    rp->off_tokp = take((size_t)P * 4);
+    rp->off_tabA = take((size_t)sh.maxA * sizeof(GemvProb));
+    rp->off_tabB = take((size_t)sh.maxB * sizeof(GemvProb));
+    rp->off_mapA = take((size_t)rp->planA.grid * 4);
+    rp->off_mapB = take((size_t)rp->planB.grid * 4);
+    rp->list_bytes = off;
+    return TFQ_OK;
+}
+}  // namespace
+
+size_t moe_routed_workspace_bytes(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E, int T, int Ktop) {
+    RoutedPlan rp{};
+    if (plan_routed(gate, up, down, E, T, Ktop, TFQ_BF16, TFQ_BF16, &rp) != TFQ_OK) return 0;
+    const size_t P = (size_t)T * Ktop, D = (size_t)gate[0]->K, F = (size_t)gate[0]->N;
+    return align256(P * D * 2) + align256((P + 1) * F * 2) + align256((P + 1) * D * 4) + align256(rp.list_bytes);
+}
+
+int moe_expert_table(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E, void* d_table) {
+    std::vector<const uint8_t*> ptrs((size_t)3 * E);
+    for (int e = 0; e < E; ++e) { ptrs[e] = gate[e]->dev; ptrs[(size_t)E + e] = up[e]->dev; ptrs[(size_t)2 * E + e] = down[e]->dev; }
+    TFQ_HIP(hipMemcpy(d_table, ptrs.data(), ptrs.size() * sizeof(void*), hipMemcpyHostToDevice));
+    return TFQ_OK;
+}
+
+int launch_moe_ffn_routed(const tfq_weight* const* gate, const tfq_weight* const* up, const tfq_weight* const* down, int E,
+                          const void* d_expert_table, const int32_t* d_topk_idx, const float* d_topk_w, int T, int Ktop,
+                          const void* x, int x_dtype, void* y, int y_dtype, int mid_dtype, void* workspace, size_t workspace_bytes,
+                          hipStream_t s) {
+    RoutedPlan rp{};
+    if (int rc = plan_routed(gate, up, down, E, T, Ktop, x_dtype, mid_dtype, &rp)) return rc;
+    const size_t P = (size_t)T * Ktop, D = (size_t)gate[0]->K, F = (size_t)gate[0]->N;
+    if (workspace_bytes < moe_routed_workspace_bytes(gate, up, down, E, T, Ktop))
+        return fail(TFQ_ERR_SHAPE, "moe routed: workspace smaller than tfq_moe_routed_workspace_bytes");
+    uint8_t* base = static_cast<uint8_t*>(workspace);
+    uint8_t* xe = base;
+    uint8_t* h = xe + align256(P * D * 2);
+    uint8_t* o = h + align256((P + 1) * F * 2);
+    uint8_t* lists = o + align256((P + 1) * D * 4);
+    int* d_first = reinterpret_cast<int*>(lists + rp.off_first);
+    int* d_rows = reinterpret_cast<int*>(lists + rp.off_rows);
+    float* d_w = reinterpret_cast<float*>(lists + rp.off_wts);
+    int* d_tokf = reinterpret_cast<int*>(lists + rp.off_tokf);
+    int* d_tokp = reinterpret_cast<int*>(lists + rp.off_tokp);
+    GemvProb* tabA = reinterpret_cast<GemvProb*>(lists + rp.off_tabA);
+    GemvProb* tabB = reinterpret_cast<GemvProb*>(lists + rp.off_tabB);
+    int* mapA = reinterpret_cast<int*>(lists + rp.off_mapA);
+    int* mapB = reinterpret_cast<int*>(lists + rp.off_mapB);
+    hipLaunchKernelGGL(routed_lists_kernel, dim3(1), dim3(1024), 0, s, d_topk_idx, d_topk_w, T, Ktop, E, d_first, d_rows, d_w, d_tokf, d_tokp,
+                       rp.sh, static_cast<const uint8_t* const*>(d_expert_table), (const uint8_t*)xe, h, o, tabA, mapA, tabB, mapB);
+    const int row_u4 = (int)(D * 2 / 16);
+    const int64_t ng = (int64_t)P * row_u4;
+    hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)((ng + 255) / 256)), dim3(256), 0, s, (const uint4*)x, (uint4*)xe, (const int*)d_rows, (int)P, row_u4);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return hip_fail(e, "moe routed launch");
+    if (int rc = launch_gemv_grouped(gate[0]->fmt, rp.planA, tabA, mapA, TFQ_BF16, s)) return rc;
+    if (int rc = launch_gemv_rows16_grouped(down[0]->fmt, rp.planB, tabB, mapB, TFQ_F32, s)) return rc;
+    const int64_t nout = (int64_t)T * (int64_t)D;
+    if (y_dtype == TFQ_BF16)
+        hipLaunchKernelGGL(combine_kernel<true>, dim3((unsigned)((nout + 255) / 256)), dim3(256), 0, s, y, (const float*)o, (const int*)d_tokf, (const int*)d_tokp, (const float*)d_w, T, (int)D, 0);
+    else
+        hipLaunchKernelGGL(combine_kernel<false>, dim3((unsigned)((nout + 255) / 256)), dim3(256), 0, s, y, (const float*)o, (const int*)d_tokf, (const int*)d_tokp, (const float*)d_w, T, (int)D, 0);
+    return hip_fail(hipGetLastError(), "moe routed launch");
+}
+
 // Dense SwiGLU feed-forward (Qwen35Engine::mlp_step, src/adapters/tools/qwen35_engine.cpp:662-672): gate and up
 // in one launch where the format has the multi-matrix kernel, the elementwise step, down.  Rows above sixteen go
 // through the prefill entry.
