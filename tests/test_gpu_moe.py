@@ -196,6 +196,42 @@ def test_moe_ffn_routed_builds_its_lists_on_the_device(O, tfq, gpu, fmt):
         wl.close()
 
 
+@pytest.mark.parametrize("T,Ktop,E", [(1, 1, 3), (7, 3, 5), (64, 2, 4), (128, 8, 16), (5, 2, 40)])
+def test_moe_ffn_routed_shapes(O, tfq, gpu, T, Ktop, E):
+    """Call shapes of the routed form: one pair, odd counts, experts with several passes of eight and sixteen
+    rows, the largest call it takes (1024 pairs), more experts than pairs.  Against tfq_moe_ffn with the same
+    routing read back to the host (which cuts the rows into passes by its own rules: equal to rounding, or to the
+    bf16 tolerance where it takes the prefill GEMM)."""
+    import torch
+    fmt, D, F = "B32S4", 256, 512
+    gate, up, down, _, _, _ = _experts(O, tfq, fmt, E, D, F, 840)
+    logits = torch.from_numpy(O.rng_normal(53, T * E, 1.0).reshape(T, E)).to(gpu)
+    _, idx, w = tfq.moe_route(logits, Ktop)
+    xt = torch.from_numpy(O.rng_normal(54, T * D, 1.0).reshape(T, D)).to(gpu).bfloat16()
+    host = tfq.moe_ffn(gate, up, down, idx.cpu().numpy().astype(np.int64), w.cpu().numpy(), xt, mid_dtype=torch.bfloat16)
+    y = torch.empty(T, D, device=gpu)
+    tfq.RoutedMoe(gate, up, down, T, Ktop)(idx, w, xt, y)
+    # with more than 32 rows on an expert the host-list call multiplies through the prefill GEMM, whose weights are
+    # rounded to bf16; the routed call always takes the decode kernels
+    counts = [int((idx == e).sum()) for e in range(E)]
+    tol = 1e-2 if max(counts) > 32 else 1e-5
+    assert float((y - host).abs().max()) <= tol * float(host.abs().max())
+    for wl in gate + up + down:
+        wl.close()
+
+
+def test_moe_ffn_routed_refuses_what_it_does_not_serve(O, tfq, gpu):
+    """More than 1024 pairs, or a format without the grouped kernels: no workspace size, and the call fails."""
+    gate, up, down, _, _, _ = _experts(O, tfq, "B32S4", 2, 256, 512, 860)
+    with pytest.raises(tfq.TfqError):
+        tfq.RoutedMoe(gate, up, down, 600, 2)
+    g3, u3, d3, _, _, _ = _experts(O, tfq, "Q_G_3", 2, 256, 512, 870)
+    with pytest.raises(tfq.TfqError):
+        tfq.RoutedMoe(g3, u3, d3, 4, 2)
+    for wl in gate + up + down + g3 + u3 + d3:
+        wl.close()
+
+
 def test_moe_ffn_routed_in_a_graph(O, tfq, gpu):
     """The routed call captured into a graph together with the router: replays with other activations (hence other
     routing) equal the eager calls bit for bit, with eager work and synchronizations between the replays."""
