@@ -9,9 +9,9 @@
 //   * copies half of a 256 x 64 activation chunk to LDS (bf16), global -> LDS without passing registers, a whole
 //     128-byte line per row (64 bytes per row, one step's worth, left L2 at half the rate: a loop of nothing
 //     but the copies and the barriers took 140 us for 14336x4096 x 2048 tokens against 85 us with whole lines),
-//   * decodes the weight tile: one lane takes one or two code dwords (8 weights each),
-//     converts the nibbles with v_cvt_f32_ubyte, applies the group's scale and
-//     offset in fp32
+//   * decodes the weight tile: one lane takes one or two code dwords (8 weights each), turns the nibbles into
+//     binary16 pairs 1024 + n with one and-or per two weights (the 8-bit formats: bytes, v_cvt_f32_ubyte), applies
+//     the group's scale and offset in fp32
 //         w = a * n + c,   (a, c) = (d, -8d) or (d*sc/15, -dm*mc)
 //     packs to bf16 (v_cvt_pk_bf16_f32) and stores the 8 weights to LDS,
 //   * runs 32, 28 or 16 v_mfma_f32_16x16x32_bf16 per wavefront (sub-tiles of 128 x 64, 64 x 112, 64 x 64:
@@ -29,8 +29,8 @@
 // reads, decode | MFMAs) and the two wavefronts of a SIMD are kept in opposite phases (PP below).
 // Where the time of a step goes (14336x4096 x 2048 tokens, B32S4, 253 us; parts taken out at compile time):
 // without the decode and its LDS stores 175 us, without the fragment reads 188 us, without the MFMAs 218 us,
-// loads and barriers alone 100 us: the decode's vector instructions (about 58 per wavefront and step beside 28
-// MFMAs) are the largest part, and they are already at one decode per weight and workgroup.
+// loads and barriers alone 100 us: the decode's vector instructions (50 per wavefront and step beside 28 MFMAs
+// then; 44 with the binary16 pairs, 244 us) are the largest part, and every weight is decoded once per workgroup.
 
 #include <algorithm>
 #include <atomic>
@@ -218,7 +218,8 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
     // too: it would wait for them with counts that leave the copies out, which are therefore too
     // strict and, where it has moved a load, drain the whole queue in the middle of the loop.
     // Loads return in the order of issue; step s issues, in this order, its XL copies, WROWS * NP code
-    // dwords and (when it starts a block) WROWS headers for step s + 3.  A register that a load is
+    // dwords and (when it starts a block) WROWS headers for step s + 3 (the copies: half a chunk, two chunks
+    // ahead).  A register that a load is
     // still writing is named by no instruction until the wait that covers it.
     uint32_t rw[WROWS][NP][4];  // ring of four: set r holds the code dwords of a step with ks % 4 == r
     u32x4_t hnext[WROWS];
