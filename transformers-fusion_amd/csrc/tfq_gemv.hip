@@ -118,7 +118,7 @@ struct GemvKernArgs {
 // column (2 T partial-sum cells), and the epilogue writes silu(gate x) * (up x) to y0.  The down product then
 // reads that vector like any other activation, instead of evaluating the exponentials in every workgroup.
 template <int FMT, bool XF32, int WD, int SETS = 1, bool GROUPED = false, int XOP = XOP_NONE, bool PAIR = false>
-__global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin_arg) {
+__global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1024 : 512) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin_arg) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
     static_assert(XOP == XOP_NONE || (XF32 && SETS == 1 && !GROUPED), "prologues take fp32 input in the plain launch");
@@ -353,7 +353,11 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
     const uint32_t M = 0x000F000Fu;
     uint32_t C = 0x43004300u;
     asm volatile("" : "+v"(C));  // keep the bias in a VGPR so (v & M) | C is one v_and_or_b32
-    uint4 av[SETS][2][4];
+    // Two slot sets: the A fragments stay in LDS and are read per MFMA (sixteen 128-bit LDS reads per unit), which
+    // leaves room for sixteen wavefronts per workgroup; one or four sets keep them in registers.
+    constexpr bool A_LDS = SETS == 2 && F::HV == 1;  // (the formats with byte headers do not fit 128 registers either way)
+    uint4 av[A_LDS ? 1 : SETS][2][4];
+    const uint4* asrc[SETS][2];
     float xv[SETS][2][PER];
     int c_ci = 0, c_t = 0;
     float* cell = part + wave * SETS * 64 + lane;  // this wavefront's cells of tile c_t, one per slot set
@@ -367,8 +371,11 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
                     const uint4* src = live ? col + (4 * st + s_a) * 32 + h * 16 + q * 4 : zero4;
+                    asrc[st][h] = src;
+                    if constexpr (!A_LDS) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) av[st][h][j] = src[j];
+                        for (int j = 0; j < 4; ++j) av[st][h][j] = src[j];
+                    }
 #pragma unroll
                     for (int t = 0; t < PER; t += 4) {
                         const float4 f = *reinterpret_cast<const float4*>(colX + (4 * st + q) * NG + h * PER + t);
@@ -416,11 +423,14 @@ __global__ __launch_bounds__(SETS == 1 ? 1024 : 512) void gemv4_kernel(GemvKernA
                     const bool second = pl == 1 || (F::GS == 16 && j >= 2);
 #pragma unroll
                     for (int st = 0; st < SETS; ++st) {
+                        uint4 afr;
+                        if constexpr (A_LDS) afr = asrc[st][h][j];
+                        else afr = av[st][h][j];
                         if (!second)
-                            DA[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[st][h][j]),
+                            DA[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, afr),
                                                                              __builtin_bit_cast(bf16x8_t, wv), DA[st], 0, 0, 0);
                         else
-                            DB[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[st][h][j]),
+                            DB[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, afr),
                                                                              __builtin_bit_cast(bf16x8_t, wv), DB[st], 0, 0, 0);
                     }
                 }
@@ -873,9 +883,13 @@ GemvPlan plan_gemv4(const GemvArgs& a, int nslot) {
     // wavefronts per workgroup.  One slot set: as many as there are (16); more wavefronts keep more fetches in
     // flight, which counts for more than an even split of the block columns (measured, B32S4 4096x14336: 8.8 us
     // with 16 wavefronts of 3 or 4 columns against 9.7-10.5 us with 14 of 4; 4096x7168 5.25 against 5.9 us).
-    // Several slot sets need the registers of two wavefronts, so at most 8 then: the count in 4..8 that splits
-    // the block columns most evenly.
-    const int max_nw = p.sets == 1 ? 16 : 8;
+    // Two slot sets of a format with a 16-byte header: sixteen as well, with the A fragments read from LDS per
+    // MFMA instead of held in registers (106-128 registers; measured against eight wavefronts with the fragments
+    // in registers, B32S4 at eight rows: q+k+v 6.6 against 8.0 us, o 5.9 against 7.2 us, gate+up 15.9 / 15.7 us;
+    // the grouped gate / up launch of a mixture layer 102.7 against 110.3 us).  Otherwise several slot sets need
+    // the registers of two wavefronts, so at most 8 then: the count in 4..8 that splits the block columns most
+    // evenly.
+    const int max_nw = p.sets == 1 || (p.sets == 2 && Fmt<FMT>::HV == 1) ? 16 : 8;
     p.NW = nblocks < max_nw ? nblocks : max_nw;
     if (nblocks > max_nw && p.sets > 1) {
         int best_waste = 1 << 30;
@@ -1138,21 +1152,20 @@ int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, 
     k.cols_base = nblocks / gp.NW; k.cols_rem = nblocks % gp.NW;
     using Kernel = void (*)(GemvKernArgs, const void*);
     constexpr int WDG = 2;  // two unit fetches in flight: every format's kernel holds that many without spilling
-    // The two-set kernel (eight wavefronts per workgroup) takes four here: with two, a compute unit has 37 KB on
-    // its way and the grouped gate / up launch of a mixture layer streams at 4.45 TB/s (118.6 us); with four,
-    // 110.3 us.  The plain launch of the same kernel is slower with four (gate + up at eight rows 16.8 against
-    // 15.7 us) and keeps two.
+    // (With eight wavefronts per workgroup the two-set kernel had only 37 KB per compute unit on their way and
+    // the grouped gate / up launch of a mixture layer streamed at 4.45 TB/s, 118.6 us; four fetches per
+    // wavefront gave 110.3 us, sixteen wavefronts of two fetches, what runs now, 102.7 us.)
     Kernel kern = gp.x_f32 ? gemv4_kernel<FMT, true, WDG, 1, true> : gemv4_kernel<FMT, false, WDG, 1, true>;
     int slot = gp.x_f32 ? 1 : 0;
     if constexpr (kWide<FMT>) {
-        if (gp.sets == 2) { kern = gemv4_kernel<FMT, false, 4, 2, true>; slot = 2; }
+        if (gp.sets == 2) { kern = gemv4_kernel<FMT, false, 2, 2, true>; slot = 2; }
         if (gp.sets == 4) { kern = gemv4_kernel<FMT, false, 1, 4, true>; slot = 3; }
     }
     if (gp.pair) {
         if constexpr (kPaired<FMT>) {
             kern = gp.x_f32 ? gemv4_kernel<FMT, true, WDG, 1, true, XOP_NONE, true> : gemv4_kernel<FMT, false, WDG, 1, true, XOP_NONE, true>;
             slot = gp.x_f32 ? 5 : 4;
-            if (gp.sets == 2) { kern = gemv4_kernel<FMT, false, 4, 2, true, XOP_NONE, true>; slot = 6; }
+            if (gp.sets == 2) { kern = gemv4_kernel<FMT, false, 2, 2, true, XOP_NONE, true>; slot = 6; }
             if (gp.sets == 4) { kern = gemv4_kernel<FMT, false, 1, 4, true, XOP_NONE, true>; slot = 7; }
         } else {
             return fail(TFQ_ERR_FORMAT, "gemv group: no paired kernel for this format");
