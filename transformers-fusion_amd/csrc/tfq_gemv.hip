@@ -359,6 +359,8 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
     uint4 av[A_LDS ? 1 : SETS][2][4];
     const uint4* asrc[SETS][2];
     float xv[SETS][2][PER];
+    float sxv[SETS][2];  // byte-header formats: the sum of a k-step's group sums, added up once per block column
+    constexpr bool SXK = tiled_header_in_bytes(FMT);
     int c_ci = 0, c_t = 0;
     float* cell = part + wave * SETS * 64 + lane;  // this wavefront's cells of tile c_t, one per slot set
     auto consume = [&](int u) __attribute__((always_inline)) {
@@ -380,6 +382,12 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
                     for (int t = 0; t < PER; t += 4) {
                         const float4 f = *reinterpret_cast<const float4*>(colX + (4 * st + q) * NG + h * PER + t);
                         xv[st][h][t] = f.x; xv[st][h][t + 1] = f.y; xv[st][h][t + 2] = f.z; xv[st][h][t + 3] = f.w;
+                    }
+                    if constexpr (SXK) {  // the same order of additions as apply_groups uses
+                        float sx = 0.0f;
+#pragma unroll
+                        for (int t = 0; t < PER; ++t) sx += xv[st][h][t];
+                        sxv[st][h] = sx;
                     }
                 }
             }
@@ -436,7 +444,10 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
                 }
             }
 #pragma unroll
-            for (int st = 0; st < SETS; ++st) res[st] += apply_groups<FMT>(hd[u], h, DA[st], DB[st], xv[st][h]);
+            for (int st = 0; st < SETS; ++st) {
+                if constexpr (SXK) res[st] += apply_groups<FMT, true>(hd[u], h, DA[st], DB[st], xv[st][h], sxv[st][h]);
+                else res[st] += apply_groups<FMT>(hd[u], h, DA[st], DB[st], xv[st][h]);
+            }
         }
         // the first block column writes the cells, later ones add to them (no zero fill, no read)
 #pragma unroll

@@ -104,8 +104,11 @@ __device__ __forceinline__ uint32_t field(const uint32_t* w, int pos, int count)
 // With 32-weight groups DA[r] is the dot product of group r; with 16-weight groups DA[r] / DB[r]
 // are the two halves of 32-slot r, i.e. groups 2r and 2r + 1, and X holds the eight activation
 // sums in group order.  For the 8-bit format DA / DB are the low / high nibble planes.
-template <int FMT>
-__device__ __forceinline__ float apply_groups(const uint4* hv, int khalf, f32x4_t DA, f32x4_t DB, const float* X) {
+// (sx_known: the sum of the k-step's activation group sums, for the formats that need it, when the caller has it
+// already: it does not depend on the weight row, so a caller that walks several tiles with one set of
+// activations adds it up once.)
+template <int FMT, bool SX_KNOWN = false>
+__device__ __forceinline__ float apply_groups(const uint4* hv, int khalf, f32x4_t DA, f32x4_t DB, const float* X, float sx_known = 0.0f) {
     constexpr Spec sp = spec_of(FMT);
     float res = 0.0f;
     if constexpr (FMT == TFQ_B32S4 || Fmt<FMT>::NP == 2) {
@@ -136,13 +139,13 @@ __device__ __forceinline__ float apply_groups(const uint4* hv, int khalf, f32x4_
                              byte_to_float<0>(sc_hi), byte_to_float<1>(sc_hi), byte_to_float<2>(sc_hi), byte_to_float<3>(sc_hi)};
         const float mc[8] = {byte_to_float<0>(mc_lo), byte_to_float<1>(mc_lo), byte_to_float<2>(mc_lo), byte_to_float<3>(mc_lo),
                              byte_to_float<0>(mc_hi), byte_to_float<1>(mc_hi), byte_to_float<2>(mc_hi), byte_to_float<3>(mc_hi)};
-        float sa = 0.0f, sm = 0.0f, sx = 0.0f;
+        float sa = 0.0f, sm = 0.0f, sx = SX_KNOWN ? sx_known : 0.0f;
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
             const float D = (t & 1) ? DB[t >> 1] : DA[t >> 1];
             sa = __builtin_fmaf(sc[t], D, sa);
             sm = __builtin_fmaf(mc[t], X[t], sm);
-            sx += X[t];
+            if constexpr (!SX_KNOWN) sx += X[t];
         }
         res = __builtin_fmaf(dtop, sa, dm * __builtin_fmaf((float)mbias, sx, -sm));
     } else {
