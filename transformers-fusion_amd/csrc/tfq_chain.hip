@@ -334,7 +334,7 @@ __global__ __launch_bounds__(1024) void chain_kernel(ChainArgs a) {
                 cc[0] = *reinterpret_cast<const uint4*>(sp + 16 * lane);
                 cc[1] = *reinterpret_cast<const uint4*>(sp + 1024 + 16 * lane);
 #pragma unroll
-                for (int i = 0; i < F::HV; ++i) hd[i] = *reinterpret_cast<const uint4*>(sp + 2048 + F::HB * n + 16 * i);
+                for (int i = 0; i < F::HV; ++i) hd[i] = *reinterpret_cast<const uint4*>(sp + tiled_header_offset(FMT, n, i));
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 issue(slot);
                 slot = slot + 1 == D ? 0 : slot + 1;

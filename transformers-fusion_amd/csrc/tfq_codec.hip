@@ -1232,7 +1232,8 @@ __global__ __launch_bounds__(256) void tile16_kernel(const uint8_t* __restrict__
             }
         }
     } else {
-        const int n = (p - CP) / HP, part = (p - CP) % HP;
+        // header pieces: one per row, or part-major planes of sixteen rows (tiled_header_offset)
+        const int n = HP == 1 ? p - CP : (p - CP) % 16, part = HP == 1 ? 0 : (p - CP) / 16;
         const int64_t row = tile * 16 + n;
         if (row < N) {
             const uint8_t* src = wire + (row * nblocks + blk) * (int64_t)BB;
@@ -1308,10 +1309,13 @@ __global__ __launch_bounds__(256) void decode_tiled_kernel(const uint8_t* __rest
         const uint32_t g = i / sp.gsz;
         float sc, mc, d, dm;
         if constexpr (tiled_header_in_bytes(FMT)) {
-            sc = (float)h[g];
-            mc = (float)h[16 + g] - (float)bias;
-            d = half_bits_to_float((uint32_t)h[32] | ((uint32_t)h[33] << 8));
-            dm = half_bits_to_float((uint32_t)h[34] | ((uint32_t)h[35] << 8));
+            const uint8_t* h0 = unit + tiled_header_offset(FMT, n, 0);
+            const uint8_t* h1 = unit + tiled_header_offset(FMT, n, 1);
+            const uint8_t* h2 = unit + tiled_header_offset(FMT, n, 2);
+            sc = (float)h0[g];
+            mc = (float)h1[g] - (float)bias;
+            d = half_bits_to_float((uint32_t)h2[0] | ((uint32_t)h2[1] << 8));
+            dm = half_bits_to_float((uint32_t)h2[2] | ((uint32_t)h2[3] << 8));
         } else {
             sc = (float)stream_bits(h, HB, g * sp.scb, sp.scb);
             mc = (float)stream_bits(h, HB, sc_bits + g * sp.mb, sp.mb) - (float)bias;

@@ -237,7 +237,8 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
     const uint8_t* col_ptr = Wm + ((size_t)tile0 * nblocks + (size_t)wave) * UB;
     const uint8_t* f_ptr = col_ptr;
     int f_t = 0, f_left = nitems;
-    const uint32_t off_c = 16u * lane, off_h = (uint32_t)F::CODE_BYTES + (uint32_t)F::HB * n;
+    const uint32_t off_c = 16u * lane, off_h = (uint32_t)tiled_header_offset(FMT, n, 0);
+    constexpr int HSTEP = tiled_header_offset(FMT, 0, 1) - tiled_header_offset(FMT, 0, 0);  // between the parts of a row's header
     auto fetch = [&](uint4 (&cc)[NC], uint4 (&hd)[F::HV]) __attribute__((always_inline)) {
         if constexpr (F::CW == 4) {
 #pragma unroll
@@ -246,7 +247,7 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
             cc[0] = stream_load16(f_ptr + off_c);
         }
 #pragma unroll
-        for (int i = 0; i < F::HV; ++i) hd[i] = stream_load16(f_ptr + off_h + 16 * i);
+        for (int i = 0; i < F::HV; ++i) hd[i] = stream_load16(f_ptr + off_h + HSTEP * i);
         if (--f_left > 0) {
             f_ptr += tile_stride;
             ++f_t;

@@ -271,7 +271,7 @@ int ensure_device();  // TFQ_OK once a gfx950 device is current and tables are l
 //            where code slot l = n + 16 q holds the 32 codes k = 32 (q + 4 kstep) .. + 31
 //            of row n as nibbles (code 2j in the low half of byte j), and header
 //            slot n holds row n's block header, the wire bytes behind the codes,
-//            zero padded to HB = 16 or 32 bytes.  2- and 3-bit codes are widened to
+//            zero padded to HB = 16 bytes (48-byte headers: see tiled_header_offset).  2- and 3-bit codes are widened to
 //            nibbles here (the matmul kernel turns a nibble into a bf16 operand with
 //            one operation; the wire bit streams straddle every register boundary).
 //            Units are ordered tile-major, so one wavefront reads one unit as a
@@ -315,6 +315,14 @@ __host__ __device__ constexpr int tiled_code_bytes(int fmt) {
     return tiled_code_width(fmt) == 2 ? 1024 : 2048 * tiled_planes(fmt);
 }
 __host__ __device__ constexpr int tiled_unit_bytes(int fmt) { return tiled_code_bytes(fmt) + 16 * tiled_header_bytes(fmt); }
+// Byte offset inside a unit of the 16-byte part `part` of row n's header.  A 16-byte header is one piece per row.
+// The 48-byte headers are stored part-major, three planes of sixteen rows: the sixteen lanes that fetch one part
+// for their rows then read 256 contiguous bytes, and the three fetches of a unit touch every cache line once
+// (row-major, every fetch touched all six lines of the header area: 14336 x 4096, one row, SB256A3 11.9 us and
+// SB256A2 10.2 us then, 11.3 us and 10.1 us now).
+__host__ __device__ constexpr int tiled_header_offset(int fmt, int n, int part) {
+    return tiled_code_bytes(fmt) + (tiled_header_bytes(fmt) == 16 ? 16 * n : 256 * part + 16 * n);
+}
 }  // namespace tfq
 
 struct tfq_weight {
