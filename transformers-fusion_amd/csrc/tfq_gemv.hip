@@ -362,6 +362,9 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
     float xv[SETS][2][PER];
     float sxv[SETS][2];  // byte-header formats: the sum of a k-step's group sums, added up once per block column
     constexpr bool SXK = tiled_header_in_bytes(FMT);
+    // symmetric formats use the group sums only as the start value -OFFS * X of the accumulators: multiplied once
+    // per block column, not per unit
+    constexpr bool XPRE = FMT == TFQ_B32S4 || F::NP == 2;
     int c_ci = 0, c_t = 0;
     float* cell = part + wave * SETS * 64 + lane;  // this wavefront's cells of tile c_t, one per slot set
     auto consume = [&](int u) __attribute__((always_inline)) {
@@ -384,6 +387,10 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
                         const float4 f = *reinterpret_cast<const float4*>(colX + (4 * st + q) * NG + h * PER + t);
                         xv[st][h][t] = f.x; xv[st][h][t + 1] = f.y; xv[st][h][t + 2] = f.z; xv[st][h][t + 3] = f.w;
                     }
+                    if constexpr (XPRE) {
+#pragma unroll
+                        for (int t = 0; t < PER; ++t) xv[st][h][t] *= -F::OFFS;
+                    }
                     if constexpr (SXK) {  // the same order of additions as apply_groups uses
                         float sx = 0.0f;
 #pragma unroll
@@ -405,7 +412,9 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
             for (int st = 0; st < SETS; ++st) {
                 const float* X = xv[st][h];
                 DB[st] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-                if constexpr (F::GS == 32) {
+                if constexpr (XPRE) {
+                    DA[st] = f32x4_t{X[0], X[1], X[2], X[3]};
+                } else if constexpr (F::GS == 32) {
                     DA[st] = f32x4_t{-F::OFFS * X[0], -F::OFFS * X[1], -F::OFFS * X[2], -F::OFFS * X[3]};
                 } else {
                     DA[st] = f32x4_t{-F::OFFS * X[0], -F::OFFS * X[2], -F::OFFS * X[4], -F::OFFS * X[6]};
