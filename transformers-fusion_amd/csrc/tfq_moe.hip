@@ -740,8 +740,10 @@ int launch_mlp_step(const tfq_weight* gate, const tfq_weight* up, const tfq_weig
         if (int rc = launch_gemm(gate, x, x_dtype, B, g, TFQ_F32, s, scratch, scratch_bytes)) return rc;
         if (int rc = launch_gemm(up, x, x_dtype, B, u, TFQ_F32, s, scratch, scratch_bytes)) return rc;
     }
-    if (B <= 16 && gemv_prologue_supported(down)) {
-        // silu(gate) * up happens while the down kernel stages its activations
+    if (B <= 16 && gemv_prologue_supported(down) && (B <= 2 || mid_dtype == TFQ_F32)) {
+        // silu(gate) * up happens while the down kernel stages its activations.  The prologue reads fp32 rows, two
+        // per pass over the matrix: with bf16 mid activations and more rows the elementwise kernel below and one
+        // pass of the sixteen-row kernel are cheaper (fp32 mid activations take two rows per pass either way)
         tfq_prologue_t pro{};
         pro.op = TFQ_PRO_SWIGLU;
         pro.up = u;
