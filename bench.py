@@ -365,7 +365,24 @@ def prefill_gemm(tfq, torch, layer, M=2048, reps=10):
         tf = 2.0 * M * W.N * W.K / (ms * 1e-3) / 1e12
         out[name] = {"shape": "%dx%d" % (W.N, W.K), "us": round(ms * 1e3, 1), "tflops": round(tf, 1),
                      "frac": round(tf / MFMA_PEAK_TFLOPS, 4)}
-        del x, y
+        # For scale, on the same box (they differ by up to 20 % on this shape): the vendor library's plain
+        # bf16 GEMM (torch.matmul) on the same matrix decoded to bf16 beforehand, i.e. with no decode in the
+        # loop and four times the weight bytes.  A comparator only: nothing in the library calls it.
+        wd = W.decode().bfloat16()
+        yl = torch.empty((M, W.N), dtype=torch.bfloat16, device="cuda")
+        for _ in range(3):
+            torch.matmul(x, wd.T, out=yl)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            torch.matmul(x, wd.T, out=yl)
+        e1.record()
+        torch.cuda.synchronize()
+        ms_lib = e0.elapsed_time(e1) / reps
+        out[name]["library_bf16_gemm_us"] = round(ms_lib * 1e3, 1)
+        out[name]["library_bf16_gemm_tflops"] = round(2.0 * M * W.N * W.K / (ms_lib * 1e-3) / 1e12, 1)
+        out[name]["max_diff_vs_library"] = float((y.float() - yl.float()).abs().max() / yl.float().abs().max())
+        del x, y, wd, yl
     return out
 
 

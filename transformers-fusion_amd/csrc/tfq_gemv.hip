@@ -1003,13 +1003,14 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     } else
     if constexpr (kWide<FMT>) {
         if (p.sets > 1) {
-            kern = p.sets == 2 ? gemv4_kernel<FMT, false, 2, 2> : gemv4_kernel<FMT, false, 1, 4>;
-            slot = p.sets == 2 ? 6 : 7;
+            if (a.x_f32 && p.sets != 2) return fail(TFQ_ERR_SHAPE, "gemv: more than four fp32 rows in one pass");
+            kern = p.sets == 2 ? (a.x_f32 ? gemv4_kernel<FMT, true, 2, 2> : gemv4_kernel<FMT, false, 2, 2>) : gemv4_kernel<FMT, false, 1, 4>;
+            slot = p.sets == 2 ? (a.x_f32 ? 18 : 6) : 7;
         }
     } else if constexpr (kTwoSets<FMT>) {
         if (p.sets == 2) {
-            kern = gemv4_kernel<FMT, false, 2, 2>;
-            slot = 6;
+            kern = a.x_f32 ? gemv4_kernel<FMT, true, 2, 2> : gemv4_kernel<FMT, false, 2, 2>;
+            slot = a.x_f32 ? 18 : 6;
         } else if (p.sets > 2) {
             return fail(TFQ_ERR_SHAPE, "gemv: more than eight rows in one pass for this format");
         }
@@ -1117,6 +1118,8 @@ int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t 
             for (int rows = kWide<FMT> ? 16 : 8; rows > 4; rows >>= 1)
                 if (plan_gemv4<FMT>(a, rows).lds != 0) { step = rows; break; }
         }
+        // fp32 rows take two slots each (high and low part): the two-set kernel carries four of them
+        if (a.x_f32 && a.xop == XOP_NONE && !a.pair && B > 2 && plan_gemv4<FMT>(a, 8).lds != 0) step = 4;
     }
     for (int b0 = 0; b0 < B; b0 += step) {
         const int nb = B - b0 < step ? B - b0 : step;
