@@ -214,7 +214,8 @@ int tfq_weight_decode(const tfq_weight_t* w, float* out, tfq_stream_t stream);
  * path (any M).  x is [B][K], y is [B][N], row-major, dtypes TFQ_F32 / TFQ_BF16.
  * A handle with K above 4096 in a format of the 16-row decode kernel (B32S4,
  * B32S8, Q_G_4, Q_G_8, Q_8) carries a small area of partial sums (16 N fp32 per
- * 4096 of K) that calls with five or more bf16 rows use: such calls on ONE
+ * 4096 of K) that calls with five or more bf16 rows or three or more fp32 rows
+ * use: such calls on ONE
  * handle must not overlap in time (issue them on one stream, as the reference's
  * gemm is called; distinct handles are independent). */
 int tfq_gemv(const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, int y_dtype,

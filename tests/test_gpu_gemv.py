@@ -49,7 +49,7 @@ def test_gemv_bf16_activations(O, tfq, gpu, fmt, N, K, B):
 
 @pytest.mark.parametrize("fmt", GEMV_FORMATS)
 @pytest.mark.parametrize("N,K,B", [(64, 256, 1), (48, 2048, 1), (96, 4096, 1), (40, 1280, 4), (24, 4096, 16),
-                                   (72, 2304, 3), (33, 6400, 7), (40, 14336, 5)])
+                                   (72, 2304, 3), (33, 6400, 7), (40, 14336, 5), (1040, 14336, 8), (2000, 4096, 13), (272, 8192, 3)])
 def test_gemv_fp32_activations(O, tfq, gpu, fmt, N, K, B):
     import torch
     print(f"gemv f32 {fmt} N={N} K={K} B={B}", flush=True)

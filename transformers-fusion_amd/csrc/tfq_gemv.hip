@@ -590,12 +590,13 @@ __device__ __forceinline__ void transpose_rows(uint32_t (&v)[4]) {
 // or four unit fetches in flight, eight wavefronts of two columns, and fewer tiles per workgroup measured equal
 // or slower.
 constexpr int kGemvbKC = 16;  // block columns per K part
-template <int FMT, bool SPLIT, bool GROUPED = false>
+template <int FMT, bool SPLIT, bool GROUPED = false, bool XF32 = false>
 __global__ __launch_bounds__(1024) void gemvb_kernel(GemvKernArgs args, const unsigned short* __restrict__ x_arg) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
     static_assert(F::GS == 32 && F::HV == 1, "32-weight groups and a 16-byte header");
     static_assert(!(SPLIT && GROUPED), "a grouped launch has no K parts");
+    static_assert(!(XF32 && GROUPED), "grouped problems take bf16 rows");
     constexpr int UB = tiled_unit_bytes(FMT), NC = 2 * F::NP, WD = 2;
     const int K = args.K, T = args.tiles_per_wg;
     const bool y_bf16 = args.y_bf16 != 0;
@@ -653,12 +654,18 @@ __global__ __launch_bounds__(1024) void gemvb_kernel(GemvKernArgs args, const un
         // pair of groups is written (two loads: rows 0..7, 8..15) and read back in fragment order.  The row index
         // is xor-ed with twice the piece index so that the sixteen lanes of a quarter hit sixteen different
         // 16-byte bank groups on the way in and on the way out.
+        // fp32 input: a row is two slots (its bf16 high part and the bf16 of the remainder, adjacent rows 2 b and
+        // 2 b + 1 of the A operand).  A lane then loads the 32 bytes of its piece from fp32 row lane / 8 (eight rows
+        // x 256 bytes per pair of loads) and splits them before the exchange: the same two 16-byte pieces per pair
+        // of groups as for bf16 rows, written to rows 2 b and 2 b + 1.
         uint4 avr[2][4];
         const int piece = lane & 7, lrow = lane >> 3;
+        const int srow0 = XF32 ? 2 * lrow : lrow, srow1 = XF32 ? 2 * lrow + 1 : 8 + lrow;  // A rows of the two pieces
         const unsigned short* xrow0 = x + (size_t)min(lrow, B - 1) * K + piece * 8;
         const unsigned short* xrow1 = x + (size_t)min(8 + lrow, B - 1) * K + piece * 8;
-        const int w_slot0 = (piece >> 2) * 64 + (piece & 3) * 16 + (lrow ^ (piece * 2));
-        const int w_slot1 = (piece >> 2) * 64 + (piece & 3) * 16 + ((8 + lrow) ^ (piece * 2));
+        const float* xrowf = reinterpret_cast<const float*>(x) + (size_t)(XF32 ? min(lrow, (B >> 1) - 1) : 0) * K + piece * 8;
+        const int w_slot0 = (piece >> 2) * 64 + (piece & 3) * 16 + (srow0 ^ (piece * 2));
+        const int w_slot1 = (piece >> 2) * 64 + (piece & 3) * 16 + (srow1 ^ (piece * 2));
         const int r_slot0 = q * 16 + (n ^ (q * 2));
         const int r_slot1 = 64 + q * 16 + (n ^ ((4 + q) * 2));
         auto load_a = [&](int col) __attribute__((always_inline)) {
@@ -667,8 +674,13 @@ __global__ __launch_bounds__(1024) void gemvb_kernel(GemvKernArgs args, const un
 #pragma unroll
                 for (int gp = 0; gp < 2; ++gp) {
                     const int o = col * 256 + h * 128 + gp * 64;
-                    avr[h][2 * gp] = *reinterpret_cast<const uint4*>(xrow0 + o);
-                    avr[h][2 * gp + 1] = *reinterpret_cast<const uint4*>(xrow1 + o);
+                    if constexpr (XF32) {
+                        avr[h][2 * gp] = *reinterpret_cast<const uint4*>(xrowf + o);
+                        avr[h][2 * gp + 1] = *reinterpret_cast<const uint4*>(xrowf + o + 4);
+                    } else {
+                        avr[h][2 * gp] = *reinterpret_cast<const uint4*>(xrow0 + o);
+                        avr[h][2 * gp + 1] = *reinterpret_cast<const uint4*>(xrow1 + o);
+                    }
                 }
         };
         auto finish_a = [&]() __attribute__((always_inline)) {
@@ -677,6 +689,18 @@ __global__ __launch_bounds__(1024) void gemvb_kernel(GemvKernArgs args, const un
             for (int h = 0; h < 2; ++h)
 #pragma unroll
                 for (int gp = 0; gp < 2; ++gp) {
+                    if constexpr (XF32) {
+                        const uint4 a0 = avr[h][2 * gp], a1 = avr[h][2 * gp + 1];
+                        const uint32_t f[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+                        uint32_t hi[8], lo[8];
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) {
+                            hi[t] = bf16_rne(__uint_as_float(f[t]));
+                            lo[t] = bf16_rne(__uint_as_float(f[t]) - __uint_as_float(hi[t] << 16));
+                        }
+                        avr[h][2 * gp] = uint4{hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16)};
+                        avr[h][2 * gp + 1] = uint4{lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16), lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16)};
+                    }
                     stg[w_slot0] = avr[h][2 * gp];
                     stg[w_slot1] = avr[h][2 * gp + 1];
                     avr[h][2 * gp] = stg[r_slot0];
@@ -817,6 +841,18 @@ __global__ __launch_bounds__(1024) void gemvb_kernel(GemvKernArgs args, const un
     auto store_out = [&](int t, const float4& v) __attribute__((always_inline)) {
         const int row = (tile0 + t) * 16 + n;
         if (row >= nrm) return;
+        if constexpr (XF32) {  // the high and the low slot of a row are adjacent registers of one lane
+            const float o[2] = {v.x + v.y, v.z + v.w};
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const int b = 2 * q + r;
+                if (2 * b >= B) continue;
+                const size_t off = (size_t)b * (size_t)nrm + (size_t)row;
+                if (y_bf16) reinterpret_cast<unsigned short*>(ym)[off] = (unsigned short)bf16_rne(o[r]);
+                else reinterpret_cast<float*>(ym)[off] = o[r];
+            }
+            return;
+        }
         const float o[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -1073,12 +1109,15 @@ int run_gemvb(GemvArgs a, const void* x, hipStream_t s) {
     k.K = a.K; k.y_bf16 = a.y_bf16; k.nslot = a.nslot; k.tiles_per_wg = T;
     const size_t lds = (size_t)NW * 2560 + (size_t)T * NW * 1024;
     using Kernel = void (*)(GemvKernArgs, const unsigned short*);
-    const Kernel kern = split ? gemvb_kernel<FMT, true> : gemvb_kernel<FMT, false>;
-    static std::atomic<bool> lds_limit_raised[2] = {};
-    if (!lds_limit_raised[split ? 1 : 0]) {
+    static const Kernel kernels[2][2] = {{gemvb_kernel<FMT, false>, gemvb_kernel<FMT, true>},
+                                         {gemvb_kernel<FMT, false, false, true>, gemvb_kernel<FMT, true, false, true>}};
+    const int ki = (a.x_f32 ? 2 : 0) + (split ? 1 : 0);
+    const Kernel kern = kernels[a.x_f32 ? 1 : 0][split ? 1 : 0];
+    static std::atomic<bool> lds_limit_raised[4] = {};
+    if (!lds_limit_raised[ki]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
-        lds_limit_raised[split ? 1 : 0] = true;
+        lds_limit_raised[ki] = true;
     }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, s, k, static_cast<const unsigned short*>(x));
     return hip_fail(hipGetLastError(), "gemv launch");
@@ -1097,12 +1136,17 @@ int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t 
         // 16 us against 41 us) and wherever those need several passes because their staged activations do not
         // fit (4096x14336: 17 us against 24 / 47 us at 8 / 16 rows); equal for five to eight rows at K = 4096
         // (q+k+v 8.1 / 8.0, o 7.6 / 7.2, gate+up 15.6 / 15.7 us), which stay with the two-set kernel.
-        bool dense_rows = !a.x_f32 && B > 8;
-        if (!a.x_f32 && B > 4 && B <= 8) dense_rows = plan_gemv4<FMT>(a, 8).lds == 0;
+        // fp32 rows count twice (a high and a low slot each): eight of them per pass, from three rows on at a K whose
+        // staging does not fit and from five rows on otherwise.
+        const int slots = a.x_f32 ? 2 * B : B, per_pass = a.x_f32 ? 8 : 16;
+        bool dense_rows = slots > 8;
+        if (slots > 4 && slots <= 8) dense_rows = plan_gemv4<FMT>(a, 8).lds == 0;
+        if (a.xop != XOP_NONE || a.pair) dense_rows = false;
         if (dense_rows) {
-            for (int b0 = 0; b0 < B; b0 += 16) {
+            for (int b0 = 0; b0 < B; b0 += per_pass) {
                 GemvArgs ab = a;
-                ab.nslot = B - b0 < 16 ? B - b0 : 16;
+                const int nb = B - b0 < per_pass ? B - b0 : per_pass;
+                ab.nslot = a.x_f32 ? 2 * nb : nb;
                 for (int m = 0; m < a.nmat; ++m) ab.y[m] = (uint8_t*)a.y[m] + (size_t)b0 * (size_t)a.nrows[m] * ye;
                 if (int rc = run_gemvb<FMT>(ab, (const uint8_t*)x + (size_t)b0 * a.K * xe, s)) return rc;
             }
