@@ -144,6 +144,32 @@ def test_gemv_multi_matches_single_launches(O, tfq, gpu, fmt, B):
         W.close()
 
 
+@pytest.mark.parametrize("fmt", GEMV_FORMATS)
+@pytest.mark.parametrize("B", [3, 4, 8, 11])
+def test_gemv_multi_fp32_rows(O, tfq, gpu, fmt, B):
+    """Three matrices on one fp32 input of several rows (four rows per pass on the two-set kernel, eight on the
+    sixteen-row kernel): the same bits as single launches, and the oracle's result."""
+    import torch
+    K = 2048
+    shapes = [72, 24, 33]
+    xh = O.rng_normal(5, B * K, 1.0).reshape(B, K)
+    x = torch.from_numpy(xh).to(gpu)
+    Ws, singles, pays = [], [], []
+    for i, N in enumerate(shapes):
+        pay = O.encode_tensor(fmt, O.rng_normal(60 + i, N * K, 0.02))
+        W = tfq.Weight(fmt, N, K, pay)
+        Ws.append(W)
+        pays.append(pay)
+        singles.append(W.gemv(x))
+    outs = [torch.zeros(B, N, device=gpu) for N in shapes]
+    tfq.gemv_multi(Ws, x, outs)
+    for got, want, pay, N in zip(outs, singles, pays, shapes):
+        assert torch.equal(got, want)
+        assert rel_err(got.cpu().numpy(), O.matmul(fmt, pay, N, K, xh)) <= TOL_F32
+    for W in Ws:
+        W.close()
+
+
 @pytest.mark.parametrize("fmt", OTHER_FORMATS)
 @pytest.mark.parametrize("N,K,B,xdt", [(48, 512, 1, "bf16"), (33, 1024, 3, "bf16"), (20, 2304, 8, "f32"), (16, 4096, 16, "bf16")])
 def test_gemv_other_formats(O, tfq, gpu, fmt, N, K, B, xdt):
