@@ -1256,17 +1256,22 @@ namespace {
 template <int FMT>
 int plan_rows16_grouped(int K, const int* nrows, int nprob, GemvGroupPlan* gp) {
     const int nblocks = K >> 8;
-    const int NW = nblocks < 16 ? nblocks : 16;
-    const int max_t = (int)((160 * 1024 - (size_t)NW * 2560) / ((size_t)NW * 1024));
-    // tiles per workgroup: the fewest rounds of 256 workgroups, counting a workgroup's start-up (its wavefronts'
-    // first A fragments) as two tiles' worth
-    int best_t = 1;
+    // Wavefronts and tiles per workgroup: the least (rounds of 256 workgroups) x (block columns of the busiest
+    // wavefront) x (tiles + 2; a column's A fragments cost about two tiles' worth).  Fewer wavefronts leave LDS
+    // for more tiles per workgroup, i.e. fewer activation bytes per weight byte: at K = 14336 fourteen wavefronts
+    // of four columns walk eight tiles where sixteen of three or four have room for seven.
+    const int nw_max = nblocks < 16 ? nblocks : 16;
+    int NW = nw_max, best_t = 1;
     long best_cost = -1;
-    for (int T = max_t; T >= 1; --T) {
-        long wgs = 0;
-        for (int i = 0; i < nprob; ++i) wgs += ((nrows[i] + 15) / 16 + T - 1) / T;
-        const long cost = (wgs + 255) / 256 * (T + 2);
-        if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_t = T; }
+    for (int w = nw_max; w >= 1 && w >= nw_max - 4; --w) {
+        const int max_t = (int)((160 * 1024 - (size_t)w * 2560) / ((size_t)w * 1024));
+        const int cols = (nblocks + w - 1) / w;
+        for (int T = max_t; T >= 1; --T) {
+            long wgs = 0;
+            for (int i = 0; i < nprob; ++i) wgs += ((nrows[i] + 15) / 16 + T - 1) / T;
+            const long cost = (wgs + 255) / 256 * (T + 2) * cols;
+            if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_t = T; NW = w; }
+        }
     }
     gp->NW = NW; gp->T = best_t; gp->sets = 4; gp->K = K; gp->x_f32 = false; gp->pair = false;
     gp->lds = (size_t)NW * 2560 + (size_t)best_t * NW * 1024;
