@@ -169,6 +169,33 @@ def test_moe_ffn_long_down_rows_five_to_sixteen(O, tfq, gpu, fmt):
         wl.close()
 
 
+@pytest.mark.parametrize("fmt,D,F", [("B32S4", 256, 6144), ("B32S4", 768, 6400), ("Q_G_4", 512, 6144), ("B32S8", 256, 6144),
+                                     ("Q_G_8", 512, 6144)])
+def test_moe_ffn_tall_gate_up_with_five_to_eight_rows(O, tfq, gpu, fmt, D, F):
+    """Gate / up matrices with thousands of rows and experts of five to eight tokens: enough tiles for the grouped
+    launch whose wavefronts own whole tiles (a workgroup per compute unit, twelve tile pairs or more each), at one,
+    two and three block columns.  Host-side and device-side routing, against the oracle."""
+    import torch
+    E, Ktop, T = 8, 2, 20
+    gate, up, down, hg, hu, hd = _experts(O, tfq, fmt, E, D, F, 1100)
+    logits = O.rng_normal(52, T * E, 1.0).reshape(T, E)
+    _, idx, w = O.softmax_topk(logits, Ktop)
+    counts = [int((idx == e).sum()) for e in range(E)]
+    assert 4 < max(counts) <= 8, counts
+    x = O.bf16_round(O.rng_normal(53, T * D, 1.0).reshape(T, D))
+    ref = O.moe_ffn(fmt, hg, hu, hd, D, F, idx, w, x, mid_bf16=True)
+    xt = torch.from_numpy(x).to(gpu).bfloat16()
+    y = tfq.moe_ffn(gate, up, down, idx, w, xt, mid_dtype=torch.bfloat16)
+    assert rel_err(y.cpu().numpy(), ref) <= 1e-2
+    routed = tfq.RoutedMoe(gate, up, down, T, Ktop)
+    yr = torch.empty(T, D, device=gpu)
+    routed(torch.from_numpy(idx.astype(np.int32)).to(gpu), torch.from_numpy(w.astype(np.float32)).to(gpu), xt, yr)
+    assert rel_err(yr.cpu().numpy(), ref) <= 1e-2
+    assert float((yr - y).abs().max()) <= 1e-5 * float(y.abs().max())
+    for wl in gate + up + down:
+        wl.close()
+
+
 @pytest.mark.parametrize("fmt", ["B32S4", "Q_G_8"])
 def test_moe_ffn_routed_builds_its_lists_on_the_device(O, tfq, gpu, fmt):
     """tfq_moe_ffn_routed: routing arrays stay on the device, lists and launch tables are built there.  Skewed

@@ -117,6 +117,10 @@ struct GemvKernArgs {
 // shape and format); a workgroup walks its T tiles of gate and then the same T tiles of up for every block
 // column (2 T partial-sum cells), and the epilogue writes silu(gate x) * (up x) to y0.  The down product then
 // reads that vector like any other activation, instead of evaluating the exponentials in every workgroup.
+// uint4 entries from one activation slot's staged A entries to the next: 32, padded to 33 for the variant that
+// reads its A fragments from LDS per MFMA (two slot sets, 16-byte header)
+__host__ __device__ constexpr int a_slot_stride(int fmt, int sets) { return sets == 2 && tiled_header_bytes(fmt) == 16 ? 33 : 32; }
+
 template <int FMT, bool XF32, int WD, int SETS = 1, bool GROUPED = false, int XOP = XOP_NONE, bool PAIR = false>
 __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1024 : 512) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin_arg) {
     extern __shared__ uint4 smem[];
@@ -174,7 +178,12 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
     // LDS: per wavefront and block column, A entries [nslot][2 k-steps][4 slots of 32][4] (uint4) and
     // group sums [4 SETS slots][NG] (float); then one zero A entry set per wavefront, then the partial
     // sums [T][NW][SETS][64].
-    const int a_per_col = nslot * 32;                   // uint4 entries
+    // Where the A fragments are read from LDS per MFMA (A_LDS below) a slot's 32 entries are followed by one unused
+    // entry: the four lanes of a 16-lane row that read A entries (slots 4 st .. 4 st + 3, same offset inside the
+    // slot) would otherwise be 512 bytes apart, on the same banks (grouped gate / up launch of a mixture layer:
+    // 101 us at a stride of 32 entries, 89 us at 33 in gemvr_kernel).
+    constexpr int SS = a_slot_stride(FMT, SETS);
+    const int a_per_col = nslot * SS;                   // uint4 entries
     const int col_stride = a_per_col + SETS * NG;       // + 4 SETS NG floats of group sums
     uint4* my = smem + (size_t)wave * ncols_max * col_stride;
     uint4* zero4 = smem + (size_t)NW * ncols_max * col_stride + 4 * wave;  // this wavefront's own zero A entries
@@ -312,7 +321,7 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
                 v.z = e[4] | (e[5] << 16); v.w = e[6] | (e[7] << 16);
             }
             const uint4 p = pair_permute(v);
-            col[s * 32 + quad] = p;  // quad = (k-step, group, dword) in that order
+            col[s * SS + quad] = p;  // quad = (k-step, group, dword) in that order
             sum = dot2(ONES, p.x, 0.0f);
             sum = dot2(ONES, p.y, sum);
             sum = dot2(ONES, p.z, sum);
@@ -376,7 +385,7 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
                 const bool live = (c_a == q) && (4 * st + s_a < nslot);
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
-                    const uint4* src = live ? col + (4 * st + s_a) * 32 + h * 16 + q * 4 : zero4;
+                    const uint4* src = live ? col + (4 * st + s_a) * SS + h * 16 + q * 4 : zero4;
                     asrc[st][h] = src;
                     if constexpr (!A_LDS) {
 #pragma unroll
@@ -526,6 +535,244 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
         if (y_bf16) reinterpret_cast<unsigned short*>(ym)[off] = (unsigned short)bf16_rne(v);
         else reinterpret_cast<float*>(ym)[off] = v;
     }
+}
+
+// ---- grouped problems with many tiles per workgroup: gemvr_kernel
+// The kernel above splits a tile's block columns over the wavefronts and needs LDS cells for the partial sums of
+// every (tile, wavefront), which caps the tiles of a workgroup (five tile pairs beside eight staged rows of
+// K = 4096): a problem of a mixture layer then takes 180 workgroups, each of which stages the activations again and
+// ends in a barrier and a round of additions while its compute unit's share of the memory stream stands still.
+// Here a wavefront owns whole tiles instead (tiles wave, wave + NW, ... of the workgroup's range) and walks all
+// block columns of a tile, whose units are adjacent in memory; its sums stay in registers from the first column to
+// the last, so there are no cells, no additions across wavefronts and no barrier at the end, and a workgroup takes
+// as many tiles as the plan gives it (one workgroup per compute unit for the whole launch).  The price: every
+// wavefront needs the staged rows of every block column, so all of them are staged first (wavefront w stages
+// columns w, w + NW, ... as above, then one barrier; the first unit fetches are already on their way), and the A
+// fragments and group sums are read from LDS per unit.  Up to eight bf16 rows (two slot sets), 16-byte headers.
+// PAIR: a tile of gate, then the same tile of up; the output is silu(gate x) * (up x).  The sum of an output runs
+// over the block columns in ascending order: deterministic, but not the order of the kernel above.
+constexpr int kSlotStride = 33;  // uint4 entries from one activation slot's A entries to the next (gemvr_kernel)
+
+template <int FMT, bool PAIR>
+__global__ __launch_bounds__(1024) void gemvr_kernel(GemvKernArgs args) {
+    extern __shared__ uint4 smem[];
+    using F = Fmt<FMT>;
+    static_assert(F::HV == 1 && F::CW == 4 && F::GS == 32, "nibble codes, 32-weight groups, a 16-byte header");
+    constexpr int SETS = 2, WD = 2;
+    constexpr int UB = tiled_unit_bytes(FMT), NC = 2 * F::NP, NG = F::NG, PER = NG / 2;
+    constexpr bool XPRE = FMT == TFQ_B32S4 || F::NP == 2;
+    const int K = args.K, T = args.tiles_per_wg;
+    const bool y_bf16 = args.y_bf16 != 0;
+    const int bid = blockIdx.x;
+    const GemvProb* table = reinterpret_cast<const GemvProb*>(args.W0);
+    const int prob = reinterpret_cast<const int*>(args.W1)[bid];
+    if (prob < 0) return;  // a workgroup beyond the problems of this call (tables built on the device)
+    const GemvProb pr = table[prob];
+    const int nrm = pr.nrows, nslot = pr.nslot;
+    const uint8_t* Wm = pr.W;
+    void* ym = pr.y;
+    const uint8_t* xbytes = static_cast<const uint8_t*>(pr.x);
+
+    const int nblocks = K >> 8;
+    const int NW = blockDim.x >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, q = lane >> 4;
+    const int tile0 = (bid - pr.wg_first) * T;
+    const int tiles_real = min(T, ((nrm + 15) >> 4) - tile0);
+    const int ntiles_w = wave < tiles_real ? (tiles_real - wave + NW - 1) / NW : 0;
+    const int nitems = ntiles_w * nblocks * (PAIR ? 2 : 1);
+
+    // LDS: per block column, A entries [nslot][2 k-steps][4 slots of 32][4] (uint4) and group sums [8 slots][NG]
+    // (float); then one zero A entry set per wavefront.  A slot's 32 entries are followed by one unused entry: the
+    // four lanes of a 16-lane row that read A entries (slots 4 st .. 4 st + 3, same offset inside the slot) would
+    // otherwise be 512 bytes apart, on the same banks.
+    // (Where the lanes off the diagonal read their zeros made no difference: one set of four entries for all.)
+    const int a_per_col = nslot * kSlotStride;
+    const int col_stride = a_per_col + SETS * NG;
+    uint4* zeros = smem + (size_t)nblocks * col_stride;  // 4 entries, shared by all wavefronts
+
+    // ---- this wavefront's share of the staging: block columns wave, wave + NW, ...; a pass covers two slots
+    const int quad = lane & 31, sl_in_pass = lane >> 5;
+    const int ncols_w = wave < nblocks ? (nblocks - wave + NW - 1) / NW : 0;
+    const int npass = ncols_w * 4;
+    auto x_load = [&](int pass) __attribute__((always_inline)) {
+        const int ci = pass >> 2;
+        const int s = min((pass & 3) * 2 + sl_in_pass, nslot - 1);
+        return *reinterpret_cast<const uint4*>(xbytes + (size_t)(wave + NW * ci) * 512 + ((uint32_t)s * (uint32_t)K + (uint32_t)quad * 8u) * 2u);
+    };
+    constexpr int XP = 4;
+    uint4 px[XP];
+#pragma unroll
+    for (int p = 0; p < XP; ++p) {
+        px[p] = uint4{0, 0, 0, 0};
+        if (p < npass) px[p] = x_load(p);
+    }
+
+    // ---- unit fetch cursor: the units of a tile are adjacent; past the end it stays on the last unit
+    const size_t tile_bytes = (size_t)nblocks * UB;
+    const ptrdiff_t pair_delta = PAIR ? pr.W2 - Wm : 0;
+    const uint8_t* f_tile = Wm + (size_t)(tile0 + min(wave, max(tiles_real - 1, 0))) * tile_bytes;
+    const uint8_t* f_ptr = f_tile;
+    int f_col = 0, f_phase = 0, f_left = nitems;
+    const uint32_t off_c = 16u * lane, off_h = (uint32_t)tiled_header_offset(FMT, n, 0);
+    auto fetch = [&](uint4 (&cc)[NC], uint4 (&hd)[1]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NC; ++i) cc[i] = stream_load16(f_ptr + off_c + 1024 * i);
+        hd[0] = stream_load16(f_ptr + off_h);
+        if (--f_left > 0) {
+            f_ptr += UB;
+            if (++f_col == nblocks) {
+                f_col = 0;
+                if (PAIR && f_phase == 0) {
+                    f_phase = 1;
+                    f_ptr = f_tile + pair_delta;
+                } else {
+                    f_phase = 0;
+                    f_tile += (size_t)NW * tile_bytes;
+                    f_ptr = f_tile;
+                }
+            }
+        }
+    };
+    uint4 cc[WD][NC], hd[WD][1];
+#pragma unroll
+    for (int u = 0; u < WD; ++u) fetch(cc[u], hd[u]);
+
+    // ---- stage: bf16 in nibble-pair order, group sums beside them (times -OFFS where that is all they are used for)
+    const uint32_t ONES = 0x3F803F80u;
+    if (tid < 4) zeros[tid] = uint4{0, 0, 0, 0};
+    auto stage = [&](int pass, uint4 v) __attribute__((always_inline)) {
+        const int ci = pass >> 2;
+        const int s = (pass & 3) * 2 + sl_in_pass;
+        uint4* col = smem + (size_t)(wave + NW * ci) * col_stride;
+        float* colX = reinterpret_cast<float*>(col + a_per_col);
+        float sum = 0.0f;
+        if (s < nslot) {
+            const uint4 p = pair_permute(v);
+            col[s * kSlotStride + quad] = p;
+            sum = dot2(ONES, p.x, 0.0f);
+            sum = dot2(ONES, p.y, sum);
+            sum = dot2(ONES, p.z, sum);
+            sum = dot2(ONES, p.w, sum);
+        }
+        sum = dpp_add<0xB1>(sum);
+        sum = dpp_add<0x4E>(sum);
+        if ((quad & 3) == 0) colX[s * NG + quad / 4] = XPRE ? -F::OFFS * sum : sum;  // zero for an unused slot
+    };
+#pragma unroll
+    for (int p = 0; p < XP; ++p)
+        if (p < npass) stage(p, px[p]);
+    for (int p = XP; p < npass; ++p) stage(p, x_load(p));
+    __syncthreads();
+    if (nitems == 0) return;
+
+    const int s_a = n >> 2, c_a = n & 3;
+    const uint32_t M = 0x000F000Fu;
+    uint32_t C = 0x43004300u;
+    asm volatile("" : "+v"(C));
+    // per-lane offsets of the A entries inside a block column (or the zero entries for a lane off the diagonal)
+    const uint4* asrc[SETS][2];
+    ptrdiff_t astep[SETS];  // what a block column adds to the pointer (0 for the zero entries)
+#pragma unroll
+    for (int st = 0; st < SETS; ++st) {
+        const bool live = (c_a == q) && (4 * st + s_a < nslot);
+        astep[st] = live ? col_stride : 0;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) asrc[st][h] = live ? smem + (4 * st + s_a) * kSlotStride + h * 16 + q * 4 : zeros;
+    }
+    const float* xsrc = reinterpret_cast<const float*>(smem + a_per_col) + q * NG;  // group sums of slot q of set 0
+
+    int c_col = 0, c_phase = 0, c_tile = wave;
+    float acc[SETS] = {0.0f, 0.0f}, gacc[SETS] = {0.0f, 0.0f};
+    auto consume = [&](int u) __attribute__((always_inline)) {
+        const float* colX = xsrc + (size_t)c_col * col_stride * 4;
+        float xv[SETS][2][PER];
+#pragma unroll
+        for (int st = 0; st < SETS; ++st)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int t = 0; t < PER; t += 4) {
+                    const float4 f = *reinterpret_cast<const float4*>(colX + st * 4 * NG + h * PER + t);
+                    xv[st][h][t] = f.x; xv[st][h][t + 1] = f.y; xv[st][h][t + 2] = f.z; xv[st][h][t + 3] = f.w;
+                }
+        float res[SETS] = {0.0f, 0.0f};
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            f32x4_t DA[SETS], DB[SETS];
+#pragma unroll
+            for (int st = 0; st < SETS; ++st) {
+                const float* X = xv[st][h];
+                DB[st] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                if constexpr (XPRE) DA[st] = f32x4_t{X[0], X[1], X[2], X[3]};
+                else DA[st] = f32x4_t{-F::OFFS * X[0], -F::OFFS * X[1], -F::OFFS * X[2], -F::OFFS * X[3]};
+            }
+#pragma unroll
+            for (int pl = 0; pl < F::NP; ++pl) {
+                const uint4 cw = cc[u][2 * pl + h];
+                const uint32_t qq[4] = {cw.x, cw.y, cw.z, cw.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t v = qq[j];
+                    const uint4 wv = {(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
+#pragma unroll
+                    for (int st = 0; st < SETS; ++st) {
+                        const uint4 afr = asrc[st][h][(size_t)c_col * astep[st] + j];
+                        if (pl == 0)
+                            DA[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, afr),
+                                                                             __builtin_bit_cast(bf16x8_t, wv), DA[st], 0, 0, 0);
+                        else
+                            DB[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, afr),
+                                                                             __builtin_bit_cast(bf16x8_t, wv), DB[st], 0, 0, 0);
+                    }
+                }
+            }
+#pragma unroll
+            for (int st = 0; st < SETS; ++st) res[st] += apply_groups<FMT>(hd[u], h, DA[st], DB[st], xv[st][h]);
+        }
+#pragma unroll
+        for (int st = 0; st < SETS; ++st) acc[st] += res[st];
+        if (++c_col == nblocks) {  // the tile is complete
+            c_col = 0;
+            if (PAIR && c_phase == 0) {
+                c_phase = 1;
+#pragma unroll
+                for (int st = 0; st < SETS; ++st) { gacc[st] = acc[st]; acc[st] = 0.0f; }
+            } else {
+                const int row = (tile0 + c_tile) * 16 + n;
+#pragma unroll
+                for (int st = 0; st < SETS; ++st) {
+                    float v = acc[st];
+                    if constexpr (PAIR) v = gacc[st] / (1.0f + expf(-gacc[st])) * v;
+                    acc[st] = 0.0f;
+                    const int slot = 4 * st + q;
+                    if (slot >= nslot || row >= nrm) continue;
+                    const size_t off = (size_t)slot * (size_t)nrm + (size_t)row;
+                    if (args.accumulate) {
+                        if (y_bf16) v += __uint_as_float((uint32_t)reinterpret_cast<const unsigned short*>(ym)[off] << 16);
+                        else v += reinterpret_cast<const float*>(ym)[off];
+                    }
+                    if (y_bf16) reinterpret_cast<unsigned short*>(ym)[off] = (unsigned short)bf16_rne(v);
+                    else reinterpret_cast<float*>(ym)[off] = v;
+                }
+                c_phase = 0;
+                c_tile += NW;
+            }
+        }
+    };
+    const int groups = (nitems + WD - 1) / WD;
+    for (int g = 1; g < groups; ++g) {
+#pragma unroll
+        for (int u = 0; u < WD; ++u) {
+            consume(u);
+            fetch(cc[u], hd[u]);
+        }
+    }
+    const int last0 = (groups - 1) * WD;
+#pragma unroll
+    for (int u = 0; u < WD; ++u)
+        if (last0 + u < nitems) consume(u);
 }
 
 // (a, off) of the four scale groups of k-step `khalf`: contribution of a group = a * D + off * X
@@ -956,7 +1203,7 @@ GemvPlan plan_gemv4(const GemvArgs& a, int nslot) {
         }
     }
     const int ncols_max = (nblocks + p.NW - 1) / p.NW;
-    const size_t x_bytes = ((size_t)p.NW * ncols_max * (nslot * 32 + p.sets * Fmt<FMT>::NG) + 4 * p.NW) * 16;
+    const size_t x_bytes = ((size_t)p.NW * ncols_max * (nslot * a_slot_stride(FMT, p.sets) + p.sets * Fmt<FMT>::NG) + 4 * p.NW) * 16;
     const size_t per_tile = (size_t)p.NW * p.sets * 256 * (a.pair ? 2 : 1);  // the paired launch keeps two cells per tile
     // tiles per workgroup: one round of workgroups over the compute units where LDS allows it;
     // every workgroup stays inside one matrix
@@ -1203,7 +1450,34 @@ int plan_grouped(int K, bool x_f32, const int* nrows, const int* nrows_x, int np
     gp->NW = p.NW; gp->T = T; gp->sets = p.sets; gp->lds = x_bytes + (size_t)T * per_tile;
     gp->x_f32 = x_f32;
     gp->pair = pair;
+    gp->rows = false;
     gp->K = K;
+    // Gate / up pairs of five to eight bf16 rows with enough tiles for every wavefront: gemvr_kernel, whose
+    // wavefronts own whole tiles.  NW wavefronts of r tile pairs each, a workgroup per compute unit if possible:
+    // the least (rounds of 256 workgroups) x (r + 1/2), then the most wavefronts at work.
+    if constexpr (kPaired<FMT>) {
+        const size_t rows_lds = ((size_t)nblocks * (nslot * kSlotStride + 2 * Fmt<FMT>::NG) + 4) * 16;
+        long tiles = 0;
+        for (int i = 0; i < nprob; ++i) tiles += (nrows[i] + 15) / 16;
+        if (pair && !x_f32 && p.sets == 2 && rows_lds <= 160 * 1024 && tiles >= 256 * 12) {
+            long best_cost = -1, best_busy = 0;
+            int best_nw = 16, best_r = 1;
+            for (int w = 16; w >= 12; --w)
+                for (int r = 1; r <= 64; ++r) {
+                    long wgs = 0;
+                    for (int i = 0; i < nprob; ++i) wgs += ((nrows[i] + 15) / 16 + w * r - 1) / (w * r);
+                    const long cost = (wgs + 255) / 256 * (2 * r + 1);
+                    const long busy = (wgs < 256 ? wgs : 256) * w;
+                    if (best_cost < 0 || cost < best_cost || (cost == best_cost && busy > best_busy)) {
+                        best_cost = cost; best_busy = busy; best_nw = w; best_r = r;
+                    }
+                }
+            gp->rows = true;
+            gp->NW = best_nw;
+            gp->T = T = best_nw * best_r;
+            gp->lds = rows_lds;
+        }
+    }
     int grid = 0;
     for (int i = 0; i < nprob; ++i) grid += ((nrows[i] + 15) / 16 + T - 1) / T;
     gp->grid = grid;
@@ -1239,7 +1513,21 @@ int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, 
             return fail(TFQ_ERR_FORMAT, "gemv group: no paired kernel for this format");
         }
     }
-    static std::atomic<bool> lds_limit_raised[8] = {};
+    static std::atomic<bool> lds_limit_raised[9] = {};
+    if (gp.rows) {
+        if constexpr (kPaired<FMT>) {
+            if (!gp.pair) return fail(TFQ_ERR_ARG, "gemv group: the tile-owning kernel serves gate / up pairs");
+            if (!lds_limit_raised[8]) {
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemvr_kernel<FMT, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
+                lds_limit_raised[8] = true;
+            }
+            hipLaunchKernelGGL((gemvr_kernel<FMT, true>), dim3(gp.grid), dim3(64 * gp.NW), gp.lds, s, k);
+            return hip_fail(hipGetLastError(), "gemv group launch");
+        } else {
+            return fail(TFQ_ERR_FORMAT, "gemv group: no paired kernel for this format");
+        }
+    }
     if (!lds_limit_raised[slot]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
@@ -1273,7 +1561,7 @@ int plan_rows16_grouped(int K, const int* nrows, int nprob, GemvGroupPlan* gp) {
             if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_t = T; NW = w; }
         }
     }
-    gp->NW = NW; gp->T = best_t; gp->sets = 4; gp->K = K; gp->x_f32 = false; gp->pair = false;
+    gp->NW = NW; gp->T = best_t; gp->sets = 4; gp->K = K; gp->x_f32 = false; gp->pair = false; gp->rows = false;
     gp->lds = (size_t)NW * 2560 + (size_t)best_t * NW * 1024;
     int grid = 0;
     for (int i = 0; i < nprob; ++i) grid += ((nrows[i] + 15) / 16 + best_t - 1) / best_t;

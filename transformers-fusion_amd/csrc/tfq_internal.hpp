@@ -411,6 +411,7 @@ struct GemvGroupPlan {
     int NW, T, sets, grid, K;
     bool x_f32;
     bool pair;  // every problem is a gate / up pair: y = silu(gate x) * (up x)
+    bool rows;  // the kernel whose wavefronts own whole tiles (many tiles per workgroup)
     size_t lds;
 };
 bool gemv_grouped_supported(int fmt);

@@ -618,16 +618,22 @@ int plan_routed(const tfq_weight* const* gate, const tfq_weight* const* up, cons
     // gate / up: the paired eight-row form where its staged rows fit, else four rows; down: sixteen rows at any K
     sh.capA = 8;
     const int nrA = (int)F, nrB = (int)D;
-    if (plan_gemv_grouped(gate[0]->fmt, (int)D, false, &nrA, &sh.capA, 1, &rp->planA, true) != TFQ_OK) {
-        sh.capA = 4;
-        if (int rc = plan_gemv_grouped(gate[0]->fmt, (int)D, false, &nrA, &sh.capA, 1, &rp->planA, true)) return rc;
+    const size_t usual = (size_t)std::min<long>(E, P);  // one problem per expert: what a decode-sized call usually has
+    {
+        const std::vector<int> nrs(usual, nrA);
+        std::vector<int> caps(usual, sh.capA);
+        if (plan_gemv_grouped(gate[0]->fmt, (int)D, false, nrs.data(), caps.data(), (int)usual, &rp->planA, true) != TFQ_OK) {
+            sh.capA = 4;
+            caps.assign(usual, sh.capA);
+            if (int rc = plan_gemv_grouped(gate[0]->fmt, (int)D, false, nrs.data(), caps.data(), (int)usual, &rp->planA, true)) return rc;
+        }
     }
     sh.capB = 16;
     {   // tiles per workgroup as for one problem per expert (what a decode-sized call usually has)
-        const std::vector<int> nrs((size_t)std::min<long>(E, P), nrB);
+        const std::vector<int> nrs(usual, nrB);
         if (int rc = plan_gemv_rows16_grouped(down[0]->fmt, (int)F, nrs.data(), (int)nrs.size(), &rp->planB)) return rc;
     }
-    sh.wgA = rp->planA.grid;  // workgroups of one problem
+    sh.wgA = (((int)F + 15) / 16 + rp->planA.T - 1) / rp->planA.T;  // workgroups of one problem
     sh.wgB = (((int)D + 15) / 16 + rp->planB.T - 1) / rp->planB.T;
     // an expert's last chunk may be short: at most one more problem per expert that has pairs than P / cap
     sh.maxA = (int)std::min<long>(P, (long)std::min<long>(E, P) + P / sh.capA);
