@@ -145,6 +145,29 @@ def test_moe_ffn_many_tokens_per_expert(O, tfq, gpu, fmt, xdt, mid_bf16, tol):
         W.close()
 
 
+@pytest.mark.parametrize("fmt", ["B32S4", "Q_G_8", "Q_G_3"])
+def test_moe_ffn_prefill_sized_with_uneven_experts(O, tfq, gpu, fmt):
+    """A prefill-sized call (bf16 rows and mid activations: the experts' products are grouped launches of the
+    matrix-core tile kernel) in which one expert holds hundreds of rows (two token tiles), others a few dozen, one
+    a handful and one none."""
+    import torch
+    E, Ktop, T, D, F = 6, 2, 300, 256, 512
+    gate, up, down, hg, hu, hd = _experts(O, tfq, fmt, E, D, F, 1300)
+    logits = O.rng_normal(54, T * E, 1.0).reshape(T, E)
+    logits[:, 1] += 6.0      # every token picks expert 1 first: 300 rows
+    logits[:, 4] -= 20.0     # nobody picks expert 4
+    logits[:, 5] -= 3.5      # a handful pick expert 5
+    _, idx, w = O.softmax_topk(logits, Ktop)
+    counts = [int((idx == e).sum()) for e in range(E)]
+    assert counts[1] == T and counts[4] == 0 and 0 < counts[5] <= 16, counts
+    x = O.bf16_round(O.rng_normal(55, T * D, 1.0).reshape(T, D))
+    ref = O.moe_ffn(fmt, hg, hu, hd, D, F, idx, w, x, mid_bf16=True)
+    y = tfq.moe_ffn(gate, up, down, idx, w, torch.from_numpy(x).to(gpu).bfloat16(), mid_dtype=torch.bfloat16).cpu().numpy()
+    assert rel_err(y, ref) <= 1e-2
+    for W in gate + up + down:
+        W.close()
+
+
 @pytest.mark.parametrize("fmt", ["B32S4", "B32S8"])
 def test_moe_ffn_long_down_rows_five_to_sixteen(O, tfq, gpu, fmt):
     """Experts with five to sixteen tokens and a down product too long for their staged rows (K = 5120: twenty

@@ -118,6 +118,16 @@ struct GemmArgs {
     int tiles_m, tiles_n;
     int ksplit;      // workgroups per output tile: each walks K / ksplit and writes an fp32 partial tile
     float* partial;  // [ksplit][M][N] when ksplit > 1
+    // A grouped launch (several products, e.g. the experts of a mixture layer, in one grid): the fields above
+    // come from entry group_map[workgroup] of group_table instead, and the workgroup index counts from the
+    // entry's first workgroup.  Null for a plain launch.
+    const void* group_table;
+    const int* group_map;
+};
+struct GemmGroupEntry {
+    GemmArgs a;
+    int wg_first;  // a multiple of 8: workgroup -> XCD stays what the tile order assumes
+    int pad;
 };
 
 // (a, c) of group g (0..7) of a block from its 16-byte header: weight = a * code + c
@@ -141,7 +151,14 @@ __device__ __forceinline__ void group_coeffs(uint4 h, int g, float& a, float& c)
 }
 
 template <int FMT, int BN, int NT, bool PP>
-__global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
+__global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args_in) {
+    GemmArgs args = args_in;
+    int wg_base = 0;
+    if (args_in.group_table != nullptr) {  // uniform: scalar loads of the entry
+        const GemmGroupEntry* entry = static_cast<const GemmGroupEntry*>(args_in.group_table) + args_in.group_map[blockIdx.x];
+        args = entry->a;
+        wg_base = entry->wg_first;
+    }
     constexpr int XL = BM * 4 / NT;     // activation copies per thread and step (rows NT / 4 apart)
     constexpr int BNA = BN > 128 ? 256 : 128;  // rows of the strip's LDS buffers and of the decode (224: the last 32 are spare)
     constexpr int WROWS = BNA * 4 / NT;        // weight rows decoded per thread and step (rows NT / 4 apart)
@@ -166,7 +183,7 @@ __global__ __launch_bounds__(NT) void gemm4_kernel(GemmArgs args) {
     // XCD is given a contiguous run of the token-tile-major work list: the workgroups that run
     // together on an XCD walk the same 256 token rows and share them through that XCD's L2, while
     // the packed weight strips stream from HBM.
-    const int wg = blockIdx.x;
+    const int wg = blockIdx.x - wg_base;
     const int xcd = wg & 7, slot = wg >> 3;
     // (with K split over several workgroups per tile, a K range of a token tile counts as a tile of its own)
     const int S = args.ksplit;
@@ -530,11 +547,108 @@ GemmPlan plan_for(const tfq_weight* w, int M, size_t scratch_bytes) {
     }
 }
 
+// ---- grouped launch: products of one format and one N x K with their own X, Y and row count in one grid
+template <int FMT, int BN>
+int run_tiles_grouped(const GemmGroupPlan& gp, const void* d_table, const int* d_map, hipStream_t s) {
+    constexpr int NT = 512;
+    constexpr size_t lds = (size_t)(4 * BM * 8 + 2 * (BN > 128 ? 256 : 128) * 4) * 16;
+    using Kernel = void (*)(GemmArgs);
+    const Kernel kern = gp.pp ? gemm4_kernel<FMT, BN, NT, true> : gemm4_kernel<FMT, BN, NT, false>;
+    static std::atomic<bool> lds_limit_raised[2] = {};
+    if (!lds_limit_raised[gp.pp]) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
+        lds_limit_raised[gp.pp] = true;
+    }
+    GemmArgs a{};
+    a.group_table = d_table;
+    a.group_map = d_map;
+    hipLaunchKernelGGL(kern, dim3(gp.grid), dim3(NT), lds, s, a);
+    return hip_fail(hipGetLastError(), "gemm group launch");
+}
+
+template <int FMT>
+int run_grouped_fmt(const GemmGroupPlan& gp, const void* d_table, const int* d_map, hipStream_t s) {
+    if (gp.bn == 256) {
+        if constexpr (tiled_planes(FMT) == 1) return run_tiles_grouped<FMT, 256>(gp, d_table, d_map, s);
+        else return fail(TFQ_ERR_SHAPE, "gemm group: no 256-wide strips for this format");
+    }
+    return gp.bn == 224 ? run_tiles_grouped<FMT, 224>(gp, d_table, d_map, s) : run_tiles_grouped<FMT, 128>(gp, d_table, d_map, s);
+}
+
 bool tile_kernel_serves(const tfq_weight* w, int x_dtype, int M) {
     return w->layout == TFQ_LAYOUT_TILED16 && tiled_header_bytes(w->fmt) == 16 && x_dtype == TFQ_BF16 && M > 16;
 }
 
 }  // namespace
+
+bool gemm_grouped_supported(const tfq_weight* w) {
+    if (w->layout != TFQ_LAYOUT_TILED16 || tiled_header_bytes(w->fmt) != 16) return false;
+    if (w->N > 0x7FFFFFF0 || w->K > 0x7FFFFFF0 || w->dev_bytes >= 0xFFFFF000ull) return false;
+    switch (canonical(w->fmt)) {
+        case TFQ_Q_G_4: case TFQ_B32S4: case TFQ_Q_G_3: case TFQ_B32S8: case TFQ_Q_G_8: case TFQ_Q_8: return true;
+        default: return false;
+    }
+}
+
+size_t gemm_group_entry_bytes() { return sizeof(GemmGroupEntry); }
+
+// Strip width of a grouped launch: the least (rounds of 256 workgroups) x (time of a step at that width), the
+// constants of plan_tiles.  No K split: the problems together are expected to fill the compute units.
+int plan_gemm_grouped(int fmt, const int* Ms, int nprob, int64_t N, int64_t K, GemmGroupPlan* gp) {
+    if (nprob <= 0) return fail(TFQ_ERR_ARG, "gemm group: no problems");
+    const int f = canonical(fmt);
+    const bool two_planes = tiled_planes(f) == 2, affine = f == TFQ_Q_G_4 || f == TFQ_Q_G_3;
+    const struct { int bn; double step; } cand[3] = {{256, 0.98}, {224, affine ? 1.0 : 0.90}, {128, 0.60}};
+    double best = 1e30;
+    for (const auto& c : cand) {
+        if (c.bn == 256 && two_planes) continue;
+        long wgs = 0;
+        for (int i = 0; i < nprob; ++i) {
+            if ((size_t)Ms[i] * (size_t)K * 2 >= 0xFFFFF000ull) return fail(TFQ_ERR_SHAPE, "gemm group: a problem's activations exceed 4 GiB");
+            const long tiles = (long)((Ms[i] + BM - 1) / BM) * (long)((N + c.bn - 1) / c.bn);
+            wgs += 8 * ((tiles + 7) / 8);
+        }
+        const double occ = wgs >= 256 ? 1.0 : (double)wgs / 256.0;
+        const double us = (double)((wgs + 255) / 256) * c.step * (0.65 + 0.35 * occ);
+        if (us < best) { best = us; gp->bn = c.bn; gp->grid = (int)wgs; gp->pp = wgs >= 256; }
+    }
+    return TFQ_OK;
+}
+
+// Host images of the entry table (nprob entries of gemm_group_entry_bytes()) and of the workgroup map (gp.grid ints)
+void fill_gemm_group(const GemmGroupPlan& gp, const tfq_weight* const* ws, const void* const* xs, void* const* ys, const int* Ms,
+                     int nprob, int y_dtype, void* table_host, int* map_host) {
+    GemmGroupEntry* t = static_cast<GemmGroupEntry*>(table_host);
+    int wg = 0;
+    for (int i = 0; i < nprob; ++i) {
+        GemmArgs a{};
+        a.W = ws[i]->dev;
+        a.X = static_cast<const unsigned short*>(xs[i]);
+        a.Y = ys[i];
+        a.M = Ms[i]; a.N = (int)ws[i]->N; a.K = (int)ws[i]->K;
+        a.y_bf16 = y_dtype == TFQ_BF16;
+        a.tiles_m = (a.M + BM - 1) / BM;
+        a.tiles_n = (a.N + gp.bn - 1) / gp.bn;
+        a.ksplit = 1;
+        const int n = 8 * ((a.tiles_m * a.tiles_n + 7) / 8);
+        t[i] = GemmGroupEntry{a, wg, 0};
+        for (int j = 0; j < n; ++j) map_host[wg + j] = i;
+        wg += n;
+    }
+}
+
+int launch_gemm_grouped(int fmt, const GemmGroupPlan& gp, const void* d_table, const int* d_map, hipStream_t s) {
+    switch (canonical(fmt)) {
+        case TFQ_Q_G_4: return run_grouped_fmt<TFQ_Q_G_4>(gp, d_table, d_map, s);
+        case TFQ_B32S4: return run_grouped_fmt<TFQ_B32S4>(gp, d_table, d_map, s);
+        case TFQ_Q_G_3: return run_grouped_fmt<TFQ_Q_G_3>(gp, d_table, d_map, s);
+        case TFQ_B32S8: return run_grouped_fmt<TFQ_B32S8>(gp, d_table, d_map, s);
+        case TFQ_Q_G_8: return run_grouped_fmt<TFQ_Q_G_8>(gp, d_table, d_map, s);
+        case TFQ_Q_8: return run_grouped_fmt<TFQ_Q_8>(gp, d_table, d_map, s);
+        default: return fail(TFQ_ERR_FORMAT, "gemm group: no tile kernel for this format");
+    }
+}
 
 // Few tokens make few workgroups for the tile kernel, while the batched decode kernel reads the matrix once
 // per 16 rows with every compute unit busy: a 16-row pass costs (us) 2.5 + 3.2 per 4096 of K (activation

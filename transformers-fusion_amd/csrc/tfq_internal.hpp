@@ -456,6 +456,19 @@ int launch_moe_ffn_capacity(const tfq_weight* const* gate, const tfq_weight* con
 int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
                 hipStream_t s, void* scratch = nullptr, size_t scratch_bytes = 0);
 size_t gemm_scratch_bytes(const tfq_weight* w, int x_dtype, int M);
+// Grouped form of the prefill tile kernel: several products over matrices of one format and one N x K, each with
+// its own bf16 X, its own Y and row count, in one grid (the experts of a mixture layer at prefill sizes).  Entry
+// table and workgroup map are built on the host (fill_gemm_group) and copied to the device by the caller.
+struct GemmGroupPlan {
+    int bn, grid;
+    bool pp;
+};
+bool gemm_grouped_supported(const tfq_weight* w);
+size_t gemm_group_entry_bytes();
+int plan_gemm_grouped(int fmt, const int* Ms, int nprob, int64_t N, int64_t K, GemmGroupPlan* gp);
+void fill_gemm_group(const GemmGroupPlan& gp, const tfq_weight* const* ws, const void* const* xs, void* const* ys, const int* Ms,
+                     int nprob, int y_dtype, void* table_host, int* map_host);
+int launch_gemm_grouped(int fmt, const GemmGroupPlan& gp, const void* d_table, const int* d_map, hipStream_t s);
 // launch_gemm with the K-split scratch in a fixed device array of the library (no allocation in the call)
 // fp32 X with more than 16 rows: X split into a bf16 high and low part in `work` (gemm_f32_split_bytes), the 2 M bf16
 // rows through the 16-row decode kernel, the two products of a row added

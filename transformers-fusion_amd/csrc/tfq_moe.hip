@@ -389,16 +389,50 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
             return rc;
         }
     }
-    const size_t eb = gemv_group_entry_bytes();
+    // A prefill-sized call with bf16 rows and bf16 mid activations: the experts' gate and up products are ONE grouped
+    // launch of the tile kernel and their down products another, instead of three launches per expert, each of
+    // which fills a fraction of the compute units (512 rows x 14336 weight rows are 128 tiles of 224).
+    bool tall_grouped = tall && x_dtype == TFQ_BF16 && mid_dtype == TFQ_BF16;
+    for (int e = 0; e < E && tall_grouped; ++e)
+        tall_grouped = gemm_grouped_supported(gate[e]) && gemm_grouped_supported(up[e]) && gemm_grouped_supported(down[e]) &&
+                       canonical(gate[e]->fmt) == canonical(gate[0]->fmt) && canonical(up[e]->fmt) == canonical(gate[0]->fmt) &&
+                       canonical(down[e]->fmt) == canonical(down[0]->fmt);
+    GemmGroupPlan gplanA{}, gplanB{};
+    std::vector<int> mA, mB;
+    if (tall_grouped) {
+        for (int e = 0; e < E; ++e) {
+            const int p0 = first[e], nt = first[e + 1] - first[e];
+            if (nt <= 0) continue;
+            for (int half = 0; half < 2; ++half) {
+                wA.push_back(half ? up[e] : gate[e]);
+                xA.push_back(ws.xe + (size_t)p0 * D * xe_bytes);
+                yA.push_back((half ? ws.u : ws.g) + (size_t)p0 * F);
+                mA.push_back(nt);
+            }
+            wB.push_back(down[e]);
+            xB.push_back(ws.h + (size_t)p0 * F * he);
+            yB.push_back(ws.o + (size_t)p0 * D);
+            mB.push_back(nt);
+        }
+        if (int rc = plan_gemm_grouped(gate[0]->fmt, mA.data(), (int)mA.size(), F, D, &gplanA)) return rc;
+        if (int rc = plan_gemm_grouped(down[0]->fmt, mB.data(), (int)mB.size(), D, F, &gplanB)) return rc;
+    }
+    const size_t eb = tall_grouped ? gemm_group_entry_bytes() : gemv_group_entry_bytes();
+    const size_t gridA = tall_grouped ? (size_t)gplanA.grid : (size_t)planA.grid, gridB = tall_grouped ? (size_t)gplanB.grid : (size_t)planB.grid;
     const size_t base_ints = ((size_t)3 * P + T + 1 + 1) & ~(size_t)1;  // tables start 8-byte aligned
     const size_t tabA = base_ints * 4, tabB = tabA + wA.size() * eb;
-    const size_t mapA = tabB + wB.size() * eb, mapB = mapA + (size_t)planA.grid * 4;
-    const size_t list_bytes = grouped ? mapB + (size_t)planB.grid * 4 : base_ints * 4;
+    const size_t mapA = tabB + wB.size() * eb, mapB = mapA + gridA * 4;
+    const size_t list_bytes = grouped || tall_grouped ? mapB + gridB * 4 : base_ints * 4;
     if (list_bytes > ws.list_bytes) return fail(TFQ_ERR_SHAPE, "moe: routing tables exceed the workspace");
     std::lock_guard<std::mutex> list_lock(g_list_mutex);
     ListSlot* slot = nullptr;
     if (int rc = acquire_list_slot(list_bytes + 8, &slot)) return rc;
     int* const lists = static_cast<int*>(slot->host);
+    if (tall_grouped) {
+        uint8_t* lb = reinterpret_cast<uint8_t*>(lists);
+        fill_gemm_group(gplanA, wA.data(), xA.data(), yA.data(), mA.data(), (int)wA.size(), TFQ_F32, lb + tabA, reinterpret_cast<int*>(lb + mapA));
+        fill_gemm_group(gplanB, wB.data(), xB.data(), yB.data(), mB.data(), (int)wB.size(), TFQ_F32, lb + tabB, reinterpret_cast<int*>(lb + mapB));
+    }
     if (grouped) {
         uint8_t* lb = reinterpret_cast<uint8_t*>(lists);
         fill_gemv_group(planA, wA.data(), xA.data(), yA.data(), rA.data(), (int)wA.size(), lb + tabA, reinterpret_cast<int*>(lb + mapA), wA2.data());
@@ -432,7 +466,10 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
     if (grouped) {
         if (int rc = launch_gemv_grouped(gate[0]->fmt, planA, d_lists + tabA, reinterpret_cast<const int*>(d_lists + mapA), mid_dtype, s)) return rc;
     }
-    for (int e = 0; e < E && !grouped; ++e) {
+    if (tall_grouped) {
+        if (int rc = launch_gemm_grouped(gate[0]->fmt, gplanA, d_lists + tabA, reinterpret_cast<const int*>(d_lists + mapA), s)) return rc;
+    }
+    for (int e = 0; e < E && !grouped && !tall_grouped; ++e) {
         const int p0 = first[e], nt = first[e + 1] - first[e];
         if (nt > 16) {  // the prefill entry: matrix cores for bf16 rows, 16-row slices otherwise
             if (int rc = launch_gemm(gate[e], ws.xe + (size_t)p0 * D * xe_bytes, x_dtype, nt, ws.g + (size_t)p0 * F, TFQ_F32, s, ws.scratch, ws.scratch_bytes)) return rc;
@@ -460,7 +497,10 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
             return rc;
         }
     }
-    for (int e = 0; e < E && !grouped; ++e) {
+    if (tall_grouped) {
+        if (int rc = launch_gemm_grouped(down[0]->fmt, gplanB, d_lists + tabB, reinterpret_cast<const int*>(d_lists + mapB), s)) return rc;
+    }
+    for (int e = 0; e < E && !grouped && !tall_grouped; ++e) {
         const int p0 = first[e], nt = first[e + 1] - first[e];
         if (nt <= 0) continue;
         // sixteen rows or fewer take the decode kernels inside
