@@ -540,8 +540,10 @@ __global__ __launch_bounds__(1024) void routed_lists_kernel(const int32_t* __res
                                                             int* __restrict__ tok_first, int* __restrict__ tok_pairs,
                                                             RoutedShape sh, const uint8_t* const* __restrict__ ptrs, const uint8_t* xe, uint8_t* h, uint8_t* o,
                                                             GemvProb* __restrict__ tabA, int* __restrict__ mapA,
-                                                            GemvProb* __restrict__ tabB, int* __restrict__ mapB) {
+                                                            GemvProb* __restrict__ tabB, int* __restrict__ mapB,
+                                                            const uint4* __restrict__ x, int row_u4) {
     __shared__ int s_idx[kRoutedMaxPairs];
+    __shared__ int s_tok[kRoutedMaxPairs];
     __shared__ int s_first[257];
     __shared__ int s_cnt[256];
     __shared__ int s_pair[kRoutedMaxPairs];
@@ -584,8 +586,17 @@ __global__ __launch_bounds__(1024) void routed_lists_kernel(const int32_t* __res
         rows[p] = t;
         wts[p] = wt;
         s_pair[sl] = p;
+        s_tok[p] = t;
     }
     __syncthreads();
+    // A decode-sized call: the pairs' activation rows are gathered here as well (x != null), which saves a launch
+    if (x != nullptr) {
+        uint4* dst = reinterpret_cast<uint4*>(const_cast<uint8_t*>(xe));
+        for (int i = tid; i < total * row_u4; i += blockDim.x) {
+            const int r = i / row_u4, c = i - r * row_u4;
+            dst[i] = x[(size_t)s_tok[r] * row_u4 + c];
+        }
+    }
     for (int t = tid; t <= T; t += blockDim.x) tok_first[t] = t * Ktop;
     for (int t = tid; t < T; t += blockDim.x) {  // the pairs of a token in ascending order (selection, Ktop is small)
         int prev = -1;
@@ -734,11 +745,14 @@ int launch_moe_ffn_routed(const tfq_weight* const* gate, const tfq_weight* const
     GemvProb* tabB = reinterpret_cast<GemvProb*>(lists + rp.off_tabB);
     int* mapA = reinterpret_cast<int*>(lists + rp.off_mapA);
     int* mapB = reinterpret_cast<int*>(lists + rp.off_mapB);
-    hipLaunchKernelGGL(routed_lists_kernel, dim3(1), dim3(1024), 0, s, d_topk_idx, d_topk_w, T, Ktop, E, d_first, d_rows, d_w, d_tokf, d_tokp,
-                       rp.sh, static_cast<const uint8_t* const*>(d_expert_table), (const uint8_t*)xe, h, o, tabA, mapA, tabB, mapB);
     const int row_u4 = (int)(D * 2 / 16);
     const int64_t ng = (int64_t)P * row_u4;
-    hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)((ng + 255) / 256)), dim3(256), 0, s, (const uint4*)x, (uint4*)xe, (const int*)d_rows, (int)P, row_u4);
+    const bool fuse_gather = ng * 16 <= 512 * 1024;  // up to 512 KB of rows ride in the list kernel's one workgroup
+    hipLaunchKernelGGL(routed_lists_kernel, dim3(1), dim3(1024), 0, s, d_topk_idx, d_topk_w, T, Ktop, E, d_first, d_rows, d_w, d_tokf, d_tokp,
+                       rp.sh, static_cast<const uint8_t* const*>(d_expert_table), (const uint8_t*)xe, h, o, tabA, mapA, tabB, mapB,
+                       fuse_gather ? (const uint4*)x : nullptr, row_u4);
+    if (!fuse_gather)
+        hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)((ng + 255) / 256)), dim3(256), 0, s, (const uint4*)x, (uint4*)xe, (const int*)d_rows, (int)P, row_u4);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return hip_fail(e, "moe routed launch");
     if (int rc = launch_gemv_grouped(gate[0]->fmt, rp.planA, tabA, mapA, TFQ_BF16, s)) return rc;
     if (int rc = launch_gemv_rows16_grouped(down[0]->fmt, rp.planB, tabB, mapB, TFQ_F32, s)) return rc;
