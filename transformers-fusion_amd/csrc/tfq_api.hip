@@ -585,19 +585,9 @@ int tfq_matmul_host(const tfq_weight_t* w, const float* X, float* Y, int B) {
     hipError_t e = hipMalloc(&dy, yb);
     if (e != hipSuccess) { (void)hipFree(dx); return hip_fail(e, "hipMalloc"); }
     int rc = hip_fail(hipMemcpy(dx, X, xb, hipMemcpyHostToDevice), "hipMemcpy H2D");
-    if (!rc && B > 16 && gemm_f32_split_serves(w, B)) {
-        // many fp32 rows: their bf16 high and low parts through the 16-row decode kernel (eight fp32 rows per pass over
-        // the weights instead of two)
-        void* work = nullptr;
-        const size_t wb = gemm_f32_split_bytes(w, B);
-        e = hipMalloc(&work, wb);
-        if (e != hipSuccess) rc = hip_fail(e, "hipMalloc");
-        if (!rc) rc = launch_gemm_f32_split(w, dx, B, dy, work, wb, nullptr);
-        if (!rc) rc = hip_fail(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
-        (void)hipFree(work);
-    } else if (!rc) {
-        rc = B <= 16 ? launch_gemv(w, dx, TFQ_F32, B, dy, TFQ_F32, nullptr) : launch_gemm(w, dx, TFQ_F32, B, dy, TFQ_F32, nullptr);
-    }
+    // more than sixteen fp32 rows: slices of sixteen through the decode path, whose sixteen-row kernel takes eight fp32
+    // rows (their bf16 high and low parts) per pass over the weights
+    if (!rc) rc = B <= 16 ? launch_gemv(w, dx, TFQ_F32, B, dy, TFQ_F32, nullptr) : launch_gemm(w, dx, TFQ_F32, B, dy, TFQ_F32, nullptr);
     if (!rc) rc = hip_fail(hipMemcpy(Y, dy, yb, hipMemcpyDeviceToHost), "hipMemcpy D2H");
     (void)hipFree(dx);
     (void)hipFree(dy);

@@ -695,56 +695,6 @@ int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y,
     return TFQ_OK;
 }
 
-// ---- fp32 activations, more than 16 rows
-// The tile kernel rounds the dequantized weights to bf16, which an fp32 product may not (its tolerance is 1e-3);
-// the decode kernels multiply the integer codes and apply the scales in fp32, but take two fp32 rows per pass
-// over the packed weights.  Here an fp32 X is split on the device into a bf16 high part and the bf16 of what is
-// left (16 significant bits of x together, exactly what the decode kernels do with an fp32 row), the 2 M bf16
-// rows go through the 16-row decode kernel, and the two products of a row are added: one pass over the weights
-// per eight fp32 rows instead of one per two.
-namespace {
-__global__ __launch_bounds__(256) void split_hi_lo_kernel(const float* __restrict__ x, unsigned short* __restrict__ hi,
-                                                          unsigned short* __restrict__ lo, long long n) {
-    const long long stride = (long long)gridDim.x * blockDim.x;
-    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-        const float v = x[i];
-        const uint32_t h = bf16_rne(v);
-        hi[i] = (unsigned short)h;
-        lo[i] = (unsigned short)bf16_rne(v - __uint_as_float(h << 16));
-    }
-}
-__global__ __launch_bounds__(256) void add_pairs_kernel(float* __restrict__ y, const float* __restrict__ a, const float* __restrict__ b, long long n) {
-    const long long stride = (long long)gridDim.x * blockDim.x;
-    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) y[i] = a[i] + b[i];
-}
-}  // namespace
-
-bool gemm_f32_split_serves(const tfq_weight* w, int M) { return M > 16 && w->layout == TFQ_LAYOUT_TILED16 && gemv_rows16_supported(w->fmt); }
-
-size_t gemm_f32_split_bytes(const tfq_weight* w, int M) {
-    // 2 M bf16 rows of X, 2 M fp32 rows of products, each part 256-byte aligned
-    const size_t planes = ((size_t)2 * M * (size_t)w->K * 2 + 255) & ~(size_t)255;
-    const size_t prods = ((size_t)2 * M * (size_t)w->N * 4 + 255) & ~(size_t)255;
-    return planes + prods;
-}
-
-int launch_gemm_f32_split(const tfq_weight* w, const float* x, int M, float* y, void* work, size_t work_bytes, hipStream_t s) {
-    if (!gemm_f32_split_serves(w, M)) return fail(TFQ_ERR_FORMAT, "gemm: no 16-row decode kernel for this matrix");
-    if (!work || work_bytes < gemm_f32_split_bytes(w, M)) return fail(TFQ_ERR_SHAPE, "gemm: work area smaller than gemm_f32_split_bytes");
-    const size_t planes = ((size_t)2 * M * (size_t)w->K * 2 + 255) & ~(size_t)255;
-    unsigned short* xs = static_cast<unsigned short*>(work);  // rows 0..M-1 high parts, M..2M-1 low parts
-    float* ys = reinterpret_cast<float*>(static_cast<uint8_t*>(work) + planes);
-    const long long nx = (long long)M * w->K, ny = (long long)M * w->N;
-    hipLaunchKernelGGL(split_hi_lo_kernel, dim3((unsigned)std::min<long long>((nx + 255) / 256, 8192)), dim3(256), 0, s, x, xs, xs + nx, nx);
-    if (hipError_t e = hipGetLastError(); e != hipSuccess) return hip_fail(e, "gemm split launch");
-    for (int m0 = 0; m0 < 2 * M; m0 += 16) {
-        const int mb = 2 * M - m0 < 16 ? 2 * M - m0 : 16;
-        if (int rc = launch_gemv(w, xs + (size_t)m0 * w->K, TFQ_BF16, mb, ys + (size_t)m0 * w->N, TFQ_F32, s)) return rc;
-    }
-    hipLaunchKernelGGL(add_pairs_kernel, dim3((unsigned)std::min<long long>((ny + 255) / 256, 8192)), dim3(256), 0, s, y, ys, ys + ny, ny);
-    return hip_fail(hipGetLastError(), "gemm add launch");
-}
-
 // ---- the prefill product for callers that cannot allocate
 // The K split of the tile kernel keeps its fp32 partial tiles in scratch memory.  tfq_gemm_ws takes that memory
 // from the caller; here it is a fixed array in the library's device image, so a call allocates nothing (no

@@ -470,11 +470,6 @@ void fill_gemm_group(const GemmGroupPlan& gp, const tfq_weight* const* ws, const
                      int nprob, int y_dtype, void* table_host, int* map_host);
 int launch_gemm_grouped(int fmt, const GemmGroupPlan& gp, const void* d_table, const int* d_map, hipStream_t s);
 // launch_gemm with the K-split scratch in a fixed device array of the library (no allocation in the call)
-// fp32 X with more than 16 rows: X split into a bf16 high and low part in `work` (gemm_f32_split_bytes), the 2 M bf16
-// rows through the 16-row decode kernel, the two products of a row added
-bool gemm_f32_split_serves(const tfq_weight* w, int M);
-size_t gemm_f32_split_bytes(const tfq_weight* w, int M);
-int launch_gemm_f32_split(const tfq_weight* w, const float* x, int M, float* y, void* work, size_t work_bytes, hipStream_t s);
 int launch_gemm_static(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype, hipStream_t s);
 size_t gemm_static_scratch_bytes();
 inline size_t gemm_scratch_bound(size_t rows, size_t cols) {
