@@ -250,7 +250,8 @@ int tfq_gemv_multi(const tfq_weight_t* const* ws, int count, const void* x, int 
                    void* const* ys, int y_dtype, tfq_stream_t stream);
 /* tfq_gemv_multi with an elementwise step of the reference engine applied to the activations while the
  * kernel stages them, so the step costs no launch and no round trip through memory.  With RMSNORM or SWIGLU
- * x is fp32 [B][K], B <= 16 (two rows ride in one pass over the weights, like every fp32 input); with
+ * x is fp32 [B][K], B <= 16 (two rows ride in one pass over the weights; fp32 rows without a prologue take
+ * four or eight per pass); with
  * TFQ_PRO_NONE (only `accumulate` set) x may be bf16 too.
  *   TFQ_PRO_RMSNORM  x * rsqrt(mean(x^2) + eps) * gamma, or * (1 + gamma) with gamma_plus_one, the form of
  *                    Qwen35Engine::rmsnorm (src/adapters/tools/qwen35_engine.cpp:46-51), in front of the
