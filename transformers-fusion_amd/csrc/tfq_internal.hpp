@@ -404,7 +404,7 @@ struct GemvProb {
     int nrows;
     int nslot;
     int wg_first;  // first workgroup of this problem
-    int pad;
+    int tiles;     // tiles per workgroup of this problem where a table built on the device chooses them (0: the launch's)
 };
 
 struct GemvGroupPlan {

@@ -355,7 +355,18 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
         // gate and up of an expert are one problem: the kernel walks the same tiles of both and its epilogue writes
         // silu(gate x) * (up x) in the mid dtype (ExpertFFN::forward, src/model/moe_core.cpp:78-92), so the two
         // products never go to memory and no elementwise launch follows
-        const int capA = chunk_cap(gate[0]->fmt, (int)D, x_dtype == TFQ_F32, (int)F, true);
+        int capA = chunk_cap(gate[0]->fmt, (int)D, x_dtype == TFQ_F32, (int)F, true);
+        if (capA > 8) {
+            // An expert with nine to sixteen rows: sixteen-row chunks would take every problem of the launch to the
+            // four-set kernel (eight wavefronts, 3.5-4.5 TB/s).  Where chunks of eight reach the kernel whose
+            // wavefronts own whole tiles, reading that expert's pair of matrices twice at 6 TB/s is the cheaper launch
+            // (16 tokens, top-2 of 8 experts, one expert with nine rows: 249 us per call with sixteen-row chunks).
+            std::vector<int> n8, r8;
+            for (int e = 0; e < E; ++e)
+                for (int nt = first[e + 1] - first[e], b0 = 0; b0 < nt; b0 += 8) { n8.push_back((int)F); r8.push_back(std::min(8, nt - b0)); }
+            GemvGroupPlan p8{};
+            if (plan_gemv_grouped(gate[0]->fmt, (int)D, false, n8.data(), r8.data(), (int)n8.size(), &p8, true) == TFQ_OK && p8.rows) capA = 8;
+        }
         int capB = chunk_cap(down[0]->fmt, (int)F, mid_dtype == TFQ_F32, (int)D, false);
         // Down at a long K: the staged activations of more than four rows do not fit, and an expert with more
         // tokens would read its matrix once per four.  With bf16 mid activations the sixteen-row kernel (A
@@ -527,6 +538,7 @@ struct RoutedShape {
     int wgA, wgB;        // workgroups per problem
     int maxA, maxB;      // problems at most
     int nrowsA, nrowsB;  // F, D
+    int nwA, rA;         // gate / up launch in the kernel whose wavefronts own tiles: its wavefronts per workgroup and tile pairs per wavefront (nwA = 0: the other kernel)
     size_t strideXA, strideYA, strideXB, strideYB;  // bytes per activation row in the gathered / mid / output buffers
 };
 
@@ -613,15 +625,29 @@ __global__ __launch_bounds__(1024) void routed_lists_kernel(const int32_t* __res
     }
     // Problem tables and workgroup maps of the two grouped launches: an expert's rows in chunks of capA / capB.
     // ptrs = device addresses of the experts' packed matrices, [gate | up | down][E].
-    __shared__ int s_nA, s_nB;
+    __shared__ int s_nA, s_nB, s_wgA;
     if (tid == 0) {
+        // The tile-owning kernel runs a workgroup per compute unit: when a call has more problems than the plan
+        // assumed (an expert's rows in several chunks), its wavefronts take more tile pairs each, so that the
+        // workgroups still fit one round.
+        int wgA = sh.wgA, tilesA = 0;
+        if (sh.nwA) {
+            int problems = 0;
+            for (int e = 0; e < E; ++e) problems += (s_first[e + 1] - s_first[e] + sh.capA - 1) / sh.capA;
+            const int tiles = (sh.nrowsA + 15) >> 4;
+            int r = sh.rA;
+            while (r < 64 && problems * ((tiles + sh.nwA * r - 1) / (sh.nwA * r)) > 256) ++r;
+            tilesA = sh.nwA * r;
+            wgA = (tiles + tilesA - 1) / tilesA;
+        }
+        s_wgA = wgA;
         int nA = 0, nB = 0;
         for (int e = 0; e < E; ++e) {
             const int p0 = s_first[e], nt = s_first[e + 1] - p0;
             for (int b0 = 0; b0 < nt; b0 += sh.capA) {
                 const int nb = min(sh.capA, nt - b0);
                 tabA[nA] = GemvProb{ptrs[e], h + (size_t)(p0 + b0) * sh.strideYA, xe + (size_t)(p0 + b0) * sh.strideXA, ptrs[E + e],
-                                    sh.nrowsA, nb, nA * sh.wgA, 0};
+                                    sh.nrowsA, nb, nA * wgA, tilesA};
                 ++nA;
             }
             for (int b0 = 0; b0 < nt; b0 += sh.capB) {
@@ -636,7 +662,8 @@ __global__ __launch_bounds__(1024) void routed_lists_kernel(const int32_t* __res
     }
     __syncthreads();
     const int nA = s_nA, nB = s_nB;
-    for (int i = tid; i < sh.maxA * sh.wgA; i += blockDim.x) mapA[i] = i / sh.wgA < nA ? i / sh.wgA : -1;
+    const int wgA = s_wgA;  // at most sh.wgA: the grid holds the problems' workgroups
+    for (int i = tid; i < sh.maxA * sh.wgA; i += blockDim.x) mapA[i] = i / wgA < nA ? i / wgA : -1;
     for (int i = tid; i < sh.maxB * sh.wgB; i += blockDim.x) mapB[i] = i / sh.wgB < nB ? i / sh.wgB : -1;
 }
 
@@ -685,6 +712,8 @@ int plan_routed(const tfq_weight* const* gate, const tfq_weight* const* up, cons
         if (int rc = plan_gemv_rows16_grouped(down[0]->fmt, (int)F, nrs.data(), (int)nrs.size(), &rp->planB)) return rc;
     }
     sh.wgA = (((int)F + 15) / 16 + rp->planA.T - 1) / rp->planA.T;  // workgroups of one problem
+    sh.nwA = rp->planA.rows ? rp->planA.NW : 0;
+    sh.rA = rp->planA.rows ? rp->planA.T / rp->planA.NW : 0;
     sh.wgB = (((int)D + 15) / 16 + rp->planB.T - 1) / rp->planB.T;
     // an expert's last chunk may be short: at most one more problem per expert that has pairs than P / cap
     sh.maxA = (int)std::min<long>(P, (long)std::min<long>(E, P) + P / sh.capA);
