@@ -670,6 +670,7 @@ __global__ __launch_bounds__(1024) void routed_lists_kernel(const int32_t* __res
 struct RoutedPlan {
     RoutedShape sh;
     GemvGroupPlan planA, planB;
+    bool down16;  // the down launch through the sixteen-row kernel
     size_t off_first, off_rows, off_wts, off_tokf, off_tokp, off_tabA, off_tabB, off_mapA, off_mapB, list_bytes;
 };
 
@@ -694,7 +695,7 @@ int plan_routed(const tfq_weight* const* gate, const tfq_weight* const* up, cons
     sh.E = E; sh.T = T; sh.Ktop = Ktop;
     sh.nrowsA = (int)F; sh.nrowsB = (int)D;
     // gate / up: the paired eight-row form where its staged rows fit, else four rows; down: sixteen rows at any K
-    sh.capA = 8;
+    sh.capA = T <= 4 ? 4 : 8;  // an expert holds at most T rows: four or fewer take the one-set kernel
     const int nrA = (int)F, nrB = (int)D;
     const size_t usual = (size_t)std::min<long>(E, P);  // one problem per expert: what a decode-sized call usually has
     {
@@ -706,10 +707,21 @@ int plan_routed(const tfq_weight* const* gate, const tfq_weight* const* up, cons
             if (int rc = plan_gemv_grouped(gate[0]->fmt, (int)D, false, nrs.data(), caps.data(), (int)usual, &rp->planA, true)) return rc;
         }
     }
+    // down: the sixteen-row kernel at any K; a call of at most four tokens takes the staged four-row kernel where
+    // its rows fit (what tfq_moe_ffn does when no expert holds more than four rows)
     sh.capB = 16;
+    rp->down16 = true;
     {   // tiles per workgroup as for one problem per expert (what a decode-sized call usually has)
         const std::vector<int> nrs(usual, nrB);
-        if (int rc = plan_gemv_rows16_grouped(down[0]->fmt, (int)F, nrs.data(), (int)nrs.size(), &rp->planB)) return rc;
+        if (T <= 4) {
+            const std::vector<int> caps(usual, 4);
+            if (plan_gemv_grouped(down[0]->fmt, (int)F, false, nrs.data(), caps.data(), (int)usual, &rp->planB, false) == TFQ_OK) {
+                sh.capB = 4;
+                rp->down16 = false;
+            }
+        }
+        if (rp->down16)
+            if (int rc = plan_gemv_rows16_grouped(down[0]->fmt, (int)F, nrs.data(), (int)nrs.size(), &rp->planB)) return rc;
     }
     sh.wgA = (((int)F + 15) / 16 + rp->planA.T - 1) / rp->planA.T;  // workgroups of one problem
     sh.nwA = rp->planA.rows ? rp->planA.NW : 0;
@@ -784,7 +796,11 @@ int launch_moe_ffn_routed(const tfq_weight* const* gate, const tfq_weight* const
         hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)((ng + 255) / 256)), dim3(256), 0, s, (const uint4*)x, (uint4*)xe, (const int*)d_rows, (int)P, row_u4);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return hip_fail(e, "moe routed launch");
     if (int rc = launch_gemv_grouped(gate[0]->fmt, rp.planA, tabA, mapA, TFQ_BF16, s)) return rc;
-    if (int rc = launch_gemv_rows16_grouped(down[0]->fmt, rp.planB, tabB, mapB, TFQ_F32, s)) return rc;
+    if (rp.down16) {
+        if (int rc = launch_gemv_rows16_grouped(down[0]->fmt, rp.planB, tabB, mapB, TFQ_F32, s)) return rc;
+    } else if (int rc = launch_gemv_grouped(down[0]->fmt, rp.planB, tabB, mapB, TFQ_F32, s)) {
+        return rc;
+    }
     const int64_t nout = (int64_t)T * (int64_t)D;
     if (y_dtype == TFQ_BF16)
         hipLaunchKernelGGL(combine_kernel<true>, dim3((unsigned)((nout + 255) / 256)), dim3(256), 0, s, y, (const float*)o, (const int*)d_tokf, (const int*)d_tokp, (const float*)d_w, T, (int)D, 0);
