@@ -441,6 +441,33 @@ def moe_layer(tfq, torch, fmt, bpw, base, E=8, top_k=2, T=16, D=4096, F=14336, r
     out["routed_on_device"] = {"us_per_call": round(dtr * 1e6, 1), "gbs": round(nbytes / dtr / 1e9, 1),
                                "frac": round(nbytes / dtr / 1e9 / HBM_PEAK_GBS, 4),
                                "note": "routing arrays on the device, lists built there, graph replays"}
+    # one token (the decode step of a single sequence): two active experts, the same entry point
+    routed1 = tfq.RoutedMoe(gate, up, down, 1, top_k)
+    _, idx1, wts1 = tfq.moe_route(logits[:1].contiguous(), top_k)
+    x1, y1 = x[:1].contiguous(), torch.empty(1, D, device="cuda")
+    for _ in range(3):
+        routed1(idx1, wts1, x1, y1)
+    torch.cuda.synchronize()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        routed1(idx1, wts1, x1, y1)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g1 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g1):
+        routed1(idx1, wts1, x1, y1)
+    for _ in range(3):
+        g1.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        g1.replay()
+    torch.cuda.synchronize()
+    dt1 = (time.perf_counter() - t0) / reps
+    active1 = len(set(idx1.cpu().numpy().reshape(-1).tolist()))
+    nbytes1 = active1 * 3 * F * D * bpw / 8
+    out["single_token"] = {"active_experts": active1, "us_per_call": round(dt1 * 1e6, 1), "gbs": round(nbytes1 / dt1 / 1e9, 1),
+                           "frac": round(nbytes1 / dt1 / 1e9 / HBM_PEAK_GBS, 4)}
     return out
 
 
