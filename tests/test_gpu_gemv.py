@@ -47,6 +47,29 @@ def test_gemv_bf16_activations(O, tfq, gpu, fmt, N, K, B):
     W.close()
 
 
+@pytest.mark.parametrize("fmt,N,K", [("B32S4", 49195, 256), ("B32S4", 49152, 768), ("Q_G_4", 49200, 512), ("B32S8", 49195, 256),
+                                     ("Q_G_8", 49168, 256)])
+def test_gemv_tall_matrix(O, tfq, gpu, fmt, N, K):
+    """A matrix of more than 3072 row tiles (an output projection over a vocabulary) with one to eight bf16 rows
+    takes the kernel whose wavefronts own whole tiles, one workgroup per compute unit; ragged last tile, fp32 and
+    bf16 outputs, against the oracle."""
+    import torch
+    w = O.rng_normal(42, N * K, 0.02)
+    pay = O.encode_tensor(fmt, w)
+    W = tfq.Weight(fmt, N, K, pay)
+    for B in (1, 3, 4, 5, 8):
+        print(f"gemv tall {fmt} N={N} K={K} B={B}", flush=True)
+        x = O.bf16_round(O.rng_normal(43 + B, B * K, 1.0).reshape(B, K))
+        ref = O.matmul(fmt, pay, N, K, x)
+        xt = torch.from_numpy(x).to(gpu).bfloat16()
+        y = W.gemv(xt).cpu().numpy()
+        assert y.shape == (B, N)
+        assert rel_err(y, ref) <= (3e-4 if fmt in ("Q_G_8", "B32S8") else 1e-4)
+        yb = W.gemv(xt, out_dtype=torch.bfloat16).float().cpu().numpy()
+        assert rel_err(yb, ref) <= TOL_BF16
+    W.close()
+
+
 @pytest.mark.parametrize("fmt", GEMV_FORMATS)
 @pytest.mark.parametrize("N,K,B", [(64, 256, 1), (48, 2048, 1), (96, 4096, 1), (40, 1280, 4), (24, 4096, 16),
                                    (72, 2304, 3), (33, 6400, 7), (40, 14336, 5), (1040, 14336, 8), (2000, 4096, 13), (272, 8192, 3)])

@@ -553,21 +553,29 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
 // over the block columns in ascending order: deterministic, but not the order of the kernel above.
 constexpr int kSlotStride = 33;  // uint4 entries from one activation slot's A entries to the next (gemvr_kernel)
 
-template <int FMT, bool PAIR>
-__global__ __launch_bounds__(1024) void gemvr_kernel(GemvKernArgs args) {
+template <int FMT, bool PAIR, int SETS = 2, bool GROUPED = true>
+__global__ __launch_bounds__(1024) void gemvr_kernel(GemvKernArgs args, const void* __restrict__ x_arg) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
     static_assert(F::HV == 1 && F::CW == 4 && F::GS == 32, "nibble codes, 32-weight groups, a 16-byte header");
-    constexpr int SETS = 2, WD = 2;
+    static_assert(SETS == 1 || SETS == 2, "four or eight activation slots");
+    static_assert(GROUPED || !PAIR, "pairs come from a problem table");
+    constexpr int WD = 2, PASSES = 2 * SETS;  // staging passes per block column, two slots each
     constexpr int UB = tiled_unit_bytes(FMT), NC = 2 * F::NP, NG = F::NG, PER = NG / 2;
     constexpr bool XPRE = FMT == TFQ_B32S4 || F::NP == 2;
     const int K = args.K;
     const bool y_bf16 = args.y_bf16 != 0;
     const int bid = blockIdx.x;
-    const GemvProb* table = reinterpret_cast<const GemvProb*>(args.W0);
-    const int prob = reinterpret_cast<const int*>(args.W1)[bid];
-    if (prob < 0) return;  // a workgroup beyond the problems of this call (tables built on the device)
-    const GemvProb pr = table[prob];
+    // the workgroup's problem: an entry of the table of a grouped launch, or the launch's one matrix
+    GemvProb pr;
+    if constexpr (GROUPED) {
+        const GemvProb* table = reinterpret_cast<const GemvProb*>(args.W0);
+        const int prob = reinterpret_cast<const int*>(args.W1)[bid];
+        if (prob < 0) return;  // a workgroup beyond the problems of this call (tables built on the device)
+        pr = table[prob];
+    } else {
+        pr = GemvProb{args.W0, args.y0, x_arg, nullptr, args.nr0, args.nslot, 0, 0};
+    }
     const int T = pr.tiles ? pr.tiles : args.tiles_per_wg;
     const int nrm = pr.nrows, nslot = pr.nslot;
     const uint8_t* Wm = pr.W;
@@ -596,10 +604,10 @@ __global__ __launch_bounds__(1024) void gemvr_kernel(GemvKernArgs args) {
     // ---- this wavefront's share of the staging: block columns wave, wave + NW, ...; a pass covers two slots
     const int quad = lane & 31, sl_in_pass = lane >> 5;
     const int ncols_w = wave < nblocks ? (nblocks - wave + NW - 1) / NW : 0;
-    const int npass = ncols_w * 4;
+    const int npass = ncols_w * PASSES;
     auto x_load = [&](int pass) __attribute__((always_inline)) {
-        const int ci = pass >> 2;
-        const int s = min((pass & 3) * 2 + sl_in_pass, nslot - 1);
+        const int ci = pass / PASSES;
+        const int s = min((pass % PASSES) * 2 + sl_in_pass, nslot - 1);
         return *reinterpret_cast<const uint4*>(xbytes + (size_t)(wave + NW * ci) * 512 + ((uint32_t)s * (uint32_t)K + (uint32_t)quad * 8u) * 2u);
     };
     constexpr int XP = 4;
@@ -644,8 +652,8 @@ __global__ __launch_bounds__(1024) void gemvr_kernel(GemvKernArgs args) {
     const uint32_t ONES = 0x3F803F80u;
     if (tid < 4) zeros[tid] = uint4{0, 0, 0, 0};
     auto stage = [&](int pass, uint4 v) __attribute__((always_inline)) {
-        const int ci = pass >> 2;
-        const int s = (pass & 3) * 2 + sl_in_pass;
+        const int ci = pass / PASSES;
+        const int s = (pass % PASSES) * 2 + sl_in_pass;
         uint4* col = smem + (size_t)(wave + NW * ci) * col_stride;
         float* colX = reinterpret_cast<float*>(col + a_per_col);
         float sum = 0.0f;
@@ -685,7 +693,7 @@ __global__ __launch_bounds__(1024) void gemvr_kernel(GemvKernArgs args) {
     const float* xsrc = reinterpret_cast<const float*>(smem + a_per_col) + q * NG;  // group sums of slot q of set 0
 
     int c_col = 0, c_phase = 0, c_tile = wave;
-    float acc[SETS] = {0.0f, 0.0f}, gacc[SETS] = {0.0f, 0.0f};
+    float acc[SETS] = {}, gacc[SETS] = {};
     auto consume = [&](int u) __attribute__((always_inline)) {
         const float* colX = xsrc + (size_t)c_col * col_stride * 4;
         float xv[SETS][2][PER];
@@ -698,7 +706,7 @@ __global__ __launch_bounds__(1024) void gemvr_kernel(GemvKernArgs args) {
                     const float4 f = *reinterpret_cast<const float4*>(colX + st * 4 * NG + h * PER + t);
                     xv[st][h][t] = f.x; xv[st][h][t + 1] = f.y; xv[st][h][t + 2] = f.z; xv[st][h][t + 3] = f.w;
                 }
-        float res[SETS] = {0.0f, 0.0f};
+        float res[SETS] = {};
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             f32x4_t DA[SETS], DB[SETS];
@@ -1216,15 +1224,67 @@ GemvPlan plan_gemv4(const GemvArgs& a, int nslot) {
     int T = (a.ntiles + num_cu - 1) / num_cu;
     while (grid_for(T) > num_cu && x_bytes + (size_t)(T + 1) * per_tile + 128 <= 160 * 1024) ++T;
     while (T > 1 && x_bytes + (size_t)T * per_tile + 128 > 160 * 1024) --T;
+    // Where LDS keeps one round of workgroups from holding all tiles, even rounds instead of a short last one
+    // (128256 x 4096 at four rows: 30 tiles per workgroup made 268 workgroups, 68.4 us; 16 make 501).
+    if (const int g = grid_for(T); g > num_cu) {
+        const int rounds = (g + num_cu - 1) / num_cu;
+        while (T > 1 && (grid_for(T - 1) + num_cu - 1) / num_cu == rounds) --T;
+    }
     p.T = T;
     p.lds = x_bytes + (size_t)T * per_tile + 128;  // + the wavefronts' sums of squares (RMSNorm prologue)
     if (p.lds > 160 * 1024) p.lds = 0;
     return p;
 }
 
+// One tall matrix (an output projection over a vocabulary: 128256 x 4096 are 8016 tiles), five to eight bf16 rows:
+// gemvr_kernel without a problem table, a workgroup per compute unit, NW wavefronts of r tiles each.
+template <int FMT>
+int run_gemv_tall(const GemvArgs& a, const void* x, hipStream_t s, bool* taken) {
+    *taken = false;
+    if constexpr (kPaired<FMT>) {
+        const int nblocks = a.K >> 8;
+        // (Up to four rows stay with the column-split kernel, which streams such a matrix as fast or faster:
+        // 128256 x 4096 at one row 46.5 us, 6.36 TB/s, against 47.1 us here; at eight rows 54.4 against 51.3 us,
+        // 49152 x 8192 60.4 against 41.7 us.)
+        if (a.nmat != 1 || a.x_f32 || a.xop != XOP_NONE || a.pair || a.nslot <= 4 || a.nslot > 8 || a.ntiles < 256 * 12) return TFQ_OK;
+        constexpr int sets = 2;
+        const size_t lds = ((size_t)nblocks * (a.nslot * kSlotStride + sets * Fmt<FMT>::NG) + 4) * 16;
+        if (lds > 160 * 1024) return TFQ_OK;
+        long best_cost = -1;
+        int nw = 16, r = 1;
+        for (int w = 16; w >= 12; --w)
+            for (int rr = 1; rr <= 256; ++rr) {
+                const long wgs = (a.ntiles + w * rr - 1) / (w * rr);
+                const long cost = (wgs + 255) / 256 * (2 * rr + 1);
+                if (best_cost < 0 || cost < best_cost) { best_cost = cost; nw = w; r = rr; }
+            }
+        GemvKernArgs k{};
+        k.W0 = a.W[0]; k.y0 = a.y[0]; k.nr0 = a.nrows[0];
+        k.K = a.K; k.y_bf16 = a.y_bf16; k.nslot = a.nslot; k.tiles_per_wg = nw * r; k.accumulate = a.accumulate;
+        const int grid = (a.ntiles + nw * r - 1) / (nw * r);
+        using Kernel = void (*)(GemvKernArgs, const void*);
+        const Kernel kern = gemvr_kernel<FMT, false, 2, false>;
+        static std::atomic<bool> lds_limit_raised{false};
+        if (!lds_limit_raised) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
+            lds_limit_raised = true;
+        }
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * nw), lds, s, k, x);
+        *taken = true;
+        return hip_fail(hipGetLastError(), "gemv launch");
+    }
+    return TFQ_OK;
+}
+
 template <int FMT>
 int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     const int nblocks = a.K >> 8;
+    {
+        bool taken = false;
+        const int rc = run_gemv_tall<FMT>(a, x, s, &taken);
+        if (rc || taken) return rc;
+    }
     const GemvPlan p = plan_gemv4<FMT>(a, a.nslot);
     if (p.lds == 0) return fail(TFQ_ERR_SHAPE, "gemv: K too large for the LDS activation stage");
     const int NW = p.NW, T = p.T;
@@ -1530,7 +1590,7 @@ int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, 
                 if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
                 lds_limit_raised[8] = true;
             }
-            hipLaunchKernelGGL((gemvr_kernel<FMT, true>), dim3(gp.grid), dim3(64 * gp.NW), gp.lds, s, k);
+            hipLaunchKernelGGL((gemvr_kernel<FMT, true>), dim3(gp.grid), dim3(64 * gp.NW), gp.lds, s, k, nullptr);
             return hip_fail(hipGetLastError(), "gemv group launch");
         } else {
             return fail(TFQ_ERR_FORMAT, "gemv group: no paired kernel for this format");
