@@ -181,6 +181,8 @@ def main():
         del layers
         torch.cuda.empty_cache()
         res["moe"] = moe_layer(tfq, torch, fmt, bpw, base)
+    if not args.no_sweep:
+        res["output_projection"] = output_projection(tfq, torch, fmt, bpw, base)
     if not args.no_cpu:
         # the reference caps its matmul at 8 threads (src/adapters/tools/qwen35_engine.cpp:60); the second
         # figure uses every core this process may use
@@ -468,6 +470,51 @@ def moe_layer(tfq, torch, fmt, bpw, base, E=8, top_k=2, T=16, D=4096, F=14336, r
     nbytes1 = active1 * 3 * F * D * bpw / 8
     out["single_token"] = {"active_experts": active1, "us_per_call": round(dt1 * 1e6, 1), "gbs": round(nbytes1 / dt1 / 1e9, 1),
                            "frac": round(nbytes1 / dt1 / 1e9 / HBM_PEAK_GBS, 4)}
+    return out
+
+
+def output_projection(tfq, torch, fmt, bpw, base, N=128256, K=4096, copies=3, reps=10):
+    """The model's largest single GEMV, the projection onto its vocabulary (128256 x 4096, 295 MB packed), at batch
+    1 and 8: three copies cut from the layer's weight stream at different offsets, called in rotation (885 MB, more
+    than the caches hold), in graph replays.  A side figure: a decode step runs it once per token, `value` covers
+    the decoder layers only."""
+    stream = torch.cat([base[n] for n in ("gate", "up", "down", "q", "o", "k", "v")])
+    need = N * K
+    reps_of_stream = (need + (copies - 1) * 1000003) // stream.numel() + 1
+    big = stream.repeat(reps_of_stream)
+    Ws = [tfq.Weight(fmt, N, K, tfq.encode(fmt, big[i * 1000003:i * 1000003 + need])) for i in range(copies)]
+    del big, stream
+    out = {"shape": "%dx%d" % (N, K), "packed_mb": round(N * K * bpw / 8 / 1e6, 1)}
+    for B in (1, 8):
+        x = torch.from_numpy(tfq.rng_normal(43, B * K)).to("cuda").reshape(B, K).bfloat16()
+        y = torch.empty(B, N, device="cuda")
+        for W in Ws:
+            W.gemv(x, out=y)
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            Ws[0].gemv(x, out=y)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        rounds = 8  # launches per replay: 24, so that the replay's own start-up does not weigh on a launch
+        with torch.cuda.graph(g):
+            for _ in range(rounds):
+                for W in Ws:
+                    W.gemv(x, out=y)
+        for _ in range(2):
+            g.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            g.replay()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / (reps * copies * rounds)
+        nbytes = N * K * bpw / 8 + B * K * 2 + B * N * 4
+        out[str(B)] = {"us": round(dt * 1e6, 2), "gbs": round(nbytes / dt / 1e9, 1), "frac": round(nbytes / dt / 1e9 / HBM_PEAK_GBS, 4)}
+    for W in Ws:
+        W.close()
     return out
 
 
