@@ -1128,46 +1128,39 @@ __global__ __launch_bounds__(1024) void gemvb_kernel(GemvKernArgs args, const un
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int slot = 4 * q + r;
-                if (slot < B)
-                    __hip_atomic_store(args.partial + (size_t)part * 16 * (size_t)nrm + (size_t)slot * (size_t)nrm + (size_t)row, o[r],
-                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (slot < B) args.partial[(size_t)part * 16 * (size_t)nrm + (size_t)slot * (size_t)nrm + (size_t)row] = o[r];
             }
         } else {
             store_out(t, v);
         }
     }
-    if constexpr (SPLIT) {
-        // The last part of a row group to arrive adds the parts in part order (the same sum whichever part
-        // that is) and puts the counter back to zero for the next launch.  Every workgroup passes through
-        // here exactly once and waits for nobody.  The partial sums are device-scope stores and are read back
-        // with device-scope loads: it is enough that every store of the workgroup has completed before its
-        // arrival is counted.
-        int& last_arrival = *reinterpret_cast<int*>(smem);  // the group sums are no longer needed
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (tid == 0) {
-            const unsigned seen = __hip_atomic_fetch_add(args.counters + rowgroup, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            last_arrival = seen == (unsigned)kparts - 1u;
-            if (last_arrival) __hip_atomic_store(args.counters + rowgroup, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        __syncthreads();
-        if (last_arrival) {
-            for (int t = wave; t < tiles_here; t += NW) {
-                const int row = (tile0 + t) * 16 + n;
-                if (row >= nrm) continue;
-                float o[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-                for (int c = 0; c < kparts; ++c) {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const int slot = 4 * q + r;
-                        if (slot < B)
-                            o[r] += __hip_atomic_load(args.partial + (size_t)c * 16 * (size_t)nrm + (size_t)slot * (size_t)nrm + (size_t)row,
-                                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
-                }
-                store_out(t, float4{o[0], o[1], o[2], o[3]});
+}
+
+// The K parts of a split launch meet in a launch of their own: y[b][n] = sum over the parts, in part order, of the
+// partial sums [part][16 slots][N] that gemvb_kernel<..., SPLIT> left (plain stores: the launch boundary orders
+// them).  fp32 rows are two adjacent slots each, added first like the unsplit kernel adds them.  (The parts used
+// to meet inside the kernel: device-scope stores, an arrival counter per row group, the last arriver reading all
+// parts back.  That chain of dependent memory round trips cost 6 us of a 17 us launch, 4096 x 14336 at sixteen
+// rows; this kernel and its launch boundary cost 3.5 us.)
+__global__ __launch_bounds__(256) void split_reduce_kernel(const float* __restrict__ partial, void* __restrict__ y, int kparts, int B,
+                                                          int nrm, int y_bf16, int x_f32) {
+    const int row = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;  // one output per lane
+    if (row >= nrm) return;
+    {
+        float v = 0.0f;
+        if (x_f32) {
+            float lo = 0.0f;
+            for (int c = 0; c < kparts; ++c) {
+                v += partial[((size_t)c * 16 + 2 * b) * (size_t)nrm + row];
+                lo += partial[((size_t)c * 16 + 2 * b + 1) * (size_t)nrm + row];
             }
+            v += lo;
+        } else {
+            for (int c = 0; c < kparts; ++c) v += partial[((size_t)c * 16 + b) * (size_t)nrm + row];
         }
+        const size_t off = (size_t)b * (size_t)nrm + (size_t)row;
+        if (y_bf16) reinterpret_cast<unsigned short*>(y)[off] = (unsigned short)bf16_rne(v);
+        else reinterpret_cast<float*>(y)[off] = v;
     }
 }
 
@@ -1428,6 +1421,9 @@ int run_gemvb(GemvArgs a, const void* x, hipStream_t s) {
         lds_limit_raised[ki] = true;
     }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, s, k, static_cast<const unsigned short*>(x));
+    if (split)
+        hipLaunchKernelGGL(split_reduce_kernel, dim3((a.nrows[0] + 255) / 256, a.x_f32 ? a.nslot / 2 : a.nslot), dim3(256), 0, s,
+                           a.split_partial, a.y[0], kparts, a.nslot, a.nrows[0], a.y_bf16, a.x_f32);
     return hip_fail(hipGetLastError(), "gemv launch");
 }
 
