@@ -255,20 +255,15 @@ static tfq_weight_t* make_weight(const char* who, uint8_t fmt, int64_t N, int64_
     if (!from_host && (uintptr_t)packed % 16) { fail(TFQ_ERR_ARG, std::string(who) + ": device payload must be 16-byte aligned"); return nullptr; }
     if (ensure_device()) return nullptr;
     const bool tiled = wants_tiled16(fmt);
-    tfq_weight_t* w = new (std::nothrow) tfq_weight_t{fmt, N, K, bytes, nullptr, 0, tiled ? TFQ_LAYOUT_TILED16 : TFQ_LAYOUT_WIRE, true, nullptr, nullptr};
+    tfq_weight_t* w = new (std::nothrow) tfq_weight_t{fmt, N, K, bytes, nullptr, 0, tiled ? TFQ_LAYOUT_TILED16 : TFQ_LAYOUT_WIRE, true, nullptr};
     if (!w) { fail(TFQ_ERR_NOMEM, std::string(who) + ": out of host memory"); return nullptr; }
     w->dev_bytes = tiled ? (size_t)((N + 15) / 16) * (size_t)(K / 256) * (size_t)tiled_unit_bytes(fmt) : bytes;
     uint8_t* staged = nullptr;  // wire payload on the device, when it has to be permuted
-    // partial sums and arrival counters of the K-split decode kernel live behind the weights
+    // the partial sums of the K-split decode kernel live behind the weights (every one is written before it is read)
     const size_t split_bytes = tiled ? gemv_rows16_split_bytes(fmt, N, K) : 0;
     const size_t split_at = (w->dev_bytes + 255) & ~(size_t)255;
     hipError_t e = hipMalloc(&w->dev, split_bytes ? split_at + split_bytes : w->dev_bytes);
-    if (e == hipSuccess && split_bytes) {
-        const size_t counter_bytes = (size_t)((N + 15) / 16) * 4;
-        w->split_partial = reinterpret_cast<float*>(w->dev + split_at);
-        w->split_counters = reinterpret_cast<unsigned*>(w->dev + split_at + split_bytes - counter_bytes);
-        e = hipMemset(w->split_counters, 0, counter_bytes);
-    }
+    if (e == hipSuccess && split_bytes) w->split_partial = reinterpret_cast<float*>(w->dev + split_at);
     if (e == hipSuccess && from_host) {
         if (tiled) {
             e = hipMalloc(&staged, bytes);
@@ -327,7 +322,7 @@ tfq_weight_t* tfq_weight_upload_mixed(int64_t N, int64_t K, const uint8_t* block
     }
     if (at != bytes) { fail(TFQ_ERR_SHAPE, std::string(who) + ": payload is " + std::to_string(bytes) + " bytes, the blocks need " + std::to_string(at)); return nullptr; }
     if (ensure_device()) return nullptr;
-    tfq_weight_t* w = new (std::nothrow) tfq_weight_t{block_formats[0], N, K, bytes, nullptr, 0, TFQ_LAYOUT_MIXED, true, nullptr, nullptr};
+    tfq_weight_t* w = new (std::nothrow) tfq_weight_t{block_formats[0], N, K, bytes, nullptr, 0, TFQ_LAYOUT_MIXED, true, nullptr};
     if (!w) { fail(TFQ_ERR_NOMEM, std::string(who) + ": out of host memory"); return nullptr; }
     // one allocation: payloads (+ 16 bytes the decoders' window reads may touch) | offsets | wire ids | layouts
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };

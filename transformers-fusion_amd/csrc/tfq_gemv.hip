@@ -64,8 +64,7 @@ struct GemvArgs {
     int nslot;         // bf16 activation rows held in LDS: B, or 2B for fp32 input (<= 4)
     int tiles_per_wg;  // T
     int cols_base, cols_rem;  // block columns per wavefront: cols_base + (wave < cols_rem)
-    float* split_partial;     // single matrix only: the handle's partial sums and arrival counters, or null
-    unsigned* split_counters;
+    float* split_partial;     // single matrix only: the handle's area for the partial sums of K parts, or null
     // prologue fused into the activation staging (fp32 input only): XOP_RMSNORM takes gamma / eps /
     // gamma_plus_one, XOP_SWIGLU takes x2 (the up product; x is the gate product) and mid_bf16
     int xop;
@@ -91,7 +90,6 @@ struct GemvKernArgs {
     int K, y_bf16, nslot, tiles_per_wg, cols_base, cols_rem;
     int kparts, kcols;  // gemvb_kernel: workgroups per row group (K parts) and block columns per part
     float* partial;
-    unsigned* counters;
     const float* gamma;  // XOP_RMSNORM
     const float* x2;     // XOP_SWIGLU: the second factor, same shape as x
     float eps;
@@ -1391,7 +1389,6 @@ int run_gemvb(GemvArgs a, const void* x, hipStream_t s) {
     k.kparts = kparts;
     k.kcols = kcols;
     k.partial = a.split_partial;
-    k.counters = a.split_counters;
     k.W0 = a.W[0]; k.W1 = a.W[1]; k.W2 = a.W[2]; k.W3 = a.W[3];
     k.y0 = a.y[0]; k.y1 = a.y[1]; k.y2 = a.y[2]; k.y3 = a.y[3];
     k.nr0 = a.nrows[0]; k.nr1 = a.nrows[1]; k.nr2 = a.nrows[2]; k.nr3 = a.nrows[3];
@@ -1689,7 +1686,7 @@ int gemv_rows16_parts(int fmt, int64_t K) {
 size_t gemv_rows16_split_bytes(int fmt, int64_t N, int64_t K) {
     const int parts = gemv_rows16_parts(fmt, K);
     if (parts < 2) return 0;
-    return (size_t)parts * 16 * (size_t)N * 4 + (size_t)((N + 15) / 16) * 4;
+    return (size_t)parts * 16 * (size_t)N * 4;
 }
 
 bool gemv_grouped_supported(int fmt) {
@@ -1801,16 +1798,15 @@ int launch_gemv_multi_fused(const tfq_weight* const* ws, int nmat, const void* x
     a.K = (int)ws[0]->K;
     if (nmat == 1) {
         a.split_partial = ws[0]->split_partial;
-        a.split_counters = ws[0]->split_counters;
     }
     if (pair) {  // one grid over the tiles of gate; the kernel walks the same tiles of up (W[1]) behind them
         a.pair = 1;
         a.nmat = 1;
         a.ntiles = (int)((ws[0]->N + 15) / 16);
-        a.split_partial = nullptr; a.split_counters = nullptr;
+        a.split_partial = nullptr;
     }
     a.accumulate = accumulate ? 1 : 0;
-    if (accumulate) { a.split_partial = nullptr; a.split_counters = nullptr; }
+    if (accumulate) a.split_partial = nullptr;
     if (fused) {
         a.xop = pro->op == TFQ_PRO_RMSNORM ? XOP_RMSNORM : XOP_SWIGLU;
         a.gamma = pro->gamma; a.x2 = pro->up; a.eps = pro->eps;

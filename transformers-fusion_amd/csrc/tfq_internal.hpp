@@ -334,10 +334,9 @@ struct tfq_weight {
     int layout;
     bool owns;
     // Behind the packed weights in the same allocation, for matrices whose K is cut into several parts by the
-    // 5..16-row decode kernel: fp32 partial sums [parts][16 rows][N] and one arrival counter per 16-row tile
-    // (zero between launches).  One call at a time per handle may use them.
+    // 5..16-row decode kernel: fp32 partial sums [parts][16 rows][N], written by one launch and added by the
+    // next.  One call at a time per handle may use them.
     float* split_partial;
-    unsigned* split_counters;
     // TFQ_LAYOUT_MIXED: every block carries its own wire id (the container's per-block format byte).  dev holds
     // the payloads one behind the other; these device arrays (behind them in the same allocation) give each
     // block's byte offset and wire id, and the block layout of every wire id.
@@ -416,7 +415,7 @@ struct GemvGroupPlan {
 };
 bool gemv_grouped_supported(int fmt);
 bool gemv_rows16_supported(int fmt);
-// K parts of the 5..16-row decode kernel (1: no split) and the bytes of partial sums and counters they need
+// K parts of the 5..16-row decode kernel (1: no split) and the bytes of partial sums they need
 int gemv_rows16_parts(int fmt, int64_t K);
 size_t gemv_rows16_split_bytes(int fmt, int64_t N, int64_t K);
 int plan_gemv_grouped(int fmt, int K, bool x_f32, const int* nrows, const int* nrows_x, int nprob, GemvGroupPlan* gp, bool pair = false);
