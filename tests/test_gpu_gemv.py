@@ -391,7 +391,7 @@ def test_gemv_rows_with_k_split_repeated_calls(O, tfq, gpu, fmt):
 
 
 def test_gemv_k_split_in_graph_replays(O, tfq, gpu):
-    """The K-split launch inside a captured graph: its arrival counters reset themselves, so every replay
+    """The K-split launches (the parts' kernel and the kernel that adds them) inside a captured graph: every replay
     (with eager launches on the same handle between replays) gives the bits of the eager result."""
     import torch
     N, K, B = 4096, 14336, 16
@@ -418,11 +418,10 @@ def test_gemv_k_split_in_graph_replays(O, tfq, gpu):
 
 
 def test_gemv_k_split_soak(O, tfq, gpu):
-    """A bounded soak of the K-split rendezvous: 3000 replays of a graph holding three K-split launches, each
-    compared bit for bit with the eager result on the device; the loop stops at the first block of replays
-    that holds a mismatch.  (The rendezvous passes partial sums between workgroups on different XCDs through
-    device-scope stores, a wait for their acknowledgement and a device-scope counter; a lost or late partial
-    sum would change bits.)"""
+    """A bounded soak of the K split: 3000 replays of a graph holding three K-split products, each compared bit
+    for bit with the eager result on the device; the loop stops at the first block of replays that holds a
+    mismatch.  (Partial sums pass from the workgroups of one launch, on different XCDs, to the launch that adds
+    them; a lost or late partial sum would change bits.)"""
     import torch
     N, K, B = 4096, 14336, 16
     g = torch.Generator(device="cuda").manual_seed(12)
