@@ -37,6 +37,12 @@
 // walks the tiles, keeps two unit fetches in flight, and adds its partial sums
 // into a private LDS cell per (tile, lane); after the only barrier the NW
 // partials of each output are added in a fixed order (deterministic results).
+//
+// Two more kernels share the arithmetic.  gemvb_kernel uses the MFMA densely for five to sixteen rows (A = the rows
+// of one scale group); over a K of more than sixteen block columns it cuts K into parts over workgroups, and
+// split_reduce_kernel, a launch of its own, adds the parts.  gemvr_kernel serves launches with at least a dozen
+// tiles per compute unit (the experts of a mixture layer, a projection onto a vocabulary): a wavefront owns whole
+// tiles and walks all their block columns, so nothing is added across wavefronts.
 
 #include <atomic>
 
