@@ -249,6 +249,47 @@ def test_moe_ffn_routed_builds_its_lists_on_the_device(O, tfq, gpu, fmt):
         wl.close()
 
 
+@pytest.mark.parametrize("fmt,D,F", [("B32S4", 512, 1024), ("Q_G_4", 256, 768), ("B32S8", 256, 512), ("Q_G_8", 512, 512), ("B32S4", 4096, 14336)])
+def test_moe_ffn_routed_single_token(O, tfq, gpu, fmt, D, F):
+    """One token, top-2: the routed call is two launches that look the slots' experts up themselves and add the
+    weighted down products into y with atomics.  Against the oracle (the small shapes), against the host-list
+    call bit for bit, and with the irregular slots: an id outside 0..E-1, a weight that is not positive, both
+    slots naming one expert; ten calls in a row give the same bits."""
+    import torch
+    E, Ktop, T = 8, 2, 1
+    small = D * F <= 1 << 20
+    if small:
+        gate, up, down, hg, hu, hd = _experts(O, tfq, fmt, E, D, F, 1500)
+    else:
+        gen = torch.Generator(device="cuda").manual_seed(3)
+        gate, up, down = [], [], []
+        for e in range(E):
+            for lst, n, k in ((gate, F, D), (up, F, D), (down, D, F)):
+                lst.append(tfq.Weight(fmt, n, k, tfq.encode(fmt, torch.randn(n * k, device=gpu, generator=gen) * 0.02)))
+    x = O.bf16_round(O.rng_normal(57, T * D, 1.0).reshape(T, D))
+    xt = torch.from_numpy(x).to(gpu).bfloat16()
+    routed = tfq.RoutedMoe(gate, up, down, T, Ktop)
+    cases = [([3, 6], [0.7, 0.3]), ([5, 0], [0.25, 0.75]), ([2, E + 1], [0.6, 0.4]), ([-1, 4], [0.5, 0.5]),
+             ([1, 7], [0.0, 1.0]), ([4, 4], [0.6, 0.4])]
+    for ids, wts in cases:
+        idx = np.array([ids], np.int64)
+        w = np.array([wts], np.float32)
+        host = tfq.moe_ffn(gate, up, down, idx, w, xt, mid_dtype=torch.bfloat16)
+        y = torch.full((T, D), 7.0, device=gpu)
+        di, dw = torch.from_numpy(idx.astype(np.int32)).to(gpu), torch.from_numpy(w).to(gpu)
+        routed(di, dw, xt, y)
+        assert torch.equal(y, host), (ids, wts, float((y - host).abs().max()))
+        if small and ids[0] != ids[1]:
+            ref = O.moe_ffn(fmt, hg, hu, hd, D, F, idx, w, x, mid_bf16=True)
+            assert rel_err(y.cpu().numpy(), ref) <= 1e-2
+        for _ in range(10):
+            y2 = torch.full((T, D), -3.0, device=gpu)
+            routed(di, dw, xt, y2)
+            assert torch.equal(y2, y)
+    for wl in gate + up + down:
+        wl.close()
+
+
 @pytest.mark.parametrize("T,Ktop,E", [(1, 1, 3), (7, 3, 5), (64, 2, 4), (128, 8, 16), (5, 2, 40)])
 def test_moe_ffn_routed_shapes(O, tfq, gpu, T, Ktop, E):
     """Call shapes of the routed form: one pair, odd counts, experts with several passes of eight and sixteen

@@ -147,15 +147,48 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
     const uint8_t* Wm2 = nullptr;  // PAIR: the second matrix
     void* ym;
     const void* xin;
+    // GROUPED, the slots of ONE token looked up here instead of in a table (W2 = the experts' matrix addresses,
+    // [gate | up | down][E]; W1 = the token's expert ids; nr2 workgroups per slot): the output is scaled by the
+    // slot's routing weight and added into one vector with atomics when y1 holds the weights.
+    float out_scale = 1.0f;
+    bool out_atomic = false;
     if constexpr (GROUPED) {
-        const GemvProb* table = reinterpret_cast<const GemvProb*>(args.W0);
-        const int* wg_map = reinterpret_cast<const int*>(args.W1);
-        const int prob = wg_map[bid];
-        if (prob < 0) return;  // a workgroup beyond the problems of this call (tables built on the device)
-        const GemvProb pr = table[prob];
-        wg_first = pr.wg_first; nrm = pr.nrows; nslot = pr.nslot;
-        Wm = pr.W; ym = pr.y; xin = pr.x;
-        Wm2 = pr.W2;
+        if (args.W2 != nullptr) {
+            if (args.y2 != nullptr) {  // the vector the next launch adds into starts at zero
+                const int i = bid * (int)blockDim.x + (int)threadIdx.x;
+                if (i < args.g2) reinterpret_cast<float*>(args.y2)[i] = 0.0f;
+            }
+            const int prob = bid / args.nr2;
+            const int* ids = reinterpret_cast<const int*>(args.W1);
+            const uint8_t* const* ptrs = reinterpret_cast<const uint8_t* const*>(args.W2);
+            const int E = args.nr1, e = ids[prob];
+            if (e < 0 || e >= E) return;  // a slot without an expert
+            if (args.y1 != nullptr) {
+                // the weight of the first slot that names the expert, as the combine step takes it; a slot whose
+                // weight is not positive adds nothing
+                const float* w = reinterpret_cast<const float*>(args.y1);
+                float wt = w[prob];
+                for (int j = prob - 1; j >= 0; --j)
+                    if (ids[j] == e) wt = w[j];
+                if (!(wt > 0.0f)) return;
+                out_scale = wt;
+                out_atomic = true;
+            }
+            wg_first = prob * args.nr2; nrm = args.nr0; nslot = 1;
+            Wm = ptrs[(size_t)args.nr3 * E + e];
+            Wm2 = ptrs[(size_t)E + e];
+            ym = static_cast<uint8_t*>(args.y0) + (size_t)prob * (size_t)args.g0;
+            xin = static_cast<const uint8_t*>(xin_arg) + (size_t)prob * (size_t)args.g1;
+        } else {
+            const GemvProb* table = reinterpret_cast<const GemvProb*>(args.W0);
+            const int* wg_map = reinterpret_cast<const int*>(args.W1);
+            const int prob = wg_map[bid];
+            if (prob < 0) return;  // a workgroup beyond the problems of this call (tables built on the device)
+            const GemvProb pr = table[prob];
+            wg_first = pr.wg_first; nrm = pr.nrows; nslot = pr.nslot;
+            Wm = pr.W; ym = pr.y; xin = pr.x;
+            Wm2 = pr.W2;
+        }
     } else {
         const int m = (bid >= args.g0) + (bid >= args.g1) + (bid >= args.g2);
         wg_first = m == 0 ? 0 : m == 1 ? args.g0 : m == 2 ? args.g1 : args.g2;
@@ -532,6 +565,12 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
         }
         if constexpr (PAIR) v = v / (1.0f + expf(-v)) * v2;
         const size_t off = (size_t)b * (size_t)nrm + (size_t)row;
+        if constexpr (GROUPED) {
+            if (out_atomic) {  // at most two slots add into a zeroed vector: the same bits in either order
+                __hip_atomic_fetch_add(reinterpret_cast<float*>(ym) + off, v * out_scale, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                continue;
+            }
+        }
         if (args.accumulate) {  // every output element belongs to one workgroup, so the update needs no atomic
             if (y_bf16) v += __uint_as_float((uint32_t)reinterpret_cast<const unsigned short*>(ym)[off] << 16);
             else v += reinterpret_cast<const float*>(ym)[off];
@@ -1552,11 +1591,22 @@ int plan_grouped(int K, bool x_f32, const int* nrows, const int* nrows_x, int np
 }
 
 template <int FMT>
-int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_bf16, hipStream_t s) {
+int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_bf16, hipStream_t s, const GemvDirect* direct = nullptr) {
     const int nblocks = gp.K >> 8;
     GemvKernArgs k{};
     k.W0 = static_cast<const uint8_t*>(d_table);
     k.W1 = reinterpret_cast<const uint8_t*>(d_map);
+    const void* xin = nullptr;
+    if (direct) {  // the slots of one token, looked up by the kernel (see its entry)
+        if (gp.rows || gp.sets != 1 || gp.x_f32) return fail(TFQ_ERR_ARG, "gemv group: the direct form takes one bf16 row per slot");
+        k.W0 = nullptr;
+        k.W1 = reinterpret_cast<const uint8_t*>(direct->ids);
+        k.W2 = reinterpret_cast<const uint8_t*>(direct->ptrs);
+        k.nr0 = direct->nrows; k.nr1 = direct->E; k.nr2 = direct->wgs_per_slot; k.nr3 = direct->matrix;
+        k.y0 = direct->y; k.y1 = const_cast<float*>(direct->weights); k.y2 = direct->zero;
+        k.g0 = (int)direct->y_stride; k.g1 = (int)direct->x_stride; k.g2 = direct->nzero;
+        xin = direct->x;
+    }
     k.K = gp.K; k.y_bf16 = y_bf16; k.nslot = 0; k.tiles_per_wg = gp.T;
     k.cols_base = nblocks / gp.NW; k.cols_rem = nblocks % gp.NW;
     using Kernel = void (*)(GemvKernArgs, const void*);
@@ -1600,7 +1650,7 @@ int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, 
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
         lds_limit_raised[slot] = true;
     }
-    hipLaunchKernelGGL(kern, dim3(gp.grid), dim3(64 * gp.NW), gp.lds, s, k, nullptr);
+    hipLaunchKernelGGL(kern, dim3(gp.grid), dim3(64 * gp.NW), gp.lds, s, k, xin);
     return hip_fail(hipGetLastError(), "gemv group launch");
 }
 
@@ -1736,6 +1786,17 @@ int launch_gemv_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, c
         case TFQ_B32S4: return run_grouped<TFQ_B32S4>(gp, d_table, d_map, yb, s);
         case TFQ_B32S8: return run_grouped<TFQ_B32S8>(gp, d_table, d_map, yb, s);
         case TFQ_Q_G_8: return run_grouped<TFQ_Q_G_8>(gp, d_table, d_map, yb, s);
+        default: return fail(TFQ_ERR_FORMAT, "gemv group: no grouped kernel for this format");
+    }
+}
+
+int launch_gemv_grouped_direct(int fmt, const GemvGroupPlan& gp, const GemvDirect& d, int y_dtype, hipStream_t s) {
+    const int yb = y_dtype == TFQ_BF16;
+    switch (canonical(fmt)) {
+        case TFQ_Q_G_4: return run_grouped<TFQ_Q_G_4>(gp, nullptr, nullptr, yb, s, &d);
+        case TFQ_B32S4: return run_grouped<TFQ_B32S4>(gp, nullptr, nullptr, yb, s, &d);
+        case TFQ_B32S8: return run_grouped<TFQ_B32S8>(gp, nullptr, nullptr, yb, s, &d);
+        case TFQ_Q_G_8: return run_grouped<TFQ_Q_G_8>(gp, nullptr, nullptr, yb, s, &d);
         default: return fail(TFQ_ERR_FORMAT, "gemv group: no grouped kernel for this format");
     }
 }

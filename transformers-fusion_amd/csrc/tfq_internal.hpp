@@ -424,6 +424,24 @@ size_t gemv_group_entry_bytes();
 void fill_gemv_group(const GemvGroupPlan& gp, const tfq_weight* const* ws, const void* const* xs, void* const* ys,
                      const int* nrows_x, int nprob, void* table_host, int* map_host, const tfq_weight* const* ws2 = nullptr);
 int launch_gemv_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s);
+// The grouped launch for the slots of ONE token (at most two when `weights` is given): no table; the kernel reads the
+// slot's expert id and takes the matrix address from `ptrs` ([gate | up | down][E] device addresses; matrix = 0 for
+// the gate / up pair, 2 for down).  Slot p reads x + p * x_stride and writes y + p * y_stride; with `weights` the
+// product times the slot's routing weight is added into y with atomics (y zeroed before: `zero` / `nzero` let the
+// launch in front do that), which for two slots gives the same bits in either order.
+struct GemvDirect {
+    const int* ids;
+    const uint8_t* const* ptrs;
+    int E, matrix, nrows, wgs_per_slot;
+    const float* weights;
+    void* y;
+    size_t y_stride;
+    const void* x;
+    size_t x_stride;
+    float* zero;
+    int nzero;
+};
+int launch_gemv_grouped_direct(int fmt, const GemvGroupPlan& gp, const GemvDirect& d, int y_dtype, hipStream_t s);
 // the same for problems of up to sixteen bf16 activation rows at any K (gemvb_kernel; tables from fill_gemv_group)
 int plan_gemv_rows16_grouped(int fmt, int K, const int* nrows, int nprob, GemvGroupPlan* gp);
 int launch_gemv_rows16_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s);

@@ -786,6 +786,22 @@ int launch_moe_ffn_routed(const tfq_weight* const* gate, const tfq_weight* const
     GemvProb* tabB = reinterpret_cast<GemvProb*>(lists + rp.off_tabB);
     int* mapA = reinterpret_cast<int*>(lists + rp.off_mapA);
     int* mapB = reinterpret_cast<int*>(lists + rp.off_mapB);
+    // One token, at most two slots, fp32 output: two launches and nothing else.  The kernels look the slots' experts
+    // up themselves (no list kernel, no gather: every slot reads the token's row), the gate / up launch zeroes y on
+    // its way, and the down launch adds routing weight x product into y with atomics: two addends onto zero, the
+    // same bits in either order (and the bits the combine step gives: 0 + w0 o0 + w1 o1).
+    if (T == 1 && Ktop <= 2 && y_dtype == TFQ_F32 && !rp.down16 && !rp.planA.rows && rp.planA.sets == 1 && rp.planB.sets == 1 &&
+        rp.planA.pair && !rp.planB.pair) {
+        GemvGroupPlan pa = rp.planA, pb = rp.planB;
+        const int wgsA = (((int)F + 15) / 16 + pa.T - 1) / pa.T, wgsB = (((int)D + 15) / 16 + pb.T - 1) / pb.T;
+        pa.grid = Ktop * wgsA;
+        pb.grid = Ktop * wgsB;
+        const uint8_t* const* ptrs = static_cast<const uint8_t* const*>(d_expert_table);
+        const GemvDirect da{d_topk_idx, ptrs, E, 0, (int)F, wgsA, nullptr, h, F * 2, x, 0, static_cast<float*>(y), (int)D};
+        if (int rc = launch_gemv_grouped_direct(gate[0]->fmt, pa, da, TFQ_BF16, s)) return rc;
+        const GemvDirect db{d_topk_idx, ptrs, E, 2, (int)D, wgsB, d_topk_w, y, 0, h, F * 2, nullptr, 0};
+        return launch_gemv_grouped_direct(down[0]->fmt, pb, db, TFQ_F32, s);
+    }
     const int row_u4 = (int)(D * 2 / 16);
     const int64_t ng = (int64_t)P * row_u4;
     const bool fuse_gather = ng * 16 <= 512 * 1024;  // up to 512 KB of rows ride in the list kernel's one workgroup
