@@ -420,6 +420,8 @@ int tfq_moe_ffn(const tfq_weight_t* const* gate, const tfq_weight_t* const* up,
  * routing.  Same results as tfq_moe_ffn to rounding (the rows of an expert may be cut into passes differently).
  * bf16 x and bf16 mid activations, experts of one tiled format per stage that has the grouped kernels (Q_G_4,
  * B32S4, B32S8, Q_G_8), T * k <= 1024, E <= 256; anything else is refused (use tfq_moe_ffn).
+ * One token with k <= 2 and an fp32 y is two launches: the kernels look the slots' experts up themselves and the
+ * down launch adds weight * product into y (two addends onto zero: the same bits in either order).
  *   tfq_moe_expert_table           writes the experts' device addresses to expert_table (device memory of
  *                                  3 * E * 8 bytes), once per set of experts (a synchronous copy)
  *   tfq_moe_routed_workspace_bytes the workspace the call needs (0: this configuration is refused) */
