@@ -254,7 +254,7 @@ def test_moe_ffn_routed_single_token(O, tfq, gpu, fmt, D, F):
     """One token, top-2: the routed call is two launches that look the slots' experts up themselves and add the
     weighted down products into y with atomics.  Against the oracle (the small shapes), against the host-list
     call bit for bit, and with the irregular slots: an id outside 0..E-1, a weight that is not positive, both
-    slots naming one expert; ten calls in a row give the same bits."""
+    slots naming one expert, no slot with an expert at all (y = 0); ten calls in a row give the same bits."""
     import torch
     E, Ktop, T = 8, 2, 1
     small = D * F <= 1 << 20
@@ -270,7 +270,7 @@ def test_moe_ffn_routed_single_token(O, tfq, gpu, fmt, D, F):
     xt = torch.from_numpy(x).to(gpu).bfloat16()
     routed = tfq.RoutedMoe(gate, up, down, T, Ktop)
     cases = [([3, 6], [0.7, 0.3]), ([5, 0], [0.25, 0.75]), ([2, E + 1], [0.6, 0.4]), ([-1, 4], [0.5, 0.5]),
-             ([1, 7], [0.0, 1.0]), ([4, 4], [0.6, 0.4])]
+             ([1, 7], [0.0, 1.0]), ([4, 4], [0.6, 0.4]), ([-1, E + 2], [0.5, 0.5])]
     for ids, wts in cases:
         idx = np.array([ids], np.int64)
         w = np.array([wts], np.float32)
