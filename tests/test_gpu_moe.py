@@ -26,6 +26,31 @@ def test_route_matches_reference_softmax_topk(O, tfq, gpu):
     assert tfq.moe_route(torch.from_numpy(logits).to(gpu), 99)[1].shape == (T, E)
 
 
+@pytest.mark.parametrize("T,E,K", [(1, 3, 2), (5, 64, 6), (16, 130, 8), (3, 257, 8), (7, 1024, 4), (2, 1100, 3)])
+def test_route_many_experts_and_ties(O, tfq, gpu, T, E, K):
+    """Expert counts around the wavefront width and the limit of the one-wavefront-per-token kernel (1100 experts take
+    the one-lane form), against the oracle; and logits with exact duplicates: equal probabilities are picked in
+    ascending expert order, the k picks of a token are distinct, and the weights are the picked probabilities."""
+    import torch
+    logits = O.rng_normal(70 + E, T * E, 1.0).reshape(T, E)
+    probs, idx, w = O.softmax_topk(logits, K)
+    p_d, i_d, w_d = tfq.moe_route(torch.from_numpy(logits).to(gpu), K)
+    assert np.array_equal(i_d.cpu().numpy().astype(np.int64), idx)
+    assert np.abs(p_d.cpu().numpy() - probs).max() <= 2e-7
+    assert np.abs(w_d.cpu().numpy() - w).max() <= 2e-7
+    tied = logits.copy()
+    tied[:, 1::2] = tied[:, 0::2][:, :tied[:, 1::2].shape[1]]  # every odd expert repeats the even one before it
+    probs, idx, w = O.softmax_topk(tied, K)
+    p_d, i_d, w_d = tfq.moe_route(torch.from_numpy(tied).to(gpu), K)
+    i_n, p_n, w_n = i_d.cpu().numpy().astype(np.int64), p_d.cpu().numpy(), w_d.cpu().numpy()
+    assert np.array_equal(i_n, idx)
+    for t in range(T):
+        assert len(set(i_n[t].tolist())) == K
+        assert np.array_equal(p_n[t, i_n[t]], w_n[t])
+        order = sorted(range(E), key=lambda e: (-p_n[t, e], e))[:K]
+        assert order == i_n[t].tolist()
+
+
 @pytest.mark.parametrize("xdt", ["f32", "bf16"])
 def test_router_linear_then_route(O, tfq, gpu, xdt):
     """tfq_moe_router: logits = x . Wr^T + b (float64 numpy as the check, 1e-5 of the largest logit), then the

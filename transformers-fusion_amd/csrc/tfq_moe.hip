@@ -79,7 +79,65 @@ __global__ __launch_bounds__(256) void combine_kernel(void* __restrict__ out, co
     else reinterpret_cast<float*>(out)[i] = acc;
 }
 
-// one lane per token; E is small (8..256)
+// One wavefront per token, up to kRouteMaxE experts (more take the one-lane form below).  The arithmetic is that of
+// the sequential loops: the maximum and the exponentials do not depend on an order, the sum of the exponentials is
+// added up by one lane in expert order (from LDS), and every round of the selection takes the largest probability
+// strictly after the previous pick, the lowest index among equals.
+constexpr int kRouteMaxE = 1024;
+__global__ __launch_bounds__(256) void route_wave_kernel(const float* __restrict__ logits, int T, int E, int k,
+                                                         float* __restrict__ probs, int* __restrict__ idx,
+                                                         float* __restrict__ wts) {
+    __shared__ float s_p[4][kRouteMaxE];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= T) return;  // a whole wavefront: the rest of the kernel has no workgroup barrier
+    const float* l = logits + (int64_t)t * E;
+    float* p = probs + (int64_t)t * E;
+    float* sp = s_p[wave];
+    float maxv = l[0];
+    for (int e = lane; e < E; e += 64) maxv = fmaxf(maxv, l[e]);
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) maxv = fmaxf(maxv, __shfl_xor(maxv, m));
+    for (int e = lane; e < E; e += 64) sp[e] = expf(l[e] - maxv);
+    __builtin_amdgcn_wave_barrier();
+    float sum = 0.0f;
+    if (lane == 0)
+        for (int e = 0; e < E; ++e) sum += sp[e];
+    sum = __shfl(sum, 0);
+    const float inv = 1.0f / sum;
+    for (int e = lane; e < E; e += 64) {
+        const float v = sp[e] * inv;
+        sp[e] = v;
+        p[e] = v;
+    }
+    __builtin_amdgcn_wave_barrier();
+    float prev = 2.0f;  // probabilities are <= 1
+    int prev_e = -1;
+    for (int j = 0; j < k; ++j) {
+        int best = -1;
+        float bv = -1.0f;
+        for (int e = lane; e < E; e += 64) {  // ascending e inside a lane: the first of equals stays
+            const float v = sp[e];
+            const bool below = v < prev || (v == prev && e > prev_e);
+            if (below && v > bv) { bv = v; best = e; }
+        }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) {
+            const float ov = __shfl_xor(bv, m);
+            const int oe = __shfl_xor(best, m);
+            const bool take = oe >= 0 && (ov > bv || (ov == bv && (best < 0 || oe < best)));
+            if (take) { bv = ov; best = oe; }
+        }
+        if (lane == 0) {
+            idx[(int64_t)t * k + j] = best;
+            wts[(int64_t)t * k + j] = bv;
+        }
+        prev = bv;
+        prev_e = best;
+    }
+}
+
+// one lane per token: any number of experts
 __global__ __launch_bounds__(64) void route_kernel(const float* __restrict__ logits, int T, int E, int k,
                                                    float* __restrict__ probs, int* __restrict__ idx,
                                                    float* __restrict__ wts) {
@@ -230,7 +288,8 @@ int launch_moe_router_logits(const void* x, int x_dtype, const float* Wr, const 
 }
 
 int launch_moe_route(const float* logits, int T, int E, int k, float* probs, int* idx, float* wts, hipStream_t s) {
-    hipLaunchKernelGGL(route_kernel, dim3((T + 63) / 64), dim3(64), 0, s, logits, T, E, k, probs, idx, wts);
+    if (E <= kRouteMaxE) hipLaunchKernelGGL(route_wave_kernel, dim3((T + 3) / 4), dim3(256), 0, s, logits, T, E, k, probs, idx, wts);
+    else hipLaunchKernelGGL(route_kernel, dim3((T + 63) / 64), dim3(64), 0, s, logits, T, E, k, probs, idx, wts);
     return hip_fail(hipGetLastError(), "route launch");
 }
 
@@ -625,40 +684,49 @@ __global__ __launch_bounds__(1024) void routed_lists_kernel(const int32_t* __res
     }
     // Problem tables and workgroup maps of the two grouped launches: an expert's rows in chunks of capA / capB.
     // ptrs = device addresses of the experts' packed matrices, [gate | up | down][E].
-    __shared__ int s_nA, s_nB, s_wgA;
+    __shared__ int s_nA, s_nB, s_wgA, s_tilesA;
+    __shared__ int s_offA[257], s_offB[257];
+    for (int e = tid; e < E; e += blockDim.x) {  // problems of an expert in either launch: its rows in chunks of capA / capB
+        const int nt = s_first[e + 1] - s_first[e];
+        s_offA[e] = (nt + sh.capA - 1) / sh.capA;
+        s_offB[e] = (nt + sh.capB - 1) / sh.capB;
+    }
+    __syncthreads();
     if (tid == 0) {
+        int nA = 0, nB = 0;  // counts -> first problem of every expert
+        for (int e = 0; e < E; ++e) {
+            const int cA = s_offA[e], cB = s_offB[e];
+            s_offA[e] = nA;
+            s_offB[e] = nB;
+            nA += cA;
+            nB += cB;
+        }
+        s_nA = nA;
+        s_nB = nB;
         // The tile-owning kernel runs a workgroup per compute unit: when a call has more problems than the plan
         // assumed (an expert's rows in several chunks), its wavefronts take more tile pairs each, so that the
         // workgroups still fit one round.
         int wgA = sh.wgA, tilesA = 0;
         if (sh.nwA) {
-            int problems = 0;
-            for (int e = 0; e < E; ++e) problems += (s_first[e + 1] - s_first[e] + sh.capA - 1) / sh.capA;
             const int tiles = (sh.nrowsA + 15) >> 4;
             int r = sh.rA;
-            while (r < 64 && problems * ((tiles + sh.nwA * r - 1) / (sh.nwA * r)) > 256) ++r;
+            while (r < 64 && nA * ((tiles + sh.nwA * r - 1) / (sh.nwA * r)) > 256) ++r;
             tilesA = sh.nwA * r;
             wgA = (tiles + tilesA - 1) / tilesA;
         }
         s_wgA = wgA;
-        int nA = 0, nB = 0;
-        for (int e = 0; e < E; ++e) {
-            const int p0 = s_first[e], nt = s_first[e + 1] - p0;
-            for (int b0 = 0; b0 < nt; b0 += sh.capA) {
-                const int nb = min(sh.capA, nt - b0);
-                tabA[nA] = GemvProb{ptrs[e], h + (size_t)(p0 + b0) * sh.strideYA, xe + (size_t)(p0 + b0) * sh.strideXA, ptrs[E + e],
-                                    sh.nrowsA, nb, nA * wgA, tilesA};
-                ++nA;
-            }
-            for (int b0 = 0; b0 < nt; b0 += sh.capB) {
-                const int nb = min(sh.capB, nt - b0);
-                tabB[nB] = GemvProb{ptrs[2 * E + e], o + (size_t)(p0 + b0) * sh.strideYB, h + (size_t)(p0 + b0) * sh.strideXB, nullptr,
-                                    sh.nrowsB, nb, nB * sh.wgB, 0};
-                ++nB;
-            }
-        }
-        s_nA = nA;
-        s_nB = nB;
+        s_tilesA = tilesA;
+    }
+    __syncthreads();
+    for (int e = tid; e < E; e += blockDim.x) {  // an expert's table entries, by one thread
+        const int p0 = s_first[e], nt = s_first[e + 1] - p0;
+        int iA = s_offA[e], iB = s_offB[e];
+        for (int b0 = 0; b0 < nt; b0 += sh.capA, ++iA)
+            tabA[iA] = GemvProb{ptrs[e], h + (size_t)(p0 + b0) * sh.strideYA, xe + (size_t)(p0 + b0) * sh.strideXA, ptrs[E + e],
+                                sh.nrowsA, min(sh.capA, nt - b0), iA * s_wgA, s_tilesA};
+        for (int b0 = 0; b0 < nt; b0 += sh.capB, ++iB)
+            tabB[iB] = GemvProb{ptrs[2 * E + e], o + (size_t)(p0 + b0) * sh.strideYB, h + (size_t)(p0 + b0) * sh.strideXB, nullptr,
+                                sh.nrowsB, min(sh.capB, nt - b0), iB * sh.wgB, 0};
     }
     __syncthreads();
     const int nA = s_nA, nB = s_nB;
@@ -804,7 +872,7 @@ int launch_moe_ffn_routed(const tfq_weight* const* gate, const tfq_weight* const
     }
     const int row_u4 = (int)(D * 2 / 16);
     const int64_t ng = (int64_t)P * row_u4;
-    const bool fuse_gather = ng * 16 <= 512 * 1024;  // up to 512 KB of rows ride in the list kernel's one workgroup
+    const bool fuse_gather = ng * 16 <= 256 * 1024;  // up to 256 KB of rows ride in the list kernel's one workgroup (about 3 us)
     hipLaunchKernelGGL(routed_lists_kernel, dim3(1), dim3(1024), 0, s, d_topk_idx, d_topk_w, T, Ktop, E, d_first, d_rows, d_w, d_tokf, d_tokp,
                        rp.sh, static_cast<const uint8_t* const*>(d_expert_table), (const uint8_t*)xe, h, o, tabA, mapA, tabB, mapB,
                        fuse_gather ? (const uint4*)x : nullptr, row_u4);
