@@ -101,6 +101,16 @@ struct GemvKernArgs {
     float eps;
     int gamma_plus_one, mid_bf16;
     int accumulate;
+    // Grouped launches of a mixture layer whose tokens have at most two slots: the launch that writes the mid
+    // activations zeroes `zero` (nzero floats) on its way, and the down launch adds routing weight x product of
+    // pair p into comb_y[comb_rows[p]][row] with atomics instead of writing a row per pair (two addends onto zero:
+    // the same bits in either order).  Null when unused.
+    float* zero;
+    int nzero;
+    const int* comb_rows;
+    const float* comb_wts;
+    float* comb_y;
+    int comb_D;
 };
 
 // WD = unit fetches in flight per wavefront; the first WD are requested unconditionally, so the host
@@ -180,6 +190,8 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
             ym = static_cast<uint8_t*>(args.y0) + (size_t)prob * (size_t)args.g0;
             xin = static_cast<const uint8_t*>(xin_arg) + (size_t)prob * (size_t)args.g1;
         } else {
+            if (args.zero != nullptr)
+                for (int i = bid * (int)blockDim.x + (int)threadIdx.x; i < args.nzero; i += (int)(gridDim.x * blockDim.x)) args.zero[i] = 0.0f;
             const GemvProb* table = reinterpret_cast<const GemvProb*>(args.W0);
             const int* wg_map = reinterpret_cast<const int*>(args.W1);
             const int prob = wg_map[bid];
@@ -612,6 +624,8 @@ __global__ __launch_bounds__(1024) void gemvr_kernel(GemvKernArgs args, const vo
     // the workgroup's problem: an entry of the table of a grouped launch, or the launch's one matrix
     GemvProb pr;
     if constexpr (GROUPED) {
+        if (args.zero != nullptr)
+            for (int i = bid * (int)blockDim.x + (int)threadIdx.x; i < args.nzero; i += (int)(gridDim.x * blockDim.x)) args.zero[i] = 0.0f;
         const GemvProb* table = reinterpret_cast<const GemvProb*>(args.W0);
         const int prob = reinterpret_cast<const int*>(args.W1)[bid];
         if (prob < 0) return;  // a workgroup beyond the problems of this call (tables built on the device)
@@ -902,7 +916,7 @@ __global__ __launch_bounds__(1024) void gemvb_kernel(GemvKernArgs args, const un
     const int bid = blockIdx.x;
     // this workgroup's matrix: selected with compares, or read from the problem table of a grouped launch
     // (W0 = table of GemvProb, W1 = map workgroup -> problem; both reads are uniform)
-    int wg_first, nrm, B;
+    int wg_first, nrm, B, pair0 = 0;
     const uint8_t* Wm;
     void* ym;
     const unsigned short* x;
@@ -914,6 +928,7 @@ __global__ __launch_bounds__(1024) void gemvb_kernel(GemvKernArgs args, const un
         const GemvProb pr = table[prob];
         wg_first = pr.wg_first; nrm = pr.nrows; B = pr.nslot;
         Wm = pr.W; ym = pr.y; x = static_cast<const unsigned short*>(pr.x);
+        pair0 = pr.tiles;  // (this kernel takes its tiles per workgroup from the launch: the field carries the first pair)
     } else {
         const int m = (bid >= args.g0) + (bid >= args.g1) + (bid >= args.g2);
         wg_first = m == 0 ? 0 : m == 1 ? args.g0 : m == 2 ? args.g1 : args.g2;
@@ -1153,6 +1168,20 @@ __global__ __launch_bounds__(1024) void gemvb_kernel(GemvKernArgs args, const un
             return;
         }
         const float o[4] = {v.x, v.y, v.z, v.w};
+        if constexpr (GROUPED) {
+            if (args.comb_y != nullptr) {  // weight x product into the token's output row (see GemvKernArgs)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int slot = 4 * q + r;
+                    if (slot >= B) continue;
+                    const float wt = args.comb_wts[pair0 + slot];
+                    if (wt > 0.0f)
+                        __hip_atomic_fetch_add(args.comb_y + (size_t)args.comb_rows[pair0 + slot] * (size_t)args.comb_D + (size_t)row, wt * o[r],
+                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                return;
+            }
+        }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int slot = 4 * q + r;
@@ -1591,7 +1620,8 @@ int plan_grouped(int K, bool x_f32, const int* nrows, const int* nrows_x, int np
 }
 
 template <int FMT>
-int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_bf16, hipStream_t s, const GemvDirect* direct = nullptr) {
+int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_bf16, hipStream_t s, const GemvDirect* direct = nullptr,
+                float* zero = nullptr, int nzero = 0) {
     const int nblocks = gp.K >> 8;
     GemvKernArgs k{};
     k.W0 = static_cast<const uint8_t*>(d_table);
@@ -1608,6 +1638,7 @@ int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, 
         xin = direct->x;
     }
     k.K = gp.K; k.y_bf16 = y_bf16; k.nslot = 0; k.tiles_per_wg = gp.T;
+    k.zero = zero; k.nzero = nzero;
     k.cols_base = nblocks / gp.NW; k.cols_rem = nblocks % gp.NW;
     using Kernel = void (*)(GemvKernArgs, const void*);
     constexpr int WDG = 2;  // two unit fetches in flight: every format's kernel holds that many without spilling
@@ -1687,8 +1718,9 @@ int plan_rows16_grouped(int K, const int* nrows, int nprob, GemvGroupPlan* gp) {
 }
 
 template <int FMT>
-int run_rows16_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_bf16, hipStream_t s) {
+int run_rows16_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_bf16, hipStream_t s, const GemvCombine* comb) {
     GemvKernArgs k{};
+    if (comb) { k.comb_rows = comb->rows; k.comb_wts = comb->weights; k.comb_y = comb->y; k.comb_D = comb->D; }
     k.W0 = static_cast<const uint8_t*>(d_table);
     k.W1 = reinterpret_cast<const uint8_t*>(d_map);
     k.K = gp.K; k.y_bf16 = y_bf16; k.tiles_per_wg = gp.T;
@@ -1715,13 +1747,14 @@ int plan_gemv_rows16_grouped(int fmt, int K, const int* nrows, int nprob, GemvGr
     }
 }
 
-int launch_gemv_rows16_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s) {
+int launch_gemv_rows16_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s,
+                               const GemvCombine* comb) {
     const int yb = y_dtype == TFQ_BF16;
     switch (canonical(fmt)) {
-        case TFQ_Q_G_4: return run_rows16_grouped<TFQ_Q_G_4>(gp, d_table, d_map, yb, s);
-        case TFQ_B32S4: return run_rows16_grouped<TFQ_B32S4>(gp, d_table, d_map, yb, s);
-        case TFQ_B32S8: return run_rows16_grouped<TFQ_B32S8>(gp, d_table, d_map, yb, s);
-        case TFQ_Q_G_8: return run_rows16_grouped<TFQ_Q_G_8>(gp, d_table, d_map, yb, s);
+        case TFQ_Q_G_4: return run_rows16_grouped<TFQ_Q_G_4>(gp, d_table, d_map, yb, s, comb);
+        case TFQ_B32S4: return run_rows16_grouped<TFQ_B32S4>(gp, d_table, d_map, yb, s, comb);
+        case TFQ_B32S8: return run_rows16_grouped<TFQ_B32S8>(gp, d_table, d_map, yb, s, comb);
+        case TFQ_Q_G_8: return run_rows16_grouped<TFQ_Q_G_8>(gp, d_table, d_map, yb, s, comb);
         default: return fail(TFQ_ERR_FORMAT, "gemv group: no sixteen-row kernel for this format");
     }
 }
@@ -1766,12 +1799,12 @@ int plan_gemv_grouped(int fmt, int K, bool x_f32, const int* nrows, const int* n
 // Fills the host images of the problem table (nprob entries of gemv_group_entry_bytes() each) and of the
 // workgroup map (gp.grid ints).
 void fill_gemv_group(const GemvGroupPlan& gp, const tfq_weight* const* ws, const void* const* xs, void* const* ys,
-                     const int* nrows_x, int nprob, void* table_host, int* map_host, const tfq_weight* const* ws2) {
+                     const int* nrows_x, int nprob, void* table_host, int* map_host, const tfq_weight* const* ws2, const int* first_pair) {
     GemvProb* t = static_cast<GemvProb*>(table_host);
     int wg = 0;
     for (int i = 0; i < nprob; ++i) {
         const int n = ((int)((ws[i]->N + 15) / 16) + gp.T - 1) / gp.T;
-        t[i] = GemvProb{ws[i]->dev, ys[i], xs[i], ws2 ? ws2[i]->dev : nullptr, (int)ws[i]->N, gp.x_f32 ? 2 * nrows_x[i] : nrows_x[i], wg, 0};
+        t[i] = GemvProb{ws[i]->dev, ys[i], xs[i], ws2 ? ws2[i]->dev : nullptr, (int)ws[i]->N, gp.x_f32 ? 2 * nrows_x[i] : nrows_x[i], wg, first_pair ? first_pair[i] : 0};
         for (int j = 0; j < n; ++j) map_host[wg + j] = i;
         wg += n;
     }
@@ -1779,13 +1812,14 @@ void fill_gemv_group(const GemvGroupPlan& gp, const tfq_weight* const* ws, const
 
 size_t gemv_group_entry_bytes() { return sizeof(GemvProb); }
 
-int launch_gemv_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s) {
+int launch_gemv_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s, float* zero,
+                        int nzero) {
     const int yb = y_dtype == TFQ_BF16;
     switch (canonical(fmt)) {
-        case TFQ_Q_G_4: return run_grouped<TFQ_Q_G_4>(gp, d_table, d_map, yb, s);
-        case TFQ_B32S4: return run_grouped<TFQ_B32S4>(gp, d_table, d_map, yb, s);
-        case TFQ_B32S8: return run_grouped<TFQ_B32S8>(gp, d_table, d_map, yb, s);
-        case TFQ_Q_G_8: return run_grouped<TFQ_Q_G_8>(gp, d_table, d_map, yb, s);
+        case TFQ_Q_G_4: return run_grouped<TFQ_Q_G_4>(gp, d_table, d_map, yb, s, nullptr, zero, nzero);
+        case TFQ_B32S4: return run_grouped<TFQ_B32S4>(gp, d_table, d_map, yb, s, nullptr, zero, nzero);
+        case TFQ_B32S8: return run_grouped<TFQ_B32S8>(gp, d_table, d_map, yb, s, nullptr, zero, nzero);
+        case TFQ_Q_G_8: return run_grouped<TFQ_Q_G_8>(gp, d_table, d_map, yb, s, nullptr, zero, nzero);
         default: return fail(TFQ_ERR_FORMAT, "gemv group: no grouped kernel for this format");
     }
 }

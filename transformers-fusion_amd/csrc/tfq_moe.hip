@@ -397,7 +397,7 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
     std::vector<const tfq_weight*> wA, wA2, wB;
     std::vector<const void*> xA, xB;
     std::vector<void*> yA, yB;
-    std::vector<int> nA, nB, rA, rB;
+    std::vector<int> nA, nB, rA, rB, pB;  // pB: first pair of a down problem
     if (grouped) {
         int max_nt = 1;
         for (int e = 0; e < E; ++e) max_nt = std::max(max_nt, first[e + 1] - first[e]);
@@ -450,6 +450,7 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
                 yB.push_back(ws.o + (size_t)(p0 + b0) * D);
                 nB.push_back((int)D);
                 rB.push_back(nb);
+                pB.push_back(p0 + b0);
             }
         }
         if (int rc = plan_gemv_grouped(gate[0]->fmt, (int)D, x_dtype == TFQ_F32, nA.data(), rA.data(), (int)nA.size(), &planA, true)) return rc;
@@ -506,7 +507,7 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
     if (grouped) {
         uint8_t* lb = reinterpret_cast<uint8_t*>(lists);
         fill_gemv_group(planA, wA.data(), xA.data(), yA.data(), rA.data(), (int)wA.size(), lb + tabA, reinterpret_cast<int*>(lb + mapA), wA2.data());
-        fill_gemv_group(planB, wB.data(), xB.data(), yB.data(), rB.data(), (int)wB.size(), lb + tabB, reinterpret_cast<int*>(lb + mapB));
+        fill_gemv_group(planB, wB.data(), xB.data(), yB.data(), rB.data(), (int)wB.size(), lb + tabB, reinterpret_cast<int*>(lb + mapB), nullptr, pB.data());
     }
     int* h_rows = lists;
     int* h_pairs = h_rows + P;
@@ -533,8 +534,15 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
                            (const uint4*)x, (uint4*)ws.xe, d_rows, P, row_u4);
     }
     const uint8_t* d_lists = reinterpret_cast<const uint8_t*>(ws.lists);
+    // Tokens of at most two slots, an fp32 y and the sixteen-row down launch: that launch adds weight x product into
+    // y itself (the gate / up launch zeroes y on its way) and no combine launch follows: two addends onto zero are the
+    // bits of the combine step in either order.  (The capacity form keeps pairs whatever their weight's sign and
+    // takes the combine launch.)
+    const bool fused_combine = grouped && down16 && Ktop <= 2 && y_dtype == TFQ_F32 && !keep_all && nout <= 0x7FFFFFFF;
     if (grouped) {
-        if (int rc = launch_gemv_grouped(gate[0]->fmt, planA, d_lists + tabA, reinterpret_cast<const int*>(d_lists + mapA), mid_dtype, s)) return rc;
+        if (int rc = launch_gemv_grouped(gate[0]->fmt, planA, d_lists + tabA, reinterpret_cast<const int*>(d_lists + mapA), mid_dtype, s,
+                                         fused_combine ? static_cast<float*>(y) : nullptr, fused_combine ? (int)nout : 0))
+            return rc;
     }
     if (tall_grouped) {
         if (int rc = launch_gemm_grouped(gate[0]->fmt, gplanA, d_lists + tabA, reinterpret_cast<const int*>(d_lists + mapA), s)) return rc;
@@ -561,6 +569,10 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
             hipLaunchKernelGGL(silu_mul_kernel<false>, dim3((unsigned)((nh + 255) / 256)), dim3(256), 0, s, ws.g, ws.u, (void*)ws.h, nh);
     }
     if (grouped) {
+        if (fused_combine) {
+            const GemvCombine comb{d_rows, d_w, static_cast<float*>(y), (int)D};
+            return launch_gemv_rows16_grouped(down[0]->fmt, planB, d_lists + tabB, reinterpret_cast<const int*>(d_lists + mapB), TFQ_F32, s, &comb);
+        }
         if (down16) {
             if (int rc = launch_gemv_rows16_grouped(down[0]->fmt, planB, d_lists + tabB, reinterpret_cast<const int*>(d_lists + mapB), TFQ_F32, s)) return rc;
         } else if (int rc = launch_gemv_grouped(down[0]->fmt, planB, d_lists + tabB, reinterpret_cast<const int*>(d_lists + mapB), TFQ_F32, s)) {
@@ -726,7 +738,7 @@ __global__ __launch_bounds__(1024) void routed_lists_kernel(const int32_t* __res
                                 sh.nrowsA, min(sh.capA, nt - b0), iA * s_wgA, s_tilesA};
         for (int b0 = 0; b0 < nt; b0 += sh.capB, ++iB)
             tabB[iB] = GemvProb{ptrs[2 * E + e], o + (size_t)(p0 + b0) * sh.strideYB, h + (size_t)(p0 + b0) * sh.strideXB, nullptr,
-                                sh.nrowsB, min(sh.capB, nt - b0), iB * sh.wgB, 0};
+                                sh.nrowsB, min(sh.capB, nt - b0), iB * sh.wgB, p0 + b0};  // (tiles: the problem's first pair)
     }
     __syncthreads();
     const int nA = s_nA, nB = s_nB;
@@ -879,13 +891,23 @@ int launch_moe_ffn_routed(const tfq_weight* const* gate, const tfq_weight* const
     if (!fuse_gather)
         hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)((ng + 255) / 256)), dim3(256), 0, s, (const uint4*)x, (uint4*)xe, (const int*)d_rows, (int)P, row_u4);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return hip_fail(e, "moe routed launch");
-    if (int rc = launch_gemv_grouped(gate[0]->fmt, rp.planA, tabA, mapA, TFQ_BF16, s)) return rc;
+    // Tokens of at most two slots and an fp32 y: no combine launch.  The gate / up launch zeroes y on its way and the
+    // down launch adds weight x product into the token's row with atomics; two addends onto zero give the bits of the
+    // combine step (0 + w0 o0 + w1 o1) in either order.
+    const int64_t nout = (int64_t)T * (int64_t)D;
+    const bool fused_combine = Ktop <= 2 && y_dtype == TFQ_F32 && rp.down16 && nout <= 0x7FFFFFFF;
+    if (int rc = launch_gemv_grouped(gate[0]->fmt, rp.planA, tabA, mapA, TFQ_BF16, s, fused_combine ? static_cast<float*>(y) : nullptr,
+                                     fused_combine ? (int)nout : 0))
+        return rc;
+    if (fused_combine) {
+        const GemvCombine comb{d_rows, d_w, static_cast<float*>(y), (int)D};
+        return launch_gemv_rows16_grouped(down[0]->fmt, rp.planB, tabB, mapB, TFQ_F32, s, &comb);
+    }
     if (rp.down16) {
         if (int rc = launch_gemv_rows16_grouped(down[0]->fmt, rp.planB, tabB, mapB, TFQ_F32, s)) return rc;
     } else if (int rc = launch_gemv_grouped(down[0]->fmt, rp.planB, tabB, mapB, TFQ_F32, s)) {
         return rc;
     }
-    const int64_t nout = (int64_t)T * (int64_t)D;
     if (y_dtype == TFQ_BF16)
         hipLaunchKernelGGL(combine_kernel<true>, dim3((unsigned)((nout + 255) / 256)), dim3(256), 0, s, y, (const float*)o, (const int*)d_tokf, (const int*)d_tokp, (const float*)d_w, T, (int)D, 0);
     else
