@@ -162,6 +162,7 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
     // slot's routing weight and added into one vector with atomics when y1 holds the weights.
     float out_scale = 1.0f;
     bool out_atomic = false;
+    int pair0 = 0;
     if constexpr (GROUPED) {
         if (args.W2 != nullptr) {
             if (args.y2 != nullptr) {  // the vector the next launch adds into starts at zero
@@ -200,6 +201,7 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
             wg_first = pr.wg_first; nrm = pr.nrows; nslot = pr.nslot;
             Wm = pr.W; ym = pr.y; xin = pr.x;
             Wm2 = pr.W2;
+            pair0 = pr.tiles;  // (a down launch that adds into the tokens' rows: the problem's first pair, see below)
         }
     } else {
         const int m = (bid >= args.g0) + (bid >= args.g1) + (bid >= args.g2);
@@ -580,6 +582,13 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
         if constexpr (GROUPED) {
             if (out_atomic) {  // at most two slots add into a zeroed vector: the same bits in either order
                 __hip_atomic_fetch_add(reinterpret_cast<float*>(ym) + off, v * out_scale, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                continue;
+            }
+            if (args.comb_y != nullptr) {  // weight x product into the token's output row (see GemvKernArgs)
+                const float wt = args.comb_wts[pair0 + b];
+                if (wt > 0.0f)
+                    __hip_atomic_fetch_add(args.comb_y + (size_t)args.comb_rows[pair0 + b] * (size_t)args.comb_D + (size_t)row, v * wt,
+                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 continue;
             }
         }
@@ -1621,7 +1630,7 @@ int plan_grouped(int K, bool x_f32, const int* nrows, const int* nrows_x, int np
 
 template <int FMT>
 int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_bf16, hipStream_t s, const GemvDirect* direct = nullptr,
-                float* zero = nullptr, int nzero = 0) {
+                float* zero = nullptr, int nzero = 0, const GemvCombine* comb = nullptr) {
     const int nblocks = gp.K >> 8;
     GemvKernArgs k{};
     k.W0 = static_cast<const uint8_t*>(d_table);
@@ -1639,6 +1648,10 @@ int run_grouped(const GemvGroupPlan& gp, const void* d_table, const int* d_map, 
     }
     k.K = gp.K; k.y_bf16 = y_bf16; k.nslot = 0; k.tiles_per_wg = gp.T;
     k.zero = zero; k.nzero = nzero;
+    if (comb) {
+        if (gp.rows || gp.x_f32 || gp.pair) return fail(TFQ_ERR_ARG, "gemv group: adding into the tokens' rows is for a plain bf16 launch");
+        k.comb_rows = comb->rows; k.comb_wts = comb->weights; k.comb_y = comb->y; k.comb_D = comb->D;
+    }
     k.cols_base = nblocks / gp.NW; k.cols_rem = nblocks % gp.NW;
     using Kernel = void (*)(GemvKernArgs, const void*);
     constexpr int WDG = 2;  // two unit fetches in flight: every format's kernel holds that many without spilling
@@ -1813,13 +1826,13 @@ void fill_gemv_group(const GemvGroupPlan& gp, const tfq_weight* const* ws, const
 size_t gemv_group_entry_bytes() { return sizeof(GemvProb); }
 
 int launch_gemv_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s, float* zero,
-                        int nzero) {
+                        int nzero, const GemvCombine* comb) {
     const int yb = y_dtype == TFQ_BF16;
     switch (canonical(fmt)) {
-        case TFQ_Q_G_4: return run_grouped<TFQ_Q_G_4>(gp, d_table, d_map, yb, s, nullptr, zero, nzero);
-        case TFQ_B32S4: return run_grouped<TFQ_B32S4>(gp, d_table, d_map, yb, s, nullptr, zero, nzero);
-        case TFQ_B32S8: return run_grouped<TFQ_B32S8>(gp, d_table, d_map, yb, s, nullptr, zero, nzero);
-        case TFQ_Q_G_8: return run_grouped<TFQ_Q_G_8>(gp, d_table, d_map, yb, s, nullptr, zero, nzero);
+        case TFQ_Q_G_4: return run_grouped<TFQ_Q_G_4>(gp, d_table, d_map, yb, s, nullptr, zero, nzero, comb);
+        case TFQ_B32S4: return run_grouped<TFQ_B32S4>(gp, d_table, d_map, yb, s, nullptr, zero, nzero, comb);
+        case TFQ_B32S8: return run_grouped<TFQ_B32S8>(gp, d_table, d_map, yb, s, nullptr, zero, nzero, comb);
+        case TFQ_Q_G_8: return run_grouped<TFQ_Q_G_8>(gp, d_table, d_map, yb, s, nullptr, zero, nzero, comb);
         default: return fail(TFQ_ERR_FORMAT, "gemv group: no grouped kernel for this format");
     }
 }

@@ -424,9 +424,18 @@ size_t gemv_group_entry_bytes();
 void fill_gemv_group(const GemvGroupPlan& gp, const tfq_weight* const* ws, const void* const* xs, void* const* ys,
                      const int* nrows_x, int nprob, void* table_host, int* map_host, const tfq_weight* const* ws2 = nullptr,
                      const int* first_pair = nullptr);  // first_pair: GemvProb::tiles of every problem (see GemvCombine)
+// With `comb` a grouped launch (either kernel) adds routing weight x product of pair (problem's first pair + slot) into
+// y[rows[pair]][.] with atomics instead of writing a row per pair: for tokens of at most two pairs and a y that starts
+// at zero the sums do not depend on the order.  The problem's first pair rides in GemvProb::tiles.
+struct GemvCombine {
+    const int* rows;
+    const float* weights;
+    float* y;
+    int D;
+};
 // (zero / nzero: fp32 words the launch sets to zero on its way, for a following launch that adds into them)
 int launch_gemv_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s,
-                        float* zero = nullptr, int nzero = 0);
+                        float* zero = nullptr, int nzero = 0, const GemvCombine* comb = nullptr);
 // The grouped launch for the slots of ONE token (at most two when `weights` is given): no table; the kernel reads the
 // slot's expert id and takes the matrix address from `ptrs` ([gate | up | down][E] device addresses; matrix = 0 for
 // the gate / up pair, 2 for down).  Slot p reads x + p * x_stride and writes y + p * y_stride; with `weights` the
@@ -447,15 +456,6 @@ struct GemvDirect {
 int launch_gemv_grouped_direct(int fmt, const GemvGroupPlan& gp, const GemvDirect& d, int y_dtype, hipStream_t s);
 // the same for problems of up to sixteen bf16 activation rows at any K (gemvb_kernel; tables from fill_gemv_group)
 int plan_gemv_rows16_grouped(int fmt, int K, const int* nrows, int nprob, GemvGroupPlan* gp);
-// With `comb` the sixteen-row launch adds routing weight x product of pair (problem's first pair + slot) into
-// y[rows[pair]][.] with atomics instead of writing a row per pair: for tokens of at most two pairs and a y that starts
-// at zero the sums do not depend on the order.  The problem's first pair rides in GemvProb::tiles.
-struct GemvCombine {
-    const int* rows;
-    const float* weights;
-    float* y;
-    int D;
-};
 int launch_gemv_rows16_grouped(int fmt, const GemvGroupPlan& gp, const void* d_table, const int* d_map, int y_dtype, hipStream_t s,
                                const GemvCombine* comb = nullptr);
 size_t moe_workspace_bytes(int T, int Ktop, int64_t D, int64_t F);

@@ -538,7 +538,7 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
     // y itself (the gate / up launch zeroes y on its way) and no combine launch follows: two addends onto zero are the
     // bits of the combine step in either order.  (The capacity form keeps pairs whatever their weight's sign and
     // takes the combine launch.)
-    const bool fused_combine = grouped && down16 && Ktop <= 2 && y_dtype == TFQ_F32 && !keep_all && nout <= 0x7FFFFFFF;
+    const bool fused_combine = grouped && mid_dtype == TFQ_BF16 && Ktop <= 2 && y_dtype == TFQ_F32 && !keep_all && nout <= 0x7FFFFFFF;
     if (grouped) {
         if (int rc = launch_gemv_grouped(gate[0]->fmt, planA, d_lists + tabA, reinterpret_cast<const int*>(d_lists + mapA), mid_dtype, s,
                                          fused_combine ? static_cast<float*>(y) : nullptr, fused_combine ? (int)nout : 0))
@@ -571,7 +571,8 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
     if (grouped) {
         if (fused_combine) {
             const GemvCombine comb{d_rows, d_w, static_cast<float*>(y), (int)D};
-            return launch_gemv_rows16_grouped(down[0]->fmt, planB, d_lists + tabB, reinterpret_cast<const int*>(d_lists + mapB), TFQ_F32, s, &comb);
+            if (down16) return launch_gemv_rows16_grouped(down[0]->fmt, planB, d_lists + tabB, reinterpret_cast<const int*>(d_lists + mapB), TFQ_F32, s, &comb);
+            return launch_gemv_grouped(down[0]->fmt, planB, d_lists + tabB, reinterpret_cast<const int*>(d_lists + mapB), TFQ_F32, s, nullptr, 0, &comb);
         }
         if (down16) {
             if (int rc = launch_gemv_rows16_grouped(down[0]->fmt, planB, d_lists + tabB, reinterpret_cast<const int*>(d_lists + mapB), TFQ_F32, s)) return rc;
@@ -895,13 +896,14 @@ int launch_moe_ffn_routed(const tfq_weight* const* gate, const tfq_weight* const
     // down launch adds weight x product into the token's row with atomics; two addends onto zero give the bits of the
     // combine step (0 + w0 o0 + w1 o1) in either order.
     const int64_t nout = (int64_t)T * (int64_t)D;
-    const bool fused_combine = Ktop <= 2 && y_dtype == TFQ_F32 && rp.down16 && nout <= 0x7FFFFFFF;
+    const bool fused_combine = Ktop <= 2 && y_dtype == TFQ_F32 && nout <= 0x7FFFFFFF;
     if (int rc = launch_gemv_grouped(gate[0]->fmt, rp.planA, tabA, mapA, TFQ_BF16, s, fused_combine ? static_cast<float*>(y) : nullptr,
                                      fused_combine ? (int)nout : 0))
         return rc;
     if (fused_combine) {
         const GemvCombine comb{d_rows, d_w, static_cast<float*>(y), (int)D};
-        return launch_gemv_rows16_grouped(down[0]->fmt, rp.planB, tabB, mapB, TFQ_F32, s, &comb);
+        if (rp.down16) return launch_gemv_rows16_grouped(down[0]->fmt, rp.planB, tabB, mapB, TFQ_F32, s, &comb);
+        return launch_gemv_grouped(down[0]->fmt, rp.planB, tabB, mapB, TFQ_F32, s, nullptr, 0, &comb);
     }
     if (rp.down16) {
         if (int rc = launch_gemv_rows16_grouped(down[0]->fmt, rp.planB, tabB, mapB, TFQ_F32, s)) return rc;
