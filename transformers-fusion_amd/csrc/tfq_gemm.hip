@@ -653,12 +653,12 @@ int launch_gemm_grouped(int fmt, const GemmGroupPlan& gp, const void* d_table, c
 // Few tokens make few workgroups for the tile kernel, while the batched decode kernel reads the matrix once
 // per 16 rows with every compute unit busy: a 16-row pass costs (us) 2.5 + 3.2 per 4096 of K (activation
 // staging) + bytes / 6.5 TB/s, plus 15 %; where that kernel splits K over workgroups (K above 4096, partial
-// sums kept with the handle) the staging is paid once and the parts' meeting costs 6 us.  Measured crossovers
+// sums kept with the handle) the staging is paid once and the launch that adds the parts costs 3.5 us.  Measured crossovers
 // without a K split of the tile kernel: 72 tokens at 14336x4096, 115 at 4096x4096, 125 at 4096x14336 (4-bit).
 static bool slices_cheaper(const tfq_weight* w, int M, double tile_us) {
     if (!gemv_rows16_supported(w->fmt)) return false;
     const double chunks = std::ceil((double)w->K / 4096.0);
-    const double staging = chunks > 1.0 && w->split_partial ? 3.2 + 6.0 : 3.2 * chunks;
+    const double staging = chunks > 1.0 && w->split_partial ? 3.2 + 3.5 : 3.2 * chunks;
     const double t16 = 1.15 * (2.5 + staging + (double)w->dev_bytes / 6.5e6);
     return (double)((M + 15) / 16) * t16 < tile_us;
 }
