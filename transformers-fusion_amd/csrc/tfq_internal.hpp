@@ -403,7 +403,9 @@ struct GemvProb {
     int nrows;
     int nslot;
     int wg_first;  // first workgroup of this problem
-    int tiles;     // tiles per workgroup of this problem where a table built on the device chooses them (0: the launch's)
+    int tiles;     // gate / up launch in gemvr_kernel: tiles per workgroup of this problem where a table built on the
+                   // device chooses them (0: the launch's); down launch that adds into the tokens' rows (GemvCombine):
+                   // the problem's first pair
 };
 
 struct GemvGroupPlan {
