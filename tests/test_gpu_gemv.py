@@ -235,6 +235,27 @@ def test_config4_lowbit_superblock_shapes(O, tfq, gpu, fmt, bits):
     W.close()
 
 
+@pytest.mark.parametrize("fmt", ["SB256A3", "SB256A2", "Q_G_2"])
+@pytest.mark.parametrize("N,K", [(4200, 1024), (40, 14336), (1000, 2304)])
+def test_one_row_of_the_byte_header_formats(O, tfq, gpu, fmt, N, K):
+    """One bf16 row of the formats with sixteen 16-weight groups runs the kernel variant in which every lane row
+    decodes the scales of its own 32 weights: several tiles per workgroup with a partial last tile, two fetches in
+    flight, uneven block columns per wavefront; the same matrix at two rows (the other variant) as a cross-check."""
+    import torch
+    w = O.rng_laplace(44, N * K, 0.015)
+    pay = O.encode_tensor(fmt, w)
+    W = tfq.Weight(fmt, N, K, pay)
+    x = O.bf16_round(O.rng_normal(43, 2 * K, 1.0).reshape(2, K))
+    ref = O.matmul(fmt, pay, N, K, x)
+    xg = torch.from_numpy(x).to(gpu).bfloat16()
+    y1 = W.gemv(xg[:1].contiguous()).cpu().numpy()
+    y2 = W.gemv(xg).cpu().numpy()
+    assert rel_err(y1, ref[:1]) <= 1e-4
+    assert rel_err(y2, ref) <= 1e-4
+    assert rel_err(y1, y2[:1]) <= 1e-5
+    W.close()
+
+
 @pytest.mark.parametrize("fmt", ["Q_G_8", "Q_8", "B32S8"])
 @pytest.mark.parametrize("N,K", [(256, 4096), (48, 14336), (1040, 1024)])
 def test_config2_eight_bit_formats(O, tfq, gpu, fmt, N, K):

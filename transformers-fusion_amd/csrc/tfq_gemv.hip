@@ -135,10 +135,18 @@ struct GemvKernArgs {
 // reads its A fragments from LDS per MFMA (two slot sets, 16-byte header)
 __host__ __device__ constexpr int a_slot_stride(int fmt, int sets) { return sets == 2 && tiled_header_bytes(fmt) == 16 ? 33 : 32; }
 
-template <int FMT, bool XF32, int WD, int SETS = 1, bool GROUPED = false, int XOP = XOP_NONE, bool PAIR = false>
+template <int FMT, bool XF32, int WD, int SETS = 1, bool GROUPED = false, int XOP = XOP_NONE, bool PAIR = false, bool GM = false>
 __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1024 : 512) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin_arg) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
+    // GM ("group-major", one bf16 activation row, formats with byte headers): A row 4 c + s instead of 4 s + c, so
+    // that lane (n, q) ends up with the product of 32-slot q alone instead of those of all four 32-slots of
+    // activation slot q.  With one row three of the four lane rows otherwise repeat the first one's scale and
+    // offset arithmetic on zeros; here every lane decodes the two scale and the two offset codes of its own 32-slot
+    // (a quarter of the conversions and multiply-adds, which is what bounds these formats) and the four lane rows
+    // are added where the wavefronts' partial sums are.
+    static_assert(!GM || (tiled_header_in_bytes(FMT) && F::GS == 16 && !XF32 && SETS == 1 && !GROUPED && XOP == XOP_NONE && !PAIR),
+                  "group-major: one bf16 row, byte headers, the plain launch");
     static_assert(XOP == XOP_NONE || (XF32 && SETS == 1 && !GROUPED), "prologues take fp32 input in the plain launch");
     static_assert(!PAIR || ((GROUPED || SETS == 1) && XOP != XOP_SWIGLU), "the paired launch: one slot set unless grouped");
     constexpr int UB = tiled_unit_bytes(FMT);  // bytes of a unit
@@ -426,11 +434,24 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
     // per block column, not per unit
     constexpr bool XPRE = FMT == TFQ_B32S4 || F::NP == 2;
     int c_ci = 0, c_t = 0;
+    const uint32_t gm_shift = (uint32_t)(q & 1) * 16u;  // GM: where the lane's two codes sit in their dword
     float* cell = part + wave * SETS * 64 + lane;  // this wavefront's cells of tile c_t, one per slot set
     auto consume = [&](int u) __attribute__((always_inline)) {
         if (c_t == 0) {  // new block column: its two k-steps' A fragments and group sums
             const uint4* col = my + (size_t)c_ci * col_stride;
             const float* colX = reinterpret_cast<const float*>(col + a_per_col);
+            if constexpr (GM) {
+                const bool live = (n >> 2) == q && (n & 3) == 0;  // A row 4 q of slot 0
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const uint4* src = live ? col + h * 16 + q * 4 : zero4;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) av[0][h][j] = src[j];
+                    const float2 f = *reinterpret_cast<const float2*>(colX + h * PER + 2 * q);  // groups 2 q, 2 q + 1
+                    xv[0][h][0] = f.x; xv[0][h][1] = f.y;
+                    xv[0][h][2] = -F::OFFS * f.x; xv[0][h][3] = -F::OFFS * f.y;
+                }
+            } else
 #pragma unroll
             for (int st = 0; st < SETS; ++st) {
                 const bool live = (c_a == q) && (4 * st + s_a < nslot);
@@ -472,7 +493,10 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
             for (int st = 0; st < SETS; ++st) {
                 const float* X = xv[st][h];
                 DB[st] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-                if constexpr (XPRE) {
+                if constexpr (GM) {
+                    DA[st] = f32x4_t{X[2], 0.0f, 0.0f, 0.0f};
+                    DB[st] = f32x4_t{X[3], 0.0f, 0.0f, 0.0f};
+                } else if constexpr (XPRE) {
                     DA[st] = f32x4_t{X[0], X[1], X[2], X[3]};
                 } else if constexpr (F::GS == 32) {
                     DA[st] = f32x4_t{-F::OFFS * X[0], -F::OFFS * X[1], -F::OFFS * X[2], -F::OFFS * X[3]};
@@ -515,7 +539,8 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
             }
 #pragma unroll
             for (int st = 0; st < SETS; ++st) {
-                if constexpr (SXK) res[st] += apply_groups<FMT, true>(hd[u], h, DA[st], DB[st], xv[st][h], sxv[st][h]);
+                if constexpr (GM) res[st] += apply_own_groups<FMT>(hd[u], h, gm_shift, q >= 2, DA[st][0], DB[st][0], xv[st][h][0], xv[st][h][1]);
+                else if constexpr (SXK) res[st] += apply_groups<FMT, true>(hd[u], h, DA[st], DB[st], xv[st][h], sxv[st][h]);
                 else res[st] += apply_groups<FMT>(hd[u], h, DA[st], DB[st], xv[st][h]);
             }
         }
@@ -559,8 +584,12 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
         const float* src = part + (t * NW * SETS + (s0 >> 2)) * 64 + (s0 & 3) * 16 + nn;
         float v = 0.0f;
         for (int w = 0; w < NW; ++w) {
+            if constexpr (GM) {  // the four lane rows hold the four 32-slots' shares of the one activation row
+                v += (src[w * 64] + src[w * 64 + 16]) + (src[w * 64 + 32] + src[w * 64 + 48]);
+            } else {
 #pragma unroll
-            for (int h = 0; h < rows_per_out; ++h) v += src[w * SETS * 64 + h * 16];
+                for (int h = 0; h < rows_per_out; ++h) v += src[w * SETS * 64 + h * 16];
+            }
         }
         float v2 = 0.0f;  // PAIR: the up product of the same output
         if constexpr (PAIR) {
@@ -1435,9 +1464,16 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     } else if (p.sets > 1) {
         return fail(TFQ_ERR_SHAPE, "gemv: more than four rows in one pass for this format");
     }
+    if constexpr (tiled_header_in_bytes(FMT) && Fmt<FMT>::GS == 16) {
+        // one bf16 row: every lane row takes the scale arithmetic of its own 32-slot (GM in the kernel)
+        if (a.nslot == 1 && !a.x_f32 && !a.pair && a.xop == XOP_NONE && p.sets == 1) {
+            kern = wd == 2 ? gemv4_kernel<FMT, false, 2, 1, false, XOP_NONE, false, true> : gemv4_kernel<FMT, false, 1, 1, false, XOP_NONE, false, true>;
+            slot = wd == 2 ? 21 : 20;
+        }
+    }
     // Raise the dynamic-LDS limit once per kernel (not per launch: the call is
     // not allowed while a stream is being captured into a graph).
-    static std::atomic<bool> lds_limit_raised[20] = {};
+    static std::atomic<bool> lds_limit_raised[22] = {};
     if (!lds_limit_raised[slot]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);

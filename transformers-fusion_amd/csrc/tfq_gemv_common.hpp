@@ -77,15 +77,14 @@ struct Fmt {
 // in the scale), which costs under a tenth of the 1e-3 output tolerance.  Decode keeps the table.
 constexpr float kComp8Gain = 1.0000742443371564f / 127.5f;
 
-// byte B of a dword as a float (v_cvt_f32_ubyteB)
+// byte B of a dword as a float: one v_cvt_f32_ubyteB.  Plain C on purpose.  Written as an inline-assembly
+// instruction it gave wrong sums in a kernel that uses one row of an accumulator only: the register allocator
+// hands the three dead rows out again while the matrix instruction that writes them is still in flight, the
+// conversion landed in one of them and was overwritten when that instruction retired; the compiler inserts the
+// wait this needs only for instructions it can see.  The optimizer picks the same instruction by itself.
 template <int B>
 __device__ __forceinline__ float byte_to_float(uint32_t v) {
-    float f;
-    if constexpr (B == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(v));
-    else if constexpr (B == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(v));
-    else if constexpr (B == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(v));
-    else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(v));
-    return f;
+    return (float)((v >> (8 * B)) & 0xFFu);
 }
 
 // `count` bits at bit `pos` (both compile-time after unrolling) of the little-endian bit string w[0], w[1], ...
@@ -173,6 +172,24 @@ __device__ __forceinline__ float apply_groups(const uint4* hv, int khalf, f32x4_
         }
     }
     return res;
+}
+
+// The same contribution for ONE 32-slot of a format with byte headers and 16-weight groups: groups 2 q and
+// 2 q + 1 of k-step `khalf`, whose code bytes sit at bit `shift` (0 or 16) of the low (q < 2) or high word of
+// the k-step's eight bytes.  D0 / D1 are the two groups' dot products, X0 / X1 their activation sums.
+template <int FMT>
+__device__ __forceinline__ float apply_own_groups(const uint4* hv, int khalf, uint32_t shift, bool high_word, float D0, float D1, float X0, float X1) {
+    constexpr Spec sp = spec_of(FMT);
+    constexpr int mbias = (1 << sp.mb) / 2;
+    constexpr float inv_top = sp.bits == 4 ? 1.0f / 15.0f : sp.bits == 3 ? 1.0f / 7.0f : 1.0f / 3.0f;
+    const uint32_t sc_lo = khalf ? hv[0].z : hv[0].x, sc_hi = khalf ? hv[0].w : hv[0].y;
+    const uint32_t mc_lo = khalf ? hv[1].z : hv[1].x, mc_hi = khalf ? hv[1].w : hv[1].y;
+    const uint32_t scw = (high_word ? sc_hi : sc_lo) >> shift, mcw = (high_word ? mc_hi : mc_lo) >> shift;
+    const float dtop = half_fast(hv[2].x & 0xFFFFu) * inv_top;
+    const float dm = half_fast(hv[2].x >> 16);
+    const float sa = __builtin_fmaf(byte_to_float<1>(scw), D1, byte_to_float<0>(scw) * D0);
+    const float sm = __builtin_fmaf(byte_to_float<1>(mcw), X1, byte_to_float<0>(mcw) * X0);
+    return __builtin_fmaf(dtop, sa, dm * __builtin_fmaf((float)mbias, X0 + X1, -sm));
 }
 
 }  // namespace gemv_detail
