@@ -254,6 +254,7 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
     // A pass covers two activation slots of one block column: lane l < 32 owns the 8-element quad l
     // of slot s0, lane l + 32 the same quad of slot s0 + 1 (clamped to the last slot: the load is
     // unconditional and staging drops what it does not need).
+    constexpr bool GM2 = GM && (F::CW == 2 || spec_of(FMT).bits == 3);  // code fields taken without shifts, see the unpack
     constexpr int XP = XOP == XOP_NONE ? 4 : 2;  // passes whose loads are issued before the weight stream
     const int quad = lane & 31, sl_in_pass = lane >> 5;
     // passes per block column: a power of two, so that a pass index splits with shifts
@@ -346,6 +347,28 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
         uint4* col = my + (size_t)ci * col_stride;
         float* colX = reinterpret_cast<float*>(col + a_per_col);
         float sum = 0.0f;
+        if constexpr (GM2) {
+            // Both halves of the wavefront hold the one row's quad.  The lower half adds up the group sums; the upper
+            // half writes the A entries, divided by the weight that the shift-free field extraction leaves on the
+            // matching code (see the unpack below), and adds up the sums of those.
+            const uint4 p = pair_permute(xlo);
+            uint32_t d[4] = {p.x, p.y, p.z, p.w};
+            if (sl_in_pass) {
+                const bool odd = quad & 1;  // MFMA 2 j' + 1 of its 32-slot
+                const float sc[4] = {F::CW == 4 ? 1.0f : odd ? 0.25f : 1.0f, F::CW == 4 ? 0.0625f : odd ? 0.0625f : 0.25f,
+                                     F::CW == 4 ? 1.0f : odd ? 1.0f : 0.0625f, F::CW == 4 ? 0.0625f : odd ? 0.25f : 1.0f};
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const float lo = __uint_as_float(d[t] << 16) * sc[t], hi = __uint_as_float(d[t] & 0xFFFF0000u) * sc[t];
+                    d[t] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xFFFF0000u);  // exact: a power of two
+                }
+                col[quad] = uint4{d[0], d[1], d[2], d[3]};
+            }
+            sum = dot2(ONES, d[0], 0.0f);
+            sum = dot2(ONES, d[1], sum);
+            sum = dot2(ONES, d[2], sum);
+            sum = dot2(ONES, d[3], sum);
+        } else
         if (s < nslot) {
             uint4 v = xlo;
             if constexpr (XF32) {
@@ -449,7 +472,9 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
                     for (int j = 0; j < 4; ++j) av[0][h][j] = src[j];
                     const float2 f = *reinterpret_cast<const float2*>(colX + h * PER + 2 * q);  // groups 2 q, 2 q + 1
                     xv[0][h][0] = f.x; xv[0][h][1] = f.y;
-                    xv[0][h][2] = -F::OFFS * f.x; xv[0][h][3] = -F::OFFS * f.y;
+                    // what the accumulators start from: the sums of the A entries as the matrix cores see them
+                    const float2 fa = GM2 ? *reinterpret_cast<const float2*>(colX + NG + h * PER + 2 * q) : f;
+                    xv[0][h][2] = -F::OFFS * fa.x; xv[0][h][3] = -F::OFFS * fa.y;
                 }
             } else
 #pragma unroll
@@ -512,9 +537,22 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     uint4 wv;
-                    if constexpr (F::CW == 4) {
+                    if constexpr (F::CW == 4 && GM2) {
+                        // 3-bit codes in nibbles: the code of an odd nibble stays at bits 4..6 of the bf16 mantissa and
+                        // makes 128 + 16 n; its A entry was divided by 16 when it was staged
+                        const uint32_t v = qq[j], w8 = v >> 8;
+                        wv = uint4{(v & 0x00070007u) | C, (v & 0x00700070u) | C, (w8 & 0x00070007u) | C, (w8 & 0x00700070u) | C};
+                    } else if constexpr (F::CW == 4) {
                         const uint32_t v = qq[j];
                         wv = uint4{(v & M) | C, ((v >> 4) & M) | C, ((v >> 8) & M) | C, ((v >> 12) & M) | C};
+                    } else if constexpr (GM2) {
+                        // 2-bit fields left where they are in the bf16 mantissa: a field at bit 0, 2 or 4 of its half
+                        // makes 128 + n, 128 + 4 n or 128 + 16 n, and the A entry of that pair was divided by 1, 4 or
+                        // 16 when it was staged: ten operations per sixteen weights instead of fifteen.
+                        const uint32_t v = qq[2 * h + (j >> 1)];
+                        const uint32_t w6 = v >> 6, w12 = v >> 12;
+                        if ((j & 1) == 0) wv = uint4{(v & 0x00030003u) | C, (v & 0x000C000Cu) | C, (v & 0x00300030u) | C, (w6 & 0x00030003u) | C};
+                        else wv = uint4{(w6 & 0x000C000Cu) | C, (w6 & 0x00300030u) | C, (w12 & 0x00030003u) | C, (w12 & 0x000C000Cu) | C};
                     } else {
                         // 2-bit fields: dword 2h + j / 2 of the lane holds the pairs of two MFMAs
                         constexpr uint32_t M2 = 0x00030003u;
