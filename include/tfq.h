@@ -217,7 +217,14 @@ int tfq_weight_decode(const tfq_weight_t* w, float* out, tfq_stream_t stream);
  * 4096 of K) that calls with five or more bf16 rows or three or more fp32 rows
  * use: such calls on ONE
  * handle must not overlap in time (issue them on one stream, as the reference's
- * gemm is called; distinct handles are independent). */
+ * gemm is called; distinct handles are independent).
+ * K: any multiple of 256 for those five formats and for every format on the wire
+ * layout.  The other tiled formats (Q_G_3, Q_G_2, SB256A3, SB256A2) stage an
+ * activation row in on-chip memory, which holds K <= 61440 for a bf16 row and
+ * K <= 32768 for an fp32 row (49152 and 28672 for the three formats with
+ * sixteen scale groups per block); beyond that the call returns TFQ_ERR_SHAPE,
+ * as do the fused calls below (tfq_gemv_multi_fused, tfq_mlp_step) for every
+ * format at K above 32768. */
 int tfq_gemv(const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, int y_dtype,
              tfq_stream_t stream);
 int tfq_gemm(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, int y_dtype,

@@ -466,6 +466,26 @@ def test_gemv_k_split_soak(O, tfq, gpu):
     W.close()
 
 
+@pytest.mark.parametrize("fmt", ["B32S4", "Q_G_4", "B32S8"])
+@pytest.mark.parametrize("K,B,xdt", [(65536, 1, "bf16"), (65536, 3, "bf16"), (40960, 1, "f32"), (65536, 2, "f32")])
+def test_very_long_k(O, tfq, gpu, fmt, K, B, xdt):
+    """K beyond what one staged activation row leaves room for in LDS (61440 for a bf16 row, 32768 for an fp32
+    row): the product goes through the kernel whose wavefronts fetch their own activation fragments."""
+    import torch
+    N = 48
+    pay = O.encode_tensor(fmt, O.rng_normal(63, N * K, 0.02))
+    W = tfq.Weight(fmt, N, K, pay)
+    x = O.rng_normal(64, B * K, 1.0).reshape(B, K)
+    if xdt == "bf16":
+        x = O.bf16_round(x)
+        y = W.gemv(torch.from_numpy(x).to(gpu).bfloat16()).cpu().numpy()
+    else:
+        y = W.gemv(torch.from_numpy(x).to(gpu)).cpu().numpy()
+    ref = O.matmul(fmt, pay, N, K, x)
+    assert float(np.abs(y - ref).max() / np.abs(ref).max()) <= (1e-4 if xdt == "bf16" else 1e-3)
+    W.close()
+
+
 @pytest.mark.parametrize("K,B,xdt", [(28672, 4, "bf16"), (28672, 2, "f32"), (20480, 4, "bf16"), (32768, 3, "f32")])
 def test_long_k_takes_fewer_rows_per_pass(O, tfq, gpu, K, B, xdt):
     """K above 16384 leaves LDS room for fewer staged rows per pass; the product must still run (and match)."""

@@ -1599,6 +1599,8 @@ int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t 
         const int slots = a.x_f32 ? 2 * B : B, per_pass = a.x_f32 ? 8 : 16;
         bool dense_rows = slots > 8;
         if (slots > 4 && slots <= 8) dense_rows = plan_gemv4<FMT>(a, 8).lds == 0;
+        // and at any row count where not even one row's staged slices fit (K above 61440, above 32768 for fp32 rows)
+        if (!dense_rows) dense_rows = plan_gemv4<FMT>(a, a.x_f32 ? 2 : 1).lds == 0;
         if (a.xop != XOP_NONE || a.pair) dense_rows = false;
         if (dense_rows) {
             for (int b0 = 0; b0 < B; b0 += per_pass) {
