@@ -486,6 +486,28 @@ def test_very_long_k(O, tfq, gpu, fmt, K, B, xdt):
     W.close()
 
 
+@pytest.mark.parametrize("fmt,K,xdt,ok", [("SB256A2", 49152, "bf16", True), ("SB256A2", 49408, "bf16", False),
+                                          ("Q_G_3", 61440, "bf16", True), ("Q_G_3", 61696, "bf16", False),
+                                          ("SB256A3", 28672, "f32", True), ("SB256A3", 28928, "f32", False)])
+def test_k_ceiling_of_the_staged_formats(O, tfq, gpu, fmt, K, xdt, ok):
+    """The tiled formats outside the sixteen-row kernel run up to the documented K and refuse the next block with
+    an error before anything is launched."""
+    import torch
+    N = 16
+    pay = O.encode_tensor(fmt, O.rng_laplace(65, N * K, 0.015))
+    W = tfq.Weight(fmt, N, K, pay)
+    x = O.rng_normal(66, K, 1.0).reshape(1, K)
+    xg = torch.from_numpy(O.bf16_round(x)).to(gpu).bfloat16() if xdt == "bf16" else torch.from_numpy(x).to(gpu)
+    if ok:
+        y = W.gemv(xg).cpu().numpy()
+        ref = O.matmul(fmt, pay, N, K, O.bf16_round(x) if xdt == "bf16" else x)
+        assert float(np.abs(y - ref).max() / np.abs(ref).max()) <= 1e-3
+    else:
+        with pytest.raises(Exception, match="K too large"):
+            W.gemv(xg)
+    W.close()
+
+
 @pytest.mark.parametrize("K,B,xdt", [(28672, 4, "bf16"), (28672, 2, "f32"), (20480, 4, "bf16"), (32768, 3, "f32")])
 def test_long_k_takes_fewer_rows_per_pass(O, tfq, gpu, K, B, xdt):
     """K above 16384 leaves LDS room for fewer staged rows per pass; the product must still run (and match)."""
