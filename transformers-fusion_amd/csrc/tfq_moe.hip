@@ -631,10 +631,17 @@ __global__ __launch_bounds__(1024) void routed_lists_kernel(const int32_t* __res
     __shared__ int s_first[257];
     __shared__ int s_cnt[256];
     __shared__ int s_pair[kRoutedMaxPairs];
+    __shared__ float s_w[kRoutedMaxPairs];
     const int P = T * Ktop, tid = threadIdx.x;
+    // Everything the kernel reads from memory that does not depend on the lists is requested at once (the launch
+    // has 1024 threads, at least one per slot and per expert): the kernel is a chain of dependent memory round
+    // trips of 1.5-2 us each, and the routing arrays, the weights and the matrix addresses were three of them.
+    const uint8_t *p_gate = nullptr, *p_up = nullptr, *p_down = nullptr;
+    if (tid < E) { p_gate = ptrs[tid]; p_up = ptrs[E + tid]; p_down = ptrs[2 * E + tid]; }
     for (int e = tid; e < E; e += blockDim.x) s_cnt[e] = 0;
     for (int sl = tid; sl < P; sl += blockDim.x) {
         const int e = idx[sl];
+        s_w[sl] = w[sl];
         s_idx[sl] = e >= 0 && e < E ? e : -1;
     }
     __syncthreads();
@@ -655,10 +662,15 @@ __global__ __launch_bounds__(1024) void routed_lists_kernel(const int32_t* __res
         s_first[E] = acc;
     }
     __syncthreads();
-    for (int e = tid; e <= E; e += blockDim.x) first[e] = s_first[e];
+    // With the gather on board the launch has several workgroups: each builds the lists in its own LDS (a few
+    // hundred operations), all of them share the rows to move, and the first one writes lists and tables.
+    const bool lead = blockIdx.x == 0;
     const int total = s_first[E];
-    for (int p = total + tid; p < P; p += blockDim.x) rows[p] = 0;
-    if (tid == 0) wts[P] = 0.0f;
+    if (lead) {
+        for (int e = tid; e <= E; e += blockDim.x) first[e] = s_first[e];
+        for (int p = total + tid; p < P; p += blockDim.x) rows[p] = 0;
+        if (tid == 0) wts[P] = 0.0f;
+    }
     for (int sl = tid; sl < P; sl += blockDim.x) {
         const int e = s_idx[sl];
         if (e < 0) { s_pair[sl] = P; continue; }
@@ -666,21 +678,30 @@ __global__ __launch_bounds__(1024) void routed_lists_kernel(const int32_t* __res
         const int t = sl / Ktop;
         float wt = 0.0f;
         for (int j = 0; j < Ktop; ++j)
-            if (s_idx[t * Ktop + j] == e) { wt = w[t * Ktop + j]; break; }
-        rows[p] = t;
-        wts[p] = wt;
+            if (s_idx[t * Ktop + j] == e) { wt = s_w[t * Ktop + j]; break; }
+        if (lead) {
+            rows[p] = t;
+            wts[p] = wt;
+        }
         s_pair[sl] = p;
         s_tok[p] = t;
     }
     __syncthreads();
     // A decode-sized call: the pairs' activation rows are gathered here as well (x != null), which saves a launch
     if (x != nullptr) {
+        // (a compute unit moves about 130 GB/s: 256 KB through one workgroup took 4 us of the kernel's 10.7)
         uint4* dst = reinterpret_cast<uint4*>(const_cast<uint8_t*>(xe));
-        for (int i = tid; i < total * row_u4; i += blockDim.x) {
-            const int r = i / row_u4, c = i - r * row_u4;
-            dst[i] = x[(size_t)s_tok[r] * row_u4 + c];
+        const int n = total * row_u4, stride = (int)blockDim.x;
+        for (int i0 = (int)blockIdx.x * 2 * stride + tid; i0 < n; i0 += 2 * stride * (int)gridDim.x) {
+            const int i1 = min(i0 + stride, n - 1);  // (past the end: the last element again, not stored)
+            const int r0 = i0 / row_u4, r1 = i1 / row_u4;
+            const uint4 v0 = x[(size_t)s_tok[r0] * row_u4 + (i0 - r0 * row_u4)];
+            const uint4 v1 = x[(size_t)s_tok[r1] * row_u4 + (i1 - r1 * row_u4)];
+            dst[i0] = v0;
+            if (i0 + stride < n) dst[i0 + stride] = v1;
         }
     }
+    if (!lead) return;
     for (int t = tid; t <= T; t += blockDim.x) tok_first[t] = t * Ktop;
     for (int t = tid; t < T; t += blockDim.x) {  // the pairs of a token in ascending order (selection, Ktop is small)
         int prev = -1;
@@ -735,10 +756,10 @@ __global__ __launch_bounds__(1024) void routed_lists_kernel(const int32_t* __res
         const int p0 = s_first[e], nt = s_first[e + 1] - p0;
         int iA = s_offA[e], iB = s_offB[e];
         for (int b0 = 0; b0 < nt; b0 += sh.capA, ++iA)
-            tabA[iA] = GemvProb{ptrs[e], h + (size_t)(p0 + b0) * sh.strideYA, xe + (size_t)(p0 + b0) * sh.strideXA, ptrs[E + e],
+            tabA[iA] = GemvProb{p_gate, h + (size_t)(p0 + b0) * sh.strideYA, xe + (size_t)(p0 + b0) * sh.strideXA, p_up,
                                 sh.nrowsA, min(sh.capA, nt - b0), iA * s_wgA, s_tilesA};
         for (int b0 = 0; b0 < nt; b0 += sh.capB, ++iB)
-            tabB[iB] = GemvProb{ptrs[2 * E + e], o + (size_t)(p0 + b0) * sh.strideYB, h + (size_t)(p0 + b0) * sh.strideXB, nullptr,
+            tabB[iB] = GemvProb{p_down, o + (size_t)(p0 + b0) * sh.strideYB, h + (size_t)(p0 + b0) * sh.strideXB, nullptr,
                                 sh.nrowsB, min(sh.capB, nt - b0), iB * sh.wgB, p0 + b0};  // (tiles: the problem's first pair)
     }
     __syncthreads();
@@ -886,7 +907,7 @@ int launch_moe_ffn_routed(const tfq_weight* const* gate, const tfq_weight* const
     const int row_u4 = (int)(D * 2 / 16);
     const int64_t ng = (int64_t)P * row_u4;
     const bool fuse_gather = ng * 16 <= 256 * 1024;  // up to 256 KB of rows ride in the list kernel's one workgroup (about 3 us)
-    hipLaunchKernelGGL(routed_lists_kernel, dim3(1), dim3(1024), 0, s, d_topk_idx, d_topk_w, T, Ktop, E, d_first, d_rows, d_w, d_tokf, d_tokp,
+    hipLaunchKernelGGL(routed_lists_kernel, dim3(fuse_gather ? 8 : 1), dim3(1024), 0, s, d_topk_idx, d_topk_w, T, Ktop, E, d_first, d_rows, d_w, d_tokf, d_tokp,
                        rp.sh, static_cast<const uint8_t* const*>(d_expert_table), (const uint8_t*)xe, h, o, tabA, mapA, tabB, mapB,
                        fuse_gather ? (const uint4*)x : nullptr, row_u4);
     if (!fuse_gather)
