@@ -48,6 +48,24 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint4* __restric
     dst[i] = src[(int64_t)rows[r] * row_u4 + c];
 }
 
+// The gather of a decode-sized call that also brings the routing lists over: the first `copy_blocks` workgroups copy
+// the list blob from pinned host memory into the workspace (the launches behind this one read it there), the others
+// gather rows with the row list read straight from the host copy.  Replaces an asynchronous copy in front of the
+// gather, which as a stream operation of its own took longer than this whole kernel.
+__global__ __launch_bounds__(256) void gather_upload_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                            const int* __restrict__ rows_host, int nrows, int row_u4,
+                                                            const uint4* __restrict__ lists_host, uint4* __restrict__ lists_dev,
+                                                            int list_u4, int copy_blocks) {
+    if ((int)blockIdx.x < copy_blocks) {
+        for (int i = (int)blockIdx.x * 256 + (int)threadIdx.x; i < list_u4; i += copy_blocks * 256) lists_dev[i] = lists_host[i];
+        return;
+    }
+    const int64_t i = (int64_t)((int)blockIdx.x - copy_blocks) * 256 + threadIdx.x;
+    if (i >= (int64_t)nrows * row_u4) return;
+    const int r = (int)(i / row_u4), c = (int)(i - (int64_t)r * row_u4);
+    dst[i] = src[(int64_t)rows_host[r] * row_u4 + c];
+}
+
 template <bool OUT_BF16>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ g, const float* __restrict__ u,
                                                        void* __restrict__ out, int64_t n) {
@@ -522,17 +540,29 @@ int moe_run(const tfq_weight* const* gate, const tfq_weight* const* up, const tf
     int* d_pairs = d_rows + P;
     int* d_first = d_pairs + P;
     float* d_w = reinterpret_cast<float*>(d_first + T + 1);
-    // The source is pinned: the copy is asynchronous, and the event tells when the slot may be filled again.
-    TFQ_HIP(hipMemcpyAsync(ws.lists, lists, list_bytes, hipMemcpyHostToDevice, s));
+    // The source is pinned, and the event tells when the slot may be filled again.  A decode-sized call lets the
+    // gather kernel fetch the lists (one launch instead of a copy and a launch); larger ones copy asynchronously.
+    const int row_u4 = (int)(D * xe_bytes / 16);
+    const int64_t ng = (int64_t)P * row_u4;
+    const bool kernel_upload = P > 0 && list_bytes <= 64 * 1024 && ng * 16 <= 4 * 1024 * 1024 && (reinterpret_cast<uintptr_t>(ws.lists) & 15) == 0 &&
+                               ((list_bytes + 15) & ~(size_t)15) <= ws.list_bytes;
+    if (kernel_upload) {
+        void* lists_dev_view = nullptr;  // the pinned buffer as the device sees it
+        TFQ_HIP(hipHostGetDevicePointer(&lists_dev_view, lists, 0));
+        const int list_u4 = (int)((list_bytes + 15) / 16);  // (the slot and the workspace area are sized in whole 16 bytes and more)
+        const int copy_blocks = (list_u4 + 255) / 256 < 4 ? (list_u4 + 255) / 256 : 4;
+        hipLaunchKernelGGL(gather_upload_kernel, dim3((unsigned)((ng + 255) / 256) + copy_blocks), dim3(256), 0, s,
+                           (const uint4*)x, (uint4*)ws.xe, static_cast<const int*>(lists_dev_view), P, row_u4,
+                           static_cast<const uint4*>(lists_dev_view), reinterpret_cast<uint4*>(ws.lists), list_u4, copy_blocks);
+    } else {
+        TFQ_HIP(hipMemcpyAsync(ws.lists, lists, list_bytes, hipMemcpyHostToDevice, s));
+        if (P)
+            hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)((ng + 255) / 256)), dim3(256), 0, s,
+                               (const uint4*)x, (uint4*)ws.xe, d_rows, P, row_u4);
+    }
     TFQ_HIP(hipEventRecord(slot->done, s));
     slot->recorded = true;
 
-    if (P) {
-        const int row_u4 = (int)(D * xe_bytes / 16);
-        const int64_t ng = (int64_t)P * row_u4;
-        hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)((ng + 255) / 256)), dim3(256), 0, s,
-                           (const uint4*)x, (uint4*)ws.xe, d_rows, P, row_u4);
-    }
     const uint8_t* d_lists = reinterpret_cast<const uint8_t*>(ws.lists);
     // Tokens of at most two slots, an fp32 y and the sixteen-row down launch: that launch adds weight x product into
     // y itself (the gate / up launch zeroes y on its way) and no combine launch follows: two addends onto zero are the
