@@ -133,10 +133,10 @@ struct GemvKernArgs {
 // reads that vector like any other activation, instead of evaluating the exponentials in every workgroup.
 // uint4 entries from one activation slot's staged A entries to the next: 32, padded to 33 for the variant that
 // reads its A fragments from LDS per MFMA (two slot sets, 16-byte header)
-__host__ __device__ constexpr int a_slot_stride(int fmt, int sets) { return sets == 2 && tiled_header_bytes(fmt) == 16 ? 33 : 32; }
+__host__ __device__ constexpr int a_slot_stride(int fmt, int sets) { return sets == 2 && (tiled_header_bytes(fmt) == 16 || tiled_header_in_bytes(fmt)) ? 33 : 32; }
 
 template <int FMT, bool XF32, int WD, int SETS = 1, bool GROUPED = false, int XOP = XOP_NONE, bool PAIR = false, bool GM = false>
-__global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1024 : 512) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin_arg) {
+__global__ __launch_bounds__((SETS == 1 || (SETS == 2 && (Fmt<FMT>::HV == 1 || (tiled_header_in_bytes(FMT) && WD == 1 && !XF32)))) ? 1024 : 512) void gemv4_kernel(GemvKernArgs args, const void* __restrict__ xin_arg) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
     // GM ("group-major", one bf16 activation row, formats with byte headers): A row 4 c + s instead of 4 s + c, so
@@ -447,7 +447,7 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && Fmt<FMT>::HV == 1)) ? 1
     asm volatile("" : "+v"(C));  // keep the bias in a VGPR so (v & M) | C is one v_and_or_b32
     // Two slot sets: the A fragments stay in LDS and are read per MFMA (sixteen 128-bit LDS reads per unit), which
     // leaves room for sixteen wavefronts per workgroup; one or four sets keep them in registers.
-    constexpr bool A_LDS = SETS == 2 && F::HV == 1;  // (the formats with byte headers do not fit 128 registers either way)
+    constexpr bool A_LDS = SETS == 2 && (F::HV == 1 || (tiled_header_in_bytes(FMT) && WD == 1 && !XF32));  // (byte headers: with one unit fetch in flight)
     uint4 av[A_LDS ? 1 : SETS][2][4];
     const uint4* asrc[SETS][2];
     float xv[SETS][2][PER];
@@ -1343,7 +1343,7 @@ GemvPlan plan_gemv4(const GemvArgs& a, int nslot) {
     // the grouped gate / up launch of a mixture layer 102.7 against 110.3 us).  Otherwise several slot sets need
     // the registers of two wavefronts, so at most 8 then: the count in 4..8 that splits the block columns most
     // evenly.
-    const int max_nw = p.sets == 1 || (p.sets == 2 && Fmt<FMT>::HV == 1) ? 16 : 8;
+    const int max_nw = p.sets == 1 || (p.sets == 2 && (Fmt<FMT>::HV == 1 || (tiled_header_in_bytes(FMT) && !a.x_f32))) ? 16 : 8;
     p.NW = nblocks < max_nw ? nblocks : max_nw;
     if (nblocks > max_nw && p.sets > 1) {
         int best_waste = 1 << 30;
@@ -1494,7 +1494,8 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
         }
     } else if constexpr (kTwoSets<FMT>) {
         if (p.sets == 2) {
-            kern = a.x_f32 ? gemv4_kernel<FMT, true, 2, 2> : gemv4_kernel<FMT, false, 2, 2>;
+            constexpr int WD2 = tiled_header_in_bytes(FMT) ? 1 : 2;
+            kern = a.x_f32 ? gemv4_kernel<FMT, true, 2, 2> : gemv4_kernel<FMT, false, WD2, 2>;
             slot = a.x_f32 ? 18 : 6;
         } else if (p.sets > 2) {
             return fail(TFQ_ERR_SHAPE, "gemv: more than eight rows in one pass for this format");
