@@ -1340,7 +1340,9 @@ GemvPlan plan_gemv4(const GemvArgs& a, int nslot) {
     // Two slot sets of a format with a 16-byte header: sixteen as well, with the A fragments read from LDS per
     // MFMA instead of held in registers (106-128 registers; measured against eight wavefronts with the fragments
     // in registers, B32S4 at eight rows: q+k+v 6.6 against 8.0 us, o 5.9 against 7.2 us, gate+up 15.9 / 15.7 us;
-    // the grouped gate / up launch of a mixture layer 102.7 against 110.3 us).  Otherwise several slot sets need
+    // the grouped gate / up launch of a mixture layer 102.7 against 110.3 us).  The formats with byte headers do the
+    // same for bf16 rows with one unit fetch in flight per wavefront, which is what fits 128 registers (SB256A2
+    // 14336x4096 at eight rows 13.6 against 15.0 us, SB256A3 14.5 against 16.2 us).  Otherwise several slot sets need
     // the registers of two wavefronts, so at most 8 then: the count in 4..8 that splits the block columns most
     // evenly.
     const int max_nw = p.sets == 1 || (p.sets == 2 && (Fmt<FMT>::HV == 1 || (tiled_header_in_bytes(FMT) && !a.x_f32))) ? 16 : 8;
