@@ -1493,6 +1493,10 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
             if (a.x_f32 && p.sets != 2) return fail(TFQ_ERR_SHAPE, "gemv: more than four fp32 rows in one pass");
             kern = p.sets == 2 ? (a.x_f32 ? gemv4_kernel<FMT, true, 2, 2> : gemv4_kernel<FMT, false, 2, 2>) : gemv4_kernel<FMT, false, 1, 4>;
             slot = p.sets == 2 ? (a.x_f32 ? 18 : 6) : 7;
+            // a wavefront with one or two units to walk keeps one fetch in flight (a second one would only repeat its
+            // last unit): 4096x4096 at eight rows B32S4 5.6 -> 5.0 us, B32S8 7.5 -> 6.6 us, 6144x4096 2-3 %; equal
+            // from four units on
+            if (p.sets == 2 && !a.x_f32 && full_items <= 2) { kern = gemv4_kernel<FMT, false, 1, 2>; slot = 19; }
         }
     } else if constexpr (kTwoSets<FMT>) {
         if (p.sets == 2) {
