@@ -979,14 +979,14 @@ __device__ __forceinline__ void transpose_rows(uint32_t (&v)[4]) {
 // or four unit fetches in flight, eight wavefronts of two columns, and fewer tiles per workgroup measured equal
 // or slower.
 constexpr int kGemvbKC = 16;  // block columns per K part
-template <int FMT, bool SPLIT, bool GROUPED = false, bool XF32 = false>
+template <int FMT, bool SPLIT, bool GROUPED = false, bool XF32 = false, int WDP = 2>
 __global__ __launch_bounds__(1024) void gemvb_kernel(GemvKernArgs args, const unsigned short* __restrict__ x_arg) {
     extern __shared__ uint4 smem[];
     using F = Fmt<FMT>;
     static_assert(F::GS == 32 && F::HV == 1, "32-weight groups and a 16-byte header");
     static_assert(!(SPLIT && GROUPED), "a grouped launch has no K parts");
     static_assert(!(XF32 && GROUPED), "grouped problems take bf16 rows");
-    constexpr int UB = tiled_unit_bytes(FMT), NC = 2 * F::NP, WD = 2;
+    constexpr int UB = tiled_unit_bytes(FMT), NC = 2 * F::NP, WD = WDP;  // unit fetches in flight per wavefront
     const int K = args.K, T = args.tiles_per_wg;
     const bool y_bf16 = args.y_bf16 != 0;
     const int bid = blockIdx.x;
@@ -1573,9 +1573,15 @@ int run_gemvb(GemvArgs a, const void* x, hipStream_t s) {
     using Kernel = void (*)(GemvKernArgs, const unsigned short*);
     static const Kernel kernels[2][2] = {{gemvb_kernel<FMT, false>, gemvb_kernel<FMT, true>},
                                          {gemvb_kernel<FMT, false, false, true>, gemvb_kernel<FMT, true, false, true>}};
-    const int ki = (a.x_f32 ? 2 : 0) + (split ? 1 : 0);
-    const Kernel kern = kernels[a.x_f32 ? 1 : 0][split ? 1 : 0];
-    static std::atomic<bool> lds_limit_raised[4] = {};
+    int ki = (a.x_f32 ? 2 : 0) + (split ? 1 : 0);
+    Kernel kern = kernels[a.x_f32 ? 1 : 0][split ? 1 : 0];
+    // a wavefront with one unit to walk (a block column of one tile): the instantiation with one fetch in flight,
+    // whose second fetch would only repeat the unit
+    if (!split && !a.x_f32 && T * ((nblocks + NW - 1) / NW) == 1) {
+        kern = gemvb_kernel<FMT, false, false, false, 1>;
+        ki = 4;
+    }
+    static std::atomic<bool> lds_limit_raised[5] = {};
     if (!lds_limit_raised[ki]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
