@@ -365,6 +365,9 @@ class Chain:
             d.y_op = ph.get("y_op", Y_PLAIN)
             ys = ph.get("y") or []
             d.y_dtype = F32
+            kinds = {_dtype_code(y) for y in ys if y is not None}
+            if len(kinds) > 1:
+                raise TfqError("Chain: the outputs of one phase must share a dtype")
             for m, y in enumerate(ys):
                 if y is not None:
                     d.y[m] = y.data_ptr()
