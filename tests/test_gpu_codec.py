@@ -132,6 +132,37 @@ def test_encode_short_blocks_golden(O, tfq, gpu):
         assert np.array_equal(back.view(np.uint32), O.decode_tensor(fmt, want, n).view(np.uint32)), fmt
 
 
+def test_encode_short_blocks_every_id_against_oracle(O, tfq, gpu):
+    """Every id the library serves x tail sizes on both sides of each layout switch (bare codes, one scale, group
+    headers, whole 32-groups) x a gaussian, a heavy-tailed, an all-zero and a constant block: the wavefront
+    encoder of a short block gives the oracle's bytes (the oracle itself is pinned by tails.npz)."""
+    import torch
+    sizes = [1, 5, 7, 8, 9, 15, 16, 17, 24, 31, 32, 33, 40, 48, 63, 64, 65, 96, 100, 127, 128, 160, 192, 200, 224, 254, 255]
+    ids = [i for i in range(0, 109) if tfq.lib().tfq_format_supported(i)]
+    srcs = [O.rng_normal(901, 256, 0.05), (O.rng_normal(902, 256, 1.0) ** 3 * 0.02).astype(np.float32),
+            np.zeros(256, np.float32), np.full(256, -0.37, np.float32)]
+    bad, checked = [], 0
+    for fmt in ids:
+        name = tfq.lib().tfq_format_name(fmt).decode()
+        mixed = name.startswith("Q_MX") or name.startswith("Q_G_MX")
+        for n in sizes:
+            try:
+                tfq.block_bytes(fmt, n)
+            except tfq.TfqError:
+                continue  # the literal block-32 formats hold whole 32-groups only
+            for k, src in enumerate(srcs):
+                if mixed and k >= 2:
+                    continue  # equal magnitudes across a tier boundary: the reference's order is its sort's
+                w = np.ascontiguousarray(src[:n])
+                want = O.encode_tensor(fmt, w)
+                got = tfq.encode(fmt, torch.from_numpy(w).to(gpu)).cpu().numpy()
+                checked += 1
+                if not np.array_equal(got, want):
+                    bad.append((name, n, k))
+    assert not bad, bad[:40]
+    assert checked > 8000, checked
+
+
 def test_half_subnormal_scales_decode_exactly(O, tfq, gpu):
     import torch
     pay = np.zeros((128, 272), np.uint8)

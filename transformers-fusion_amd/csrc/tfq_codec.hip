@@ -1048,13 +1048,24 @@ __global__ __launch_bounds__(64) void decode_mix_kernel(MixLayout L, const uint8
 }
 
 __device__ __forceinline__ float mix_level(int bits, uint32_t code) {
-    return bits == 3 ? fixed_value(3, code) : grid_value(bits, code);
+    return (bits == 3 || bits == 6 || bits == 12) ? fixed_value(bits, code) : grid_value(bits, code);
 }
 // nearest_level / nearest_fixed_level for the widths the mixes use (src/codec/block_codec.cpp:190-203, :596-606)
 __device__ __forceinline__ uint32_t mix_nearest(int bits, float v) {
     if (bits == 8) {
         const float c = fmaxf(-8.0f, fminf(8.0f, v));
         return (uint32_t)lroundf((c + 8.0f) * 255.0f / 16.0f);
+    }
+    if (bits == 6 || bits == 12) {  // ascending quantile tables: search |v| in the upper half (:596-622)
+        const int half = 1 << (bits - 1);
+        const float a = fabsf(v);
+        int lo = half, hi = 2 * half - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi) / 2;
+            if (fixed_value(bits, (uint32_t)mid) < a) lo = mid + 1; else hi = mid;
+        }
+        if (lo > half && fixed_value(bits, (uint32_t)lo) - a >= a - fixed_value(bits, (uint32_t)lo - 1u)) --lo;
+        return v >= 0.0f ? (uint32_t)lo : (uint32_t)(half - 1 - (lo - half));
     }
     uint32_t best = 0;
     float bd = fabsf(v - mix_level(bits, 0));
@@ -1065,7 +1076,7 @@ __device__ __forceinline__ uint32_t mix_nearest(int bits, float v) {
     return best;
 }
 
-// Encoder of a full block (quant_quad_mix, src/codec/block_codec.cpp:2102-2205): weights ranked by
+// Encoder of a block of L.n <= 256 weights (quant_quad_mix, src/codec/block_codec.cpp:2102-2205): weights ranked by
 // magnitude, the c[3] largest into tier 3 and so on down; per tier (per 32 values of the most populated
 // tier of a grouped id) s = max / top level and two least-squares refits on the first 32 values the scale
 // covers; then tiers, values and scales as laid out in MixLayout.  Equal magnitudes rank by index here;
@@ -1079,17 +1090,18 @@ __global__ __launch_bounds__(64) void encode_mix_kernel(MixLayout L, const float
     __shared__ uint32_t words[200];  // the largest block is 784 bytes
     const uint32_t lane = threadIdx.x;
     const int64_t blk = blockIdx.x;
-    for (int i = lane; i < 256; i += 64) { const float x = wg[blk * 256 + i]; w[i] = x; mag[i] = __float_as_uint(x) & 0x7FFFFFFFu; }
+    const int n = L.n, valid = max(0, min(4, n - 4 * (int)lane));  // lane l holds weights 4 l .. 4 l + 3
+    for (int i = lane; i < 256; i += 64) { const float x = i < n ? wg[blk * n + i] : 0.0f; w[i] = x; mag[i] = __float_as_uint(x) & 0x7FFFFFFFu; }
     for (int i = lane; i < 200; i += 64) words[i] = 0;
     if (lane < 32) sc[lane >> 3][lane & 7] = 0.0f;
     __syncthreads();
     const int n3 = L.c[3], n2 = n3 + L.c[2], n1 = n2 + L.c[1];
     uint32_t tiers = 0;
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < valid; ++k) {
         const int i = 4 * lane + k;
         const uint32_t m = mag[i];
         int rank = 0;
-        for (int j = 0; j < 256; ++j) {
+        for (int j = 0; j < n; ++j) {
             const uint32_t mj = mag[j];
             rank += (mj > m || (mj == m && j < i)) ? 1 : 0;
         }
@@ -1097,10 +1109,10 @@ __global__ __launch_bounds__(64) void encode_mix_kernel(MixLayout L, const float
         tiers |= t << (2 * k);
     }
     uint32_t before[4], total[4];
-    mix_scan(tiers, 4, lane, before, total);
+    mix_scan(tiers, valid, lane, before, total);
     const int first[4] = {0, L.c[0], L.c[0] + L.c[1], L.c[0] + L.c[1] + L.c[2]};  // tier runs inside tv
-    uint32_t rk[4];
-    for (int k = 0; k < 4; ++k) {
+    uint32_t rk[4] = {0, 0, 0, 0};
+    for (int k = 0; k < valid; ++k) {
         const uint32_t t = (tiers >> (2 * k)) & 3u;
         rk[k] = before[t]++;
         tv[first[t] + rk[k]] = w[4 * lane + k];
@@ -1110,7 +1122,8 @@ __global__ __launch_bounds__(64) void encode_mix_kernel(MixLayout L, const float
         const int nsc = L.nsc[t];
         if (nsc == 0) continue;
         const int bits = L.bits[t], cnt = min(L.c[t], nsc * 32);
-        const float top = bits == 2 ? 1.5104f : bits == 3 ? 3.0776f : bits == 4 ? 2.7178f : bits == 8 ? 8.0f : 1.0f;
+        const float top = bits == 2 ? 1.5104f : bits == 3 ? 3.0776f : bits == 4 ? 2.7178f : bits == 8 ? 8.0f
+                                                                  : (bits == 6 || bits == 12) ? fixed_value(bits, (1u << bits) - 1u) : 1.0f;
         const float* x = tv + first[t];
         if ((int)lane < nsc) {
             float maxa = 0.0f;
@@ -1142,9 +1155,9 @@ __global__ __launch_bounds__(64) void encode_mix_kernel(MixLayout L, const float
     // the stream: byte l holds the tiers of lane l's weights, values at (start of the tier's run) + rank * width
     atomicOr(&words[lane >> 2], tiers << (8 * (lane & 3u)));
     uint32_t start[4];
-    uint32_t at = 512;
+    uint32_t at = 2u * (uint32_t)n;
     for (int t = 0; t < 4; ++t) { start[t] = at; at += (uint32_t)(L.c[t] * L.bits[t]); }
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < valid; ++k) {
         const uint32_t t = (tiers >> (2 * k)) & 3u;
         const int bits = L.bits[t];
         const float v = w[4 * lane + k];
@@ -1410,6 +1423,11 @@ bool block_layout(int fmt, int n, BlockLayout* L) {
             return true;
         default: return false;
     }
+}
+
+int launch_encode_mix(const MixLayout& L, const float* w, uint8_t* dst, hipStream_t s) {
+    hipLaunchKernelGGL(encode_mix_kernel, dim3(1), dim3(64), 0, s, L, w, dst);
+    return hip_fail(hipGetLastError(), "encode launch");
 }
 
 int launch_decode_short(const BlockLayout& L, const uint8_t* src, float* out, hipStream_t s) {
