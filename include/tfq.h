@@ -212,12 +212,11 @@ int tfq_weight_decode(const tfq_weight_t* w, float* out, tfq_stream_t stream);
  * Replaces Qwen35Engine::gemm (src/adapters/tools/qwen35_engine.cpp:54-101):
  * tfq_gemv is the decode path (B rows, 1 <= B <= 16), tfq_gemm the prefill
  * path (any M).  x is [B][K], y is [B][N], row-major, dtypes TFQ_F32 / TFQ_BF16.
- * A handle with K above 4096 in a format of the 16-row decode kernel (B32S4,
- * B32S8, Q_G_4, Q_G_8, Q_8) carries a small area of partial sums (16 N fp32 per
- * 4096 of K) that calls with five or more bf16 rows or three or more fp32 rows
- * use: such calls on ONE
- * handle must not overlap in time (issue them on one stream, as the reference's
- * gemm is called; distinct handles are independent).
+ * A handle is read-only for every call that takes it as `const`: like the
+ * reference's gemm, which is const and may run concurrently on one matrix
+ * (qwen35_engine.cpp:54-75), calls on one handle may overlap on different
+ * streams.  Scratch memory, where a call uses any, comes from the caller
+ * (tfq_gemv_ws, tfq_gemm_ws) and must not be shared by overlapping calls.
  * K: any multiple of 256 for those five formats and for every format on the wire
  * layout.  The other tiled formats (Q_G_3, Q_G_2, SB256A3, SB256A2) stage an
  * activation row in on-chip memory, which holds K <= 61440 for a bf16 row and
@@ -229,6 +228,17 @@ int tfq_gemv(const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, 
              tfq_stream_t stream);
 int tfq_gemm(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
              tfq_stream_t stream);
+/* tfq_gemv with scratch memory.  With five or more rows and K above 4096 in a format of the 16-row decode
+ * kernel (B32S4, B32S8, Q_G_4, Q_G_8, Q_8), the kernel cuts K into parts of at most 4096 over separate
+ * workgroups, so that a workgroup reads a quarter of the activations instead of all of them; the parts' fp32
+ * partial sums [parts][16][N] go to `workspace` (device memory, 256-byte aligned) and a second launch adds them
+ * in part order.  tfq_gemv_workspace_bytes returns what a call with these arguments uses (0: none).  A null or
+ * smaller workspace is legal: the product then runs unsplit (tfq_gemv is that call), same results to the stated
+ * tolerance, slower (Llama-3-8B down projection, 16 rows: about 20 us against 16 us).  Replaces the same
+ * reference loop as tfq_gemv (qwen35_engine.cpp:54-101); the workspace has no counterpart there. */
+size_t tfq_gemv_workspace_bytes(const tfq_weight_t* w, int x_dtype, int B);
+int tfq_gemv_ws(const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, int y_dtype, void* workspace,
+                size_t workspace_bytes, tfq_stream_t stream);
 /* tfq_gemm with scratch memory.  When M rows make fewer output tiles than the GPU has compute units
  * (a tall K with few weight rows, or a few hundred tokens), the prefill kernel can split K over several
  * workgroups per tile; the fp32 partial tiles go to `workspace` (device memory) and are added in a fixed

@@ -372,11 +372,11 @@ def test_gemv_multi_with_eight_rows(O, tfq, gpu):
 
 @pytest.mark.parametrize("fmt", ["B32S4", "B32S8"])
 def test_gemv_rows_with_k_split_repeated_calls(O, tfq, gpu, fmt):
-    """K above 4096 with five or more rows: the workgroups of a row group split K and meet through partial sums
-    and an arrival counter kept with the handle.  The counter must be back at zero after every launch: calls in
-    a row on one handle (other activations, fewer rows, bf16 output, 40 rows through tfq_gemm) each match a dense
-    product of the decoded matrix, a repeated call gives the same bits (the parts are added in a fixed order),
-    and two matrices of such a K in one launch (no split there) agree with the single launches."""
+    """K above 4096 with five or more rows: the workgroups of a row group split K, write their partial sums to the
+    call's workspace, and a second launch adds the parts in part order.  Calls in a row on one handle (other
+    activations, fewer rows, bf16 output, 40 rows through tfq_gemm) each match a dense product of the decoded
+    matrix, a repeated call gives the same bits, and two matrices of such a K in one launch (no split there)
+    agree with the single launches."""
     import torch
     N, K = 1000, 14336  # 63 tiles, the last one short; 56 block columns in 4 parts of 14
     g = torch.Generator(device="cuda").manual_seed(77)
@@ -435,6 +435,38 @@ def test_gemv_k_split_in_graph_replays(O, tfq, gpu):
         for want, got in zip(eager, outs):
             assert torch.equal(want, got)
         assert torch.equal(W.gemv(xs[rep % 3]), eager[rep % 3])  # eager work between the replays
+    W.close()
+
+
+def test_gemv_one_handle_on_two_streams(O, tfq, gpu):
+    """Qwen35Engine::gemm is const and may run concurrently on one matrix (qwen35_engine.cpp:54-75): calls on
+    one handle overlap on two streams, each with a workspace of its own, and give the bits of the serial
+    result; so does the call without a workspace (unsplit) to the matmul tolerance."""
+    import torch
+    N, K, B = 4096, 14336, 16
+    g = torch.Generator(device="cuda").manual_seed(21)
+    W = tfq.Weight("B32S4", N, K, tfq.encode("B32S4", torch.randn(N * K, device=gpu, generator=g) * 0.02))
+    xs = [torch.randn(B, K, device=gpu, generator=g).bfloat16() for _ in range(2)]
+    need = W.gemv_workspace_bytes(tfq.BF16, B)
+    assert need > 0
+    wss = [torch.empty(need, dtype=torch.uint8, device=gpu) for _ in range(2)]
+    serial = [W.gemv(x, workspace=wss[0]).clone() for x in xs]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [torch.empty(B, N, device=gpu) for _ in range(2)]
+    for rep in range(50):
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                W.gemv(xs[i], out=outs[i], workspace=wss[i])
+        torch.cuda.synchronize()
+        for want, got in zip(serial, outs):
+            assert torch.equal(want, got), rep
+    # no workspace: the unsplit kernel, the same product to the tolerance of bf16 activations
+    y = torch.empty(B, N, device=gpu)
+    rc = tfq.lib().tfq_gemv(W.handle, xs[0].data_ptr(), tfq.BF16, B, y.data_ptr(), tfq.F32, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert float((y - serial[0]).abs().max()) <= 1e-4 * float(serial[0].abs().max())
     W.close()
 
 

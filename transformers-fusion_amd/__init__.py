@@ -71,6 +71,8 @@ def _load():
         "tfq_weight_decode": (i32, [vp, vp, vp]),
         "tfq_gemv": (i32, [vp, vp, i32, i32, vp, i32, vp]),
         "tfq_gemm": (i32, [vp, vp, i32, i32, vp, i32, vp]),
+        "tfq_gemv_workspace_bytes": (sz, [vp, i32, i32]),
+        "tfq_gemv_ws": (i32, [vp, vp, i32, i32, vp, i32, vp, sz, vp]),
         "tfq_gemm_workspace_bytes": (sz, [vp, i32, i32]),
         "tfq_gemm_ws": (i32, [vp, vp, i32, i32, vp, i32, vp, sz, vp]),
         "tfq_gemm_static": (i32, [vp, vp, i32, i32, vp, i32, vp]),
@@ -293,14 +295,29 @@ class Weight:
         _check(fn(self.handle, x.data_ptr(), _dtype_code(x), B, y.data_ptr(), _dtype_code(y), _stream()))
         return y
 
-    def gemv(self, x, out_dtype=None, out=None):
-        """y[B][N] = x[B][K] . W^T for 1 <= B <= 16 (decode)."""
-        if out is not None:
-            B = x.numel() // self.K
-            _check(lib().tfq_gemv(self.handle, x.data_ptr(), _dtype_code(x), B, out.data_ptr(),
-                                  _dtype_code(out), _stream()))
+    def gemv(self, x, out_dtype=None, out=None, workspace=None):
+        """y[B][N] = x[B][K] . W^T for 1 <= B <= 16 (decode).  Calls that cut K into parts (five or more rows, K above
+        4096) go through tfq_gemv_ws; `workspace` is a uint8 tensor of tfq_gemv_workspace_bytes or more (one is made
+        per call when none is given; pass one when the call is captured into a graph and replayed)."""
+        import torch
+        x = x.contiguous()
+        assert x.is_cuda and x.shape[-1] == self.K
+        B = x.numel() // self.K
+        if out is None:
+            out = torch.empty((B, self.N), dtype=out_dtype or torch.float32, device=x.device)
+        need = int(lib().tfq_gemv_workspace_bytes(self.handle, _dtype_code(x), B))
+        if need == 0:
+            _check(lib().tfq_gemv(self.handle, x.data_ptr(), _dtype_code(x), B, out.data_ptr(), _dtype_code(out), _stream()))
             return out
-        return self._mm(lib().tfq_gemv, x, out_dtype)
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+        assert workspace.numel() >= need and workspace.data_ptr() % 256 == 0
+        _check(lib().tfq_gemv_ws(self.handle, x.data_ptr(), _dtype_code(x), B, out.data_ptr(), _dtype_code(out),
+                                 workspace.data_ptr(), workspace.numel(), _stream()))
+        return out
+
+    def gemv_workspace_bytes(self, x_dtype_code: int, B: int) -> int:
+        return int(lib().tfq_gemv_workspace_bytes(self.handle, x_dtype_code, B))
 
     def gemm(self, x, out_dtype=None, workspace=True):
         """y[M][N] = x[M][K] . W^T for any M (prefill).  With `workspace` the call goes through tfq_gemm_ws with

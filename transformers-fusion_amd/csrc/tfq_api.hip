@@ -255,15 +255,11 @@ static tfq_weight_t* make_weight(const char* who, uint8_t fmt, int64_t N, int64_
     if (!from_host && (uintptr_t)packed % 16) { fail(TFQ_ERR_ARG, std::string(who) + ": device payload must be 16-byte aligned"); return nullptr; }
     if (ensure_device()) return nullptr;
     const bool tiled = wants_tiled16(fmt);
-    tfq_weight_t* w = new (std::nothrow) tfq_weight_t{fmt, N, K, bytes, nullptr, 0, tiled ? TFQ_LAYOUT_TILED16 : TFQ_LAYOUT_WIRE, true, nullptr};
+    tfq_weight_t* w = new (std::nothrow) tfq_weight_t{fmt, N, K, bytes, nullptr, 0, tiled ? TFQ_LAYOUT_TILED16 : TFQ_LAYOUT_WIRE, true};
     if (!w) { fail(TFQ_ERR_NOMEM, std::string(who) + ": out of host memory"); return nullptr; }
     w->dev_bytes = tiled ? (size_t)((N + 15) / 16) * (size_t)(K / 256) * (size_t)tiled_unit_bytes(fmt) : bytes;
     uint8_t* staged = nullptr;  // wire payload on the device, when it has to be permuted
-    // the partial sums of the K-split decode kernel live behind the weights (every one is written before it is read)
-    const size_t split_bytes = tiled ? gemv_rows16_split_bytes(fmt, N, K) : 0;
-    const size_t split_at = (w->dev_bytes + 255) & ~(size_t)255;
-    hipError_t e = hipMalloc(&w->dev, split_bytes ? split_at + split_bytes : w->dev_bytes);
-    if (e == hipSuccess && split_bytes) w->split_partial = reinterpret_cast<float*>(w->dev + split_at);
+    hipError_t e = hipMalloc(&w->dev, w->dev_bytes);
     if (e == hipSuccess && from_host) {
         if (tiled) {
             e = hipMalloc(&staged, bytes);
@@ -385,6 +381,20 @@ int tfq_gemv(const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, 
     if (int r = check_matmul("tfq_gemv", w, x, x_dtype, B, y, y_dtype)) return r;
     if (B > 16) return fail(TFQ_ERR_SHAPE, "tfq_gemv: batch above 16, use tfq_gemm");
     return launch_gemv(w, x, x_dtype, B, y, y_dtype, (hipStream_t)stream);
+}
+
+size_t tfq_gemv_workspace_bytes(const tfq_weight_t* w, int x_dtype, int B) {
+    (void)x_dtype;
+    if (!w || B < 5 || B > 16 || w->layout != TFQ_LAYOUT_TILED16) return 0;
+    return gemv_rows16_split_bytes(w->fmt, w->N, w->K);
+}
+
+int tfq_gemv_ws(const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, int y_dtype, void* workspace,
+                size_t workspace_bytes, tfq_stream_t stream) {
+    if (int r = check_matmul("tfq_gemv_ws", w, x, x_dtype, B, y, y_dtype)) return r;
+    if (B > 16) return fail(TFQ_ERR_SHAPE, "tfq_gemv_ws: batch above 16, use tfq_gemm_ws");
+    if (workspace && (uintptr_t)workspace % 256) return fail(TFQ_ERR_ARG, "tfq_gemv_ws: workspace must be 256-byte aligned");
+    return launch_gemv(w, x, x_dtype, B, y, y_dtype, (hipStream_t)stream, workspace, workspace ? workspace_bytes : 0);
 }
 
 int tfq_gemv_multi(const tfq_weight_t* const* ws, int count, const void* x, int x_dtype, int B, void* const* ys,

@@ -653,26 +653,34 @@ int launch_gemm_grouped(int fmt, const GemmGroupPlan& gp, const void* d_table, c
 // Few tokens make few workgroups for the tile kernel, while the batched decode kernel reads the matrix once
 // per 16 rows with every compute unit busy: a 16-row pass costs (us) 2.5 + 3.2 per 4096 of K (activation
 // staging) + bytes / 6.5 TB/s, plus 15 %; where that kernel splits K over workgroups (K above 4096, partial
-// sums kept with the handle) the staging is paid once and the launch that adds the parts costs 3.5 us.  Measured crossovers
+// sums in the caller's scratch) the staging is paid once and the launch that adds the parts costs 3.5 us.  Measured crossovers
 // without a K split of the tile kernel: 72 tokens at 14336x4096, 115 at 4096x4096, 125 at 4096x14336 (4-bit).
-static bool slices_cheaper(const tfq_weight* w, int M, double tile_us) {
+static bool slices_cheaper(const tfq_weight* w, int M, double tile_us, bool split_scratch) {
     if (!gemv_rows16_supported(w->fmt)) return false;
     const double chunks = std::ceil((double)w->K / 4096.0);
-    const double staging = chunks > 1.0 && w->split_partial ? 3.2 + 3.5 : 3.2 * chunks;
+    const double staging = chunks > 1.0 && split_scratch ? 3.2 + 3.5 : 3.2 * chunks;
     const double t16 = 1.15 * (2.5 + staging + (double)w->dev_bytes / 6.5e6);
     return (double)((M + 15) / 16) * t16 < tile_us;
 }
 
+// bytes of partial sums a 16-row slice of the decode kernel keeps in scratch (0: it does not split K)
+static size_t slice_split_bytes(const tfq_weight* w) {
+    return w->layout == TFQ_LAYOUT_TILED16 ? gemv_rows16_split_bytes(w->fmt, w->N, w->K) : 0;
+}
+
 size_t gemm_scratch_bytes(const tfq_weight* w, int x_dtype, int M) {
-    if (!tile_kernel_serves(w, x_dtype, M)) return 0;
+    if (!tile_kernel_serves(w, x_dtype, M)) return M > 4 ? slice_split_bytes(w) : 0;
     const GemmPlan p = plan_for(w, M, ~(size_t)0);
-    if (p.ksplit == 1 || slices_cheaper(w, M, p.us)) return 0;
+    if (slices_cheaper(w, M, p.us, true)) return slice_split_bytes(w);
+    if (p.ksplit == 1) return 0;
     return (size_t)p.ksplit * (size_t)M * (size_t)w->N * 4;
 }
 
 int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y, int y_dtype, hipStream_t s, void* scratch,
                 size_t scratch_bytes) {
-    if (tile_kernel_serves(w, x_dtype, M) && !slices_cheaper(w, M, plan_for(w, M, scratch ? scratch_bytes : 0).us)) {
+    const size_t slice_ws = slice_split_bytes(w);
+    const bool slices_split = scratch && slice_ws && scratch_bytes >= slice_ws;
+    if (tile_kernel_serves(w, x_dtype, M) && !slices_cheaper(w, M, plan_for(w, M, scratch ? scratch_bytes : 0).us, slices_split)) {
         if (w->N > 0x7FFFFFF0 || w->K > 0x7FFFFFF0 || w->dev_bytes >= 0xFFFFF000ull) return fail(TFQ_ERR_SHAPE, "gemm: matrix too large");
         switch (canonical(w->fmt)) {
             case TFQ_Q_G_4: return run<TFQ_Q_G_4>(w, x, M, y, y_dtype, scratch, scratch_bytes, s);
@@ -689,7 +697,8 @@ int launch_gemm(const tfq_weight* w, const void* x, int x_dtype, int M, void* y,
     for (int m0 = 0; m0 < M; m0 += 16) {
         const int mb = M - m0 < 16 ? M - m0 : 16;
         const int rc = launch_gemv(w, (const uint8_t*)x + (size_t)m0 * w->K * xe, x_dtype, mb,
-                                   (uint8_t*)y + (size_t)m0 * w->N * ye, y_dtype, s);
+                                   (uint8_t*)y + (size_t)m0 * w->N * ye, y_dtype, s, slices_split ? scratch : nullptr,
+                                   slices_split ? scratch_bytes : 0);
         if (rc) return rc;
     }
     return TFQ_OK;

@@ -70,7 +70,7 @@ struct GemvArgs {
     int nslot;         // bf16 activation rows held in LDS: B, or 2B for fp32 input (<= 4)
     int tiles_per_wg;  // T
     int cols_base, cols_rem;  // block columns per wavefront: cols_base + (wave < cols_rem)
-    float* split_partial;     // single matrix only: the handle's area for the partial sums of K parts, or null
+    float* split_partial;     // single matrix only: the caller's area for the partial sums of K parts, or null
     // prologue fused into the activation staging (fp32 input only): XOP_RMSNORM takes gamma / eps /
     // gamma_plus_one, XOP_SWIGLU takes x2 (the up product; x is the gate product) and mid_bf16
     int xop;
@@ -1938,8 +1938,8 @@ int launch_gemv_grouped_direct(int fmt, const GemvGroupPlan& gp, const GemvDirec
 }
 
 int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
-                      void* const* ys, int y_dtype, hipStream_t s) {
-    return launch_gemv_multi_fused(ws, nmat, x, x_dtype, B, ys, y_dtype, nullptr, s);
+                      void* const* ys, int y_dtype, hipStream_t s, void* split_ws, size_t split_ws_bytes) {
+    return launch_gemv_multi_fused(ws, nmat, x, x_dtype, B, ys, y_dtype, nullptr, s, split_ws, split_ws_bytes);
 }
 
 bool gemv_prologue_supported(const tfq_weight* w) { return w->layout == TFQ_LAYOUT_TILED16; }
@@ -1951,7 +1951,8 @@ bool gemv_pair_supported(const tfq_weight* w) {
 }
 
 int launch_gemv_multi_fused(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
-                            void* const* ys, int y_dtype, const tfq_prologue_t* pro, hipStream_t s) {
+                            void* const* ys, int y_dtype, const tfq_prologue_t* pro, hipStream_t s, void* split_ws,
+                            size_t split_ws_bytes) {
     const bool fused = pro && pro->op != TFQ_PRO_NONE;
     const bool accumulate = pro && pro->accumulate;
     const bool pair = pro && pro->pair_swiglu;
@@ -1999,8 +2000,8 @@ int launch_gemv_multi_fused(const tfq_weight* const* ws, int nmat, const void* x
     a.ntiles = (int)tiles;
     a.nmat = nmat;
     a.K = (int)ws[0]->K;
-    if (nmat == 1) {
-        a.split_partial = ws[0]->split_partial;
+    if (nmat == 1 && split_ws && split_ws_bytes >= gemv_rows16_split_bytes(ws[0]->fmt, ws[0]->N, ws[0]->K)) {
+        a.split_partial = static_cast<float*>(split_ws);
     }
     if (pair) {  // one grid over the tiles of gate; the kernel walks the same tiles of up (W[1]) behind them
         a.pair = 1;
@@ -2031,8 +2032,9 @@ int launch_gemv_multi_fused(const tfq_weight* const* ws, int nmat, const void* x
 }
 
 
-int launch_gemv(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype, hipStream_t s) {
-    return launch_gemv_multi(&w, 1, x, x_dtype, B, &y, y_dtype, s);
+int launch_gemv(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype, hipStream_t s, void* split_ws,
+                size_t split_ws_bytes) {
+    return launch_gemv_multi(&w, 1, x, x_dtype, B, &y, y_dtype, s, split_ws, split_ws_bytes);
 }
 
 }  // namespace tfq

@@ -333,10 +333,6 @@ struct tfq_weight {
     size_t dev_bytes;
     int layout;
     bool owns;
-    // Behind the packed weights in the same allocation, for matrices whose K is cut into several parts by the
-    // 5..16-row decode kernel: fp32 partial sums [parts][16 rows][N], written by one launch and added by the
-    // next.  One call at a time per handle may use them.
-    float* split_partial;
     // TFQ_LAYOUT_MIXED: every block carries its own wire id (the container's per-block format byte).  dev holds
     // the payloads one behind the other; these device arrays (behind them in the same allocation) give each
     // block's byte offset and wire id, and the block layout of every wire id.
@@ -373,13 +369,18 @@ int launch_decode_tiled(int fmt, const uint8_t* tiled, int64_t N, int64_t K, flo
 int launch_encode(int fmt, const float* w, int64_t nblocks, uint8_t* dst, hipStream_t s);
 // one block of L.n < 256 weights (the last block of a tensor) in the layout L = block_layout(fmt, L.n)
 int launch_encode_short(int fmt, const BlockLayout& L, const float* w, uint8_t* dst, hipStream_t s);
+// split_ws (optional, device memory, 256-byte aligned): where the 5..16-row kernel of a single matrix with K above
+// 4096 keeps the partial sums of its K parts (gemv_rows16_split_bytes says how many bytes); without it such a call
+// runs unsplit, every workgroup reading whole activation rows.  A handle owns no scratch memory, so calls on one
+// handle may overlap on different streams as long as their workspaces differ.
 int launch_gemv(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype,
-                hipStream_t s);
+                hipStream_t s, void* split_ws = nullptr, size_t split_ws_bytes = 0);
 int launch_gemv_multi(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
-                      void* const* ys, int y_dtype, hipStream_t s);
+                      void* const* ys, int y_dtype, hipStream_t s, void* split_ws = nullptr, size_t split_ws_bytes = 0);
 // the same with a prologue on the (fp32) activations; pro == null or TFQ_PRO_NONE is launch_gemv_multi
 int launch_gemv_multi_fused(const tfq_weight* const* ws, int nmat, const void* x, int x_dtype, int B,
-                            void* const* ys, int y_dtype, const tfq_prologue_t* pro, hipStream_t s);
+                            void* const* ys, int y_dtype, const tfq_prologue_t* pro, hipStream_t s, void* split_ws = nullptr,
+                            size_t split_ws_bytes = 0);
 bool gemv_prologue_supported(const tfq_weight* w);
 bool gemv_pair_supported(const tfq_weight* w);  // the paired gate / up launch with the SwiGLU epilogue
 int launch_gemv_generic(const tfq_weight* w, const void* x, int x_dtype, int B, void* y, int y_dtype,

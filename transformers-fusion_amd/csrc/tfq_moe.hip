@@ -1021,7 +1021,15 @@ int launch_mlp_step(const tfq_weight* gate, const tfq_weight* up, const tfq_weig
     else
         hipLaunchKernelGGL(silu_mul_kernel<false>, dim3((unsigned)((nh + 255) / 256)), dim3(256), 0, s, g, u, h, nh);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return hip_fail(e, "mlp_step launch");
-    return launch_gemm(down, h, mid_dtype, B, y, y_dtype, s, scratch, scratch_bytes);  // sixteen rows or fewer take the decode kernels inside
+    if (B <= 16) {
+        // the decode kernels; the gate and up products are spent once silu(gate) * up is written, so their two areas
+        // hold the partial sums of the down product's K parts when they are large enough (else a longer workspace
+        // than tfq_mlp_workspace_bytes asks for does; else the product runs unsplit)
+        const size_t have_tail = workspace_bytes - 3 * part;
+        void* split_ws = 2 * part >= have_tail ? (void*)g : (void*)((uint8_t*)workspace + 3 * part);
+        return launch_gemm(down, h, mid_dtype, B, y, y_dtype, s, split_ws, 2 * part >= have_tail ? 2 * part : have_tail);
+    }
+    return launch_gemm(down, h, mid_dtype, B, y, y_dtype, s, scratch, scratch_bytes);
 }
 
 }  // namespace tfq
