@@ -221,9 +221,13 @@ int tfq_weight_decode(const tfq_weight_t* w, float* out, tfq_stream_t stream);
  * layout.  The other tiled formats (Q_G_3, Q_G_2, SB256A3, SB256A2) stage an
  * activation row in on-chip memory, which holds K <= 61440 for a bf16 row and
  * K <= 32768 for an fp32 row (49152 and 28672 for the three formats with
- * sixteen scale groups per block); beyond that the call returns TFQ_ERR_SHAPE,
- * as do the fused calls below (tfq_gemv_multi_fused, tfq_mlp_step) for every
- * format at K above 32768. */
+ * sixteen scale groups per block).  Beyond that an fp32 y is still served: the
+ * row is walked in windows of at most 16384 elements of K, one round of launches
+ * per window, each after the first adding into y (so y holds partial sums while
+ * the call runs).  A bf16 y cannot be added to without a second rounding: that
+ * combination returns TFQ_ERR_SHAPE above the limit, as do the fused calls below
+ * (tfq_gemv_multi_fused, tfq_mlp_step) for every format at K above 32768, whose
+ * RMSNorm prologue needs the whole row at once. */
 int tfq_gemv(const tfq_weight_t* w, const void* x, int x_dtype, int B, void* y, int y_dtype,
              tfq_stream_t stream);
 int tfq_gemm(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, int y_dtype,

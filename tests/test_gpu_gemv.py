@@ -518,25 +518,54 @@ def test_very_long_k(O, tfq, gpu, fmt, K, B, xdt):
     W.close()
 
 
-@pytest.mark.parametrize("fmt,K,xdt,ok", [("SB256A2", 49152, "bf16", True), ("SB256A2", 49408, "bf16", False),
-                                          ("Q_G_3", 61440, "bf16", True), ("Q_G_3", 61696, "bf16", False),
-                                          ("SB256A3", 28672, "f32", True), ("SB256A3", 28928, "f32", False)])
-def test_k_ceiling_of_the_staged_formats(O, tfq, gpu, fmt, K, xdt, ok):
-    """The tiled formats outside the sixteen-row kernel run up to the documented K and refuse the next block with
-    an error before anything is launched."""
+@pytest.mark.parametrize("fmt,K,xdt,one_launch", [("SB256A2", 49152, "bf16", True), ("SB256A2", 49408, "bf16", False),
+                                                  ("Q_G_3", 61440, "bf16", True), ("Q_G_3", 61696, "bf16", False),
+                                                  ("SB256A3", 28672, "f32", True), ("SB256A3", 28928, "f32", False)])
+def test_k_ceiling_of_the_staged_formats(O, tfq, gpu, fmt, K, xdt, one_launch):
+    """The tiled formats outside the sixteen-row kernel stage a whole activation row up to a K that depends on the
+    format; one block more and the row is walked in windows of K that add into an fp32 output.  Both sides of the
+    step match the oracle; a bf16 output, which cannot be added to, is refused above the step before any launch."""
     import torch
     N = 16
     pay = O.encode_tensor(fmt, O.rng_laplace(65, N * K, 0.015))
     W = tfq.Weight(fmt, N, K, pay)
     x = O.rng_normal(66, K, 1.0).reshape(1, K)
     xg = torch.from_numpy(O.bf16_round(x)).to(gpu).bfloat16() if xdt == "bf16" else torch.from_numpy(x).to(gpu)
-    if ok:
-        y = W.gemv(xg).cpu().numpy()
-        ref = O.matmul(fmt, pay, N, K, O.bf16_round(x) if xdt == "bf16" else x)
-        assert float(np.abs(y - ref).max() / np.abs(ref).max()) <= 1e-3
+    y = W.gemv(xg).cpu().numpy()
+    ref = O.matmul(fmt, pay, N, K, O.bf16_round(x) if xdt == "bf16" else x)
+    assert float(np.abs(y - ref).max() / np.abs(ref).max()) <= 1e-3
+    if one_launch:
+        assert W.gemv(xg, out_dtype=torch.bfloat16).shape == (1, N)
     else:
         with pytest.raises(Exception, match="K too large"):
-            W.gemv(xg)
+            W.gemv(xg, out_dtype=torch.bfloat16)
+    W.close()
+
+
+@pytest.mark.parametrize("fmt", ["SB256A2", "SB256A3", "Q_G_3", "Q_G_2", "Q_G_6"])
+@pytest.mark.parametrize("K,B,xdt", [(65536, 1, "bf16"), (65536, 8, "bf16"), (65536, 3, "f32"), (70400, 5, "bf16")])
+def test_k_above_the_staging_ceiling_in_windows(O, tfq, gpu, fmt, K, B, xdt):
+    """K = 65536 and a K that no even split divides, one row to eight: windows of block columns, each a round of
+    launches that adds into y, against the oracle's product.  (Q_G_6 is not held as tiles and takes the generic
+    kernel, which has no K limit: it rides along as the control.)"""
+    import torch
+    N = 40
+    pay = O.encode_tensor(fmt, O.rng_laplace(67, N * K, 0.015))
+    W = tfq.Weight(fmt, N, K, pay)
+    x = O.rng_normal(68, B * K, 1.0).reshape(B, K)
+    if xdt == "bf16":
+        x = O.bf16_round(x)
+        xg = torch.from_numpy(x).to(gpu).bfloat16()
+    else:
+        xg = torch.from_numpy(x).to(gpu)
+    y = W.gemv(xg).cpu().numpy()
+    ref = O.matmul(fmt, pay, N, K, x)
+    assert float(np.abs(y - ref).max() / np.abs(ref).max()) <= 1e-3
+    # the same call adds nothing to a second run's result (every window but the first accumulates: y must be
+    # overwritten by the first window, not added to)
+    out = torch.full((B, N), 7.0, device=gpu)
+    W.gemv(xg, out=out)
+    assert np.array_equal(out.cpu().numpy(), y)
     W.close()
 
 

@@ -65,6 +65,7 @@ struct GemvArgs {
     int ntiles;  // all matrices together
     int nmat;
     int K;
+    int kstride;       // 0, or the K of the whole matrix when this launch walks a window of its block columns
     int y_bf16;
     int x_f32;
     int nslot;         // bf16 activation rows held in LDS: B, or 2B for fp32 input (<= 4)
@@ -94,6 +95,7 @@ struct GemvKernArgs {
     int g0, g1, g2;
     int nr0, nr1, nr2, nr3;
     int K, y_bf16, nslot, tiles_per_wg, cols_base, cols_rem;
+    int kstride;  // elements between activation rows and (/ 256) units between tiles when K is a window of a longer row; 0: K
     int kparts, kcols;  // gemvb_kernel: workgroups per row group (K parts) and block columns per part
     float* partial;
     const float* gamma;  // XOP_RMSNORM
@@ -270,7 +272,7 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && (Fmt<FMT>::HV == 1 || (
         const int s0 = (pass & (npc - 1)) * 2;
         const int s = min(s0 + sl_in_pass, nslot - 1);
         const int row = XF32 ? s >> 1 : s;
-        const uint32_t lane_off = ((uint32_t)row * (uint32_t)K + (uint32_t)quad * 8u) * XE;
+        const uint32_t lane_off = ((uint32_t)row * (uint32_t)(args.kstride ? args.kstride : K) + (uint32_t)quad * 8u) * XE;
         const size_t col_off = (size_t)(wave + NW * ci) * (256 * XE);
         const uint4* src = reinterpret_cast<const uint4*>(xbytes + col_off + lane_off);
         lo = src[0];
@@ -301,9 +303,10 @@ __global__ __launch_bounds__((SETS == 1 || (SETS == 2 && (Fmt<FMT>::HV == 1 || (
     // number of loads younger than any operand is a compile-time constant, staging waits for the
     // activations alone and a unit is consumed as soon as IT has arrived (behind a conditional
     // fetch the compiler waits for everything in flight).
-    const size_t tile_stride = (size_t)nblocks * UB;
+    const int nblocks_row = args.kstride ? args.kstride >> 8 : nblocks;  // units between consecutive tiles
+    const size_t tile_stride = (size_t)nblocks_row * UB;
     const ptrdiff_t pair_delta = PAIR ? Wm2 - Wm : 0;
-    const uint8_t* col_ptr = Wm + ((size_t)tile0 * nblocks + (size_t)wave) * UB;
+    const uint8_t* col_ptr = Wm + ((size_t)tile0 * nblocks_row + (size_t)wave) * UB;
     const uint8_t* f_ptr = col_ptr;
     int f_t = 0, f_left = nitems;
     const uint32_t off_c = 16u * lane, off_h = (uint32_t)tiled_header_offset(FMT, n, 0);
@@ -1389,7 +1392,7 @@ int run_gemv_tall(const GemvArgs& a, const void* x, hipStream_t s, bool* taken) 
         // (Up to four rows stay with the column-split kernel, which streams such a matrix as fast or faster:
         // 128256 x 4096 at one row 46.5 us, 6.36 TB/s, against 47.1 us here; at eight rows 54.4 against 51.3 us,
         // 49152 x 8192 60.4 against 41.7 us.)
-        if (a.nmat != 1 || a.x_f32 || a.xop != XOP_NONE || a.pair || a.nslot <= 4 || a.nslot > 8 || a.ntiles < 256 * 12) return TFQ_OK;
+        if (a.nmat != 1 || a.x_f32 || a.xop != XOP_NONE || a.pair || a.kstride || a.nslot <= 4 || a.nslot > 8 || a.ntiles < 256 * 12) return TFQ_OK;
         constexpr int sets = 2;
         const size_t lds = ((size_t)nblocks * (a.nslot * kSlotStride + sets * Fmt<FMT>::NG) + 4) * 16;
         if (lds > 160 * 1024) return TFQ_OK;
@@ -1446,7 +1449,7 @@ int run_gemv4(GemvArgs a, const void* x, hipStream_t s) {
     k.g0 = ends[0]; k.g1 = ends[1]; k.g2 = ends[2];
     int grid = g;
     if (a.nmat == 4) grid += ((a.nrows[3] + 15) / 16 + T - 1) / T;
-    k.K = a.K; k.y_bf16 = a.y_bf16; k.nslot = a.nslot; k.tiles_per_wg = T;
+    k.K = a.K; k.kstride = a.kstride; k.y_bf16 = a.y_bf16; k.nslot = a.nslot; k.tiles_per_wg = T;
     k.cols_base = a.cols_base; k.cols_rem = a.cols_rem;
     k.gamma = a.gamma; k.x2 = a.x2; k.eps = a.eps; k.gamma_plus_one = a.gamma_plus_one; k.mid_bf16 = a.mid_bf16;
     k.accumulate = a.accumulate;
@@ -1627,6 +1630,30 @@ int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t 
         }
     }
     int step = a.x_f32 ? 2 : 4;
+    // Not even one row's staged slices fit (and the format has no sixteen-row kernel): the row is walked in windows
+    // of block columns short enough for a full pass of rows, a round of launches per window, the later windows
+    // adding into y.  That takes fp32 outputs (a bf16 sum cannot be added to without rounding twice) and no
+    // prologue (RMSNorm needs the sum of squares of the whole row).
+    if (a.kstride == 0 && a.xop == XOP_NONE && !a.pair && !a.y_bf16 && plan_gemv4<FMT>(a, a.x_f32 ? 2 : 1).lds == 0) {
+        const int nblocks = a.K >> 8;
+        int wb = nblocks < 64 ? nblocks : 64;
+        GemvArgs wnd = a;
+        wnd.kstride = a.K;
+        for (;; --wb) {
+            wnd.K = wb * 256;
+            if (plan_gemv4<FMT>(wnd, 4).lds != 0) break;
+            if (wb == 1) return fail(TFQ_ERR_SHAPE, "gemv: no window of K fits the LDS activation stage");
+        }
+        const int nwin = (nblocks + wb - 1) / wb;
+        wb = (nblocks + nwin - 1) / nwin;  // windows of even length
+        for (int b0 = 0; b0 < nblocks; b0 += wb) {
+            wnd.K = (nblocks - b0 < wb ? nblocks - b0 : wb) * 256;
+            for (int m = 0; m < a.nmat; ++m) wnd.W[m] = a.W[m] + (size_t)b0 * tiled_unit_bytes(FMT);
+            wnd.accumulate = a.accumulate || b0 != 0;
+            if (int rc = gemv4_batched<FMT>(wnd, (const uint8_t*)x + (size_t)b0 * 256 * xe, xd, B, yd, s)) return rc;
+        }
+        return TFQ_OK;
+    }
     // A long K leaves LDS room for fewer staged rows: halve the rows per pass until the plan fits
     // (K = 16640..20480 takes three or two bf16 rows, one fp32 row up to 32768, one bf16 row up to 61440).
     while (step > 1 && plan_gemv4<FMT>(a, a.x_f32 ? 2 * step : step).lds == 0) step >>= 1;
@@ -1643,7 +1670,7 @@ int gemv4_batched(GemvArgs a, const void* x, int xd, int B, int yd, hipStream_t 
         GemvArgs ab = a;
         ab.nslot = a.x_f32 ? 2 * nb : nb;
         for (int m = 0; m < a.nmat; ++m) ab.y[m] = (uint8_t*)a.y[m] + (size_t)b0 * (size_t)a.nrows[m] * ye;
-        const void* xb = (const uint8_t*)x + (size_t)b0 * a.K * xe;
+        const void* xb = (const uint8_t*)x + (size_t)b0 * (a.kstride ? a.kstride : a.K) * xe;
         if (a.x2) ab.x2 = a.x2 + (size_t)b0 * a.K;
         if (int rc = run_gemv4<FMT>(ab, xb, s)) return rc;
     }
