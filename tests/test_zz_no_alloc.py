@@ -37,19 +37,20 @@ def test_gemm_static_equals_workspace_form(O, tfq, gpu, fmt):
 
 
 def test_gemm_static_refuses_what_does_not_fit(O, tfq, gpu):
+    """4096x14336 at 2048 rows splits K in two: 64 MiB of partial tiles, more than the static area holds.  The call
+    is refused with TFQ_ERR_SHAPE before anything is launched, and y stays as it was."""
     import torch
     fmt, N, K, M = "B32S4", 4096, 14336, 2048
     lib = tfq.lib()
     w = torch.randn(N * K, device=gpu) * 0.02
     W = tfq.Weight(fmt, N, K, tfq.encode(fmt, w))
     need = int(lib.tfq_gemm_workspace_bytes(W.handle, tfq.BF16, M))
+    assert need > 32 << 20, "the case must ask for more than the static area"
     x = torch.zeros(M, K, device=gpu).bfloat16()
-    y = torch.empty(M, N, device=gpu)
+    y = torch.full((M, N), 3.0, device=gpu)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     rc = lib.tfq_gemm_static(W.handle, x.data_ptr(), tfq.BF16, M, y.data_ptr(), tfq.F32, stream)
-    if need > 32 << 20:
-        assert rc == 3 and b"static area" in lib.tfq_last_error()
-    else:
-        assert rc == 0
+    assert rc == 3 and b"static area" in lib.tfq_last_error()
     torch.cuda.synchronize()
+    assert bool((y == 3.0).all())
     W.close()
