@@ -259,7 +259,9 @@ int tfq_gemm_ws(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* 
  * its copy until the process ends); the call itself allocates nothing.  A product whose split would use more
  * (tfq_gemm_workspace_bytes above that size) is refused with TFQ_ERR_SHAPE.  Same results as tfq_gemm_ws with
  * a workspace of tfq_gemm_workspace_bytes.  All calls on one GPU share the array: calls that overlap in time
- * on one GPU race (issue them on one stream).  No counterpart in the reference. */
+ * on one GPU race (issue them on one stream).  The first call on a device resolves the array's address and
+ * raises the kernel's LDS limit, which a capturing stream does not allow: make one call of the same shape
+ * before a capture starts.  No counterpart in the reference: it is for callers that cannot allocate. */
 int tfq_gemm_static(const tfq_weight_t* w, const void* x, int x_dtype, int M, void* y, int y_dtype,
                     tfq_stream_t stream);
 size_t tfq_gemm_static_scratch_bytes(void);

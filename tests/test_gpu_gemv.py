@@ -235,6 +235,28 @@ def test_config4_lowbit_superblock_shapes(O, tfq, gpu, fmt, bits):
     W.close()
 
 
+@pytest.mark.parametrize("fmt", ["SB256A3", "SB256A2"])
+def test_config4_lowbit_superblock_full_size(tfq, gpu, fmt):
+    """The whole 14336x4096 matrix of the benchmark's low-bit configuration (Laplace(0, 0.015) weights encoded on
+    the device), batch 1 and batch 8, against the float64 product of the device-decoded matrix; the decoded matrix
+    itself is pinned bit for bit against the oracle by the tests above."""
+    import torch
+    N, K = 14336, 4096
+    g = torch.Generator(device="cuda").manual_seed(44)
+    u = torch.rand(N * K, device=gpu, generator=g) - 0.5
+    w = -0.015 * torch.sign(u) * torch.log1p(-2 * u.abs().clamp(max=0.4999999))
+    W = tfq.Weight(fmt, N, K, tfq.encode(fmt, w))
+    dense = W.decode().double()
+    for B in (1, 8):
+        x = torch.randn(B, K, device=gpu, generator=g).bfloat16()
+        want = x.double() @ dense.T
+        y = W.gemv(x)
+        assert float((y.double() - want).abs().max() / want.abs().max()) <= 1e-4
+        yb = W.gemv(x, out_dtype=torch.bfloat16)
+        assert float((yb.double() - want).abs().max() / want.abs().max()) <= 1e-2
+    W.close()
+
+
 @pytest.mark.parametrize("fmt", ["SB256A3", "SB256A2", "Q_G_2"])
 @pytest.mark.parametrize("N,K", [(4200, 1024), (40, 14336), (1000, 2304)])
 def test_one_row_of_the_byte_header_formats(O, tfq, gpu, fmt, N, K):
