@@ -331,7 +331,8 @@ int tfq_mlp_step(const tfq_weight_t* gate, const tfq_weight_t* up, const tfq_wei
  * while the arithmetic of a phase waits for the phase before it.
  *
  * A phase multiplies up to four matrices (one format per chain: B32S4 or Q_G_4; equal K inside
- * a phase, K <= 14336) with the same B <= 2 activation rows.
+ * a phase, K <= 16384; dtypes TFQ_F32 or TFQ_BF16, one output dtype per chain; tfq_chain_create
+ * refuses anything else with TFQ_ERR_SHAPE or TFQ_ERR_ARG) with the same B <= 2 activation rows.
  *   x          first phase: device pointer [B][K] (x_dtype).  Every later phase: NULL; it reads the
  *              result of the phase before it, which is the concatenation of that phase's outputs
  *              [B][N0 + N1 + ...] (its first K columns are used), the SwiGLU product [B][N], or the
